@@ -1,0 +1,130 @@
+/*
+ * libternaspmm.so -- C ABI of the TernaSpMM path, MI355X (gfx950) build.
+ *
+ * The first eight symbols are the ones the reference library exports and that its
+ * callers bind (model.py:21,76-89 through ctypes; tests/test_kernel.cu:51-76).  Names,
+ * argument order and argument meaning are unchanged; "bf16" is 16-bit bfloat storage and
+ * the stream argument is a hipStream_t (PyTorch-ROCm's stream.cuda_stream).  The symbols
+ * after them are additions of this build and have no counterpart in the reference.
+ *
+ * Conventions shared by every compute entry point:
+ *   - all pointers are device memory owned by the caller; `out` [M][N] row-major bf16 is
+ *     fully overwritten; nothing is allocated, freed or synchronised on the call path;
+ *   - W is [N][K] ternary in the compressed format (bitmap / TileOffsets_global /
+ *     TileOffsets_median / sign words), N % 64 == 0 and K % 64 == 0;
+ *   - calls only enqueue work on `stream` and are safe under stream capture;
+ *   - on a HIP runtime error the library prints the error and exits the process, as the
+ *     reference does (kernels/TernaSpMM.cu:15-22).
+ */
+#ifndef TERNASPMM_H
+#define TERNASPMM_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef uint16_t terna_bf16;   /* bfloat16 storage                                   */
+typedef void*    terna_stream; /* hipStream_t                                        */
+
+/* ---- reference symbols ------------------------------------------------------------- */
+
+/* kernels/TernaSpMM.cu:15 -- print and exit(1) if the runtime holds a pending error. */
+void checkLastCudaError(int line);
+
+/* kernels/TernaSpMM.cu:25 -- out = bf16( (x_q . W^T) scaled ), int8 activations.
+ *   x       int8  [M][K] row-major (quantised activations)
+ *   s       bf16  [M]    per-row activation scale (x_q = round(x*s))
+ *   ws      bf16  [>=ws_num] weight-group scales, ws_num groups along N
+ *   M <= 64 : epilogue bf16((acc / s[m]) * ws[g])        (Reduction_Kernel.cuh:60)
+ *   M  > 64 : epilogue bf16(acc * (ws[g] / s[m])), 0 if s[m]==0, g per 128-column tile
+ *                                                        (epilogue_visitor_scale_ws.h:135-205)
+ *   SPLIT_K and workspace are accepted for compatibility; this build reduces split-K
+ *   partials on chip and never touches `workspace`. */
+void bitlinear_TernaSpMM(int8_t* x, uint64_t* bitmap, int* tile_offsets_global,
+                         uint16_t* tile_offsets_median, uint32_t* sign_words,
+                         terna_bf16* out, terna_bf16* s, terna_bf16* ws, int ws_num,
+                         int M, int N, int K, int SPLIT_K, int32_t* workspace, terna_stream stream);
+
+/* kernels/TernaSpMM.cu:79 -- as above, always the decode epilogue. */
+void bitlinear_TernaSpMM_decode(int8_t* x, uint64_t* bitmap, int* tile_offsets_global,
+                                uint16_t* tile_offsets_median, uint32_t* sign_words,
+                                terna_bf16* out, terna_bf16* s, terna_bf16* ws, int ws_num,
+                                int M, int N, int K, int SPLIT_K, int32_t* workspace, terna_stream stream);
+
+/* kernels/TernaSpMM.cu:110 -- as above, always the prefill epilogue. */
+void bitlinear_TernaSpMM_prefill(int8_t* x, uint64_t* bitmap, int* tile_offsets_global,
+                                 uint16_t* tile_offsets_median, uint32_t* sign_words,
+                                 terna_bf16* out, terna_bf16* s, terna_bf16* ws, int ws_num,
+                                 int M, int N, int K, int SPLIT_K, int32_t* workspace, terna_stream stream);
+
+/* kernels/TernaSpMM.cu:141 -- mode 0/1/2 = auto/prefill/decode; warm-up, event-timed loop,
+ * prints "Shape(M=, N=, K=): %.2f us (avg over %d iters, warmup=%d)".  Synchronises. */
+void bitlinear_TernaSpMM_benchmark(int mode, int warmup_iters, int bench_iters,
+                                   int8_t* x, uint64_t* bitmap, int* tile_offsets_global,
+                                   uint16_t* tile_offsets_median, uint32_t* sign_words,
+                                   terna_bf16* out, terna_bf16* s, terna_bf16* ws, int ws_num,
+                                   int M, int N, int K, int SPLIT_K, int32_t* workspace, terna_stream stream);
+
+/* kernels/TernaSpMM.cu:241 -- host only: 16x16 block permutation of a bf16 [N][K] matrix. */
+void reorder_WT_h(terna_bf16* W, terna_bf16* W_reordered, int N, int K);
+
+/* kernels/TernaSpMM.cu:282 -- host only: encode an already reordered bf16 [N][K] matrix.
+ * The tile-size arguments must be 64,16,8,64,64,8 (the only values the reference passes,
+ * tests/test_kernel.cu:255); anything else returns -1.  Returns the number of 64x64 tiles.
+ * *bitmap is pinned host memory (free with hipHostFree); the other three are malloc'd
+ * (free with free()).  max_nnz_count is the reference's `int&`. */
+int convert_reorderd(terna_bf16* A_h, int N, int K, int tile_N, int warp_subtile_N, int subtile_N,
+                     int tile_K, int warp_subtile_K, int subtile_K,
+                     uint64_t** bitmap, int** tile_offsets_global, uint16_t** tile_offsets_median,
+                     uint32_t** sign_words, int* max_nnz_count);
+
+/* kernels/TernaSpMM.cu:454 -- enqueue a kernel that spins for about `us` microseconds. */
+void gpu_sleep(double us, terna_stream stream);
+
+/* ---- additions of this build (no counterpart in the reference) ---------------------- */
+
+/* bf16-activation family: out = bf16( (x . W^T) * scale[g(n)] ), fp32 accumulate.
+ *   x bf16 [M][K], any M >= 1 (no padding rows needed); scale fp32 [ws_num];
+ *   group rule of the decode path (Reduction_Kernel.cuh:46-54).
+ * The plain symbol picks a kernel by M; _decode / _prefill force the small-M dot-product
+ * kernel or the MFMA-tiled kernel.  workspace may be NULL. */
+void bitlinear_TernaSpMM_bf16(const terna_bf16* x, const uint64_t* bitmap, const int* tile_offsets_global,
+                              const uint16_t* tile_offsets_median, const uint32_t* sign_words,
+                              terna_bf16* out, const float* scale, int ws_num,
+                              int M, int N, int K, int SPLIT_K, void* workspace, terna_stream stream);
+void bitlinear_TernaSpMM_bf16_decode(const terna_bf16* x, const uint64_t* bitmap, const int* tile_offsets_global,
+                                     const uint16_t* tile_offsets_median, const uint32_t* sign_words,
+                                     terna_bf16* out, const float* scale, int ws_num,
+                                     int M, int N, int K, int SPLIT_K, void* workspace, terna_stream stream);
+void bitlinear_TernaSpMM_bf16_prefill(const terna_bf16* x, const uint64_t* bitmap, const int* tile_offsets_global,
+                                      const uint16_t* tile_offsets_median, const uint32_t* sign_words,
+                                      terna_bf16* out, const float* scale, int ws_num,
+                                      int M, int N, int K, int SPLIT_K, void* workspace, terna_stream stream);
+
+/* Host only: sizes of the four format arrays for an [N][K] matrix.  sign_words_capacity is
+ * the worst case (all weights nonzero).  Returns 0, or -1 if N or K is not a multiple of 64. */
+int ternaspmm_encode_sizes(int N, int K, int64_t* bitmap_len, int64_t* tile_offsets_global_len,
+                           int64_t* tile_offsets_median_len, int64_t* sign_words_capacity);
+
+/* Host only: reorder + encode an ORIGINAL (not reordered) ternary int8 [N][K] matrix into
+ * caller-provided arrays of the sizes above.  Returns the number of sign words written
+ * (= tile_offsets_global[last] / 32), or -1 on a bad shape or a value outside {-1,0,1}.
+ * Output is bit-identical to reorder_weight + compress_weight (convert/convert_utils.py:9-228). */
+int64_t ternaspmm_encode_i8(const int8_t* W, int N, int K, uint64_t* bitmap, int* tile_offsets_global,
+                            uint16_t* tile_offsets_median, uint32_t* sign_words);
+
+/* Device: expand the compressed format to a dense row-major bf16 [N][K] matrix of
+ * {-1, 0, +1} on `stream` (load-time inspection and round-trip checks). */
+void ternaspmm_decompress_bf16(const uint64_t* bitmap, const int* tile_offsets_global,
+                               const uint16_t* tile_offsets_median, const uint32_t* sign_words,
+                               terna_bf16* W_dense, int N, int K, terna_stream stream);
+
+/* Library version string, e.g. "ternaspmm-gfx950 0.1". */
+const char* ternaspmm_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TERNASPMM_H */

@@ -1,0 +1,8 @@
+"""MI355X-native TernaSpMM: ternary-weight sparse x dense matmul behind libternaspmm.so."""
+from . import _lib  # noqa: F401
+from .convert_utils import compress_weight, reorder_weight, quant_weight_int8, pack_weight_scale  # noqa: F401
+from .linear import (  # noqa: F401
+    BF16BitLinear, SpBitLinear, SpBitLinearBF16, TernaInfer_linear, TernaInfer_linear_bf16,
+    get_global_workspace)
+
+__version__ = "0.1"

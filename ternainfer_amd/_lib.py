@@ -1,0 +1,57 @@
+"""ctypes loader for ``kernels/libternaspmm.so`` (the C-ABI boundary of the TernaSpMM path).
+
+The reference binds the library with ``ctypes.CDLL('./kernels/libternaspmm.so')`` and no
+prototypes (model.py:21).  Here the path is resolved from the package location so that the
+import works from any directory, and prototypes are declared so that a wrong argument count
+fails in Python instead of corrupting the call.  There is no fallback: if the library has
+not been built the import raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.environ.get("TERNASPMM_LIB", os.path.join(_ROOT, "kernels", "libternaspmm.so"))
+
+_vp, _ci = ctypes.c_void_p, ctypes.c_int
+_i8_args = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _vp]
+_bf16_args = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _vp]
+
+#: every symbol include/ternaspmm.h declares -> (argtypes, restype)
+PROTOTYPES = {
+    "checkLastCudaError": ([_ci], None),
+    "bitlinear_TernaSpMM": (_i8_args, None),
+    "bitlinear_TernaSpMM_decode": (_i8_args, None),
+    "bitlinear_TernaSpMM_prefill": (_i8_args, None),
+    "bitlinear_TernaSpMM_benchmark": ([_ci, _ci, _ci] + _i8_args, None),
+    "reorder_WT_h": ([_vp, _vp, _ci, _ci], None),
+    "convert_reorderd": ([_vp, _ci, _ci, _ci, _ci, _ci, _ci, _ci, _ci, _vp, _vp, _vp, _vp, _vp], _ci),
+    "gpu_sleep": ([ctypes.c_double, _vp], None),
+    "bitlinear_TernaSpMM_bf16": (_bf16_args, None),
+    "bitlinear_TernaSpMM_bf16_decode": (_bf16_args, None),
+    "bitlinear_TernaSpMM_bf16_prefill": (_bf16_args, None),
+    "ternaspmm_encode_sizes": ([_ci, _ci, _vp, _vp, _vp, _vp], _ci),
+    "ternaspmm_encode_i8": ([_vp, _ci, _ci, _vp, _vp, _vp, _vp], ctypes.c_int64),
+    "ternaspmm_decompress_bf16": ([_vp, _vp, _vp, _vp, _vp, _ci, _ci, _vp], None),
+    "ternaspmm_version": ([], ctypes.c_char_p),
+}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library once and attach prototypes.  Raises if it is missing."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} not found: build it with `bash kernels/compile.sh` "
+                "(hipcc --offload-arch=gfx950); there is no fallback path")
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (argtypes, restype) in PROTOTYPES.items():
+            fn = getattr(lib, name)          # AttributeError if the symbol is not exported
+            fn.argtypes = argtypes
+            fn.restype = restype
+        _lib = lib
+    return _lib

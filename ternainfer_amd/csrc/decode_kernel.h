@@ -1,0 +1,237 @@
+// Small-M TernaSpMM kernel for gfx950: streams the compressed weight format once and
+// multiplies it by a handful of activation rows.
+//
+// Work split.  One workgroup owns one 16-row band of W (a "median tile" row of the
+// format, the smallest unit with its own sign-stream offset) over the whole K, for up
+// to 16*MB batch rows.  Its WAVES wavefronts take the band's 64-column tiles round
+// robin, accumulate in MFMA registers, and are summed through LDS in a fixed order.
+// The scale epilogue and the bf16 store are fused behind that sum: one launch, no
+// global workspace, no atomics, bit-reproducible.
+//
+// Lane mapping for one 16x64 band-tile (16 bitmaps b = 4*g + 2*sk + sm, bit = 8*r + c
+// <-> row 8*sk + r, column 16*g + 4*(c>>1) + 2*sm + (c&1)):
+//   lane L: i = L & 15 (W row inside the band, also the batch row of the B operand),
+//           g = L >> 4 (16-column group).
+//   One byte of a bitmap is 8 weights of one row, which is exactly one lane's share of a
+//   16x16x32 MFMA A operand.  MFMA number t (t = sm = 0,1) therefore takes byte r = i&7
+//   of bitmap 4g + 2(i>>3) + t.  The matching B operand is dwords t, 2+t, 4+t, 6+t of the
+//   32 contiguous bytes X[m][64*gk + 16*g ..], so X needs no shuffling at all.
+//   Sign bits: position of a lane's byte in the stream = tile offset + band offset
+//   + popcounts of earlier bitmaps (16-lane DPP prefix scan) + popcount of the lower bytes.
+//   The (nonzero nibble, next 4 sign bits) pair indexes a 256-entry LDS table that yields the
+//   four bf16 (or int8) operand values in one read.
+#pragma once
+
+#include "terna_common.h"
+
+namespace terna {
+
+template <typename Act> struct ActTraits;
+
+template <> struct ActTraits<uint16_t> {        // bf16 activations, fp32 accumulate
+    using Acc = f32x4;
+    using AccScalar = float;
+    using Lut = uint2;
+    static constexpr int kXVecs = 2;             // 2 x 16 B = 16 bf16 per (row, 16-col group)
+    __device__ static Lut make_lut(int e) { return make_lut_bf16(e); }
+};
+
+template <> struct ActTraits<int8_t> {          // int8 activations, int32 accumulate
+    using Acc = i32x4;
+    using AccScalar = int;
+    using Lut = uint32_t;
+    static constexpr int kXVecs = 1;             // 16 B = 16 int8
+    __device__ static Lut make_lut(int e) { return make_lut_i8(e); }
+};
+
+__device__ __forceinline__ int row16_inclusive_scan(int v)
+{
+    // Inclusive prefix sum inside each row of 16 lanes: row_shr:n with bound_ctrl (zeros shifted in).
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, true);
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, true);
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, true);
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, true);
+    return v;
+}
+
+// Per-lane constants of the band-tile mapping described at the top of this file.
+struct LaneGeom {
+    int i, g, sk, r, b0;
+    uint32_t lo_mask, hi_mask;     // bits of a bitmap that precede byte r
+    __device__ explicit LaneGeom(int lane)
+    {
+        i = lane & 15;
+        g = lane >> 4;
+        sk = i >> 3;
+        r = i & 7;
+        b0 = 4 * g + 2 * sk;       // bitmap for t = 0; t = 1 is the next one
+        lo_mask = r >= 4 ? 0xffffffffu : ((1u << (8 * r)) - 1u);
+        hi_mask = r > 4 ? ((1u << (8 * (r - 4))) - 1u) : 0u;
+    }
+};
+
+// For one band-tile: the two bytes (t = 0, 1) of nonzero flags this lane owns and the four
+// expansion-table indices that turn them into operand values.
+//   scan_bm   bitmap (lane & 15) of the band-tile, bm[t] bitmap b0 + t
+//   sign_base stream position (in bits) where the band-tile's signs start
+__device__ __forceinline__ void band_tile_indices(const LaneGeom& q, uint64_t scan_bm, const uint64_t bm[2],
+                                                  int sign_base, const uint32_t* __restrict__ sign_words,
+                                                  int last_word, uint32_t idx[2][2])
+{
+    const int pc = __popcll(scan_bm);
+    const int excl = row16_inclusive_scan(pc) - pc;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const uint32_t lo = static_cast<uint32_t>(bm[t]);
+        const uint32_t hi = static_cast<uint32_t>(bm[t] >> 32);
+        const uint32_t nzb = ((q.r >= 4 ? hi : lo) >> (8 * (q.r & 3))) & 0xffu;
+        const int below = __popc(lo & q.lo_mask) + __popc(hi & q.hi_mask);
+        const int before = __builtin_amdgcn_ds_bpermute((q.b0 + t) << 2, excl);
+        const int pos = sign_base + before + below;
+        uint32_t w0 = 0, w1 = 0;
+        if (nzb) {                          // a set bit guarantees pos>>5 is a valid word
+            const int wi = pos >> 5;
+            w0 = sign_words[wi];
+            w1 = sign_words[wi < last_word ? wi + 1 : last_word];
+        }
+        const uint32_t sbits = __builtin_amdgcn_alignbit(w1, w0, pos & 31);
+        const uint32_t n_lo = nzb & 15u;
+        idx[t][0] = (n_lo << 4) | (sbits & 15u);
+        idx[t][1] = (nzb & 0xf0u) | ((sbits >> __popc(n_lo)) & 15u);
+    }
+}
+
+// What a lane fetches for one band-tile before any arithmetic.
+template <typename Act, int MB>
+struct BandTileRaw {
+    uint64_t scan_bm;                       // bitmap (L & 15), for the prefix scan
+    uint64_t bm[2];                         // bitmaps 4g + 2sk + t
+    uint4    x[MB][ActTraits<Act>::kXVecs]; // activation bytes of (row, group g)
+    int      sign_base;                     // tile offset + band offset, in sign bits
+};
+
+template <typename Act, int WAVES, int MB>
+__global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
+    const Act* __restrict__ x, const uint64_t* __restrict__ bitmap, const int* __restrict__ tile_off,
+    const uint16_t* __restrict__ median_off, const uint32_t* __restrict__ sign_words,
+    uint16_t* __restrict__ out, Epilogue ep, int M, int N, int K)
+{
+    using T = ActTraits<Act>;
+    using Acc = typename T::Acc;
+    using Lut = typename T::Lut;
+
+    __shared__ Lut lut[256];
+    __shared__ Acc red[WAVES][MB][64];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    for (int e = tid; e < 256; e += WAVES * 64) lut[e] = T::make_lut(e);
+
+    const int band = blockIdx.x;            // 16-row band of W
+    const int gm = band >> 2, med = band & 3;
+    const int m_base = blockIdx.y * (16 * MB);
+    const int ktiles = K >> 6;
+    const int last_word = (tile_off[(N >> 6) * ktiles] >> 5) - 1;   // index of the last sign word
+
+    const LaneGeom q(lane);
+    const int i = q.i, g = q.g, b0 = q.b0;
+
+    int xrow[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        const int m = m_base + mb * 16 + i;
+        xrow[mb] = m < M ? m : M - 1;       // rows past M repeat the last one; never stored
+    }
+
+    auto fetch = [&](int gk, BandTileRaw<Act, MB>& raw) {
+        const int tile = gm * ktiles + gk;
+        const uint64_t* bmp = bitmap + static_cast<size_t>(tile) * 64 + med * 16;
+        raw.scan_bm = bmp[i];
+        raw.bm[0] = bmp[b0];
+        raw.bm[1] = bmp[b0 + 1];
+        int base = tile_off[tile];
+        if (med) base += median_off[3 * tile + med - 1];
+        raw.sign_base = base;
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            const Act* xp = x + static_cast<size_t>(xrow[mb]) * K + gk * 64 + g * 16;
+#pragma unroll
+            for (int v = 0; v < T::kXVecs; ++v) raw.x[mb][v] = reinterpret_cast<const uint4*>(xp)[v];
+        }
+    };
+
+    Acc acc[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb] = Acc{0, 0, 0, 0};
+
+    BandTileRaw<Act, MB> cur, nxt;
+    int gk = wave;
+    if (gk < ktiles) fetch(gk, cur);
+    __syncthreads();                        // expansion table ready
+
+    for (; gk < ktiles; gk += WAVES) {
+        const bool more = gk + WAVES < ktiles;
+        if (more) fetch(gk + WAVES, nxt);
+
+        uint32_t idx[2][2];
+        band_tile_indices(q, cur.scan_bm, cur.bm, cur.sign_base, sign_words, last_word, idx);
+
+        if constexpr (sizeof(Act) == 2) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const uint2 a_lo = lut[idx[t][0]];
+                const uint2 a_hi = lut[idx[t][1]];
+                const uint4 a_bits = make_uint4(a_lo.x, a_lo.y, a_hi.x, a_hi.y);
+                const bf16x8 a = __builtin_bit_cast(bf16x8, a_bits);
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    const uint4 x0 = cur.x[mb][0], x1 = cur.x[mb][1];
+                    const uint4 b_bits = t == 0 ? make_uint4(x0.x, x0.z, x1.x, x1.z)
+                                                : make_uint4(x0.y, x0.w, x1.y, x1.w);
+                    const bf16x8 b = __builtin_bit_cast(bf16x8, b_bits);
+                    acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mb], 0, 0, 0);
+                }
+            }
+        } else {
+            // k order of the 16x16x64 operand: (t, c) -> column 4*(c>>1) + 2*t + (c&1)
+            const i32x4 a = {static_cast<int>(lut[idx[0][0]]), static_cast<int>(lut[idx[0][1]]),
+                             static_cast<int>(lut[idx[1][0]]), static_cast<int>(lut[idx[1][1]])};
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                const uint4 xv = cur.x[mb][0];       // dword j = columns 4j .. 4j+3
+                const i32x4 b = {
+                    static_cast<int>(__builtin_amdgcn_perm(xv.y, xv.x, 0x05040100u)),   // t=0, c=0..3
+                    static_cast<int>(__builtin_amdgcn_perm(xv.w, xv.z, 0x05040100u)),   // t=0, c=4..7
+                    static_cast<int>(__builtin_amdgcn_perm(xv.y, xv.x, 0x07060302u)),   // t=1, c=0..3
+                    static_cast<int>(__builtin_amdgcn_perm(xv.w, xv.z, 0x07060302u))};  // t=1, c=4..7
+                acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[mb], 0, 0, 0);
+            }
+        }
+        if (more) cur = nxt;
+    }
+
+    // Cross-wave sum in wave order, then the fused epilogue.  The accumulator layout of a
+    // 16x16 MFMA: lane L holds output rows 4*(L>>4) .. +3 of column L & 15.
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) red[wave][mb][lane] = acc[mb];
+    __syncthreads();
+    for (int mb = wave; mb < MB; mb += WAVES) {
+        Acc sum = red[0][mb][lane];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) sum += red[w][mb][lane];
+        const int m = m_base + mb * 16 + i;
+        if (m < M) {
+            const int n0 = band * 16 + 4 * g;
+            uint16_t o[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                o[v] = apply_epilogue<typename T::AccScalar>(ep, sum[v], m, n0 + v, N);
+            uint2 packed = make_uint2(o[0] | (static_cast<uint32_t>(o[1]) << 16),
+                                      o[2] | (static_cast<uint32_t>(o[3]) << 16));
+            *reinterpret_cast<uint2*>(out + static_cast<size_t>(m) * N + n0) = packed;
+        }
+    }
+}
+
+}  // namespace terna

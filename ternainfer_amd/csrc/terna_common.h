@@ -1,0 +1,120 @@
+// Shared device-side definitions for the TernaSpMM kernels (gfx950, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace terna {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+
+constexpr int kWave = 64;
+
+// Which scaling rule the epilogue applies; each follows one reference source.
+enum EpilogueKind : int {
+    EP_I8_DECODE  = 0,  // bf16((float(acc) / s[m]) * ws[g])           Reduction_Kernel.cuh:45-60
+    EP_I8_PREFILL = 1,  // bf16(float(acc) * (ws[g] / s[m])), 0 if s==0  epilogue_visitor_scale_ws.h:135-205
+    EP_BF16       = 2,  // bf16(acc * scale[g]), fp32 scale             (bf16-activation family)
+};
+
+struct Epilogue {
+    const uint16_t* s;      // bf16 [M]       (int8 family)
+    const uint16_t* ws;     // bf16 [ws_num]  (int8 family)
+    const float*    scale;  // fp32 [ws_num]  (bf16 family)
+    int             ws_num;
+    int             kind;
+};
+
+__device__ __forceinline__ float bf16_bits_to_float(uint16_t h)
+{
+    return __uint_as_float(static_cast<uint32_t>(h) << 16);
+}
+
+// Round to nearest even, NaN kept quiet: the rounding of __float2bfloat16_rn.
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return static_cast<uint16_t>(u >> 16);
+}
+
+// Weight-scale group of output column n on the decode path (Reduction_Kernel.cuh:46-54).
+__device__ __forceinline__ int ws_group_decode(int n, int N, int ws_num)
+{
+    if (ws_num == 3 && N == 3840) return n < 2560 ? 0 : (n < 3200 ? 1 : 2);
+    return n / (N / ws_num);
+}
+
+// Prefill path: the group of the first column of the 128-wide tile that holds n, clamped
+// (epilogue_visitor_scale_ws.h:135-148).
+__device__ __forceinline__ int ws_group_prefill(int n, int N, int ws_num)
+{
+    const int c0 = n & ~127;
+    int g;
+    if (N == 3840) g = c0 < 2560 ? 0 : (c0 < 3200 ? 1 : 2);
+    else g = c0 / (N / ws_num);
+    return g < ws_num ? g : ws_num - 1;
+}
+
+// One output element: integer or float accumulator -> bf16 storage.
+template <typename Acc>
+__device__ __forceinline__ uint16_t apply_epilogue(const Epilogue& ep, Acc acc, int m, int n, int N)
+{
+    float r;
+    if (ep.kind == EP_BF16) {
+        r = static_cast<float>(acc) * ep.scale[ws_group_decode(n, N, ep.ws_num)];
+    } else if (ep.kind == EP_I8_DECODE) {
+        const float sv = bf16_bits_to_float(ep.s[m]);
+        const float wv = bf16_bits_to_float(ep.ws[ws_group_decode(n, N, ep.ws_num)]);
+        const float q = __fdiv_rn(static_cast<float>(acc), sv);
+        r = __fmul_rn(q, wv);
+    } else {
+        const float sv = bf16_bits_to_float(ep.s[m]);
+        const float wv = bf16_bits_to_float(ep.ws[ws_group_prefill(n, N, ep.ws_num)]);
+        const float coeff = (sv != 0.0f) ? __fdiv_rn(wv, sv) : 0.0f;
+        r = __fmul_rn(static_cast<float>(acc), coeff);
+    }
+    return float_to_bf16_bits(r);
+}
+
+// Expansion tables: index = (nonzero nibble << 4) | (next 4 sign bits of the stream).
+// The j-th set bit of the nibble takes sign bit number popcount(nibble below j).
+//   bf16 table: 4 x bf16 (+1 = 0x3F80, -1 = 0xBF80) in 8 bytes
+//   int8 table: 4 x int8 (+1 = 0x01,  -1 = 0xFF)   in 4 bytes
+__device__ __forceinline__ uint2 make_lut_bf16(int e)
+{
+    const int nz = e >> 4, sg = e & 15;
+    uint32_t v[4];
+    int used = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if ((nz >> j) & 1) {
+            v[j] = ((sg >> used) & 1) ? 0xBF80u : 0x3F80u;
+            ++used;
+        } else {
+            v[j] = 0u;
+        }
+    }
+    return make_uint2(v[0] | (v[1] << 16), v[2] | (v[3] << 16));
+}
+
+__device__ __forceinline__ uint32_t make_lut_i8(int e)
+{
+    const int nz = e >> 4, sg = e & 15;
+    uint32_t r = 0;
+    int used = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if ((nz >> j) & 1) {
+            r |= (((sg >> used) & 1) ? 0xFFu : 0x01u) << (8 * j);
+            ++used;
+        }
+    }
+    return r;
+}
+
+}  // namespace terna

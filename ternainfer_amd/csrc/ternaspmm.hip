@@ -1,0 +1,265 @@
+// libternaspmm.so: the extern "C" boundary of the TernaSpMM path on MI355X (gfx950).
+// Declarations and the reference interface each symbol stands for: include/ternaspmm.h.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+
+#include "../../include/ternaspmm.h"
+#include "decode_kernel.h"
+#include "decompress_kernel.h"
+#include "format_host.h"
+
+using namespace terna;
+
+namespace {
+
+constexpr int kDecodeWaves = 8;
+
+[[noreturn]] void die(const char* what, hipError_t e, int line)
+{
+    std::printf("Last Cuda Error Detected at line: %d, Error: %s (%s).\n", line, hipGetErrorString(e), what);
+    std::fflush(stdout);
+    std::exit(EXIT_FAILURE);
+}
+
+bool shape_ok(int M, int N, int K)
+{
+    if (M < 1 || N < 64 || K < 64 || (N % 64) || (K % 64)) {
+        std::printf("TernaSpMM Error: unsupported shape M=%d N=%d K=%d (need M >= 1, N %% 64 == 0, K %% 64 == 0)\n",
+                    M, N, K);
+        std::fflush(stdout);
+        return false;
+    }
+    return true;
+}
+
+struct Weights {
+    const uint64_t* bitmap;
+    const int* tile_off;
+    const uint16_t* median_off;
+    const uint32_t* sign_words;
+};
+
+// Small-M kernel: one workgroup per 16-row band; up to 64 batch rows per workgroup.
+template <typename Act>
+void launch_decode(const Act* x, const Weights& w, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                   hipStream_t st)
+{
+    const dim3 block(kDecodeWaves * 64);
+    if (M <= 16) {
+        terna_decode_kernel<Act, kDecodeWaves, 1><<<dim3(N / 16, 1), block, 0, st>>>(
+            x, w.bitmap, w.tile_off, w.median_off, w.sign_words, out, ep, M, N, K);
+    } else if (M <= 32) {
+        terna_decode_kernel<Act, kDecodeWaves, 2><<<dim3(N / 16, 1), block, 0, st>>>(
+            x, w.bitmap, w.tile_off, w.median_off, w.sign_words, out, ep, M, N, K);
+    } else {
+        terna_decode_kernel<Act, kDecodeWaves, 4><<<dim3(N / 16, (M + 63) / 64), block, 0, st>>>(
+            x, w.bitmap, w.tile_off, w.median_off, w.sign_words, out, ep, M, N, K);
+    }
+}
+
+template <typename Act>
+void launch_prefill(const Act* x, const Weights& w, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                    hipStream_t st)
+{
+    // Until the MFMA-tiled kernel covers this range the small-M kernel computes it; the
+    // epilogue rule is the caller's, so results are unchanged.
+    launch_decode(x, w, out, ep, M, N, K, st);
+}
+
+enum Route { ROUTE_AUTO, ROUTE_DECODE, ROUTE_PREFILL };
+
+void run_i8(Route route, int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* median_off, uint32_t* sign_words,
+            uint16_t* out, uint16_t* s, uint16_t* ws, int ws_num, int M, int N, int K, hipStream_t st, int line)
+{
+    if (!shape_ok(M, N, K) || ws_num < 1) return;
+    // The reference picks its path, and with it the epilogue arithmetic, by M <= 64
+    // (kernels/TernaSpMM.cu:34); the forced entry points pin one of the two.
+    const bool decode_rule = route == ROUTE_DECODE || (route == ROUTE_AUTO && M <= 64);
+    const Epilogue ep{s, ws, nullptr, ws_num, decode_rule ? EP_I8_DECODE : EP_I8_PREFILL};
+    const Weights w{bitmap, tile_off, median_off, sign_words};
+    if (M <= 64) launch_decode<int8_t>(x, w, out, ep, M, N, K, st);
+    else launch_prefill<int8_t>(x, w, out, ep, M, N, K, st);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("bitlinear_TernaSpMM", e, line);
+}
+
+void run_bf16(Route route, const uint16_t* x, const uint64_t* bitmap, const int* tile_off,
+              const uint16_t* median_off, const uint32_t* sign_words, uint16_t* out, const float* scale,
+              int ws_num, int M, int N, int K, hipStream_t st, int line)
+{
+    if (!shape_ok(M, N, K) || ws_num < 1) return;
+    const Epilogue ep{nullptr, nullptr, scale, ws_num, EP_BF16};
+    const Weights w{bitmap, tile_off, median_off, sign_words};
+    const bool small = route == ROUTE_DECODE || (route == ROUTE_AUTO && M <= 64);
+    if (small) launch_decode<uint16_t>(x, w, out, ep, M, N, K, st);
+    else launch_prefill<uint16_t>(x, w, out, ep, M, N, K, st);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("bitlinear_TernaSpMM_bf16", e, line);
+}
+
+__global__ void sleep_kernel(long long ticks)
+{
+    // wall_clock64 counts at a fixed 100 MHz; every lane leaves once the span has passed.
+    const long long start = wall_clock64();
+    while (wall_clock64() - start < ticks) __builtin_amdgcn_s_sleep(8);
+}
+
+}  // namespace
+
+extern "C" {
+
+void checkLastCudaError(int line)
+{
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("checkLastCudaError", e, line);
+}
+
+void bitlinear_TernaSpMM(int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* median_off, uint32_t* sign_words,
+                         terna_bf16* out, terna_bf16* s, terna_bf16* ws, int ws_num, int M, int N, int K,
+                         int /*SPLIT_K*/, int32_t* /*workspace*/, terna_stream stream)
+{
+    run_i8(ROUTE_AUTO, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K,
+           static_cast<hipStream_t>(stream), __LINE__);
+}
+
+void bitlinear_TernaSpMM_decode(int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* median_off,
+                                uint32_t* sign_words, terna_bf16* out, terna_bf16* s, terna_bf16* ws, int ws_num,
+                                int M, int N, int K, int /*SPLIT_K*/, int32_t* /*workspace*/, terna_stream stream)
+{
+    run_i8(ROUTE_DECODE, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K,
+           static_cast<hipStream_t>(stream), __LINE__);
+}
+
+void bitlinear_TernaSpMM_prefill(int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* median_off,
+                                 uint32_t* sign_words, terna_bf16* out, terna_bf16* s, terna_bf16* ws, int ws_num,
+                                 int M, int N, int K, int /*SPLIT_K*/, int32_t* /*workspace*/, terna_stream stream)
+{
+    run_i8(ROUTE_PREFILL, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K,
+           static_cast<hipStream_t>(stream), __LINE__);
+}
+
+void bitlinear_TernaSpMM_benchmark(int mode, int warmup_iters, int bench_iters, int8_t* x, uint64_t* bitmap,
+                                   int* tile_off, uint16_t* median_off, uint32_t* sign_words, terna_bf16* out,
+                                   terna_bf16* s, terna_bf16* ws, int ws_num, int M, int N, int K, int SPLIT_K,
+                                   int32_t* workspace, terna_stream stream)
+{
+    // mode 0 = auto, 1 = prefill, 2 = decode (kernels/TernaSpMM.cu:165-173)
+    const Route route = mode == 1 ? ROUTE_PREFILL : (mode == 2 ? ROUTE_DECODE : ROUTE_AUTO);
+    (void)SPLIT_K;
+    (void)workspace;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    for (int it = 0; it < warmup_iters; ++it)
+        run_i8(route, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K, st, __LINE__);
+    hipError_t e = hipStreamSynchronize(st);
+    if (e != hipSuccess) die("benchmark warm-up", e, __LINE__);
+
+    hipEvent_t start, stop;
+    if ((e = hipEventCreate(&start)) != hipSuccess) die("hipEventCreate", e, __LINE__);
+    if ((e = hipEventCreate(&stop)) != hipSuccess) die("hipEventCreate", e, __LINE__);
+    (void)hipEventRecord(start, st);
+    for (int it = 0; it < bench_iters; ++it)
+        run_i8(route, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K, st, __LINE__);
+    (void)hipEventRecord(stop, st);
+    if ((e = hipEventSynchronize(stop)) != hipSuccess) die("benchmark loop", e, __LINE__);
+    float total_ms = 0.0f;
+    (void)hipEventElapsedTime(&total_ms, start, stop);
+    const float avg_us = bench_iters > 0 ? total_ms * 1000.0f / bench_iters : 0.0f;
+    std::printf("Shape(M=%d, N=%d, K=%d): %.2f us (avg over %d iters, warmup=%d)\n", M, N, K, avg_us, bench_iters,
+                warmup_iters);
+    std::fflush(stdout);
+    (void)hipEventDestroy(start);
+    (void)hipEventDestroy(stop);
+}
+
+void reorder_WT_h(terna_bf16* W, terna_bf16* W_reordered, int N, int K) { reorder_bf16(W, W_reordered, N, K); }
+
+int convert_reorderd(terna_bf16* A_h, int N, int K, int tile_N, int warp_subtile_N, int subtile_N, int tile_K,
+                     int warp_subtile_K, int subtile_K, uint64_t** bitmap, int** tile_off, uint16_t** median_off,
+                     uint32_t** sign_words, int* max_nnz_count)
+{
+    if (tile_N != 64 || warp_subtile_N != 16 || subtile_N != 8 || tile_K != 64 || warp_subtile_K != 64 ||
+        subtile_K != 8)
+        return -1;
+    int64_t n_bitmap, n_off, n_med, cap_words;
+    if (encode_sizes(N, K, &n_bitmap, &n_off, &n_med, &cap_words) != 0) return -1;
+    *sign_words = static_cast<uint32_t*>(std::malloc(static_cast<size_t>(cap_words) * 4 + 4));
+    *tile_off = static_cast<int*>(std::malloc(static_cast<size_t>(n_off) * sizeof(int)));
+    // three trailing entries of slack: the reference's consumer reads that far past the end
+    *median_off = static_cast<uint16_t*>(std::calloc(static_cast<size_t>(n_med) + 4, sizeof(uint16_t)));
+    *bitmap = nullptr;
+    // pinned, as the reference allocates it (kernels/TernaSpMM.cu:317); callers release it with hipHostFree
+    if (hipHostMalloc(reinterpret_cast<void**>(bitmap), static_cast<size_t>(n_bitmap) * 8, hipHostMallocDefault) !=
+        hipSuccess) {
+        (void)hipGetLastError();
+        *bitmap = nullptr;
+    }
+    if (!*sign_words || !*tile_off || !*median_off || !*bitmap) return -1;
+    int max_nnz = 0;
+    const int64_t words = encode_reordered_bf16(A_h, N, K, *bitmap, *tile_off, *median_off, *sign_words, &max_nnz);
+    if (words < 0) return -1;
+    if (max_nnz_count) *max_nnz_count = max_nnz;
+    uint32_t* shrunk = static_cast<uint32_t*>(std::realloc(*sign_words, static_cast<size_t>(words) * 4 + 4));
+    if (shrunk) *sign_words = shrunk;
+    return (N / 64) * (K / 64);
+}
+
+void gpu_sleep(double us, terna_stream stream)
+{
+    const long long ticks = us > 0 ? static_cast<long long>(us * 100.0) : 0;
+    sleep_kernel<<<1, 64, 0, static_cast<hipStream_t>(stream)>>>(ticks);
+}
+
+void bitlinear_TernaSpMM_bf16(const terna_bf16* x, const uint64_t* bitmap, const int* tile_off,
+                              const uint16_t* median_off, const uint32_t* sign_words, terna_bf16* out,
+                              const float* scale, int ws_num, int M, int N, int K, int /*SPLIT_K*/,
+                              void* /*workspace*/, terna_stream stream)
+{
+    run_bf16(ROUTE_AUTO, x, bitmap, tile_off, median_off, sign_words, out, scale, ws_num, M, N, K,
+             static_cast<hipStream_t>(stream), __LINE__);
+}
+
+void bitlinear_TernaSpMM_bf16_decode(const terna_bf16* x, const uint64_t* bitmap, const int* tile_off,
+                                     const uint16_t* median_off, const uint32_t* sign_words, terna_bf16* out,
+                                     const float* scale, int ws_num, int M, int N, int K, int /*SPLIT_K*/,
+                                     void* /*workspace*/, terna_stream stream)
+{
+    run_bf16(ROUTE_DECODE, x, bitmap, tile_off, median_off, sign_words, out, scale, ws_num, M, N, K,
+             static_cast<hipStream_t>(stream), __LINE__);
+}
+
+void bitlinear_TernaSpMM_bf16_prefill(const terna_bf16* x, const uint64_t* bitmap, const int* tile_off,
+                                      const uint16_t* median_off, const uint32_t* sign_words, terna_bf16* out,
+                                      const float* scale, int ws_num, int M, int N, int K, int /*SPLIT_K*/,
+                                      void* /*workspace*/, terna_stream stream)
+{
+    run_bf16(ROUTE_PREFILL, x, bitmap, tile_off, median_off, sign_words, out, scale, ws_num, M, N, K,
+             static_cast<hipStream_t>(stream), __LINE__);
+}
+
+int ternaspmm_encode_sizes(int N, int K, int64_t* bitmap_len, int64_t* tile_off_len, int64_t* median_len,
+                           int64_t* sign_words_capacity)
+{
+    return encode_sizes(N, K, bitmap_len, tile_off_len, median_len, sign_words_capacity);
+}
+
+int64_t ternaspmm_encode_i8(const int8_t* W, int N, int K, uint64_t* bitmap, int* tile_off, uint16_t* median_off,
+                            uint32_t* sign_words)
+{
+    return encode_i8(W, N, K, bitmap, tile_off, median_off, sign_words);
+}
+
+void ternaspmm_decompress_bf16(const uint64_t* bitmap, const int* tile_off, const uint16_t* median_off,
+                               const uint32_t* sign_words, terna_bf16* W_dense, int N, int K, terna_stream stream)
+{
+    if (!shape_ok(1, N, K)) return;
+    terna_decompress_kernel<4><<<dim3(N / 16), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+        bitmap, tile_off, median_off, sign_words, W_dense, N, K);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_decompress_bf16", e, __LINE__);
+}
+
+const char* ternaspmm_version(void) { return "ternaspmm-gfx950 0.1"; }
+
+}  // extern "C"

@@ -1,0 +1,154 @@
+"""Call site of the TernaSpMM path: the host-side mirror of the reference's ``model.py:21-153``.
+
+``TernaInfer_linear`` / ``SpBitLinear`` / ``BF16BitLinear`` / ``get_global_workspace`` keep the
+reference's names, arguments and behaviour (row padding to ``max(8, next_pow2(M))``,
+``SPLIT_K = 7``, raw device pointers and the current stream handed to the C ABI).
+``TernaInfer_linear_bf16`` / ``SpBitLinearBF16`` are the same call site for the
+bf16-activation entry points this build adds.  PyTorch is only the owner of device memory
+and streams here; all arithmetic happens in libternaspmm.so.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+from torch import nn
+from torch.nn import functional as F
+
+from . import _lib
+
+MAX_MATRIX_ELEMENTS = 13824 * 2560          # ModelArgs.max_matrix_elements, model.py:34
+
+_GLOBAL_WORKSPACE = None
+
+
+def get_global_workspace(device="cuda"):
+    """One int8 scratch buffer shared by every layer (model.py:37-42).  This build's kernels
+    never touch it; it is still passed so the ABI stays the reference's."""
+    global _GLOBAL_WORKSPACE
+    if _GLOBAL_WORKSPACE is None:
+        _GLOBAL_WORKSPACE = torch.empty(MAX_MATRIX_ELEMENTS, dtype=torch.int8, device=device)
+    return _GLOBAL_WORKSPACE
+
+
+def _p(t: torch.Tensor):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def TernaInfer_linear(input, compressed_val, TileOffsets_global, TileOffsets_median, bitmap,
+                      workspace, s, ws, ws_num, out_features):
+    """int8 activations x compressed ternary weight -> bf16 (model.py:45-92)."""
+    lib = _lib.load()
+    out_shape = list(input.shape)
+    out_shape[-1] = out_features
+    stream = torch.cuda.current_stream()
+
+    M = input.shape[0]
+    if len(out_shape) == 3:
+        M *= input.shape[1]
+    N = out_features
+    K = input.shape[-1]
+    SPLIT_K = 7
+
+    M_padded = max(8, 1 << (M - 1).bit_length())
+    pad_rows = M_padded - M
+    if pad_rows > 0:
+        input_padded = torch.cat([
+            input.reshape(M, K),
+            torch.empty((pad_rows, K), dtype=input.dtype, device=input.device)], dim=0)
+        # the reference also reads s for the padding rows; give those reads memory to land in
+        s_padded = torch.cat([s.reshape(M), torch.ones(pad_rows, dtype=s.dtype, device=s.device)])
+    else:
+        input_padded = input.reshape(M, K).contiguous()
+        s_padded = s.reshape(M).contiguous()
+
+    ret_padded = torch.empty((M_padded, N), dtype=torch.bfloat16, device=input.device)
+    lib.bitlinear_TernaSpMM(
+        _p(input_padded), _p(bitmap), _p(TileOffsets_global), _p(TileOffsets_median), _p(compressed_val),
+        _p(ret_padded), _p(s_padded), _p(ws), ws_num, M_padded, N, K, SPLIT_K, _p(workspace),
+        ctypes.c_void_p(stream.cuda_stream))
+    return ret_padded[:M, :].reshape(*out_shape)
+
+
+def TernaInfer_linear_bf16(input, compressed_val, TileOffsets_global, TileOffsets_median, bitmap,
+                           scale, ws_num, out_features, route: str = "auto"):
+    """bf16 activations x compressed ternary weight -> bf16, fp32 accumulate, fp32 scale[ws_num].
+    No row padding: the entry point takes the true M."""
+    lib = _lib.load()
+    fn = {"auto": lib.bitlinear_TernaSpMM_bf16, "decode": lib.bitlinear_TernaSpMM_bf16_decode,
+          "prefill": lib.bitlinear_TernaSpMM_bf16_prefill}[route]
+    out_shape = list(input.shape)
+    out_shape[-1] = out_features
+    K = input.shape[-1]
+    x = input.reshape(-1, K).contiguous()
+    M = x.shape[0]
+    assert x.dtype == torch.bfloat16 and scale.dtype == torch.float32
+    out = torch.empty((M, out_features), dtype=torch.bfloat16, device=input.device)
+    stream = torch.cuda.current_stream()
+    fn(_p(x), _p(bitmap), _p(TileOffsets_global), _p(TileOffsets_median), _p(compressed_val), _p(out),
+       _p(scale), ws_num, M, out_features, K, 1, None, ctypes.c_void_p(stream.cuda_stream))
+    return out.reshape(*out_shape)
+
+
+class _CompressedWeight(nn.Module):
+    """Holds the four format tensors + ``weight_scale`` under the reference's checkpoint keys
+    (convert_TernaInfer.py:204-209, model.py:110-116)."""
+
+    def __init__(self, in_features: int, out_features: int, dic: dict, key: str):
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        dev = "cuda"
+        mk = lambda t: torch.nn.Parameter(t.to(dev), requires_grad=False)
+        self.weight_compressed_val = mk(dic[key + ".weight_compressed_val"])
+        self.weight_TileOffsets_global = mk(dic[key + ".weight_TileOffsets_global"])
+        self.weight_TileOffsets_median = mk(dic[key + ".weight_TileOffsets_median"])
+        self.weight_bitmap = mk(dic[key + ".weight_bitmap"])
+        ws = dic[key + ".weight_scale"]
+        self.weight_scale = mk(ws)
+        self.ws_num = len(ws[ws != 0])
+
+
+class SpBitLinear(_CompressedWeight):
+    """Ternary linear on int8-quantised activations (model.py:96-133)."""
+
+    def quant_input(self, input):
+        s = 127 / input.abs().max(dim=-1, keepdim=True).values.clamp_(min=1e-5)
+        return (input * s).round().clamp(-128, 127).to(torch.int8), s
+
+    def forward(self, input):
+        input, s = self.quant_input(input)
+        return TernaInfer_linear(
+            input, self.weight_compressed_val, self.weight_TileOffsets_global, self.weight_TileOffsets_median,
+            self.weight_bitmap, get_global_workspace(), s, self.weight_scale, self.ws_num, self.out_features)
+
+
+class SpBitLinearBF16(_CompressedWeight):
+    """Ternary linear on bf16 activations (no activation quantisation)."""
+
+    def __init__(self, in_features: int, out_features: int, dic: dict, key: str):
+        super().__init__(in_features, out_features, dic, key)
+        self.scale_f32 = torch.nn.Parameter(self.weight_scale.float(), requires_grad=False)
+
+    def forward(self, input):
+        return TernaInfer_linear_bf16(
+            input, self.weight_compressed_val, self.weight_TileOffsets_global, self.weight_TileOffsets_median,
+            self.weight_bitmap, self.scale_f32, self.ws_num, self.out_features)
+
+
+class BF16BitLinear(nn.Module):
+    """Dense reference semantics (model.py:135-153): quantise activations, bf16 GEMM, divide by s."""
+
+    def __init__(self, in_features: int, out_features: int, dic: dict, key: str):
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.weight = torch.nn.Parameter(dic[key + ".weight"].cuda(), requires_grad=False)
+
+    def quant_input(self, input):
+        s = 127 / input.abs().max(dim=-1, keepdim=True).values.clamp_(min=1e-5)
+        return (input * s).round().clamp(-128, 127).to(torch.int8), s
+
+    def forward(self, input):
+        input, s = self.quant_input(input)
+        return F.linear(input.to(torch.bfloat16), self.weight) / s

@@ -1,0 +1,59 @@
+"""The C-ABI library loads without a GPU and exports every symbol include/ternaspmm.h declares."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "ternaspmm.h")
+
+REFERENCE_SYMBOLS = ["checkLastCudaError", "bitlinear_TernaSpMM", "bitlinear_TernaSpMM_decode",
+                     "bitlinear_TernaSpMM_prefill", "bitlinear_TernaSpMM_benchmark", "reorder_WT_h",
+                     "convert_reorderd", "gpu_sleep"]
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(r"^\s*(?:const\s+)?[A-Za-z_][\w\s\*]*?\b([A-Za-z_]\w*)\s*\(", text, flags=re.M)
+
+
+def test_header_declares_the_reference_symbols():
+    names = declared_symbols()
+    for sym in REFERENCE_SYMBOLS:
+        assert sym in names, sym
+
+
+def test_library_exports_every_declared_symbol():
+    from ternainfer_amd import _lib
+    lib = _lib.load()
+    names = declared_symbols()
+    assert len(names) >= 15
+    for sym in names:
+        assert hasattr(lib, sym), f"{sym} declared in include/ternaspmm.h but not exported"
+        assert sym in _lib.PROTOTYPES, f"{sym} has no ctypes prototype"
+    assert set(_lib.PROTOTYPES) == set(names)
+
+
+def test_version_string():
+    from ternainfer_amd import _lib
+    assert _lib.load().ternaspmm_version().startswith(b"ternaspmm-gfx950")
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    from ternainfer_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libternaspmm.so")
+    with pytest.raises(ImportError):
+        _lib.load()
+
+
+def test_encode_sizes_rejects_bad_shapes():
+    from ternainfer_amd import _lib
+    lib = _lib.load()
+    out = (ctypes.c_int64 * 4)()
+    ptrs = [ctypes.byref(out, 8 * j) for j in range(4)]
+    assert lib.ternaspmm_encode_sizes(64, 100, *ptrs) == -1
+    assert lib.ternaspmm_encode_sizes(128, 192, *ptrs) == 0
+    assert list(out) == [128 * 192 // 64, 128 * 192 // 4096 + 1, 3 * 128 * 192 // 4096, 128 * 192 // 32]

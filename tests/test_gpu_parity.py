@@ -1,0 +1,278 @@
+"""Parity of the HIP path against the CPU oracle, through the C ABI, on a real MI355X.
+
+  int8 family : bit-exact (integer accumulate + the reference's fp32 epilogue arithmetic)
+  bf16 family : max|err| <= 1e-2 * max|ref| and median error <= 1 bf16 ULP against the fp64 golden
+  format      : device decompression of the compressed format is bit-exact
+"""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import terna_oracle as O
+from tests._util import (DeviceFormat, check_against_fp64, make_bf16_activations, make_int8_activations,
+                         make_row_skewed, make_ternary, seed_for, vp)
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from ternainfer_amd import _lib
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return _lib.load()
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def run_i8(lib, fmt, xq, s_bits, ws_bits, ws_num, entry="bitlinear_TernaSpMM"):
+    m, k = xq.shape
+    x = torch.from_numpy(xq).cuda()
+    s = torch.from_numpy(s_bits.view(np.int16)).cuda()
+    ws = torch.from_numpy(ws_bits.view(np.int16)).cuda()
+    out = torch.full((m, fmt.n), -1, dtype=torch.int16, device="cuda")      # poison: must be overwritten
+    work = torch.empty(16, dtype=torch.int32, device="cuda")
+    print(f"[case] {entry} M={m} N={fmt.n} K={k} ws_num={ws_num}", flush=True)
+    getattr(lib, entry)(vp(x), vp(fmt.bm), vp(fmt.off), vp(fmt.med), vp(fmt.vals), vp(out), vp(s), vp(ws),
+                        ws_num, m, fmt.n, k, 7, vp(work), _stream())
+    torch.cuda.synchronize()
+    return out.cpu().numpy().view(np.uint16)
+
+
+def run_bf16(lib, fmt, x_bits, scale, ws_num, entry="bitlinear_TernaSpMM_bf16"):
+    m, k = x_bits.shape
+    x = torch.from_numpy(x_bits.view(np.int16)).cuda()
+    sc = torch.from_numpy(scale).cuda()
+    out = torch.full((m, fmt.n), -1, dtype=torch.int16, device="cuda")
+    print(f"[case] {entry} M={m} N={fmt.n} K={k} ws_num={ws_num}", flush=True)
+    getattr(lib, entry)(vp(x), vp(fmt.bm), vp(fmt.off), vp(fmt.med), vp(fmt.vals), vp(out), vp(sc), ws_num,
+                        m, fmt.n, k, 1, None, _stream())
+    torch.cuda.synchronize()
+    return out.cpu().numpy().view(np.uint16)
+
+
+WS = O.f32_to_bf16_bits(np.array([0.8125, 1.59375, 2.71875, 0.3359375], np.float32))
+
+
+# ------------------------------------------------------------------------------- format
+@pytest.mark.parametrize("kind", ["iid40", "iid45", "skewed", "dense", "empty", "sparse97"])
+def test_device_decompress_is_bit_exact(lib, kind):
+    n, k = 256, 320
+    w = {"iid40": lambda: make_ternary(n, k, 0.40, 1), "iid45": lambda: make_ternary(n, k, 0.45, 2),
+         "skewed": lambda: make_row_skewed(n, k, 3), "dense": lambda: make_ternary(n, k, 0.0, 4),
+         "empty": lambda: np.zeros((n, k), np.int8), "sparse97": lambda: make_ternary(n, k, 0.97, 5)}[kind]()
+    fmt = DeviceFormat(w)
+    dense = torch.full((n, k), 0x7FC0, dtype=torch.int16, device="cuda")
+    print(f"[case] decompress {kind} N={n} K={k}", flush=True)
+    lib.ternaspmm_decompress_bf16(vp(fmt.bm), vp(fmt.off), vp(fmt.med), vp(fmt.vals), vp(dense), n, k, _stream())
+    torch.cuda.synchronize()
+    got = O.bf16_bits_to_f32(dense.cpu().numpy().view(np.uint16))
+    assert (got == w.astype(np.float32)).all()
+
+
+def test_device_decompress_full_size_round_trip(lib):
+    """BitNet-2B gate+up shape: decompress(encode(W)) == W on the device."""
+    n, k = 13824, 2560
+    w = make_ternary(n, k, 0.40, seed_for(2, 3))
+    fmt = DeviceFormat(w)
+    dense = torch.empty((n, k), dtype=torch.bfloat16, device="cuda")
+    lib.ternaspmm_decompress_bf16(vp(fmt.bm), vp(fmt.off), vp(fmt.med), vp(fmt.vals), vp(dense), n, k, _stream())
+    torch.cuda.synchronize()
+    assert torch.equal(dense.cpu(), torch.from_numpy(w).to(torch.bfloat16))
+
+
+# ------------------------------------------------------------------------------- int8 family
+@pytest.mark.parametrize("m", [1, 8, 16, 24, 32, 64])
+@pytest.mark.parametrize("n,k,ws_num", [(128, 192, 1), (256, 320, 2), (256, 64, 4)])
+def test_int8_small_m_bit_exact(lib, coracle, m, n, k, ws_num):
+    w = make_ternary(n, k, 0.40, 10 + m + n)
+    fmt = DeviceFormat(w)
+    xq, s = make_int8_activations(m, k, 20 + m + k)
+    got = run_i8(lib, fmt, xq, s, WS, ws_num)
+    want = coracle.spmm_i8(xq, w, s, WS, ws_num, 0)
+    assert (got == want).all()
+
+
+@pytest.mark.parametrize("entry,mode,m", [("bitlinear_TernaSpMM_decode", 0, 8), ("bitlinear_TernaSpMM_decode", 0, 128),
+                                          ("bitlinear_TernaSpMM_prefill", 1, 8), ("bitlinear_TernaSpMM_prefill", 1, 128),
+                                          ("bitlinear_TernaSpMM", 1, 128), ("bitlinear_TernaSpMM", 1, 200)])
+def test_int8_forced_paths_follow_their_epilogue(lib, coracle, entry, mode, m):
+    n, k = 384, 256
+    w = make_ternary(n, k, 0.40, 31)
+    fmt = DeviceFormat(w)
+    xq, s = make_int8_activations(m, k, 32 + m)
+    s = s.copy()
+    if mode == 1:
+        s[m // 2] = 0                     # prefill rule: coefficient 0 where s == 0
+    got = run_i8(lib, fmt, xq, s, WS, 3, entry)
+    want = coracle.spmm_i8(xq, w, s, WS, 3, mode)
+    if mode == 0:
+        assert (got == want).all()
+    else:
+        row = m // 2
+        keep = np.arange(m) != row
+        assert (got[keep] == want[keep]).all()
+        assert not (got[row] & 0x7FFF).any() and (got[row] == want[row]).all()
+
+
+def test_int8_qkv_groups_bit_exact(lib, coracle):
+    """N = 3840 with three scales: the 2560 / 640 / 640 split of the fused QKV matrix."""
+    n, k, m = 3840, 256, 8
+    w = make_ternary(n, k, 0.40, 41)
+    fmt = DeviceFormat(w)
+    xq, s = make_int8_activations(m, k, 42)
+    got = run_i8(lib, fmt, xq, s, WS, 3)
+    assert (got == coracle.spmm_i8(xq, w, s, WS, 3, 0)).all()
+
+
+def test_int8_reference_test_construction(lib):
+    """tests/test_kernel.cu 8 2560 2560 45 7: x == 1, unit scales, ws_num = 4 -> exact row sums of W."""
+    n = k = 2560
+    m = 8
+    w = make_ternary(n, k, 0.45, seed_for(1, 0))
+    fmt = DeviceFormat(w)
+    x = np.ones((m, k), np.int8)
+    one = O.f32_to_bf16_bits(np.ones(4, np.float32))
+    got = run_i8(lib, fmt, x, one[:1].repeat(m), one, 4)
+    want = O.f32_to_bf16_bits(np.tile(w.sum(axis=1, dtype=np.int64).astype(np.float32), (m, 1)))
+    assert (got == want).all()
+
+
+@pytest.mark.parametrize("n,k", [(3840, 2560), (2560, 2560), (13824, 2560), (2560, 6912)])
+@pytest.mark.parametrize("m", [1, 8, 16])
+def test_int8_2b_layer_shapes_bit_exact(lib, m, n, k):
+    w = make_ternary(n, k, 0.40, seed_for(2, n % 7))
+    fmt = DeviceFormat(w)
+    xq, s = make_int8_activations(m, k, seed_for(2, 10 + m))
+    ws_num = 3 if n == 3840 else (2 if n == 13824 else 1)
+    mp = max(8, 1 << (m - 1).bit_length())          # the call site pads rows (model.py:64)
+    xq_p = np.concatenate([xq, np.zeros((mp - m, k), np.int8)])
+    s_p = np.concatenate([s, O.f32_to_bf16_bits(np.ones(mp - m, np.float32))])
+    got = run_i8(lib, fmt, xq_p, s_p, WS, ws_num)[:m]
+    want = O.spmm_i8(xq, w, s, WS, ws_num, 0)
+    assert (got == want).all()
+
+
+# ------------------------------------------------------------------------------- bf16 family
+def _check_bf16(got, ref):
+    max_err, max_ref, med_ulp, max_ulp = check_against_fp64(got, ref)
+    assert max_err <= 1e-2 * max_ref, (max_err, max_ref)
+    assert med_ulp <= 1, med_ulp
+    return max_err / max_ref, med_ulp, max_ulp
+
+
+@pytest.mark.parametrize("m", [1, 3, 8, 16, 17, 40, 64])
+def test_bf16_small_m(lib, coracle, m):
+    n, k = 256, 320
+    w = make_ternary(n, k, 0.40, 50 + m)
+    fmt = DeviceFormat(w)
+    x = make_bf16_activations(m, k, 60 + m)
+    scale = np.array([0.7, 1.9], np.float32)
+    got = run_bf16(lib, fmt, x, scale, 2)
+    _check_bf16(got, coracle.spmm_bf16(x, w, scale, 2))
+
+
+def test_bf16_golden_fixture(lib):
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "linear_8x128x192.npz"))
+    f = np.load(os.path.join(os.path.dirname(__file__), "golden", "format_128x192.npz"))
+    fmt = DeviceFormat(f["w"])
+    _check_bf16(run_bf16(lib, fmt, g["x_bf16"], g["scale"], 1), g["ref_fp64"])
+    ws_num = int(g["ws_num"])
+    assert (run_i8(lib, fmt, g["x_q"], g["s"], g["ws"], ws_num, "bitlinear_TernaSpMM_decode") == g["out_i8_decode"]).all()
+    assert (run_i8(lib, fmt, g["x_q"], g["s"], g["ws"], ws_num, "bitlinear_TernaSpMM_prefill") == g["out_i8_prefill"]).all()
+
+
+def test_bf16_config1(lib):
+    """M=8, K=N=2560, P(0)=0.45, one fp32 scale ~ U[0.5, 2]."""
+    n = k = 2560
+    m = 8
+    w = make_ternary(n, k, 0.45, seed_for(1, 0))
+    fmt = DeviceFormat(w)
+    x = make_bf16_activations(m, k, seed_for(1, 1))
+    scale = np.random.default_rng(seed_for(1, 2)).uniform(0.5, 2.0, 1).astype(np.float32)
+    got = run_bf16(lib, fmt, x, scale, 1)
+    _check_bf16(got, O.spmm_bf16_golden(x, w, scale, 1))
+
+
+@pytest.mark.parametrize("n,k", [(3840, 2560), (2560, 2560), (13824, 2560), (2560, 6912)])
+@pytest.mark.parametrize("m", [1, 8, 16])
+def test_bf16_2b_layer_shapes(lib, m, n, k):
+    w = make_ternary(n, k, 0.40, seed_for(2, n % 7))
+    fmt = DeviceFormat(w)
+    x = make_bf16_activations(m, k, seed_for(2, 20 + m))
+    scale = np.array([1.37], np.float32)
+    got = run_bf16(lib, fmt, x, scale, 1)
+    _check_bf16(got, O.spmm_bf16_golden(x, w, scale, 1))
+
+
+@pytest.mark.parametrize("n,k", [(2560, 2560), (2560, 6912)])
+@pytest.mark.parametrize("kind", ["p20", "p33", "p45", "p60", "skewed"])
+def test_bf16_sparsity_sweep_m16(lib, n, k, kind):
+    seed = seed_for(4, len(kind) + k % 5)
+    w = make_row_skewed(n, k, seed) if kind == "skewed" else make_ternary(n, k, int(kind[1:]) / 100.0, seed)
+    fmt = DeviceFormat(w)
+    x = make_bf16_activations(16, k, seed + 1)
+    scale = np.array([0.93], np.float32)
+    got = run_bf16(lib, fmt, x, scale, 1)
+    _check_bf16(got, O.spmm_bf16_golden(x, w, scale, 1))
+
+
+def test_bf16_linearity_and_zero_weights(lib):
+    """Properties that hold at any size: W == 0 -> output exactly 0; doubling the scale doubles
+    every output exactly (power of two); negating x negates the output bit for bit."""
+    n, k, m = 2560, 2560, 8
+    fmt0 = DeviceFormat(np.zeros((n, k), np.int8))
+    x = make_bf16_activations(m, k, 71)
+    assert not run_bf16(lib, fmt0, x, np.array([1.0], np.float32), 1).any()
+    fmt = DeviceFormat(make_ternary(n, k, 0.4, 72))
+    a = run_bf16(lib, fmt, x, np.array([0.75], np.float32), 1)
+    b = run_bf16(lib, fmt, x, np.array([1.5], np.float32), 1)
+    assert (O.bf16_bits_to_f32(b) == 2 * O.bf16_bits_to_f32(a)).all()
+    c = run_bf16(lib, fmt, x ^ np.uint16(0x8000), np.array([0.75], np.float32), 1)
+    assert ((c ^ np.uint16(0x8000)) == a).all()
+
+
+def test_call_site_mirror_pads_and_slices(lib, coracle):
+    """TernaInfer_linear (the model.py:45-92 mirror): M=3 is padded to 8 rows and sliced back."""
+    import ternainfer_amd as T
+    n, k, m = 256, 192, 3
+    w = make_ternary(n, k, 0.4, 81)
+    fmt = DeviceFormat(w)
+    xq, s = make_int8_activations(m, k, 82)
+    out = T.TernaInfer_linear(torch.from_numpy(xq).cuda(), fmt.vals, fmt.off, fmt.med, fmt.bm,
+                              T.get_global_workspace(), torch.from_numpy(s.view(np.int16)).cuda().view(torch.bfloat16),
+                              torch.from_numpy(WS.view(np.int16)).cuda().view(torch.bfloat16), 2, n)
+    torch.cuda.synchronize()
+    assert out.shape == (m, n) and out.dtype == torch.bfloat16
+    got = out.view(torch.int16).cpu().numpy().view(np.uint16)
+    assert (got == coracle.spmm_i8(xq, w, s, WS, 2, 0)).all()
+
+
+def test_graph_capture_replays(lib):
+    """The entry point only enqueues: capture it in a HIP graph, replay with eager work between."""
+    n, k, m = 2560, 2560, 8
+    w = make_ternary(n, k, 0.4, 91)
+    fmt = DeviceFormat(w)
+    x_bits = make_bf16_activations(m, k, 92)
+    scale = np.array([1.1], np.float32)
+    eager = run_bf16(lib, fmt, x_bits, scale, 1)
+    x = torch.from_numpy(x_bits.view(np.int16)).cuda()
+    sc = torch.from_numpy(scale).cuda()
+    out = torch.zeros((m, n), dtype=torch.int16, device="cuda")
+    st = torch.cuda.Stream()
+    st.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(st):
+        with torch.cuda.graph(g, stream=st):
+            lib.bitlinear_TernaSpMM_bf16(vp(x), vp(fmt.bm), vp(fmt.off), vp(fmt.med), vp(fmt.vals), vp(out), vp(sc),
+                                         1, m, n, k, 1, None, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    for _ in range(3):
+        out.fill_(0)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert (out.cpu().numpy().view(np.uint16) == eager).all()

@@ -1,0 +1,103 @@
+"""Pins the oracle's linear-layer arithmetic (no GPU).
+
+  int8 family - the integer matmul is exact; with x == 1 and unit scales the output is the row
+                sums of W, the construction the reference's own tests/test_kernel.cu:79-92 uses
+                (glibc rand() without srand, reproduced here through libc);
+                epilogue: C (volatile float, one operation at a time) == numpy float32, and the
+                two rounding orders are shown to differ on some element (so a swapped formula fails)
+  bf16 family - C fp64 loop == numpy fp64 matmul; linear in the scale; sign flip of W flips the output
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+from oracle import terna_oracle as O
+from tests._util import make_bf16_activations, make_int8_activations, make_ternary
+
+
+def glibc_rand_ternary(n, k, sparsity_pct):
+    """W as tests/test_kernel.cu:83-91 builds it: r = rand()%100; nonzero iff r >= sparsity,
+    then sign = (rand()%2)*2-1, row-major, from glibc's default seed."""
+    libc = ctypes.CDLL("libc.so.6")
+    libc.srand(1)                      # the state a program has when it never calls srand
+    w = np.zeros((n, k), dtype=np.int8)
+    for i in range(n):
+        for j in range(k):
+            if libc.rand() % 100 >= sparsity_pct:
+                w[i, j] = (libc.rand() % 2) * 2 - 1
+    return w
+
+
+def test_x_equal_one_gives_row_sums(coracle):
+    n, k, m = 64, 128, 8
+    w = glibc_rand_ternary(n, k, 45)
+    x = np.ones((m, k), dtype=np.int8)
+    one = O.f32_to_bf16_bits(np.ones(4, np.float32))
+    out = coracle.spmm_i8(x, w, one[:1].repeat(m), one, 4, 0)
+    want = O.f32_to_bf16_bits(np.tile(w.sum(axis=1, dtype=np.int64).astype(np.float32), (m, 1)))
+    assert (out == want).all()
+    assert (O.spmm_i8(x, w, one[:1].repeat(m), one, 4, 0) == want).all()
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("n,ws_num", [(128, 1), (128, 2), (256, 4), (3840, 3), (3840, 1)])
+def test_int8_epilogue_c_equals_numpy(coracle, mode, n, ws_num):
+    k, m = 192, 5
+    w = make_ternary(n, k, 0.4, 100 + n + ws_num)
+    xq, s = make_int8_activations(m, k, 200 + n)
+    ws = O.f32_to_bf16_bits(np.array([0.8125, 1.59375, 2.71875, 0.3359375], np.float32))
+    a = coracle.spmm_i8(xq, w, s, ws, ws_num, mode)
+    b = O.spmm_i8(xq, w, s, ws, ws_num, mode)
+    assert (a == b).all()
+
+
+def test_the_two_epilogue_orders_differ_somewhere(coracle):
+    n, k, m = 256, 192, 16
+    w = make_ternary(n, k, 0.4, 7)
+    xq, s = make_int8_activations(m, k, 8)
+    ws = O.f32_to_bf16_bits(np.array([1.59375], np.float32))
+    a = coracle.spmm_i8(xq, w, s, ws, 1, 0)
+    b = coracle.spmm_i8(xq, w, s, ws, 1, 1)
+    assert (a != b).any()
+
+
+def test_prefill_epilogue_zero_scale_gives_zero(coracle):
+    n, k, m = 128, 64, 2
+    w = make_ternary(n, k, 0.4, 9)
+    xq, s = make_int8_activations(m, k, 10)
+    s = s.copy()
+    s[1] = 0
+    ws = O.f32_to_bf16_bits(np.array([1.5], np.float32))
+    out = coracle.spmm_i8(xq, w, s, ws, 1, 1)
+    # float(acc) * 0 keeps acc's sign: the row is all +0.0 / -0.0
+    assert not (out[1] & 0x7FFF).any() and out[0].any()
+
+
+def test_prefill_group_is_per_128_column_tile():
+    # N = 192, ws_num = 3: groups of 64 columns on the decode path; the prefill path looks only
+    # at the first column of each 128-wide tile
+    cols = np.arange(192)
+    assert O.ws_group_decode(cols, 192, 3).tolist() == [0] * 64 + [1] * 64 + [2] * 64
+    assert O.ws_group_prefill(cols, 192, 3).tolist() == [0] * 128 + [2] * 64
+    assert O.ws_group_prefill(np.arange(3840), 3840, 1).max() == 0
+
+
+def test_bf16_golden_c_equals_numpy_and_is_linear(coracle):
+    n, k, m = 128, 256, 4
+    w = make_ternary(n, k, 0.4, 11)
+    x = make_bf16_activations(m, k, 12, outlier_frac=0.01)
+    sc = np.array([0.7, 1.9], np.float32)
+    a = coracle.spmm_bf16(x, w, sc, 2)
+    b = O.spmm_bf16_golden(x, w, sc, 2)
+    assert np.allclose(a, b, rtol=1e-12, atol=1e-9)
+    assert np.allclose(coracle.spmm_bf16(x, -w, sc, 2), -a, rtol=0, atol=0)
+    assert np.allclose(coracle.spmm_bf16(x, w, 2 * sc, 2), 2 * a, rtol=1e-15)
+
+
+def test_quant_input_c_equals_numpy(coracle):
+    x = make_bf16_activations(6, 320, 13, outlier_frac=0.02)
+    q1, s1 = coracle.quant_input(x)
+    q2, s2 = O.quant_input(x)
+    assert (q1 == q2).all() and (s1 == s2).all()
+    assert np.abs(q1).max() <= 127 and (np.abs(q1).max(axis=1) >= 126).all()
