@@ -1,0 +1,250 @@
+#!/usr/bin/env python3
+"""Benchmark of the TernaSpMM path on one MI355X.
+
+A step is one decode pass over the BitNet-b1.58-2B ternary layer set -- QKV 2560->3840,
+O 2560->2560, gate+up 2560->13824, down 6912->2560 -- for `--layers` layers (default 30, the
+model's depth) at M = `--m` activation rows (default 8), bf16 activations, fp32 accumulate, one
+fp32 scale per matrix.  Every layer has its own copy of the compressed weights, so one step
+streams ~417 MB of distinct weight bytes: more than the 256 MB last-level cache, i.e. the
+weights come from HBM on every step ("cold stream").  The step is captured once in a HIP graph
+(as the reference's generate.py does for its forward) and replayed.
+
+Prints ONE JSON line.  `value` is algorithmic GB/s: bytes of the reference-format tensors
+(bitmaps, sign words, both offset arrays), activations in, scales, bf16 out -- never the
+dense matrix -- divided by the measured time.  `roofline` prices the same bytes against the
+8 TB/s HBM peak; `cpu_baseline` times decode-to-dense + torch.matmul on the host cores for one
+layer of the same workload and doubles as the correctness gate of the run.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+BF16_MFMA_PEAK_TFLOPS = 2500.0
+LAYER_SET = [("wqkv", 3840, 2560), ("wo", 2560, 2560), ("w13", 13824, 2560), ("w2", 2560, 6912)]   # (name, N, K)
+
+# HBM bytes per launch of the small-M kernel on this workload, from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs scaled by a copy kernel of known size; None until measured.
+TRAFFIC_BYTES_PER_LAUNCH = None
+
+
+def vp(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def make_ternary(n, k, p0, seed):
+    """iid ternary from 16-bit draws: zero iff draw < p0 * 65536 (P(0) = 0.40 to 1e-5), sign = bit 0,
+    which is balanced and independent of the zero test."""
+    rng = np.random.default_rng(seed)
+    b = rng.integers(0, 65536, size=(n, k), dtype=np.uint16)
+    nz = (b >= np.uint16(int(p0 * 65536))).astype(np.int8)
+    return nz * (1 - 2 * (b & 1).astype(np.int8))
+
+
+def f32_to_bf16_bits(x):
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+class Matrix:
+    """One ternary matrix: host copy, `copies` device copies of the format, activations, output."""
+
+    def __init__(self, name, n, k, m, copies, seed, torch, T):
+        self.name, self.n, self.k, self.m = name, n, k, m
+        self.w = make_ternary(n, k, 0.40, seed)
+        vals, off, med, bm = T.compress_weight(torch.from_numpy(self.w))
+        self.host_format = (vals.numpy(), off.numpy(), med.numpy(), bm.numpy())
+        self.n_sign_words = int(vals.numel())
+        base = [t.cuda() for t in (vals, off, med, bm)]
+        self.dev = [base] + [[t.clone() for t in base] for _ in range(copies - 1)]
+        rng = np.random.default_rng(seed + 1)
+        self.x_bits = f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
+        self.x = torch.from_numpy(self.x_bits.view(np.int16)).cuda()
+        self.scale_host = rng.uniform(0.5, 2.0, 1).astype(np.float32)
+        self.scale = torch.from_numpy(self.scale_host).cuda()
+        self.out = torch.zeros((m, n), dtype=torch.int16, device="cuda")
+        # reference-format bytes one call has to move
+        self.alg_bytes = (8 * (n * k // 64) + 4 * self.n_sign_words + 4 * (n * k // 4096 + 1)
+                          + 2 * (3 * n * k // 4096) + 2 * m * k + 4 + 2 * m * n)
+
+    def launch(self, lib, copy, stream):
+        vals, off, med, bm = self.dev[copy]
+        lib.bitlinear_TernaSpMM_bf16(vp(self.x), vp(bm), vp(off), vp(med), vp(vals), vp(self.out), vp(self.scale),
+                                     1, self.m, self.n, self.k, 1, None, stream)
+
+
+def time_graph(torch, graph, replays, warmup):
+    for _ in range(warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(replays):
+        graph.replay()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / replays       # ms per replay
+
+
+def capture(torch, fn):
+    """Capture fn(stream_handle) into a graph on a side stream (events are recorded on the
+    stream the replays are issued to, the current one)."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            fn(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.current_stream().wait_stream(side)
+    return g
+
+
+def cpu_baseline(mats, torch):
+    """Decode the compressed format to dense on the host (C oracle, one thread), then
+    torch.matmul(X.float(), W.T) * scale on all host cores; one layer set, median of 5.
+    Also the correctness gate: the GPU outputs of layer copy 0 must match this golden."""
+    from oracle import terna_oracle as O
+    orc = O.COracle()
+    # the GPU box grants a share of its host cores and exports it as OMP_NUM_THREADS
+    cores = int(os.environ.get("OMP_NUM_THREADS", 0)) or min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    t_decode, t_matmul, alg = [], [], 0
+    parity = {}
+    for mat in mats:
+        alg += mat.alg_bytes
+    for rep in range(5):
+        td = tm = 0.0
+        for mat in mats:
+            t0 = time.perf_counter()
+            w = orc.decode(*mat.host_format, mat.n, mat.k)
+            t1 = time.perf_counter()
+            xf = torch.from_numpy(O.bf16_bits_to_f32(mat.x_bits))
+            wf = torch.from_numpy(w).float()
+            ref = torch.matmul(xf, wf.t()) * float(mat.scale_host[0])
+            t2 = time.perf_counter()
+            td += t1 - t0
+            tm += t2 - t1
+            if rep == 0:
+                assert (w == mat.w).all(), f"{mat.name}: decode(encode(W)) != W"
+                golden = O.spmm_bf16_golden(mat.x_bits, w, mat.scale_host, 1)
+                got = O.bf16_bits_to_f32(mat.out.cpu().numpy().view(np.uint16)).astype(np.float64)
+                max_ref = np.abs(golden).max()
+                max_err = np.abs(got - golden).max()
+                assert max_err <= 1e-2 * max_ref, f"{mat.name}: max_err {max_err} vs max_ref {max_ref}"
+                assert np.abs(ref.double().numpy() - golden).max() <= 1e-3 * max_ref
+                parity[mat.name] = float(max_err / max_ref)
+        t_decode.append(td)
+        t_matmul.append(tm)
+    total = float(np.median(np.array(t_decode) + np.array(t_matmul)))
+    return {
+        "value": alg / total / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+        "sample": (f"one layer set (4 matrices, M={mats[0].m}), median of 5: C-oracle decode to dense on 1 thread "
+                   f"({float(np.median(t_decode)) * 1e3:.1f} ms) + torch.matmul fp32 on {cores} threads "
+                   f"({float(np.median(t_matmul)) * 1e3:.1f} ms)"),
+        "decode_ms": float(np.median(t_decode)) * 1e3, "matmul_ms": float(np.median(t_matmul)) * 1e3,
+        "parity_max_err_over_max_ref": parity,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--m", type=int, default=8, help="activation rows per call (decode batch)")
+    ap.add_argument("--layers", type=int, default=30, help="distinct weight copies per matrix")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-per-shape", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import ternainfer_amd as T
+    assert torch.cuda.is_available(), "bench.py needs the MI355X"
+    lib = T._lib.load()
+    torch.cuda.set_device(0)
+
+    mats = [Matrix(name, n, k, args.m, args.layers, 20260200 + 10 * j, torch, T)
+            for j, (name, n, k) in enumerate(LAYER_SET)]
+    step_bytes = args.layers * sum(mt.alg_bytes for mt in mats)
+    launches_per_step = args.layers * len(mats)
+
+    def step(stream):
+        for layer in range(args.layers):
+            for mt in mats:
+                mt.launch(lib, layer, stream)
+
+    # eager pass first (loads code objects, fills outputs for the correctness gate)
+    step(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    graph = capture(torch, step)
+
+    # ---- the timed region: W warm-up replays, then exactly K steps between two synchronised events
+    for _ in range(args.warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(args.steps):
+        graph.replay()
+    ev1.record()
+    torch.cuda.synchronize()
+    ms_per_step = ev0.elapsed_time(ev1) / args.steps
+    gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
+    launch_us = ms_per_step * 1e3 / launches_per_step
+
+    result = {
+        "metric": "TernaSpMM GB/s + %HBM roofline (M=8,K=N=2560); 2B-shape decode tok/s",
+        "value": gbps, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": (f"configs[1]: BitNet-b1.58-2B decode layer set (QKV 2560->3840, O 2560->2560, "
+                                f"gate+up 2560->13824, down 6912->2560), M={args.m}, P(0)=0.40, bf16 activations, "
+                                f"{args.layers} layers with distinct weight copies (cold stream), HIP-graph replay"),
+                   "m": args.m, "layers": args.layers, "launches_per_step": launches_per_step,
+                   "algorithmic_bytes_per_step": step_bytes},
+        "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": gbps / HBM_PEAK_GBPS, "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+                     "kernel": "terna_decode_kernel<bf16, 8 waves, 1 m-block>",
+                     "algorithmic_bytes_per_launch": step_bytes / launches_per_step,
+                     "avg_launch_us": launch_us},
+        "tokens_per_s_linear_layers_only": args.m / (ms_per_step * 1e-3) if args.layers == 30 else None,
+    }
+
+    # ---- per-shape detail: cold (rotating copies) and hot (one copy, cache resident)
+    if not args.no_per_shape:
+        shapes = {}
+        for mt in mats:
+            cold = capture(torch, lambda s, mt=mt: [mt.launch(lib, c, s) for c in range(args.layers)])
+            hot = capture(torch, lambda s, mt=mt: [mt.launch(lib, 0, s) for _ in range(args.layers)])
+            cold_us = time_graph(torch, cold, 20, 3) * 1e3 / args.layers
+            hot_us = time_graph(torch, hot, 20, 3) * 1e3 / args.layers
+            shapes[f"{mt.name}_{mt.k}x{mt.n}"] = {
+                "alg_bytes": mt.alg_bytes, "cold_us": cold_us, "cold_GBps": mt.alg_bytes / cold_us / 1e3,
+                "cold_frac": mt.alg_bytes / cold_us / 1e3 / HBM_PEAK_GBPS,
+                "hot_us": hot_us, "hot_GBps": mt.alg_bytes / hot_us / 1e3,
+                "tflops": 2.0 * mt.m * mt.n * mt.k / cold_us / 1e6}
+        result["per_shape"] = shapes
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(mats, torch)
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
