@@ -24,6 +24,11 @@
 
 #include "terna_common.h"
 
+// Phase timestamps for tuning builds; expands to nothing in the shipped library.
+#ifndef TERNA_TS
+#define TERNA_TS(slot)
+#endif
+
 namespace terna {
 
 template <typename Act> struct ActTraits;
@@ -31,9 +36,9 @@ template <typename Act> struct ActTraits;
 template <> struct ActTraits<uint16_t> {        // bf16 activations, fp32 accumulate
     using Acc = f32x4;
     using AccScalar = float;
-    using Lut = uint2;
+    using Lut = u32x2;
     static constexpr int kXVecs = 2;             // 2 x 16 B = 16 bf16 per (row, 16-col group)
-    __device__ static Lut make_lut(int e) { return make_lut_bf16(e); }
+    __device__ static Lut make_lut(int e) { const uint2 v = make_lut_bf16(e); return u32x2{v.x, v.y}; }
 };
 
 template <> struct ActTraits<int8_t> {          // int8 activations, int32 accumulate
@@ -101,16 +106,64 @@ __device__ __forceinline__ void band_tile_indices(const LaneGeom& q, uint64_t sc
     }
 }
 
+// Stream position (relative to the band-tile start) of bitmap 4g + 2sk for every lane, from
+// nothing but the lane's own two bitmaps and three DPP moves:
+//   lanes i and i^8 of a 16-lane row hold the two halves (sk = 0, 1) of 16-column group g, so
+//   row_ror:8 hands each lane the other half's popcount; the group totals are then prefix-summed
+//   across the four rows with row_bcast15 / row_bcast31, the cross-row steps of a wave scan.
+__device__ __forceinline__ int band_tile_prefix(const LaneGeom& q, int pc_pair)
+{
+    const int other = __builtin_amdgcn_update_dpp(0, pc_pair, 0x128, 0xf, 0xf, false);     // row_ror:8
+    const int group_total = pc_pair + other;
+    int incl = group_total;
+    incl += __builtin_amdgcn_update_dpp(0, incl, 0x142, 0xa, 0xf, false);                  // row_bcast15 -> rows 1,3
+    incl += __builtin_amdgcn_update_dpp(0, incl, 0x143, 0xc, 0xf, false);                  // row_bcast31 -> rows 2,3
+    return incl - group_total + (q.sk ? other : 0);
+}
+
+// For one band-tile: the two bytes (t = 0, 1) of nonzero flags this lane owns and the four
+// expansion-table indices that turn them into operand values.  The sign bits come from a
+// register-resident window: lane j of `win` holds sign word (sign_base >> 5) + j.  A band-tile has
+// at most 1024 sign bits, so its stream lies inside words 0..32 of that window, and the window
+// address depends only on the offset arrays, never on the bitmaps.
+__device__ __forceinline__ void band_tile_indices_win(const LaneGeom& q, const uint64_t bm[2], int sign_base,
+                                                      uint32_t win, uint32_t idx[2][2])
+{
+    uint32_t lo[2], hi[2];
+    int pc[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        lo[t] = static_cast<uint32_t>(bm[t]);
+        hi[t] = static_cast<uint32_t>(bm[t] >> 32);
+        pc[t] = __popc(lo[t]) + __popc(hi[t]);
+    }
+    int before = band_tile_prefix(q, pc[0] + pc[1]) + (sign_base & 31);   // relative to the window start
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const uint32_t nzb = ((q.r >= 4 ? hi[t] : lo[t]) >> (8 * (q.r & 3))) & 0xffu;
+        const int pos = before + __popc(lo[t] & q.lo_mask) + __popc(hi[t] & q.hi_mask);   // <= 31 + 1024
+        before += pc[t];
+        const int wsel = (pos >> 5) << 2;
+        const uint32_t w0 = __builtin_amdgcn_ds_bpermute(wsel, static_cast<int>(win));
+        const uint32_t w1 = __builtin_amdgcn_ds_bpermute(wsel + 4, static_cast<int>(win));
+        const uint32_t sbits = __builtin_amdgcn_alignbit(w1, w0, pos & 31);
+        const uint32_t n_lo = nzb & 15u;
+        idx[t][0] = (n_lo << 4) | (sbits & 15u);
+        idx[t][1] = (nzb & 0xf0u) | ((sbits >> __popc(n_lo)) & 15u);
+    }
+}
+
 // What a lane fetches for one band-tile before any arithmetic.
 template <typename Act, int MB>
 struct BandTileRaw {
-    uint64_t scan_bm;                       // bitmap (L & 15), for the prefix scan
     uint64_t bm[2];                         // bitmaps 4g + 2sk + t
-    uint4    x[MB][ActTraits<Act>::kXVecs]; // activation bytes of (row, group g)
+    u32x4    x[MB][ActTraits<Act>::kXVecs]; // activation bytes of (row, group g)
+    uint32_t win;                           // sign word (sign_base >> 5) + L
     int      sign_base;                     // tile offset + band offset, in sign bits
 };
 
-template <typename Act, int WAVES, int MB>
+// DEPTH = how many band-tiles ahead a wave keeps its global loads in flight.
+template <typename Act, int WAVES, int MB, int DEPTH>
 __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
     const Act* __restrict__ x, const uint64_t* __restrict__ bitmap, const int* __restrict__ tile_off,
     const uint16_t* __restrict__ median_off, const uint32_t* __restrict__ sign_words,
@@ -119,14 +172,18 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
     using T = ActTraits<Act>;
     using Acc = typename T::Acc;
     using Lut = typename T::Lut;
+    constexpr int NBUF = DEPTH + 1;
 
-    __shared__ Lut lut[256];
+    // One private copy of the 256-entry expansion table per wave: filling it needs no
+    // workgroup barrier, and it happens while the first loads are in flight.
+    __shared__ Lut lut_all[WAVES][256];
     __shared__ Acc red[WAVES][MB][64];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    for (int e = tid; e < 256; e += WAVES * 64) lut[e] = T::make_lut(e);
+    TERNA_TS(0);
+    Lut* lut = lut_all[wave];
 
     const int band = blockIdx.x;            // 16-row band of W
     const int gm = band >> 2, med = band & 3;
@@ -144,51 +201,74 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
         xrow[mb] = m < M ? m : M - 1;       // rows past M repeat the last one; never stored
     }
 
-    auto fetch = [&](int gk, BandTileRaw<Act, MB>& raw) {
-        const int tile = gm * ktiles + gk;
-        const uint64_t* bmp = bitmap + static_cast<size_t>(tile) * 64 + med * 16;
-        raw.scan_bm = bmp[i];
-        raw.bm[0] = bmp[b0];
-        raw.bm[1] = bmp[b0 + 1];
-        int base = tile_off[tile];
-        if (med) base += median_off[3 * tile + med - 1];
-        raw.sign_base = base;
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-            const Act* xp = x + static_cast<size_t>(xrow[mb]) * K + gk * 64 + g * 16;
-#pragma unroll
-            for (int v = 0; v < T::kXVecs; ++v) raw.x[mb][v] = reinterpret_cast<const uint4*>(xp)[v];
-        }
-    };
-
     Acc acc[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[mb] = Acc{0, 0, 0, 0};
 
-    BandTileRaw<Act, MB> cur, nxt;
-    int gk = wave;
-    if (gk < ktiles) fetch(gk, cur);
-    __syncthreads();                        // expansion table ready
+    // Wave w finishes m-block w (and w + WAVES, ...): fetch that block's scale factors now.
+    const int n0 = band * 16 + 4 * g;
+    EpilogueRegs eregs[(MB + WAVES - 1) / WAVES];
+#pragma unroll
+    for (int e = 0; e < (MB + WAVES - 1) / WAVES; ++e) {
+        const int m = m_base + (wave + e * WAVES) * 16 + i;
+        eregs[e] = load_epilogue(ep, m < M ? m : M - 1, n0, N);
+    }
 
-    for (; gk < ktiles; gk += WAVES) {
-        const bool more = gk + WAVES < ktiles;
-        if (more) fetch(gk + WAVES, nxt);
+    // This wave's band-tiles: gk = wave, wave + WAVES, ...  (cnt of them)
+    const int cnt = ktiles > wave ? (ktiles - wave + WAVES - 1) / WAVES : 0;
 
+    // Sign-stream start of band-tile number (c0 + lane) of this wave, held one per lane.
+    auto load_bases = [&](int c0) -> int {
+        const int j = c0 + lane;
+        int base = 0;
+        if (j < cnt) {
+            const int tile = gm * ktiles + wave + j * WAVES;
+            base = tile_off[tile];
+            if (med) base += median_off[3 * tile + med - 1];
+        }
+        return base;
+    };
+
+    // Loads that need no offset: the band-tile's bitmaps and the activation slab.
+    auto fetch_tile = [&](int j, BandTileRaw<Act, MB>& raw) {
+        const int gk = wave + j * WAVES;
+        const int tile = gm * ktiles + gk;
+        const uint64_t* bmp = bitmap + static_cast<size_t>(tile) * 64 + med * 16;
+        raw.bm[0] = bmp[b0];
+        raw.bm[1] = bmp[b0 + 1];
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            const Act* xp = x + static_cast<size_t>(xrow[mb]) * K + gk * 64 + g * 16;
+#pragma unroll
+            for (int v = 0; v < T::kXVecs; ++v) raw.x[mb][v] = reinterpret_cast<const u32x4*>(xp)[v];
+        }
+    };
+    // The sign window: needs the band-tile's stream offset.
+    auto fetch_signs = [&](int base, BandTileRaw<Act, MB>& raw) {
+        raw.sign_base = base;
+        uint32_t win = 0;
+        if (last_word >= 0) {
+            const int wi = (base >> 5) + lane;
+            win = sign_words[wi < last_word ? wi : last_word];
+        }
+        raw.win = win;
+    };
+
+    auto process = [&](const BandTileRaw<Act, MB>& cur) {
         uint32_t idx[2][2];
-        band_tile_indices(q, cur.scan_bm, cur.bm, cur.sign_base, sign_words, last_word, idx);
+        band_tile_indices_win(q, cur.bm, cur.sign_base, cur.win, idx);
 
         if constexpr (sizeof(Act) == 2) {
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-                const uint2 a_lo = lut[idx[t][0]];
-                const uint2 a_hi = lut[idx[t][1]];
-                const uint4 a_bits = make_uint4(a_lo.x, a_lo.y, a_hi.x, a_hi.y);
+                const u32x2 a_lo = lut[idx[t][0]];
+                const u32x2 a_hi = lut[idx[t][1]];
+                const u32x4 a_bits = {a_lo.x, a_lo.y, a_hi.x, a_hi.y};
                 const bf16x8 a = __builtin_bit_cast(bf16x8, a_bits);
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) {
-                    const uint4 x0 = cur.x[mb][0], x1 = cur.x[mb][1];
-                    const uint4 b_bits = t == 0 ? make_uint4(x0.x, x0.z, x1.x, x1.z)
-                                                : make_uint4(x0.y, x0.w, x1.y, x1.w);
+                    const u32x4 x0 = cur.x[mb][0], x1 = cur.x[mb][1];
+                    const u32x4 b_bits = t == 0 ? u32x4{x0.x, x0.z, x1.x, x1.z} : u32x4{x0.y, x0.w, x1.y, x1.w};
                     const bf16x8 b = __builtin_bit_cast(bf16x8, b_bits);
                     acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mb], 0, 0, 0);
                 }
@@ -199,7 +279,7 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
                              static_cast<int>(lut[idx[1][0]]), static_cast<int>(lut[idx[1][1]])};
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
-                const uint4 xv = cur.x[mb][0];       // dword j = columns 4j .. 4j+3
+                const u32x4 xv = cur.x[mb][0];       // dword j = columns 4j .. 4j+3
                 const i32x4 b = {
                     static_cast<int>(__builtin_amdgcn_perm(xv.y, xv.x, 0x05040100u)),   // t=0, c=0..3
                     static_cast<int>(__builtin_amdgcn_perm(xv.w, xv.z, 0x05040100u)),   // t=0, c=4..7
@@ -208,30 +288,82 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
                 acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[mb], 0, 0, 0);
             }
         }
-        if (more) cur = nxt;
+    };
+
+    // Ring of DEPTH + 1 register buffers, named one by one so that they stay in registers.
+    static_assert(DEPTH == 1 || DEPTH == 2, "prefetch distance");
+    BandTileRaw<Act, MB> ring0, ring1, ring2;
+    int c0 = 0, vbase = 0, ccnt = 0;
+    // One ring slot: start the loads of band-tile j + DEPTH into `pre`, then consume `cur`.
+    auto slot = [&](int j, const BandTileRaw<Act, MB>& cur, BandTileRaw<Act, MB>& pre) {
+        if (j < ccnt) {
+            if (j + DEPTH < ccnt) {
+                fetch_tile(c0 + j + DEPTH, pre);
+                fetch_signs(__builtin_amdgcn_readlane(vbase, j + DEPTH), pre);
+            }
+            process(cur);
+            TERNA_TS(3 + (j < 5 ? j : 5));
+        }
+    };
+    // Start of a round: offset-free loads go out first so they overlap the offset fetch.
+    auto prime = [&]() {
+        if (0 < ccnt) fetch_tile(c0, ring0);
+        if (DEPTH == 2 && 1 < ccnt) fetch_tile(c0 + 1, ring1);
+        if (0 < ccnt) fetch_signs(__builtin_amdgcn_readlane(vbase, 0), ring0);
+        if (DEPTH == 2 && 1 < ccnt) fetch_signs(__builtin_amdgcn_readlane(vbase, 1), ring1);
+    };
+
+    // Offsets come 64 band-tiles at a time (one per lane); K <= 4096 * WAVES needs one round.
+    ccnt = cnt < 64 ? cnt : 64;
+    vbase = load_bases(0);
+    prime();
+    TERNA_TS(1);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) lut[lane + 64 * e] = T::make_lut(lane + 64 * e);
+    TERNA_TS(2);
+    while (ccnt > 0) {
+        for (int j0 = 0; j0 < ccnt; j0 += NBUF) {
+            if constexpr (DEPTH == 2) {
+                slot(j0, ring0, ring2);
+                slot(j0 + 1, ring1, ring0);
+                slot(j0 + 2, ring2, ring1);
+            } else {
+                slot(j0, ring0, ring1);
+                slot(j0 + 1, ring1, ring0);
+            }
+        }
+        c0 += 64;
+        ccnt = cnt - c0 < 64 ? cnt - c0 : 64;
+        if (ccnt > 0) {
+            vbase = load_bases(c0);
+            prime();
+        }
     }
 
     // Cross-wave sum in wave order, then the fused epilogue.  The accumulator layout of a
     // 16x16 MFMA: lane L holds output rows 4*(L>>4) .. +3 of column L & 15.
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) red[wave][mb][lane] = acc[mb];
+    TERNA_TS(9);
     __syncthreads();
-    for (int mb = wave; mb < MB; mb += WAVES) {
+    TERNA_TS(10);
+#pragma unroll
+    for (int e = 0; e < (MB + WAVES - 1) / WAVES; ++e) {
+        const int mb = wave + e * WAVES;
+        if (mb >= MB) break;
         Acc sum = red[0][mb][lane];
 #pragma unroll
         for (int w = 1; w < WAVES; ++w) sum += red[w][mb][lane];
         const int m = m_base + mb * 16 + i;
         if (m < M) {
-            const int n0 = band * 16 + 4 * g;
             uint16_t o[4];
 #pragma unroll
-            for (int v = 0; v < 4; ++v)
-                o[v] = apply_epilogue<typename T::AccScalar>(ep, sum[v], m, n0 + v, N);
-            uint2 packed = make_uint2(o[0] | (static_cast<uint32_t>(o[1]) << 16),
-                                      o[2] | (static_cast<uint32_t>(o[3]) << 16));
-            *reinterpret_cast<uint2*>(out + static_cast<size_t>(m) * N + n0) = packed;
+            for (int v = 0; v < 4; ++v) o[v] = apply_epilogue<typename T::AccScalar>(ep.kind, eregs[e], v, sum[v]);
+            const u32x2 packed = {o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16)};
+            *reinterpret_cast<u32x2*>(out + static_cast<size_t>(m) * N + n0) = packed;
         }
     }
+    TERNA_TS(11);
 }
 
 }  // namespace terna

@@ -10,6 +10,8 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 constexpr int kWave = 64;
 
@@ -60,22 +62,43 @@ __device__ __forceinline__ int ws_group_prefill(int n, int N, int ws_num)
     return g < ws_num ? g : ws_num - 1;
 }
 
+// Scale factors of one output row m and four consecutive output columns n0..n0+3, fetched
+// ahead of the main loop so that no global load sits between the last MFMA and the store.
+struct EpilogueRegs {
+    float s;        // activation scale of row m (int8 family)
+    float w[4];     // weight-group scale of each column (bf16 family: the fp32 scale)
+};
+
+__device__ __forceinline__ EpilogueRegs load_epilogue(const Epilogue& ep, int m, int n0, int N)
+{
+    EpilogueRegs r;
+    r.s = 1.0f;
+    if (ep.kind == EP_BF16) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) r.w[v] = ep.scale[ws_group_decode(n0 + v, N, ep.ws_num)];
+    } else {
+        r.s = bf16_bits_to_float(ep.s[m]);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int g = ep.kind == EP_I8_DECODE ? ws_group_decode(n0 + v, N, ep.ws_num)
+                                                  : ws_group_prefill(n0 + v, N, ep.ws_num);
+            r.w[v] = bf16_bits_to_float(ep.ws[g]);
+        }
+    }
+    return r;
+}
+
 // One output element: integer or float accumulator -> bf16 storage.
 template <typename Acc>
-__device__ __forceinline__ uint16_t apply_epilogue(const Epilogue& ep, Acc acc, int m, int n, int N)
+__device__ __forceinline__ uint16_t apply_epilogue(int kind, const EpilogueRegs& e, int v, Acc acc)
 {
     float r;
-    if (ep.kind == EP_BF16) {
-        r = static_cast<float>(acc) * ep.scale[ws_group_decode(n, N, ep.ws_num)];
-    } else if (ep.kind == EP_I8_DECODE) {
-        const float sv = bf16_bits_to_float(ep.s[m]);
-        const float wv = bf16_bits_to_float(ep.ws[ws_group_decode(n, N, ep.ws_num)]);
-        const float q = __fdiv_rn(static_cast<float>(acc), sv);
-        r = __fmul_rn(q, wv);
+    if (kind == EP_BF16) {
+        r = static_cast<float>(acc) * e.w[v];
+    } else if (kind == EP_I8_DECODE) {
+        r = __fmul_rn(__fdiv_rn(static_cast<float>(acc), e.s), e.w[v]);
     } else {
-        const float sv = bf16_bits_to_float(ep.s[m]);
-        const float wv = bf16_bits_to_float(ep.ws[ws_group_prefill(n, N, ep.ws_num)]);
-        const float coeff = (sv != 0.0f) ? __fdiv_rn(wv, sv) : 0.0f;
+        const float coeff = (e.s != 0.0f) ? __fdiv_rn(e.w[v], e.s) : 0.0f;
         r = __fmul_rn(static_cast<float>(acc), coeff);
     }
     return float_to_bf16_bits(r);

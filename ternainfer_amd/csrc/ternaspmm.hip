@@ -14,8 +14,6 @@ using namespace terna;
 
 namespace {
 
-constexpr int kDecodeWaves = 8;
-
 [[noreturn]] void die(const char* what, hipError_t e, int line)
 {
     std::printf("Last Cuda Error Detected at line: %d, Error: %s (%s).\n", line, hipGetErrorString(e), what);
@@ -42,20 +40,44 @@ struct Weights {
 };
 
 // Small-M kernel: one workgroup per 16-row band; up to 64 batch rows per workgroup.
+template <typename Act, int WAVES, int MB, int DEPTH>
+void launch_decode_as(const Act* x, const Weights& w, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                      hipStream_t st)
+{
+    const dim3 grid(N / 16, (M + 16 * MB - 1) / (16 * MB));
+    terna_decode_kernel<Act, WAVES, MB, DEPTH><<<grid, dim3(WAVES * 64), 0, st>>>(
+        x, w.bitmap, w.tile_off, w.median_off, w.sign_words, out, ep, M, N, K);
+}
+
+// Shape of the small-M launch.  With one workgroup per 16-row band, a matrix with few bands
+// (N/16 <= 256: at most one workgroup per CU) is bound by each wave's serial share of K, so it
+// gets 16 waves and a deeper prefetch ring; a matrix with many bands is bound by how many
+// workgroups fit on the chip at once, so it gets 8 waves and the leaner ring (<= 64 VGPRs).
+// TERNASPMM_DECODE_WAVES=8|16 forces one variant (tuning aid).
+int decode_waves_override()
+{
+    static const int waves = [] {
+        const char* v = std::getenv("TERNASPMM_DECODE_WAVES");
+        const int w = v ? std::atoi(v) : 0;
+        return (w == 8 || w == 16) ? w : 0;
+    }();
+    return waves;
+}
+
 template <typename Act>
 void launch_decode(const Act* x, const Weights& w, uint16_t* out, const Epilogue& ep, int M, int N, int K,
                    hipStream_t st)
 {
-    const dim3 block(kDecodeWaves * 64);
+    const int forced = decode_waves_override();
+    const bool wide = forced ? forced == 16 : (N / 16 <= 256);
     if (M <= 16) {
-        terna_decode_kernel<Act, kDecodeWaves, 1><<<dim3(N / 16, 1), block, 0, st>>>(
-            x, w.bitmap, w.tile_off, w.median_off, w.sign_words, out, ep, M, N, K);
+        if (wide) launch_decode_as<Act, 16, 1, 2>(x, w, out, ep, M, N, K, st);
+        else launch_decode_as<Act, 8, 1, 1>(x, w, out, ep, M, N, K, st);
     } else if (M <= 32) {
-        terna_decode_kernel<Act, kDecodeWaves, 2><<<dim3(N / 16, 1), block, 0, st>>>(
-            x, w.bitmap, w.tile_off, w.median_off, w.sign_words, out, ep, M, N, K);
+        if (wide) launch_decode_as<Act, 16, 2, 1>(x, w, out, ep, M, N, K, st);
+        else launch_decode_as<Act, 8, 2, 1>(x, w, out, ep, M, N, K, st);
     } else {
-        terna_decode_kernel<Act, kDecodeWaves, 4><<<dim3(N / 16, (M + 63) / 64), block, 0, st>>>(
-            x, w.bitmap, w.tile_off, w.median_off, w.sign_words, out, ep, M, N, K);
+        launch_decode_as<Act, 8, 4, 1>(x, w, out, ep, M, N, K, st);
     }
 }
 
