@@ -189,7 +189,8 @@ def spmm_i8(x_q: np.ndarray, w: np.ndarray, s_bits: np.ndarray, ws_bits: np.ndar
     """
     m, _ = x_q.shape
     n = w.shape[0]
-    acc = x_q.astype(np.int64) @ w.astype(np.int64).T
+    # integer matmul through fp64 BLAS: exact while |acc| < 2^53 (here |acc| <= 128*K)
+    acc = np.rint(x_q.astype(np.float64) @ w.astype(np.float64).T).astype(np.int64)
     assert np.abs(acc).max(initial=0) < 2 ** 24
     accf = acc.astype(np.float32)
     s = bf16_bits_to_f32(s_bits).reshape(m, 1).astype(np.float32)

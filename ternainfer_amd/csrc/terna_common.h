@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace terna {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -68,6 +70,33 @@ struct EpilogueRegs {
     float s;        // activation scale of row m (int8 family)
     float w[4];     // weight-group scale of each column (bf16 family: the fp32 scale)
 };
+
+// Compile-time loop: the body receives the index as a constant, so register arrays indexed by it
+// never need dynamic addressing.
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+// Weight-group scales of the four consecutive output columns n0..n0+3.
+__device__ __forceinline__ void load_col_scales(const Epilogue& ep, int n0, int N, float w[4])
+{
+    if (ep.ws_num == 1) {                       // one scale per matrix: no group arithmetic
+        const float v = ep.kind == EP_BF16 ? ep.scale[0] : bf16_bits_to_float(ep.ws[0]);
+        w[0] = w[1] = w[2] = w[3] = v;
+        return;
+    }
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const int g = ep.kind == EP_I8_PREFILL ? ws_group_prefill(n0 + v, N, ep.ws_num)
+                                               : ws_group_decode(n0 + v, N, ep.ws_num);
+        w[v] = ep.kind == EP_BF16 ? ep.scale[g] : bf16_bits_to_float(ep.ws[g]);
+    }
+}
 
 __device__ __forceinline__ EpilogueRegs load_epilogue(const Epilogue& ep, int m, int n0, int N)
 {

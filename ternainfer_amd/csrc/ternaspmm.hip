@@ -8,6 +8,7 @@
 #include "../../include/ternaspmm.h"
 #include "decode_kernel.h"
 #include "decompress_kernel.h"
+#include "prefill_kernel.h"
 #include "format_host.h"
 
 using namespace terna;
@@ -81,13 +82,33 @@ void launch_decode(const Act* x, const Weights& w, uint16_t* out, const Epilogue
     }
 }
 
+// Large-M kernel: 256 output features x 64*MT batch rows per workgroup, MFMA-tiled.
+template <typename Act, int MT>
+void launch_prefill_as(const Act* x, const Weights& w, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                       hipStream_t st)
+{
+    using S = PrefillSmem<MT>;
+    auto kernel = terna_prefill_kernel<Act, MT>;
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, S::kBytes);
+    if (attr != hipSuccess) die("hipFuncSetAttribute(prefill)", attr, __LINE__);
+    const dim3 grid((N + kPrefillBN - 1) / kPrefillBN, (M + S::BM - 1) / S::BM);
+    kernel<<<grid, dim3(256), S::kBytes, st>>>(x, w.bitmap, w.tile_off, w.median_off, w.sign_words, out, ep, M, N, K);
+}
+
 template <typename Act>
 void launch_prefill(const Act* x, const Weights& w, uint16_t* out, const Epilogue& ep, int M, int N, int K,
                     hipStream_t st)
 {
-    // Until the MFMA-tiled kernel covers this range the small-M kernel computes it; the
-    // epilogue rule is the caller's, so results are unchanged.
-    launch_decode(x, w, out, ep, M, N, K, st);
+    if (K > 128 * 64) {                     // the MFMA kernel keeps per-step offsets for at most 128 steps
+        launch_decode(x, w, out, ep, M, N, K, st);
+        return;
+    }
+    // Largest batch tile that still gives every CU a workgroup; small problems take the smallest.
+    const int n_tiles = (N + kPrefillBN - 1) / kPrefillBN;
+    if (n_tiles * ((M + 255) / 256) >= 256) launch_prefill_as<Act, 4>(x, w, out, ep, M, N, K, st);
+    else if (n_tiles * ((M + 127) / 128) >= 256) launch_prefill_as<Act, 2>(x, w, out, ep, M, N, K, st);
+    else launch_prefill_as<Act, 1>(x, w, out, ep, M, N, K, st);
 }
 
 enum Route { ROUTE_AUTO, ROUTE_DECODE, ROUTE_PREFILL };

@@ -158,6 +158,17 @@ def test_int8_2b_layer_shapes_bit_exact(lib, m, n, k):
 
 
 # ------------------------------------------------------------------------------- bf16 family
+def _assert_negation_symmetric(out_bits, out_of_negated_x_bits):
+    """out(-x) == -out(x): exactly on all but a sliver of the outputs, and there to within one bf16
+    step of the value (or of the cancellation noise floor for sums that nearly cancel) -- the
+    matrix cores' internal fp32 summation is not exactly sign-symmetric."""
+    a = O.bf16_bits_to_f32(out_bits).astype(np.float64)
+    b = O.bf16_bits_to_f32(out_of_negated_x_bits).astype(np.float64)
+    diff = np.abs(a + b)
+    assert (diff != 0).mean() < 1e-4, float((diff != 0).mean())
+    assert (diff <= 2.0 ** -7 * np.abs(a) + 1e-4 * np.abs(a).max()).all(), float(diff.max())
+
+
 def _check_bf16(got, ref):
     max_err, max_ref, med_ulp, max_ulp = check_against_fp64(got, ref)
     assert max_err <= 1e-2 * max_ref, (max_err, max_ref)
@@ -223,7 +234,8 @@ def test_bf16_sparsity_sweep_m16(lib, n, k, kind):
 
 def test_bf16_linearity_and_zero_weights(lib):
     """Properties that hold at any size: W == 0 -> output exactly 0; doubling the scale doubles
-    every output exactly (power of two); negating x negates the output bit for bit."""
+    every output exactly (power of two); negating x negates the output (to within one bf16 step:
+    the matrix cores' internal fp32 summation is not exactly sign-symmetric)."""
     n, k, m = 2560, 2560, 8
     fmt0 = DeviceFormat(np.zeros((n, k), np.int8))
     x = make_bf16_activations(m, k, 71)
@@ -233,7 +245,7 @@ def test_bf16_linearity_and_zero_weights(lib):
     b = run_bf16(lib, fmt, x, np.array([1.5], np.float32), 1)
     assert (O.bf16_bits_to_f32(b) == 2 * O.bf16_bits_to_f32(a)).all()
     c = run_bf16(lib, fmt, x ^ np.uint16(0x8000), np.array([0.75], np.float32), 1)
-    assert ((c ^ np.uint16(0x8000)) == a).all()
+    _assert_negation_symmetric(a, c)
 
 
 def test_call_site_mirror_pads_and_slices(lib, coracle):
@@ -276,3 +288,59 @@ def test_graph_capture_replays(lib):
         g.replay()
         torch.cuda.synchronize()
         assert (out.cpu().numpy().view(np.uint16) == eager).all()
+
+
+# ------------------------------------------------------------------------------- MFMA-tiled (large-M) kernel
+@pytest.mark.parametrize("m", [1, 8, 33, 64, 100, 256, 300])
+@pytest.mark.parametrize("n,k", [(256, 64), (320, 128), (512, 320)])
+def test_bf16_prefill_kernel_small_shapes(lib, coracle, m, n, k):
+    """The forced _prefill entry runs the MFMA-tiled kernel at any M: ragged M, N not a multiple
+    of the 256-wide tile, one to five k-steps."""
+    w = make_ternary(n, k, 0.40, 300 + m + n)
+    fmt = DeviceFormat(w)
+    x = make_bf16_activations(m, k, 310 + m + k, outlier_frac=0.01)
+    scale = np.array([0.7, 1.9], np.float32)
+    got = run_bf16(lib, fmt, x, scale, 2, "bitlinear_TernaSpMM_bf16_prefill")
+    _check_bf16(got, coracle.spmm_bf16(x, w, scale, 2))
+
+
+@pytest.mark.parametrize("m", [65, 128, 256, 384])
+@pytest.mark.parametrize("n,k,ws_num", [(256, 192, 1), (3840, 128, 3), (640, 320, 2)])
+def test_int8_prefill_kernel_bit_exact(lib, m, n, k, ws_num):
+    """int8 activations through the bf16 MFMA tiles: every product and partial sum is an integer
+    below 2^24, so the result must equal the integer oracle bit for bit."""
+    w = make_ternary(n, k, 0.40, 320 + m + n)
+    fmt = DeviceFormat(w)
+    xq, s = make_int8_activations(m, k, 330 + m + k)
+    got = run_i8(lib, fmt, xq, s, WS, ws_num)                      # M > 64 -> prefill rule and kernel
+    assert (got == O.spmm_i8(xq, w, s, WS, ws_num, 1)).all()
+    got_d = run_i8(lib, fmt, xq, s, WS, ws_num, "bitlinear_TernaSpMM_decode")
+    assert (got_d == O.spmm_i8(xq, w, s, WS, ws_num, 0)).all()
+
+
+def test_prefill_entry_beyond_128_k_steps_falls_back(lib, coracle):
+    n, k, m = 64, 64 * 130, 70
+    w = make_ternary(n, k, 0.40, 341)
+    fmt = DeviceFormat(w)
+    x = make_bf16_activations(m, k, 342)
+    scale = np.array([1.0], np.float32)
+    got = run_bf16(lib, fmt, x, scale, 1, "bitlinear_TernaSpMM_bf16_prefill")
+    _check_bf16(got, O.spmm_bf16_golden(x, w, scale, 1))
+
+
+@pytest.mark.parametrize("n,k", [(3840, 2560), (2560, 2560), (13824, 2560), (2560, 6912)])
+@pytest.mark.parametrize("m", [256, 512, 2048])
+def test_bf16_prefill_2b_layer_shapes(lib, m, n, k):
+    """Prefill shapes with 1% outlier channels (x20).  The fp64 golden is taken on a seeded sample
+    of 192 output columns (all rows), which keeps the host matmul small; the whole output is
+    also checked for the size-independent property out(-x) == -out(x)."""
+    w = make_ternary(n, k, 0.40, seed_for(3, n % 7))
+    fmt = DeviceFormat(w)
+    x = make_bf16_activations(m, k, seed_for(3, 30 + m % 97), outlier_frac=0.01)
+    scale = np.array([1.37], np.float32)
+    got = run_bf16(lib, fmt, x, scale, 1)
+    cols = np.sort(np.random.default_rng(seed_for(3, 99)).permutation(n)[:192])
+    ref = O.bf16_bits_to_f32(x).astype(np.float64) @ w[cols].astype(np.float64).T * float(scale[0])
+    _check_bf16(got[:, cols], ref)
+    neg = run_bf16(lib, fmt, x ^ np.uint16(0x8000), scale, 1)
+    _assert_negation_symmetric(got, neg)
