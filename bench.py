@@ -157,6 +157,67 @@ def cpu_baseline(mats, torch):
     }
 
 
+def run_prefill(args, torch, T, lib):
+    """configs[2]: the four BitNet-2B matrices at M in {256, 512, 2048}, bf16 activations with 1% of
+    the channels scaled x20.  A step is one pass over the four matrices at M = --m (default 2048
+    when --workload prefill is given without --m)."""
+    m_main = args.m if args.m >= 64 else 2048
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rng = np.random.default_rng(20260300)
+    mats = []
+    for j, (name, n, k) in enumerate(LAYER_SET):
+        mt = Matrix(name, n, k, 8, 1, 20260300 + 10 * j, torch, T)
+        xs = {}
+        for m in sorted({256, 512, 2048, m_main}):
+            xf = rng.standard_normal((m, k)).astype(np.float32)
+            ch = rng.permutation(k)[: int(np.ceil(0.01 * k))]
+            xf[:, ch] *= 20.0
+            xs[m] = (torch.from_numpy(f32_to_bf16_bits(xf).view(np.int16)).cuda(),
+                     torch.zeros((m, n), dtype=torch.int16, device="cuda"))
+        mats.append((mt, xs))
+
+    def launch(mt, xs, m, s):
+        x, out = xs[m]
+        vals, off, med, bm = mt.dev[0]
+        lib.bitlinear_TernaSpMM_bf16(vp(x), vp(bm), vp(off), vp(med), vp(vals), vp(out), vp(mt.scale),
+                                     1, m, mt.n, mt.k, 1, None, s)
+
+    per_shape = {}
+    for mt, xs in mats:
+        for m in sorted(xs):
+            launch(mt, xs, m, stream)
+            torch.cuda.synchronize()
+            g = capture(torch, lambda s, mt=mt, xs=xs, m=m: [launch(mt, xs, m, s) for _ in range(10)])
+            us = time_graph(torch, g, 5, 2) * 1e3 / 10
+            tf = 2.0 * m * mt.n * mt.k / us / 1e6
+            per_shape[f"{mt.name}_{mt.k}x{mt.n}_M{m}"] = {"us": us, "tflops": tf, "frac": tf / BF16_MFMA_PEAK_TFLOPS}
+
+    graph = capture(torch, lambda s: [launch(mt, xs, m_main, s) for mt, xs in mats])
+    for _ in range(args.warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(args.steps):
+        graph.replay()
+    ev1.record()
+    torch.cuda.synchronize()
+    ms = ev0.elapsed_time(ev1) / args.steps
+    flops = sum(2.0 * m_main * mt.n * mt.k for mt, _ in mats)
+    tf = flops / (ms * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "TernaSpMM prefill TFLOP/s + %bf16 MFMA peak (M=2048, BitNet-2B layer set)",
+        "value": tf, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"configs[2]: four BitNet-b1.58-2B matrices at M={m_main}, P(0)=0.40, bf16 activations "
+                               "with 1% outlier channels (x20), HIP-graph replay", "m": m_main},
+        "roofline": {"bound": "mfma", "achieved": tf, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tf / BF16_MFMA_PEAK_TFLOPS, "traffic": None,
+                     "kernel": "terna_prefill_kernel<bf16>", "algorithmic_flops_per_step": flops},
+        "per_shape": per_shape}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -164,6 +225,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--m", type=int, default=8, help="activation rows per call (decode batch)")
     ap.add_argument("--layers", type=int, default=30, help="distinct weight copies per matrix")
+    ap.add_argument("--workload", choices=["decode", "prefill"], default="decode",
+                    help="decode: the headline small-M HBM-bound pass; prefill: the M>=256 MFMA-bound pass")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-per-shape", action="store_true")
     args = ap.parse_args()
@@ -177,6 +240,10 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs the MI355X"
     lib = T._lib.load()
     torch.cuda.set_device(0)
+
+    if args.workload == "prefill":
+        run_prefill(args, torch, T, lib)
+        return
 
     mats = [Matrix(name, n, k, args.m, args.layers, 20260200 + 10 * j, torch, T)
             for j, (name, n, k) in enumerate(LAYER_SET)]
