@@ -40,8 +40,9 @@ void checkLastCudaError(int line);
  *   M <= 64 : epilogue bf16((acc / s[m]) * ws[g])        (Reduction_Kernel.cuh:60)
  *   M  > 64 : epilogue bf16(acc * (ws[g] / s[m])), 0 if s[m]==0, g per 128-column tile
  *                                                        (epilogue_visitor_scale_ws.h:135-205)
- *   SPLIT_K and workspace are accepted for compatibility; this build reduces split-K
- *   partials on chip and never touches `workspace`. */
+ *   SPLIT_K is accepted for compatibility (split-K partials are reduced on chip).  `workspace`
+ *   is used only for M > 64: if it is non-NULL and 16-byte aligned, N*K/4 bytes of it receive a
+ *   transcoded copy of the weights for the duration of the call; pass NULL to keep it untouched. */
 void bitlinear_TernaSpMM(int8_t* x, uint64_t* bitmap, int* tile_offsets_global,
                          uint16_t* tile_offsets_median, uint32_t* sign_words,
                          terna_bf16* out, terna_bf16* s, terna_bf16* ws, int ws_num,
@@ -89,7 +90,8 @@ void gpu_sleep(double us, terna_stream stream);
  *   x bf16 [M][K], any M >= 1 (no padding rows needed); scale fp32 [ws_num];
  *   group rule of the decode path (Reduction_Kernel.cuh:46-54).
  * The plain symbol picks a kernel by M; _decode / _prefill force the small-M dot-product
- * kernel or the MFMA-tiled kernel.  workspace may be NULL. */
+ * kernel or the MFMA-tiled kernel.  workspace may be NULL; if given (16-byte aligned, N*K/4
+ * bytes) the MFMA-tiled path transcodes the weights into it first, which is faster. */
 void bitlinear_TernaSpMM_bf16(const terna_bf16* x, const uint64_t* bitmap, const int* tile_offsets_global,
                               const uint16_t* tile_offsets_median, const uint32_t* sign_words,
                               terna_bf16* out, const float* scale, int ws_num,
@@ -120,6 +122,30 @@ int64_t ternaspmm_encode_i8(const int8_t* W, int N, int K, uint64_t* bitmap, int
 void ternaspmm_decompress_bf16(const uint64_t* bitmap, const int* tile_offsets_global,
                                const uint16_t* tile_offsets_median, const uint32_t* sign_words,
                                terna_bf16* W_dense, int N, int K, terna_stream stream);
+
+/* ---- load-time repack ("P2" layout, 2 bits per weight, N*K/4 bytes) ----------------------------
+ * The reference format stays the on-disk and interchange format.  P2 is a device-side layout
+ * this library can derive from it, bit-exactly, once at load time; its kernels need no offset
+ * arrays and no sign-stream arithmetic.  Callers that keep to the reference entry points never
+ * see it, except that the large-M path (M > 64) transcodes into `workspace` when one is given:
+ * it needs N*K/4 bytes there, within the N*K bytes the reference's call site guarantees
+ * (model.py:34-42). */
+
+/* Bytes of a P2 buffer for an [N][K] matrix, or -1 if N or K is not a multiple of 64. */
+int64_t ternaspmm_packed_bytes(int N, int K);
+
+/* Device: reference format -> P2 into `packed` (16-byte aligned, ternaspmm_packed_bytes(N,K) bytes). */
+void ternaspmm_repack(const uint64_t* bitmap, const int* tile_offsets_global, const uint16_t* tile_offsets_median,
+                      const uint32_t* sign_words, void* packed, int N, int K, terna_stream stream);
+
+/* bf16-activation linear on a P2 buffer.  route: 0 = pick by M, 1 = MFMA-tiled kernel, 2 = small-M kernel. */
+void bitlinear_TernaSpMM_bf16_packed(const terna_bf16* x, const void* packed, terna_bf16* out, const float* scale,
+                                     int ws_num, int M, int N, int K, int route, terna_stream stream);
+
+/* int8-activation linear on a P2 buffer; arguments as bitlinear_TernaSpMM.  route: 0 = the reference's
+ * rule (decode epilogue for M <= 64, prefill epilogue above), 1 = prefill epilogue, 2 = decode epilogue. */
+void bitlinear_TernaSpMM_packed(const int8_t* x, const void* packed, terna_bf16* out, const terna_bf16* s,
+                                const terna_bf16* ws, int ws_num, int M, int N, int K, int route, terna_stream stream);
 
 /* Library version string, e.g. "ternaspmm-gfx950 0.1". */
 const char* ternaspmm_version(void);

@@ -34,6 +34,10 @@ PROTOTYPES = {
     "ternaspmm_encode_sizes": ([_ci, _ci, _vp, _vp, _vp, _vp], _ci),
     "ternaspmm_encode_i8": ([_vp, _ci, _ci, _vp, _vp, _vp, _vp], ctypes.c_int64),
     "ternaspmm_decompress_bf16": ([_vp, _vp, _vp, _vp, _vp, _ci, _ci, _vp], None),
+    "ternaspmm_packed_bytes": ([_ci, _ci], ctypes.c_int64),
+    "ternaspmm_repack": ([_vp, _vp, _vp, _vp, _vp, _ci, _ci, _vp], None),
+    "bitlinear_TernaSpMM_bf16_packed": ([_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp], None),
+    "bitlinear_TernaSpMM_packed": ([_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp], None),
     "ternaspmm_version": ([], ctypes.c_char_p),
 }
 

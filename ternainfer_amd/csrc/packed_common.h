@@ -1,0 +1,107 @@
+// The load-time layout "P2" and its expansion to MFMA operands (gfx950).
+//
+// P2 is this library's own device layout of a ternary matrix; the reference has no counterpart.
+// It is produced from the reference's compressed format by terna_repack_kernel (bit-exact,
+// checked by round trip) either once at load time or, on the reference's prefill entry points,
+// per call into the caller's workspace.  It costs 2 bits per weight (N*K/4 bytes, vs ~1.6 bits
+// in the reference format) and buys a decode with no offsets, no popcounts and no LDS:
+//
+//   uint32 packed[N/16][K/64][64]
+//   element [band][gk][4*i + g] : row 16*band + i, columns 64*gk + 16*g .. +15, 2 bits each
+//                                 (bit0 = nonzero, bit1 = negative)
+//   weight (t, c) of the group  : column 16g + 4*(c>>1) + 2t + (c&1)   (the format's own
+//                                 coordinates: byte pair t, bit c of a bitmap row)
+//                                 sits at bit 8*(c&3) + 2*(2t + (c>>2)).
+//
+// So `(word >> 2*(2t+h)) & 0x03030303` is four 2-bit codes in four bytes -- exactly a v_perm_b32
+// selector.  One v_perm against a 4-entry byte table turns it into four int8 weights
+// (0x00 / 0x01 / 0xFF) or four bf16 high bytes (0x00 / 0x3F / 0xBF), and two more v_perm
+// interleave the high bytes with zero low bytes into bf16 pairs.  bf16 weights are therefore
+// +-0.5 (0x3F00 / 0xBF00), not +-1: every product and partial sum is exactly half of what +-1
+// would give, and the epilogue multiplies the accumulator by 2, which is exact.
+#pragma once
+
+#include "decode_kernel.h"
+
+namespace terna {
+
+constexpr uint32_t kCodeMask = 0x03030303u;
+constexpr uint32_t kTableBf16Hi = 0xBF003F00u;   // code 0 -> 0x00, 1 -> 0x3F, 3 -> 0xBF
+constexpr uint32_t kTableI8 = 0xFF000100u;       // code 0 -> 0x00, 1 -> 0x01, 3 -> 0xFF
+constexpr uint32_t kPair01 = 0x010C000Cu;        // [0, b0, 0, b1]: two bf16 with zero low bytes
+constexpr uint32_t kPair23 = 0x030C020Cu;        // [0, b2, 0, b3]
+
+// Eight bf16 weights (+-0.5 / 0) of byte pair t of a packed word `dd` already shifted right by 4t:
+// k order c = 0..7, i.e. dword j holds the weights that meet activation dword (2j + t) of the group.
+__device__ __forceinline__ u32x4 expand_chunk_bf16(uint32_t dd)
+{
+    const uint32_t hi0 = __builtin_amdgcn_perm(0u, kTableBf16Hi, dd & kCodeMask);
+    const uint32_t hi1 = __builtin_amdgcn_perm(0u, kTableBf16Hi, (dd >> 2) & kCodeMask);
+    return u32x4{__builtin_amdgcn_perm(0u, hi0, kPair01), __builtin_amdgcn_perm(0u, hi0, kPair23),
+                 __builtin_amdgcn_perm(0u, hi1, kPair01), __builtin_amdgcn_perm(0u, hi1, kPair23)};
+}
+
+// Sixteen int8 weights (+-1 / 0) of a packed word: dword (2t + h) holds (t, c = 4h .. 4h+3).
+__device__ __forceinline__ i32x4 expand_word_i8(uint32_t d)
+{
+    return i32x4{static_cast<int>(__builtin_amdgcn_perm(0u, kTableI8, d & kCodeMask)),
+                 static_cast<int>(__builtin_amdgcn_perm(0u, kTableI8, (d >> 2) & kCodeMask)),
+                 static_cast<int>(__builtin_amdgcn_perm(0u, kTableI8, (d >> 4) & kCodeMask)),
+                 static_cast<int>(__builtin_amdgcn_perm(0u, kTableI8, (d >> 6) & kCodeMask))};
+}
+
+// Repack table: (nonzero nibble, next 4 sign bits of the stream) -> four 2-bit codes, one per byte.
+__device__ __forceinline__ uint32_t make_lut_code(int e)
+{
+    const int nz = e >> 4, sg = e & 15;
+    uint32_t r = 0;
+    int used = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if ((nz >> j) & 1) {
+            r |= (1u | (((sg >> used) & 1) << 1)) << (8 * j);
+            ++used;
+        }
+    }
+    return r;
+}
+
+// Reference format -> P2.  One wave per 16x64 band-tile; lane (i, g) produces word 4*i + g.
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void terna_repack_kernel(
+    const uint64_t* __restrict__ bitmap, const int* __restrict__ tile_off,
+    const uint16_t* __restrict__ median_off, const uint32_t* __restrict__ sign_words,
+    uint32_t* __restrict__ packed, int N, int K)
+{
+    __shared__ uint32_t lut[256];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    for (int e = tid; e < 256; e += WAVES * 64) lut[e] = make_lut_code(e);
+    __syncthreads();
+
+    const int band = blockIdx.x;
+    const int gm = band >> 2, med = band & 3;
+    const int ktiles = K >> 6;
+    const int last_word = (tile_off[(N >> 6) * ktiles] >> 5) - 1;
+    const LaneGeom q(lane);
+
+    for (int gk = wave; gk < ktiles; gk += WAVES) {
+        const int tile = gm * ktiles + gk;
+        const uint64_t* bmp = bitmap + static_cast<size_t>(tile) * 64 + med * 16;
+        const uint64_t bm[2] = {bmp[q.b0], bmp[q.b0 + 1]};
+        int base = tile_off[tile];
+        if (med) base += median_off[3 * tile + med - 1];
+        uint32_t win = 0;
+        if (last_word >= 0) {
+            const int wi = (base >> 5) + lane;
+            win = sign_words[wi < last_word ? wi : last_word];
+        }
+        uint32_t idx[2][2];
+        band_tile_indices_win(q, bm, base, win, idx);
+        const uint32_t word = lut[idx[0][0]] | (lut[idx[0][1]] << 2) | (lut[idx[1][0]] << 4) | (lut[idx[1][1]] << 6);
+        packed[(static_cast<size_t>(band) * ktiles + gk) * 64 + q.i * 4 + q.g] = word;
+    }
+}
+
+}  // namespace terna

@@ -96,97 +96,88 @@ __global__ __launch_bounds__(256, 1) void terna_prefill_kernel(
     const LaneGeom q(lane);
 
     // ---- this wave's four band-tiles per step: bands 4*wave .. 4*wave+3 of the tile
-    int band_gm[4], band_med[4];
+    int band_med[4];
+    const uint64_t* bm_ptr[4];                         // this lane's first bitmap of band u at k-step 0
+    int vbase[4][2];                                   // sign-stream start of (band u, k-step lane / 64 + lane)
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
         int band = (n0 >> 4) + 4 * wave + u;
-        band = band < last_band ? band : last_band;  // a tile hanging over N re-decodes the last band; never stored
-        band_gm[u] = band >> 2;
+        band = band < last_band ? band : last_band;    // a tile hanging over N re-decodes the last band; never stored
+        const int gm = band >> 2;
         band_med[u] = band & 3;
-    }
-    // sign-stream start of (band u, k-step lane) and (band u, k-step 64 + lane), one per lane
-    int vbase[4][2];
-#pragma unroll
-    for (int u = 0; u < 4; ++u)
+        bm_ptr[u] = bitmap + (static_cast<size_t>(gm) * ktiles * 64 + band_med[u] * 16 + q.b0);
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int gk = 64 * h + lane;
             int base = 0;
             if (gk < ktiles) {
-                const int tile = band_gm[u] * ktiles + gk;
+                const int tile = gm * ktiles + gk;
                 base = tile_off[tile];
                 if (band_med[u]) base += median_off[3 * tile + band_med[u] - 1];
             }
             vbase[u][h] = base;
         }
+    }
 
     // ---- activation items of this thread: item = tid + 256*it -> (row = item / 4, group = item % 4)
-    int x_row[Raw::XI], x_g[Raw::XI];
+    int x_lds[Raw::XI];                                // byte offset of the item's sm = 0 chunk in the X tile
     const Act* x_ptr[Raw::XI];
 #pragma unroll
     for (int it = 0; it < Raw::XI; ++it) {
         const int item = tid + 256 * it;
-        x_row[it] = item >> 2;
-        x_g[it] = item & 3;
-        int m = m0 + x_row[it];
+        const int row = item >> 2, g = item & 3;
+        x_lds[it] = (g * 2) * PX + row * 16;
+        int m = m0 + row;
         m = m < M ? m : M - 1;
-        x_ptr[it] = x + static_cast<size_t>(m) * K + x_g[it] * 16;
+        x_ptr[it] = x + static_cast<size_t>(m) * K + g * 16;
     }
 
-    auto fetch = [&](int gk, Raw& raw) {
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int tile = band_gm[u] * ktiles + gk;
-            const uint64_t* bmp = bitmap + static_cast<size_t>(tile) * 64 + band_med[u] * 16;
-            raw.bm[u][0] = bmp[q.b0];
-            raw.bm[u][1] = bmp[q.b0 + 1];
-            const int base = gk < 64 ? __builtin_amdgcn_readlane(vbase[u][0], gk & 63)
-                                     : __builtin_amdgcn_readlane(vbase[u][1], gk & 63);
-            raw.base[u] = base;
-            uint32_t win = 0;
-            if (last_word >= 0) {
-                const int wi = (base >> 5) + lane;
-                win = sign_words[wi < last_word ? wi : last_word];
-            }
-            raw.win[u] = win;
+    // Global loads of k-step gk, one quarter (u) at a time.
+    auto fetch_w = [&](int u, int gk, Raw& raw) {
+        const uint64_t* bmp = bm_ptr[u] + static_cast<size_t>(gk) * 64;
+        raw.bm[u][0] = bmp[0];
+        raw.bm[u][1] = bmp[1];
+        const int base = gk < 64 ? __builtin_amdgcn_readlane(vbase[u][0], gk & 63)
+                                 : __builtin_amdgcn_readlane(vbase[u][1], gk & 63);
+        raw.base[u] = base;
+        uint32_t win = 0;
+        if (last_word >= 0) {
+            const int wi = (base >> 5) + lane;
+            win = sign_words[wi < last_word ? wi : last_word];
         }
+        raw.win[u] = win;
+    };
+    auto fetch_x = [&](int it, int gk, Raw& raw) {
+        const u32x4* p = reinterpret_cast<const u32x4*>(x_ptr[it] + gk * 64);
 #pragma unroll
-        for (int it = 0; it < Raw::XI; ++it) {
-            const u32x4* p = reinterpret_cast<const u32x4*>(x_ptr[it] + gk * 64);
-#pragma unroll
-            for (int v = 0; v < T::kXVecs; ++v) raw.x[it][v] = p[v];
-        }
+        for (int v = 0; v < T::kXVecs; ++v) raw.x[it][v] = p[v];
     };
 
-    // Decode the prefetched band-tiles and stage the activations into LDS stage `st`.
-    auto stage_in = [&](const Raw& raw, int st) {
+    // Decode one prefetched band-tile into stage `st` of the W tile.
+    auto decode_w = [&](int u, const Raw& raw, int st) {
         uint8_t* ws = smem + st * S::kStage;
-        uint8_t* xs = ws + 8 * PW;
+        uint32_t idx[2][2];
+        band_tile_indices_win(q, raw.bm[u], raw.base[u], raw.win[u], idx);
+        const int row = 16 * (4 * wave + u) + q.i;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            uint32_t idx[2][2];
-            band_tile_indices_win(q, raw.bm[u], raw.base[u], raw.win[u], idx);
-            const int row = 16 * (4 * wave + u) + q.i;
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                const u32x2 lo = lut[idx[t][0]], hi = lut[idx[t][1]];
-                *reinterpret_cast<u32x4*>(ws + (q.g * 2 + t) * PW + row * 16) = u32x4{lo.x, lo.y, hi.x, hi.y};
-            }
+        for (int t = 0; t < 2; ++t) {
+            const u32x2 lo = lut[idx[t][0]], hi = lut[idx[t][1]];
+            *reinterpret_cast<u32x4*>(ws + (q.g * 2 + t) * PW + row * 16) = u32x4{lo.x, lo.y, hi.x, hi.y};
         }
-#pragma unroll
-        for (int it = 0; it < Raw::XI; ++it) {
-            u32x4 c0, c1;
-            if constexpr (sizeof(Act) == 2) {
-                const u32x4 a = raw.x[it][0], b = raw.x[it][1];
-                c0 = u32x4{a.x, a.z, b.x, b.z};
-                c1 = u32x4{a.y, a.w, b.y, b.w};
-            } else {
-                int8_group_to_chunks(raw.x[it][0], c0, c1);
-            }
-            uint8_t* dst = xs + (x_g[it] * 2) * PX + x_row[it] * 16;
-            *reinterpret_cast<u32x4*>(dst) = c0;
-            *reinterpret_cast<u32x4*>(dst + PX) = c1;
+    };
+    // Split one prefetched activation group into its two chunks in stage `st` of the X tile.
+    auto stage_x = [&](int it, const Raw& raw, int st) {
+        u32x4 c0, c1;
+        if constexpr (sizeof(Act) == 2) {
+            const u32x4 a = raw.x[it][0], b = raw.x[it][1];
+            c0 = u32x4{a.x, a.z, b.x, b.z};
+            c1 = u32x4{a.y, a.w, b.y, b.w};
+        } else {
+            int8_group_to_chunks(raw.x[it][0], c0, c1);
         }
+        uint8_t* dst = smem + st * S::kStage + 8 * PW + x_lds[it];
+        *reinterpret_cast<u32x4*>(dst) = c0;
+        *reinterpret_cast<u32x4*>(dst + PX) = c1;
     };
 
     f32x16 acc[4][MT];
@@ -199,49 +190,90 @@ __global__ __launch_bounds__(256, 1) void terna_prefill_kernel(
     }
 
     const int kb = lane >> 5, l32 = lane & 31;
-    auto mma_stage = [&](int st) {
-        const uint8_t* ws = smem + st * S::kStage;
-        const uint8_t* xs = ws + 8 * PW;
+    struct Operands {
+        bf16x8 a[4];
+        bf16x8 b[MT];
+    };
+    const int a_off = kb * PW + (128 * wn + l32) * 16;            // + g*2*PW + a*512
+    const int b_off = 8 * PW + kb * PX + (32 * MT * wm + l32) * 16;  // + g*2*PX + b*512
+    auto load_operands = [&](int st, int g, Operands& r) {
+        const uint8_t* base = smem + st * S::kStage;
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            bf16x8 af[4], bfr[MT];
+        for (int a = 0; a < 4; ++a)
+            r.a[a] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(base + a_off + g * 2 * PW + a * 512));
 #pragma unroll
-            for (int a = 0; a < 4; ++a)
-                af[a] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(
-                            ws + (g * 2 + kb) * PW + (128 * wn + 32 * a + l32) * 16));
+        for (int b = 0; b < MT; ++b)
+            r.b[b] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(base + b_off + g * 2 * PX + b * 512));
+    };
+    auto mfma_block = [&](const Operands& r) {
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
 #pragma unroll
             for (int b = 0; b < MT; ++b)
-                bfr[b] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(
-                             xs + (g * 2 + kb) * PX + (32 * MT * wm + 32 * b + l32) * 16));
-#pragma unroll
-            for (int a = 0; a < 4; ++a)
-#pragma unroll
-                for (int b = 0; b < MT; ++b)
-                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[a], bfr[b], acc[a][b], 0, 0, 0);
-        }
+                acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(r.a[a], r.b[b], acc[a][b], 0, 0, 0);
     };
 
-    // ---- pipeline: loads two steps ahead, decode one step ahead, MFMA on the current stage
+    // One k-step = four g-steps.  G-step j multiplies 16-column group j of stage `cur` while it
+    // decodes band-tile j and stages activation item j of the NEXT k-step into stage `cur ^ 1`,
+    // starts quarter j of the global loads two k-steps ahead, and reads the operands of group j+1.
+    // The sched_group_barrier sequence asks the scheduler to deal those side jobs out between the
+    // matrix instructions instead of in front of them.
     Raw raw;
-    fetch(0, raw);
+    Operands ops;
+    auto k_step = [&](int k, auto has_next, auto has_next2) {
+        const int cur = k & 1;
+        static_for<0, 4>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            Operands nxt;
+            if constexpr (j < 3) load_operands(cur, j + 1, nxt);
+            if constexpr (decltype(has_next)::value) {
+                decode_w(j, raw, cur ^ 1);
+                static_for<0, Raw::XI>([&](auto ic) {
+                    constexpr int it = decltype(ic)::value;
+                    if constexpr (it * (4 / MT) == j) stage_x(it, raw, cur ^ 1);
+                });
+            }
+            if constexpr (decltype(has_next2)::value) {
+                fetch_w(j, k + 2, raw);
+                static_for<0, Raw::XI>([&](auto ic) {
+                    constexpr int it = decltype(ic)::value;
+                    if constexpr (it * (4 / MT) == j) fetch_x(it, k + 2, raw);
+                });
+            }
+            mfma_block(ops);
+#pragma unroll
+            for (int r = 0; r < 4 * MT; ++r) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               // one MFMA
+                __builtin_amdgcn_sched_group_barrier(0x002, 16 / MT, 0);         // vector ALU
+                __builtin_amdgcn_sched_group_barrier(0x100, MT >= 2 ? 1 : 3, 0); // LDS reads
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);               // LDS write
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);               // global read
+            }
+            if constexpr (j < 3) ops = nxt;
+        });
+        __syncthreads();
+        if constexpr (decltype(has_next)::value) load_operands(cur ^ 1, 0, ops);
+    };
+
+    // ---- pipeline: global loads two k-steps ahead, decode one k-step ahead
+    static_for<0, 4>([&](auto uc) { fetch_w(decltype(uc)::value, 0, raw); });
+    static_for<0, Raw::XI>([&](auto ic) { fetch_x(decltype(ic)::value, 0, raw); });
     __syncthreads();                                  // expansion table ready
-    stage_in(raw, 0);
-    if (ktiles > 1) fetch(1, raw);
-    __syncthreads();
-    int k = 0;
-    for (; k + 2 < ktiles; ++k) {
-        stage_in(raw, (k + 1) & 1);
-        fetch(k + 2, raw);
-        mma_stage(k & 1);
-        __syncthreads();
+    static_for<0, 4>([&](auto uc) { decode_w(decltype(uc)::value, raw, 0); });
+    static_for<0, Raw::XI>([&](auto ic) { stage_x(decltype(ic)::value, raw, 0); });
+    if (ktiles > 1) {
+        static_for<0, 4>([&](auto uc) { fetch_w(decltype(uc)::value, 1, raw); });
+        static_for<0, Raw::XI>([&](auto ic) { fetch_x(decltype(ic)::value, 1, raw); });
     }
+    __syncthreads();
+    load_operands(0, 0, ops);
+    int k = 0;
+    for (; k + 2 < ktiles; ++k) k_step(k, std::true_type{}, std::true_type{});
     if (k + 1 < ktiles) {
-        stage_in(raw, (k + 1) & 1);
-        mma_stage(k & 1);
-        __syncthreads();
+        k_step(k, std::true_type{}, std::false_type{});
         ++k;
     }
-    mma_stage(k & 1);
+    k_step(k, std::false_type{}, std::false_type{});
 
     // ---- epilogue: lane holds, per accumulator tile, column m = l32 and rows n = (v&3) + 8(v>>2) + 4kb
     EpilogueRegs e[MT];

@@ -9,6 +9,8 @@
 #include "decode_kernel.h"
 #include "decompress_kernel.h"
 #include "prefill_kernel.h"
+#include "decode_packed_kernel.h"
+#include "prefill_packed_kernel.h"
 #include "format_host.h"
 
 using namespace terna;
@@ -111,10 +113,83 @@ void launch_prefill(const Act* x, const Weights& w, uint16_t* out, const Epilogu
     else launch_prefill_as<Act, 1>(x, w, out, ep, M, N, K, st);
 }
 
+// ---- P2 layout (load-time repack): see packed_common.h -------------------------------------------
+void launch_repack(const Weights& w, uint32_t* packed, int N, int K, hipStream_t st)
+{
+    terna_repack_kernel<4><<<dim3(N / 16), dim3(256), 0, st>>>(w.bitmap, w.tile_off, w.median_off, w.sign_words,
+                                                              packed, N, K);
+}
+
+template <typename Act, int WAVES, int MB, int DEPTH>
+void launch_decode_packed_as(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N,
+                             int K, hipStream_t st)
+{
+    const dim3 grid(N / 16, (M + 16 * MB - 1) / (16 * MB));
+    terna_decode_packed_kernel<Act, WAVES, MB, DEPTH><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, ep, M, N, K);
+}
+
+template <typename Act>
+void launch_decode_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                          hipStream_t st)
+{
+    const int forced = decode_waves_override();
+    const bool wide = forced ? forced == 16 : (N / 16 <= 256);
+    if (M <= 16) {
+        if (wide) launch_decode_packed_as<Act, 16, 1, 3>(x, packed, out, ep, M, N, K, st);
+        else launch_decode_packed_as<Act, 8, 1, 2>(x, packed, out, ep, M, N, K, st);
+    } else if (M <= 32) {
+        if (wide) launch_decode_packed_as<Act, 16, 2, 2>(x, packed, out, ep, M, N, K, st);
+        else launch_decode_packed_as<Act, 8, 2, 2>(x, packed, out, ep, M, N, K, st);
+    } else {
+        launch_decode_packed_as<Act, 8, 4, 1>(x, packed, out, ep, M, N, K, st);
+    }
+}
+
+template <typename Act, int MT>
+void launch_prefill_packed_as(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N,
+                              int K, hipStream_t st)
+{
+    using S = PackedPrefillSmem<MT>;
+    auto kernel = terna_prefill_packed_kernel<Act, MT>;
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, S::kBytes);
+    if (attr != hipSuccess) die("hipFuncSetAttribute(prefill packed)", attr, __LINE__);
+    const dim3 grid((N + kPrefillBN - 1) / kPrefillBN, (M + S::BM - 1) / S::BM);
+    kernel<<<grid, dim3(256), S::kBytes, st>>>(x, packed, out, ep, M, N, K);
+}
+
+template <typename Act>
+void launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                           hipStream_t st)
+{
+    // Largest batch tile that still gives every CU a workgroup; small problems take the smallest.
+    const int n_tiles = (N + kPrefillBN - 1) / kPrefillBN;
+    if (n_tiles * ((M + 255) / 256) >= 256) launch_prefill_packed_as<Act, 4>(x, packed, out, ep, M, N, K, st);
+    else if (n_tiles * ((M + 127) / 128) >= 256) launch_prefill_packed_as<Act, 2>(x, packed, out, ep, M, N, K, st);
+    else launch_prefill_packed_as<Act, 1>(x, packed, out, ep, M, N, K, st);
+}
+
+// Large-M call on reference-format pointers: with a 16-byte aligned workspace of N*K/4 bytes the
+// weights are first transcoded to P2 there (one cheap pass) and the P2 kernel does the GEMM;
+// without one the fused reference-format kernel runs.
+template <typename Act>
+void launch_large_m(const Act* x, const Weights& w, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                    void* workspace, hipStream_t st)
+{
+    if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
+        uint32_t* packed = static_cast<uint32_t*>(workspace);
+        launch_repack(w, packed, N, K, st);
+        launch_prefill_packed(x, packed, out, ep, M, N, K, st);
+    } else {
+        launch_prefill(x, w, out, ep, M, N, K, st);
+    }
+}
+
 enum Route { ROUTE_AUTO, ROUTE_DECODE, ROUTE_PREFILL };
 
 void run_i8(Route route, int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* median_off, uint32_t* sign_words,
-            uint16_t* out, uint16_t* s, uint16_t* ws, int ws_num, int M, int N, int K, hipStream_t st, int line)
+            uint16_t* out, uint16_t* s, uint16_t* ws, int ws_num, int M, int N, int K, void* workspace,
+            hipStream_t st, int line)
 {
     if (!shape_ok(M, N, K) || ws_num < 1) return;
     // The reference picks its path, and with it the epilogue arithmetic, by M <= 64
@@ -123,21 +198,21 @@ void run_i8(Route route, int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* m
     const Epilogue ep{s, ws, nullptr, ws_num, decode_rule ? EP_I8_DECODE : EP_I8_PREFILL};
     const Weights w{bitmap, tile_off, median_off, sign_words};
     if (M <= 64) launch_decode<int8_t>(x, w, out, ep, M, N, K, st);
-    else launch_prefill<int8_t>(x, w, out, ep, M, N, K, st);
+    else launch_large_m<int8_t>(x, w, out, ep, M, N, K, workspace, st);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("bitlinear_TernaSpMM", e, line);
 }
 
 void run_bf16(Route route, const uint16_t* x, const uint64_t* bitmap, const int* tile_off,
               const uint16_t* median_off, const uint32_t* sign_words, uint16_t* out, const float* scale,
-              int ws_num, int M, int N, int K, hipStream_t st, int line)
+              int ws_num, int M, int N, int K, void* workspace, hipStream_t st, int line)
 {
     if (!shape_ok(M, N, K) || ws_num < 1) return;
     const Epilogue ep{nullptr, nullptr, scale, ws_num, EP_BF16};
     const Weights w{bitmap, tile_off, median_off, sign_words};
     const bool small = route == ROUTE_DECODE || (route == ROUTE_AUTO && M <= 64);
     if (small) launch_decode<uint16_t>(x, w, out, ep, M, N, K, st);
-    else launch_prefill<uint16_t>(x, w, out, ep, M, N, K, st);
+    else launch_large_m<uint16_t>(x, w, out, ep, M, N, K, workspace, st);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("bitlinear_TernaSpMM_bf16", e, line);
 }
@@ -161,25 +236,25 @@ void checkLastCudaError(int line)
 
 void bitlinear_TernaSpMM(int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* median_off, uint32_t* sign_words,
                          terna_bf16* out, terna_bf16* s, terna_bf16* ws, int ws_num, int M, int N, int K,
-                         int /*SPLIT_K*/, int32_t* /*workspace*/, terna_stream stream)
+                         int /*SPLIT_K*/, int32_t* workspace, terna_stream stream)
 {
-    run_i8(ROUTE_AUTO, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K,
+    run_i8(ROUTE_AUTO, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K, workspace,
            static_cast<hipStream_t>(stream), __LINE__);
 }
 
 void bitlinear_TernaSpMM_decode(int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* median_off,
                                 uint32_t* sign_words, terna_bf16* out, terna_bf16* s, terna_bf16* ws, int ws_num,
-                                int M, int N, int K, int /*SPLIT_K*/, int32_t* /*workspace*/, terna_stream stream)
+                                int M, int N, int K, int /*SPLIT_K*/, int32_t* workspace, terna_stream stream)
 {
-    run_i8(ROUTE_DECODE, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K,
+    run_i8(ROUTE_DECODE, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K, workspace,
            static_cast<hipStream_t>(stream), __LINE__);
 }
 
 void bitlinear_TernaSpMM_prefill(int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* median_off,
                                  uint32_t* sign_words, terna_bf16* out, terna_bf16* s, terna_bf16* ws, int ws_num,
-                                 int M, int N, int K, int /*SPLIT_K*/, int32_t* /*workspace*/, terna_stream stream)
+                                 int M, int N, int K, int /*SPLIT_K*/, int32_t* workspace, terna_stream stream)
 {
-    run_i8(ROUTE_PREFILL, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K,
+    run_i8(ROUTE_PREFILL, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K, workspace,
            static_cast<hipStream_t>(stream), __LINE__);
 }
 
@@ -191,10 +266,9 @@ void bitlinear_TernaSpMM_benchmark(int mode, int warmup_iters, int bench_iters, 
     // mode 0 = auto, 1 = prefill, 2 = decode (kernels/TernaSpMM.cu:165-173)
     const Route route = mode == 1 ? ROUTE_PREFILL : (mode == 2 ? ROUTE_DECODE : ROUTE_AUTO);
     (void)SPLIT_K;
-    (void)workspace;
     hipStream_t st = static_cast<hipStream_t>(stream);
     for (int it = 0; it < warmup_iters; ++it)
-        run_i8(route, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K, st, __LINE__);
+        run_i8(route, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K, workspace, st, __LINE__);
     hipError_t e = hipStreamSynchronize(st);
     if (e != hipSuccess) die("benchmark warm-up", e, __LINE__);
 
@@ -203,7 +277,7 @@ void bitlinear_TernaSpMM_benchmark(int mode, int warmup_iters, int bench_iters, 
     if ((e = hipEventCreate(&stop)) != hipSuccess) die("hipEventCreate", e, __LINE__);
     (void)hipEventRecord(start, st);
     for (int it = 0; it < bench_iters; ++it)
-        run_i8(route, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K, st, __LINE__);
+        run_i8(route, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K, workspace, st, __LINE__);
     (void)hipEventRecord(stop, st);
     if ((e = hipEventSynchronize(stop)) != hipSuccess) die("benchmark loop", e, __LINE__);
     float total_ms = 0.0f;
@@ -257,27 +331,27 @@ void gpu_sleep(double us, terna_stream stream)
 void bitlinear_TernaSpMM_bf16(const terna_bf16* x, const uint64_t* bitmap, const int* tile_off,
                               const uint16_t* median_off, const uint32_t* sign_words, terna_bf16* out,
                               const float* scale, int ws_num, int M, int N, int K, int /*SPLIT_K*/,
-                              void* /*workspace*/, terna_stream stream)
+                              void* workspace, terna_stream stream)
 {
-    run_bf16(ROUTE_AUTO, x, bitmap, tile_off, median_off, sign_words, out, scale, ws_num, M, N, K,
+    run_bf16(ROUTE_AUTO, x, bitmap, tile_off, median_off, sign_words, out, scale, ws_num, M, N, K, workspace,
              static_cast<hipStream_t>(stream), __LINE__);
 }
 
 void bitlinear_TernaSpMM_bf16_decode(const terna_bf16* x, const uint64_t* bitmap, const int* tile_off,
                                      const uint16_t* median_off, const uint32_t* sign_words, terna_bf16* out,
                                      const float* scale, int ws_num, int M, int N, int K, int /*SPLIT_K*/,
-                                     void* /*workspace*/, terna_stream stream)
+                                     void* workspace, terna_stream stream)
 {
-    run_bf16(ROUTE_DECODE, x, bitmap, tile_off, median_off, sign_words, out, scale, ws_num, M, N, K,
+    run_bf16(ROUTE_DECODE, x, bitmap, tile_off, median_off, sign_words, out, scale, ws_num, M, N, K, workspace,
              static_cast<hipStream_t>(stream), __LINE__);
 }
 
 void bitlinear_TernaSpMM_bf16_prefill(const terna_bf16* x, const uint64_t* bitmap, const int* tile_off,
                                       const uint16_t* median_off, const uint32_t* sign_words, terna_bf16* out,
                                       const float* scale, int ws_num, int M, int N, int K, int /*SPLIT_K*/,
-                                      void* /*workspace*/, terna_stream stream)
+                                      void* workspace, terna_stream stream)
 {
-    run_bf16(ROUTE_PREFILL, x, bitmap, tile_off, median_off, sign_words, out, scale, ws_num, M, N, K,
+    run_bf16(ROUTE_PREFILL, x, bitmap, tile_off, median_off, sign_words, out, scale, ws_num, M, N, K, workspace,
              static_cast<hipStream_t>(stream), __LINE__);
 }
 
@@ -301,6 +375,50 @@ void ternaspmm_decompress_bf16(const uint64_t* bitmap, const int* tile_off, cons
         bitmap, tile_off, median_off, sign_words, W_dense, N, K);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_decompress_bf16", e, __LINE__);
+}
+
+int64_t ternaspmm_packed_bytes(int N, int K)
+{
+    if (N < 64 || K < 64 || (N % 64) || (K % 64)) return -1;
+    return static_cast<int64_t>(N) * K / 4;
+}
+
+void ternaspmm_repack(const uint64_t* bitmap, const int* tile_off, const uint16_t* median_off,
+                      const uint32_t* sign_words, void* packed, int N, int K, terna_stream stream)
+{
+    if (!shape_ok(1, N, K)) return;
+    launch_repack(Weights{bitmap, tile_off, median_off, sign_words}, static_cast<uint32_t*>(packed), N, K,
+                  static_cast<hipStream_t>(stream));
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_repack", e, __LINE__);
+}
+
+void bitlinear_TernaSpMM_bf16_packed(const terna_bf16* x, const void* packed, terna_bf16* out, const float* scale,
+                                     int ws_num, int M, int N, int K, int route, terna_stream stream)
+{
+    if (!shape_ok(M, N, K) || ws_num < 1) return;
+    const Epilogue ep{nullptr, nullptr, scale, ws_num, EP_BF16};
+    const uint32_t* p = static_cast<const uint32_t*>(packed);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool small = route == 2 || (route != 1 && M <= 64);
+    if (small) launch_decode_packed<uint16_t>(x, p, out, ep, M, N, K, st);
+    else launch_prefill_packed<uint16_t>(x, p, out, ep, M, N, K, st);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("bitlinear_TernaSpMM_bf16_packed", e, __LINE__);
+}
+
+void bitlinear_TernaSpMM_packed(const int8_t* x, const void* packed, terna_bf16* out, const terna_bf16* s,
+                                const terna_bf16* ws, int ws_num, int M, int N, int K, int route, terna_stream stream)
+{
+    if (!shape_ok(M, N, K) || ws_num < 1) return;
+    const bool decode_rule = route == 2 || (route != 1 && M <= 64);
+    const Epilogue ep{s, ws, nullptr, ws_num, decode_rule ? EP_I8_DECODE : EP_I8_PREFILL};
+    const uint32_t* p = static_cast<const uint32_t*>(packed);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (M <= 64) launch_decode_packed<int8_t>(x, p, out, ep, M, N, K, st);
+    else launch_prefill_packed<int8_t>(x, p, out, ep, M, N, K, st);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("bitlinear_TernaSpMM_packed", e, __LINE__);
 }
 
 const char* ternaspmm_version(void) { return "ternaspmm-gfx950 0.1"; }

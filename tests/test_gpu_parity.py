@@ -29,28 +29,69 @@ def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
-def run_i8(lib, fmt, xq, s_bits, ws_bits, ws_num, entry="bitlinear_TernaSpMM"):
+def _workspace(m, n, k):
+    """What the reference's call site guarantees (model.py:34-42): room for 7 int32 split-K partials
+    and for N*K bytes.  The large-M path transcodes the weights into its first N*K/4 bytes."""
+    return torch.empty(max(4 * m * n * 7, n * k) + 256, dtype=torch.int8, device="cuda")
+
+
+def run_i8(lib, fmt, xq, s_bits, ws_bits, ws_num, entry="bitlinear_TernaSpMM", workspace=True):
     m, k = xq.shape
     x = torch.from_numpy(xq).cuda()
     s = torch.from_numpy(s_bits.view(np.int16)).cuda()
     ws = torch.from_numpy(ws_bits.view(np.int16)).cuda()
     out = torch.full((m, fmt.n), -1, dtype=torch.int16, device="cuda")      # poison: must be overwritten
-    work = torch.empty(16, dtype=torch.int32, device="cuda")
-    print(f"[case] {entry} M={m} N={fmt.n} K={k} ws_num={ws_num}", flush=True)
+    work = _workspace(m, fmt.n, k) if workspace else None
+    print(f"[case] {entry} M={m} N={fmt.n} K={k} ws_num={ws_num} workspace={workspace}", flush=True)
     getattr(lib, entry)(vp(x), vp(fmt.bm), vp(fmt.off), vp(fmt.med), vp(fmt.vals), vp(out), vp(s), vp(ws),
-                        ws_num, m, fmt.n, k, 7, vp(work), _stream())
+                        ws_num, m, fmt.n, k, 7, vp(work) if workspace else None, _stream())
     torch.cuda.synchronize()
     return out.cpu().numpy().view(np.uint16)
 
 
-def run_bf16(lib, fmt, x_bits, scale, ws_num, entry="bitlinear_TernaSpMM_bf16"):
+def run_bf16(lib, fmt, x_bits, scale, ws_num, entry="bitlinear_TernaSpMM_bf16", workspace=False):
     m, k = x_bits.shape
     x = torch.from_numpy(x_bits.view(np.int16)).cuda()
     sc = torch.from_numpy(scale).cuda()
     out = torch.full((m, fmt.n), -1, dtype=torch.int16, device="cuda")
-    print(f"[case] {entry} M={m} N={fmt.n} K={k} ws_num={ws_num}", flush=True)
+    work = _workspace(m, fmt.n, k) if workspace else None
+    print(f"[case] {entry} M={m} N={fmt.n} K={k} ws_num={ws_num} workspace={workspace}", flush=True)
     getattr(lib, entry)(vp(x), vp(fmt.bm), vp(fmt.off), vp(fmt.med), vp(fmt.vals), vp(out), vp(sc), ws_num,
-                        m, fmt.n, k, 1, None, _stream())
+                        m, fmt.n, k, 1, vp(work) if workspace else None, _stream())
+    torch.cuda.synchronize()
+    return out.cpu().numpy().view(np.uint16)
+
+
+def repack(lib, fmt):
+    """Reference format -> P2 on the device."""
+    nbytes = lib.ternaspmm_packed_bytes(fmt.n, fmt.k)
+    assert nbytes == fmt.n * fmt.k // 4
+    packed = torch.full((nbytes // 4,), -1, dtype=torch.int32, device="cuda")
+    print(f"[case] ternaspmm_repack N={fmt.n} K={fmt.k}", flush=True)
+    lib.ternaspmm_repack(vp(fmt.bm), vp(fmt.off), vp(fmt.med), vp(fmt.vals), vp(packed), fmt.n, fmt.k, _stream())
+    torch.cuda.synchronize()
+    return packed
+
+
+def run_bf16_packed(lib, packed, n, x_bits, scale, ws_num, route=0):
+    m, k = x_bits.shape
+    x = torch.from_numpy(x_bits.view(np.int16)).cuda()
+    sc = torch.from_numpy(scale).cuda()
+    out = torch.full((m, n), -1, dtype=torch.int16, device="cuda")
+    print(f"[case] bitlinear_TernaSpMM_bf16_packed M={m} N={n} K={k} ws_num={ws_num} route={route}", flush=True)
+    lib.bitlinear_TernaSpMM_bf16_packed(vp(x), vp(packed), vp(out), vp(sc), ws_num, m, n, k, route, _stream())
+    torch.cuda.synchronize()
+    return out.cpu().numpy().view(np.uint16)
+
+
+def run_i8_packed(lib, packed, n, xq, s_bits, ws_bits, ws_num, route=0):
+    m, k = xq.shape
+    x = torch.from_numpy(xq).cuda()
+    s = torch.from_numpy(s_bits.view(np.int16)).cuda()
+    ws = torch.from_numpy(ws_bits.view(np.int16)).cuda()
+    out = torch.full((m, n), -1, dtype=torch.int16, device="cuda")
+    print(f"[case] bitlinear_TernaSpMM_packed M={m} N={n} K={k} ws_num={ws_num} route={route}", flush=True)
+    lib.bitlinear_TernaSpMM_packed(vp(x), vp(packed), vp(out), vp(s), vp(ws), ws_num, m, n, k, route, _stream())
     torch.cuda.synchronize()
     return out.cpu().numpy().view(np.uint16)
 
@@ -312,8 +353,11 @@ def test_int8_prefill_kernel_bit_exact(lib, m, n, k, ws_num):
     w = make_ternary(n, k, 0.40, 320 + m + n)
     fmt = DeviceFormat(w)
     xq, s = make_int8_activations(m, k, 330 + m + k)
-    got = run_i8(lib, fmt, xq, s, WS, ws_num)                      # M > 64 -> prefill rule and kernel
-    assert (got == O.spmm_i8(xq, w, s, WS, ws_num, 1)).all()
+    want = O.spmm_i8(xq, w, s, WS, ws_num, 1)
+    got = run_i8(lib, fmt, xq, s, WS, ws_num)                      # M > 64 -> prefill rule; transcode + P2 kernel
+    assert (got == want).all()
+    got_nw = run_i8(lib, fmt, xq, s, WS, ws_num, workspace=False)  # no workspace -> fused reference-format kernel
+    assert (got_nw == want).all()
     got_d = run_i8(lib, fmt, xq, s, WS, ws_num, "bitlinear_TernaSpMM_decode")
     assert (got_d == O.spmm_i8(xq, w, s, WS, ws_num, 0)).all()
 
@@ -344,3 +388,74 @@ def test_bf16_prefill_2b_layer_shapes(lib, m, n, k):
     _check_bf16(got[:, cols], ref)
     neg = run_bf16(lib, fmt, x ^ np.uint16(0x8000), scale, 1)
     _assert_negation_symmetric(got, neg)
+
+
+# ------------------------------------------------------------------------------- P2 layout (load-time repack)
+@pytest.mark.parametrize("kind", ["iid40", "skewed", "dense", "empty", "sparse97"])
+def test_repack_is_bit_exact(lib, kind):
+    """repack(encode(W)) == pack(W): the device transcoder against the oracle's packing of the
+    original matrix, and unpack(pack(W)) == W closes the round trip."""
+    n, k = 256, 320
+    w = {"iid40": lambda: make_ternary(n, k, 0.40, 1), "skewed": lambda: make_row_skewed(n, k, 3),
+         "dense": lambda: make_ternary(n, k, 0.0, 4), "empty": lambda: np.zeros((n, k), np.int8),
+         "sparse97": lambda: make_ternary(n, k, 0.97, 5)}[kind]()
+    got = repack(lib, DeviceFormat(w)).cpu().numpy().view(np.uint32)
+    assert (got == O.pack_p2(w).reshape(-1)).all()
+    assert (O.unpack_p2(got, n, k) == w).all()
+
+
+@pytest.mark.parametrize("n,k", [(13824, 2560), (2560, 6912)])
+def test_repack_full_size_round_trip(lib, n, k):
+    w = make_ternary(n, k, 0.40, seed_for(2, 50 + n % 7))
+    got = repack(lib, DeviceFormat(w)).cpu().numpy().view(np.uint32)
+    assert (O.unpack_p2(got, n, k) == w).all()
+
+
+@pytest.mark.parametrize("m", [1, 8, 16, 24, 64, 65, 128, 300])
+@pytest.mark.parametrize("n,k,ws_num", [(256, 192, 1), (640, 320, 2), (3840, 128, 3)])
+def test_packed_int8_bit_exact(lib, m, n, k, ws_num):
+    w = make_ternary(n, k, 0.40, 400 + m + n)
+    packed = repack(lib, DeviceFormat(w))
+    xq, s = make_int8_activations(m, k, 410 + m + k)
+    mode = 0 if m <= 64 else 1
+    assert (run_i8_packed(lib, packed, n, xq, s, WS, ws_num) == O.spmm_i8(xq, w, s, WS, ws_num, mode)).all()
+    assert (run_i8_packed(lib, packed, n, xq, s, WS, ws_num, 2) == O.spmm_i8(xq, w, s, WS, ws_num, 0)).all()
+    assert (run_i8_packed(lib, packed, n, xq, s, WS, ws_num, 1) == O.spmm_i8(xq, w, s, WS, ws_num, 1)).all()
+
+
+@pytest.mark.parametrize("route", [1, 2])
+@pytest.mark.parametrize("m", [1, 3, 16, 17, 64, 100, 256, 300])
+@pytest.mark.parametrize("n,k", [(256, 64), (320, 128), (512, 320)])
+def test_packed_bf16_both_kernels(lib, coracle, route, m, n, k):
+    """route 1 = MFMA-tiled kernel, route 2 = small-M kernel, each at every M."""
+    w = make_ternary(n, k, 0.40, 420 + m + n)
+    packed = repack(lib, DeviceFormat(w))
+    x = make_bf16_activations(m, k, 430 + m + k, outlier_frac=0.01)
+    scale = np.array([0.7, 1.9], np.float32)
+    _check_bf16(run_bf16_packed(lib, packed, n, x, scale, 2, route), coracle.spmm_bf16(x, w, scale, 2))
+
+
+@pytest.mark.parametrize("n,k", [(3840, 2560), (2560, 2560), (13824, 2560), (2560, 6912)])
+@pytest.mark.parametrize("m", [1, 8, 16, 256, 2048])
+def test_packed_bf16_2b_layer_shapes(lib, m, n, k):
+    w = make_ternary(n, k, 0.40, seed_for(2, n % 7))
+    packed = repack(lib, DeviceFormat(w))
+    x = make_bf16_activations(m, k, seed_for(2, 60 + m % 97), outlier_frac=0.01 if m >= 256 else 0.0)
+    scale = np.array([1.37], np.float32)
+    got = run_bf16_packed(lib, packed, n, x, scale, 1)
+    cols = np.sort(np.random.default_rng(seed_for(2, 98)).permutation(n)[:192]) if m >= 256 else np.arange(n)
+    ref = O.bf16_bits_to_f32(x).astype(np.float64) @ w[cols].astype(np.float64).T * float(scale[0])
+    _check_bf16(got[:, cols], ref)
+
+
+def test_large_m_with_workspace_matches_without(lib):
+    """The transcode-into-workspace route and the fused route compute the same sums in a different
+    order; both must sit within tolerance of the golden, and the int8 family must agree bit for bit."""
+    n, k, m = 512, 640, 200
+    w = make_ternary(n, k, 0.40, 441)
+    fmt = DeviceFormat(w)
+    x = make_bf16_activations(m, k, 442, outlier_frac=0.01)
+    scale = np.array([1.0], np.float32)
+    ref = O.spmm_bf16_golden(x, w, scale, 1)
+    _check_bf16(run_bf16(lib, fmt, x, scale, 1, workspace=True), ref)
+    _check_bf16(run_bf16(lib, fmt, x, scale, 1, workspace=False), ref)

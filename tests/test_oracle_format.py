@@ -144,3 +144,24 @@ def test_bf16_rounding_helpers(coracle):
     # ties to even: 1 + 2^-8 is halfway between 1.0 (even mantissa) and 1 + 2^-7
     assert O.f32_to_bf16_bits(np.array([1.00390625], np.float32))[0] == 0x3F80
     assert O.f32_to_bf16_bits(np.array([1.01171875], np.float32))[0] == 0x3F82
+
+
+def test_p2_pack_round_trip_and_field_positions():
+    """The library's load-time layout: unpack(pack(W)) == W, and one weight at (row, col) sets
+    exactly the 2-bit field the layout definition names."""
+    w = make_ternary(128, 192, 0.4, 51)
+    p = O.pack_p2(w)
+    assert p.shape == (8, 3, 64) and p.dtype == np.uint32 and (O.unpack_p2(p, 128, 192) == w).all()
+    rng = np.random.default_rng(52)
+    for _ in range(64):
+        row, col = int(rng.integers(0, 128)), int(rng.integers(0, 192))
+        sign = -1 if rng.random() < 0.5 else 1
+        one = np.zeros((128, 192), np.int8)
+        one[row, col] = sign
+        p = O.pack_p2(one)
+        q = col & 15
+        t, c = (q >> 1) & 1, 2 * (q >> 2) + (q & 1)
+        bit = 8 * (c & 3) + 2 * (2 * t + (c >> 2))
+        want = np.zeros_like(p)
+        want[row >> 4, col >> 6, 4 * (row & 15) + ((col >> 4) & 3)] = (3 if sign < 0 else 1) << bit
+        assert (p == want).all()
