@@ -68,6 +68,14 @@ class Matrix:
         self.n_sign_words = int(vals.numel())
         base = [t.cuda() for t in (vals, off, med, bm)]
         self.dev = [base] + [[t.clone() for t in base] for _ in range(copies - 1)]
+        # load-time repack (P2 layout), one buffer per weight copy
+        lib = T._lib.load()
+        self.packed = []
+        for vals_d, off_d, med_d, bm_d in self.dev:
+            buf = torch.empty(lib.ternaspmm_packed_bytes(n, k) // 4, dtype=torch.int32, device="cuda")
+            lib.ternaspmm_repack(vp(bm_d), vp(off_d), vp(med_d), vp(vals_d), vp(buf), n, k, None)
+            self.packed.append(buf)
+        torch.cuda.synchronize()
         rng = np.random.default_rng(seed + 1)
         self.x_bits = f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
         self.x = torch.from_numpy(self.x_bits.view(np.int16)).cuda()
@@ -78,10 +86,14 @@ class Matrix:
         self.alg_bytes = (8 * (n * k // 64) + 4 * self.n_sign_words + 4 * (n * k // 4096 + 1)
                           + 2 * (3 * n * k // 4096) + 2 * m * k + 4 + 2 * m * n)
 
-    def launch(self, lib, copy, stream):
-        vals, off, med, bm = self.dev[copy]
-        lib.bitlinear_TernaSpMM_bf16(vp(self.x), vp(bm), vp(off), vp(med), vp(vals), vp(self.out), vp(self.scale),
-                                     1, self.m, self.n, self.k, 1, None, stream)
+    def launch(self, lib, copy, stream, layout="packed"):
+        if layout == "packed":
+            lib.bitlinear_TernaSpMM_bf16_packed(vp(self.x), vp(self.packed[copy]), vp(self.out), vp(self.scale),
+                                                1, self.m, self.n, self.k, 0, stream)
+        else:
+            vals, off, med, bm = self.dev[copy]
+            lib.bitlinear_TernaSpMM_bf16(vp(self.x), vp(bm), vp(off), vp(med), vp(vals), vp(self.out), vp(self.scale),
+                                         1, self.m, self.n, self.k, 1, None, stream)
 
 
 def time_graph(torch, graph, replays, warmup):
@@ -176,11 +188,16 @@ def run_prefill(args, torch, T, lib):
                      torch.zeros((m, n), dtype=torch.int16, device="cuda"))
         mats.append((mt, xs))
 
+    work = torch.empty(13824 * 2560, dtype=torch.int8, device="cuda")      # the reference's global workspace
+
     def launch(mt, xs, m, s):
         x, out = xs[m]
-        vals, off, med, bm = mt.dev[0]
-        lib.bitlinear_TernaSpMM_bf16(vp(x), vp(bm), vp(off), vp(med), vp(vals), vp(out), vp(mt.scale),
-                                     1, m, mt.n, mt.k, 1, None, s)
+        if args.layout == "packed":
+            lib.bitlinear_TernaSpMM_bf16_packed(vp(x), vp(mt.packed[0]), vp(out), vp(mt.scale), 1, m, mt.n, mt.k, 0, s)
+        else:                      # reference-format pointers + workspace: transcode per call, then the P2 kernel
+            vals, off, med, bm = mt.dev[0]
+            lib.bitlinear_TernaSpMM_bf16(vp(x), vp(bm), vp(off), vp(med), vp(vals), vp(out), vp(mt.scale),
+                                         1, m, mt.n, mt.k, 1, vp(work), s)
 
     per_shape = {}
     for mt, xs in mats:
@@ -211,10 +228,13 @@ def run_prefill(args, torch, T, lib):
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": f"configs[2]: four BitNet-b1.58-2B matrices at M={m_main}, P(0)=0.40, bf16 activations "
-                               "with 1% outlier channels (x20), HIP-graph replay", "m": m_main},
+                               "with 1% outlier channels (x20), HIP-graph replay; weight layout: "
+                               + ("P2, repacked once at load time" if args.layout == "packed"
+                                  else "reference format, transcoded into the workspace on every call"),
+                   "m": m_main, "layout": args.layout},
         "roofline": {"bound": "mfma", "achieved": tf, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": tf / BF16_MFMA_PEAK_TFLOPS, "traffic": None,
-                     "kernel": "terna_prefill_kernel<bf16>", "algorithmic_flops_per_step": flops},
+                     "kernel": "terna_prefill_packed_kernel<bf16>", "algorithmic_flops_per_step": flops},
         "per_shape": per_shape}))
 
 
@@ -227,6 +247,9 @@ def main():
     ap.add_argument("--layers", type=int, default=30, help="distinct weight copies per matrix")
     ap.add_argument("--workload", choices=["decode", "prefill"], default="decode",
                     help="decode: the headline small-M HBM-bound pass; prefill: the M>=256 MFMA-bound pass")
+    ap.add_argument("--layout", choices=["packed", "reference"], default="packed",
+                    help="packed: weights repacked once at load time to the library's P2 layout (bit-exact); "
+                         "reference: kernels read the reference's compressed format directly")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-per-shape", action="store_true")
     args = ap.parse_args()
@@ -250,10 +273,10 @@ def main():
     step_bytes = args.layers * sum(mt.alg_bytes for mt in mats)
     launches_per_step = args.layers * len(mats)
 
-    def step(stream):
+    def step(stream, layout=args.layout):
         for layer in range(args.layers):
             for mt in mats:
-                mt.launch(lib, layer, stream)
+                mt.launch(lib, layer, stream, layout)
 
     # eager pass first (loads code objects, fills outputs for the correctness gate)
     step(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
@@ -281,12 +304,15 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": (f"configs[1]: BitNet-b1.58-2B decode layer set (QKV 2560->3840, O 2560->2560, "
                                 f"gate+up 2560->13824, down 6912->2560), M={args.m}, P(0)=0.40, bf16 activations, "
-                                f"{args.layers} layers with distinct weight copies (cold stream), HIP-graph replay"),
-                   "m": args.m, "layers": args.layers, "launches_per_step": launches_per_step,
+                                f"{args.layers} layers with distinct weight copies (cold stream), HIP-graph replay; weight layout: "
+                                + ("P2, repacked once at load time from the reference format" if args.layout == "packed"
+                                   else "reference format read directly")),
+                   "m": args.m, "layers": args.layers, "layout": args.layout, "launches_per_step": launches_per_step,
                    "algorithmic_bytes_per_step": step_bytes},
         "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": gbps / HBM_PEAK_GBPS, "traffic": TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "terna_decode_kernel<bf16, 8 waves, 1 m-block>",
+                     "kernel": ("terna_decode_packed_kernel<bf16>" if args.layout == "packed"
+                                else "terna_decode_kernel<bf16>"),
                      "algorithmic_bytes_per_launch": step_bytes / launches_per_step,
                      "avg_launch_us": launch_us},
         "tokens_per_s_linear_layers_only": args.m / (ms_per_step * 1e-3) if args.layers == 30 else None,
@@ -296,14 +322,17 @@ def main():
     if not args.no_per_shape:
         shapes = {}
         for mt in mats:
-            cold = capture(torch, lambda s, mt=mt: [mt.launch(lib, c, s) for c in range(args.layers)])
-            hot = capture(torch, lambda s, mt=mt: [mt.launch(lib, 0, s) for _ in range(args.layers)])
+            cold = capture(torch, lambda s, mt=mt: [mt.launch(lib, c, s, args.layout) for c in range(args.layers)])
+            hot = capture(torch, lambda s, mt=mt: [mt.launch(lib, 0, s, args.layout) for _ in range(args.layers)])
+            other = "reference" if args.layout == "packed" else "packed"
+            alt = capture(torch, lambda s, mt=mt: [mt.launch(lib, c, s, other) for c in range(args.layers)])
             cold_us = time_graph(torch, cold, 20, 3) * 1e3 / args.layers
             hot_us = time_graph(torch, hot, 20, 3) * 1e3 / args.layers
+            alt_us = time_graph(torch, alt, 20, 3) * 1e3 / args.layers
             shapes[f"{mt.name}_{mt.k}x{mt.n}"] = {
                 "alg_bytes": mt.alg_bytes, "cold_us": cold_us, "cold_GBps": mt.alg_bytes / cold_us / 1e3,
                 "cold_frac": mt.alg_bytes / cold_us / 1e3 / HBM_PEAK_GBPS,
-                "hot_us": hot_us, "hot_GBps": mt.alg_bytes / hot_us / 1e3,
+                "hot_us": hot_us, "hot_GBps": mt.alg_bytes / hot_us / 1e3, f"cold_us_{other}_layout": alt_us,
                 "tflops": 2.0 * mt.m * mt.n * mt.k / cold_us / 1e6}
         result["per_shape"] = shapes
 

@@ -194,11 +194,14 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
     const LaneGeom q(lane);
     const int i = q.i, g = q.g, b0 = q.b0;
 
+    // Lanes whose batch row does not exist load nothing (zero operand, output never stored).
     int xrow[MB];
+    bool x_ok[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
         const int m = m_base + mb * 16 + i;
-        xrow[mb] = m < M ? m : M - 1;       // rows past M repeat the last one; never stored
+        x_ok[mb] = m < M;
+        xrow[mb] = x_ok[mb] ? m : 0;
     }
 
     Acc acc[MB];
@@ -240,7 +243,8 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
         for (int mb = 0; mb < MB; ++mb) {
             const Act* xp = x + static_cast<size_t>(xrow[mb]) * K + gk * 64 + g * 16;
 #pragma unroll
-            for (int v = 0; v < T::kXVecs; ++v) raw.x[mb][v] = reinterpret_cast<const u32x4*>(xp)[v];
+            for (int v = 0; v < T::kXVecs; ++v)
+                raw.x[mb][v] = x_ok[mb] ? reinterpret_cast<const u32x4*>(xp)[v] : u32x4{0u, 0u, 0u, 0u};
         }
     };
     // The sign window: needs the band-tile's stream offset.

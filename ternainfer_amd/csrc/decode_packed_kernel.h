@@ -13,10 +13,30 @@
 
 namespace terna {
 
+// Activations reach the MFMA B operand through a wave-private LDS slot.  The operand wants lane
+// (m = L & 15, g = L >> 4) to hold 32 bytes of batch row m -- sixteen different rows in sixteen
+// adjacent lanes, which a global load can only serve one cache line per lane.  So the wave loads
+// its [16 rows][64 columns] slab the other way round (adjacent lanes walk along a row: 8 lanes per
+// 128-byte row segment, fully coalesced), drops it into LDS with a padded row pitch, and reads
+// it back in operand order; both LDS accesses are bank-conflict free.
+template <typename Act> struct XSlab;
+template <> struct XSlab<uint16_t> {              // bf16: a row segment is 128 B = 8 lanes x 16 B
+    static constexpr int kPitch = 144, kLoads = 2;   // two loads: rows 0-7 and rows 8-15
+    __device__ static int row_of(int lane, int h) { return 8 * h + (lane >> 3); }
+    __device__ static int col_of(int lane) { return (lane & 7) * 8; }             // in elements
+    __device__ static int write_off(int lane, int h) { return row_of(lane, h) * kPitch + (lane & 7) * 16; }
+};
+template <> struct XSlab<int8_t> {                // int8: a row segment is 64 B = 4 lanes x 16 B
+    static constexpr int kPitch = 80, kLoads = 1;    // one load covers all 16 rows
+    __device__ static int row_of(int lane, int) { return lane >> 2; }
+    __device__ static int col_of(int lane) { return (lane & 3) * 16; }
+    __device__ static int write_off(int lane, int) { return (lane >> 2) * kPitch + (lane & 3) * 16; }
+};
+
 template <typename Act, int MB>
 struct PackedRaw {
-    uint32_t word;                          // 16 weights: row (L & 15), 16-column group (L >> 4)
-    u32x4    x[MB][ActTraits<Act>::kXVecs]; // activation bytes of (batch row L & 15, group L >> 4)
+    uint32_t word;                           // 16 weights: row (L & 15), 16-column group (L >> 4)
+    u32x4    x[MB][XSlab<Act>::kLoads];      // coalesced pieces of the activation slab
 };
 
 template <typename Act, int WAVES, int MB, int DEPTH>
@@ -27,68 +47,81 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
     using T = ActTraits<Act>;
     using Acc = typename T::Acc;
     using Raw = PackedRaw<Act, MB>;
+    using XS = XSlab<Act>;
     constexpr int NBUF = DEPTH + 1;
     static_assert(DEPTH >= 1 && DEPTH <= 3, "prefetch distance");
 
     __shared__ Acc red[WAVES][MB][64];
+    __shared__ __align__(16) uint8_t xslab_all[WAVES][MB][16 * XS::kPitch];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    TERNA_TS(0);
     const int band = blockIdx.x;
     const int m_base = blockIdx.y * (16 * MB);
     const int ktiles = K >> 6;
     const int i = lane & 15, g = lane >> 4;
 
     const uint32_t* wp = packed + (static_cast<size_t>(band) * ktiles + wave) * 64 + i * 4 + g;
-    const Act* xp[MB];
+    // Coalesced activation pieces of this lane; rows past M are not loaded (their operand is zero
+    // and their output column is never stored).
+    const Act* xp[MB][XS::kLoads];
+    bool x_ok[MB][XS::kLoads];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-        const int m = m_base + mb * 16 + i;
-        xp[mb] = x + static_cast<size_t>(m < M ? m : M - 1) * K + wave * 64 + g * 16;   // rows past M repeat the last
-    }
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int h = 0; h < XS::kLoads; ++h) {
+            const int m = m_base + mb * 16 + XS::row_of(lane, h);
+            x_ok[mb][h] = m < M;
+            xp[mb][h] = x + static_cast<size_t>(x_ok[mb][h] ? m : 0) * K + wave * 64 + XS::col_of(lane);
+        }
 
     const int cnt = ktiles > wave ? (ktiles - wave + WAVES - 1) / WAVES : 0;   // this wave's band-tiles
+#ifdef TERNA_TS_ENABLED
+    if (reinterpret_cast<uintptr_t>(wp) == 1 || cnt < -1) return;   // force the kernarg wait before the stamp
+    TERNA_TS(2);
+#endif
     auto fetch = [&](int j, Raw& raw) {
         raw.word = wp[static_cast<size_t>(j) * (WAVES * 64)];
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-            const u32x4* p = reinterpret_cast<const u32x4*>(xp[mb] + static_cast<size_t>(j) * (WAVES * 64));
+        for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-            for (int v = 0; v < T::kXVecs; ++v) raw.x[mb][v] = p[v];
-        }
+            for (int h = 0; h < XS::kLoads; ++h) {
+                const u32x4* p = reinterpret_cast<const u32x4*>(xp[mb][h] + static_cast<size_t>(j) * (WAVES * 64));
+                raw.x[mb][h] = x_ok[mb][h] ? *p : u32x4{0u, 0u, 0u, 0u};
+            }
     };
 
     Acc acc[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[mb] = Acc{0, 0, 0, 0};
 
-    // Wave w finishes m-block w (and w + WAVES, ...): fetch that block's scale factors now.
-    const int n0 = band * 16 + 4 * g;
-    EpilogueRegs eregs[(MB + WAVES - 1) / WAVES];
-#pragma unroll
-    for (int e = 0; e < (MB + WAVES - 1) / WAVES; ++e) {
-        const int m = m_base + (wave + e * WAVES) * 16 + i;
-        eregs[e] = load_epilogue(ep, m < M ? m : M - 1, n0, N);
-    }
-
+    uint8_t* slab = xslab_all[wave][0];
     auto process = [&](const Raw& cur) {
+        // slab in (coalesced order), operands out (MFMA order); same wave, so LDS ordering suffices
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int h = 0; h < XS::kLoads; ++h)
+                *reinterpret_cast<u32x4*>(slab + mb * (16 * XS::kPitch) + XS::write_off(lane, h)) = cur.x[mb][h];
         if constexpr (sizeof(Act) == 2) {
+            const bf16x8 a0 = __builtin_bit_cast(bf16x8, expand_chunk_bf16(cur.word));
+            const bf16x8 a1 = __builtin_bit_cast(bf16x8, expand_chunk_bf16(cur.word >> 4));
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                const bf16x8 a = __builtin_bit_cast(bf16x8, expand_chunk_bf16(cur.word >> (4 * t)));
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb) {
-                    const u32x4 x0 = cur.x[mb][0], x1 = cur.x[mb][1];
-                    const u32x4 b_bits = t == 0 ? u32x4{x0.x, x0.z, x1.x, x1.z} : u32x4{x0.y, x0.w, x1.y, x1.w};
-                    acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, b_bits), acc[mb], 0, 0, 0);
-                }
+            for (int mb = 0; mb < MB; ++mb) {
+                const uint8_t* src = slab + mb * (16 * XS::kPitch) + i * XS::kPitch + g * 32;
+                const u32x4 x0 = *reinterpret_cast<const u32x4*>(src);
+                const u32x4 x1 = *reinterpret_cast<const u32x4*>(src + 16);
+                const u32x4 b0 = {x0.x, x0.z, x1.x, x1.z}, b1 = {x0.y, x0.w, x1.y, x1.w};
+                acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, __builtin_bit_cast(bf16x8, b0), acc[mb], 0, 0, 0);
+                acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, __builtin_bit_cast(bf16x8, b1), acc[mb], 0, 0, 0);
             }
         } else {
             const i32x4 a = expand_word_i8(cur.word);
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
-                const u32x4 xv = cur.x[mb][0];       // dword j = columns 4j .. 4j+3
+                const u32x4 xv = *reinterpret_cast<const u32x4*>(slab + mb * (16 * XS::kPitch) + i * XS::kPitch + g * 16);
                 const i32x4 b = {
                     static_cast<int>(__builtin_amdgcn_perm(xv.y, xv.x, 0x05040100u)),   // t=0, c=0..3
                     static_cast<int>(__builtin_amdgcn_perm(xv.w, xv.z, 0x05040100u)),   // t=0, c=4..7
@@ -105,11 +138,24 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
         if (j < cnt) {
             if (j + DEPTH < cnt) fetch(j + DEPTH, pre);
             process(cur);
+            TERNA_TS(3 + (j < 5 ? j : 5));
         }
     };
     if (0 < cnt) fetch(0, ring0);
     if (DEPTH >= 2 && 1 < cnt) fetch(1, ring1);
     if (DEPTH >= 3 && 2 < cnt) fetch(2, ring2);
+    TERNA_TS(1);
+
+    // Wave w finishes m-block w (and w + WAVES, ...): with the data loads in flight, fetch that
+    // block's scale factors so that no global load sits between the last MFMA and the store.
+    const int n0 = band * 16 + 4 * g;
+    EpilogueRegs eregs[(MB + WAVES - 1) / WAVES];
+#pragma unroll
+    for (int e = 0; e < (MB + WAVES - 1) / WAVES; ++e) {
+        const int m = m_base + (wave + e * WAVES) * 16 + i;
+        eregs[e] = load_epilogue(ep, m < M ? m : M - 1, n0, N);
+    }
+
     for (int j0 = 0; j0 < cnt; j0 += NBUF) {
         if constexpr (DEPTH == 3) {
             slot(j0, ring0, ring3);
@@ -130,7 +176,9 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
     // output rows 4*(L>>4) .. +3 of column L & 15).  bf16 weights were +-0.5: undo with an exact x2.
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) red[wave][mb][lane] = acc[mb];
+    TERNA_TS(9);
     __syncthreads();
+    TERNA_TS(10);
 #pragma unroll
     for (int e = 0; e < (MB + WAVES - 1) / WAVES; ++e) {
         const int mb = wave + e * WAVES;
@@ -150,6 +198,7 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
             *reinterpret_cast<u32x2*>(out + static_cast<size_t>(m) * N + n0) = pk;
         }
     }
+    TERNA_TS(11);
 }
 
 }  // namespace terna

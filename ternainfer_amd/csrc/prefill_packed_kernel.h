@@ -4,15 +4,16 @@
 //
 //   out[m][n] = epilogue( 2 * sum_k X[m][k] * Whalf[n][k] ),   Whalf = W / 2 in {-0.5, 0, +0.5}
 //
-// Tiling.  One workgroup (4 waves, 2 (n) x 2 (m)) owns 256 output features x 64*MT batch rows and
-// walks K in steps of 64.  A wave owns 128 x 32*MT outputs as 4 x MT accumulator tiles of
-// v_mfma_f32_32x32x16_bf16, W as the A operand.  A-operand lane (row = L%32, kb = L/32) of
-// accumulator row-tile a needs, for 16-column group g, the eight weights of byte pair t = kb of
-// packed word (band, gk, i, g): the four words g = 0..3 of a row are adjacent, so one 16-byte
-// load per row-tile and k-step brings everything the lane needs, and ten VALU ops turn each word
-// into an operand.  Only the activation tile goes through LDS (two stages, chunk order
-// [g][sm][row], see the reference-format kernel), staged one k-step ahead; global loads of both
-// operands run two k-steps ahead.
+// Tiling.  One workgroup (4 waves) owns 256 output features x BM = 32*MB batch rows and walks K in
+// steps of 64.  The waves split the output features only: wave w owns rows 64w .. 64w+63 and ALL
+// BM batch rows, i.e. 2 x MB accumulator tiles of v_mfma_f32_32x32x16_bf16 with W as the A
+// operand -- so every weight is expanded exactly once per workgroup, and one expansion (ten VALU
+// ops) feeds MB matrix instructions.  A-operand lane (row = L%32, kb = L/32) of row-tile a needs,
+// for 16-column group g, the eight weights of byte pair t = kb of packed word (band, gk, i, g): the
+// four words g = 0..3 of a row are adjacent, so one 16-byte load per row-tile and k-step brings
+// everything the lane needs.  Only the activation tile goes through LDS (two stages, chunk order
+// [g][sm][row], see the reference-format kernel), staged one k-step ahead; B operands are read one
+// group ahead of the MFMAs that use them; weight registers are refilled two k-steps ahead.
 #pragma once
 
 #include "packed_common.h"
@@ -20,40 +21,40 @@
 
 namespace terna {
 
-template <int MT>
+template <int MB>
 struct PackedPrefillSmem {
-    static constexpr int BM = 64 * MT;
+    static constexpr int BM = 32 * MB;
     static constexpr int PX = BM * 16 + 16;           // bytes between chunk rows of the X tile (padded)
     static constexpr int kStage = 8 * PX;
     static constexpr int kBytes = 2 * kStage;
 };
 
-template <typename Act, int MT>
-__global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void terna_prefill_packed_kernel(
+template <typename Act, int MB>
+__global__ __launch_bounds__(256, MB == 8 ? 1 : 2) void terna_prefill_packed_kernel(
     const Act* __restrict__ x, const uint32_t* __restrict__ packed, uint16_t* __restrict__ out,
     Epilogue ep, int M, int N, int K)
 {
     using T = ActTraits<Act>;
-    using S = PackedPrefillSmem<MT>;
+    using S = PackedPrefillSmem<MB>;
     constexpr int BN = kPrefillBN, BM = S::BM, PX = S::PX;
-    constexpr int XI = MT;                            // (row, group) activation items per thread and k-step
+    constexpr int XI = BM / 64;                       // (row, group) activation items per thread and k-step
+    static_assert(MB == 2 || MB == 4 || MB == 8, "batch tile of 64, 128 or 256 rows");
 
     extern __shared__ __align__(16) uint8_t smem[];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wn = wave & 1, wm = wave >> 1;
     const int n0 = blockIdx.x * BN, m0 = blockIdx.y * BM;
     const int ktiles = K >> 6;
     const int last_band = (N >> 4) - 1;
     const int kb = lane >> 5, l32 = lane & 31;
 
-    // ---- weight words of this lane: row-tile a -> band (n0/16 + 8*wn + 2a + l32/16), row i = l32 % 16
-    const u32x4* w_ptr[4];
+    // ---- weight words of this lane: row-tile a -> band (n0/16 + 4*wave + 2a + l32/16), row i = l32 % 16
+    const u32x4* w_ptr[2];                             // running: advanced one k-step per fetch
 #pragma unroll
-    for (int a = 0; a < 4; ++a) {
-        int band = (n0 >> 4) + 8 * wn + 2 * a + (l32 >> 4);
+    for (int a = 0; a < 2; ++a) {
+        int band = (n0 >> 4) + 4 * wave + 2 * a + (l32 >> 4);
         band = band < last_band ? band : last_band;   // a tile hanging over N re-reads the last band; never stored
         w_ptr[a] = reinterpret_cast<const u32x4*>(packed + (static_cast<size_t>(band) * ktiles) * 64 + (l32 & 15) * 4);
     }
@@ -70,18 +71,23 @@ __global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void terna_prefill_packed_ker
         x_ptr[it] = x + static_cast<size_t>(m) * K + g * 16;
     }
 
-    struct RawW { u32x4 w[4]; };                      // [a] -> words g = 0..3
+    struct RawW { u32x4 w[2]; };                      // [a] -> words g = 0..3
     struct RawX { u32x4 x[XI][T::kXVecs]; };
-    auto fetch_w = [&](int gk, RawW& r) {
+    // Both fetches walk running pointers: one k-step is 16 u32x4 of weights and 64 activations.
+    auto fetch_w = [&](RawW& r) {
 #pragma unroll
-        for (int a = 0; a < 4; ++a) r.w[a] = w_ptr[a][static_cast<size_t>(gk) * 16];
+        for (int a = 0; a < 2; ++a) {
+            r.w[a] = *w_ptr[a];
+            w_ptr[a] += 16;
+        }
     };
-    auto fetch_x = [&](int gk, RawX& r) {
+    auto fetch_x = [&](RawX& r) {
 #pragma unroll
         for (int it = 0; it < XI; ++it) {
-            const u32x4* p = reinterpret_cast<const u32x4*>(x_ptr[it] + gk * 64);
+            const u32x4* p = reinterpret_cast<const u32x4*>(x_ptr[it]);
 #pragma unroll
             for (int v = 0; v < T::kXVecs; ++v) r.x[it][v] = p[v];
+            x_ptr[it] += 64;
         }
     };
     auto stage_x = [&](const RawX& r, int st) {
@@ -101,78 +107,96 @@ __global__ __launch_bounds__(256, MT == 4 ? 1 : 2) void terna_prefill_packed_ker
         }
     };
 
-    f32x16 acc[4][MT];
+    f32x16 acc[2][MB];
     {
         const f32x16 zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int a = 0; a < 4; ++a)
+        for (int a = 0; a < 2; ++a)
 #pragma unroll
-            for (int b = 0; b < MT; ++b) acc[a][b] = zero;
+            for (int b = 0; b < MB; ++b) acc[a][b] = zero;
     }
 
-    const int b_off = kb * PX + (32 * MT * wm + l32) * 16;   // + g*2*PX + b*512
+    const int b_off = kb * PX + l32 * 16;                    // + g*2*PX + b*512
     const int wshift = 4 * kb;                               // byte pair t = kb of every word
 
-    // One k-step: for each 16-column group g, expand the four A operands from registers, read the
-    // MT B operands from the current X stage, and issue 4*MT MFMAs.
+    struct BOps { bf16x8 b[MB]; };
+    auto load_b = [&](int st, int g, BOps& r) {
+        const uint8_t* xs = smem + st * S::kStage + b_off + g * 2 * PX;
+#pragma unroll
+        for (int b = 0; b < MB; ++b) r.b[b] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(xs + b * 512));
+    };
+    // One k-step: for each 16-column group g, expand the two A operands from registers and issue
+    // 2*MB MFMAs against B operands that were read from LDS one group earlier.
     auto mma_step = [&](const RawW& rw, int st) {
-        const uint8_t* xs = smem + st * S::kStage;
+        BOps bcur;
+        load_b(st, 0, bcur);
         static_for<0, 4>([&](auto gc) {
             constexpr int g = decltype(gc)::value;
-            bf16x8 bfr[MT];
+            BOps bnxt;
+            if constexpr (g < 3) load_b(st, g + 1, bnxt);
 #pragma unroll
-            for (int b = 0; b < MT; ++b)
-                bfr[b] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(xs + b_off + g * 2 * PX + b * 512));
-#pragma unroll
-            for (int a = 0; a < 4; ++a) {
+            for (int a = 0; a < 2; ++a) {
                 const bf16x8 af = __builtin_bit_cast(bf16x8, expand_chunk_bf16(rw.w[a][g] >> wshift));
 #pragma unroll
-                for (int b = 0; b < MT; ++b)
-                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bfr[b], acc[a][b], 0, 0, 0);
+                for (int b = 0; b < MB; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bcur.b[b], acc[a][b], 0, 0, 0);
             }
+            if constexpr (g < 3) bcur = bnxt;
         });
     };
 
-    // ---- pipeline: global loads two k-steps ahead; X staged one k-step ahead (double-buffered LDS)
-    RawW w_cur, w_nxt;
+    // ---- pipeline.  Two weight buffers: w0 serves even k-steps, w1 odd ones; each is refilled
+    // for k + 2 as soon as step k has consumed it, so its loads have a whole k-step to land.
+    // Activations: raw registers hold step k + 1 while LDS stage (k & 1) feeds the MFMAs of step k.
+    RawW w0, w1;
     RawX x_raw;
-    fetch_w(0, w_cur);
-    fetch_x(0, x_raw);
+    fetch_w(w0);
+    fetch_x(x_raw);
     stage_x(x_raw, 0);
     if (ktiles > 1) {
-        fetch_w(1, w_nxt);
-        fetch_x(1, x_raw);
+        fetch_w(w1);
+        fetch_x(x_raw);
     }
     __syncthreads();
-    for (int k = 0; k < ktiles; ++k) {
-        const int st = k & 1;
-        if (k + 1 < ktiles) stage_x(x_raw, st ^ 1);       // k+1 activations -> other stage
-        RawW w_nn;
-        if (k + 2 < ktiles) {
-            fetch_w(k + 2, w_nn);
-            fetch_x(k + 2, x_raw);
-        }
-        mma_step(w_cur, st);
-        w_cur = w_nxt;
-        w_nxt = w_nn;
+    // k-step k with both look-aheads in range (k + 2 < ktiles)
+    auto body_full = [&](int k, RawW& w) {
+        stage_x(x_raw, (k + 1) & 1);
+        fetch_x(x_raw);
+        mma_step(w, k & 1);
+        fetch_w(w);
         __syncthreads();
+    };
+    auto body_tail = [&](int k, RawW& w) {
+        if (k + 1 < ktiles) stage_x(x_raw, (k + 1) & 1);
+        if (k + 2 < ktiles) fetch_x(x_raw);
+        mma_step(w, k & 1);
+        if (k + 2 < ktiles) fetch_w(w);
+        __syncthreads();
+    };
+    int k = 0;
+    for (; k + 3 < ktiles; k += 2) {
+        body_full(k, w0);
+        body_full(k + 1, w1);
     }
+    if (k < ktiles) body_tail(k++, w0);
+    if (k < ktiles) body_tail(k++, w1);
+    if (k < ktiles) body_tail(k++, w0);
 
     // ---- epilogue: lane holds, per accumulator tile, column m = l32 and rows n = (v&3) + 8(v>>2) + 4kb.
     // The accumulator is half the true sum (weights were +-0.5); x2 is exact.
-    EpilogueRegs e[MT];
-    int m_of[MT];
-    static_for<0, MT>([&](auto bc) {
+    EpilogueRegs e[MB];
+    int m_of[MB];
+    static_for<0, MB>([&](auto bc) {
         constexpr int b = decltype(bc)::value;
-        m_of[b] = m0 + 32 * MT * wm + 32 * b + l32;
+        m_of[b] = m0 + 32 * b + l32;
         e[b].s = ep.kind == EP_BF16 ? 1.0f : bf16_bits_to_float(ep.s[m_of[b] < M ? m_of[b] : M - 1]);
     });
-    static_for<0, 16>([&](auto tc) {
+    static_for<0, 8>([&](auto tc) {
         constexpr int a = decltype(tc)::value >> 2, vq = decltype(tc)::value & 3;
-        const int n = n0 + 128 * wn + 32 * a + 8 * vq + 4 * kb;
+        const int n = n0 + 64 * wave + 32 * a + 8 * vq + 4 * kb;
         float wv[4];
         load_col_scales(ep, n < N ? n : N - 4, N, wv);
-        static_for<0, MT>([&](auto bc) {
+        static_for<0, MB>([&](auto bc) {
             constexpr int b = decltype(bc)::value;
             EpilogueRegs eb = e[b];
 #pragma unroll

@@ -101,19 +101,8 @@ __device__ __forceinline__ void load_col_scales(const Epilogue& ep, int n0, int 
 __device__ __forceinline__ EpilogueRegs load_epilogue(const Epilogue& ep, int m, int n0, int N)
 {
     EpilogueRegs r;
-    r.s = 1.0f;
-    if (ep.kind == EP_BF16) {
-#pragma unroll
-        for (int v = 0; v < 4; ++v) r.w[v] = ep.scale[ws_group_decode(n0 + v, N, ep.ws_num)];
-    } else {
-        r.s = bf16_bits_to_float(ep.s[m]);
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            const int g = ep.kind == EP_I8_DECODE ? ws_group_decode(n0 + v, N, ep.ws_num)
-                                                  : ws_group_prefill(n0 + v, N, ep.ws_num);
-            r.w[v] = bf16_bits_to_float(ep.ws[g]);
-        }
-    }
+    r.s = ep.kind == EP_BF16 ? 1.0f : bf16_bits_to_float(ep.s[m]);
+    load_col_scales(ep, n0, N, r.w);
     return r;
 }
 

@@ -145,12 +145,12 @@ void launch_decode_packed(const Act* x, const uint32_t* packed, uint16_t* out, c
     }
 }
 
-template <typename Act, int MT>
+template <typename Act, int MB>
 void launch_prefill_packed_as(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N,
                               int K, hipStream_t st)
 {
-    using S = PackedPrefillSmem<MT>;
-    auto kernel = terna_prefill_packed_kernel<Act, MT>;
+    using S = PackedPrefillSmem<MB>;
+    auto kernel = terna_prefill_packed_kernel<Act, MB>;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, S::kBytes);
     if (attr != hipSuccess) die("hipFuncSetAttribute(prefill packed)", attr, __LINE__);
@@ -162,11 +162,18 @@ template <typename Act>
 void launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
                            hipStream_t st)
 {
-    // Largest batch tile that still gives every CU a workgroup; small problems take the smallest.
-    const int n_tiles = (N + kPrefillBN - 1) / kPrefillBN;
-    if (n_tiles * ((M + 255) / 256) >= 256) launch_prefill_packed_as<Act, 4>(x, packed, out, ep, M, N, K, st);
-    else if (n_tiles * ((M + 127) / 128) >= 256) launch_prefill_packed_as<Act, 2>(x, packed, out, ep, M, N, K, st);
-    else launch_prefill_packed_as<Act, 1>(x, packed, out, ep, M, N, K, st);
+    // Batch rows per workgroup (64 / 128 / 256).  Measured on MI355X the 64-row tile wins at every
+    // BitNet-2B shape: it runs four waves per SIMD, and occupancy hides more latency than the taller
+    // tiles save in weight expansion.  TERNASPMM_PREFILL_BM=64|128|256 forces one (tuning aid).
+    static const int forced = [] {
+        const char* v = std::getenv("TERNASPMM_PREFILL_BM");
+        const int bm = v ? std::atoi(v) : 0;
+        return (bm == 64 || bm == 128 || bm == 256) ? bm : 0;
+    }();
+    const int bm = forced ? forced : 64;
+    if (bm == 256) launch_prefill_packed_as<Act, 8>(x, packed, out, ep, M, N, K, st);
+    else if (bm == 128) launch_prefill_packed_as<Act, 4>(x, packed, out, ep, M, N, K, st);
+    else launch_prefill_packed_as<Act, 2>(x, packed, out, ep, M, N, K, st);
 }
 
 // Large-M call on reference-format pointers: with a 16-byte aligned workspace of N*K/4 bytes the
