@@ -49,6 +49,26 @@ template <> struct ActTraits<int8_t> {          // int8 activations, int32 accum
     __device__ static Lut make_lut(int e) { return make_lut_i8(e); }
 };
 
+// Activations reach the MFMA B operand through a wave-private LDS slot.  The operand wants lane
+// (m = L & 15, g = L >> 4) to hold 32 bytes of batch row m -- sixteen different rows in sixteen
+// adjacent lanes, which a global load can only serve one cache line per lane.  So a wave loads
+// its [16 rows][64 columns] slab the other way round (adjacent lanes walk along a row: 8 lanes per
+// 128-byte row segment, fully coalesced), drops it into LDS with a padded row pitch, and reads
+// it back in operand order; both LDS accesses are bank-conflict free.
+template <typename Act> struct XSlab;
+template <> struct XSlab<uint16_t> {              // bf16: a row segment is 128 B = 8 lanes x 16 B
+    static constexpr int kPitch = 144, kLoads = 2;   // two loads: rows 0-7 and rows 8-15
+    __device__ static int row_of(int lane, int h) { return 8 * h + (lane >> 3); }
+    __device__ static int col_of(int lane) { return (lane & 7) * 8; }             // in elements
+    __device__ static int write_off(int lane, int h) { return row_of(lane, h) * kPitch + (lane & 7) * 16; }
+};
+template <> struct XSlab<int8_t> {                // int8: a row segment is 64 B = 4 lanes x 16 B
+    static constexpr int kPitch = 80, kLoads = 1;    // one load covers all 16 rows
+    __device__ static int row_of(int lane, int) { return lane >> 2; }
+    __device__ static int col_of(int lane) { return (lane & 3) * 16; }
+    __device__ static int write_off(int lane, int) { return (lane >> 2) * kPitch + (lane & 3) * 16; }
+};
+
 __device__ __forceinline__ int row16_inclusive_scan(int v)
 {
     // Inclusive prefix sum inside each row of 16 lanes: row_shr:n with bound_ctrl (zeros shifted in).
@@ -157,7 +177,7 @@ __device__ __forceinline__ void band_tile_indices_win(const LaneGeom& q, const u
 template <typename Act, int MB>
 struct BandTileRaw {
     uint64_t bm[2];                         // bitmaps 4g + 2sk + t
-    u32x4    x[MB][ActTraits<Act>::kXVecs]; // activation bytes of (row, group g)
+    u32x4    x[MB][XSlab<Act>::kLoads];     // coalesced pieces of the activation slab
     uint32_t win;                           // sign word (sign_base >> 5) + L
     int      sign_base;                     // tile offset + band offset, in sign bits
 };
@@ -178,6 +198,8 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
     // workgroup barrier, and it happens while the first loads are in flight.
     __shared__ Lut lut_all[WAVES][256];
     __shared__ Acc red[WAVES][MB][64];
+    using XS = XSlab<Act>;
+    __shared__ __align__(16) uint8_t xslab_all[WAVES][MB][16 * XS::kPitch];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -194,15 +216,18 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
     const LaneGeom q(lane);
     const int i = q.i, g = q.g, b0 = q.b0;
 
-    // Lanes whose batch row does not exist load nothing (zero operand, output never stored).
-    int xrow[MB];
-    bool x_ok[MB];
+    // Coalesced activation pieces of this lane; rows past M are not loaded (their operand is zero
+    // and their output column is never stored).
+    const Act* xp[MB][XS::kLoads];
+    bool x_ok[MB][XS::kLoads];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-        const int m = m_base + mb * 16 + i;
-        x_ok[mb] = m < M;
-        xrow[mb] = x_ok[mb] ? m : 0;
-    }
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int h = 0; h < XS::kLoads; ++h) {
+            const int m = m_base + mb * 16 + XS::row_of(lane, h);
+            x_ok[mb][h] = m < M;
+            xp[mb][h] = x + static_cast<size_t>(x_ok[mb][h] ? m : 0) * K + XS::col_of(lane);
+        }
 
     Acc acc[MB];
 #pragma unroll
@@ -240,12 +265,10 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
         raw.bm[0] = bmp[b0];
         raw.bm[1] = bmp[b0 + 1];
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-            const Act* xp = x + static_cast<size_t>(xrow[mb]) * K + gk * 64 + g * 16;
+        for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-            for (int v = 0; v < T::kXVecs; ++v)
-                raw.x[mb][v] = x_ok[mb] ? reinterpret_cast<const u32x4*>(xp)[v] : u32x4{0u, 0u, 0u, 0u};
-        }
+            for (int h = 0; h < XS::kLoads; ++h)
+                raw.x[mb][h] = x_ok[mb][h] ? *reinterpret_cast<const u32x4*>(xp[mb][h] + gk * 64) : u32x4{0u, 0u, 0u, 0u};
     };
     // The sign window: needs the band-tile's stream offset.
     auto fetch_signs = [&](int base, BandTileRaw<Act, MB>& raw) {
@@ -258,7 +281,14 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
         raw.win = win;
     };
 
+    uint8_t* slab = xslab_all[wave][0];
     auto process = [&](const BandTileRaw<Act, MB>& cur) {
+        // slab in (coalesced order), operands out (MFMA order); same wave, so LDS ordering suffices
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int h = 0; h < XS::kLoads; ++h)
+                *reinterpret_cast<u32x4*>(slab + mb * (16 * XS::kPitch) + XS::write_off(lane, h)) = cur.x[mb][h];
         uint32_t idx[2][2];
         band_tile_indices_win(q, cur.bm, cur.sign_base, cur.win, idx);
 
@@ -271,7 +301,9 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
                 const bf16x8 a = __builtin_bit_cast(bf16x8, a_bits);
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) {
-                    const u32x4 x0 = cur.x[mb][0], x1 = cur.x[mb][1];
+                    const uint8_t* src = slab + mb * (16 * XS::kPitch) + i * XS::kPitch + g * 32;
+                    const u32x4 x0 = *reinterpret_cast<const u32x4*>(src);
+                    const u32x4 x1 = *reinterpret_cast<const u32x4*>(src + 16);
                     const u32x4 b_bits = t == 0 ? u32x4{x0.x, x0.z, x1.x, x1.z} : u32x4{x0.y, x0.w, x1.y, x1.w};
                     const bf16x8 b = __builtin_bit_cast(bf16x8, b_bits);
                     acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mb], 0, 0, 0);
@@ -283,8 +315,8 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
                              static_cast<int>(lut[idx[1][0]]), static_cast<int>(lut[idx[1][1]])};
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
-                const u32x4 xv = cur.x[mb][0];       // dword j = columns 4j .. 4j+3
-                const i32x4 b = {
+                const u32x4 xv = *reinterpret_cast<const u32x4*>(slab + mb * (16 * XS::kPitch) + i * XS::kPitch + g * 16);
+                const i32x4 b = {   // dword j of xv = columns 4j .. 4j+3
                     static_cast<int>(__builtin_amdgcn_perm(xv.y, xv.x, 0x05040100u)),   // t=0, c=0..3
                     static_cast<int>(__builtin_amdgcn_perm(xv.w, xv.z, 0x05040100u)),   // t=0, c=4..7
                     static_cast<int>(__builtin_amdgcn_perm(xv.y, xv.x, 0x07060302u)),   // t=1, c=0..3

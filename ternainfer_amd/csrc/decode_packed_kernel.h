@@ -13,26 +13,6 @@
 
 namespace terna {
 
-// Activations reach the MFMA B operand through a wave-private LDS slot.  The operand wants lane
-// (m = L & 15, g = L >> 4) to hold 32 bytes of batch row m -- sixteen different rows in sixteen
-// adjacent lanes, which a global load can only serve one cache line per lane.  So the wave loads
-// its [16 rows][64 columns] slab the other way round (adjacent lanes walk along a row: 8 lanes per
-// 128-byte row segment, fully coalesced), drops it into LDS with a padded row pitch, and reads
-// it back in operand order; both LDS accesses are bank-conflict free.
-template <typename Act> struct XSlab;
-template <> struct XSlab<uint16_t> {              // bf16: a row segment is 128 B = 8 lanes x 16 B
-    static constexpr int kPitch = 144, kLoads = 2;   // two loads: rows 0-7 and rows 8-15
-    __device__ static int row_of(int lane, int h) { return 8 * h + (lane >> 3); }
-    __device__ static int col_of(int lane) { return (lane & 7) * 8; }             // in elements
-    __device__ static int write_off(int lane, int h) { return row_of(lane, h) * kPitch + (lane & 7) * 16; }
-};
-template <> struct XSlab<int8_t> {                // int8: a row segment is 64 B = 4 lanes x 16 B
-    static constexpr int kPitch = 80, kLoads = 1;    // one load covers all 16 rows
-    __device__ static int row_of(int lane, int) { return lane >> 2; }
-    __device__ static int col_of(int lane) { return (lane & 3) * 16; }
-    __device__ static int write_off(int lane, int) { return (lane >> 2) * kPitch + (lane & 3) * 16; }
-};
-
 template <typename Act, int MB>
 struct PackedRaw {
     uint32_t word;                           // 16 weights: row (L & 15), 16-column group (L >> 4)
