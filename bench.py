@@ -34,9 +34,12 @@ HBM_PEAK_GBPS = 8000.0
 BF16_MFMA_PEAK_TFLOPS = 2500.0
 LAYER_SET = [("wqkv", 3840, 2560), ("wo", 2560, 2560), ("w13", 13824, 2560), ("w2", 2560, 6912)]   # (name, N, K)
 
-# HBM bytes per launch of the small-M kernel on this workload, from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE runs scaled by a copy kernel of known size; None until measured.
-TRAFFIC_BYTES_PER_LAUNCH = None
+# HBM bytes per launch of the small-M kernel on the default workload (M=8, average over the four
+# matrices), from two rocprofv3 --pmc runs (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each
+# scaled by what the same counter reads for a plain 256 MiB device copy / fill in the same run
+# (FETCH_SIZE reads 131088 for 262144 KiB -> x2.0; WRITE_SIZE reads 262144 -> x1.0).  Per layer:
+# 19209 KiB fetched + 356 KiB written over 4 launches.  None where not collected.
+TRAFFIC_BYTES_PER_LAUNCH = {"packed": (19209.3 + 356.0) * 1024 / 4, "reference": None}
 
 
 def vp(t):
@@ -169,6 +172,33 @@ def cpu_baseline(mats, torch):
     }
 
 
+def run_model(args, torch):
+    """configs[4]: 2B-shaped random-init model, prompt of 128 uniform random ids, greedy decode of 256
+    tokens; tokens/s = generated tokens / decode-phase time (as the reference's stats.py:19-27)."""
+    from ternainfer_amd.model import ModelArgs, Transformer, greedy_decode
+    margs = ModelArgs()
+    t0 = time.perf_counter()
+    model = Transformer(margs, seed=20260500, act=args.act)
+    torch.cuda.synchronize()
+    build_s = time.perf_counter() - t0
+    gen = torch.Generator(device="cuda").manual_seed(20260501)
+    prompt = torch.randint(0, margs.vocab_size, (args.batch, 128), generator=gen, device="cuda")
+    greedy_decode(model, prompt, 8)                                   # warm-up (code objects, allocator)
+    toks, prefill_s, decode_s = greedy_decode(model, prompt, 256)
+    tps = args.batch * 256 / decode_s
+    print(json.dumps({
+        "metric": "2B-shape decode tok/s", "value": tps, "unit": "tokens/s", "n_gpus": 1, "steps": 256, "warmup": 8,
+        "ms_per_step": decode_s * 1e3 / 256, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"configs[4]: BitNet-b1.58-2B-shaped random-init decoder (30 layers, hidden 2560, 20/5 heads, "
+                               f"FFN 6912, vocab 128256), batch {args.batch}, 128-token prompt, 256 greedy tokens, "
+                               f"{args.act} activations into the ternary linears, weights in P2 layout, one HIP graph per "
+                               "decode step; attention / norms / RoPE / LM head are plain PyTorch ops",
+                   "batch": args.batch, "act": args.act},
+        "prefill_tokens_per_s": args.batch * 128 / prefill_s, "prefill_s": prefill_s, "decode_s": decode_s,
+        "model_build_s": build_s, "first_tokens": toks[0, :8].tolist()}))
+
+
 def run_prefill(args, torch, T, lib):
     """configs[2]: the four BitNet-2B matrices at M in {256, 512, 2048}, bf16 activations with 1% of
     the channels scaled x20.  A step is one pass over the four matrices at M = --m (default 2048
@@ -245,13 +275,19 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--m", type=int, default=8, help="activation rows per call (decode batch)")
     ap.add_argument("--layers", type=int, default=30, help="distinct weight copies per matrix")
-    ap.add_argument("--workload", choices=["decode", "prefill"], default="decode",
-                    help="decode: the headline small-M HBM-bound pass; prefill: the M>=256 MFMA-bound pass")
+    ap.add_argument("--workload", choices=["decode", "prefill", "model"], default="decode",
+                    help="decode: the headline small-M HBM-bound pass; prefill: the M>=256 MFMA-bound pass; "
+                         "model: random-init BitNet-2B-shaped decoder, 128-token prompt + 256 greedy tokens")
+    ap.add_argument("--batch", type=int, default=1, help="sequences decoded together (model workload)")
+    ap.add_argument("--act", choices=["int8", "bf16"], default="int8",
+                    help="model workload: int8-quantised activations (the reference's SpBitLinear) or bf16")
     ap.add_argument("--layout", choices=["packed", "reference"], default="packed",
                     help="packed: weights repacked once at load time to the library's P2 layout (bit-exact); "
                          "reference: kernels read the reference's compressed format directly")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-per-shape", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one plain 256 MiB device copy (calibrates FETCH_SIZE / WRITE_SIZE under rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
@@ -264,8 +300,17 @@ def main():
     lib = T._lib.load()
     torch.cuda.set_device(0)
 
+    if args.copy_probe:
+        a = torch.empty(256 << 20, dtype=torch.int8, device="cuda")
+        b = torch.ones(256 << 20, dtype=torch.int8, device="cuda")
+        torch.cuda.synchronize()
+        a.copy_(b)                                     # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
     if args.workload == "prefill":
         run_prefill(args, torch, T, lib)
+        return
+    if args.workload == "model":
+        run_model(args, torch)
         return
 
     mats = [Matrix(name, n, k, args.m, args.layers, 20260200 + 10 * j, torch, T)
@@ -310,7 +355,8 @@ def main():
                    "m": args.m, "layers": args.layers, "layout": args.layout, "launches_per_step": launches_per_step,
                    "algorithmic_bytes_per_step": step_bytes},
         "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": gbps / HBM_PEAK_GBPS, "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+                     "frac": gbps / HBM_PEAK_GBPS,
+                     "traffic": TRAFFIC_BYTES_PER_LAUNCH[args.layout] if args.m == 8 and args.layers == 30 else None,
                      "kernel": ("terna_decode_packed_kernel<bf16>" if args.layout == "packed"
                                 else "terna_decode_kernel<bf16>"),
                      "algorithmic_bytes_per_launch": step_bytes / launches_per_step,

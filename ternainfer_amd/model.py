@@ -1,0 +1,217 @@
+"""Measurement harness: a BitNet-b1.58-2B-shaped decoder whose linear layers run through TernaSpMM.
+
+This is NOT a port of the reference's transformer (model.py:155-471); it exists so that the
+2B-shape decode tokens/s of the benchmark configuration can be measured with every ternary linear
+going through libternaspmm.so.  It keeps the reference's block structure -- fused wqkv / w13,
+attention and FFN sub-norms, squared-ReLU gating, tied bf16 LM head (model.py:198-239, 277-282,
+323-335, 367) -- and, like the reference's SpBitLinear (model.py:120-133), quantises activations
+per row to int8 in front of every ternary linear.  Attention, RoPE, norms and the LM head are
+plain PyTorch-ROCm ops; one decode step is captured in a HIP graph, as generate.py:204-224 does.
+"""
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+from typing import List, Optional
+
+import torch
+from torch.nn import functional as F
+
+from . import _lib
+
+
+@dataclass
+class ModelArgs:                      # model.py:23-34
+    dim: int = 2560
+    n_layers: int = 30
+    n_heads: int = 20
+    n_kv_heads: int = 5
+    vocab_size: int = 128256
+    ffn_dim: int = 6912
+    norm_eps: float = 1e-5
+    rope_theta: float = 500000.0
+
+    @property
+    def head_dim(self) -> int:
+        return self.dim // self.n_heads
+
+
+def _p(t: Optional[torch.Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def random_p2_weight(n: int, k: int, p_zero: float, gen: torch.Generator, device="cuda") -> torch.Tensor:
+    """Random ternary [n, k] matrix, generated on the device directly in the library's P2 layout
+    (uint32 [n/16][k/64][64], see csrc/packed_common.h): P(0) = p_zero, signs balanced."""
+    u = torch.rand((n // 16, 16, k // 64, 4, 16), generator=gen, device=device)           # band, i, gk, g, q
+    neg = torch.rand(u.shape, generator=gen, device=device) < 0.5
+    code = (u >= p_zero).to(torch.int64) | ((u >= p_zero) & neg).to(torch.int64) << 1
+    q = torch.arange(16, device=device)
+    t, c = (q >> 1) & 1, 2 * (q >> 2) + (q & 1)
+    shift = 8 * (c & 3) + 2 * (2 * t + (c >> 2))
+    words = (code << shift).sum(dim=-1)                                                     # band, i, gk, g
+    words = words.permute(0, 2, 1, 3).contiguous().view(n // 16, k // 64, 64)
+    return (words - ((words >> 31) << 32)).to(torch.int32)                                  # same 32 bits, signed storage
+
+
+class TernaryLinear:
+    """One ternary matrix in P2 layout + its weight-group scales; forward = TernaSpMM."""
+
+    def __init__(self, in_features: int, out_features: int, packed: torch.Tensor, weight_scale: torch.Tensor,
+                 act: str = "int8"):
+        self.k, self.n = in_features, out_features
+        self.packed = packed
+        self.ws = weight_scale.to(torch.bfloat16).contiguous()                  # bf16[4], zero padded (convert_TernaInfer.py:176-194)
+        self.ws_num = int((self.ws != 0).sum().item())
+        self.scale_f32 = self.ws.float().contiguous()
+        self.act = act
+        self.lib = _lib.load()
+
+    def __call__(self, x: torch.Tensor) -> torch.Tensor:
+        m = x.shape[0]
+        out = torch.empty((m, self.n), dtype=torch.bfloat16, device=x.device)
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        if self.act == "int8":                                                   # model.py:120-133
+            s = 127 / x.abs().max(dim=-1, keepdim=True).values.clamp_(min=1e-5)
+            xq = (x * s).round().clamp(-128, 127).to(torch.int8)
+            self.lib.bitlinear_TernaSpMM_packed(_p(xq), _p(self.packed), _p(out), _p(s.to(torch.bfloat16).contiguous()),
+                                                _p(self.ws), self.ws_num, m, self.n, self.k, 0, stream)
+        else:
+            self.lib.bitlinear_TernaSpMM_bf16_packed(_p(x.contiguous()), _p(self.packed), _p(out), _p(self.scale_f32),
+                                                     self.ws_num, m, self.n, self.k, 0, stream)
+        return out
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).to(x.dtype) * weight
+
+
+def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """x [B, H, T, D]; rotate-half convention; cos/sin [B, 1, T, D/2] in fp32."""
+    x1, x2 = x.float().chunk(2, dim=-1)
+    return torch.cat([x1 * cos - x2 * sin, x2 * cos + x1 * sin], dim=-1).to(x.dtype)
+
+
+class Block:
+    def __init__(self, args: ModelArgs, gen: torch.Generator, act: str, p_zero: float):
+        d, hd = args.dim, args.head_dim
+        qkv_n = (args.n_heads + 2 * args.n_kv_heads) * hd
+        bf = lambda v: torch.tensor(v + [0.0] * (4 - len(v)), dtype=torch.bfloat16, device="cuda")
+        sc = lambda: float(torch.empty(1).uniform_(0.5, 2.0, generator=gen_cpu))
+        gen_cpu = torch.Generator().manual_seed(int(torch.randint(0, 2 ** 31, (1,), generator=gen, device="cuda").item()))
+        self.wqkv = TernaryLinear(d, qkv_n, random_p2_weight(qkv_n, d, p_zero, gen), bf([sc(), sc(), sc()]), act)
+        self.wo = TernaryLinear(args.n_heads * hd, d, random_p2_weight(d, args.n_heads * hd, p_zero, gen), bf([sc()]), act)
+        self.w13 = TernaryLinear(d, 2 * args.ffn_dim, random_p2_weight(2 * args.ffn_dim, d, p_zero, gen), bf([sc(), sc()]), act)
+        self.w2 = TernaryLinear(args.ffn_dim, d, random_p2_weight(d, args.ffn_dim, p_zero, gen), bf([sc()]), act)
+        ones = lambda n: torch.ones(n, dtype=torch.bfloat16, device="cuda")
+        self.attention_norm, self.ffn_norm = ones(d), ones(d)
+        self.attn_sub_norm, self.ffn_sub_norm = ones(d), ones(args.ffn_dim)
+        self.args = args
+
+    def forward(self, x, cache_k, cache_v, pos_idx, cos, sin, mask):
+        """x [B*T, dim] (T new tokens per sequence); cache_* [B, n_kv, S, hd]; pos_idx int64 [T] cache slots."""
+        a = self.args
+        bsz = cache_k.shape[0]
+        t = x.shape[0] // bsz
+        h = rms_norm(x, self.attention_norm, a.norm_eps)
+        qkv = self.wqkv(h).view(bsz, t, a.n_heads + 2 * a.n_kv_heads, a.head_dim).transpose(1, 2)
+        q, k, v = qkv[:, :a.n_heads], qkv[:, a.n_heads:a.n_heads + a.n_kv_heads], qkv[:, a.n_heads + a.n_kv_heads:]
+        q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
+        cache_k.index_copy_(2, pos_idx, k)
+        cache_v.index_copy_(2, pos_idx, v)
+        rep = a.n_heads // a.n_kv_heads
+        kk = cache_k.repeat_interleave(rep, dim=1)
+        vv = cache_v.repeat_interleave(rep, dim=1)
+        o = F.scaled_dot_product_attention(q, kk, vv, attn_mask=mask)
+        o = o.transpose(1, 2).reshape(bsz * t, a.n_heads * a.head_dim)
+        x = x + self.wo(rms_norm(o, self.attn_sub_norm, a.norm_eps))
+        h = rms_norm(x, self.ffn_norm, a.norm_eps)
+        x1, x3 = self.w13(h).chunk(2, dim=-1)
+        inner = rms_norm(F.relu(x1) ** 2 * x3, self.ffn_sub_norm, a.norm_eps)
+        return x + self.w2(inner)
+
+
+class Transformer:
+    """Random-init decoder; `act` selects int8-quantised (reference semantics) or bf16 activations."""
+
+    def __init__(self, args: ModelArgs, seed: int = 0, act: str = "int8", p_zero: float = 0.40):
+        gen = torch.Generator(device="cuda").manual_seed(seed)
+        self.args = args
+        self.tok_embeddings = (torch.randn((args.vocab_size, args.dim), generator=gen, device="cuda") * 0.02).to(torch.bfloat16)
+        self.layers: List[Block] = [Block(args, gen, act, p_zero) for _ in range(args.n_layers)]
+        self.norm = torch.ones(args.dim, dtype=torch.bfloat16, device="cuda")
+
+    def make_cache(self, bsz: int, max_seq: int):
+        a = self.args
+        shape = (bsz, a.n_kv_heads, max_seq, a.head_dim)
+        dev = self.tok_embeddings.device
+        return [(torch.zeros(shape, dtype=torch.bfloat16, device=dev), torch.zeros(shape, dtype=torch.bfloat16, device=dev))
+                for _ in range(a.n_layers)]
+
+    def forward(self, tokens: torch.Tensor, cache, pos_idx: torch.Tensor) -> torch.Tensor:
+        """tokens int64 [B, T]; pos_idx int64 [T] = cache slots of the new tokens.  Returns logits [B, vocab]
+        of the last new token."""
+        a = self.args
+        bsz, t = tokens.shape
+        max_seq = cache[0][0].shape[2]
+        dev = tokens.device
+        inv = 1.0 / (a.rope_theta ** (torch.arange(0, a.head_dim, 2, device=dev, dtype=torch.float32) / a.head_dim))
+        ang = pos_idx.float()[:, None] * inv[None, :]
+        cos, sin = ang.cos()[None, None], ang.sin()[None, None]
+        # causal over cache slots: new token at slot p sees slots <= p
+        mask = torch.arange(max_seq, device=dev)[None, :] <= pos_idx[:, None]
+        x = self.tok_embeddings[tokens.reshape(-1)]
+        for layer, (ck, cv) in zip(self.layers, cache):
+            x = layer.forward(x, ck, cv, pos_idx, cos, sin, mask[None, None])
+        x = rms_norm(x.view(bsz, t, a.dim)[:, -1], self.norm, a.norm_eps)
+        return F.linear(x, self.tok_embeddings)                               # tied LM head (model.py:367)
+
+
+@torch.inference_mode()
+def greedy_decode(model: Transformer, prompt: torch.Tensor, gen_tokens: int, use_graph: bool = True):
+    """Prefill `prompt` [B, P], then `gen_tokens` greedy steps.  Returns (tokens [B, gen_tokens],
+    prefill seconds, decode seconds).  The decode step (model forward + argmax + position bump) is
+    captured once and replayed, so the host issues one graph launch per token."""
+    bsz, plen = prompt.shape
+    cache = model.make_cache(bsz, plen + gen_tokens)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+    ev[0].record()
+    logits = model.forward(prompt, cache, torch.arange(plen, device="cuda"))
+    tok = logits.argmax(dim=-1, keepdim=True)
+    ev[1].record()
+    pos = torch.full((1,), plen, dtype=torch.int64, device="cuda")
+    out = torch.empty((bsz, gen_tokens), dtype=torch.int64, device="cuda")
+    step_idx = torch.zeros(1, dtype=torch.int64, device="cuda")
+
+    def step():
+        out.index_copy_(1, step_idx, tok)
+        nxt = model.forward(tok, cache, pos).argmax(dim=-1, keepdim=True)
+        tok.copy_(nxt)
+        pos.add_(1)
+        step_idx.add_(1)
+
+    graph = None
+    if use_graph:
+        # warm up on a side stream (allocator, lazy inits), then restore the state and capture
+        snap = (tok.clone(), pos.clone(), step_idx.clone())
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        tok.copy_(snap[0]); pos.copy_(snap[1]); step_idx.copy_(snap[2])
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        tok.copy_(snap[0]); pos.copy_(snap[1]); step_idx.copy_(snap[2])
+    torch.cuda.synchronize()
+    ev[2].record()
+    for _ in range(gen_tokens):
+        if graph is not None:
+            graph.replay()
+        else:
+            step()
+    ev[3].record()
+    torch.cuda.synchronize()
+    return out, ev[0].elapsed_time(ev[1]) * 1e-3, ev[2].elapsed_time(ev[3]) * 1e-3
