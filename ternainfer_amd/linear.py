@@ -90,6 +90,36 @@ def TernaInfer_linear_bf16(input, compressed_val, TileOffsets_global, TileOffset
     return out.reshape(*out_shape)
 
 
+def repack_weight(compressed_val, TileOffsets_global, TileOffsets_median, bitmap, out_features, in_features):
+    """Load-time repack of one matrix from the reference format to the library's P2 device layout
+    (2 bits per weight, bit-exact; one kernel launch).  Returns an int8 device tensor of N*K/4 bytes."""
+    lib = _lib.load()
+    nbytes = lib.ternaspmm_packed_bytes(out_features, in_features)
+    if nbytes < 0:
+        raise ValueError(f"repack_weight: N and K must be multiples of 64, got {out_features}x{in_features}")
+    packed = torch.empty(nbytes, dtype=torch.int8, device=bitmap.device)
+    stream = torch.cuda.current_stream()
+    lib.ternaspmm_repack(_p(bitmap), _p(TileOffsets_global), _p(TileOffsets_median), _p(compressed_val), _p(packed),
+                         out_features, in_features, ctypes.c_void_p(stream.cuda_stream))
+    return packed
+
+
+def TernaInfer_linear_packed(input, packed, s, ws, ws_num, out_features):
+    """int8 activations x P2-layout ternary weight -> bf16; the reference's epilogue rule by M
+    (decode arithmetic for M <= 64, prefill arithmetic above).  No row padding needed."""
+    lib = _lib.load()
+    out_shape = list(input.shape)
+    out_shape[-1] = out_features
+    K = input.shape[-1]
+    x = input.reshape(-1, K).contiguous()
+    M = x.shape[0]
+    out = torch.empty((M, out_features), dtype=torch.bfloat16, device=input.device)
+    stream = torch.cuda.current_stream()
+    lib.bitlinear_TernaSpMM_packed(_p(x), _p(packed), _p(out), _p(s.reshape(M).contiguous()), _p(ws), ws_num,
+                                   M, out_features, K, 0, ctypes.c_void_p(stream.cuda_stream))
+    return out.reshape(*out_shape)
+
+
 class _CompressedWeight(nn.Module):
     """Holds the four format tensors + ``weight_scale`` under the reference's checkpoint keys
     (convert_TernaInfer.py:204-209, model.py:110-116)."""
@@ -110,7 +140,18 @@ class _CompressedWeight(nn.Module):
 
 
 class SpBitLinear(_CompressedWeight):
-    """Ternary linear on int8-quantised activations (model.py:96-133)."""
+    """Ternary linear on int8-quantised activations (model.py:96-133).  With ``repack=True`` the
+    weight is repacked once at construction and every call runs on the P2 layout."""
+
+    def __init__(self, in_features: int, out_features: int, dic: dict, key: str, bias: bool = False,
+                 repack: bool = False):
+        super().__init__(in_features, out_features, dic, key)
+        self.weight_packed = None
+        if repack:
+            self.weight_packed = torch.nn.Parameter(
+                repack_weight(self.weight_compressed_val, self.weight_TileOffsets_global,
+                              self.weight_TileOffsets_median, self.weight_bitmap, out_features, in_features),
+                requires_grad=False)
 
     def quant_input(self, input):
         s = 127 / input.abs().max(dim=-1, keepdim=True).values.clamp_(min=1e-5)
@@ -118,6 +159,9 @@ class SpBitLinear(_CompressedWeight):
 
     def forward(self, input):
         input, s = self.quant_input(input)
+        if self.weight_packed is not None:
+            return TernaInfer_linear_packed(input, self.weight_packed, s.to(torch.bfloat16), self.weight_scale,
+                                            self.ws_num, self.out_features)
         return TernaInfer_linear(
             input, self.weight_compressed_val, self.weight_TileOffsets_global, self.weight_TileOffsets_median,
             self.weight_bitmap, get_global_workspace(), s, self.weight_scale, self.ws_num, self.out_features)

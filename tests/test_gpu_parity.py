@@ -459,3 +459,40 @@ def test_large_m_with_workspace_matches_without(lib):
     ref = O.spmm_bf16_golden(x, w, scale, 1)
     _check_bf16(run_bf16(lib, fmt, x, scale, 1, workspace=True), ref)
     _check_bf16(run_bf16(lib, fmt, x, scale, 1, workspace=False), ref)
+
+
+def test_spbitlinear_module_reference_and_repacked_agree(lib, coracle):
+    """The call-site mirror: SpBitLinear from a reference-format checkpoint dict, with and without
+    the load-time repack, against the oracle on the module's own quantised activations."""
+    import ternainfer_amd as T
+    n, k, m = 384, 256, 5
+    w = make_ternary(n, k, 0.4, 451)
+    vals, off, med, bm = T.compress_weight(torch.from_numpy(w))
+    ws = torch.tensor([1.59375, 0.8125, 0.0, 0.0], dtype=torch.bfloat16)
+    dic = {"l.weight_compressed_val": vals, "l.weight_TileOffsets_global": off, "l.weight_TileOffsets_median": med,
+           "l.weight_bitmap": bm, "l.weight_scale": ws}
+    x = torch.from_numpy(O.bf16_bits_to_f32(make_bf16_activations(m, k, 452))).to(torch.bfloat16).cuda()
+    print("[case] SpBitLinear reference-format vs repacked", flush=True)
+    a = T.SpBitLinear(k, n, dic, "l")(x)
+    b = T.SpBitLinear(k, n, dic, "l", repack=True)(x)
+    torch.cuda.synchronize()
+    assert a.shape == (m, n) and torch.equal(a, b)
+    xq, s = T.SpBitLinear(k, n, dic, "l").quant_input(x)
+    want = coracle.spmm_i8(xq.cpu().numpy(), w, s.to(torch.bfloat16).view(torch.int16).cpu().numpy().view(np.uint16).reshape(-1),
+                           ws.view(torch.int16).numpy().view(np.uint16), 2, 0)
+    assert (a.view(torch.int16).cpu().numpy().view(np.uint16) == want).all()
+
+
+def test_kernel_binary_reference_command_line():
+    """tests/test_kernel (HIP build of the reference's micro-test, same CLI): the documented
+    invocation `8 2560 2560 45 7` must agree exactly with the dense bf16 GEMM (x == 1 makes every
+    output an integer row sum), for both families and the repacked layout."""
+    import subprocess
+    exe = os.path.join(os.path.dirname(__file__), "test_kernel")
+    if not os.path.exists(exe):
+        pytest.fail("tests/test_kernel is not built: run `bash kernels/compile.sh`")
+    print("[case] tests/test_kernel 8 2560 2560 45 7", flush=True)
+    r = subprocess.run([exe, "8", "2560", "2560", "45", "7"], capture_output=True, text=True, timeout=120)
+    print(r.stdout)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert r.stdout.count("TotalError: 0.00") == 4
