@@ -167,17 +167,15 @@ def pack_p2(w: np.ndarray) -> np.ndarray:
 
     uint32 packed[N/16][K/64][64]; element [band][gk][4*i + g] holds the 16 weights of row
     16*band + i, columns 64*gk + 16*g .. +15, two bits each (bit0 = nonzero, bit1 = negative).
-    Column q of the group sits at bit 8*(c & 3) + 2*(2*t + (c >> 2)) with t = (q >> 1) & 1 and
-    c = 2*(q >> 2) + (q & 1) -- (t, c) are the format's own coordinates of a weight inside a
-    bitmap byte pair, so a repack from the reference format never moves a weight across lanes."""
+    Column j of the group sits at bit 8*(j & 3) + 2*(j >> 2): byte j & 3, 2-bit field j >> 2.  The 16
+    weights of a word are the two bitmap bytes (sm = 0, 1) that one lane of the reference kernel
+    decodes, so a repack from the reference format never moves a weight across lanes."""
     w = np.ascontiguousarray(w, dtype=np.int8)
     n, k = w.shape
     assert n % 16 == 0 and k % 64 == 0
     code = ((w != 0).astype(np.uint32) | ((w < 0).astype(np.uint32) << 1))
-    q = np.arange(16)
-    t = (q >> 1) & 1
-    c = 2 * (q >> 2) + (q & 1)
-    shift = (8 * (c & 3) + 2 * (2 * t + (c >> 2))).astype(np.uint32)
+    j = np.arange(16)
+    shift = (8 * (j & 3) + 2 * (j >> 2)).astype(np.uint32)
     blocks = code.reshape(n // 16, 16, k // 64, 4, 16)                # band, i, gk, g, q
     words = np.bitwise_or.reduce(blocks << shift, axis=-1)            # band, i, gk, g
     return np.ascontiguousarray(words.transpose(0, 2, 1, 3)).reshape(n // 16, k // 64, 64).astype(np.uint32)
@@ -186,10 +184,8 @@ def pack_p2(w: np.ndarray) -> np.ndarray:
 def unpack_p2(packed: np.ndarray, n: int, k: int) -> np.ndarray:
     """Inverse of :func:`pack_p2`."""
     words = np.asarray(packed, dtype=np.uint32).reshape(n // 16, k // 64, 16, 4)   # band, gk, i, g
-    q = np.arange(16)
-    t = (q >> 1) & 1
-    c = 2 * (q >> 2) + (q & 1)
-    shift = (8 * (c & 3) + 2 * (2 * t + (c >> 2))).astype(np.uint32)
+    j = np.arange(16)
+    shift = (8 * (j & 3) + 2 * (j >> 2)).astype(np.uint32)
     code = (words[..., None] >> shift) & 3                                            # band, gk, i, g, q
     val = np.where(code & 1, np.where(code & 2, -1, 1), 0).astype(np.int8)
     return np.ascontiguousarray(val.transpose(0, 2, 1, 3, 4)).reshape(n, k)

@@ -91,9 +91,8 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
                 const uint8_t* src = slab + mb * (16 * XS::kPitch) + i * XS::kPitch + g * 32;
-                const u32x4 x0 = *reinterpret_cast<const u32x4*>(src);
-                const u32x4 x1 = *reinterpret_cast<const u32x4*>(src + 16);
-                const u32x4 b0 = {x0.x, x0.z, x1.x, x1.z}, b1 = {x0.y, x0.w, x1.y, x1.w};
+                const u32x4 b0 = *reinterpret_cast<const u32x4*>(src);        // columns 16g .. 16g+7
+                const u32x4 b1 = *reinterpret_cast<const u32x4*>(src + 16);   // columns 16g+8 .. 16g+15
                 acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, __builtin_bit_cast(bf16x8, b0), acc[mb], 0, 0, 0);
                 acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, __builtin_bit_cast(bf16x8, b1), acc[mb], 0, 0, 0);
             }
@@ -101,12 +100,8 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
             const i32x4 a = expand_word_i8(cur.word);
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
-                const u32x4 xv = *reinterpret_cast<const u32x4*>(slab + mb * (16 * XS::kPitch) + i * XS::kPitch + g * 16);
-                const i32x4 b = {
-                    static_cast<int>(__builtin_amdgcn_perm(xv.y, xv.x, 0x05040100u)),   // t=0, c=0..3
-                    static_cast<int>(__builtin_amdgcn_perm(xv.w, xv.z, 0x05040100u)),   // t=0, c=4..7
-                    static_cast<int>(__builtin_amdgcn_perm(xv.y, xv.x, 0x07060302u)),   // t=1, c=0..3
-                    static_cast<int>(__builtin_amdgcn_perm(xv.w, xv.z, 0x07060302u))};  // t=1, c=4..7
+                const i32x4 b = __builtin_bit_cast(
+                    i32x4, *reinterpret_cast<const u32x4*>(slab + mb * (16 * XS::kPitch) + i * XS::kPitch + g * 16));
                 acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[mb], 0, 0, 0);
             }
         }

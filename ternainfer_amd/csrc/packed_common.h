@@ -9,12 +9,11 @@
 //   uint32 packed[N/16][K/64][64]
 //   element [band][gk][4*i + g] : row 16*band + i, columns 64*gk + 16*g .. +15, 2 bits each
 //                                 (bit0 = nonzero, bit1 = negative)
-//   weight (t, c) of the group  : column 16g + 4*(c>>1) + 2t + (c&1)   (the format's own
-//                                 coordinates: byte pair t, bit c of a bitmap row)
-//                                 sits at bit 8*(c&3) + 2*(2t + (c>>2)).
+//   column j of the group       : byte j & 3, 2-bit field j >> 2, i.e. bit 8*(j&3) + 2*(j>>2).
 //
-// So `(word >> 2*(2t+h)) & 0x03030303` is four 2-bit codes in four bytes -- exactly a v_perm_b32
-// selector.  One v_perm against a 4-entry byte table turns it into four int8 weights
+// So `(word >> 2*q) & 0x03030303` is the four 2-bit codes of columns 4q .. 4q+3 in four bytes --
+// exactly a v_perm_b32 selector, and its result is in natural column order: the matching
+// activation operand is a plain contiguous piece of the activation row.  One v_perm against a 4-entry byte table turns it into four int8 weights
 // (0x00 / 0x01 / 0xFF) or four bf16 high bytes (0x00 / 0x3F / 0xBF), and two more v_perm
 // interleave the high bytes with zero low bytes into bf16 pairs.  bf16 weights are therefore
 // +-0.5 (0x3F00 / 0xBF00), not +-1: every product and partial sum is exactly half of what +-1
@@ -31,8 +30,8 @@ constexpr uint32_t kTableI8 = 0xFF000100u;       // code 0 -> 0x00, 1 -> 0x01, 3
 constexpr uint32_t kPair01 = 0x010C000Cu;        // [0, b0, 0, b1]: two bf16 with zero low bytes
 constexpr uint32_t kPair23 = 0x030C020Cu;        // [0, b2, 0, b3]
 
-// Eight bf16 weights (+-0.5 / 0) of byte pair t of a packed word `dd` already shifted right by 4t:
-// k order c = 0..7, i.e. dword j holds the weights that meet activation dword (2j + t) of the group.
+// Eight bf16 weights (+-0.5 / 0), columns 8h .. 8h+7 of the group, of a packed word `dd` already
+// shifted right by 4h: dword j holds columns 8h + 2j, 8h + 2j + 1.
 __device__ __forceinline__ u32x4 expand_chunk_bf16(uint32_t dd)
 {
     const uint32_t hi0 = __builtin_amdgcn_perm(0u, kTableBf16Hi, dd & kCodeMask);
@@ -41,7 +40,7 @@ __device__ __forceinline__ u32x4 expand_chunk_bf16(uint32_t dd)
                  __builtin_amdgcn_perm(0u, hi1, kPair01), __builtin_amdgcn_perm(0u, hi1, kPair23)};
 }
 
-// Sixteen int8 weights (+-1 / 0) of a packed word: dword (2t + h) holds (t, c = 4h .. 4h+3).
+// Sixteen int8 weights (+-1 / 0) of a packed word in column order: dword q holds columns 4q .. 4q+3.
 __device__ __forceinline__ i32x4 expand_word_i8(uint32_t d)
 {
     return i32x4{static_cast<int>(__builtin_amdgcn_perm(0u, kTableI8, d & kCodeMask)),
@@ -50,16 +49,19 @@ __device__ __forceinline__ i32x4 expand_word_i8(uint32_t d)
                  static_cast<int>(__builtin_amdgcn_perm(0u, kTableI8, (d >> 6) & kCodeMask))};
 }
 
-// Repack table: (nonzero nibble, next 4 sign bits of the stream) -> four 2-bit codes, one per byte.
+// Repack table: (nonzero nibble, next 4 sign bits of the stream) -> the nibble's four 2-bit codes
+// where P2 wants them, up to a shift.  Bit cb of nibble hh of bitmap byte sm is column
+// j = 4*(2hh + (cb>>1)) + 2sm + (cb&1) of the group: byte 2sm + (cb&1), field 2hh + (cb>>1).  The
+// table holds byte (cb&1), field (cb>>1); the caller shifts by 16*sm + 4*hh.
 __device__ __forceinline__ uint32_t make_lut_code(int e)
 {
     const int nz = e >> 4, sg = e & 15;
     uint32_t r = 0;
     int used = 0;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        if ((nz >> j) & 1) {
-            r |= (1u | (((sg >> used) & 1) << 1)) << (8 * j);
+    for (int cb = 0; cb < 4; ++cb) {
+        if ((nz >> cb) & 1) {
+            r |= (1u | (((sg >> used) & 1) << 1)) << (8 * (cb & 1) + 2 * (cb >> 1));
             ++used;
         }
     }
@@ -99,7 +101,7 @@ __global__ __launch_bounds__(WAVES * 64) void terna_repack_kernel(
         }
         uint32_t idx[2][2];
         band_tile_indices_win(q, bm, base, win, idx);
-        const uint32_t word = lut[idx[0][0]] | (lut[idx[0][1]] << 2) | (lut[idx[1][0]] << 4) | (lut[idx[1][1]] << 6);
+        const uint32_t word = lut[idx[0][0]] | (lut[idx[0][1]] << 4) | (lut[idx[1][0]] << 16) | (lut[idx[1][1]] << 20);
         packed[(static_cast<size_t>(band) * ktiles + gk) * 64 + q.i * 4 + q.g] = word;
     }
 }

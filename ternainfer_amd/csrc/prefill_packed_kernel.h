@@ -4,15 +4,15 @@
 //
 //   out[m][n] = epilogue( 2 * sum_k X[m][k] * Whalf[n][k] ),   Whalf = W / 2 in {-0.5, 0, +0.5}
 //
-// Tiling.  One workgroup (4 waves) owns 256 output features x BM = 32*MB batch rows and walks K in
-// steps of 64.  The waves split the output features only: wave w owns rows 64w .. 64w+63 and ALL
-// BM batch rows, i.e. 2 x MB accumulator tiles of v_mfma_f32_32x32x16_bf16 with W as the A
+// Tiling.  One workgroup (4 waves) owns BN = 128*NA output features x BM = 32*MB batch rows and walks
+// K in steps of 64.  The waves split the output features only: wave w owns rows 32*NA*w .. +32*NA-1 and
+// ALL BM batch rows, i.e. NA x MB accumulator tiles of v_mfma_f32_32x32x16_bf16 with W as the A
 // operand -- so every weight is expanded exactly once per workgroup, and one expansion (ten VALU
 // ops) feeds MB matrix instructions.  A-operand lane (row = L%32, kb = L/32) of row-tile a needs,
-// for 16-column group g, the eight weights of byte pair t = kb of packed word (band, gk, i, g): the
+// for 16-column group g, columns 8kb .. 8kb+7 of packed word (band, gk, i, g): the
 // four words g = 0..3 of a row are adjacent, so one 16-byte load per row-tile and k-step brings
 // everything the lane needs.  Only the activation tile goes through LDS (two stages, chunk order
-// [g][sm][row], see the reference-format kernel), staged one k-step ahead; B operands are read one
+// [g][half][row]: 16-byte pieces of 8 columns), staged one k-step ahead; B operands are read one
 // group ahead of the MFMAs that use them; weight registers are refilled two k-steps ahead.
 #pragma once
 
@@ -20,6 +20,58 @@
 #include "prefill_kernel.h"
 
 namespace terna {
+
+// 16 int8 -> 16 bf16 in column order (exact: the upper half of the float).
+__device__ __forceinline__ void int8x16_to_bf16(const u32x4& v, u32x4& c0, u32x4& c1)
+{
+    const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+    uint32_t o[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float f[4];
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+            f[b] = static_cast<float>(static_cast<int>(static_cast<int8_t>((d[j] >> (8 * b)) & 0xff)));
+        o[2 * j] = (__float_as_uint(f[0]) >> 16) | (__float_as_uint(f[1]) & 0xffff0000u);
+        o[2 * j + 1] = (__float_as_uint(f[2]) >> 16) | (__float_as_uint(f[3]) & 0xffff0000u);
+    }
+    c0 = u32x4{o[0], o[1], o[2], o[3]};
+    c1 = u32x4{o[4], o[5], o[6], o[7]};
+}
+
+// Fused epilogue of one wave's NA x MB accumulator tiles (v_mfma_f32_32x32x16 layout: lane holds
+// column m = L % 32 and rows n = (v&3) + 8(v>>2) + 4(L/32) of each tile).  The accumulator is half
+// the true sum (weights were +-0.5); x2 is exact.
+template <int MB, int NA>
+__device__ __forceinline__ void packed_prefill_epilogue(f32x16 (&acc)[NA][MB], uint16_t* __restrict__ out,
+                                                        const Epilogue& ep, int M, int N, int n_wave, int m0, int lane)
+{
+    const int kb = lane >> 5, l32 = lane & 31;
+    EpilogueRegs e[MB];
+    int m_of[MB];
+    static_for<0, MB>([&](auto bc) {
+        constexpr int b = decltype(bc)::value;
+        m_of[b] = m0 + 32 * b + l32;
+        e[b].s = ep.kind == EP_BF16 ? 1.0f : bf16_bits_to_float(ep.s[m_of[b] < M ? m_of[b] : M - 1]);
+    });
+    static_for<0, 4 * NA>([&](auto tc) {
+        constexpr int a = decltype(tc)::value >> 2, vq = decltype(tc)::value & 3;
+        const int n = n_wave + 32 * a + 8 * vq + 4 * kb;
+        float wv[4];
+        load_col_scales(ep, n < N ? n : N - 4, N, wv);
+        static_for<0, MB>([&](auto bc) {
+            constexpr int b = decltype(bc)::value;
+            EpilogueRegs eb = e[b];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) eb.w[v] = wv[v];
+            uint16_t o[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) o[v] = apply_epilogue<float>(ep.kind, eb, v, acc[a][b][4 * vq + v] * 2.0f);
+            const u32x2 pk = {o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16)};
+            if (m_of[b] < M && n < N) *reinterpret_cast<u32x2*>(out + static_cast<size_t>(m_of[b]) * N + n) = pk;
+        });
+    });
+}
 
 template <int MB>
 struct PackedPrefillSmem {
@@ -29,16 +81,17 @@ struct PackedPrefillSmem {
     static constexpr int kBytes = 2 * kStage;
 };
 
-template <typename Act, int MB>
-__global__ __launch_bounds__(256, MB == 8 ? 1 : 2) void terna_prefill_packed_kernel(
+template <typename Act, int MB, int NA>
+__global__ __launch_bounds__(256, MB == 8 ? 1 : (MB == 3 ? 3 : 2)) void terna_prefill_packed_kernel(
     const Act* __restrict__ x, const uint32_t* __restrict__ packed, uint16_t* __restrict__ out,
     Epilogue ep, int M, int N, int K)
 {
     using T = ActTraits<Act>;
     using S = PackedPrefillSmem<MB>;
-    constexpr int BN = kPrefillBN, BM = S::BM, PX = S::PX;
-    constexpr int XI = BM / 64;                       // (row, group) activation items per thread and k-step
-    static_assert(MB == 2 || MB == 4 || MB == 8, "batch tile of 64, 128 or 256 rows");
+    constexpr int BN = 128 * NA, BM = S::BM, PX = S::PX;
+    static_assert(NA == 1 || NA == 2, "32 or 64 output features per wave");
+    constexpr int XI = (BM + 63) / 64;                // (row, group) activation items per thread and k-step
+    static_assert(MB == 2 || MB == 3 || MB == 4 || MB == 8, "batch tile of 64, 96, 128 or 256 rows");
 
     extern __shared__ __align__(16) uint8_t smem[];
 
@@ -51,10 +104,10 @@ __global__ __launch_bounds__(256, MB == 8 ? 1 : 2) void terna_prefill_packed_ker
     const int kb = lane >> 5, l32 = lane & 31;
 
     // ---- weight words of this lane: row-tile a -> band (n0/16 + 4*wave + 2a + l32/16), row i = l32 % 16
-    const u32x4* w_ptr[2];                             // running: advanced one k-step per fetch
+    const u32x4* w_ptr[NA];                            // running: advanced one k-step per fetch
 #pragma unroll
-    for (int a = 0; a < 2; ++a) {
-        int band = (n0 >> 4) + 4 * wave + 2 * a + (l32 >> 4);
+    for (int a = 0; a < NA; ++a) {
+        int band = (n0 >> 4) + 2 * NA * wave + 2 * a + (l32 >> 4);
         band = band < last_band ? band : last_band;   // a tile hanging over N re-reads the last band; never stored
         w_ptr[a] = reinterpret_cast<const u32x4*>(packed + (static_cast<size_t>(band) * ktiles) * 64 + (l32 & 15) * 4);
     }
@@ -64,19 +117,21 @@ __global__ __launch_bounds__(256, MB == 8 ? 1 : 2) void terna_prefill_packed_ker
 #pragma unroll
     for (int it = 0; it < XI; ++it) {
         const int item = tid + 256 * it;
-        const int row = item >> 2, g = item & 3;
+        int row = item >> 2;
+        const int g = item & 3;
+        row = row < BM ? row : BM - 1;                // 96-row tile: the spare half-item restages the last row
         x_lds[it] = (g * 2) * PX + row * 16;
         int m = m0 + row;
         m = m < M ? m : M - 1;
         x_ptr[it] = x + static_cast<size_t>(m) * K + g * 16;
     }
 
-    struct RawW { u32x4 w[2]; };                      // [a] -> words g = 0..3
+    struct RawW { u32x4 w[NA]; };                     // [a] -> words g = 0..3
     struct RawX { u32x4 x[XI][T::kXVecs]; };
     // Both fetches walk running pointers: one k-step is 16 u32x4 of weights and 64 activations.
     auto fetch_w = [&](RawW& r) {
 #pragma unroll
-        for (int a = 0; a < 2; ++a) {
+        for (int a = 0; a < NA; ++a) {
             r.w[a] = *w_ptr[a];
             w_ptr[a] += 16;
         }
@@ -93,13 +148,12 @@ __global__ __launch_bounds__(256, MB == 8 ? 1 : 2) void terna_prefill_packed_ker
     auto stage_x = [&](const RawX& r, int st) {
 #pragma unroll
         for (int it = 0; it < XI; ++it) {
-            u32x4 c0, c1;
+            u32x4 c0, c1;                              // columns 16g .. 16g+7 and 16g+8 .. 16g+15 as bf16
             if constexpr (sizeof(Act) == 2) {
-                const u32x4 a = r.x[it][0], b = r.x[it][1];
-                c0 = u32x4{a.x, a.z, b.x, b.z};
-                c1 = u32x4{a.y, a.w, b.y, b.w};
+                c0 = r.x[it][0];
+                c1 = r.x[it][1];
             } else {
-                int8_group_to_chunks(r.x[it][0], c0, c1);
+                int8x16_to_bf16(r.x[it][0], c0, c1);
             }
             uint8_t* dst = smem + st * S::kStage + x_lds[it];
             *reinterpret_cast<u32x4*>(dst) = c0;
@@ -107,17 +161,17 @@ __global__ __launch_bounds__(256, MB == 8 ? 1 : 2) void terna_prefill_packed_ker
         }
     };
 
-    f32x16 acc[2][MB];
+    f32x16 acc[NA][MB];
     {
         const f32x16 zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int a = 0; a < 2; ++a)
+        for (int a = 0; a < NA; ++a)
 #pragma unroll
             for (int b = 0; b < MB; ++b) acc[a][b] = zero;
     }
 
     const int b_off = kb * PX + l32 * 16;                    // + g*2*PX + b*512
-    const int wshift = 4 * kb;                               // byte pair t = kb of every word
+    const int wshift = 4 * kb;                               // columns 8kb .. 8kb+7 of every word
 
     struct BOps { bf16x8 b[MB]; };
     auto load_b = [&](int st, int g, BOps& r) {
@@ -135,7 +189,7 @@ __global__ __launch_bounds__(256, MB == 8 ? 1 : 2) void terna_prefill_packed_ker
             BOps bnxt;
             if constexpr (g < 3) load_b(st, g + 1, bnxt);
 #pragma unroll
-            for (int a = 0; a < 2; ++a) {
+            for (int a = 0; a < NA; ++a) {
                 const bf16x8 af = __builtin_bit_cast(bf16x8, expand_chunk_bf16(rw.w[a][g] >> wshift));
 #pragma unroll
                 for (int b = 0; b < MB; ++b)
@@ -154,8 +208,8 @@ __global__ __launch_bounds__(256, MB == 8 ? 1 : 2) void terna_prefill_packed_ker
     fetch_x(x_raw);
     stage_x(x_raw, 0);
     if (ktiles > 1) {
+        fetch_x(x_raw);                               // activations first: the loop waits for them before the weights
         fetch_w(w1);
-        fetch_x(x_raw);
     }
     __syncthreads();
     // k-step k with both look-aheads in range (k + 2 < ktiles)
@@ -182,32 +236,198 @@ __global__ __launch_bounds__(256, MB == 8 ? 1 : 2) void terna_prefill_packed_ker
     if (k < ktiles) body_tail(k++, w1);
     if (k < ktiles) body_tail(k++, w0);
 
-    // ---- epilogue: lane holds, per accumulator tile, column m = l32 and rows n = (v&3) + 8(v>>2) + 4kb.
-    // The accumulator is half the true sum (weights were +-0.5); x2 is exact.
-    EpilogueRegs e[MB];
-    int m_of[MB];
-    static_for<0, MB>([&](auto bc) {
-        constexpr int b = decltype(bc)::value;
-        m_of[b] = m0 + 32 * b + l32;
-        e[b].s = ep.kind == EP_BF16 ? 1.0f : bf16_bits_to_float(ep.s[m_of[b] < M ? m_of[b] : M - 1]);
-    });
-    static_for<0, 8>([&](auto tc) {
-        constexpr int a = decltype(tc)::value >> 2, vq = decltype(tc)::value & 3;
-        const int n = n0 + 64 * wave + 32 * a + 8 * vq + 4 * kb;
-        float wv[4];
-        load_col_scales(ep, n < N ? n : N - 4, N, wv);
-        static_for<0, MB>([&](auto bc) {
-            constexpr int b = decltype(bc)::value;
-            EpilogueRegs eb = e[b];
+    packed_prefill_epilogue<MB, NA>(acc, out, ep, M, N, n0 + 32 * NA * wave, m0, lane);
+}
+
+// ------------------------------------------------------------------------------------------------
+// bf16-activation variant whose activation tile goes global memory -> LDS directly
+// (global_load_lds_dwordx4), with every load of the main loop issued and awaited by hand.
+//
+// Why by hand: the loop keeps two k-steps of loads in flight and each wait must leave exactly the
+// younger ones outstanding; the counters are in-order, so that is one `s_waitcnt vmcnt(n)` with a
+// known n per k-step -- folded into the step's only barrier.  Loads written as ordinary C++ get
+// their waits from the compiler, which at loop headers settles for far stricter ones.
+//
+// Activation tile in LDS: NST stages of BM rows x 128 bytes (one k-step = 64 bf16 per row), as 8
+// pieces of 16 bytes; piece p of row r sits at position p ^ swizzle(r), so that the 16-byte
+// operand reads of 32 consecutive rows spread over all banks.  One direct load writes 64 lanes x
+// 16 bytes = 8 whole rows (lane = 8*row + position) and reads whole 128-byte lines from memory.
+//
+// Per k-step k (stage k % 3, weight buffer k & 1):
+//   issue X(k+2) -> stage (k+2) % 3        (last read in step k-1, before that step's barrier)
+//   MFMAs of step k
+//   issue W(k+2) -> the buffer step k just used
+//   s_waitcnt vmcnt(MB + NA): everything but X(k+2), W(k+2) has landed, i.e. X(k+1) and W(k+1)
+//   s_barrier                               (also orders step k's operand reads before X(k+3))
+constexpr int kXSwizzleShift = 1;
+__device__ __forceinline__ constexpr int x_swizzle(int row) { return (row >> kXSwizzleShift) & 7; }
+
+// LDS[lds_addr + 16*lane .. +15] <- global[sbase + voff .. +15]; completion is counted by vmcnt.
+__device__ __forceinline__ void lds_dma_b128(const void* sbase, uint32_t voff, uint32_t lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
+// d <- global[sbase + voff .. +15] without a compiler-generated wait: d may be read only after a
+// later wait_loads<>() and a landed(d).
+__device__ __forceinline__ void global_load_b128_nowait(u32x4& d, const void* sbase, uint32_t voff)
+{
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(d) : "v"(voff), "s"(sbase) : "memory");
+}
+__device__ __forceinline__ void landed(u32x4& d) { asm volatile("" : "+v"(d)); }
+template <int VM>
+__device__ __forceinline__ void wait_loads_and_barrier()
+{
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(VM) : "memory");
+}
+
+template <int MB>
+struct PackedPrefillDmaSmem {
+    static constexpr int BM = 32 * MB;
+    static constexpr int kStages = 3;
+    static constexpr int kStage = BM * 128;
+    static constexpr int kBytes = kStages * kStage;
+};
+
+template <int MB, int NA>
+__global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) void terna_prefill_packed_dma_kernel(
+    const uint16_t* __restrict__ x, const uint32_t* __restrict__ packed, uint16_t* __restrict__ out,
+    Epilogue ep, int M, int N, int K)
+{
+    using S = PackedPrefillDmaSmem<MB>;
+    constexpr int BN = 128 * NA, BM = S::BM;
+    static_assert(NA == 1 || NA == 2, "32 or 64 output features per wave");
+    static_assert(MB == 2 || MB == 4, "batch tile of 64 or 128 rows (all stages below 64 KiB of LDS)");
+
+    extern __shared__ __align__(16) uint8_t smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n0 = blockIdx.x * BN, m0 = blockIdx.y * BM;
+    const int ktiles = K >> 6;
+    const int last_band = (N >> 4) - 1;
+    const int kb = lane >> 5, l32 = lane & 31;
+
+    // ---- weights: row-tile a -> band (n0/16 + 2*NA*wave + 2a + l32/16), row l32 % 16; one k-step is 256 bytes
+    uint32_t w_off[NA];
 #pragma unroll
-            for (int v = 0; v < 4; ++v) eb.w[v] = wv[v];
-            uint16_t o[4];
+    for (int a = 0; a < NA; ++a) {
+        int band = (n0 >> 4) + 2 * NA * wave + 2 * a + (l32 >> 4);
+        band = band < last_band ? band : last_band;   // a tile hanging over N re-reads the last band; never stored
+        w_off[a] = static_cast<uint32_t>(band) * static_cast<uint32_t>(ktiles) * 256u + (l32 & 15) * 16;
+    }
+    const uint8_t* w_base = reinterpret_cast<const uint8_t*>(packed);
+    // ---- activations: direct load j of this wave fills rows 8*(wave + 4j) .. +7 of the stage
+    uint32_t x_off[MB];
 #pragma unroll
-            for (int v = 0; v < 4; ++v) o[v] = apply_epilogue<float>(ep.kind, eb, v, acc[a][b][4 * vq + v] * 2.0f);
-            const u32x2 pk = {o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16)};
-            if (m_of[b] < M && n < N) *reinterpret_cast<u32x2*>(out + static_cast<size_t>(m_of[b]) * N + n) = pk;
+    for (int j = 0; j < MB; ++j) {
+        const int row = 8 * (wave + 4 * j) + (lane >> 3);
+        const int piece = (lane & 7) ^ x_swizzle(row);
+        int m = m0 + row;
+        m = m < M ? m : M - 1;
+        x_off[j] = static_cast<uint32_t>(m) * static_cast<uint32_t>(K) * 2u + piece * 16;
+    }
+    const uint8_t* x_base = reinterpret_cast<const uint8_t*>(x);
+    const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem)) + wave * 1024;
+
+    // Stage of k-step kk is kk % 3, kept as running byte offsets (no division in the loop).
+    auto next_stage = [](int st) { return st == 2 * S::kStage ? 0 : st + S::kStage; };
+    auto issue_x = [&](int kk, int st) {
+        const uint8_t* base = x_base + static_cast<size_t>(kk) * 128;
+#pragma unroll
+        for (int j = 0; j < MB; ++j) lds_dma_b128(base, x_off[j], lds0 + st + j * 4096);
+    };
+    struct RawW { u32x4 w[NA]; };
+    auto fetch_w = [&](RawW& r, int kk) {
+        const uint8_t* base = w_base + static_cast<size_t>(kk) * 256;
+#pragma unroll
+        for (int a = 0; a < NA; ++a) global_load_b128_nowait(r.w[a], base, w_off[a]);
+    };
+
+    f32x16 acc[NA][MB];
+    {
+        const f32x16 zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int a = 0; a < NA; ++a)
+#pragma unroll
+            for (int b = 0; b < MB; ++b) acc[a][b] = zero;
+    }
+
+    // B operand of (group g, tile b): row 32b + l32, piece 2g + kb; swizzle(32b + l32) == swizzle(l32)
+    int b_off[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) b_off[g] = l32 * 128 + (((2 * g + kb) ^ x_swizzle(l32)) * 16);
+    const int wshift = 4 * kb;                               // columns 8kb .. 8kb+7 of every word
+
+    struct BOps { bf16x8 b[MB]; };
+    auto load_b = [&](const uint8_t* stage, int g, BOps& r) {
+#pragma unroll
+        for (int b = 0; b < MB; ++b)
+            r.b[b] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(stage + b_off[g] + b * 4096));
+    };
+    // The scheduling fences keep the operand reads one group ahead of their MFMAs (hoisting all
+    // of them to the top costs 8*MB registers) and every MFMA of the step before its barrier.
+    auto mma_step = [&](const RawW& rw, int st) {
+        const uint8_t* stage = smem + st;
+        BOps bcur;
+        load_b(stage, 0, bcur);
+        static_for<0, 4>([&](auto gc) {
+            constexpr int g = decltype(gc)::value;
+            BOps bnxt;
+            if constexpr (g < 3) load_b(stage, g + 1, bnxt);
+#pragma unroll
+            for (int a = 0; a < NA; ++a) {
+                const bf16x8 af = __builtin_bit_cast(bf16x8, expand_chunk_bf16(rw.w[a][g] >> wshift));
+#pragma unroll
+                for (int b = 0; b < MB; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bcur.b[b], acc[a][b], 0, 0, 0);
+            }
+            if constexpr (g < 3) bcur = bnxt;
+            __builtin_amdgcn_sched_barrier(0);
         });
-    });
+    };
+
+    // A hand-issued load writes its registers (or LDS) whenever it lands, which the compiler does
+    // not know: every one of them must be followed, on every path, by a wait that covers it
+    // before its destination can be reused -- so none is issued for steps past the end, and the
+    // last two steps wait for everything.
+    RawW w0, w1;
+    int st_mma = 0;                                          // stage of the step being multiplied
+    int st_dma = 2 * S::kStage;                              // stage that the next direct load fills
+    issue_x(0, 0);
+    fetch_w(w0, 0);
+    if (ktiles > 1) {
+        issue_x(1, S::kStage);
+        fetch_w(w1, 1);
+        wait_loads_and_barrier<MB + NA>();
+    } else {
+        wait_loads_and_barrier<0>();
+    }
+    auto body = [&](int k, RawW& w) {
+        const bool more = k + 2 < ktiles;                    // uniform
+        if (more) issue_x(k + 2, st_dma);
+#pragma unroll
+        for (int a = 0; a < NA; ++a) landed(w.w[a]);
+        __builtin_amdgcn_sched_barrier(0);
+        mma_step(w, st_mma);
+        if (more) {
+            fetch_w(w, k + 2);
+            wait_loads_and_barrier<MB + NA>();
+        } else {
+            wait_loads_and_barrier<0>();
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        st_mma = next_stage(st_mma);
+        st_dma = next_stage(st_dma);
+    };
+    int k = 0;
+    for (; k + 1 < ktiles; k += 2) {
+        body(k, w0);
+        body(k + 1, w1);
+    }
+    if (k < ktiles) body(k, w0);
+
+    packed_prefill_epilogue<MB, NA>(acc, out, ep, M, N, n0 + 32 * NA * wave, m0, lane);
 }
 
 }  // namespace terna

@@ -145,17 +145,44 @@ void launch_decode_packed(const Act* x, const uint32_t* packed, uint16_t* out, c
     }
 }
 
-template <typename Act, int MB>
+template <typename Act, int MB, int NA = 2>
 void launch_prefill_packed_as(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N,
                               int K, hipStream_t st)
 {
     using S = PackedPrefillSmem<MB>;
-    auto kernel = terna_prefill_packed_kernel<Act, MB>;
+    auto kernel = terna_prefill_packed_kernel<Act, MB, NA>;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, S::kBytes);
     if (attr != hipSuccess) die("hipFuncSetAttribute(prefill packed)", attr, __LINE__);
-    const dim3 grid((N + kPrefillBN - 1) / kPrefillBN, (M + S::BM - 1) / S::BM);
+    constexpr int BN = 128 * NA;
+    const dim3 grid((N + BN - 1) / BN, (M + S::BM - 1) / S::BM);
     kernel<<<grid, dim3(256), S::kBytes, st>>>(x, packed, out, ep, M, N, K);
+}
+
+template <int MB, int NA>
+void launch_prefill_packed_dma_as(const uint16_t* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M,
+                                  int N, int K, hipStream_t st)
+{
+    using S = PackedPrefillDmaSmem<MB>;
+    auto kernel = terna_prefill_packed_dma_kernel<MB, NA>;
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, S::kBytes);
+    if (attr != hipSuccess) die("hipFuncSetAttribute(prefill packed dma)", attr, __LINE__);
+    constexpr int BN = 128 * NA;
+    const dim3 grid((N + BN - 1) / BN, (M + S::BM - 1) / S::BM);
+    kernel<<<grid, dim3(256), S::kBytes, st>>>(x, packed, out, ep, M, N, K);
+}
+
+// The direct-to-LDS kernel addresses both operands as a 64-bit base plus a 32-bit byte offset and
+// loads 16-byte pieces of the activation rows.
+inline bool prefill_dma_ok(const void* x, int M, int N, int K)
+{
+    static const bool off = [] {
+        const char* v = std::getenv("TERNASPMM_PREFILL_DMA");
+        return v && std::atoi(v) == 0;
+    }();
+    return !off && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && static_cast<uint64_t>(M) * K * 2 < (1ull << 32) &&
+           static_cast<uint64_t>(N) * K / 4 < (1ull << 32);
 }
 
 template <typename Act>
@@ -168,10 +195,30 @@ void launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, 
     static const int forced = [] {
         const char* v = std::getenv("TERNASPMM_PREFILL_BM");
         const int bm = v ? std::atoi(v) : 0;
-        return (bm == 64 || bm == 128 || bm == 256) ? bm : 0;
+        return (bm == 64 || bm == 96 || bm == 128 || bm == 256) ? bm : 0;
+    }();
+    static const int forced_bn = [] {
+        const char* v = std::getenv("TERNASPMM_PREFILL_BN");
+        const int bn = v ? std::atoi(v) : 0;
+        return (bn == 128 || bn == 256) ? bn : 0;
     }();
     const int bm = forced ? forced : 64;
-    if (bm == 256) launch_prefill_packed_as<Act, 8>(x, packed, out, ep, M, N, K, st);
+    // 256-feature tiles expand every weight once per 64 batch rows with two MFMAs per operand read;
+    // when they would leave most of the 1024 workgroup slots of the chip empty, 128-feature tiles
+    // double the workgroup count instead.  TERNASPMM_PREFILL_BN=128|256 forces one (tuning aid).
+    const long wg256 = static_cast<long>((N + 255) / 256) * ((M + 63) / 64);
+    const int bn = forced_bn ? forced_bn : (wg256 <= 640 ? 128 : 256);
+    if constexpr (sizeof(Act) == 2) {
+        if (prefill_dma_ok(x, M, N, K) && (bm == 64 || bm == 128)) {
+            if (bm == 64 && bn == 128) launch_prefill_packed_dma_as<2, 1>(x, packed, out, ep, M, N, K, st);
+            else if (bm == 128) launch_prefill_packed_dma_as<4, 2>(x, packed, out, ep, M, N, K, st);
+            else launch_prefill_packed_dma_as<2, 2>(x, packed, out, ep, M, N, K, st);
+            return;
+        }
+    }
+    if (bm == 64 && bn == 128) launch_prefill_packed_as<Act, 2, 1>(x, packed, out, ep, M, N, K, st);
+    else if (bm == 256) launch_prefill_packed_as<Act, 8>(x, packed, out, ep, M, N, K, st);
+    else if (bm == 96) launch_prefill_packed_as<Act, 3>(x, packed, out, ep, M, N, K, st);
     else if (bm == 128) launch_prefill_packed_as<Act, 4>(x, packed, out, ep, M, N, K, st);
     else launch_prefill_packed_as<Act, 2>(x, packed, out, ep, M, N, K, st);
 }

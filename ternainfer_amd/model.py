@@ -46,9 +46,8 @@ def random_p2_weight(n: int, k: int, p_zero: float, gen: torch.Generator, device
     u = torch.rand((n // 16, 16, k // 64, 4, 16), generator=gen, device=device)           # band, i, gk, g, q
     neg = torch.rand(u.shape, generator=gen, device=device) < 0.5
     code = (u >= p_zero).to(torch.int64) | ((u >= p_zero) & neg).to(torch.int64) << 1
-    q = torch.arange(16, device=device)
-    t, c = (q >> 1) & 1, 2 * (q >> 2) + (q & 1)
-    shift = 8 * (c & 3) + 2 * (2 * t + (c >> 2))
+    j = torch.arange(16, device=device)
+    shift = 8 * (j & 3) + 2 * (j >> 2)
     words = (code << shift).sum(dim=-1)                                                     # band, i, gk, g
     words = words.permute(0, 2, 1, 3).contiguous().view(n // 16, k // 64, 64)
     return (words - ((words >> 31) << 32)).to(torch.int32)                                  # same 32 bits, signed storage

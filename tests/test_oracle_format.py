@@ -159,9 +159,8 @@ def test_p2_pack_round_trip_and_field_positions():
         one = np.zeros((128, 192), np.int8)
         one[row, col] = sign
         p = O.pack_p2(one)
-        q = col & 15
-        t, c = (q >> 1) & 1, 2 * (q >> 2) + (q & 1)
-        bit = 8 * (c & 3) + 2 * (2 * t + (c >> 2))
+        j = col & 15
+        bit = 8 * (j & 3) + 2 * (j >> 2)
         want = np.zeros_like(p)
         want[row >> 4, col >> 6, 4 * (row & 15) + ((col >> 4) & 3)] = (3 if sign < 0 else 1) << bit
         assert (p == want).all()
