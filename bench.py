@@ -32,6 +32,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 BF16_MFMA_PEAK_TFLOPS = 2500.0
+INT8_MFMA_PEAK_TOPS = 5000.0
 LAYER_SET = [("wqkv", 3840, 2560), ("wo", 2560, 2560), ("w13", 13824, 2560), ("w2", 2560, 6912)]   # (name, N, K)
 
 # HBM bytes per launch of the small-M kernel on the default workload (M=8, average over the four
@@ -178,6 +179,7 @@ def run_model(args, torch):
     from ternainfer_amd.model import ModelArgs, Transformer, greedy_decode
     margs = ModelArgs()
     t0 = time.perf_counter()
+    args.act = args.act or "int8"
     model = Transformer(margs, seed=20260500, act=args.act)
     torch.cuda.synchronize()
     build_s = time.perf_counter() - t0
@@ -201,9 +203,14 @@ def run_model(args, torch):
 
 def run_prefill(args, torch, T, lib):
     """configs[2]: the four BitNet-2B matrices at M in {256, 512, 2048}, bf16 activations with 1% of
-    the channels scaled x20.  A step is one pass over the four matrices at M = --m (default 2048
-    when --workload prefill is given without --m)."""
+    the channels scaled x20 (--act int8: the same activations quantised per row to int8, the
+    reference's own prefill input).  A step is one pass over the four matrices at M = --m (default
+    2048 when --workload prefill is given without --m).  Next to every shape the vendor's dense GEMM
+    (torch.matmul / torch._int_mm on already expanded weights) is timed as a yardstick."""
     m_main = args.m if args.m >= 64 else 2048
+    act = args.act or "bf16"
+    if act == "int8" and args.layout != "packed":
+        sys.exit("bench.py: --workload prefill --act int8 runs on the packed layout")
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     rng = np.random.default_rng(20260300)
     mats = []
@@ -214,13 +221,24 @@ def run_prefill(args, torch, T, lib):
             xf = rng.standard_normal((m, k)).astype(np.float32)
             ch = rng.permutation(k)[: int(np.ceil(0.01 * k))]
             xf[:, ch] *= 20.0
-            xs[m] = (torch.from_numpy(f32_to_bf16_bits(xf).view(np.int16)).cuda(),
-                     torch.zeros((m, n), dtype=torch.int16, device="cuda"))
+            if act == "bf16":
+                xs[m] = (torch.from_numpy(f32_to_bf16_bits(xf).view(np.int16)).cuda(),
+                         torch.zeros((m, n), dtype=torch.int16, device="cuda"))
+            else:                  # per-row absmax quantisation, as the reference's quant_input (model.py:60-63)
+                sc = 127.0 / np.maximum(np.abs(xf).max(axis=1, keepdims=True), 1e-5)
+                xq = np.clip(np.rint(xf * sc), -128, 127).astype(np.int8)
+                xs[m] = (torch.from_numpy(xq).cuda(), torch.zeros((m, n), dtype=torch.int16, device="cuda"),
+                         torch.from_numpy(f32_to_bf16_bits(sc.astype(np.float32).ravel()).view(np.int16)).cuda())
+        mt.ws = torch.from_numpy(f32_to_bf16_bits(mt.scale_host).view(np.int16)).cuda()
         mats.append((mt, xs))
 
     work = torch.empty(13824 * 2560, dtype=torch.int8, device="cuda")      # the reference's global workspace
 
     def launch(mt, xs, m, s):
+        if act == "int8":
+            x, out, srow = xs[m]
+            lib.bitlinear_TernaSpMM_packed(vp(x), vp(mt.packed[0]), vp(out), vp(srow), vp(mt.ws), 1, m, mt.n, mt.k, 0, s)
+            return
         x, out = xs[m]
         if args.layout == "packed":
             lib.bitlinear_TernaSpMM_bf16_packed(vp(x), vp(mt.packed[0]), vp(out), vp(mt.scale), 1, m, mt.n, mt.k, 0, s)
@@ -229,7 +247,33 @@ def run_prefill(args, torch, T, lib):
             lib.bitlinear_TernaSpMM_bf16(vp(x), vp(bm), vp(off), vp(med), vp(vals), vp(out), vp(mt.scale),
                                          1, m, mt.n, mt.k, 1, vp(work), s)
 
+    peak = BF16_MFMA_PEAK_TFLOPS if act == "bf16" else INT8_MFMA_PEAK_TOPS
+
+    def dense_us(m, n, k):
+        """Vendor dense GEMM of the same shape on expanded weights (not part of the product)."""
+        if act == "bf16":
+            a = torch.randn(m, k, device="cuda", dtype=torch.bfloat16)
+            b = torch.randn(n, k, device="cuda", dtype=torch.bfloat16).t()
+            f = lambda: torch.matmul(a, b)
+        else:
+            a = torch.randint(-127, 128, (m, k), device="cuda", dtype=torch.int8)
+            b = torch.randint(-1, 2, (n, k), device="cuda", dtype=torch.int8).t()
+            f = lambda: torch._int_mm(a, b)
+        try:
+            for _ in range(3):
+                f()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(10):
+                f()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e3 / 10
+        except Exception:                                   # no such vendor kernel in this build
+            return None
+
     per_shape = {}
+    dense_main_us = 0.0
     for mt, xs in mats:
         for m in sorted(xs):
             launch(mt, xs, m, stream)
@@ -237,7 +281,13 @@ def run_prefill(args, torch, T, lib):
             g = capture(torch, lambda s, mt=mt, xs=xs, m=m: [launch(mt, xs, m, s) for _ in range(10)])
             us = time_graph(torch, g, 5, 2) * 1e3 / 10
             tf = 2.0 * m * mt.n * mt.k / us / 1e6
-            per_shape[f"{mt.name}_{mt.k}x{mt.n}_M{m}"] = {"us": us, "tflops": tf, "frac": tf / BF16_MFMA_PEAK_TFLOPS}
+            d_us = None if args.no_per_shape else dense_us(m, mt.n, mt.k)
+            per_shape[f"{mt.name}_{mt.k}x{mt.n}_M{m}"] = {"us": us, "tflops": tf, "frac": tf / peak,
+                                                         "vendor_dense_gemm_us": d_us}
+            if m == m_main and d_us is not None and dense_main_us is not None:
+                dense_main_us += d_us
+            elif m == m_main:
+                dense_main_us = None
 
     graph = capture(torch, lambda s: [launch(mt, xs, m_main, s) for mt, xs in mats])
     for _ in range(args.warmup):
@@ -253,18 +303,24 @@ def run_prefill(args, torch, T, lib):
     flops = sum(2.0 * m_main * mt.n * mt.k for mt, _ in mats)
     tf = flops / (ms * 1e-3) / 1e12
     print(json.dumps({
-        "metric": "TernaSpMM prefill TFLOP/s + %bf16 MFMA peak (M=2048, BitNet-2B layer set)",
-        "value": tf, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "metric": "TernaSpMM prefill TFLOP/s + %bf16 MFMA peak (M=2048, BitNet-2B layer set)" if act == "bf16"
+                  else "TernaSpMM prefill TOP/s, int8 activations (M=2048, BitNet-2B layer set)",
+        "value": tf, "unit": "TFLOP/s" if act == "bf16" else "TOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if act == "bf16" else "int8",
         "data": "synthetic",
-        "config": {"workload": f"configs[2]: four BitNet-b1.58-2B matrices at M={m_main}, P(0)=0.40, bf16 activations "
+        "config": {"workload": f"configs[2]: four BitNet-b1.58-2B matrices at M={m_main}, P(0)=0.40, {act} activations "
                                "with 1% outlier channels (x20), HIP-graph replay; weight layout: "
                                + ("P2, repacked once at load time" if args.layout == "packed"
                                   else "reference format, transcoded into the workspace on every call"),
                    "m": m_main, "layout": args.layout},
-        "roofline": {"bound": "mfma", "achieved": tf, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tf / BF16_MFMA_PEAK_TFLOPS, "traffic": None,
-                     "kernel": "terna_prefill_packed_kernel<bf16>", "algorithmic_flops_per_step": flops},
+        "roofline": {"bound": "mfma", "achieved": tf, "peak": peak, "unit": "TFLOP/s" if act == "bf16" else "TOP/s",
+                     "frac": tf / peak, "traffic": None,
+                     "kernel": f"terna_prefill_packed_dma_kernel<{act}>", "algorithmic_flops_per_step": flops},
+        "vendor_dense_gemm": None if not dense_main_us else {
+            "what": "torch.matmul (bf16) / torch._int_mm (int8) on already expanded weights, same four shapes, eager",
+            "ms_per_step": dense_main_us * 1e-3, "rate": flops / (dense_main_us * 1e-6) / 1e12},
         "per_shape": per_shape}))
 
 
@@ -279,8 +335,9 @@ def main():
                     help="decode: the headline small-M HBM-bound pass; prefill: the M>=256 MFMA-bound pass; "
                          "model: random-init BitNet-2B-shaped decoder, 128-token prompt + 256 greedy tokens")
     ap.add_argument("--batch", type=int, default=1, help="sequences decoded together (model workload)")
-    ap.add_argument("--act", choices=["int8", "bf16"], default="int8",
-                    help="model workload: int8-quantised activations (the reference's SpBitLinear) or bf16")
+    ap.add_argument("--act", choices=["int8", "bf16"], default=None,
+                    help="activations into the ternary linears: int8 + per-row scale (the reference's SpBitLinear; "
+                         "default of the model workload) or bf16 (default of the prefill workload)")
     ap.add_argument("--layout", choices=["packed", "reference"], default="packed",
                     help="packed: weights repacked once at load time to the library's P2 layout (bit-exact); "
                          "reference: kernels read the reference's compressed format directly")

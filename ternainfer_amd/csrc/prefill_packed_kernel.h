@@ -40,10 +40,10 @@ __device__ __forceinline__ void int8x16_to_bf16(const u32x4& v, u32x4& c0, u32x4
 }
 
 // Fused epilogue of one wave's NA x MB accumulator tiles (v_mfma_f32_32x32x16 layout: lane holds
-// column m = L % 32 and rows n = (v&3) + 8(v>>2) + 4(L/32) of each tile).  The accumulator is half
-// the true sum (weights were +-0.5); x2 is exact.
-template <int MB, int NA>
-__device__ __forceinline__ void packed_prefill_epilogue(f32x16 (&acc)[NA][MB], uint16_t* __restrict__ out,
+// column m = L % 32 and rows n = (v&3) + 8(v>>2) + 4(L/32) of each tile).  A float accumulator is
+// half the true sum (weights were +-0.5; x2 is exact); an integer one is the sum itself.
+template <int MB, int NA, typename AccV>
+__device__ __forceinline__ void packed_prefill_epilogue(AccV (&acc)[NA][MB], uint16_t* __restrict__ out,
                                                         const Epilogue& ep, int M, int N, int n_wave, int m0, int lane)
 {
     const int kb = lane >> 5, l32 = lane & 31;
@@ -66,7 +66,12 @@ __device__ __forceinline__ void packed_prefill_epilogue(f32x16 (&acc)[NA][MB], u
             for (int v = 0; v < 4; ++v) eb.w[v] = wv[v];
             uint16_t o[4];
 #pragma unroll
-            for (int v = 0; v < 4; ++v) o[v] = apply_epilogue<float>(ep.kind, eb, v, acc[a][b][4 * vq + v] * 2.0f);
+            for (int v = 0; v < 4; ++v) {
+                if constexpr (std::is_same<AccV, f32x16>::value)
+                    o[v] = apply_epilogue<float>(ep.kind, eb, v, acc[a][b][4 * vq + v] * 2.0f);
+                else
+                    o[v] = apply_epilogue<int>(ep.kind, eb, v, acc[a][b][4 * vq + v]);
+            }
             const u32x2 pk = {o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16)};
             if (m_of[b] < M && n < N) *reinterpret_cast<u32x2*>(out + static_cast<size_t>(m_of[b]) * N + n) = pk;
         });
@@ -240,7 +245,7 @@ __global__ __launch_bounds__(256, MB == 8 ? 1 : (MB == 3 ? 3 : 2)) void terna_pr
 }
 
 // ------------------------------------------------------------------------------------------------
-// bf16-activation variant whose activation tile goes global memory -> LDS directly
+// Variant (bf16 or int8 activations) whose activation tile goes global memory -> LDS directly
 // (global_load_lds_dwordx4), with every load of the main loop issued and awaited by hand.
 //
 // Why by hand: the loop keeps two k-steps of loads in flight and each wait must leave exactly the
@@ -248,17 +253,13 @@ __global__ __launch_bounds__(256, MB == 8 ? 1 : (MB == 3 ? 3 : 2)) void terna_pr
 // known n per k-step -- folded into the step's only barrier.  Loads written as ordinary C++ get
 // their waits from the compiler, which at loop headers settles for far stricter ones.
 //
-// Activation tile in LDS: NST stages of BM rows x 128 bytes (one k-step = 64 bf16 per row), as 8
+// Activation tile in LDS: three stages of BM rows x 128 bytes (one step = 64 bf16 or 128 int8), as 8
 // pieces of 16 bytes; piece p of row r sits at position p ^ swizzle(r), so that the 16-byte
 // operand reads of 32 consecutive rows spread over all banks.  One direct load writes 64 lanes x
 // 16 bytes = 8 whole rows (lane = 8*row + position) and reads whole 128-byte lines from memory.
 //
-// Per k-step k (stage k % 3, weight buffer k & 1):
-//   issue X(k+2) -> stage (k+2) % 3        (last read in step k-1, before that step's barrier)
-//   MFMAs of step k
-//   issue W(k+2) -> the buffer step k just used
-//   s_waitcnt vmcnt(MB + NA): everything but X(k+2), W(k+2) has landed, i.e. X(k+1) and W(k+1)
-//   s_barrier                               (also orders step k's operand reads before X(k+3))
+// Three stages: while step k multiplies out of stage k % 3, X(k+1) is landing in the next one and
+// X(k+2) is issued into the third (see the step description inside the kernel).
 constexpr int kXSwizzleShift = 1;
 __device__ __forceinline__ constexpr int x_swizzle(int row) { return (row >> kXSwizzleShift) & 7; }
 
@@ -288,13 +289,18 @@ struct PackedPrefillDmaSmem {
     static constexpr int kBytes = kStages * kStage;
 };
 
-template <int MB, int NA>
+template <typename Act, int MB, int NA>
 __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) void terna_prefill_packed_dma_kernel(
-    const uint16_t* __restrict__ x, const uint32_t* __restrict__ packed, uint16_t* __restrict__ out,
+    const Act* __restrict__ x, const uint32_t* __restrict__ packed, uint16_t* __restrict__ out,
     Epilogue ep, int M, int N, int K)
 {
     using S = PackedPrefillDmaSmem<MB>;
     constexpr int BN = 128 * NA, BM = S::BM;
+    // One step is 128 bytes of every activation row: 64 bf16 columns (one 64-column weight tile,
+    // v_mfma_f32_32x32x16_bf16) or 128 int8 columns (two tiles, v_mfma_i32_32x32x32_i8; the lanes
+    // of k-half kb take tile 2*step + kb whole, one 16-column word per MFMA).
+    constexpr bool I8 = sizeof(Act) == 1;
+    using AccV = typename std::conditional<I8, i32x16, f32x16>::type;
     static_assert(NA == 1 || NA == 2, "32 or 64 output features per wave");
     static_assert(MB == 2 || MB == 4, "batch tile of 64 or 128 rows (all stages below 64 KiB of LDS)");
 
@@ -305,27 +311,33 @@ __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) voi
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n0 = blockIdx.x * BN, m0 = blockIdx.y * BM;
     const int ktiles = K >> 6;
+    const int steps = I8 ? (ktiles + 1) >> 1 : ktiles;
+    // int8 with an odd tile count: in the last step the kb = 1 half has no tile.  Its loads are
+    // pulled back onto the kb = 0 half's addresses (in bounds) and its weights are zeroed.
+    const bool half_tail = I8 && (ktiles & 1);
     const int last_band = (N >> 4) - 1;
     const int kb = lane >> 5, l32 = lane & 31;
 
-    // ---- weights: row-tile a -> band (n0/16 + 2*NA*wave + 2a + l32/16), row l32 % 16; one k-step is 256 bytes
+    // ---- weights: row-tile a -> band (n0/16 + 2*NA*wave + 2a + l32/16), row l32 % 16; a tile is 256 bytes
+    constexpr int kWStep = I8 ? 512 : 256;
     uint32_t w_off[NA];
 #pragma unroll
     for (int a = 0; a < NA; ++a) {
         int band = (n0 >> 4) + 2 * NA * wave + 2 * a + (l32 >> 4);
         band = band < last_band ? band : last_band;   // a tile hanging over N re-reads the last band; never stored
-        w_off[a] = static_cast<uint32_t>(band) * static_cast<uint32_t>(ktiles) * 256u + (l32 & 15) * 16;
+        w_off[a] = static_cast<uint32_t>(band) * static_cast<uint32_t>(ktiles) * 256u + (l32 & 15) * 16 + (I8 ? kb * 256 : 0);
     }
     const uint8_t* w_base = reinterpret_cast<const uint8_t*>(packed);
     // ---- activations: direct load j of this wave fills rows 8*(wave + 4j) .. +7 of the stage
-    uint32_t x_off[MB];
+    uint32_t x_off[MB], x_tail[MB];
 #pragma unroll
     for (int j = 0; j < MB; ++j) {
         const int row = 8 * (wave + 4 * j) + (lane >> 3);
         const int piece = (lane & 7) ^ x_swizzle(row);
         int m = m0 + row;
         m = m < M ? m : M - 1;
-        x_off[j] = static_cast<uint32_t>(m) * static_cast<uint32_t>(K) * 2u + piece * 16;
+        x_off[j] = static_cast<uint32_t>(m) * static_cast<uint32_t>(K) * static_cast<uint32_t>(sizeof(Act)) + piece * 16;
+        x_tail[j] = piece >= 4 ? 64 : 0;
     }
     const uint8_t* x_base = reinterpret_cast<const uint8_t*>(x);
     const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem)) + wave * 1024;
@@ -334,98 +346,127 @@ __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) voi
     auto next_stage = [](int st) { return st == 2 * S::kStage ? 0 : st + S::kStage; };
     auto issue_x = [&](int kk, int st) {
         const uint8_t* base = x_base + static_cast<size_t>(kk) * 128;
+        const bool pull_back = half_tail && kk == steps - 1;
 #pragma unroll
-        for (int j = 0; j < MB; ++j) lds_dma_b128(base, x_off[j], lds0 + st + j * 4096);
+        for (int j = 0; j < MB; ++j)
+            lds_dma_b128(base, pull_back ? x_off[j] - x_tail[j] : x_off[j], lds0 + st + j * 4096);
     };
     struct RawW { u32x4 w[NA]; };
     auto fetch_w = [&](RawW& r, int kk) {
-        const uint8_t* base = w_base + static_cast<size_t>(kk) * 256;
+        const uint8_t* base = w_base + static_cast<size_t>(kk) * kWStep;
+        const bool pull_back = half_tail && kk == steps - 1;
 #pragma unroll
-        for (int a = 0; a < NA; ++a) global_load_b128_nowait(r.w[a], base, w_off[a]);
+        for (int a = 0; a < NA; ++a) global_load_b128_nowait(r.w[a], base, pull_back ? w_off[a] - kb * 256 : w_off[a]);
     };
 
-    f32x16 acc[NA][MB];
-    {
-        const f32x16 zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    AccV acc[NA][MB];
 #pragma unroll
-        for (int a = 0; a < NA; ++a)
-#pragma unroll
-            for (int b = 0; b < MB; ++b) acc[a][b] = zero;
-    }
-
-    // B operand of (group g, tile b): row 32b + l32, piece 2g + kb; swizzle(32b + l32) == swizzle(l32)
-    int b_off[4];
-#pragma unroll
-    for (int g = 0; g < 4; ++g) b_off[g] = l32 * 128 + (((2 * g + kb) ^ x_swizzle(l32)) * 16);
-    const int wshift = 4 * kb;                               // columns 8kb .. 8kb+7 of every word
-
-    struct BOps { bf16x8 b[MB]; };
-    auto load_b = [&](const uint8_t* stage, int g, BOps& r) {
+    for (int a = 0; a < NA; ++a)
 #pragma unroll
         for (int b = 0; b < MB; ++b)
-            r.b[b] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(stage + b_off[g] + b * 4096));
-    };
-    // The scheduling fences keep the operand reads one group ahead of their MFMAs (hoisting all
-    // of them to the top costs 8*MB registers) and every MFMA of the step before its barrier.
-    auto mma_step = [&](const RawW& rw, int st) {
-        const uint8_t* stage = smem + st;
-        BOps bcur;
-        load_b(stage, 0, bcur);
-        static_for<0, 4>([&](auto gc) {
-            constexpr int g = decltype(gc)::value;
-            BOps bnxt;
-            if constexpr (g < 3) load_b(stage, g + 1, bnxt);
 #pragma unroll
-            for (int a = 0; a < NA; ++a) {
+            for (int v = 0; v < 16; ++v) acc[a][b][v] = 0;
+
+    // B operand of (group g, tile b): row 32b + l32, piece 2g + kb (bf16: columns 16g + 8kb .. +7)
+    // or 4kb + g (int8: columns 64kb + 16g .. +15); swizzle(32b + l32) == swizzle(l32)
+    int b_off[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) b_off[g] = l32 * 128 + ((((I8 ? 4 * kb + g : 2 * g + kb)) ^ x_swizzle(l32)) * 16);
+    const int wshift = 4 * kb;                               // bf16: columns 8kb .. 8kb+7 of every word
+
+    struct BOps { u32x4 b[MB]; };
+    auto load_b = [&](int st, int g, BOps& r) {
+        const uint8_t* stage = smem + st;
+#pragma unroll
+        for (int b = 0; b < MB; ++b) r.b[b] = *reinterpret_cast<const u32x4*>(stage + b_off[g] + b * 4096);
+    };
+    // One 16-column group: expand the NA weight operands and issue NA*MB MFMAs against `bcur`.
+    auto mma_group = [&](const RawW& rw, auto gc, const BOps& bcur) {
+        constexpr int g = decltype(gc)::value;
+#pragma unroll
+        for (int a = 0; a < NA; ++a) {
+            if constexpr (I8) {
+                const i32x4 af = expand_word_i8(rw.w[a][g]);
+#pragma unroll
+                for (int b = 0; b < MB; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, __builtin_bit_cast(i32x4, bcur.b[b]), acc[a][b], 0, 0, 0);
+            } else {
                 const bf16x8 af = __builtin_bit_cast(bf16x8, expand_chunk_bf16(rw.w[a][g] >> wshift));
 #pragma unroll
                 for (int b = 0; b < MB; ++b)
-                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bcur.b[b], acc[a][b], 0, 0, 0);
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, __builtin_bit_cast(bf16x8, bcur.b[b]), acc[a][b], 0, 0, 0);
             }
-            if constexpr (g < 3) bcur = bnxt;
-            __builtin_amdgcn_sched_barrier(0);
-        });
+        }
     };
 
     // A hand-issued load writes its registers (or LDS) whenever it lands, which the compiler does
     // not know: every one of them must be followed, on every path, by a wait that covers it
-    // before its destination can be reused -- so none is issued for steps past the end, and the
-    // last two steps wait for everything.
+    // before its destination can be reused -- so none is issued for steps past the end.
+    //
+    // Step k, with its one barrier in the middle (so that the operand reads of the next group
+    // are always in flight across it and across the step boundary):
+    //   groups 0, 1                       operands of group g+1 are read while group g multiplies
+    //   s_waitcnt vmcnt(NA); s_barrier    own part of X(k+1) landed; everybody is past step k-1
+    //   issue X(k+2) -> stage (k+2) % 3   == stage of step k-1, which nobody reads any more
+    //   groups 2, 3                       group 3 reads group 0 of step k+1
+    //   issue W(k+2); s_waitcnt vmcnt(MB + NA)   W(k+1) landed; X(k+2), W(k+2) stay in flight
+    // The scheduling fences keep the compiler from hoisting operand reads (8*MB registers if all
+    // go to the top) or sinking MFMAs across the hand-placed waits.
     RawW w0, w1;
+    BOps b_a, b_b;
     int st_mma = 0;                                          // stage of the step being multiplied
     int st_dma = 2 * S::kStage;                              // stage that the next direct load fills
     issue_x(0, 0);
     fetch_w(w0, 0);
-    if (ktiles > 1) {
+    if (steps > 1) {
         issue_x(1, S::kStage);
         fetch_w(w1, 1);
         wait_loads_and_barrier<MB + NA>();
     } else {
         wait_loads_and_barrier<0>();
     }
+    load_b(0, 0, b_a);
     auto body = [&](int k, RawW& w) {
-        const bool more = k + 2 < ktiles;                    // uniform
-        if (more) issue_x(k + 2, st_dma);
+        const bool more1 = k + 1 < steps, more2 = k + 2 < steps;        // uniform
+        const int st_next = next_stage(st_mma);
 #pragma unroll
         for (int a = 0; a < NA; ++a) landed(w.w[a]);
-        __builtin_amdgcn_sched_barrier(0);
-        mma_step(w, st_mma);
-        if (more) {
-            fetch_w(w, k + 2);
-            wait_loads_and_barrier<MB + NA>();
-        } else {
-            wait_loads_and_barrier<0>();
+        if (half_tail && !more1 && kb) {
+#pragma unroll
+            for (int a = 0; a < NA; ++a) w.w[a] = u32x4{0u, 0u, 0u, 0u};
         }
         __builtin_amdgcn_sched_barrier(0);
-        st_mma = next_stage(st_mma);
+        load_b(st_mma, 1, b_b);
+        mma_group(w, std::integral_constant<int, 0>{}, b_a);
+        __builtin_amdgcn_sched_barrier(0);
+        load_b(st_mma, 2, b_a);
+        mma_group(w, std::integral_constant<int, 1>{}, b_b);
+        __builtin_amdgcn_sched_barrier(0);
+        if (more1) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(NA) : "memory");
+        if (more2) issue_x(k + 2, st_dma);
+        __builtin_amdgcn_sched_barrier(0);
+        load_b(st_mma, 3, b_b);
+        mma_group(w, std::integral_constant<int, 2>{}, b_a);
+        __builtin_amdgcn_sched_barrier(0);
+        if (more1) load_b(st_next, 0, b_a);
+        mma_group(w, std::integral_constant<int, 3>{}, b_b);
+        __builtin_amdgcn_sched_barrier(0);
+        if (more2) {
+            fetch_w(w, k + 2);
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(MB + NA) : "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        st_mma = st_next;
         st_dma = next_stage(st_dma);
     };
     int k = 0;
-    for (; k + 1 < ktiles; k += 2) {
+    for (; k + 1 < steps; k += 2) {
         body(k, w0);
         body(k + 1, w1);
     }
-    if (k < ktiles) body(k, w0);
+    if (k < steps) body(k, w0);
 
     packed_prefill_epilogue<MB, NA>(acc, out, ep, M, N, n0 + 32 * NA * wave, m0, lane);
 }

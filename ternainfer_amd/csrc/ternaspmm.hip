@@ -159,12 +159,12 @@ void launch_prefill_packed_as(const Act* x, const uint32_t* packed, uint16_t* ou
     kernel<<<grid, dim3(256), S::kBytes, st>>>(x, packed, out, ep, M, N, K);
 }
 
-template <int MB, int NA>
-void launch_prefill_packed_dma_as(const uint16_t* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M,
+template <typename Act, int MB, int NA>
+void launch_prefill_packed_dma_as(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M,
                                   int N, int K, hipStream_t st)
 {
     using S = PackedPrefillDmaSmem<MB>;
-    auto kernel = terna_prefill_packed_dma_kernel<MB, NA>;
+    auto kernel = terna_prefill_packed_dma_kernel<Act, MB, NA>;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, S::kBytes);
     if (attr != hipSuccess) die("hipFuncSetAttribute(prefill packed dma)", attr, __LINE__);
@@ -175,13 +175,13 @@ void launch_prefill_packed_dma_as(const uint16_t* x, const uint32_t* packed, uin
 
 // The direct-to-LDS kernel addresses both operands as a 64-bit base plus a 32-bit byte offset and
 // loads 16-byte pieces of the activation rows.
-inline bool prefill_dma_ok(const void* x, int M, int N, int K)
+inline bool prefill_dma_ok(const void* x, size_t act_bytes, int M, int N, int K)
 {
     static const bool off = [] {
         const char* v = std::getenv("TERNASPMM_PREFILL_DMA");
         return v && std::atoi(v) == 0;
     }();
-    return !off && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && static_cast<uint64_t>(M) * K * 2 < (1ull << 32) &&
+    return !off && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && static_cast<uint64_t>(M) * K * act_bytes < (1ull << 32) &&
            static_cast<uint64_t>(N) * K / 4 < (1ull << 32);
 }
 
@@ -208,13 +208,12 @@ void launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, 
     // double the workgroup count instead.  TERNASPMM_PREFILL_BN=128|256 forces one (tuning aid).
     const long wg256 = static_cast<long>((N + 255) / 256) * ((M + 63) / 64);
     const int bn = forced_bn ? forced_bn : (wg256 <= 640 ? 128 : 256);
-    if constexpr (sizeof(Act) == 2) {
-        if (prefill_dma_ok(x, M, N, K) && (bm == 64 || bm == 128)) {
-            if (bm == 64 && bn == 128) launch_prefill_packed_dma_as<2, 1>(x, packed, out, ep, M, N, K, st);
-            else if (bm == 128) launch_prefill_packed_dma_as<4, 2>(x, packed, out, ep, M, N, K, st);
-            else launch_prefill_packed_dma_as<2, 2>(x, packed, out, ep, M, N, K, st);
-            return;
-        }
+    if (prefill_dma_ok(x, sizeof(Act), M, N, K) && (bm == 64 || bm == 128)) {
+        if (bm == 64 && bn == 128) launch_prefill_packed_dma_as<Act, 2, 1>(x, packed, out, ep, M, N, K, st);
+        else if (bm == 128 && forced_bn == 128) launch_prefill_packed_dma_as<Act, 4, 1>(x, packed, out, ep, M, N, K, st);
+        else if (bm == 128) launch_prefill_packed_dma_as<Act, 4, 2>(x, packed, out, ep, M, N, K, st);
+        else launch_prefill_packed_dma_as<Act, 2, 2>(x, packed, out, ep, M, N, K, st);
+        return;
     }
     if (bm == 64 && bn == 128) launch_prefill_packed_as<Act, 2, 1>(x, packed, out, ep, M, N, K, st);
     else if (bm == 256) launch_prefill_packed_as<Act, 8>(x, packed, out, ep, M, N, K, st);

@@ -423,6 +423,17 @@ def test_packed_int8_bit_exact(lib, m, n, k, ws_num):
     assert (run_i8_packed(lib, packed, n, xq, s, WS, ws_num, 1) == O.spmm_i8(xq, w, s, WS, ws_num, 1)).all()
 
 
+@pytest.mark.parametrize("m", [1, 70, 256])
+@pytest.mark.parametrize("n,k,ws_num", [(64, 64, 1), (192, 448, 1), (3840, 2560, 3), (2560, 6912, 1)])
+def test_packed_int8_mfma_kernel_tile_counts_and_2b_shapes(lib, m, n, k, ws_num):
+    """The large-M int8 kernel walks K two 64-column tiles at a time: one tile (K = 64), an odd count
+    (K = 448), and the even counts of the 2B matrices, forced onto that kernel at every M."""
+    w = make_ternary(n, k, 0.40, 440 + m + n)
+    packed = repack(lib, DeviceFormat(w))
+    xq, s = make_int8_activations(m, k, 450 + m + k)
+    assert (run_i8_packed(lib, packed, n, xq, s, WS, ws_num, 1) == O.spmm_i8(xq, w, s, WS, ws_num, 1)).all()
+
+
 @pytest.mark.parametrize("route", [1, 2])
 @pytest.mark.parametrize("m", [1, 3, 16, 17, 64, 100, 256, 300])
 @pytest.mark.parametrize("n,k", [(256, 64), (320, 128), (512, 320)])
