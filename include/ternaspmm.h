@@ -147,6 +147,24 @@ void bitlinear_TernaSpMM_bf16_packed(const terna_bf16* x, const void* packed, te
 void bitlinear_TernaSpMM_packed(const int8_t* x, const void* packed, terna_bf16* out, const terna_bf16* s,
                                 const terna_bf16* ws, int ws_num, int M, int N, int K, int route, terna_stream stream);
 
+/* ---- Fused prologue of a ternary linear (no counterpart in the reference's library) -----------------
+ * One launch replaces the PyTorch / xformers / Inductor kernels the reference runs between two bitlinear
+ * calls: the residual add and block norm (model.py:330, :334), the sub-norms (model.py:236, :280), the
+ * gate squared_relu(x1) * x3 (model.py:279-280) and SpBitLinear.quant_input (model.py:120-123).  Per row:
+ *   h = x, or bf16(x + residual) when residual != NULL (written to sum_out when that is non-NULL)
+ *   y = bf16(h * rsqrt(mean(h^2) + eps) * weight)                       fp32 inside
+ *   s = bf16(127 / max(max|y|, 1e-5)),  xq = clamp(rint(y * s), -128, 127)
+ * y_out (bf16 [M][K]) and the pair xq_out (int8 [M][K]) / s_out (bf16 [M]) are each optional (NULL = not
+ * written); xq_out / s_out feed bitlinear_TernaSpMM* directly.  K % 8 == 0, K <= 8192.  Only enqueues. */
+void ternaspmm_rmsnorm_quant(const terna_bf16* x, const terna_bf16* residual, terna_bf16* sum_out,
+                             const terna_bf16* weight, float eps, terna_bf16* y_out, int8_t* xq_out,
+                             terna_bf16* s_out, int M, int K, terna_stream stream);
+
+/* Same with h = bf16(bf16(relu(x1)^2) * x3), x1 = x13[m][0:F], x3 = x13[m][F:2F] (x13 is the gate/up
+ * linear's output, bf16 [M][2F]); the norm and the quantisation run over F columns. */
+void ternaspmm_relu2_mul_rmsnorm_quant(const terna_bf16* x13, const terna_bf16* weight, float eps, terna_bf16* y_out,
+                                       int8_t* xq_out, terna_bf16* s_out, int M, int F, terna_stream stream);
+
 /* Library version string, e.g. "ternaspmm-gfx950 0.1". */
 const char* ternaspmm_version(void);
 

@@ -21,7 +21,12 @@ Reference files restated (paths relative to the reference checkout):
 
 Parity status: every function is pinned by a test in tests/test_oracle_*.py except
 ``quant_input``'s intermediate precision, which the reference leaves open
-("parity unpinned" beyond the two-line formula).
+("parity unpinned" beyond the two-line formula), and ``rmsnorm``: the reference takes
+RMSNorm from xformers.ops (model.py:16), a third-party dependency that is not part of
+the reference checkout and not installed here, so "parity unpinned"; the formula
+y = x * rsqrt(mean(x^2) + eps) * weight, fp32 inside and one rounding to the tensor's
+dtype, restates that operator's published definition and is checked against what the
+mathematics fixes (tests/test_oracle_linear.py).
 """
 from __future__ import annotations
 
@@ -253,6 +258,31 @@ def quant_input(x_bits: np.ndarray):
     s = bf16_bits_to_f32(s_bits)
     q = np.clip(np.rint((x * s).astype(np.float32)), -128, 127).astype(np.int8)
     return q, s_bits.reshape(-1)
+
+
+# --------------------------------------------------------------------------- glue between two linears
+def residual_add(x_bits: np.ndarray, r_bits: np.ndarray) -> np.ndarray:
+    """model.py:330, :334: bf16 + bf16 -> bf16 (the fp32 sum rounded once more to bf16)."""
+    return f32_to_bf16_bits(bf16_bits_to_f32(x_bits) + bf16_bits_to_f32(r_bits))
+
+
+def relu2_mul(x13_bits: np.ndarray) -> np.ndarray:
+    """model.py:243, :279-280: squared_relu(x1) * x3 on bf16 tensors, every op rounded to bf16."""
+    f = x13_bits.shape[-1] // 2
+    x1 = bf16_bits_to_f32(x13_bits[..., :f])
+    x3 = bf16_bits_to_f32(x13_bits[..., f:])
+    r = np.maximum(x1, np.float32(0))
+    sq = bf16_bits_to_f32(f32_to_bf16_bits(r * r))
+    return f32_to_bf16_bits(sq * x3)
+
+
+def rmsnorm(h_bits: np.ndarray, w_bits: np.ndarray, eps: float) -> np.ndarray:
+    """RMSNorm over the last axis, evaluated in float64 and rounded to bf16 (see the module header:
+    parity unpinned, xformers is absent).  Returns bf16 storage."""
+    h = bf16_bits_to_f32(h_bits).astype(np.float64)
+    w = bf16_bits_to_f32(w_bits).astype(np.float64)
+    y = h / np.sqrt((h * h).mean(axis=-1, keepdims=True) + float(eps)) * w
+    return f32_to_bf16_bits(y.astype(np.float32))
 
 
 def quant_weight_int8(w: np.ndarray):

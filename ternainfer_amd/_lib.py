@@ -38,6 +38,8 @@ PROTOTYPES = {
     "ternaspmm_repack": ([_vp, _vp, _vp, _vp, _vp, _ci, _ci, _vp], None),
     "bitlinear_TernaSpMM_bf16_packed": ([_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp], None),
     "bitlinear_TernaSpMM_packed": ([_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp], None),
+    "ternaspmm_rmsnorm_quant": ([_vp, _vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _ci, _ci, _vp], None),
+    "ternaspmm_relu2_mul_rmsnorm_quant": ([_vp, _vp, ctypes.c_float, _vp, _vp, _vp, _ci, _ci, _vp], None),
     "ternaspmm_version": ([], ctypes.c_char_p),
 }
 

@@ -1,0 +1,144 @@
+// Fused prologue of a ternary linear: [residual add | relu(x1)^2 * x3] -> RMSNorm -> per-row
+// absmax int8 quantisation, one workgroup per activation row.
+//
+// This is the glue the reference runs as separate PyTorch / xformers / Inductor kernels between two
+// bitlinear calls (model.py:120-123 quant_input; model.py:236 attn_sub_norm; :280 ffn_sub_norm over
+// squared_relu(x1) * x3; :330, :334 the residual adds and the two block norms).  Per row:
+//
+//   h  = x                                   (plain)
+//      = bf16(x + residual)                  (residual add; h is also written back as the new stream)
+//      = bf16(bf16(relu(x1)^2) * x3)         (gated FFN; x1 = row[0:F], x3 = row[F:2F])
+//   y  = bf16(h * rsqrt(mean(h^2) + eps) * weight)          fp32 inside, one rounding at the end
+//   s  = bf16(127 / max(max|y|, 1e-5));  q = clamp(rint(y * s), -128, 127)   (fp32 inside)
+//
+// The row stays in registers between the three passes; HBM sees each input element once and each
+// output element once.  Rows are independent, so the grid is M workgroups of 256 threads.
+#pragma once
+
+#include "terna_common.h"
+
+namespace terna {
+
+constexpr int kNormThreads = 256;
+constexpr int kNormMaxVecs = 4;                       // 8-element vectors per thread: K <= 8192
+
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+    return v;
+}
+
+__device__ __forceinline__ void unpack_bf16x8(const u32x4& v, float f[8])
+{
+    const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        f[2 * j] = __uint_as_float(d[j] << 16);
+        f[2 * j + 1] = __uint_as_float(d[j] & 0xffff0000u);
+    }
+}
+__device__ __forceinline__ u32x4 pack_bf16x8(const float f[8])
+{
+    uint32_t d[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        d[j] = float_to_bf16_bits(f[2 * j]) | (static_cast<uint32_t>(float_to_bf16_bits(f[2 * j + 1])) << 16);
+    return u32x4{d[0], d[1], d[2], d[3]};
+}
+__device__ __forceinline__ float round_bf16(float v) { return bf16_bits_to_float(float_to_bf16_bits(v)); }
+
+// GLU = false: x [M][K], optional residual [M][K] and sum_out [M][K].
+// GLU = true : x [M][2K] holding x1 | x3; residual / sum_out unused.
+template <bool GLU>
+__global__ __launch_bounds__(kNormThreads) void terna_norm_quant_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, uint16_t* __restrict__ sum_out,
+    const uint16_t* __restrict__ weight, float eps, uint16_t* __restrict__ y_out, int8_t* __restrict__ xq_out,
+    uint16_t* __restrict__ s_out, int K)
+{
+    __shared__ float red[2][kNormThreads / 64];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const size_t row = blockIdx.x;
+    const int nvec = K >> 3;
+    const uint16_t* xr = x + row * static_cast<size_t>(GLU ? 2 * K : K);
+
+    float h[kNormMaxVecs][8];
+    float ssq = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kNormMaxVecs; ++i) {
+        const int v = tid + i * kNormThreads;
+        if (v < nvec) {
+            unpack_bf16x8(*reinterpret_cast<const u32x4*>(xr + 8 * v), h[i]);
+            if constexpr (GLU) {
+                float g[8];
+                unpack_bf16x8(*reinterpret_cast<const u32x4*>(xr + K + 8 * v), g);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float r = fmaxf(h[i][j], 0.0f);
+                    h[i][j] = round_bf16(round_bf16(r * r) * g[j]);
+                }
+            } else if (residual != nullptr) {
+                float r[8];
+                unpack_bf16x8(*reinterpret_cast<const u32x4*>(residual + row * K + 8 * v), r);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) h[i][j] = round_bf16(h[i][j] + r[j]);
+                if (sum_out != nullptr) *reinterpret_cast<u32x4*>(sum_out + row * K + 8 * v) = pack_bf16x8(h[i]);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) ssq = fmaf(h[i][j], h[i][j], ssq);
+        }
+    }
+    ssq = wave_sum(ssq);
+    if (lane == 0) red[0][wave] = ssq;
+    __syncthreads();
+    const float total = (red[0][0] + red[0][1]) + (red[0][2] + red[0][3]);
+    const float rstd = rsqrtf(total / static_cast<float>(K) + eps);
+
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kNormMaxVecs; ++i) {
+        const int v = tid + i * kNormThreads;
+        if (v < nvec) {
+            float w[8];
+            unpack_bf16x8(*reinterpret_cast<const u32x4*>(weight + 8 * v), w);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                h[i][j] = round_bf16(h[i][j] * rstd * w[j]);
+                amax = fmaxf(amax, fabsf(h[i][j]));
+            }
+            if (y_out != nullptr) *reinterpret_cast<u32x4*>(y_out + row * K + 8 * v) = pack_bf16x8(h[i]);
+        }
+    }
+    if (xq_out == nullptr) return;
+
+    amax = wave_max(amax);
+    if (lane == 0) red[1][wave] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red[1][0], red[1][1]), fmaxf(red[1][2], red[1][3]));
+    const uint16_t s_bits = float_to_bf16_bits(__fdiv_rn(127.0f, fmaxf(amax, 1e-5f)));
+    const float s = bf16_bits_to_float(s_bits);
+    if (tid == 0) s_out[row] = s_bits;
+#pragma unroll
+    for (int i = 0; i < kNormMaxVecs; ++i) {
+        const int v = tid + i * kNormThreads;
+        if (v < nvec) {
+            uint32_t q[2] = {0u, 0u};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float r = rintf(__fmul_rn(h[i][j], s));
+                r = fminf(fmaxf(r, -128.0f), 127.0f);
+                q[j >> 2] |= (static_cast<uint32_t>(static_cast<int>(r)) & 0xffu) << (8 * (j & 3));
+            }
+            *reinterpret_cast<u32x2*>(xq_out + row * K + 8 * v) = u32x2{q[0], q[1]};
+        }
+    }
+}
+
+}  // namespace terna

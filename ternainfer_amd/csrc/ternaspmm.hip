@@ -11,6 +11,7 @@
 #include "prefill_kernel.h"
 #include "decode_packed_kernel.h"
 #include "prefill_packed_kernel.h"
+#include "norm_quant_kernel.h"
 #include "format_host.h"
 
 using namespace terna;
@@ -207,7 +208,9 @@ void launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, 
     // when they would leave most of the 1024 workgroup slots of the chip empty, 128-feature tiles
     // double the workgroup count instead.  TERNASPMM_PREFILL_BN=128|256 forces one (tuning aid).
     const long wg256 = static_cast<long>((N + 255) / 256) * ((M + 63) / 64);
-    const int bn = forced_bn ? forced_bn : (wg256 <= 640 ? 128 : 256);
+    // int8 activations: a step is half as many MFMA cycles per byte loaded, and the extra waves of
+    // the small tile hide more latency than its extra operand reads cost -- 128 wins at every shape.
+    const int bn = forced_bn ? forced_bn : ((sizeof(Act) == 1 || wg256 <= 640) ? 128 : 256);
     if (prefill_dma_ok(x, sizeof(Act), M, N, K) && (bm == 64 || bm == 128)) {
         if (bm == 64 && bn == 128) launch_prefill_packed_dma_as<Act, 2, 1>(x, packed, out, ep, M, N, K, st);
         else if (bm == 128 && forced_bn == 128) launch_prefill_packed_dma_as<Act, 4, 1>(x, packed, out, ep, M, N, K, st);
@@ -472,6 +475,33 @@ void bitlinear_TernaSpMM_packed(const int8_t* x, const void* packed, terna_bf16*
     else launch_prefill_packed<int8_t>(x, p, out, ep, M, N, K, st);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("bitlinear_TernaSpMM_packed", e, __LINE__);
+}
+
+void ternaspmm_rmsnorm_quant(const terna_bf16* x, const terna_bf16* residual, terna_bf16* sum_out,
+                             const terna_bf16* weight, float eps, terna_bf16* y_out, int8_t* xq_out,
+                             terna_bf16* s_out, int M, int K, terna_stream stream)
+{
+    if (M < 1 || K < 8 || (K & 7) || K > 8 * kNormThreads * kNormMaxVecs || (xq_out != nullptr) != (s_out != nullptr)) {
+        std::fprintf(stderr, "ternaspmm_rmsnorm_quant: unsupported arguments (M=%d K=%d)\n", M, K);
+        return;
+    }
+    terna_norm_quant_kernel<false><<<dim3(M), dim3(kNormThreads), 0, static_cast<hipStream_t>(stream)>>>(
+        x, residual, sum_out, weight, eps, y_out, xq_out, s_out, K);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_rmsnorm_quant", e, __LINE__);
+}
+
+void ternaspmm_relu2_mul_rmsnorm_quant(const terna_bf16* x13, const terna_bf16* weight, float eps, terna_bf16* y_out,
+                                       int8_t* xq_out, terna_bf16* s_out, int M, int F, terna_stream stream)
+{
+    if (M < 1 || F < 8 || (F & 7) || F > 8 * kNormThreads * kNormMaxVecs || (xq_out != nullptr) != (s_out != nullptr)) {
+        std::fprintf(stderr, "ternaspmm_relu2_mul_rmsnorm_quant: unsupported arguments (M=%d F=%d)\n", M, F);
+        return;
+    }
+    terna_norm_quant_kernel<true><<<dim3(M), dim3(kNormThreads), 0, static_cast<hipStream_t>(stream)>>>(
+        x13, nullptr, nullptr, weight, eps, y_out, xq_out, s_out, F);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_relu2_mul_rmsnorm_quant", e, __LINE__);
 }
 
 const char* ternaspmm_version(void) { return "ternaspmm-gfx950 0.1"; }

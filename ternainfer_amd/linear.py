@@ -120,6 +120,51 @@ def TernaInfer_linear_packed(input, packed, s, ws, ws_num, out_features):
     return out.reshape(*out_shape)
 
 
+def rmsnorm_quant(x, weight, eps, residual=None, quant=True):
+    """Fused [residual add] -> RMSNorm -> [SpBitLinear.quant_input] in one launch
+    (model.py:330/334 + the norm + model.py:120-123).  x, residual: bf16 [M, K]; weight: bf16 [K].
+    Returns (xq int8 [M, K], s bf16 [M], h) when quant else (y bf16 [M, K], h); h is the bf16 sum
+    x + residual (x itself when residual is None)."""
+    m, k = x.shape
+    x = x.contiguous()
+    lib = _lib.load()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    h = x
+    if residual is not None:
+        residual = residual.contiguous()
+        h = torch.empty_like(x)
+    if quant:
+        xq = torch.empty((m, k), dtype=torch.int8, device=x.device)
+        s = torch.empty(m, dtype=torch.bfloat16, device=x.device)
+        lib.ternaspmm_rmsnorm_quant(_p(x), _p(residual) if residual is not None else None,
+                                    _p(h) if residual is not None else None, _p(weight), float(eps), None, _p(xq),
+                                    _p(s), m, k, stream)
+        return xq, s, h
+    y = torch.empty_like(x)
+    lib.ternaspmm_rmsnorm_quant(_p(x), _p(residual) if residual is not None else None,
+                                _p(h) if residual is not None else None, _p(weight), float(eps), _p(y), None, None,
+                                m, k, stream)
+    return y, h
+
+
+def relu2_mul_rmsnorm_quant(x13, weight, eps, quant=True):
+    """Fused squared_relu(x1) * x3 -> ffn_sub_norm -> [quant_input] (model.py:279-281 + 120-123).
+    x13: bf16 [M, 2F].  Returns (xq int8 [M, F], s bf16 [M]) when quant else y bf16 [M, F]."""
+    m, f2 = x13.shape
+    f = f2 // 2
+    x13 = x13.contiguous()
+    lib = _lib.load()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    if quant:
+        xq = torch.empty((m, f), dtype=torch.int8, device=x13.device)
+        s = torch.empty(m, dtype=torch.bfloat16, device=x13.device)
+        lib.ternaspmm_relu2_mul_rmsnorm_quant(_p(x13), _p(weight), float(eps), None, _p(xq), _p(s), m, f, stream)
+        return xq, s
+    y = torch.empty((m, f), dtype=torch.bfloat16, device=x13.device)
+    lib.ternaspmm_relu2_mul_rmsnorm_quant(_p(x13), _p(weight), float(eps), _p(y), None, None, m, f, stream)
+    return y
+
+
 class _CompressedWeight(nn.Module):
     """Holds the four format tensors + ``weight_scale`` under the reference's checkpoint keys
     (convert_TernaInfer.py:204-209, model.py:110-116)."""

@@ -5,8 +5,10 @@ This is NOT a port of the reference's transformer (model.py:155-471); it exists 
 going through libternaspmm.so.  It keeps the reference's block structure -- fused wqkv / w13,
 attention and FFN sub-norms, squared-ReLU gating, tied bf16 LM head (model.py:198-239, 277-282,
 323-335, 367) -- and, like the reference's SpBitLinear (model.py:120-133), quantises activations
-per row to int8 in front of every ternary linear.  Attention, RoPE, norms and the LM head are
-plain PyTorch-ROCm ops; one decode step is captured in a HIP graph, as generate.py:204-224 does.
+per row to int8 in front of every ternary linear.  The residual adds, the four norms, the gate and
+that quantisation run as the library's fused prologue kernels (one launch in front of each
+linear); attention, RoPE and the LM head are plain PyTorch-ROCm ops; one decode step is captured
+in a HIP graph, as generate.py:204-224 does.
 """
 from __future__ import annotations
 
@@ -18,6 +20,7 @@ import torch
 from torch.nn import functional as F
 
 from . import _lib
+from .linear import relu2_mul_rmsnorm_quant, rmsnorm_quant
 
 
 @dataclass
@@ -66,24 +69,37 @@ class TernaryLinear:
         self.act = act
         self.lib = _lib.load()
 
-    def __call__(self, x: torch.Tensor) -> torch.Tensor:
+    def quantised(self, xq: torch.Tensor, s: torch.Tensor) -> torch.Tensor:
+        """int8 activations [M, K] + per-row scale bf16 [M] (as the fused prologue kernels write them)."""
+        m = xq.shape[0]
+        out = torch.empty((m, self.n), dtype=torch.bfloat16, device=xq.device)
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        self.lib.bitlinear_TernaSpMM_packed(_p(xq), _p(self.packed), _p(out), _p(s), _p(self.ws), self.ws_num,
+                                            m, self.n, self.k, 0, stream)
+        return out
+
+    def dense(self, x: torch.Tensor) -> torch.Tensor:
+        """bf16 activations [M, K]."""
         m = x.shape[0]
         out = torch.empty((m, self.n), dtype=torch.bfloat16, device=x.device)
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-        if self.act == "int8":                                                   # model.py:120-133
-            s = 127 / x.abs().max(dim=-1, keepdim=True).values.clamp_(min=1e-5)
-            xq = (x * s).round().clamp(-128, 127).to(torch.int8)
-            self.lib.bitlinear_TernaSpMM_packed(_p(xq), _p(self.packed), _p(out), _p(s.to(torch.bfloat16).contiguous()),
-                                                _p(self.ws), self.ws_num, m, self.n, self.k, 0, stream)
-        else:
-            self.lib.bitlinear_TernaSpMM_bf16_packed(_p(x.contiguous()), _p(self.packed), _p(out), _p(self.scale_f32),
-                                                     self.ws_num, m, self.n, self.k, 0, stream)
+        self.lib.bitlinear_TernaSpMM_bf16_packed(_p(x.contiguous()), _p(self.packed), _p(out), _p(self.scale_f32),
+                                                 self.ws_num, m, self.n, self.k, 0, stream)
         return out
+
+    def __call__(self, x: torch.Tensor) -> torch.Tensor:
+        if self.act == "int8":                # model.py:120-133, fp32 inside, the bf16-rounded s used throughout
+            xf = x.float()
+            s = (127 / xf.abs().amax(dim=-1, keepdim=True).clamp_(min=1e-5)).to(torch.bfloat16)
+            xq = (xf * s.float()).round().clamp(-128, 127).to(torch.int8)
+            return self.quantised(xq, s.reshape(-1).contiguous())
+        return self.dense(x)
 
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """fp32 inside, one rounding to the input's dtype (the fused kernels compute the same)."""
     xf = x.float()
-    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).to(x.dtype) * weight
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * weight.float()).to(x.dtype)
 
 
 def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
@@ -107,14 +123,39 @@ class Block:
         self.attention_norm, self.ffn_norm = ones(d), ones(d)
         self.attn_sub_norm, self.ffn_sub_norm = ones(d), ones(args.ffn_dim)
         self.args = args
+        self.act = act
+        self.fused = True          # norms / gate / activation quantisation through the fused prologue kernels
 
-    def forward(self, x, cache_k, cache_v, pos_idx, cos, sin, mask):
-        """x [B*T, dim] (T new tokens per sequence); cache_* [B, n_kv, S, hd]; pos_idx int64 [T] cache slots."""
+    def _norm_linear(self, lin, x, weight, residual=None, glu=False):
+        """[x + residual | relu(x1)^2 * x3] -> RMSNorm -> lin.  Returns (lin output, x + residual)."""
+        eps = self.args.norm_eps
+        if not self.fused:
+            if glu:
+                x1, x3 = x.chunk(2, dim=-1)
+                h = F.relu(x1) ** 2 * x3
+            else:
+                h = x if residual is None else x + residual
+            return lin(rms_norm(h, weight, eps)), h
+        if glu:
+            if self.act == "int8":
+                return lin.quantised(*relu2_mul_rmsnorm_quant(x, weight, eps)), None
+            return lin.dense(relu2_mul_rmsnorm_quant(x, weight, eps, quant=False)), None
+        if self.act == "int8":
+            xq, s, h = rmsnorm_quant(x, weight, eps, residual=residual)
+            return lin.quantised(xq, s), h
+        y, h = rmsnorm_quant(x, weight, eps, residual=residual, quant=False)
+        return lin.dense(y), h
+
+    def forward(self, x, pending, cache_k, cache_v, pos_idx, cos, sin, mask):
+        """x [B*T, dim] (T new tokens per sequence) and `pending`, the previous block's FFN output that
+        has not been added to the stream yet (None for the first block): the add is part of this
+        block's first fused kernel.  cache_* [B, n_kv, S, hd]; pos_idx int64 [T] cache slots.
+        Returns (stream, pending) for the next block."""
         a = self.args
         bsz = cache_k.shape[0]
         t = x.shape[0] // bsz
-        h = rms_norm(x, self.attention_norm, a.norm_eps)
-        qkv = self.wqkv(h).view(bsz, t, a.n_heads + 2 * a.n_kv_heads, a.head_dim).transpose(1, 2)
+        qkv, x = self._norm_linear(self.wqkv, x, self.attention_norm, residual=pending)
+        qkv = qkv.view(bsz, t, a.n_heads + 2 * a.n_kv_heads, a.head_dim).transpose(1, 2)
         q, k, v = qkv[:, :a.n_heads], qkv[:, a.n_heads:a.n_heads + a.n_kv_heads], qkv[:, a.n_heads + a.n_kv_heads:]
         q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
         cache_k.index_copy_(2, pos_idx, k)
@@ -124,11 +165,10 @@ class Block:
         vv = cache_v.repeat_interleave(rep, dim=1)
         o = F.scaled_dot_product_attention(q, kk, vv, attn_mask=mask)
         o = o.transpose(1, 2).reshape(bsz * t, a.n_heads * a.head_dim)
-        x = x + self.wo(rms_norm(o, self.attn_sub_norm, a.norm_eps))
-        h = rms_norm(x, self.ffn_norm, a.norm_eps)
-        x1, x3 = self.w13(h).chunk(2, dim=-1)
-        inner = rms_norm(F.relu(x1) ** 2 * x3, self.ffn_sub_norm, a.norm_eps)
-        return x + self.w2(inner)
+        attn, _ = self._norm_linear(self.wo, o.contiguous(), self.attn_sub_norm)
+        x13, x = self._norm_linear(self.w13, x, self.ffn_norm, residual=attn)
+        ffn, _ = self._norm_linear(self.w2, x13, self.ffn_sub_norm, glu=True)
+        return x, ffn
 
 
 class Transformer:
@@ -161,8 +201,10 @@ class Transformer:
         # causal over cache slots: new token at slot p sees slots <= p
         mask = torch.arange(max_seq, device=dev)[None, :] <= pos_idx[:, None]
         x = self.tok_embeddings[tokens.reshape(-1)]
+        pending = None
         for layer, (ck, cv) in zip(self.layers, cache):
-            x = layer.forward(x, ck, cv, pos_idx, cos, sin, mask[None, None])
+            x, pending = layer.forward(x, pending, ck, cv, pos_idx, cos, sin, mask[None, None])
+        x = x + pending
         x = rms_norm(x.view(bsz, t, a.dim)[:, -1], self.norm, a.norm_eps)
         return F.linear(x, self.tok_embeddings)                               # tied LM head (model.py:367)
 

@@ -22,10 +22,11 @@ class DenseLinearCPU:
 
     def __call__(self, x):
         if self.act == "int8":
-            s = 127 / x.abs().max(dim=-1, keepdim=True).values.clamp_(min=1e-5)
-            xq = (x * s).round().clamp(-128, 127)
+            xf = x.float()
+            s = (127 / xf.abs().amax(dim=-1, keepdim=True).clamp_(min=1e-5)).to(torch.bfloat16)
+            xq = (xf * s.float()).round().clamp(-128, 127)
             acc = xq.double() @ self.w.T
-            return ((acc / s.to(torch.bfloat16).double()) * self.ws).to(torch.bfloat16)
+            return ((acc / s.double()) * self.ws).to(torch.bfloat16)
         return ((x.double() @ self.w.T) * self.ws).to(torch.bfloat16)
 
 
@@ -46,6 +47,7 @@ def test_toy_model_matches_cpu_golden(act):
         twin.layers = []
         for blk in model.layers:
             b = copy.copy(blk)
+            b.fused = False                      # the CPU twin runs the same block with plain torch ops
             for name in ("wqkv", "wo", "w13", "w2"):
                 setattr(b, name, DenseLinearCPU(getattr(blk, name), act))
             for name in ("attention_norm", "ffn_norm", "attn_sub_norm", "ffn_sub_norm"):
@@ -56,6 +58,23 @@ def test_toy_model_matches_cpu_golden(act):
     ref = want.abs().max().item()
     assert err <= 3e-2 * ref, (err, ref)
     assert torch.nn.functional.cosine_similarity(got.flatten(), want.flatten(), dim=0).item() > 0.999
+
+
+def test_toy_model_fused_prologue_equals_torch_ops():
+    """Same model, norms / gate / quantisation through the fused kernels vs through torch ops."""
+    from ternainfer_amd.model import ModelArgs, Transformer
+    args = ModelArgs(dim=256, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=1024, ffn_dim=384)
+    tokens = torch.randint(0, args.vocab_size, (2, 24), generator=torch.Generator().manual_seed(11)).cuda()
+    outs = []
+    model = Transformer(args, seed=12, act="int8")
+    for fused in (True, False):
+        for blk in model.layers:
+            blk.fused = fused
+        with torch.inference_mode():
+            outs.append(model.forward(tokens, model.make_cache(2, 32), torch.arange(24, device="cuda")).float())
+    err = (outs[0] - outs[1]).abs().max().item()
+    assert err <= 3e-2 * outs[1].abs().max().item()
+    assert torch.nn.functional.cosine_similarity(outs[0].flatten(), outs[1].flatten(), dim=0).item() > 0.999
 
 
 def test_toy_model_greedy_decode_graph_equals_eager():

@@ -1,0 +1,135 @@
+"""GPU tests of the fused prologue kernels (residual add / gate -> RMSNorm -> int8 quantisation)
+through the C ABI, against the CPU oracle.
+
+Bars: the residual stream and the int8 quantisation are bit-exact (their arithmetic is fully
+defined); the norm output is within one bf16 step of the float64 evaluation, the tolerance a
+parallel fp32 sum of squares leaves (RMSNorm parity is unpinned: xformers is absent)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import terna_oracle as O
+from tests._util import make_bf16_activations
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from ternainfer_amd import _lib
+    return _lib.load()
+
+
+def _dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int16) if a.dtype == np.uint16 else np.ascontiguousarray(a)).cuda()
+
+
+def _vp(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _run(lib, x, w, eps, residual=None, glu=False, want_y=True, want_q=True):
+    m = x.shape[0]
+    k = x.shape[1] // 2 if glu else x.shape[1]
+    xd, wd = _dev(x), _dev(w)
+    rd = _dev(residual) if residual is not None else None
+    hd = torch.zeros((m, k), dtype=torch.int16, device="cuda") if residual is not None else None
+    yd = torch.zeros((m, k), dtype=torch.int16, device="cuda") if want_y else None
+    qd = torch.zeros((m, k), dtype=torch.int8, device="cuda") if want_q else None
+    sd = torch.zeros(m, dtype=torch.int16, device="cuda") if want_q else None
+    if glu:
+        lib.ternaspmm_relu2_mul_rmsnorm_quant(_vp(xd), _vp(wd), eps, _vp(yd), _vp(qd), _vp(sd), m, k, None)
+    else:
+        lib.ternaspmm_rmsnorm_quant(_vp(xd), _vp(rd), _vp(hd), _vp(wd), eps, _vp(yd), _vp(qd), _vp(sd), m, k, None)
+    torch.cuda.synchronize()
+    get = lambda t, dt: None if t is None else t.cpu().numpy().view(dt)
+    return get(hd, np.uint16), get(yd, np.uint16), get(qd, np.int8), get(sd, np.uint16)
+
+
+def _assert_within_one_bf16_step(got_bits, want_bits):
+    """Monotone integer image of bf16 storage: adjacent values differ by 1."""
+    def key(b):
+        b = b.astype(np.int32)
+        return np.where(b & 0x8000, -(b & 0x7FFF), b & 0x7FFF)
+    d = np.abs(key(got_bits) - key(want_bits))
+    assert d.max() <= 1, f"max distance {d.max()} bf16 steps"
+    assert (d != 0).mean() < 0.02, f"{(d != 0).mean():.4f} of the outputs are one step off"
+
+
+def _weight(k, seed):
+    return O.f32_to_bf16_bits(np.random.default_rng(seed).uniform(0.5, 1.5, k).astype(np.float32))
+
+
+@pytest.mark.parametrize("m", [1, 8, 37, 256])
+@pytest.mark.parametrize("k", [64, 2560, 6912, 8192])
+def test_rmsnorm_quant_plain(lib, m, k):
+    x = make_bf16_activations(m, k, 600 + m + k, outlier_frac=0.01)
+    w = _weight(k, 601 + k)
+    _, y, q, s = _run(lib, x, w, 1e-5)
+    _assert_within_one_bf16_step(y, O.rmsnorm(x, w, 1e-5))
+    want_q, want_s = O.quant_input(y)                         # the quantiser, on the kernel's own norm output
+    assert (s == want_s).all() and (q == want_q).all()
+
+
+@pytest.mark.parametrize("m,k", [(8, 2560), (300, 2560), (5, 640)])
+def test_rmsnorm_quant_with_residual(lib, m, k):
+    x = make_bf16_activations(m, k, 610 + m)
+    r = make_bf16_activations(m, k, 611 + m, outlier_frac=0.01)
+    w = _weight(k, 612)
+    h, y, q, s = _run(lib, x, w, 1e-5, residual=r)
+    want_h = O.residual_add(x, r)
+    assert (h == want_h).all()
+    _assert_within_one_bf16_step(y, O.rmsnorm(want_h, w, 1e-5))
+    want_q, want_s = O.quant_input(y)
+    assert (s == want_s).all() and (q == want_q).all()
+
+
+@pytest.mark.parametrize("m,f", [(1, 6912), (8, 6912), (100, 6912), (16, 64)])
+def test_relu2_mul_rmsnorm_quant(lib, m, f):
+    x13 = make_bf16_activations(m, 2 * f, 620 + m + f, outlier_frac=0.01)
+    w = _weight(f, 621)
+    _, y, q, s = _run(lib, x13, w, 1e-5, glu=True)
+    _assert_within_one_bf16_step(y, O.rmsnorm(O.relu2_mul(x13), w, 1e-5))
+    want_q, want_s = O.quant_input(y)
+    assert (s == want_s).all() and (q == want_q).all()
+
+
+def test_optional_outputs_do_not_change_the_others(lib):
+    x = make_bf16_activations(9, 2560, 630)
+    w = _weight(2560, 631)
+    _, y, q, s = _run(lib, x, w, 1e-5)
+    _, y2, _, _ = _run(lib, x, w, 1e-5, want_q=False)
+    _, _, q2, s2 = _run(lib, x, w, 1e-5, want_y=False)
+    assert (y == y2).all() and (q == q2).all() and (s == s2).all()
+
+
+def test_zero_row_quantises_to_zero_with_the_clamped_scale(lib):
+    """max|y| = 0 -> s = bf16(127 / 1e-5), q = 0 (model.py:121's clamp_(min=1e-5))."""
+    x = np.zeros((2, 128), np.uint16)
+    _, y, q, s = _run(lib, x, _weight(128, 640), 1e-5)
+    assert (y & 0x7FFF == 0).all() and (q == 0).all()
+    assert (s == O.f32_to_bf16_bits(np.array([127.0 / 1e-5], np.float32))[0]).all()
+
+
+def test_python_wrappers_feed_the_linear(lib):
+    """rmsnorm_quant -> TernaInfer_linear_packed equals the unfused sequence on the same inputs."""
+    import ternainfer_amd as T
+    from tests._util import make_ternary
+    n, k, m = 256, 320, 8
+    w = make_ternary(n, k, 0.4, 650)
+    vals, off, med, bm = [t.cuda() for t in T.compress_weight(torch.from_numpy(w))]
+    packed = T.repack_weight(vals, off, med, bm, n, k)
+    x = make_bf16_activations(m, k, 651)
+    g = _weight(k, 652)
+    xt = torch.from_numpy(x.view(np.int16)).cuda().view(torch.bfloat16)
+    gt = torch.from_numpy(g.view(np.int16)).cuda().view(torch.bfloat16)
+    ws = torch.tensor([1.25, 0, 0, 0], dtype=torch.bfloat16, device="cuda")
+    xq, s, h = T.rmsnorm_quant(xt, gt, 1e-5)
+    out = T.TernaInfer_linear_packed(xq, packed, s, ws, 1, n)
+    y, _ = T.rmsnorm_quant(xt, gt, 1e-5, quant=False)
+    yq, ys = O.quant_input(y.view(torch.int16).cpu().numpy().view(np.uint16))
+    assert (xq.cpu().numpy() == yq).all()
+    want = O.spmm_i8(yq, w, ys, O.f32_to_bf16_bits(np.array([1.25, 0, 0, 0], np.float32)), 1, 0)
+    assert (out.view(torch.int16).cpu().numpy().view(np.uint16) == want).all()

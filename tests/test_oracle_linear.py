@@ -101,3 +101,30 @@ def test_quant_input_c_equals_numpy(coracle):
     q2, s2 = O.quant_input(x)
     assert (q1 == q2).all() and (s1 == s2).all()
     assert np.abs(q1).max() <= 127 and (np.abs(q1).max(axis=1) >= 126).all()
+
+
+# ------------------------------------------------------------------ glue between two linears
+def test_rmsnorm_closed_forms():
+    """What the mathematics fixes for RMSNorm: a constant row maps to sign * weight, a power-of-two
+    rescale of the row changes nothing when eps = 0, and a 4-element case equals the hand formula."""
+    w = O.f32_to_bf16_bits(np.linspace(0.5, 2.0, 64, dtype=np.float32))
+    ones = O.f32_to_bf16_bits(np.full((1, 64), -3.0, np.float32))
+    assert (O.rmsnorm(ones, w, 0.0) == O.f32_to_bf16_bits(-O.bf16_bits_to_f32(w))).all()
+    x = make_bf16_activations(5, 64, 71)
+    x4 = O.f32_to_bf16_bits(O.bf16_bits_to_f32(x) * np.float32(4.0))
+    assert (O.rmsnorm(x, w, 0.0) == O.rmsnorm(x4, w, 0.0)).all()
+    v = np.array([[1.0, -2.0, 3.0, 0.5]], np.float32)
+    want = v / np.sqrt((1 + 4 + 9 + 0.25) / 4 + 1e-5) * np.array([1.0, 0.5, 2.0, 1.0])
+    got = O.bf16_bits_to_f32(O.rmsnorm(O.f32_to_bf16_bits(v), O.f32_to_bf16_bits(np.array([1.0, 0.5, 2.0, 1.0], np.float32)), 1e-5))
+    assert (got == O.bf16_bits_to_f32(O.f32_to_bf16_bits(want.astype(np.float32)))).all()
+
+
+def test_relu2_mul_and_residual_add_small_cases():
+    x13 = O.f32_to_bf16_bits(np.array([[-1.0, 0.0, 1.5, 3.0, 2.0, 2.0, -2.0, 0.5]], np.float32))
+    assert O.bf16_bits_to_f32(O.relu2_mul(x13)).tolist() == [[0.0, 0.0, -4.5, 4.5]]
+    # 1 + 2^-8 is not a bf16 value: the sum rounds to even
+    a = O.f32_to_bf16_bits(np.array([1.0], np.float32))
+    b = O.f32_to_bf16_bits(np.array([2.0 ** -8], np.float32))
+    assert O.bf16_bits_to_f32(O.residual_add(a, b)).tolist() == [1.0]
+    c = O.f32_to_bf16_bits(np.array([3 * 2.0 ** -8], np.float32))
+    assert O.bf16_bits_to_f32(O.residual_add(a, c)).tolist() == [1.0 + 2.0 ** -6]
