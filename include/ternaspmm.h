@@ -165,6 +165,25 @@ void ternaspmm_rmsnorm_quant(const terna_bf16* x, const terna_bf16* residual, te
 void ternaspmm_relu2_mul_rmsnorm_quant(const terna_bf16* x13, const terna_bf16* weight, float eps, terna_bf16* y_out,
                                        int8_t* xq_out, terna_bf16* s_out, int M, int F, terna_stream stream);
 
+/* ---- Attention-side kernels of a decode step (no counterpart in the reference's library) -----------
+ * They stand where the reference calls xformers' rope_padded (model.py:218-229) and
+ * fmha.memory_efficient_attention_forward (model.py:231-233).
+ *
+ * ternaspmm_rope_kv_store: rotary embedding of the q and k heads of the fused qkv linear's output
+ * (bf16 [B*T][(H + 2*KV)*D], row b*T + t), pairs (j, j + D/2) rotated by the angle whose cosine / sine is
+ * cos[t][j] / sin[t][j] (fp32 [T][D/2]); q goes to q_out (bf16 [B][H][T][D]); k and v go into the caches
+ * (bf16 [B][KV][S][D]) at slot pos[t] (int64 [T], device memory).
+ *
+ * ternaspmm_decode_attention: one new token per sequence.  q bf16 [B][H][D]; head h reads kv head
+ * h / (H/KV) at slots 0 .. pos[0]; out bf16 [B][H*D] = softmax(scale * q K^T) V.  D is 64 or 128,
+ * S <= 8192.  Both only enqueue. */
+void ternaspmm_rope_kv_store(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
+                             terna_bf16* q_out, terna_bf16* cache_k, terna_bf16* cache_v, int B, int T, int H,
+                             int KV, int D, int S, terna_stream stream);
+void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
+                                const long long* pos, terna_bf16* out, int B, int H, int KV, int D, int S,
+                                float scale, terna_stream stream);
+
 /* Library version string, e.g. "ternaspmm-gfx950 0.1". */
 const char* ternaspmm_version(void);
 

@@ -285,6 +285,33 @@ def rmsnorm(h_bits: np.ndarray, w_bits: np.ndarray, eps: float) -> np.ndarray:
     return f32_to_bf16_bits(y.astype(np.float32))
 
 
+def rope_rotate_half(x_bits: np.ndarray, cos: np.ndarray, sin: np.ndarray) -> np.ndarray:
+    """Rotary embedding of bf16 x [..., D] by angles given as cos / sin [..., D/2] (fp32): pair j is
+    (x[j], x[j + D/2]).  Stands for xformers' rope_padded (model.py:218-229; absent dependency,
+    parity unpinned).  fp32 arithmetic in the order x1*c - x2*s, x2*c + x1*s, one rounding to bf16."""
+    x = bf16_bits_to_f32(x_bits)
+    half = x.shape[-1] // 2
+    x1, x2 = x[..., :half], x[..., half:]
+    c, s = cos.astype(np.float32), sin.astype(np.float32)
+    return f32_to_bf16_bits(np.concatenate([x1 * c - x2 * s, x2 * c + x1 * s], axis=-1).astype(np.float32))
+
+
+def attention_one_token(q_bits: np.ndarray, k_bits: np.ndarray, v_bits: np.ndarray, n: int, scale: float) -> np.ndarray:
+    """softmax(scale * q K^T) V in float64 for one query per (sequence, head): q [B, H, D],
+    k / v [B, KV, S, D], keys 0 .. n-1 valid, head h reads kv head h // (H // KV).  Stands for
+    fmha.memory_efficient_attention_forward on the padded cache (model.py:231-233; absent
+    dependency, parity unpinned).  Returns float64 [B, H, D]."""
+    q = bf16_bits_to_f32(q_bits).astype(np.float64)
+    k = bf16_bits_to_f32(k_bits).astype(np.float64)[:, :, :n]
+    v = bf16_bits_to_f32(v_bits).astype(np.float64)[:, :, :n]
+    rep = q.shape[1] // k.shape[1]
+    k, v = np.repeat(k, rep, axis=1), np.repeat(v, rep, axis=1)
+    sc = np.einsum("bhd,bhsd->bhs", q, k) * scale
+    p = np.exp(sc - sc.max(axis=-1, keepdims=True))
+    p /= p.sum(axis=-1, keepdims=True)
+    return np.einsum("bhs,bhsd->bhd", p, v)
+
+
 def quant_weight_int8(w: np.ndarray):
     """convert_TernaInfer.py:159-163: ternarise by 1/mean(|W|); returns (int8 W, fp32 scale=1/s)."""
     w = np.asarray(w, dtype=np.float32)

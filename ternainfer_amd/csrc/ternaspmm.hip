@@ -12,6 +12,7 @@
 #include "decode_packed_kernel.h"
 #include "prefill_packed_kernel.h"
 #include "norm_quant_kernel.h"
+#include "attention_kernel.h"
 #include "format_host.h"
 
 using namespace terna;
@@ -502,6 +503,38 @@ void ternaspmm_relu2_mul_rmsnorm_quant(const terna_bf16* x13, const terna_bf16* 
         x13, nullptr, nullptr, weight, eps, y_out, xq_out, s_out, F);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_relu2_mul_rmsnorm_quant", e, __LINE__);
+}
+
+void ternaspmm_rope_kv_store(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
+                             terna_bf16* q_out, terna_bf16* cache_k, terna_bf16* cache_v, int B, int T, int H,
+                             int KV, int D, int S, terna_stream stream)
+{
+    if (B < 1 || T < 1 || H < 1 || KV < 1 || D < 2 || (D & 1) || S < 1) {
+        std::fprintf(stderr, "ternaspmm_rope_kv_store: unsupported arguments\n");
+        return;
+    }
+    terna_rope_kv_store_kernel<<<dim3(B * T), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+        qkv, cos, sin, pos, q_out, cache_k, cache_v, T, H, KV, D, S);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_rope_kv_store", e, __LINE__);
+}
+
+void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
+                                const long long* pos, terna_bf16* out, int B, int H, int KV, int D, int S,
+                                float scale, terna_stream stream)
+{
+    if (B < 1 || H < 1 || KV < 1 || H % KV != 0 || (D != 64 && D != 128) || S < 1 || S > 8192) {
+        std::fprintf(stderr, "ternaspmm_decode_attention: unsupported arguments (H=%d KV=%d D=%d S=%d)\n", H, KV, D, S);
+        return;
+    }
+    const size_t lds = (static_cast<size_t>(S) + 16 * D) * sizeof(float);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (D == 128)
+        terna_decode_attention_kernel<128><<<dim3(B * H), dim3(256), lds, st>>>(q, cache_k, cache_v, pos, out, H, KV, S, scale);
+    else
+        terna_decode_attention_kernel<64><<<dim3(B * H), dim3(256), lds, st>>>(q, cache_k, cache_v, pos, out, H, KV, S, scale);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_decode_attention", e, __LINE__);
 }
 
 const char* ternaspmm_version(void) { return "ternaspmm-gfx950 0.1"; }

@@ -7,8 +7,9 @@ attention and FFN sub-norms, squared-ReLU gating, tied bf16 LM head (model.py:19
 323-335, 367) -- and, like the reference's SpBitLinear (model.py:120-133), quantises activations
 per row to int8 in front of every ternary linear.  The residual adds, the four norms, the gate and
 that quantisation run as the library's fused prologue kernels (one launch in front of each
-linear); attention, RoPE and the LM head are plain PyTorch-ROCm ops; one decode step is captured
-in a HIP graph, as generate.py:204-224 does.
+linear); RoPE + KV-cache write and single-token attention are library kernels too, multi-token
+(prefill) attention and the LM head are PyTorch-ROCm ops; one decode step is captured in a HIP
+graph, as generate.py:204-224 does.
 """
 from __future__ import annotations
 
@@ -103,7 +104,7 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
 
 
 def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
-    """x [B, H, T, D]; rotate-half convention; cos/sin [B, 1, T, D/2] in fp32."""
+    """x [B, H, T, D]; rotate-half convention; cos/sin broadcastable to [B, H, T, D/2], fp32."""
     x1, x2 = x.float().chunk(2, dim=-1)
     return torch.cat([x1 * cos - x2 * sin, x2 * cos + x1 * sin], dim=-1).to(x.dtype)
 
@@ -155,16 +156,28 @@ class Block:
         bsz = cache_k.shape[0]
         t = x.shape[0] // bsz
         qkv, x = self._norm_linear(self.wqkv, x, self.attention_norm, residual=pending)
-        qkv = qkv.view(bsz, t, a.n_heads + 2 * a.n_kv_heads, a.head_dim).transpose(1, 2)
-        q, k, v = qkv[:, :a.n_heads], qkv[:, a.n_heads:a.n_heads + a.n_kv_heads], qkv[:, a.n_heads + a.n_kv_heads:]
-        q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
-        cache_k.index_copy_(2, pos_idx, k)
-        cache_v.index_copy_(2, pos_idx, v)
         rep = a.n_heads // a.n_kv_heads
-        kk = cache_k.repeat_interleave(rep, dim=1)
-        vv = cache_v.repeat_interleave(rep, dim=1)
-        o = F.scaled_dot_product_attention(q, kk, vv, attn_mask=mask)
-        o = o.transpose(1, 2).reshape(bsz * t, a.n_heads * a.head_dim)
+        if self.fused:
+            lib = self.wqkv.lib
+            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            q = torch.empty((bsz, a.n_heads, t, a.head_dim), dtype=torch.bfloat16, device=x.device)
+            lib.ternaspmm_rope_kv_store(_p(qkv), _p(cos), _p(sin), _p(pos_idx), _p(q), _p(cache_k), _p(cache_v),
+                                        bsz, t, a.n_heads, a.n_kv_heads, a.head_dim, cache_k.shape[2], stream)
+        else:
+            qkv = qkv.view(bsz, t, a.n_heads + 2 * a.n_kv_heads, a.head_dim).transpose(1, 2)
+            q, k, v = qkv[:, :a.n_heads], qkv[:, a.n_heads:a.n_heads + a.n_kv_heads], qkv[:, a.n_heads + a.n_kv_heads:]
+            q, k = apply_rope(q, cos[None, None], sin[None, None]), apply_rope(k, cos[None, None], sin[None, None])
+            cache_k.index_copy_(2, pos_idx, k)
+            cache_v.index_copy_(2, pos_idx, v)
+        if self.fused and t == 1 and a.head_dim in (64, 128) and cache_k.shape[2] <= 8192:
+            o = torch.empty((bsz, a.n_heads * a.head_dim), dtype=torch.bfloat16, device=x.device)
+            lib.ternaspmm_decode_attention(_p(q), _p(cache_k), _p(cache_v), _p(pos_idx), _p(o), bsz, a.n_heads,
+                                           a.n_kv_heads, a.head_dim, cache_k.shape[2], a.head_dim ** -0.5, stream)
+        else:
+            kk = cache_k.repeat_interleave(rep, dim=1)
+            vv = cache_v.repeat_interleave(rep, dim=1)
+            o = F.scaled_dot_product_attention(q, kk, vv, attn_mask=mask)
+            o = o.transpose(1, 2).reshape(bsz * t, a.n_heads * a.head_dim)
         attn, _ = self._norm_linear(self.wo, o.contiguous(), self.attn_sub_norm)
         x13, x = self._norm_linear(self.w13, x, self.ffn_norm, residual=attn)
         ffn, _ = self._norm_linear(self.w2, x13, self.ffn_sub_norm, glu=True)
@@ -197,7 +210,7 @@ class Transformer:
         dev = tokens.device
         inv = 1.0 / (a.rope_theta ** (torch.arange(0, a.head_dim, 2, device=dev, dtype=torch.float32) / a.head_dim))
         ang = pos_idx.float()[:, None] * inv[None, :]
-        cos, sin = ang.cos()[None, None], ang.sin()[None, None]
+        cos, sin = ang.cos().contiguous(), ang.sin().contiguous()            # fp32 [T, head_dim / 2]
         # causal over cache slots: new token at slot p sees slots <= p
         mask = torch.arange(max_seq, device=dev)[None, :] <= pos_idx[:, None]
         x = self.tok_embeddings[tokens.reshape(-1)]

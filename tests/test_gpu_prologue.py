@@ -133,3 +133,50 @@ def test_python_wrappers_feed_the_linear(lib):
     assert (xq.cpu().numpy() == yq).all()
     want = O.spmm_i8(yq, w, ys, O.f32_to_bf16_bits(np.array([1.25, 0, 0, 0], np.float32)), 1, 0)
     assert (out.view(torch.int16).cpu().numpy().view(np.uint16) == want).all()
+
+
+# ------------------------------------------------------------------ attention-side kernels
+@pytest.mark.parametrize("b,t,h,kv,d,s_max", [(1, 1, 20, 5, 128, 64), (2, 24, 4, 2, 64, 32), (3, 5, 20, 5, 128, 40)])
+def test_rope_kv_store(lib, b, t, h, kv, d, s_max):
+    rng = np.random.default_rng(700 + b + t)
+    qkv = make_bf16_activations(b * t, (h + 2 * kv) * d, 701 + t)
+    pos = np.sort(rng.choice(s_max, t, replace=False)).astype(np.int64)
+    ang = (pos[:, None] * (1.0 / 500000.0 ** (np.arange(0, d, 2) / d))[None, :]).astype(np.float32)
+    cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    sentinel = 0x7FC1
+    ck = np.full((b, kv, s_max, d), sentinel, np.uint16)
+    cv = np.full((b, kv, s_max, d), sentinel, np.uint16)
+    qd, ckd, cvd = torch.zeros((b, h, t, d), dtype=torch.int16, device="cuda"), _dev(ck), _dev(cv)
+    xd, cd, sd, pd = _dev(qkv), _dev(cos), _dev(sin), _dev(pos)      # named: they must outlive the launch
+    lib.ternaspmm_rope_kv_store(_vp(xd), _vp(cd), _vp(sd), _vp(pd), _vp(qd), _vp(ckd), _vp(cvd), b, t, h, kv, d,
+                                s_max, None)
+    torch.cuda.synchronize()
+    x = qkv.reshape(b, t, h + 2 * kv, d)
+    want_q = O.rope_rotate_half(x[:, :, :h], cos[None, :, None], sin[None, :, None]).transpose(0, 2, 1, 3)
+    want_k = O.rope_rotate_half(x[:, :, h:h + kv], cos[None, :, None], sin[None, :, None]).transpose(0, 2, 1, 3)
+    want_v = x[:, :, h + kv:].transpose(0, 2, 1, 3)
+    got_q = qd.cpu().numpy().view(np.uint16)
+    got_k, got_v = ckd.cpu().numpy().view(np.uint16), cvd.cpu().numpy().view(np.uint16)
+    assert (got_q == want_q).all()
+    assert (got_k[:, :, pos] == want_k).all()
+    assert (got_v[:, :, pos] == want_v).all()
+    untouched = np.setdiff1d(np.arange(s_max), pos)
+    assert (got_k[:, :, untouched] == sentinel).all() and (got_v[:, :, untouched] == sentinel).all()
+
+
+@pytest.mark.parametrize("b,h,kv,d,s_max,n", [(1, 20, 5, 128, 256, 1), (1, 20, 5, 128, 256, 160), (8, 20, 5, 128, 512, 512),
+                                              (2, 4, 2, 64, 40, 17), (1, 20, 5, 128, 4096, 4000)])
+def test_decode_attention(lib, b, h, kv, d, s_max, n):
+    q = make_bf16_activations(b * h, d, 710 + n).reshape(b, h, d)
+    k = make_bf16_activations(b * kv * s_max, d, 711 + n).reshape(b, kv, s_max, d)
+    v = make_bf16_activations(b * kv * s_max, d, 712 + n, outlier_frac=0.01).reshape(b, kv, s_max, d)
+    pos = np.array([n - 1], np.int64)
+    od = torch.zeros((b, h * d), dtype=torch.int16, device="cuda")
+    qd, kd, vd, pd = _dev(q), _dev(k), _dev(v), _dev(pos)            # named: they must outlive the launch
+    lib.ternaspmm_decode_attention(_vp(qd), _vp(kd), _vp(vd), _vp(pd), _vp(od), b, h, kv, d, s_max, float(d) ** -0.5, None)
+    torch.cuda.synchronize()
+    got = O.bf16_bits_to_f32(od.cpu().numpy().view(np.uint16)).reshape(b, h, d).astype(np.float64)
+    want = O.attention_one_token(q, k, v, n, float(d) ** -0.5)
+    # fp32 softmax and accumulation, bf16 output: relative to the largest output of the head
+    tol = 2.0 ** -7 * np.abs(want).max(axis=-1, keepdims=True) + 1e-6
+    assert (np.abs(got - want) <= tol).all(), float((np.abs(got - want) / tol).max())

@@ -128,3 +128,25 @@ def test_relu2_mul_and_residual_add_small_cases():
     assert O.bf16_bits_to_f32(O.residual_add(a, b)).tolist() == [1.0]
     c = O.f32_to_bf16_bits(np.array([3 * 2.0 ** -8], np.float32))
     assert O.bf16_bits_to_f32(O.residual_add(a, c)).tolist() == [1.0 + 2.0 ** -6]
+
+
+def test_rope_and_attention_closed_forms():
+    """Angle 0 is the identity, angle pi/2 maps (x1, x2) to (-x2, x1); attention over identical value
+    rows returns that row, and a key that dominates the softmax returns its value row."""
+    x = make_bf16_activations(3, 64, 81)
+    zero, one = np.zeros((3, 32), np.float32), np.ones((3, 32), np.float32)
+    assert (O.rope_rotate_half(x, one, zero) == x).all()
+    xf = O.bf16_bits_to_f32(x)
+    want = np.concatenate([-xf[:, 32:], xf[:, :32]], axis=-1)
+    assert (O.bf16_bits_to_f32(O.rope_rotate_half(x, zero, one)) == want).all()
+    q = make_bf16_activations(2 * 4, 64, 82).reshape(2, 4, 64)
+    k = make_bf16_activations(2 * 2 * 10, 64, 83).reshape(2, 2, 10, 64)
+    v = np.broadcast_to(make_bf16_activations(1, 64, 84), (2, 2, 10, 64)).copy()
+    got = O.attention_one_token(q, k, v, 7, 0.125)
+    assert np.allclose(got, np.broadcast_to(O.bf16_bits_to_f32(v[0, 0, 0]), got.shape), rtol=0, atol=1e-12)
+    k2 = np.zeros((1, 1, 5, 64), np.uint16)
+    k2[0, 0, 3] = O.f32_to_bf16_bits(np.full(64, 8.0, np.float32))
+    q2 = O.f32_to_bf16_bits(np.full((1, 1, 64), 8.0, np.float32))
+    v2 = make_bf16_activations(5, 64, 85).reshape(1, 1, 5, 64)
+    assert np.allclose(O.attention_one_token(q2, k2, v2, 5, 1.0)[0, 0], O.bf16_bits_to_f32(v2[0, 0, 3]), atol=1e-9)
+    assert not np.allclose(O.attention_one_token(q2, k2, v2, 3, 1.0)[0, 0], O.bf16_bits_to_f32(v2[0, 0, 3]), atol=1e-3)
