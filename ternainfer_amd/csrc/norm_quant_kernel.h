@@ -69,16 +69,31 @@ __global__ __launch_bounds__(kNormThreads) void terna_norm_quant_kernel(
     const int nvec = K >> 3;
     const uint16_t* xr = x + row * static_cast<size_t>(GLU ? 2 * K : K);
 
+    // Every global load of the row -- input, second operand, norm weight -- is issued before the
+    // first use: with one row per workgroup the kernel's time is its chain of memory round trips.
+    u32x4 raw_x[kNormMaxVecs], raw_b[kNormMaxVecs], raw_w[kNormMaxVecs];
+    const bool has_b = GLU || residual != nullptr;
+    const uint16_t* br = GLU ? xr + K : residual + row * K;
+#pragma unroll
+    for (int i = 0; i < kNormMaxVecs; ++i) {
+        const int v = tid + i * kNormThreads;
+        if (v < nvec) {
+            raw_x[i] = *reinterpret_cast<const u32x4*>(xr + 8 * v);
+            if (has_b) raw_b[i] = *reinterpret_cast<const u32x4*>(br + 8 * v);
+            raw_w[i] = *reinterpret_cast<const u32x4*>(weight + 8 * v);
+        }
+    }
+
     float h[kNormMaxVecs][8];
     float ssq = 0.0f;
 #pragma unroll
     for (int i = 0; i < kNormMaxVecs; ++i) {
         const int v = tid + i * kNormThreads;
         if (v < nvec) {
-            unpack_bf16x8(*reinterpret_cast<const u32x4*>(xr + 8 * v), h[i]);
+            unpack_bf16x8(raw_x[i], h[i]);
             if constexpr (GLU) {
                 float g[8];
-                unpack_bf16x8(*reinterpret_cast<const u32x4*>(xr + K + 8 * v), g);
+                unpack_bf16x8(raw_b[i], g);
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const float r = fmaxf(h[i][j], 0.0f);
@@ -86,7 +101,7 @@ __global__ __launch_bounds__(kNormThreads) void terna_norm_quant_kernel(
                 }
             } else if (residual != nullptr) {
                 float r[8];
-                unpack_bf16x8(*reinterpret_cast<const u32x4*>(residual + row * K + 8 * v), r);
+                unpack_bf16x8(raw_b[i], r);
 #pragma unroll
                 for (int j = 0; j < 8; ++j) h[i][j] = round_bf16(h[i][j] + r[j]);
                 if (sum_out != nullptr) *reinterpret_cast<u32x4*>(sum_out + row * K + 8 * v) = pack_bf16x8(h[i]);
@@ -107,7 +122,7 @@ __global__ __launch_bounds__(kNormThreads) void terna_norm_quant_kernel(
         const int v = tid + i * kNormThreads;
         if (v < nvec) {
             float w[8];
-            unpack_bf16x8(*reinterpret_cast<const u32x4*>(weight + 8 * v), w);
+            unpack_bf16x8(raw_w[i], w);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 h[i][j] = round_bf16(h[i][j] * rstd * w[j]);
