@@ -48,8 +48,7 @@ __device__ __forceinline__ u32x4 pack_bf16x8(const float f[8])
 {
     uint32_t d[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-        d[j] = float_to_bf16_bits(f[2 * j]) | (static_cast<uint32_t>(float_to_bf16_bits(f[2 * j + 1])) << 16);
+    for (int j = 0; j < 4; ++j) d[j] = pack_bf16x2(f[2 * j], f[2 * j + 1]);
     return u32x4{d[0], d[1], d[2], d[3]};
 }
 __device__ __forceinline__ float round_bf16(float v) { return bf16_bits_to_float(float_to_bf16_bits(v)); }

@@ -38,13 +38,17 @@ __device__ __forceinline__ float bf16_bits_to_float(uint16_t h)
     return __uint_as_float(static_cast<uint32_t>(h) << 16);
 }
 
-// Round to nearest even, NaN kept quiet: the rounding of __float2bfloat16_rn.
+// Round to nearest even (the rounding of __float2bfloat16_rn): gfx950's v_cvt_pk_bf16_f32.
 __device__ __forceinline__ uint16_t float_to_bf16_bits(float f)
 {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return static_cast<uint16_t>(u >> 16);
+    return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
+}
+// Two at once: lo in bits 0..15, hi in bits 16..31 (one instruction).
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
+{
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
 }
 
 // Weight-scale group of output column n on the decode path (Reduction_Kernel.cuh:46-54).
