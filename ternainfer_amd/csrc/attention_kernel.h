@@ -85,12 +85,10 @@ __global__ __launch_bounds__(256) void terna_rope_kv_store_kernel(
 }
 
 // One workgroup per (sequence, head).  q bf16 [B][H][D]; keys / values of kv head h / (H/KV) at
-// slots 0 .. pos[0]; out bf16 [B][H*D].  Dynamic LDS: (S + D + 16*D) floats.
-//   pass 1  one thread per cache slot: the whole key row is fetched with D/8 independent 16-byte
-//           loads (all in flight together) and multiplied with q, which every lane reads from
-//           LDS at the same address (a broadcast)
+// slots 0 .. pos[0]; out bf16 [B][H*D].  Dynamic LDS: (S + 2048) floats.
+//   pass 1  q K^T on the matrix cores, 16 slots per MFMA tile, four tiles per wave requested up front
 //   pass 2  softmax over the scores in LDS
-//   pass 3  thread (slice, chunk): slots slice, slice+S', ... x 8 dimensions of V, four rows in
+//   pass 3  thread (slice, chunk): slots slice, slice+S', ... x 8 dimensions of V, eight rows in
 //           flight per thread; the slices are summed through LDS
 template <int D>
 __global__ __launch_bounds__(256) void terna_decode_attention_kernel(
@@ -101,9 +99,8 @@ __global__ __launch_bounds__(256) void terna_decode_attention_kernel(
     constexpr int CH = D / 8;                    // 8-dimension chunks of a row
     constexpr int SLICES = 256 / CH;
     extern __shared__ __align__(16) float lds[];
-    float* qs = lds;                             // [D]  q * scale
-    float* part = lds + D;                       // [SLICES][D]
-    float* score = lds + D + SLICES * D;         // [S]
+    float* part = lds;                           // [SLICES][D]
+    float* score = lds + SLICES * D;             // [S]
     __shared__ float red[8];
 
     const int tid = threadIdx.x;
@@ -114,29 +111,65 @@ __global__ __launch_bounds__(256) void terna_decode_attention_kernel(
     const uint16_t* kbase = cache_k + (static_cast<size_t>(b) * KV + kvh) * S * D;
     const uint16_t* vbase = cache_v + (static_cast<size_t>(b) * KV + kvh) * S * D;
 
-    if (tid < D) qs[tid] = bf16_bits_to_float(q[(static_cast<size_t>(b) * H + h) * D + tid]) * scale;
-    __syncthreads();
+    // Everything the first round of each pass needs is requested before anything is used: KT key
+    // tiles per wave, the first VU value rows of this thread's slice, q.  Slots >= n hold stale or
+    // unwritten cache lines; they are read (the cache is S slots long) and masked out below.
+    //
+    // ---- pass 1: scores on the matrix cores.  A tile is 16 cache slots; v_mfma_f32_16x16x32_bf16
+    // takes the key rows as A (lane: slot L & 15, dimensions 32j + 8(L >> 4) .. +7 -- the 16 bytes
+    // the lane loads) and q as B, the same in all 16 columns, so every column of the result holds
+    // the 16 scores and column 0 (lanes 0, 16, 32, 48: four slots each) writes them.  No shuffles.
+    constexpr int NJ = D / 32;                   // MFMAs (32 dimensions each) per tile
+    constexpr int KT = 4;                        // key tiles in flight per wave: slots 0 .. 255
+    constexpr int VU = 8;                        // value rows in flight per thread
+    const int r16 = lane & 15, kblk = lane >> 4;
+    const int chunk = tid % CH, slice = tid / CH;
+    u32x4 kr[KT][NJ], vr[VU], qr[NJ];
+#pragma unroll
+    for (int t = 0; t < KT; ++t) {
+        const int sk = 16 * (wave + 4 * t) + r16;
+        const uint16_t* kp = kbase + static_cast<size_t>(sk < S ? sk : 0) * D + 8 * kblk;
+#pragma unroll
+        for (int jj = 0; jj < NJ; ++jj) kr[t][jj] = *reinterpret_cast<const u32x4*>(kp + 32 * jj);
+    }
+#pragma unroll
+    for (int u = 0; u < VU; ++u) {
+        const int sv = slice + u * SLICES;
+        vr[u] = *reinterpret_cast<const u32x4*>(vbase + static_cast<size_t>(sv < S ? sv : 0) * D + chunk * 8);
+    }
+#pragma unroll
+    for (int jj = 0; jj < NJ; ++jj)
+        qr[jj] = *reinterpret_cast<const u32x4*>(q + (static_cast<size_t>(b) * H + h) * D + 32 * jj + 8 * kblk);
 
-    // ---- pass 1: scores
     float mx = -INFINITY;
-    for (int s = tid; s < n; s += 256) {
-        const u32x4* kp = reinterpret_cast<const u32x4*>(kbase + static_cast<size_t>(s) * D);
-        u32x4 kr[CH];
+    auto score_tile = [&](int tile, const u32x4 (&k)[NJ]) {
+        f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int c = 0; c < CH; ++c) kr[c] = kp[c];
-        float d = 0.0f;
+        for (int jj = 0; jj < NJ; ++jj)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, k[jj]), __builtin_bit_cast(bf16x8, qr[jj]), acc, 0, 0, 0);
+        if (r16 == 0) {
 #pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            float kf[8];
-            unpack_bf16x8(kr[c], kf);
-            const f32x4 q0 = *reinterpret_cast<const f32x4*>(qs + 8 * c), q1 = *reinterpret_cast<const f32x4*>(qs + 8 * c + 4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) d = fmaf(q0[e], kf[e], d);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) d = fmaf(q1[e], kf[4 + e], d);
+            for (int v = 0; v < 4; ++v) {
+                const int sk = 16 * tile + 4 * kblk + v;
+                if (sk < n) {
+                    const float d = acc[v] * scale;
+                    score[sk] = d;
+                    mx = fmaxf(mx, d);
+                }
+            }
         }
-        score[s] = d;
-        mx = fmaxf(mx, d);
+    };
+    const int tiles = (n + 15) >> 4;
+#pragma unroll
+    for (int t = 0; t < KT; ++t)
+        if (wave + 4 * t < tiles) score_tile(wave + 4 * t, kr[t]);
+    for (int tile = wave + 4 * KT; tile < tiles; tile += 4) {     // beyond 256 slots: plain loop
+        u32x4 k[NJ];
+        const int sk = 16 * tile + r16;
+        const uint16_t* kp = kbase + static_cast<size_t>(sk < S ? sk : 0) * D + 8 * kblk;
+#pragma unroll
+        for (int jj = 0; jj < NJ; ++jj) k[jj] = *reinterpret_cast<const u32x4*>(kp + 32 * jj);
+        score_tile(tile, k);
     }
     mx = wave_max(mx);
     if (lane == 0) red[wave] = mx;
@@ -155,21 +188,22 @@ __global__ __launch_bounds__(256) void terna_decode_attention_kernel(
     __syncthreads();
     sum = (red[4] + red[5]) + (red[6] + red[7]);
 
-    // ---- pass 3: weighted sum of the value rows
-    const int chunk = tid % CH, slice = tid / CH;
+    // ---- pass 3: weighted sum of the value rows, VU rows per round (the first round is already here)
     float acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-    for (int s0 = slice; s0 < n; s0 += 4 * SLICES) {
-        u32x4 vr[4];
-        float p[4];
+    for (int s0 = slice; s0 < n; s0 += VU * SLICES) {
+        float p[VU];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < VU; ++u) {
             const int s = s0 + u * SLICES;
-            const int sc = s < n ? s : s0;       // past the end: re-read a valid row with weight 0
-            vr[u] = *reinterpret_cast<const u32x4*>(vbase + static_cast<size_t>(sc) * D + chunk * 8);
+            if (s0 != slice) {
+                const int sc = s < n ? s : s0;   // past the end: re-read a valid row with weight 0
+                vr[u] = *reinterpret_cast<const u32x4*>(vbase + static_cast<size_t>(sc) * D + chunk * 8);
+            }
             p[u] = s < n ? score[s] : 0.0f;
+            if (!(s < n)) vr[u] = u32x4{0u, 0u, 0u, 0u};     // never multiply stale cache contents (could be NaN)
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < VU; ++u) {
             float vf[8];
             unpack_bf16x8(vr[u], vf);
 #pragma unroll

@@ -527,7 +527,7 @@ void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, 
         std::fprintf(stderr, "ternaspmm_decode_attention: unsupported arguments (H=%d KV=%d D=%d S=%d)\n", H, KV, D, S);
         return;
     }
-    const size_t lds = (static_cast<size_t>(S) + D + (256 / (D / 8)) * D) * sizeof(float);
+    const size_t lds = (static_cast<size_t>(S) + (256 / (D / 8)) * D) * sizeof(float);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (D == 128)
         terna_decode_attention_kernel<128><<<dim3(B * H), dim3(256), lds, st>>>(q, cache_k, cache_v, pos, out, H, KV, S, scale);
