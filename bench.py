@@ -275,13 +275,13 @@ def run_prefill(args, torch, T, lib):
     per_shape = {}
     dense_main_us = 0.0
     for mt, xs in mats:
-        for m in sorted(xs):
+        for m in ([] if args.no_per_shape else sorted(xs)):
             launch(mt, xs, m, stream)
             torch.cuda.synchronize()
             g = capture(torch, lambda s, mt=mt, xs=xs, m=m: [launch(mt, xs, m, s) for _ in range(10)])
             us = time_graph(torch, g, 5, 2) * 1e3 / 10
             tf = 2.0 * m * mt.n * mt.k / us / 1e6
-            d_us = None if args.no_per_shape else dense_us(m, mt.n, mt.k)
+            d_us = dense_us(m, mt.n, mt.k)
             per_shape[f"{mt.name}_{mt.k}x{mt.n}_M{m}"] = {"us": us, "tflops": tf, "frac": tf / peak,
                                                          "vendor_dense_gemm_us": d_us}
             if m == m_main and d_us is not None and dense_main_us is not None:
