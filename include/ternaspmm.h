@@ -165,6 +165,19 @@ void ternaspmm_rmsnorm_quant(const terna_bf16* x, const terna_bf16* residual, te
 void ternaspmm_relu2_mul_rmsnorm_quant(const terna_bf16* x13, const terna_bf16* weight, float eps, terna_bf16* y_out,
                                        int8_t* xq_out, terna_bf16* s_out, int M, int F, terna_stream stream);
 
+/* The same prologue inside the small-M linear: [residual add] -> RMSNorm -> quant_input -> ternary matmul ->
+ * decode epilogue in ONE launch (x, residual, sum_out, norm_weight, eps as ternaspmm_rmsnorm_quant; packed, out,
+ * ws, ws_num as bitlinear_TernaSpMM_packed).  xq_out / s_out are optional copies of the quantised activations
+ * (NULL = not written).  sum_out must not alias x or residual (every workgroup reads both).  Supported: M <= 16
+ * and K <= 3072 (K <= 2560 when N > 4096); returns 1 when the launch was enqueued, 0 when the shape is outside
+ * that range and nothing was done -- the caller then runs ternaspmm_rmsnorm_quant + bitlinear_TernaSpMM_packed.
+ * Every workgroup repeats the prologue arithmetic, so the single launch pays for M = 1 (measured on MI355X:
+ * 5.2-5.6 us against 7.2-7.5 us for the pair) and is no faster than the pair from M = 8 on. */
+int bitlinear_TernaSpMM_packed_fused(const terna_bf16* x, const terna_bf16* residual, terna_bf16* sum_out,
+                                     const terna_bf16* norm_weight, float eps, const void* packed, terna_bf16* out,
+                                     const terna_bf16* ws, int ws_num, int8_t* xq_out, terna_bf16* s_out, int M,
+                                     int N, int K, terna_stream stream);
+
 /* ---- Attention-side kernels of a decode step (no counterpart in the reference's library) -----------
  * They stand where the reference calls xformers' rope_padded (model.py:218-229) and
  * fmha.memory_efficient_attention_forward (model.py:231-233).

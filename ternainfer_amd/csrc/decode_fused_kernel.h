@@ -1,0 +1,235 @@
+// Small-M TernaSpMM on the P2 layout with its prologue inside: [residual add] -> RMSNorm ->
+// per-row int8 quantisation -> ternary matmul -> scale epilogue, one launch.
+//
+// In terna_decode_packed_kernel every workgroup (one 16-row band of W) already reads the whole
+// activation row block: its waves take the band's 64-column tiles round robin.  So the row
+// statistics the prologue needs (sum of squares, then max |y|) cost each workgroup two
+// reductions over data it holds anyway, and the separate norm/quantise launch -- 4 us of a
+// 9 us pair in a decode step -- disappears.  Every workgroup recomputes the same statistics from
+// the same values in the same order, so all bands see identical int8 activations.
+//
+//   h  = x, or bf16(x + residual)            (band 0 also writes h to sum_out: the new stream)
+//   y  = bf16(h * rsqrt(mean(h^2) + eps) * norm_w)
+//   s  = bf16(127 / max(max|y|, 1e-5)),  q = clamp(rint(y * s), -128, 127)
+//   out[m][n] = bf16((sum_k q[m][k] W[n][k] / s[m]) * ws[group(n)])      (decode epilogue)
+//
+// Phases of a wave (T = its tiles, at most TMAX):
+//   A  request everything: T weight words, T activation pieces (x, residual), then the norm
+//      weights of its columns; h -> registers (packed bf16), sum of squares per row
+//   B  rows' sums: the lanes that share a row (shuffles), then the waves in LDS  -- barrier 1
+//   C  y -> registers, max |y| per row, same reduction                      -- barrier 2
+//   D  per tile: quantise, int8 slab -> wave-private LDS -> operand order, MFMA
+//   E  cross-wave sum of the accumulators + epilogue (wave 0)               -- barrier 3
+#pragma once
+
+#include "decode_packed_kernel.h"
+#include "norm_quant_kernel.h"
+
+namespace terna {
+
+// MP consecutive columns of one activation row, as a lane holds them: bf16 storage in, floats out.
+template <int MP> struct RowPiece;
+template <> struct RowPiece<16> {
+    u32x4 v[2];
+    __device__ void load(const uint16_t* p) { v[0] = reinterpret_cast<const u32x4*>(p)[0]; v[1] = reinterpret_cast<const u32x4*>(p)[1]; }
+    __device__ void store(uint16_t* p) const { reinterpret_cast<u32x4*>(p)[0] = v[0]; reinterpret_cast<u32x4*>(p)[1] = v[1]; }
+    __device__ void zero() { v[0] = v[1] = u32x4{0u, 0u, 0u, 0u}; }
+    __device__ void unpack(float f[16]) const { unpack_bf16x8(v[0], f); unpack_bf16x8(v[1], f + 8); }
+    __device__ void pack(const float f[16]) { v[0] = pack_bf16x8(f); v[1] = pack_bf16x8(f + 8); }
+};
+template <> struct RowPiece<8> {
+    u32x4 v;
+    __device__ void load(const uint16_t* p) { v = *reinterpret_cast<const u32x4*>(p); }
+    __device__ void store(uint16_t* p) const { *reinterpret_cast<u32x4*>(p) = v; }
+    __device__ void zero() { v = u32x4{0u, 0u, 0u, 0u}; }
+    __device__ void unpack(float f[8]) const { unpack_bf16x8(v, f); }
+    __device__ void pack(const float f[8]) { v = pack_bf16x8(f); }
+};
+template <> struct RowPiece<1> {
+    uint16_t v;
+    __device__ void load(const uint16_t* p) { v = *p; }
+    __device__ void store(uint16_t* p) const { *p = v; }
+    __device__ void zero() { v = 0; }
+    __device__ void unpack(float f[1]) const { f[0] = bf16_bits_to_float(v); }
+    __device__ void pack(const float f[1]) { v = float_to_bf16_bits(f[0]); }
+};
+
+// MP = rows a wave's 64 lanes cover at once (M <= MP): 64/MP lanes walk along a row, MP columns
+// each, so a lane handles MP elements per tile -- the prologue arithmetic, which every workgroup
+// repeats, costs in proportion to the batch rows that exist, not to the 16 the MFMA tile has.
+template <int WAVES, int TMAX, bool RES, int MP>
+__global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, uint16_t* __restrict__ sum_out,
+    const uint16_t* __restrict__ norm_w, float eps, const uint32_t* __restrict__ packed,
+    uint16_t* __restrict__ out, const uint16_t* __restrict__ ws, int ws_num, int8_t* __restrict__ xq_out,
+    uint16_t* __restrict__ s_out, int M, int N, int K)
+{
+    using XQ = XSlab<int8_t>;
+    using Piece = RowPiece<MP>;
+    constexpr int LPR = 64 / MP;                     // lanes per row
+    __shared__ i32x4 red[WAVES][64];
+    __shared__ __align__(16) uint8_t slab_all[WAVES][16 * XQ::kPitch];
+    __shared__ __align__(16) float stat[2][16][WAVES];
+    __shared__ float s_row[16];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int band = blockIdx.x;
+    const int ktiles = K >> 6;
+    const int i = lane & 15, g = lane >> 4;          // operand coordinates: weight row / batch row i, 16-column group g
+    const int row = lane / LPR, cl = (lane % LPR) * MP;   // load coordinates: batch row, first of MP columns
+    const bool row_ok = row < M;
+    const bool writer = band == 0;                   // the workgroup that publishes h, q and s
+
+    // ---- phase A: request everything
+    uint32_t wword[TMAX];
+    Piece xr[TMAX], rr[TMAX], nw[TMAX];
+#pragma unroll
+    for (int t = 0; t < TMAX; ++t) {
+        const int j = wave + WAVES * t;
+        const bool valid = j < ktiles;
+        wword[t] = valid ? packed[(static_cast<size_t>(band) * ktiles + j) * 64 + i * 4 + g] : 0u;
+        const size_t off = static_cast<size_t>(row_ok ? row : 0) * K + (valid ? j : 0) * 64 + cl;
+        if (valid && row_ok) {
+            xr[t].load(x + off);
+            if constexpr (RES) rr[t].load(residual + off);
+        } else {
+            xr[t].zero();
+            if constexpr (RES) rr[t].zero();
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < TMAX; ++t) {
+        const int j = wave + WAVES * t;
+        nw[t].load(norm_w + (j < ktiles ? j : 0) * 64 + cl);
+    }
+    // this wave's LDS slot: rows the batch does not have stay zero
+    uint8_t* slab = slab_all[wave];
+    for (int o = lane * 16; o < 16 * XQ::kPitch; o += 64 * 16) *reinterpret_cast<u32x4*>(slab + o) = u32x4{0u, 0u, 0u, 0u};
+
+    float ssq = 0.0f;
+#pragma unroll
+    for (int t = 0; t < TMAX; ++t) {
+        const int j = wave + WAVES * t;
+        float f[MP];
+        xr[t].unpack(f);
+        if constexpr (RES) {
+            float r[MP];
+            rr[t].unpack(r);
+#pragma unroll
+            for (int e = 0; e < MP; ++e) f[e] = round_bf16(f[e] + r[e]);
+            xr[t].pack(f);
+            if (writer && sum_out != nullptr && j < ktiles && row_ok)
+                xr[t].store(sum_out + static_cast<size_t>(row) * K + j * 64 + cl);
+        }
+#pragma unroll
+        for (int e = 0; e < MP; ++e) ssq = fmaf(f[e], f[e], ssq);
+    }
+
+    // ---- phase B: sum of squares per row (LPR lanes share a row, then the waves)
+    auto row_reduce = [&](float v, int which, bool is_max) {
+#pragma unroll
+        for (int off = 1; off < LPR; off <<= 1) {
+            const float o = __shfl_xor(v, off);
+            v = is_max ? fmaxf(v, o) : v + o;
+        }
+        if ((lane % LPR) == 0) stat[which][row][wave] = v;
+        __syncthreads();
+        const f32x4* p = reinterpret_cast<const f32x4*>(stat[which][row]);
+        float r = 0.0f;
+#pragma unroll
+        for (int q4 = 0; q4 < WAVES / 4; ++q4) {
+            const f32x4 c = p[q4];
+            if (is_max) r = fmaxf(fmaxf(r, fmaxf(c.x, c.y)), fmaxf(c.z, c.w));
+            else r += (c.x + c.y) + (c.z + c.w);
+        }
+        return r;
+    };
+    ssq = row_reduce(ssq, 0, false);
+    const float rstd = rsqrtf(ssq / static_cast<float>(K) + eps);
+
+    // ---- phase C: y in place of h, max |y| per row
+    float amax = 0.0f;
+#pragma unroll
+    for (int t = 0; t < TMAX; ++t) {
+        float w[MP], f[MP];
+        nw[t].unpack(w);
+        xr[t].unpack(f);
+        const bool valid = wave + WAVES * t < ktiles;
+#pragma unroll
+        for (int e = 0; e < MP; ++e) {
+            f[e] = round_bf16(f[e] * rstd * w[e]);
+            if (valid) amax = fmaxf(amax, fabsf(f[e]));
+        }
+        xr[t].pack(f);
+    }
+    amax = row_reduce(amax, 1, true);
+    const uint16_t s_bits = float_to_bf16_bits(__fdiv_rn(127.0f, fmaxf(amax, 1e-5f)));
+    const float s = bf16_bits_to_float(s_bits);
+    if (wave == 0 && (lane % LPR) == 0) {
+        s_row[row] = s;
+        if (writer && s_out != nullptr && row_ok) s_out[row] = s_bits;
+    }
+
+    // ---- phase D: quantise a tile, turn it into operand order through the wave's LDS slot, multiply
+    i32x4 acc = {0, 0, 0, 0};
+#pragma unroll
+    for (int t = 0; t < TMAX; ++t) {
+        const int j = wave + WAVES * t;
+        if (j < ktiles) {
+            float f[MP];
+            xr[t].unpack(f);
+            uint8_t q[MP];
+#pragma unroll
+            for (int e = 0; e < MP; ++e) {
+                const float r = __builtin_amdgcn_fmed3f(rintf(__fmul_rn(f[e], s)), -128.0f, 127.0f);
+                q[e] = static_cast<uint8_t>(static_cast<int>(r) & 0xff);
+            }
+            uint8_t* dst = slab + row * XQ::kPitch + cl;
+            int8_t* gdst = xq_out + static_cast<size_t>(row_ok ? row : 0) * K + j * 64 + cl;
+            const bool publish = writer && xq_out != nullptr && row_ok;
+            if constexpr (MP == 1) {
+                *dst = q[0];
+                if (publish) *gdst = static_cast<int8_t>(q[0]);
+            } else {
+                uint32_t d[MP / 4];
+#pragma unroll
+                for (int e = 0; e < MP / 4; ++e)
+                    d[e] = q[4 * e] | (q[4 * e + 1] << 8) | (q[4 * e + 2] << 16) | (static_cast<uint32_t>(q[4 * e + 3]) << 24);
+                if constexpr (MP == 8) {
+                    *reinterpret_cast<u32x2*>(dst) = u32x2{d[0], d[1]};
+                    if (publish) *reinterpret_cast<u32x2*>(gdst) = u32x2{d[0], d[1]};
+                } else {
+                    *reinterpret_cast<u32x4*>(dst) = u32x4{d[0], d[1], d[2], d[3]};
+                    if (publish) *reinterpret_cast<u32x4*>(gdst) = u32x4{d[0], d[1], d[2], d[3]};
+                }
+            }
+            const i32x4 bq = __builtin_bit_cast(i32x4, *reinterpret_cast<const u32x4*>(slab + i * XQ::kPitch + g * 16));
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(expand_word_i8(wword[t]), bq, acc, 0, 0, 0);
+        }
+    }
+
+    // ---- phase E: cross-wave sum in wave order + the decode epilogue (lane: batch row i, output rows 4g .. 4g+3)
+    red[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0) {
+        i32x4 sum = red[0][lane];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) sum += red[w][lane];
+        if (i < M) {
+            const int n0 = band * 16 + 4 * g;
+            const Epilogue ep{nullptr, ws, nullptr, ws_num, EP_I8_DECODE};
+            EpilogueRegs e;
+            e.s = s_row[i];
+            load_col_scales(ep, n0, N, e.w);
+            uint16_t o[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) o[v] = apply_epilogue<int>(EP_I8_DECODE, e, v, sum[v]);
+            const u32x2 pk = {o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16)};
+            *reinterpret_cast<u32x2*>(out + static_cast<size_t>(i) * N + n0) = pk;
+        }
+    }
+}
+
+}  // namespace terna

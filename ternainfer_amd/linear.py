@@ -147,6 +147,30 @@ def rmsnorm_quant(x, weight, eps, residual=None, quant=True):
     return y, h
 
 
+def rmsnorm_linear_packed(x, norm_weight, eps, packed, ws, ws_num, out_features, residual=None):
+    """[residual add] -> RMSNorm -> quant_input -> int8 TernaSpMM on a P2 weight.  One launch for a single
+    row where the library supports the shape (every workgroup of the fused kernel repeats the prologue
+    arithmetic, which pays at M = 1: 5.2-5.6 us against 7.2-7.5 us on MI355X, and no longer at M = 8),
+    else rmsnorm_quant + TernaInfer_linear_packed.
+    x, residual: bf16 [M, K].  Returns (out bf16 [M, out_features], h = x + residual)."""
+    m, k = x.shape
+    x = x.contiguous()
+    lib = _lib.load()
+    h = x
+    if residual is not None:
+        residual = residual.contiguous()
+        h = torch.empty_like(x)
+    out = torch.empty((m, out_features), dtype=torch.bfloat16, device=x.device)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    done = m == 1 and lib.bitlinear_TernaSpMM_packed_fused(
+        _p(x), _p(residual) if residual is not None else None, _p(h) if residual is not None else None,
+        _p(norm_weight), float(eps), _p(packed), _p(out), _p(ws), ws_num, None, None, m, out_features, k, stream)
+    if done:
+        return out, h
+    xq, s, h = rmsnorm_quant(x, norm_weight, eps, residual=residual)
+    return TernaInfer_linear_packed(xq, packed, s, ws, ws_num, out_features), h
+
+
 def relu2_mul_rmsnorm_quant(x13, weight, eps, quant=True):
     """Fused squared_relu(x1) * x3 -> ffn_sub_norm -> [quant_input] (model.py:279-281 + 120-123).
     x13: bf16 [M, 2F].  Returns (xq int8 [M, F], s bf16 [M]) when quant else y bf16 [M, F]."""

@@ -21,7 +21,7 @@ import torch
 from torch.nn import functional as F
 
 from . import _lib
-from .linear import relu2_mul_rmsnorm_quant, rmsnorm_quant
+from .linear import relu2_mul_rmsnorm_quant, rmsnorm_linear_packed, rmsnorm_quant
 
 
 @dataclass
@@ -142,6 +142,8 @@ class Block:
                 return lin.quantised(*relu2_mul_rmsnorm_quant(x, weight, eps)), None
             return lin.dense(relu2_mul_rmsnorm_quant(x, weight, eps, quant=False)), None
         if self.act == "int8":
+            if x.shape[0] == 1:            # single-row decode step: prologue and linear in one launch
+                return rmsnorm_linear_packed(x, weight, eps, lin.packed, lin.ws, lin.ws_num, lin.n, residual=residual)
             xq, s, h = rmsnorm_quant(x, weight, eps, residual=residual)
             return lin.quantised(xq, s), h
         y, h = rmsnorm_quant(x, weight, eps, residual=residual, quant=False)
