@@ -178,6 +178,13 @@ int bitlinear_TernaSpMM_packed_fused(const terna_bf16* x, const terna_bf16* resi
                                      const terna_bf16* ws, int ws_num, int8_t* xq_out, terna_bf16* s_out, int M,
                                      int N, int K, terna_stream stream);
 
+/* Gated-FFN variant: h = bf16(bf16(relu(x1)^2) * x3) from x13 (bf16 [M][2F], as ternaspmm_relu2_mul_rmsnorm_quant),
+ * norm and quantisation over F columns, then the [N][F] ternary linear.  Supported: M = 1, N <= 4096, F <= 7168;
+ * returns 0 otherwise (caller: ternaspmm_relu2_mul_rmsnorm_quant + bitlinear_TernaSpMM_packed). */
+int bitlinear_TernaSpMM_packed_fused_glu(const terna_bf16* x13, const terna_bf16* norm_weight, float eps,
+                                         const void* packed, terna_bf16* out, const terna_bf16* ws, int ws_num,
+                                         int8_t* xq_out, terna_bf16* s_out, int M, int N, int F, terna_stream stream);
+
 /* ---- Attention-side kernels of a decode step (no counterpart in the reference's library) -----------
  * They stand where the reference calls xformers' rope_padded (model.py:218-229) and
  * fmha.memory_efficient_attention_forward (model.py:231-233).

@@ -3,6 +3,6 @@ from . import _lib  # noqa: F401
 from .convert_utils import compress_weight, reorder_weight, quant_weight_int8, pack_weight_scale  # noqa: F401
 from .linear import (  # noqa: F401
     BF16BitLinear, SpBitLinear, SpBitLinearBF16, TernaInfer_linear, TernaInfer_linear_bf16,
-    TernaInfer_linear_packed, get_global_workspace, relu2_mul_rmsnorm_quant, repack_weight, rmsnorm_linear_packed, rmsnorm_quant)
+    TernaInfer_linear_packed, get_global_workspace, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant, repack_weight, rmsnorm_linear_packed, rmsnorm_quant)
 
 __version__ = "0.1"

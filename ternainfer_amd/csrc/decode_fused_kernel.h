@@ -8,7 +8,8 @@
 // 9 us pair in a decode step -- disappears.  Every workgroup recomputes the same statistics from
 // the same values in the same order, so all bands see identical int8 activations.
 //
-//   h  = x, or bf16(x + residual)            (band 0 also writes h to sum_out: the new stream)
+//   h  = x, or bf16(x + residual)            (band 0 also writes h to sum_out: the new stream),
+//        or bf16(bf16(relu(x1)^2) * x3)      (gated FFN: x = [x1 | x3], 2K columns per row)
 //   y  = bf16(h * rsqrt(mean(h^2) + eps) * norm_w)
 //   s  = bf16(127 / max(max|y|, 1e-5)),  q = clamp(rint(y * s), -128, 127)
 //   out[m][n] = bf16((sum_k q[m][k] W[n][k] / s[m]) * ws[group(n)])      (decode epilogue)
@@ -57,7 +58,9 @@ template <> struct RowPiece<1> {
 // MP = rows a wave's 64 lanes cover at once (M <= MP): 64/MP lanes walk along a row, MP columns
 // each, so a lane handles MP elements per tile -- the prologue arithmetic, which every workgroup
 // repeats, costs in proportion to the batch rows that exist, not to the 16 the MFMA tile has.
-template <int WAVES, int TMAX, bool RES, int MP>
+enum FusedMode { FUSED_PLAIN, FUSED_RESIDUAL, FUSED_GLU };
+
+template <int WAVES, int TMAX, int MODE, int MP>
 __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, uint16_t* __restrict__ sum_out,
     const uint16_t* __restrict__ norm_w, float eps, const uint32_t* __restrict__ packed,
@@ -81,6 +84,9 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
     const int row = lane / LPR, cl = (lane % LPR) * MP;   // load coordinates: batch row, first of MP columns
     const bool row_ok = row < M;
     const bool writer = band == 0;                   // the workgroup that publishes h, q and s
+    constexpr bool RES = MODE != FUSED_PLAIN;        // a second operand: the residual, or x3 of the gate
+    const size_t pitch = MODE == FUSED_GLU ? 2 * static_cast<size_t>(K) : K;
+    const uint16_t* second = MODE == FUSED_GLU ? x + K : residual;
 
     // ---- phase A: request everything
     uint32_t wword[TMAX];
@@ -90,10 +96,10 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
         const int j = wave + WAVES * t;
         const bool valid = j < ktiles;
         wword[t] = valid ? packed[(static_cast<size_t>(band) * ktiles + j) * 64 + i * 4 + g] : 0u;
-        const size_t off = static_cast<size_t>(row_ok ? row : 0) * K + (valid ? j : 0) * 64 + cl;
+        const size_t off = static_cast<size_t>(row_ok ? row : 0) * pitch + (valid ? j : 0) * 64 + cl;
         if (valid && row_ok) {
             xr[t].load(x + off);
-            if constexpr (RES) rr[t].load(residual + off);
+            if constexpr (RES) rr[t].load(second + off);
         } else {
             xr[t].zero();
             if constexpr (RES) rr[t].zero();
@@ -114,7 +120,7 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
         const int j = wave + WAVES * t;
         float f[MP];
         xr[t].unpack(f);
-        if constexpr (RES) {
+        if constexpr (MODE == FUSED_RESIDUAL) {
             float r[MP];
             rr[t].unpack(r);
 #pragma unroll
@@ -122,6 +128,15 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
             xr[t].pack(f);
             if (writer && sum_out != nullptr && j < ktiles && row_ok)
                 xr[t].store(sum_out + static_cast<size_t>(row) * K + j * 64 + cl);
+        } else if constexpr (MODE == FUSED_GLU) {
+            float r[MP];
+            rr[t].unpack(r);
+#pragma unroll
+            for (int e = 0; e < MP; ++e) {
+                const float p = fmaxf(f[e], 0.0f);
+                f[e] = round_bf16(round_bf16(p * p) * r[e]);
+            }
+            xr[t].pack(f);
         }
 #pragma unroll
         for (int e = 0; e < MP; ++e) ssq = fmaf(f[e], f[e], ssq);

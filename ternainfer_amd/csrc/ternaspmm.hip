@@ -506,39 +506,61 @@ void ternaspmm_relu2_mul_rmsnorm_quant(const terna_bf16* x13, const terna_bf16* 
     if (e != hipSuccess) die("ternaspmm_relu2_mul_rmsnorm_quant", e, __LINE__);
 }
 
-int bitlinear_TernaSpMM_packed_fused(const terna_bf16* x, const terna_bf16* residual, terna_bf16* sum_out,
-                                     const terna_bf16* norm_weight, float eps, const void* packed, terna_bf16* out,
-                                     const terna_bf16* ws, int ws_num, int8_t* xq_out, terna_bf16* s_out, int M,
-                                     int N, int K, terna_stream stream)
+// mode: FUSED_PLAIN / FUSED_RESIDUAL / FUSED_GLU.  Returns 1 when a launch was enqueued.
+static int launch_decode_fused(int mode, const terna_bf16* x, const terna_bf16* residual, terna_bf16* sum_out,
+                               const terna_bf16* norm_weight, float eps, const void* packed, terna_bf16* out,
+                               const terna_bf16* ws, int ws_num, int8_t* xq_out, terna_bf16* s_out, int M, int N,
+                               int K, hipStream_t st)
 {
     if (!shape_ok(M, N, K) || ws_num < 1 || M > 16) return 0;
     const int ktiles = K / 64;
     const bool wide = N / 16 <= 256;                  // same split as the unfused small-M kernel
-    if (wide ? ktiles > 16 * 3 : ktiles > 8 * 5) return 0;
-    hipStream_t st = static_cast<hipStream_t>(stream);
     const uint32_t* p = static_cast<const uint32_t*>(packed);
     const dim3 grid(N / 16);
-#define TERNA_FUSED(WAVES, TMAX, RES, MP)                                                                          \
-    terna_decode_fused_kernel<WAVES, TMAX, RES, MP><<<grid, dim3(WAVES * 64), 0, st>>>(                            \
+#define TERNA_FUSED(WAVES, TMAX, MODE, MP)                                                                         \
+    terna_decode_fused_kernel<WAVES, TMAX, MODE, MP><<<grid, dim3(WAVES * 64), 0, st>>>(                           \
         x, residual, sum_out, norm_weight, eps, p, out, ws, ws_num, xq_out, s_out, M, N, K)
-#define TERNA_FUSED_M(WAVES, TMAX, RES)                                                                            \
+#define TERNA_FUSED_M(WAVES, TMAX, MODE)                                                                           \
     do {                                                                                                           \
-        if (M == 1) TERNA_FUSED(WAVES, TMAX, RES, 1);                                                              \
-        else if (M <= 8) TERNA_FUSED(WAVES, TMAX, RES, 8);                                                         \
-        else TERNA_FUSED(WAVES, TMAX, RES, 16);                                                                    \
+        if (M == 1) TERNA_FUSED(WAVES, TMAX, MODE, 1);                                                             \
+        else if (M <= 8) TERNA_FUSED(WAVES, TMAX, MODE, 8);                                                        \
+        else TERNA_FUSED(WAVES, TMAX, MODE, 16);                                                                   \
     } while (0)
-    if (wide) {
-        if (residual) TERNA_FUSED_M(16, 3, true);
-        else TERNA_FUSED_M(16, 3, false);
+    if (mode == FUSED_GLU) {
+        // long K (the down projection): only the single-row variant, whose per-lane state is tiny
+        if (M != 1 || !wide || ktiles > 16 * 7) return 0;
+        TERNA_FUSED(16, 7, FUSED_GLU, 1);
+    } else if (wide) {
+        if (ktiles > 16 * 3) return 0;
+        if (mode == FUSED_RESIDUAL) TERNA_FUSED_M(16, 3, FUSED_RESIDUAL);
+        else TERNA_FUSED_M(16, 3, FUSED_PLAIN);
     } else {
-        if (residual) TERNA_FUSED_M(8, 5, true);
-        else TERNA_FUSED_M(8, 5, false);
+        if (ktiles > 8 * 5) return 0;
+        if (mode == FUSED_RESIDUAL) TERNA_FUSED_M(8, 5, FUSED_RESIDUAL);
+        else TERNA_FUSED_M(8, 5, FUSED_PLAIN);
     }
 #undef TERNA_FUSED_M
 #undef TERNA_FUSED
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("bitlinear_TernaSpMM_packed_fused", e, __LINE__);
     return 1;
+}
+
+int bitlinear_TernaSpMM_packed_fused(const terna_bf16* x, const terna_bf16* residual, terna_bf16* sum_out,
+                                     const terna_bf16* norm_weight, float eps, const void* packed, terna_bf16* out,
+                                     const terna_bf16* ws, int ws_num, int8_t* xq_out, terna_bf16* s_out, int M,
+                                     int N, int K, terna_stream stream)
+{
+    return launch_decode_fused(residual ? FUSED_RESIDUAL : FUSED_PLAIN, x, residual, sum_out, norm_weight, eps, packed, out,
+                               ws, ws_num, xq_out, s_out, M, N, K, static_cast<hipStream_t>(stream));
+}
+
+int bitlinear_TernaSpMM_packed_fused_glu(const terna_bf16* x13, const terna_bf16* norm_weight, float eps,
+                                         const void* packed, terna_bf16* out, const terna_bf16* ws, int ws_num,
+                                         int8_t* xq_out, terna_bf16* s_out, int M, int N, int F, terna_stream stream)
+{
+    return launch_decode_fused(FUSED_GLU, x13, nullptr, nullptr, norm_weight, eps, packed, out, ws, ws_num, xq_out, s_out,
+                               M, N, F, static_cast<hipStream_t>(stream));
 }
 
 void ternaspmm_rope_kv_store(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,

@@ -171,6 +171,22 @@ def rmsnorm_linear_packed(x, norm_weight, eps, packed, ws, ws_num, out_features,
     return TernaInfer_linear_packed(xq, packed, s, ws, ws_num, out_features), h
 
 
+def relu2_mul_rmsnorm_linear_packed(x13, norm_weight, eps, packed, ws, ws_num, out_features):
+    """squared_relu(x1) * x3 -> RMSNorm -> quant_input -> int8 TernaSpMM on a P2 weight: one launch for a single
+    row where the library supports the shape, else relu2_mul_rmsnorm_quant + TernaInfer_linear_packed.
+    x13: bf16 [M, 2F].  Returns out bf16 [M, out_features]."""
+    m, f2 = x13.shape
+    x13 = x13.contiguous()
+    lib = _lib.load()
+    out = torch.empty((m, out_features), dtype=torch.bfloat16, device=x13.device)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    if m == 1 and lib.bitlinear_TernaSpMM_packed_fused_glu(_p(x13), _p(norm_weight), float(eps), _p(packed), _p(out), _p(ws),
+                                                         ws_num, None, None, m, out_features, f2 // 2, stream):
+        return out
+    xq, s = relu2_mul_rmsnorm_quant(x13, norm_weight, eps)
+    return TernaInfer_linear_packed(xq, packed, s, ws, ws_num, out_features)
+
+
 def relu2_mul_rmsnorm_quant(x13, weight, eps, quant=True):
     """Fused squared_relu(x1) * x3 -> ffn_sub_norm -> [quant_input] (model.py:279-281 + 120-123).
     x13: bf16 [M, 2F].  Returns (xq int8 [M, F], s bf16 [M]) when quant else y bf16 [M, F]."""

@@ -21,7 +21,8 @@ import torch
 from torch.nn import functional as F
 
 from . import _lib
-from .linear import relu2_mul_rmsnorm_quant, rmsnorm_linear_packed, rmsnorm_quant
+from .linear import (relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant, rmsnorm_linear_packed,
+                     rmsnorm_quant)
 
 
 @dataclass
@@ -139,6 +140,8 @@ class Block:
             return lin(rms_norm(h, weight, eps)), h
         if glu:
             if self.act == "int8":
+                if x.shape[0] == 1:
+                    return relu2_mul_rmsnorm_linear_packed(x, weight, eps, lin.packed, lin.ws, lin.ws_num, lin.n), None
                 return lin.quantised(*relu2_mul_rmsnorm_quant(x, weight, eps)), None
             return lin.dense(relu2_mul_rmsnorm_quant(x, weight, eps, quant=False)), None
         if self.act == "int8":

@@ -263,3 +263,34 @@ def test_rmsnorm_linear_wrapper_matches_two_launch_sequence(lib):
         assert torch.equal(h, h2)
         err = (out.float() - out2.float()).abs().max().item()
         assert err <= 2e-2 * out2.float().abs().max().item()
+
+
+@pytest.mark.parametrize("n,f,ws_num", [(2560, 6912, 1), (256, 192, 2), (320, 7168, 1)])
+def test_fused_gate_prologue_linear(lib, n, f, ws_num):
+    """Single row: squared_relu(x1) * x3 -> norm -> quantise -> matmul in one launch; same bars as above."""
+    from tests._util import DeviceFormat, make_ternary
+    w = make_ternary(n, f, 0.40, 870 + n)
+    fmt = DeviceFormat(w)
+    packed = torch.empty(n * f // 16, dtype=torch.int32, device="cuda")
+    lib.ternaspmm_repack(_vp(fmt.bm), _vp(fmt.off), _vp(fmt.med), _vp(fmt.vals), _vp(packed), n, f, None)
+    x13 = make_bf16_activations(1, 2 * f, 871 + f, outlier_frac=0.01)
+    g = _weight(f, 872)
+    ws = O.f32_to_bf16_bits(np.array([1.25, 0.75, 0.0, 0.0], np.float32))
+    xd, gd, wsd = _dev(x13), _dev(g), _dev(ws)
+    od = torch.zeros((1, n), dtype=torch.int16, device="cuda")
+    qd = torch.zeros((1, f), dtype=torch.int8, device="cuda")
+    sd = torch.zeros(1, dtype=torch.int16, device="cuda")
+    print(f"[case] fused gate prologue linear n={n} f={f}", flush=True)
+    assert lib.bitlinear_TernaSpMM_packed_fused_glu(_vp(xd), _vp(gd), 1e-5, _vp(packed), _vp(od), _vp(wsd), ws_num, _vp(qd),
+                                                    _vp(sd), 1, n, f, None) == 1
+    torch.cuda.synchronize()
+    q, s = qd.cpu().numpy(), sd.cpu().numpy().view(np.uint16)
+    y64 = O.rmsnorm(O.relu2_mul(x13), g, 1e-5)
+    _, s_want = O.quant_input(y64)
+    assert np.abs(_bf16_key(s) - _bf16_key(s_want)).max() <= 1
+    q_ref = np.clip(np.rint(O.bf16_bits_to_f32(y64) * O.bf16_bits_to_f32(s)[:, None]), -128, 127)
+    dq = np.abs(q.astype(np.int32) - q_ref.astype(np.int32))
+    assert dq.max() <= 1 and (dq != 0).mean() < 0.02
+    assert (od.cpu().numpy().view(np.uint16) == O.spmm_i8(q, w, s, ws, ws_num, 0)).all()
+    z = torch.zeros(64, dtype=torch.int32, device="cuda")
+    assert lib.bitlinear_TernaSpMM_packed_fused_glu(_vp(z), _vp(z), 1e-5, _vp(z), _vp(z), _vp(z), 1, None, None, 2, n, f, None) == 0
