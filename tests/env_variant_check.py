@@ -1,0 +1,35 @@
+"""Run under pytest by tests/test_gpu_parity.py::test_tile_and_path_overrides in a child process whose
+environment pins one of the library's tuning overrides (they are read once per process): large-M
+parity of both families on shapes with ragged M, N tails and odd / even tile counts."""
+import sys
+
+import numpy as np
+import torch
+
+from oracle import terna_oracle as O
+from tests._util import DeviceFormat, make_bf16_activations, make_int8_activations, make_ternary
+from tests.test_gpu_parity import WS, _check_bf16, repack, run_bf16_packed, run_i8_packed
+from ternainfer_amd import _lib
+
+
+def main() -> int:
+    lib = _lib.load()
+    co = O.COracle()
+    for m, n, k in [(100, 320, 192), (300, 512, 320), (65, 256, 64), (256, 3840, 128)]:
+        w = make_ternary(n, k, 0.40, 900 + m + n)
+        packed = repack(lib, DeviceFormat(w))
+        xq, s = make_int8_activations(m, k, 901 + m)
+        print(f"[case] override check m={m} n={n} k={k}", flush=True)
+        if not (run_i8_packed(lib, packed, n, xq, s, WS, 1, 1) == O.spmm_i8(xq, w, s, WS, 1, 1)).all():
+            print("int8 mismatch", m, n, k)
+            return 1
+        x = make_bf16_activations(m, k, 902 + m, outlier_frac=0.01)
+        scale = np.array([0.7], np.float32)
+        _check_bf16(run_bf16_packed(lib, packed, n, x, scale, 1, 1), co.spmm_bf16(x, w, scale, 1))
+    torch.cuda.synchronize()
+    print("override check ok")
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

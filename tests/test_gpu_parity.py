@@ -507,3 +507,21 @@ def test_kernel_binary_reference_command_line():
     print(r.stdout)
     assert r.returncode == 0, r.stdout + r.stderr
     assert r.stdout.count("TotalError: 0.00") == 4
+
+
+@pytest.mark.parametrize("env", [{"TERNASPMM_PREFILL_DMA": "0"},
+                                 {"TERNASPMM_PREFILL_DMA": "0", "TERNASPMM_PREFILL_BM": "128"},
+                                 {"TERNASPMM_PREFILL_BM": "128", "TERNASPMM_PREFILL_BN": "256"},
+                                 {"TERNASPMM_PREFILL_BM": "128", "TERNASPMM_PREFILL_BN": "128"},
+                                 {"TERNASPMM_PREFILL_BN": "256"}, {"TERNASPMM_PREFILL_BN": "128"},
+                                 {"TERNASPMM_DECODE_WAVES": "8"}, {"TERNASPMM_DECODE_WAVES": "16"}])
+def test_tile_and_path_overrides(env):
+    """Every large-M tile shape and the register-staged path behind the library's tuning overrides
+    (read once per process, hence a child process): tests/env_variant_check.py must pass under each."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    print(f"[case] override {env}", flush=True)
+    r = subprocess.run([sys.executable, "-u", "-m", "tests.env_variant_check"], cwd=root, env={**os.environ, **env},
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "override check ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
