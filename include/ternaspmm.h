@@ -204,6 +204,15 @@ void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, 
                                 const long long* pos, terna_bf16* out, int B, int H, int KV, int D, int S,
                                 float scale, terna_stream stream);
 
+/* Opt-in repack cache for unmodified call sites: with TERNASPMM_REPACK_CACHE=1 in the environment the
+ * reference-format entry points above (bitlinear_TernaSpMM*, bitlinear_TernaSpMM_bf16*) keep a device-side P2
+ * copy (N*K/4 bytes) of every weight they have seen -- keyed by device, the bitmap / sign / offset pointers and
+ * the shape -- and run the P2 kernels from the second sight on; the first sight allocates, repacks and waits
+ * (during stream capture, where nothing may be allocated, it runs the reference-format kernels instead).  The
+ * cache trusts the pointers: after freeing or rewriting weight tensors call this function, which releases every
+ * cached copy. */
+void ternaspmm_repack_cache_clear(void);
+
 /* Library version string, e.g. "ternaspmm-gfx950 0.1". */
 const char* ternaspmm_version(void);
 

@@ -46,6 +46,7 @@ PROTOTYPES = {
                                              ctypes.c_int),
     "ternaspmm_rope_kv_store": ([_vp] * 7 + [_ci] * 6 + [_vp], None),
     "ternaspmm_decode_attention": ([_vp] * 5 + [_ci] * 5 + [ctypes.c_float, _vp], None),
+    "ternaspmm_repack_cache_clear": ([], None),
     "ternaspmm_version": ([], ctypes.c_char_p),
 }
 

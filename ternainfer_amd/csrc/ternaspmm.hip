@@ -4,6 +4,8 @@
 
 #include <cstdio>
 #include <cstdlib>
+#include <mutex>
+#include <unordered_map>
 
 #include "../../include/ternaspmm.h"
 #include "decode_kernel.h"
@@ -245,6 +247,64 @@ void launch_large_m(const Act* x, const Weights& w, uint16_t* out, const Epilogu
 
 enum Route { ROUTE_AUTO, ROUTE_DECODE, ROUTE_PREFILL };
 
+// ---- opt-in repack cache behind the reference-format entry points (TERNASPMM_REPACK_CACHE=1).
+// An unmodified call site keeps passing the four format tensors; the first call that sees a weight
+// (identified by device, pointers and shape) allocates N*K/4 bytes, repacks into them and waits for
+// the repack; every later call runs the P2 kernels.  The cache trusts the pointers: a caller that
+// frees or rewrites weights must call ternaspmm_repack_cache_clear().  A first sight during stream
+// capture (where nothing may be allocated) is served by the reference-format kernels instead.
+struct RepackKey {
+    int device;
+    const void* bitmap;
+    const void* signs;
+    const void* offsets;
+    int n, k;
+    bool operator==(const RepackKey& o) const
+    {
+        return device == o.device && bitmap == o.bitmap && signs == o.signs && offsets == o.offsets && n == o.n && k == o.k;
+    }
+};
+struct RepackKeyHash {
+    size_t operator()(const RepackKey& key) const
+    {
+        size_t h = std::hash<const void*>()(key.bitmap);
+        h = h * 1000003u ^ std::hash<const void*>()(key.signs);
+        h = h * 1000003u ^ std::hash<const void*>()(key.offsets);
+        return h * 1000003u ^ (static_cast<size_t>(key.n) << 20) ^ static_cast<size_t>(key.k) ^ (static_cast<size_t>(key.device) << 40);
+    }
+};
+std::mutex g_repack_mutex;
+std::unordered_map<RepackKey, void*, RepackKeyHash> g_repack_cache;
+
+const uint32_t* cached_packed(const Weights& w, int N, int K, hipStream_t st)
+{
+    static const bool on = [] {
+        const char* v = std::getenv("TERNASPMM_REPACK_CACHE");
+        return v && std::atoi(v) != 0;
+    }();
+    if (!on) return nullptr;
+    RepackKey key{0, w.bitmap, w.sign_words, w.tile_off, N, K};
+    if (hipGetDevice(&key.device) != hipSuccess) return nullptr;
+    std::lock_guard<std::mutex> lock(g_repack_mutex);
+    const auto it = g_repack_cache.find(key);
+    if (it != g_repack_cache.end()) return static_cast<const uint32_t*>(it->second);
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    void* buf = nullptr;
+    if (hipMalloc(&buf, static_cast<size_t>(N) * K / 4) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    launch_repack(w, static_cast<uint32_t*>(buf), N, K, st);
+    const hipError_t e = hipStreamSynchronize(st);       // later calls may come on other streams
+    if (e != hipSuccess) die("repack cache", e, __LINE__);
+    g_repack_cache.emplace(key, buf);
+    return static_cast<const uint32_t*>(buf);
+}
+
 void run_i8(Route route, int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* median_off, uint32_t* sign_words,
             uint16_t* out, uint16_t* s, uint16_t* ws, int ws_num, int M, int N, int K, void* workspace,
             hipStream_t st, int line)
@@ -255,7 +315,10 @@ void run_i8(Route route, int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* m
     const bool decode_rule = route == ROUTE_DECODE || (route == ROUTE_AUTO && M <= 64);
     const Epilogue ep{s, ws, nullptr, ws_num, decode_rule ? EP_I8_DECODE : EP_I8_PREFILL};
     const Weights w{bitmap, tile_off, median_off, sign_words};
-    if (M <= 64) launch_decode<int8_t>(x, w, out, ep, M, N, K, st);
+    if (const uint32_t* p2 = cached_packed(w, N, K, st)) {
+        if (M <= 64) launch_decode_packed<int8_t>(x, p2, out, ep, M, N, K, st);
+        else launch_prefill_packed<int8_t>(x, p2, out, ep, M, N, K, st);
+    } else if (M <= 64) launch_decode<int8_t>(x, w, out, ep, M, N, K, st);
     else launch_large_m<int8_t>(x, w, out, ep, M, N, K, workspace, st);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("bitlinear_TernaSpMM", e, line);
@@ -269,7 +332,10 @@ void run_bf16(Route route, const uint16_t* x, const uint64_t* bitmap, const int*
     const Epilogue ep{nullptr, nullptr, scale, ws_num, EP_BF16};
     const Weights w{bitmap, tile_off, median_off, sign_words};
     const bool small = route == ROUTE_DECODE || (route == ROUTE_AUTO && M <= 64);
-    if (small) launch_decode<uint16_t>(x, w, out, ep, M, N, K, st);
+    if (const uint32_t* p2 = cached_packed(w, N, K, st)) {
+        if (small) launch_decode_packed<uint16_t>(x, p2, out, ep, M, N, K, st);
+        else launch_prefill_packed<uint16_t>(x, p2, out, ep, M, N, K, st);
+    } else if (small) launch_decode<uint16_t>(x, w, out, ep, M, N, K, st);
     else launch_large_m<uint16_t>(x, w, out, ep, M, N, K, workspace, st);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("bitlinear_TernaSpMM_bf16", e, line);
@@ -593,6 +659,13 @@ void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, 
         terna_decode_attention_kernel<64><<<dim3(B * H), dim3(256), lds, st>>>(q, cache_k, cache_v, pos, out, H, KV, S, scale);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_decode_attention", e, __LINE__);
+}
+
+void ternaspmm_repack_cache_clear(void)
+{
+    std::lock_guard<std::mutex> lock(g_repack_mutex);
+    for (auto& kv : g_repack_cache) (void)hipFree(kv.second);
+    g_repack_cache.clear();
 }
 
 const char* ternaspmm_version(void) { return "ternaspmm-gfx950 0.1"; }

@@ -1,0 +1,72 @@
+"""Run by tests/test_gpu_parity.py::test_repack_cache_behind_reference_entry_points in a child process with
+TERNASPMM_REPACK_CACHE=1: the reference-format entry points must give the same results as without the
+cache, on first sight (allocate + repack), on later sights (P2 kernels), under graph capture, and after
+ternaspmm_repack_cache_clear() when a different weight reuses the same device memory."""
+import ctypes
+import sys
+
+import numpy as np
+import torch
+
+from oracle import terna_oracle as O
+from tests._util import DeviceFormat, make_bf16_activations, make_int8_activations, make_ternary, vp
+from tests.test_gpu_parity import WS, _check_bf16, run_bf16, run_i8
+from ternainfer_amd import _lib
+
+
+def main() -> int:
+    lib = _lib.load()
+    co = O.COracle()
+    n, k = 320, 192
+    weights = [make_ternary(n, k, 0.40, seed) for seed in (950, 951)]
+    sources = [DeviceFormat(w) for w in weights]
+    fmt = sources[0]                             # its device buffers are reused for the second weight
+    shared_vals = torch.zeros(max(f.vals.numel() for f in sources), dtype=fmt.vals.dtype, device="cuda")
+    fmt_vals0 = sources[0].vals.clone()
+    fmt.vals = shared_vals
+    for round_no, w in enumerate(weights):
+        src_vals = fmt_vals0 if round_no == 0 else sources[1].vals
+        fmt.vals.zero_()
+        fmt.vals[: src_vals.numel()].copy_(src_vals)
+        if round_no == 1:                        # same device pointers, new contents: the stale-pointer case
+            fmt.bm.copy_(sources[1].bm); fmt.off.copy_(sources[1].off); fmt.med.copy_(sources[1].med)
+            lib.ternaspmm_repack_cache_clear()
+        torch.cuda.synchronize()
+        for m in (8, 8, 100, 100):               # first sight, cached sight, both kernel families
+            print(f"[case] repack cache weight {round_no} m={m}", flush=True)
+            xq, s = make_int8_activations(m, k, 960 + m)
+            mode = 0 if m <= 64 else 1
+            if not (run_i8(lib, fmt, xq, s, WS, 2) == O.spmm_i8(xq, w, s, WS, 2, mode)).all():
+                print("int8 mismatch", round_no, m)
+                return 1
+            x = make_bf16_activations(m, k, 961 + m)
+            scale = np.array([0.7, 1.9], np.float32)
+            _check_bf16(run_bf16(lib, fmt, x, scale, 2), co.spmm_bf16(x, w, scale, 2))
+    # a weight first seen during capture: served without allocating, replays stay correct
+    w = make_ternary(256, 128, 0.40, 970)
+    f2 = DeviceFormat(w)
+    xq, s = make_int8_activations(8, 128, 971)
+    xd = torch.from_numpy(xq).cuda(); sd = torch.from_numpy(s.view(np.int16)).cuda()
+    wsd = torch.from_numpy(WS.view(np.int16)).cuda()
+    out = torch.zeros((8, 256), dtype=torch.int16, device="cuda")
+    work = torch.empty(256 * 128, dtype=torch.int8, device="cuda")
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            lib.bitlinear_TernaSpMM(vp(xd), vp(f2.bm), vp(f2.off), vp(f2.med), vp(f2.vals), vp(out), vp(sd), vp(wsd), 1,
+                                    8, 256, 128, 1, vp(work), ctypes.c_void_p(side.cuda_stream))
+    for _ in range(2):
+        out.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        if not (out.cpu().numpy().view(np.uint16) == O.spmm_i8(xq, w, s, WS, 1, 0)).all():
+            print("graph replay mismatch")
+            return 1
+    lib.ternaspmm_repack_cache_clear()
+    print("repack cache check ok")
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

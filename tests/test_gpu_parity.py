@@ -525,3 +525,13 @@ def test_tile_and_path_overrides(env):
     r = subprocess.run([sys.executable, "-u", "-m", "tests.env_variant_check"], cwd=root, env={**os.environ, **env},
                        capture_output=True, text=True, timeout=300)
     assert r.returncode == 0 and "override check ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+
+
+def test_repack_cache_behind_reference_entry_points():
+    """TERNASPMM_REPACK_CACHE=1 (read once per process, hence a child process): tests/repack_cache_check.py."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-u", "-m", "tests.repack_cache_check"], cwd=root,
+                       env={**os.environ, "TERNASPMM_REPACK_CACHE": "1"}, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "repack cache check ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
