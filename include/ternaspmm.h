@@ -203,6 +203,12 @@ void ternaspmm_rope_kv_store(const terna_bf16* qkv, const float* cos, const floa
 void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
                                 const long long* pos, terna_bf16* out, int B, int H, int KV, int D, int S,
                                 float scale, terna_stream stream);
+/* Both of the above in one launch for T = 1: qkv bf16 [B][(H + 2*KV)*D], cos / sin fp32 [D/2] of the new
+ * token's position; writes slot pos[0] of the caches and out.  Results are bit-identical to
+ * ternaspmm_rope_kv_store followed by ternaspmm_decode_attention. */
+void ternaspmm_rope_decode_attention(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
+                                     terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
+                                     int D, int S, float scale, terna_stream stream);
 
 /* Opt-in repack cache for unmodified call sites: with TERNASPMM_REPACK_CACHE=1 in the environment the
  * reference-format entry points above (bitlinear_TernaSpMM*, bitlinear_TernaSpMM_bf16*) keep a device-side P2

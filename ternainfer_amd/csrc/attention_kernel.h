@@ -90,9 +90,16 @@ __global__ __launch_bounds__(256) void terna_rope_kv_store_kernel(
 //   pass 2  softmax over the scores in LDS
 //   pass 3  thread (slice, chunk): slots slice, slice+S', ... x 8 dimensions of V, eight rows in
 //           flight per thread; the slices are summed through LDS
-template <int D>
+//
+// ROPE = true folds terna_rope_kv_store_kernel (one token per sequence) into the same launch: `q` is
+// then the fused qkv row of the new token (bf16 [B][(H + 2*KV)*D]); every workgroup rotates its own
+// q head and the new key row of its kv head in registers (same arithmetic, bit for bit), uses them
+// -- and the new value row -- in place of cache slot pos[0], and the first workgroup of each kv
+// group writes the new key / value rows into the cache for the steps to come.
+template <int D, bool ROPE>
 __global__ __launch_bounds__(256) void terna_decode_attention_kernel(
-    const uint16_t* __restrict__ q, const uint16_t* __restrict__ cache_k, const uint16_t* __restrict__ cache_v,
+    const uint16_t* __restrict__ q, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
+    const float* __restrict__ cosv, const float* __restrict__ sinv,
     const long long* __restrict__ pos, uint16_t* __restrict__ out, int H, int KV, int S, float scale)
 {
     static_assert(D == 64 || D == 128, "head dimension");
@@ -137,12 +144,70 @@ __global__ __launch_bounds__(256) void terna_decode_attention_kernel(
         const int sv = slice + u * SLICES;
         vr[u] = *reinterpret_cast<const u32x4*>(vbase + static_cast<size_t>(sv < S ? sv : 0) * D + chunk * 8);
     }
+    u32x4 knew[NJ], vnew;                        // ROPE: the new token's key chunks of this lane, value chunk of this thread
+    if constexpr (!ROPE) {
 #pragma unroll
-    for (int jj = 0; jj < NJ; ++jj)
-        qr[jj] = *reinterpret_cast<const u32x4*>(q + (static_cast<size_t>(b) * H + h) * D + 32 * jj + 8 * kblk);
+        for (int jj = 0; jj < NJ; ++jj)
+            qr[jj] = *reinterpret_cast<const u32x4*>(q + (static_cast<size_t>(b) * H + h) * D + 32 * jj + 8 * kblk);
+    } else {
+        // chunk c = 4jj + kblk (dimensions 8c .. 8c+7) and its rotation partner c +- CH/2
+        const uint16_t* row = q + static_cast<size_t>(b) * (H + 2 * KV) * D;
+        u32x4 q_own[NJ], q_par[NJ], k_own[NJ], k_par[NJ];
+        f32x4 cs[NJ][2], sn[NJ][2];
+#pragma unroll
+        for (int jj = 0; jj < NJ; ++jj) {
+            const int c = 4 * jj + kblk, cp = (c + CH / 2) % CH, ca = c % (CH / 2);
+            q_own[jj] = *reinterpret_cast<const u32x4*>(row + h * D + 8 * c);
+            q_par[jj] = *reinterpret_cast<const u32x4*>(row + h * D + 8 * cp);
+            k_own[jj] = *reinterpret_cast<const u32x4*>(row + (H + kvh) * D + 8 * c);
+            k_par[jj] = *reinterpret_cast<const u32x4*>(row + (H + kvh) * D + 8 * cp);
+            cs[jj][0] = *reinterpret_cast<const f32x4*>(cosv + 8 * ca);
+            cs[jj][1] = *reinterpret_cast<const f32x4*>(cosv + 8 * ca + 4);
+            sn[jj][0] = *reinterpret_cast<const f32x4*>(sinv + 8 * ca);
+            sn[jj][1] = *reinterpret_cast<const f32x4*>(sinv + 8 * ca + 4);
+        }
+        vnew = *reinterpret_cast<const u32x4*>(row + (H + KV + kvh) * D + 8 * chunk);
+        auto rotate = [&](const u32x4& own, const u32x4& par, int jj, bool first_half) {
+            float a[8], p[8], o[8];
+            unpack_bf16x8(own, a);
+            unpack_bf16x8(par, p);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+#pragma clang fp contract(off)                   // as terna_rope_kv_store_kernel: every product and sum rounded once
+                const float c = cs[jj][e >> 2][e & 3], sv = sn[jj][e >> 2][e & 3];
+                const float lo = a[e] * c - p[e] * sv;     // own chunk in the first half:  x1 c - x2 s
+                const float hi = a[e] * c + p[e] * sv;     // own chunk in the second half: x2 c + x1 s
+                o[e] = first_half ? lo : hi;
+            }
+            return pack_bf16x8(o);
+        };
+#pragma unroll
+        for (int jj = 0; jj < NJ; ++jj) {
+            const bool first_half = 4 * jj + kblk < CH / 2;
+            qr[jj] = rotate(q_own[jj], q_par[jj], jj, first_half);
+            knew[jj] = rotate(k_own[jj], k_par[jj], jj, first_half);
+        }
+        if (h % (H / KV) == 0) {                 // this kv group's writer: slot pos[0] of both caches
+            const size_t slot_off = ((static_cast<size_t>(b) * KV + kvh) * S + (n - 1)) * D;
+            if (wave == 0 && r16 == 0) {
+#pragma unroll
+                for (int jj = 0; jj < NJ; ++jj) *reinterpret_cast<u32x4*>(cache_k + slot_off + 8 * (4 * jj + kblk)) = knew[jj];
+            }
+            if (tid < CH) *reinterpret_cast<u32x4*>(cache_v + slot_off + 8 * chunk) = vnew;
+        }
+    }
 
     float mx = -INFINITY;
-    auto score_tile = [&](int tile, const u32x4 (&k)[NJ]) {
+    auto score_tile = [&](int tile, const u32x4 (&kin)[NJ]) {
+        u32x4 k[NJ];
+#pragma unroll
+        for (int jj = 0; jj < NJ; ++jj) k[jj] = kin[jj];
+        if constexpr (ROPE) {
+            if (16 * tile + r16 == n - 1) {      // the new token's slot: its key row is in registers, not in the cache yet
+#pragma unroll
+                for (int jj = 0; jj < NJ; ++jj) k[jj] = knew[jj];
+            }
+        }
         f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int jj = 0; jj < NJ; ++jj)
@@ -201,6 +266,9 @@ __global__ __launch_bounds__(256) void terna_decode_attention_kernel(
             }
             p[u] = s < n ? score[s] : 0.0f;
             if (!(s < n)) vr[u] = u32x4{0u, 0u, 0u, 0u};     // never multiply stale cache contents (could be NaN)
+            if constexpr (ROPE) {
+                if (s == n - 1) vr[u] = vnew;
+            }
         }
 #pragma unroll
         for (int u = 0; u < VU; ++u) {

@@ -653,12 +653,32 @@ void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, 
     }
     const size_t lds = (static_cast<size_t>(S) + (256 / (D / 8)) * D) * sizeof(float);
     hipStream_t st = static_cast<hipStream_t>(stream);
+    uint16_t* ck = const_cast<uint16_t*>(cache_k);      // the kernel writes the caches only in its ROPE variant
+    uint16_t* cv = const_cast<uint16_t*>(cache_v);
     if (D == 128)
-        terna_decode_attention_kernel<128><<<dim3(B * H), dim3(256), lds, st>>>(q, cache_k, cache_v, pos, out, H, KV, S, scale);
+        terna_decode_attention_kernel<128, false><<<dim3(B * H), dim3(256), lds, st>>>(q, ck, cv, nullptr, nullptr, pos, out, H, KV, S, scale);
     else
-        terna_decode_attention_kernel<64><<<dim3(B * H), dim3(256), lds, st>>>(q, cache_k, cache_v, pos, out, H, KV, S, scale);
+        terna_decode_attention_kernel<64, false><<<dim3(B * H), dim3(256), lds, st>>>(q, ck, cv, nullptr, nullptr, pos, out, H, KV, S, scale);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_decode_attention", e, __LINE__);
+}
+
+void ternaspmm_rope_decode_attention(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
+                                     terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
+                                     int D, int S, float scale, terna_stream stream)
+{
+    if (B < 1 || H < 1 || KV < 1 || H % KV != 0 || (D != 64 && D != 128) || S < 1 || S > 8192) {
+        std::fprintf(stderr, "ternaspmm_rope_decode_attention: unsupported arguments (H=%d KV=%d D=%d S=%d)\n", H, KV, D, S);
+        return;
+    }
+    const size_t lds = (static_cast<size_t>(S) + (256 / (D / 8)) * D) * sizeof(float);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (D == 128)
+        terna_decode_attention_kernel<128, true><<<dim3(B * H), dim3(256), lds, st>>>(qkv, cache_k, cache_v, cos, sin, pos, out, H, KV, S, scale);
+    else
+        terna_decode_attention_kernel<64, true><<<dim3(B * H), dim3(256), lds, st>>>(qkv, cache_k, cache_v, cos, sin, pos, out, H, KV, S, scale);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_rope_decode_attention", e, __LINE__);
 }
 
 void ternaspmm_repack_cache_clear(void)

@@ -162,7 +162,15 @@ class Block:
         t = x.shape[0] // bsz
         qkv, x = self._norm_linear(self.wqkv, x, self.attention_norm, residual=pending)
         rep = a.n_heads // a.n_kv_heads
-        if self.fused:
+        one_token = self.fused and t == 1 and a.head_dim in (64, 128) and cache_k.shape[2] <= 8192
+        if one_token:                       # RoPE, cache write and attention over the cache prefix: one launch
+            lib = self.wqkv.lib
+            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            o = torch.empty((bsz, a.n_heads * a.head_dim), dtype=torch.bfloat16, device=x.device)
+            lib.ternaspmm_rope_decode_attention(_p(qkv), _p(cos), _p(sin), _p(pos_idx), _p(cache_k), _p(cache_v), _p(o),
+                                                bsz, a.n_heads, a.n_kv_heads, a.head_dim, cache_k.shape[2],
+                                                a.head_dim ** -0.5, stream)
+        elif self.fused:
             lib = self.wqkv.lib
             stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
             q = torch.empty((bsz, a.n_heads, t, a.head_dim), dtype=torch.bfloat16, device=x.device)
@@ -174,11 +182,7 @@ class Block:
             q, k = apply_rope(q, cos[None, None], sin[None, None]), apply_rope(k, cos[None, None], sin[None, None])
             cache_k.index_copy_(2, pos_idx, k)
             cache_v.index_copy_(2, pos_idx, v)
-        if self.fused and t == 1 and a.head_dim in (64, 128) and cache_k.shape[2] <= 8192:
-            o = torch.empty((bsz, a.n_heads * a.head_dim), dtype=torch.bfloat16, device=x.device)
-            lib.ternaspmm_decode_attention(_p(q), _p(cache_k), _p(cache_v), _p(pos_idx), _p(o), bsz, a.n_heads,
-                                           a.n_kv_heads, a.head_dim, cache_k.shape[2], a.head_dim ** -0.5, stream)
-        else:
+        if not one_token:
             kk = cache_k.repeat_interleave(rep, dim=1)
             vv = cache_v.repeat_interleave(rep, dim=1)
             o = F.scaled_dot_product_attention(q, kk, vv, attn_mask=mask)

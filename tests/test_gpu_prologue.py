@@ -294,3 +294,34 @@ def test_fused_gate_prologue_linear(lib, n, f, ws_num):
     assert (od.cpu().numpy().view(np.uint16) == O.spmm_i8(q, w, s, ws, ws_num, 0)).all()
     z = torch.zeros(64, dtype=torch.int32, device="cuda")
     assert lib.bitlinear_TernaSpMM_packed_fused_glu(_vp(z), _vp(z), 1e-5, _vp(z), _vp(z), _vp(z), 1, None, None, 2, n, f, None) == 0
+
+
+@pytest.mark.parametrize("b,h,kv,d,s_max,n", [(1, 20, 5, 128, 256, 1), (1, 20, 5, 128, 256, 160), (8, 20, 5, 128, 300, 290),
+                                              (2, 4, 2, 64, 40, 17), (1, 20, 5, 128, 600, 513)])
+def test_rope_decode_attention_equals_the_two_launches(lib, b, h, kv, d, s_max, n):
+    """One launch (RoPE + cache write + attention) against ternaspmm_rope_kv_store followed by
+    ternaspmm_decode_attention on the same inputs: outputs and both caches bit-identical."""
+    rng = np.random.default_rng(720 + n)
+    qkv = make_bf16_activations(b, (h + 2 * kv) * d, 721 + n)
+    k0 = make_bf16_activations(b * kv * s_max, d, 722 + n).reshape(b, kv, s_max, d)
+    v0 = make_bf16_activations(b * kv * s_max, d, 723 + n, outlier_frac=0.01).reshape(b, kv, s_max, d)
+    pos = np.array([n - 1], np.int64)
+    ang = (pos[:, None] * (1.0 / 500000.0 ** (np.arange(0, d, 2) / d))[None, :]).astype(np.float32)
+    cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    xd, cd, sd, pd = _dev(qkv), _dev(cos), _dev(sin), _dev(pos)
+    scale = float(d) ** -0.5
+    # two launches
+    ck1, cv1 = _dev(k0), _dev(v0)
+    q1 = torch.zeros((b, h, 1, d), dtype=torch.int16, device="cuda")
+    o1 = torch.zeros((b, h * d), dtype=torch.int16, device="cuda")
+    lib.ternaspmm_rope_kv_store(_vp(xd), _vp(cd), _vp(sd), _vp(pd), _vp(q1), _vp(ck1), _vp(cv1), b, 1, h, kv, d, s_max, None)
+    lib.ternaspmm_decode_attention(_vp(q1), _vp(ck1), _vp(cv1), _vp(pd), _vp(o1), b, h, kv, d, s_max, scale, None)
+    # one launch
+    ck2, cv2 = _dev(k0), _dev(v0)
+    o2 = torch.zeros((b, h * d), dtype=torch.int16, device="cuda")
+    print(f"[case] rope + decode attention b={b} h={h} kv={kv} d={d} S={s_max} n={n}", flush=True)
+    lib.ternaspmm_rope_decode_attention(_vp(xd), _vp(cd), _vp(sd), _vp(pd), _vp(ck2), _vp(cv2), _vp(o2), b, h, kv, d, s_max,
+                                        scale, None)
+    torch.cuda.synchronize()
+    assert torch.equal(ck1, ck2) and torch.equal(cv1, cv2)
+    assert torch.equal(o1, o2)
