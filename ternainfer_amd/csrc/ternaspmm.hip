@@ -61,13 +61,13 @@ void launch_decode_as(const Act* x, const Weights& w, uint16_t* out, const Epilo
 // (N/16 <= 256: at most one workgroup per CU) is bound by each wave's serial share of K, so it
 // gets 16 waves and a deeper prefetch ring; a matrix with many bands is bound by how many
 // workgroups fit on the chip at once, so it gets 8 waves and the leaner ring (<= 64 VGPRs).
-// TERNASPMM_DECODE_WAVES=8|16 forces one variant (tuning aid).
+// TERNASPMM_DECODE_WAVES=4|8|16 forces one variant (tuning aid).
 int decode_waves_override()
 {
     static const int waves = [] {
         const char* v = std::getenv("TERNASPMM_DECODE_WAVES");
         const int w = v ? std::atoi(v) : 0;
-        return (w == 8 || w == 16) ? w : 0;
+        return (w == 4 || w == 8 || w == 16) ? w : 0;
     }();
     return waves;
 }
@@ -140,7 +140,11 @@ void launch_decode_packed(const Act* x, const uint32_t* packed, uint16_t* out, c
     const int forced = decode_waves_override();
     const bool wide = forced ? forced == 16 : (N / 16 <= 256);
     if (M <= 16) {
-        if (wide) launch_decode_packed_as<Act, 16, 1, 3>(x, packed, out, ep, M, N, K, st);
+        // more than 512 bands (gate+up): per-wave set-up is as expensive as a few band-tiles, so fewer waves
+        // with more band-tiles each win (measured 7.4 against 8.2 us)
+        const bool narrow = forced ? forced == 4 : (N / 16 > 512);
+        if (narrow) launch_decode_packed_as<Act, 4, 1, 3>(x, packed, out, ep, M, N, K, st);
+        else if (wide) launch_decode_packed_as<Act, 16, 1, 3>(x, packed, out, ep, M, N, K, st);
         else launch_decode_packed_as<Act, 8, 1, 2>(x, packed, out, ep, M, N, K, st);
     } else if (M <= 32) {
         if (wide) launch_decode_packed_as<Act, 16, 2, 2>(x, packed, out, ep, M, N, K, st);

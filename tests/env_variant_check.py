@@ -26,6 +26,21 @@ def main() -> int:
         x = make_bf16_activations(m, k, 902 + m, outlier_frac=0.01)
         scale = np.array([0.7], np.float32)
         _check_bf16(run_bf16_packed(lib, packed, n, x, scale, 1, 1), co.spmm_bf16(x, w, scale, 1))
+    from tests.test_gpu_parity import run_bf16, run_i8
+    for m, n, k in [(8, 320, 192), (16, 256, 64), (1, 8256, 128)]:      # small-M kernels, both layouts
+        w = make_ternary(n, k, 0.40, 910 + m + n)
+        fmt = DeviceFormat(w)
+        packed = repack(lib, fmt)
+        xq, s = make_int8_activations(m, k, 911 + m)
+        x = make_bf16_activations(m, k, 912 + m)
+        scale = np.array([0.7], np.float32)
+        want = O.spmm_i8(xq, w, s, WS, 1, 0)
+        if not ((run_i8_packed(lib, packed, n, xq, s, WS, 1) == want).all() and (run_i8(lib, fmt, xq, s, WS, 1) == want).all()):
+            print("int8 small-M mismatch", m, n, k)
+            return 1
+        gold = co.spmm_bf16(x, w, scale, 1)
+        _check_bf16(run_bf16_packed(lib, packed, n, x, scale, 1), gold)
+        _check_bf16(run_bf16(lib, fmt, x, scale, 1), gold)
     torch.cuda.synchronize()
     print("override check ok")
     return 0
