@@ -110,6 +110,9 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
         const int j = wave + WAVES * t;
         nw[t].load(norm_w + (j < ktiles ? j : 0) * 64 + cl);
     }
+    // wave 0 finishes the band: its weight-group scales are requested now, converted at the very end
+    const Epilogue ep{nullptr, ws, nullptr, ws_num, EP_I8_DECODE};
+    EpilogueRaw eraw = load_epilogue_raw_scales(ep, band * 16 + 4 * g, N);
     // this wave's LDS slot: rows the batch does not have stay zero
     uint8_t* slab = slab_all[wave];
     for (int o = lane * 16; o < 16 * XQ::kPitch; o += 64 * 16) *reinterpret_cast<u32x4*>(slab + o) = u32x4{0u, 0u, 0u, 0u};
@@ -234,10 +237,8 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
         for (int w = 1; w < WAVES; ++w) sum += red[w][lane];
         if (i < M) {
             const int n0 = band * 16 + 4 * g;
-            const Epilogue ep{nullptr, ws, nullptr, ws_num, EP_I8_DECODE};
-            EpilogueRegs e;
+            EpilogueRegs e = finish_epilogue(ep, eraw);
             e.s = s_row[i];
-            load_col_scales(ep, n0, N, e.w);
             uint16_t o[4];
 #pragma unroll
             for (int v = 0; v < 4; ++v) o[v] = apply_epilogue<int>(EP_I8_DECODE, e, v, sum[v]);

@@ -235,11 +235,11 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
 
     // Wave w finishes m-block w (and w + WAVES, ...): fetch that block's scale factors now.
     const int n0 = band * 16 + 4 * g;
-    EpilogueRegs eregs[(MB + WAVES - 1) / WAVES];
+    EpilogueRaw eraw[(MB + WAVES - 1) / WAVES];
 #pragma unroll
     for (int e = 0; e < (MB + WAVES - 1) / WAVES; ++e) {
         const int m = m_base + (wave + e * WAVES) * 16 + i;
-        eregs[e] = load_epilogue(ep, m < M ? m : M - 1, n0, N);
+        eraw[e] = load_epilogue_raw(ep, m < M ? m : M - 1, n0, N);
     }
 
     // This wave's band-tiles: gk = wave, wave + WAVES, ...  (cnt of them)
@@ -392,9 +392,10 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
         for (int w = 1; w < WAVES; ++w) sum += red[w][mb][lane];
         const int m = m_base + mb * 16 + i;
         if (m < M) {
+            const EpilogueRegs eregs = finish_epilogue(ep, eraw[e]);
             uint16_t o[4];
 #pragma unroll
-            for (int v = 0; v < 4; ++v) o[v] = apply_epilogue<typename T::AccScalar>(ep.kind, eregs[e], v, sum[v]);
+            for (int v = 0; v < 4; ++v) o[v] = apply_epilogue<typename T::AccScalar>(ep.kind, eregs, v, sum[v]);
             const u32x2 packed = {o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16)};
             *reinterpret_cast<u32x2*>(out + static_cast<size_t>(m) * N + n0) = packed;
         }

@@ -124,11 +124,11 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
     // Wave w finishes m-block w (and w + WAVES, ...): with the data loads in flight, fetch that
     // block's scale factors so that no global load sits between the last MFMA and the store.
     const int n0 = band * 16 + 4 * g;
-    EpilogueRegs eregs[(MB + WAVES - 1) / WAVES];
+    EpilogueRaw eraw[(MB + WAVES - 1) / WAVES];
 #pragma unroll
     for (int e = 0; e < (MB + WAVES - 1) / WAVES; ++e) {
         const int m = m_base + (wave + e * WAVES) * 16 + i;
-        eregs[e] = load_epilogue(ep, m < M ? m : M - 1, n0, N);
+        eraw[e] = load_epilogue_raw(ep, m < M ? m : M - 1, n0, N);
     }
 
     for (int j0 = 0; j0 < cnt; j0 += NBUF) {
@@ -163,11 +163,12 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
         for (int w = 1; w < WAVES; ++w) sum += red[w][mb][lane];
         const int m = m_base + mb * 16 + i;
         if (m < M) {
+            const EpilogueRegs eregs = finish_epilogue(ep, eraw[e]);
             uint16_t o[4];
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-                if constexpr (sizeof(Act) == 2) o[v] = apply_epilogue<float>(ep.kind, eregs[e], v, sum[v] * 2.0f);
-                else o[v] = apply_epilogue<int>(ep.kind, eregs[e], v, sum[v]);
+                if constexpr (sizeof(Act) == 2) o[v] = apply_epilogue<float>(ep.kind, eregs, v, sum[v] * 2.0f);
+                else o[v] = apply_epilogue<int>(ep.kind, eregs, v, sum[v]);
             }
             const u32x2 pk = {o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16)};
             *reinterpret_cast<u32x2*>(out + static_cast<size_t>(m) * N + n0) = pk;

@@ -111,6 +111,71 @@ __device__ __forceinline__ EpilogueRegs load_epilogue(const Epilogue& ep, int m,
     return r;
 }
 
+// The same scale factors as they come out of memory -- bf16 storage (int8 family) or fp32 bits (bf16
+// family) -- with no arithmetic on them: a kernel that requests them ahead of its main loop must not
+// touch the values before the loop is over, or it waits for them (and for every load issued before
+// them) on the spot.  finish_epilogue() converts once the data is certainly there.
+struct EpilogueRaw {
+    uint32_t s;
+    uint32_t w[4];      // one scale per matrix: only w[0] is loaded
+};
+
+__device__ __forceinline__ EpilogueRaw load_epilogue_raw(const Epilogue& ep, int m, int n0, int N)
+{
+    EpilogueRaw r;
+    r.s = 0u;
+    r.w[0] = r.w[1] = r.w[2] = r.w[3] = 0u;
+    if (ep.kind == EP_BF16) {
+        if (ep.ws_num == 1) {
+            r.w[0] = __float_as_uint(ep.scale[0]);
+        } else {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) r.w[v] = __float_as_uint(ep.scale[ws_group_decode(n0 + v, N, ep.ws_num)]);
+        }
+    } else {
+        r.s = ep.s[m];
+        if (ep.ws_num == 1) {
+            r.w[0] = ep.ws[0];
+        } else {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int g = ep.kind == EP_I8_PREFILL ? ws_group_prefill(n0 + v, N, ep.ws_num)
+                                                       : ws_group_decode(n0 + v, N, ep.ws_num);
+                r.w[v] = ep.ws[g];
+            }
+        }
+    }
+    return r;
+}
+
+// Only the weight-group scales (the caller has the activation scale from elsewhere).
+__device__ __forceinline__ EpilogueRaw load_epilogue_raw_scales(const Epilogue& ep, int n0, int N)
+{
+    EpilogueRaw r;
+    r.s = 0u;
+    r.w[0] = r.w[1] = r.w[2] = r.w[3] = 0u;
+    if (ep.ws_num == 1) {
+        r.w[0] = ep.ws[0];
+    } else {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) r.w[v] = ep.ws[ws_group_decode(n0 + v, N, ep.ws_num)];
+    }
+    return r;
+}
+
+__device__ __forceinline__ EpilogueRegs finish_epilogue(const Epilogue& ep, const EpilogueRaw& r)
+{
+    EpilogueRegs e;
+    const bool f32 = ep.kind == EP_BF16;
+    e.s = f32 ? 1.0f : __uint_as_float(r.s << 16);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const uint32_t bits = r.w[ep.ws_num == 1 ? 0 : v];
+        e.w[v] = f32 ? __uint_as_float(bits) : __uint_as_float(bits << 16);
+    }
+    return e;
+}
+
 // One output element: integer or float accumulator -> bf16 storage.
 template <typename Acc>
 __device__ __forceinline__ uint16_t apply_epilogue(int kind, const EpilogueRegs& e, int v, Acc acc)
