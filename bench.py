@@ -191,11 +191,13 @@ def run_model(args, torch):
     print(json.dumps({
         "metric": "2B-shape decode tok/s", "value": tps, "unit": "tokens/s", "n_gpus": 1, "steps": 256, "warmup": 8,
         "ms_per_step": decode_s * 1e3 / 256, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
+        "dtype": args.act, "data": "synthetic",
         "config": {"workload": f"configs[4]: BitNet-b1.58-2B-shaped random-init decoder (30 layers, hidden 2560, 20/5 heads, "
                                f"FFN 6912, vocab 128256), batch {args.batch}, 128-token prompt, 256 greedy tokens, "
                                f"{args.act} activations into the ternary linears, weights in P2 layout, one HIP graph per "
-                               "decode step; attention / norms / RoPE / LM head are plain PyTorch ops",
+                               "decode step; norms, gate, activation quantisation, RoPE, cache write and "
+                               "single-token attention are library kernels, prefill attention and the bf16 LM head "
+                               "are PyTorch-ROCm ops",
                    "batch": args.batch, "act": args.act},
         "prefill_tokens_per_s": args.batch * 128 / prefill_s, "prefill_s": prefill_s, "decode_s": decode_s,
         "model_build_s": build_s, "first_tokens": toks[0, :8].tolist()}))
