@@ -535,3 +535,43 @@ def test_repack_cache_behind_reference_entry_points():
     r = subprocess.run([sys.executable, "-u", "-m", "tests.repack_cache_check"], cwd=root,
                        env={**os.environ, "TERNASPMM_REPACK_CACHE": "1"}, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0 and "repack cache check ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+
+
+def test_benchmark_entry_point_times_and_leaves_the_result(lib, capfd):
+    """bitlinear_TernaSpMM_benchmark(mode, warmup, iters, <the 15 arguments>) (kernels/TernaSpMM.cu:141-236):
+    runs the chosen path, prints one 'Shape(M=.., N=.., K=..): <t> us' line, and `out` holds the result."""
+    import re
+    n, k = 256, 192
+    w = make_ternary(n, k, 0.40, 980)
+    fmt = DeviceFormat(w)
+    for mode, m, ep_mode in [(0, 8, 0), (2, 8, 0), (1, 8, 1), (0, 100, 1), (2, 100, 0)]:
+        xq, s = make_int8_activations(m, k, 981 + m)
+        x, sd = torch.from_numpy(xq).cuda(), torch.from_numpy(s.view(np.int16)).cuda()
+        ws = torch.from_numpy(WS.view(np.int16)).cuda()
+        out = torch.full((m, n), -1, dtype=torch.int16, device="cuda")
+        work = _workspace(m, n, k)
+        print(f"[case] benchmark entry mode={mode} M={m}", flush=True)
+        capfd.readouterr()
+        lib.bitlinear_TernaSpMM_benchmark(mode, 2, 5, vp(x), vp(fmt.bm), vp(fmt.off), vp(fmt.med), vp(fmt.vals), vp(out),
+                                          vp(sd), vp(ws), 2, m, n, k, 7, vp(work), _stream())
+        torch.cuda.synchronize()
+        text = capfd.readouterr().out
+        match = re.search(r"Shape\(M=(\d+), N=(\d+), K=(\d+)\): ([0-9.]+) us", text)
+        assert match, text
+        assert (int(match.group(1)), int(match.group(2)), int(match.group(3))) == (m, n, k)
+        assert 0.0 < float(match.group(4)) < 1e4
+        assert (out.cpu().numpy().view(np.uint16) == O.spmm_i8(xq, w, s, WS, 2, ep_mode)).all()
+
+
+def test_gpu_sleep_and_error_check(lib):
+    """gpu_sleep(us, stream) (kernels/TernaSpMM.cu:454) occupies the stream for about that long;
+    checkLastCudaError(line) returns quietly when nothing went wrong."""
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    lib.gpu_sleep(ctypes.c_double(100.0), _stream())             # warm-up: code object load
+    torch.cuda.synchronize()
+    e0.record()
+    lib.gpu_sleep(ctypes.c_double(3000.0), _stream())
+    e1.record()
+    torch.cuda.synchronize()
+    assert 2.5 <= e0.elapsed_time(e1) <= 30.0
+    lib.checkLastCudaError(123)
