@@ -79,7 +79,9 @@ void launch_decode(const Act* x, const Weights& w, uint16_t* out, const Epilogue
     const int forced = decode_waves_override();
     const bool wide = forced ? forced == 16 : (N / 16 <= 256);
     if (M <= 16) {
-        if (wide) launch_decode_as<Act, 16, 1, 2>(x, w, out, ep, M, N, K, st);
+        const bool narrow = forced ? forced == 4 : (N / 16 > 512);      // as on the P2 layout: fewer, longer-lived waves
+        if (narrow) launch_decode_as<Act, 4, 1, 2>(x, w, out, ep, M, N, K, st);
+        else if (wide) launch_decode_as<Act, 16, 1, 2>(x, w, out, ep, M, N, K, st);
         else launch_decode_as<Act, 8, 1, 1>(x, w, out, ep, M, N, K, st);
     } else if (M <= 32) {
         if (wide) launch_decode_as<Act, 16, 2, 1>(x, w, out, ep, M, N, K, st);
