@@ -47,13 +47,62 @@ __device__ __forceinline__ void packed_prefill_epilogue(AccV (&acc)[NA][MB], uin
                                                         const Epilogue& ep, int M, int N, int n_wave, int m0, int lane)
 {
     const int kb = lane >> 5, l32 = lane & 31;
-    EpilogueRegs e[MB];
+    constexpr bool kFloatAcc = std::is_same<AccV, f32x16>::value;
+    auto value = [&](auto ac, auto bc, int idx) {
+        constexpr int a = decltype(ac)::value, b = decltype(bc)::value;
+        if constexpr (kFloatAcc) return acc[a][b][idx] * 2.0f;
+        else return static_cast<float>(acc[a][b][idx]);
+    };
     int m_of[MB];
+    float s_of[MB];
     static_for<0, MB>([&](auto bc) {
         constexpr int b = decltype(bc)::value;
         m_of[b] = m0 + 32 * b + l32;
-        e[b].s = ep.kind == EP_BF16 ? 1.0f : bf16_bits_to_float(ep.s[m_of[b] < M ? m_of[b] : M - 1]);
+        s_of[b] = ep.kind == EP_BF16 ? 1.0f : bf16_bits_to_float(ep.s[m_of[b] < M ? m_of[b] : M - 1]);
     });
+    auto store4 = [&](int b_m, int n, float r0, float r1, float r2, float r3) {
+        if (b_m < M && n < N)
+            *reinterpret_cast<u32x2*>(out + static_cast<size_t>(b_m) * N + n) = u32x2{pack_bf16x2(r0, r1), pack_bf16x2(r2, r3)};
+    };
+
+    // One weight-group scale per 32-feature tile whenever the group boundaries fall on multiples of
+    // 32 (always for the per-128-column rule of the prefill epilogue): the per-element work is then
+    // one multiply (bf16 family, prefill rule) or one divide and one multiply (decode rule), with
+    // the same operations in the same order as apply_epilogue.
+    const bool tile_groups = ep.kind == EP_I8_PREFILL || ep.ws_num == 1 || (N == 3840 && ep.ws_num == 3) ||
+                             (N / ep.ws_num) % 32 == 0;
+    if (tile_groups) {
+        float w_of[NA];
+        static_for<0, NA>([&](auto ac) {
+            constexpr int a = decltype(ac)::value;
+            int n_a = n_wave + 32 * a;
+            n_a = n_a < N ? n_a : N - 4;
+            const int g = ep.ws_num == 1 ? 0 : (ep.kind == EP_I8_PREFILL ? ws_group_prefill(n_a, N, ep.ws_num)
+                                                                       : ws_group_decode(n_a, N, ep.ws_num));
+            w_of[a] = ep.kind == EP_BF16 ? ep.scale[g] : bf16_bits_to_float(ep.ws[g]);
+        });
+        static_for<0, NA>([&](auto ac) {
+            constexpr int a = decltype(ac)::value;
+            static_for<0, MB>([&](auto bc) {
+                constexpr int b = decltype(bc)::value;
+                float coeff = w_of[a];
+                if (ep.kind == EP_I8_PREFILL) coeff = s_of[b] != 0.0f ? __fdiv_rn(w_of[a], s_of[b]) : 0.0f;
+                static_for<0, 4>([&](auto vc) {
+                    constexpr int vq = decltype(vc)::value;
+                    const int n = n_wave + 32 * a + 8 * vq + 4 * kb;
+                    float r[4];
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const float x = value(ac, bc, 4 * vq + v);
+                        r[v] = ep.kind == EP_I8_DECODE ? __fmul_rn(__fdiv_rn(x, s_of[b]), coeff) : __fmul_rn(x, coeff);
+                    }
+                    store4(m_of[b], n, r[0], r[1], r[2], r[3]);
+                });
+            });
+        });
+        return;
+    }
+    // group boundaries inside a tile: per-column scales
     static_for<0, 4 * NA>([&](auto tc) {
         constexpr int a = decltype(tc)::value >> 2, vq = decltype(tc)::value & 3;
         const int n = n_wave + 32 * a + 8 * vq + 4 * kb;
@@ -61,19 +110,15 @@ __device__ __forceinline__ void packed_prefill_epilogue(AccV (&acc)[NA][MB], uin
         load_col_scales(ep, n < N ? n : N - 4, N, wv);
         static_for<0, MB>([&](auto bc) {
             constexpr int b = decltype(bc)::value;
-            EpilogueRegs eb = e[b];
+            EpilogueRegs eb;
+            eb.s = s_of[b];
 #pragma unroll
             for (int v = 0; v < 4; ++v) eb.w[v] = wv[v];
-            uint16_t o[4];
+            float r[4];
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                if constexpr (std::is_same<AccV, f32x16>::value)
-                    o[v] = apply_epilogue<float>(ep.kind, eb, v, acc[a][b][4 * vq + v] * 2.0f);
-                else
-                    o[v] = apply_epilogue<int>(ep.kind, eb, v, acc[a][b][4 * vq + v]);
-            }
-            const u32x2 pk = {o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16)};
-            if (m_of[b] < M && n < N) *reinterpret_cast<u32x2*>(out + static_cast<size_t>(m_of[b]) * N + n) = pk;
+            for (int v = 0; v < 4; ++v)
+                r[v] = bf16_bits_to_float(apply_epilogue<float>(ep.kind, eb, v, value(std::integral_constant<int, a>{}, bc, 4 * vq + v)));
+            store4(m_of[b], n, r[0], r[1], r[2], r[3]);
         });
     });
 }
