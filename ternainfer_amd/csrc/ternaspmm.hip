@@ -218,9 +218,7 @@ void launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, 
     // when they would leave most of the 1024 workgroup slots of the chip empty, 128-feature tiles
     // double the workgroup count instead.  TERNASPMM_PREFILL_BN=128|256 forces one (tuning aid).
     const long wg256 = static_cast<long>((N + 255) / 256) * ((M + 63) / 64);
-    // int8 activations: a step is half as many MFMA cycles per byte loaded, and the extra waves of
-    // the small tile hide more latency than its extra operand reads cost -- 128 wins at every shape.
-    const int bn = forced_bn ? forced_bn : ((sizeof(Act) == 1 || wg256 <= 640) ? 128 : 256);
+    const int bn = forced_bn ? forced_bn : (wg256 <= 640 ? 128 : 256);
     if (prefill_dma_ok(x, sizeof(Act), M, N, K) && (bm == 64 || bm == 128)) {
         if (bm == 64 && bn == 128) launch_prefill_packed_dma_as<Act, 2, 1>(x, packed, out, ep, M, N, K, st);
         else if (bm == 128 && forced_bn == 128) launch_prefill_packed_dma_as<Act, 4, 1>(x, packed, out, ep, M, N, K, st);
