@@ -81,25 +81,47 @@ __device__ __forceinline__ void packed_prefill_epilogue(AccV (&acc)[NA][MB], uin
                                                                        : ws_group_decode(n_a, N, ep.ws_num));
             w_of[a] = ep.kind == EP_BF16 ? ep.scale[g] : bf16_bits_to_float(ep.ws[g]);
         });
-        static_for<0, NA>([&](auto ac) {
-            constexpr int a = decltype(ac)::value;
-            static_for<0, MB>([&](auto bc) {
-                constexpr int b = decltype(bc)::value;
-                float coeff = w_of[a];
-                if (ep.kind == EP_I8_PREFILL) coeff = s_of[b] != 0.0f ? __fdiv_rn(w_of[a], s_of[b]) : 0.0f;
-                static_for<0, 4>([&](auto vc) {
-                    constexpr int vq = decltype(vc)::value;
-                    const int n = n_wave + 32 * a + 8 * vq + 4 * kb;
-                    float r[4];
+        // Two separate loops under a uniform branch: written as a select, the compiler evaluates the
+        // IEEE division of the decode rule for every element of every kind.
+        auto tiles = [&](auto&& element) {
+            static_for<0, NA>([&](auto ac) {
+                constexpr int a = decltype(ac)::value;
+                static_for<0, MB>([&](auto bc) {
+                    constexpr int b = decltype(bc)::value;
+                    static_for<0, 4>([&](auto vc) {
+                        constexpr int vq = decltype(vc)::value;
+                        float r[4];
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        const float x = value(ac, bc, 4 * vq + v);
-                        r[v] = ep.kind == EP_I8_DECODE ? __fmul_rn(__fdiv_rn(x, s_of[b]), coeff) : __fmul_rn(x, coeff);
-                    }
-                    store4(m_of[b], n, r[0], r[1], r[2], r[3]);
+                        for (int v = 0; v < 4; ++v) r[v] = element(w_of[a], s_of[b], value(ac, bc, 4 * vq + v));
+                        store4(m_of[b], n_wave + 32 * a + 8 * vq + 4 * kb, r[0], r[1], r[2], r[3]);
+                    });
                 });
             });
-        });
+        };
+        if (ep.kind == EP_I8_DECODE) {
+            tiles([](float w, float sm, float x) { return __fmul_rn(__fdiv_rn(x, sm), w); });
+        } else if (ep.kind == EP_I8_PREFILL) {
+            float coeff[NA][MB];
+#pragma unroll
+            for (int a = 0; a < NA; ++a)
+#pragma unroll
+                for (int b = 0; b < MB; ++b) coeff[a][b] = s_of[b] != 0.0f ? __fdiv_rn(w_of[a], s_of[b]) : 0.0f;
+            static_for<0, NA>([&](auto ac) {
+                constexpr int a = decltype(ac)::value;
+                static_for<0, MB>([&](auto bc) {
+                    constexpr int b = decltype(bc)::value;
+                    static_for<0, 4>([&](auto vc) {
+                        constexpr int vq = decltype(vc)::value;
+                        float r[4];
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) r[v] = __fmul_rn(value(ac, bc, 4 * vq + v), coeff[a][b]);
+                        store4(m_of[b], n_wave + 32 * a + 8 * vq + 4 * kb, r[0], r[1], r[2], r[3]);
+                    });
+                });
+            });
+        } else {
+            tiles([](float w, float, float x) { return __fmul_rn(x, w); });
+        }
         return;
     }
     // group boundaries inside a tile: per-column scales
