@@ -359,7 +359,7 @@ struct PackedPrefillDmaSmem {
 template <typename Act, int MB, int NA>
 __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) void terna_prefill_packed_dma_kernel(
     const Act* __restrict__ x, const uint32_t* __restrict__ packed, uint16_t* __restrict__ out,
-    Epilogue ep, int M, int N, int K)
+    Epilogue ep, int M, int N, int K, int xcd_map)
 {
     using S = PackedPrefillDmaSmem<MB>;
     constexpr int BN = 128 * NA, BM = S::BM;
@@ -376,7 +376,20 @@ __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) voi
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int n0 = blockIdx.x * BN, m0 = blockIdx.y * BM;
+    // Workgroup -> tile.  Workgroups go to the 8 XCDs round robin by their linear index, and each XCD
+    // has its own L2: when the batch tiles divide by 8, XCD c gets batch tiles c*T/8 .. and walks
+    // through them feature tile by feature tile, so its share of the activations (a few MB) stays in
+    // its L2 and a weight tile is fetched once per XCD per pass instead of the activations being
+    // streamed again for every feature tile.
+    int n_tile = blockIdx.x, m_tile = blockIdx.y;
+    if (xcd_map) {
+        const int linear = blockIdx.y * gridDim.x + blockIdx.x;
+        const int per_xcd = gridDim.y >> 3;          // batch tiles per XCD
+        const int xcd = linear & 7, idx = linear >> 3;
+        m_tile = xcd * per_xcd + idx % per_xcd;
+        n_tile = idx / per_xcd;
+    }
+    const int n0 = n_tile * BN, m0 = m_tile * BM;
     const int ktiles = K >> 6;
     const int steps = I8 ? (ktiles + 1) >> 1 : ktiles;
     // int8 with an odd tile count: in the last step the kb = 1 half has no tile.  Its loads are

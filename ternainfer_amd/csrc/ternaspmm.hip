@@ -181,7 +181,16 @@ void launch_prefill_packed_dma_as(const Act* x, const uint32_t* packed, uint16_t
     if (attr != hipSuccess) die("hipFuncSetAttribute(prefill packed dma)", attr, __LINE__);
     constexpr int BN = 128 * NA;
     const dim3 grid((N + BN - 1) / BN, (M + S::BM - 1) / S::BM);
-    kernel<<<grid, dim3(256), S::kBytes, st>>>(x, packed, out, ep, M, N, K);
+    static const int xcd_forced = [] {
+        const char* v = std::getenv("TERNASPMM_PREFILL_XCD_MAP");
+        return v ? std::atoi(v) : -1;
+    }();
+    // XCD-aware tile order (see the kernel): pays once the activations no longer fit one XCD's 4 MiB L2 --
+    // below that the default order, which fetches every weight tile on one XCD only, moves less data.
+    // TERNASPMM_PREFILL_XCD_MAP=0|1 forces it off / on (tuning aid).
+    const bool big_x = static_cast<size_t>(M) * K * sizeof(Act) > (4u << 20);
+    const int xcd_map = (grid.y % 8 == 0) && (xcd_forced < 0 ? big_x : xcd_forced != 0);
+    kernel<<<grid, dim3(256), S::kBytes, st>>>(x, packed, out, ep, M, N, K, xcd_map);
 }
 
 // The direct-to-LDS kernel addresses both operands as a 64-bit base plus a 32-bit byte offset and

@@ -15,7 +15,7 @@ from ternainfer_amd import _lib
 def main() -> int:
     lib = _lib.load()
     co = O.COracle()
-    for m, n, k in [(100, 320, 192), (300, 512, 320), (65, 256, 64), (256, 3840, 128)]:
+    for m, n, k in [(100, 320, 192), (300, 512, 320), (65, 256, 64), (256, 3840, 128), (512, 384, 128), (1024, 320, 64)]:
         w = make_ternary(n, k, 0.40, 900 + m + n)
         packed = repack(lib, DeviceFormat(w))
         xq, s = make_int8_activations(m, k, 901 + m)

@@ -515,6 +515,7 @@ def test_kernel_binary_reference_command_line():
                                  {"TERNASPMM_PREFILL_BM": "128", "TERNASPMM_PREFILL_BN": "128"},
                                  {"TERNASPMM_PREFILL_BN": "256"}, {"TERNASPMM_PREFILL_BN": "128"},
                                  {"TERNASPMM_PREFILL_BM": "256"}, {"TERNASPMM_PREFILL_BM": "96"},
+                                 {"TERNASPMM_PREFILL_XCD_MAP": "1"}, {"TERNASPMM_PREFILL_XCD_MAP": "1", "TERNASPMM_PREFILL_BM": "128"},
                                  {"TERNASPMM_DECODE_WAVES": "4"}, {"TERNASPMM_DECODE_WAVES": "8"}, {"TERNASPMM_DECODE_WAVES": "16"}])
 def test_tile_and_path_overrides(env):
     """Every large-M tile shape and the register-staged path behind the library's tuning overrides
