@@ -190,16 +190,17 @@ int bitlinear_TernaSpMM_packed_fused_glu(const terna_bf16* x13, const terna_bf16
  * fmha.memory_efficient_attention_forward (model.py:231-233).
  *
  * ternaspmm_rope_kv_store: rotary embedding of the q and k heads of the fused qkv linear's output
- * (bf16 [B*T][(H + 2*KV)*D], row b*T + t), pairs (j, j + D/2) rotated by the angle whose cosine / sine is
- * cos[t][j] / sin[t][j] (fp32 [T][D/2]); q goes to q_out (bf16 [B][H][T][D]); k and v go into the caches
- * (bf16 [B][KV][S][D]) at slot pos[t] (int64 [T], device memory).
+ * (bf16 [B*T][(H + 2*KV)*D], row b*T + t): pair j of a head -- dimensions (2j, 2j + 1) when `adjacent` is
+ * non-zero (rope_padded's default and the order of the reference's checkpoints), (j, j + D/2) otherwise -- is
+ * rotated by the angle whose cosine / sine is cos[t][j] / sin[t][j] (fp32 [T][D/2]); q goes to q_out
+ * (bf16 [B][H][T][D]); k and v go into the caches (bf16 [B][KV][S][D]) at slot pos[t] (int64 [T], device memory).
  *
  * ternaspmm_decode_attention: one new token per sequence.  q bf16 [B][H][D]; head h reads kv head
  * h / (H/KV) at slots 0 .. pos[0]; out bf16 [B][H*D] = softmax(scale * q K^T) V.  D is 64 or 128,
  * S <= 8192.  Both only enqueue. */
 void ternaspmm_rope_kv_store(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
                              terna_bf16* q_out, terna_bf16* cache_k, terna_bf16* cache_v, int B, int T, int H,
-                             int KV, int D, int S, terna_stream stream);
+                             int KV, int D, int S, int adjacent, terna_stream stream);
 void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
                                 const long long* pos, terna_bf16* out, int B, int H, int KV, int D, int S,
                                 float scale, terna_stream stream);
@@ -208,7 +209,7 @@ void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, 
  * ternaspmm_rope_kv_store followed by ternaspmm_decode_attention. */
 void ternaspmm_rope_decode_attention(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
                                      terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
-                                     int D, int S, float scale, terna_stream stream);
+                                     int D, int S, float scale, int adjacent, terna_stream stream);
 
 /* Opt-in repack cache for unmodified call sites: with TERNASPMM_REPACK_CACHE=1 in the environment the
  * reference-format entry points above (bitlinear_TernaSpMM*, bitlinear_TernaSpMM_bf16*) keep a device-side P2

@@ -21,12 +21,14 @@ Reference files restated (paths relative to the reference checkout):
 
 Parity status: every function is pinned by a test in tests/test_oracle_*.py except
 ``quant_input``'s intermediate precision, which the reference leaves open
-("parity unpinned" beyond the two-line formula), and ``rmsnorm``: the reference takes
-RMSNorm from xformers.ops (model.py:16), a third-party dependency that is not part of
-the reference checkout and not installed here, so "parity unpinned"; the formula
-y = x * rsqrt(mean(x^2) + eps) * weight, fp32 inside and one rounding to the tensor's
-dtype, restates that operator's published definition and is checked against what the
-mathematics fixes (tests/test_oracle_linear.py).
+("parity unpinned" beyond the two-line formula), and ``rmsnorm``, ``rope_rotate_half``,
+``rope_adjacent`` and ``attention_one_token``: the reference takes RMSNorm, rope_padded
+and the attention forward from xformers.ops (model.py:16), a third-party dependency that
+is not part of the reference checkout and not installed here, so "parity unpinned"; the
+formulas (y = x * rsqrt(mean(x^2) + eps) * weight, fp32 inside and one rounding to the
+tensor's dtype; rotation of dimension pairs by position-dependent angles; softmax(q K^T
+scale) V over the valid cache slots) restate those operators' published definitions and
+are checked against what the mathematics fixes (tests/test_oracle_linear.py).
 """
 from __future__ import annotations
 
@@ -294,6 +296,19 @@ def rope_rotate_half(x_bits: np.ndarray, cos: np.ndarray, sin: np.ndarray) -> np
     x1, x2 = x[..., :half], x[..., half:]
     c, s = cos.astype(np.float32), sin.astype(np.float32)
     return f32_to_bf16_bits(np.concatenate([x1 * c - x2 * s, x2 * c + x1 * s], axis=-1).astype(np.float32))
+
+
+def rope_adjacent(x_bits: np.ndarray, cos: np.ndarray, sin: np.ndarray) -> np.ndarray:
+    """As rope_rotate_half with pair j = (x[2j], x[2j + 1]): rope_padded's default pairing, the one the
+    reference's checkpoints are laid out for (convert_TernaInfer.py:46-50 undoes the rotate-half row
+    order of the source checkpoint).  Same arithmetic order and rounding; parity unpinned likewise."""
+    x = bf16_bits_to_f32(x_bits)
+    x1, x2 = x[..., 0::2], x[..., 1::2]
+    c, s = cos.astype(np.float32), sin.astype(np.float32)
+    out = np.empty_like(x)
+    out[..., 0::2] = x1 * c - x2 * s
+    out[..., 1::2] = x2 * c + x1 * s
+    return f32_to_bf16_bits(out.astype(np.float32))
 
 
 def attention_one_token(q_bits: np.ndarray, k_bits: np.ndarray, v_bits: np.ndarray, n: int, scale: float) -> np.ndarray:

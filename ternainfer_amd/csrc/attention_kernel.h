@@ -6,8 +6,10 @@
 //
 // They stand where the reference calls xformers' rope_padded (model.py:218-229) and
 // fmha.memory_efficient_attention_forward (model.py:231-233); both are absent third-party
-// operators, restated here from their definitions (rotate-half RoPE with given cos/sin tables;
-// softmax(q K^T / sqrt(D)) V over the valid cache slots).  fp32 inside, bf16 storage.
+// operators, restated here from their definitions (RoPE with given cos/sin tables, pairing either
+// adjacent dimensions -- rope_padded's default, which the reference's checkpoints are laid out for
+// -- or the two halves of a head; softmax(q K^T / sqrt(D)) V over the valid cache slots).
+// fp32 inside, bf16 storage.
 #pragma once
 
 #include "norm_quant_kernel.h"
@@ -19,8 +21,9 @@ namespace terna {
 // pos   int64 [T]                    cache slot of token t (same for every sequence)
 // q_out bf16 [B][H][T][D]
 // cache_k, cache_v  bf16 [B][KV][S][D]
-// Pair j of a head is (x[j], x[j + D/2]):  x[j]' = x[j] cos - x[j + D/2] sin,
-//                                          x[j + D/2]' = x[j + D/2] cos + x[j] sin.
+// Pair j of a head is (a, b) = (x[2j], x[2j + 1]) when ADJACENT, else (x[j], x[j + D/2]):
+//   a' = a cos - b sin,   b' = b cos + a sin.
+template <bool ADJACENT>
 __global__ __launch_bounds__(256) void terna_rope_kv_store_kernel(
     const uint16_t* __restrict__ qkv, const float* __restrict__ cosv, const float* __restrict__ sinv,
     const long long* __restrict__ pos, uint16_t* __restrict__ q_out, uint16_t* __restrict__ cache_k,
@@ -36,20 +39,33 @@ __global__ __launch_bounds__(256) void terna_rope_kv_store_kernel(
         // 8 pairs per thread: 16-byte loads and stores, for the 2B model one pass of 240 threads
         const int per = half >> 3;
         for (int i = threadIdx.x; i < slots * per; i += blockDim.x) {
-            const int hs = i / per, j = (i - hs * per) * 8;
+            const int hs = i / per, j = (i - hs * per) * 8;          // pairs j .. j+7
+            // the two 8-element chunks that hold those pairs
+            const int off1 = ADJACENT ? 2 * j : j, off2 = ADJACENT ? 2 * j + 8 : j + half;
             float x1[8], x2[8], o1[8], o2[8];
-            unpack_bf16x8(*reinterpret_cast<const u32x4*>(src + hs * D + j), x1);
-            unpack_bf16x8(*reinterpret_cast<const u32x4*>(src + hs * D + j + half), x2);
+            unpack_bf16x8(*reinterpret_cast<const u32x4*>(src + hs * D + off1), x1);
+            unpack_bf16x8(*reinterpret_cast<const u32x4*>(src + hs * D + off2), x2);
             if (hs < H + KV) {
                 const f32x4* cp = reinterpret_cast<const f32x4*>(cosv + t * half + j);
                 const f32x4* sp = reinterpret_cast<const f32x4*>(sinv + t * half + j);
                 const f32x4 c0 = cp[0], c1 = cp[1], s0 = sp[0], s1 = sp[1];
+                if constexpr (ADJACENT) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
+                    for (int m = 0; m < 4; ++m) {
 #pragma clang fp contract(off)                   // every product and sum rounded once: a defined result
-                    const float c = e < 4 ? c0[e & 3] : c1[e & 3], sn = e < 4 ? s0[e & 3] : s1[e & 3];
-                    o1[e] = x1[e] * c - x2[e] * sn;
-                    o2[e] = x2[e] * c + x1[e] * sn;
+                        o1[2 * m] = x1[2 * m] * c0[m] - x1[2 * m + 1] * s0[m];
+                        o1[2 * m + 1] = x1[2 * m + 1] * c0[m] + x1[2 * m] * s0[m];
+                        o2[2 * m] = x2[2 * m] * c1[m] - x2[2 * m + 1] * s1[m];
+                        o2[2 * m + 1] = x2[2 * m + 1] * c1[m] + x2[2 * m] * s1[m];
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+#pragma clang fp contract(off)
+                        const float c = e < 4 ? c0[e & 3] : c1[e & 3], sn = e < 4 ? s0[e & 3] : s1[e & 3];
+                        o1[e] = x1[e] * c - x2[e] * sn;
+                        o2[e] = x2[e] * c + x1[e] * sn;
+                    }
                 }
             } else {
 #pragma unroll
@@ -59,15 +75,16 @@ __global__ __launch_bounds__(256) void terna_rope_kv_store_kernel(
             if (hs < H) dst = q_out + ((static_cast<size_t>(b) * H + hs) * T + t) * D;
             else if (hs < H + KV) dst = cache_k + ((static_cast<size_t>(b) * KV + (hs - H)) * S + slot) * D;
             else dst = cache_v + ((static_cast<size_t>(b) * KV + (hs - H - KV)) * S + slot) * D;
-            *reinterpret_cast<u32x4*>(dst + j) = pack_bf16x8(o1);
-            *reinterpret_cast<u32x4*>(dst + j + half) = pack_bf16x8(o2);
+            *reinterpret_cast<u32x4*>(dst + off1) = pack_bf16x8(o1);
+            *reinterpret_cast<u32x4*>(dst + off2) = pack_bf16x8(o2);
         }
         return;
     }
     for (int i = threadIdx.x; i < slots * half; i += blockDim.x) {
         const int hs = i / half, j = i - hs * half;
-        const float x1 = bf16_bits_to_float(src[hs * D + j]);
-        const float x2 = bf16_bits_to_float(src[hs * D + j + half]);
+        const int ia = ADJACENT ? 2 * j : j, ib = ADJACENT ? 2 * j + 1 : j + half;
+        const float x1 = bf16_bits_to_float(src[hs * D + ia]);
+        const float x2 = bf16_bits_to_float(src[hs * D + ib]);
         uint16_t* dst;
         float o1 = x1, o2 = x2;
         if (hs < H + KV) {
@@ -79,8 +96,8 @@ __global__ __launch_bounds__(256) void terna_rope_kv_store_kernel(
         if (hs < H) dst = q_out + ((static_cast<size_t>(b) * H + hs) * T + t) * D;
         else if (hs < H + KV) dst = cache_k + ((static_cast<size_t>(b) * KV + (hs - H)) * S + slot) * D;
         else dst = cache_v + ((static_cast<size_t>(b) * KV + (hs - H - KV)) * S + slot) * D;
-        dst[j] = float_to_bf16_bits(o1);
-        dst[j + half] = float_to_bf16_bits(o2);
+        dst[ia] = float_to_bf16_bits(o1);
+        dst[ib] = float_to_bf16_bits(o2);
     }
 }
 
@@ -95,8 +112,9 @@ __global__ __launch_bounds__(256) void terna_rope_kv_store_kernel(
 // then the fused qkv row of the new token (bf16 [B][(H + 2*KV)*D]); every workgroup rotates its own
 // q head and the new key row of its kv head in registers (same arithmetic, bit for bit), uses them
 // -- and the new value row -- in place of cache slot pos[0], and the first workgroup of each kv
-// group writes the new key / value rows into the cache for the steps to come.
-template <int D, bool ROPE>
+// group writes the new key / value rows into the cache for the steps to come.  ADJACENT selects
+// the pairing of the rotation, as in terna_rope_kv_store_kernel.
+template <int D, bool ROPE, bool ADJACENT = false>
 __global__ __launch_bounds__(256) void terna_decode_attention_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
     const float* __restrict__ cosv, const float* __restrict__ sinv,
@@ -150,42 +168,72 @@ __global__ __launch_bounds__(256) void terna_decode_attention_kernel(
         for (int jj = 0; jj < NJ; ++jj)
             qr[jj] = *reinterpret_cast<const u32x4*>(q + (static_cast<size_t>(b) * H + h) * D + 32 * jj + 8 * kblk);
     } else {
-        // chunk c = 4jj + kblk (dimensions 8c .. 8c+7) and its rotation partner c +- CH/2
         const uint16_t* row = q + static_cast<size_t>(b) * (H + 2 * KV) * D;
-        u32x4 q_own[NJ], q_par[NJ], k_own[NJ], k_par[NJ];
-        f32x4 cs[NJ][2], sn[NJ][2];
-#pragma unroll
-        for (int jj = 0; jj < NJ; ++jj) {
-            const int c = 4 * jj + kblk, cp = (c + CH / 2) % CH, ca = c % (CH / 2);
-            q_own[jj] = *reinterpret_cast<const u32x4*>(row + h * D + 8 * c);
-            q_par[jj] = *reinterpret_cast<const u32x4*>(row + h * D + 8 * cp);
-            k_own[jj] = *reinterpret_cast<const u32x4*>(row + (H + kvh) * D + 8 * c);
-            k_par[jj] = *reinterpret_cast<const u32x4*>(row + (H + kvh) * D + 8 * cp);
-            cs[jj][0] = *reinterpret_cast<const f32x4*>(cosv + 8 * ca);
-            cs[jj][1] = *reinterpret_cast<const f32x4*>(cosv + 8 * ca + 4);
-            sn[jj][0] = *reinterpret_cast<const f32x4*>(sinv + 8 * ca);
-            sn[jj][1] = *reinterpret_cast<const f32x4*>(sinv + 8 * ca + 4);
-        }
         vnew = *reinterpret_cast<const u32x4*>(row + (H + KV + kvh) * D + 8 * chunk);
-        auto rotate = [&](const u32x4& own, const u32x4& par, int jj, bool first_half) {
-            float a[8], p[8], o[8];
-            unpack_bf16x8(own, a);
-            unpack_bf16x8(par, p);
+        if constexpr (ADJACENT) {
+            // chunk c = 4jj + kblk (dimensions 8c .. 8c+7) holds pairs 4c .. 4c+3 whole
+            u32x4 q_own[NJ], k_own[NJ];
+            f32x4 cs[NJ], sn[NJ];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-#pragma clang fp contract(off)                   // as terna_rope_kv_store_kernel: every product and sum rounded once
-                const float c = cs[jj][e >> 2][e & 3], sv = sn[jj][e >> 2][e & 3];
-                const float lo = a[e] * c - p[e] * sv;     // own chunk in the first half:  x1 c - x2 s
-                const float hi = a[e] * c + p[e] * sv;     // own chunk in the second half: x2 c + x1 s
-                o[e] = first_half ? lo : hi;
+            for (int jj = 0; jj < NJ; ++jj) {
+                const int c = 4 * jj + kblk;
+                q_own[jj] = *reinterpret_cast<const u32x4*>(row + h * D + 8 * c);
+                k_own[jj] = *reinterpret_cast<const u32x4*>(row + (H + kvh) * D + 8 * c);
+                cs[jj] = *reinterpret_cast<const f32x4*>(cosv + 4 * c);
+                sn[jj] = *reinterpret_cast<const f32x4*>(sinv + 4 * c);
             }
-            return pack_bf16x8(o);
-        };
+            auto rotate = [&](const u32x4& own, int jj) {
+                float a[8], o[8];
+                unpack_bf16x8(own, a);
 #pragma unroll
-        for (int jj = 0; jj < NJ; ++jj) {
-            const bool first_half = 4 * jj + kblk < CH / 2;
-            qr[jj] = rotate(q_own[jj], q_par[jj], jj, first_half);
-            knew[jj] = rotate(k_own[jj], k_par[jj], jj, first_half);
+                for (int m = 0; m < 4; ++m) {
+#pragma clang fp contract(off)                   // as terna_rope_kv_store_kernel: every product and sum rounded once
+                    o[2 * m] = a[2 * m] * cs[jj][m] - a[2 * m + 1] * sn[jj][m];
+                    o[2 * m + 1] = a[2 * m + 1] * cs[jj][m] + a[2 * m] * sn[jj][m];
+                }
+                return pack_bf16x8(o);
+            };
+#pragma unroll
+            for (int jj = 0; jj < NJ; ++jj) {
+                qr[jj] = rotate(q_own[jj], jj);
+                knew[jj] = rotate(k_own[jj], jj);
+            }
+        } else {
+            // chunk c = 4jj + kblk (dimensions 8c .. 8c+7) and its rotation partner c +- CH/2
+            u32x4 q_own[NJ], q_par[NJ], k_own[NJ], k_par[NJ];
+            f32x4 cs[NJ][2], sn[NJ][2];
+#pragma unroll
+            for (int jj = 0; jj < NJ; ++jj) {
+                const int c = 4 * jj + kblk, cp = (c + CH / 2) % CH, ca = c % (CH / 2);
+                q_own[jj] = *reinterpret_cast<const u32x4*>(row + h * D + 8 * c);
+                q_par[jj] = *reinterpret_cast<const u32x4*>(row + h * D + 8 * cp);
+                k_own[jj] = *reinterpret_cast<const u32x4*>(row + (H + kvh) * D + 8 * c);
+                k_par[jj] = *reinterpret_cast<const u32x4*>(row + (H + kvh) * D + 8 * cp);
+                cs[jj][0] = *reinterpret_cast<const f32x4*>(cosv + 8 * ca);
+                cs[jj][1] = *reinterpret_cast<const f32x4*>(cosv + 8 * ca + 4);
+                sn[jj][0] = *reinterpret_cast<const f32x4*>(sinv + 8 * ca);
+                sn[jj][1] = *reinterpret_cast<const f32x4*>(sinv + 8 * ca + 4);
+            }
+            auto rotate = [&](const u32x4& own, const u32x4& par, int jj, bool first_half) {
+                float a[8], p[8], o[8];
+                unpack_bf16x8(own, a);
+                unpack_bf16x8(par, p);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+#pragma clang fp contract(off)
+                    const float c = cs[jj][e >> 2][e & 3], sv = sn[jj][e >> 2][e & 3];
+                    const float lo = a[e] * c - p[e] * sv;     // own chunk in the first half:  x1 c - x2 s
+                    const float hi = a[e] * c + p[e] * sv;     // own chunk in the second half: x2 c + x1 s
+                    o[e] = first_half ? lo : hi;
+                }
+                return pack_bf16x8(o);
+            };
+#pragma unroll
+            for (int jj = 0; jj < NJ; ++jj) {
+                const bool first_half = 4 * jj + kblk < CH / 2;
+                qr[jj] = rotate(q_own[jj], q_par[jj], jj, first_half);
+                knew[jj] = rotate(k_own[jj], k_par[jj], jj, first_half);
+            }
         }
         if (h % (H / KV) == 0) {                 // this kv group's writer: slot pos[0] of both caches
             const size_t slot_off = ((static_cast<size_t>(b) * KV + kvh) * S + (n - 1)) * D;

@@ -47,6 +47,26 @@ struct Weights {
     const uint32_t* sign_words;
 };
 
+// Dynamic-LDS opt-in of one kernel, once per (kernel, device) of the process: the attribute is per device.
+void allow_dynamic_lds_ptr(const void* kernel, int bytes, const char* what, int line)
+{
+    static std::mutex mutex;
+    static std::unordered_map<const void*, uint64_t> done;       // kernel -> bit per device ordinal
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
+    std::lock_guard<std::mutex> lock(mutex);
+    uint64_t& mask = done[kernel];
+    if (dev >= 0 && ((mask >> dev) & 1u)) return;
+    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) die(what, e, line);
+    if (dev >= 0) mask |= uint64_t{1} << dev;
+}
+template <typename Kernel>
+void allow_dynamic_lds(Kernel kernel, int bytes, const char* what, int line)
+{
+    allow_dynamic_lds_ptr(reinterpret_cast<const void*>(kernel), bytes, what, line);
+}
+
 // Small-M kernel: one workgroup per 16-row band; up to 64 batch rows per workgroup.
 template <typename Act, int WAVES, int MB, int DEPTH>
 void launch_decode_as(const Act* x, const Weights& w, uint16_t* out, const Epilogue& ep, int M, int N, int K,
@@ -98,9 +118,7 @@ void launch_prefill_as(const Act* x, const Weights& w, uint16_t* out, const Epil
 {
     using S = PrefillSmem<MT>;
     auto kernel = terna_prefill_kernel<Act, MT>;
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, S::kBytes);
-    if (attr != hipSuccess) die("hipFuncSetAttribute(prefill)", attr, __LINE__);
+    allow_dynamic_lds(kernel, S::kBytes, "hipFuncSetAttribute(prefill)", __LINE__);
     const dim3 grid((N + kPrefillBN - 1) / kPrefillBN, (M + S::BM - 1) / S::BM);
     kernel<<<grid, dim3(256), S::kBytes, st>>>(x, w.bitmap, w.tile_off, w.median_off, w.sign_words, out, ep, M, N, K);
 }
@@ -162,9 +180,7 @@ void launch_prefill_packed_as(const Act* x, const uint32_t* packed, uint16_t* ou
 {
     using S = PackedPrefillSmem<MB>;
     auto kernel = terna_prefill_packed_kernel<Act, MB, NA>;
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, S::kBytes);
-    if (attr != hipSuccess) die("hipFuncSetAttribute(prefill packed)", attr, __LINE__);
+    allow_dynamic_lds(kernel, S::kBytes, "hipFuncSetAttribute(prefill packed)", __LINE__);
     constexpr int BN = 128 * NA;
     const dim3 grid((N + BN - 1) / BN, (M + S::BM - 1) / S::BM);
     kernel<<<grid, dim3(256), S::kBytes, st>>>(x, packed, out, ep, M, N, K);
@@ -176,9 +192,7 @@ void launch_prefill_packed_dma_as(const Act* x, const uint32_t* packed, uint16_t
 {
     using S = PackedPrefillDmaSmem<MB>;
     auto kernel = terna_prefill_packed_dma_kernel<Act, MB, NA>;
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, S::kBytes);
-    if (attr != hipSuccess) die("hipFuncSetAttribute(prefill packed dma)", attr, __LINE__);
+    allow_dynamic_lds(kernel, S::kBytes, "hipFuncSetAttribute(prefill packed dma)", __LINE__);
     constexpr int BN = 128 * NA;
     const dim3 grid((N + BN - 1) / BN, (M + S::BM - 1) / S::BM);
     static const int xcd_forced = [] {
@@ -644,14 +658,17 @@ int bitlinear_TernaSpMM_packed_fused_glu(const terna_bf16* x13, const terna_bf16
 
 void ternaspmm_rope_kv_store(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
                              terna_bf16* q_out, terna_bf16* cache_k, terna_bf16* cache_v, int B, int T, int H,
-                             int KV, int D, int S, terna_stream stream)
+                             int KV, int D, int S, int adjacent, terna_stream stream)
 {
     if (B < 1 || T < 1 || H < 1 || KV < 1 || D < 2 || (D & 1) || S < 1) {
         std::fprintf(stderr, "ternaspmm_rope_kv_store: unsupported arguments\n");
         return;
     }
-    terna_rope_kv_store_kernel<<<dim3(B * T), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
-        qkv, cos, sin, pos, q_out, cache_k, cache_v, T, H, KV, D, S);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (adjacent)
+        terna_rope_kv_store_kernel<true><<<dim3(B * T), dim3(256), 0, st>>>(qkv, cos, sin, pos, q_out, cache_k, cache_v, T, H, KV, D, S);
+    else
+        terna_rope_kv_store_kernel<false><<<dim3(B * T), dim3(256), 0, st>>>(qkv, cos, sin, pos, q_out, cache_k, cache_v, T, H, KV, D, S);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_rope_kv_store", e, __LINE__);
 }
@@ -678,7 +695,7 @@ void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, 
 
 void ternaspmm_rope_decode_attention(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
                                      terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
-                                     int D, int S, float scale, terna_stream stream)
+                                     int D, int S, float scale, int adjacent, terna_stream stream)
 {
     if (B < 1 || H < 1 || KV < 1 || H % KV != 0 || (D != 64 && D != 128) || S < 1 || S > 8192) {
         std::fprintf(stderr, "ternaspmm_rope_decode_attention: unsupported arguments (H=%d KV=%d D=%d S=%d)\n", H, KV, D, S);
@@ -686,10 +703,17 @@ void ternaspmm_rope_decode_attention(const terna_bf16* qkv, const float* cos, co
     }
     const size_t lds = (static_cast<size_t>(S) + (256 / (D / 8)) * D) * sizeof(float);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (D == 128)
-        terna_decode_attention_kernel<128, true><<<dim3(B * H), dim3(256), lds, st>>>(qkv, cache_k, cache_v, cos, sin, pos, out, H, KV, S, scale);
-    else
-        terna_decode_attention_kernel<64, true><<<dim3(B * H), dim3(256), lds, st>>>(qkv, cache_k, cache_v, cos, sin, pos, out, H, KV, S, scale);
+#define TERNA_ROPE_ATTN(DIM, ADJ)                                                                                  \
+    terna_decode_attention_kernel<DIM, true, ADJ><<<dim3(B * H), dim3(256), lds, st>>>(qkv, cache_k, cache_v, cos, sin, \
+                                                                                        pos, out, H, KV, S, scale)
+    if (D == 128) {
+        if (adjacent) TERNA_ROPE_ATTN(128, true);
+        else TERNA_ROPE_ATTN(128, false);
+    } else {
+        if (adjacent) TERNA_ROPE_ATTN(64, true);
+        else TERNA_ROPE_ATTN(64, false);
+    }
+#undef TERNA_ROPE_ATTN
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_rope_decode_attention", e, __LINE__);
 }

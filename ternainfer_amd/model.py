@@ -21,7 +21,7 @@ import torch
 from torch.nn import functional as F
 
 from . import _lib
-from .linear import (relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant, rmsnorm_linear_packed,
+from .linear import (relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant, repack_weight, rmsnorm_linear_packed,
                      rmsnorm_quant)
 
 
@@ -35,6 +35,7 @@ class ModelArgs:                      # model.py:23-34
     ffn_dim: int = 6912
     norm_eps: float = 1e-5
     rope_theta: float = 500000.0
+    rope_adjacent: bool = True        # pairs (2j, 2j+1), rope_padded's default (model.py:221-229); False = (j, j + D/2)
 
     @property
     def head_dim(self) -> int:
@@ -104,14 +105,24 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * weight.float()).to(x.dtype)
 
 
-def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
-    """x [B, H, T, D]; rotate-half convention; cos/sin broadcastable to [B, H, T, D/2], fp32."""
-    x1, x2 = x.float().chunk(2, dim=-1)
+def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, adjacent: bool = True) -> torch.Tensor:
+    """x [B, H, T, D]; cos/sin broadcastable to [B, H, T, D/2], fp32; pair j = (x[2j], x[2j+1]) when
+    `adjacent`, else (x[j], x[j + D/2])."""
+    xf = x.float()
+    if adjacent:
+        x1, x2 = xf[..., 0::2], xf[..., 1::2]
+        return torch.stack([x1 * cos - x2 * sin, x2 * cos + x1 * sin], dim=-1).flatten(-2).to(x.dtype)
+    x1, x2 = xf.chunk(2, dim=-1)
     return torch.cat([x1 * cos - x2 * sin, x2 * cos + x1 * sin], dim=-1).to(x.dtype)
 
 
 class Block:
-    def __init__(self, args: ModelArgs, gen: torch.Generator, act: str, p_zero: float):
+    def __init__(self, args: ModelArgs, gen: Optional[torch.Generator], act: str, p_zero: float = 0.40):
+        self.args = args
+        self.act = act
+        self.fused = True          # norms / gate / activation quantisation through the fused prologue kernels
+        if gen is None:            # filled in by from_checkpoint
+            return
         d, hd = args.dim, args.head_dim
         qkv_n = (args.n_heads + 2 * args.n_kv_heads) * hd
         bf = lambda v: torch.tensor(v + [0.0] * (4 - len(v)), dtype=torch.bfloat16, device="cuda")
@@ -124,9 +135,26 @@ class Block:
         ones = lambda n: torch.ones(n, dtype=torch.bfloat16, device="cuda")
         self.attention_norm, self.ffn_norm = ones(d), ones(d)
         self.attn_sub_norm, self.ffn_sub_norm = ones(d), ones(args.ffn_dim)
-        self.args = args
-        self.act = act
-        self.fused = True          # norms / gate / activation quantisation through the fused prologue kernels
+
+    @classmethod
+    def from_checkpoint(cls, args: ModelArgs, dic: dict, layer_prefix: str, act: str = "int8") -> "Block":
+        """One block from the merged checkpoint dictionary (keys as model.py:110-116, 195, 275, 320-321):
+        the four format tensors of each linear are uploaded, repacked to P2 once and dropped."""
+        blk = cls(args, None, act)
+        d, hd = args.dim, args.head_dim
+        shapes = {"attention.wqkv": (d, (args.n_heads + 2 * args.n_kv_heads) * hd), "attention.wo": (args.n_heads * hd, d),
+                  "feed_forward.w13": (d, 2 * args.ffn_dim), "feed_forward.w2": (args.ffn_dim, d)}
+        for name, (k, n) in shapes.items():
+            key = f"{layer_prefix}.{name}"
+            parts = [dic[key + ".weight" + suffix].cuda()
+                     for suffix in ("_compressed_val", "_TileOffsets_global", "_TileOffsets_median", "_bitmap")]
+            packed = repack_weight(*parts, n, k)
+            torch.cuda.synchronize()       # the format tensors are released below; the repack must have read them
+            setattr(blk, name.split(".")[1], TernaryLinear(k, n, packed, dic[key + ".weight_scale"].cuda(), act))
+        norm = lambda name: dic[f"{layer_prefix}.{name}.weight"].to(device="cuda", dtype=torch.bfloat16).contiguous()
+        blk.attention_norm, blk.ffn_norm = norm("attention_norm"), norm("ffn_norm")
+        blk.attn_sub_norm, blk.ffn_sub_norm = norm("attention.attn_sub_norm"), norm("feed_forward.ffn_sub_norm")
+        return blk
 
     def _norm_linear(self, lin, x, weight, residual=None, glu=False):
         """[x + residual | relu(x1)^2 * x3] -> RMSNorm -> lin.  Returns (lin output, x + residual)."""
@@ -169,17 +197,19 @@ class Block:
             o = torch.empty((bsz, a.n_heads * a.head_dim), dtype=torch.bfloat16, device=x.device)
             lib.ternaspmm_rope_decode_attention(_p(qkv), _p(cos), _p(sin), _p(pos_idx), _p(cache_k), _p(cache_v), _p(o),
                                                 bsz, a.n_heads, a.n_kv_heads, a.head_dim, cache_k.shape[2],
-                                                a.head_dim ** -0.5, stream)
+                                                a.head_dim ** -0.5, int(a.rope_adjacent), stream)
         elif self.fused:
             lib = self.wqkv.lib
             stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
             q = torch.empty((bsz, a.n_heads, t, a.head_dim), dtype=torch.bfloat16, device=x.device)
             lib.ternaspmm_rope_kv_store(_p(qkv), _p(cos), _p(sin), _p(pos_idx), _p(q), _p(cache_k), _p(cache_v),
-                                        bsz, t, a.n_heads, a.n_kv_heads, a.head_dim, cache_k.shape[2], stream)
+                                        bsz, t, a.n_heads, a.n_kv_heads, a.head_dim, cache_k.shape[2],
+                                        int(a.rope_adjacent), stream)
         else:
             qkv = qkv.view(bsz, t, a.n_heads + 2 * a.n_kv_heads, a.head_dim).transpose(1, 2)
             q, k, v = qkv[:, :a.n_heads], qkv[:, a.n_heads:a.n_heads + a.n_kv_heads], qkv[:, a.n_heads + a.n_kv_heads:]
-            q, k = apply_rope(q, cos[None, None], sin[None, None]), apply_rope(k, cos[None, None], sin[None, None])
+            q = apply_rope(q, cos[None, None], sin[None, None], a.rope_adjacent)
+            k = apply_rope(k, cos[None, None], sin[None, None], a.rope_adjacent)
             cache_k.index_copy_(2, pos_idx, k)
             cache_v.index_copy_(2, pos_idx, v)
         if not one_token:
@@ -202,6 +232,17 @@ class Transformer:
         self.tok_embeddings = (torch.randn((args.vocab_size, args.dim), generator=gen, device="cuda") * 0.02).to(torch.bfloat16)
         self.layers: List[Block] = [Block(args, gen, act, p_zero) for _ in range(args.n_layers)]
         self.norm = torch.ones(args.dim, dtype=torch.bfloat16, device="cuda")
+
+    @classmethod
+    def from_checkpoint(cls, args: ModelArgs, dic: dict, act: str = "int8") -> "Transformer":
+        """The model of a converted checkpoint: `dic` is the ternary and the non-ternary file merged
+        (generate.py:69-71; ternainfer_amd.convert_utils.load_checkpoint)."""
+        model = cls.__new__(cls)
+        model.args = args
+        model.tok_embeddings = dic["tok_embeddings.weight"].to(device="cuda", dtype=torch.bfloat16).contiguous()
+        model.layers = [Block.from_checkpoint(args, dic, f"layers.{n}", act) for n in range(args.n_layers)]
+        model.norm = dic["norm.weight"].to(device="cuda", dtype=torch.bfloat16).contiguous()
+        return model
 
     def make_cache(self, bsz: int, max_seq: int):
         a = self.args

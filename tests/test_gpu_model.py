@@ -13,10 +13,13 @@ class DenseLinearCPU:
     """CPU stand-in for TernaryLinear: same activation quantisation, integer matmul in fp64,
     the decode-path epilogue (acc / s) * ws[g] with the reference's group rule."""
 
-    def __init__(self, lin, act):
+    def __init__(self, lin, act, w=None):
+        """`w`: the dense ternary matrix if the caller has it from elsewhere; else unpacked from lin.packed."""
         self.n, self.k, self.act = lin.n, lin.k, act
-        packed = lin.packed.cpu().numpy().view(np.uint32)
-        self.w = torch.from_numpy(O.unpack_p2(packed, lin.n, lin.k).astype(np.float64))
+        if w is None:
+            packed = lin.packed.cpu().numpy().view(np.uint32)
+            w = O.unpack_p2(packed, lin.n, lin.k)
+        self.w = torch.from_numpy(np.asarray(w).astype(np.float64))
         groups = O.ws_group_decode(np.arange(lin.n), lin.n, lin.ws_num)
         self.ws = lin.ws.float().cpu().double()[torch.from_numpy(groups)]
 
@@ -86,3 +89,43 @@ def test_toy_model_greedy_decode_graph_equals_eager():
     a, _, _ = greedy_decode(model, prompt, 12, use_graph=True)
     b, _, _ = greedy_decode(model, prompt, 12, use_graph=False)
     assert torch.equal(a, b)
+
+
+def test_converted_checkpoint_loads_and_matches_cpu_golden(tmp_path):
+    """fp32 state dict -> converter -> three files -> Transformer.from_checkpoint; the CPU golden is built
+    from the converter's int8 matrices (not from the packed buffers), so the loader and the repack are
+    inside the comparison."""
+    import copy
+    import ternainfer_amd as T
+    from ternainfer_amd.model import ModelArgs, Transformer
+    from tests.test_checkpoint_convert import toy_state
+    cfg = T.CheckpointShape(dim=256, n_heads=4, n_kv_heads=2, ffn_dim=384, n_layers=2)
+    args = ModelArgs(dim=256, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=512, ffn_dim=384)
+    state = toy_state(cfg, vocab=512, seed=21)
+    T.save_checkpoint(str(tmp_path), *T.convert_checkpoint(state, cfg, workers=2))
+    dic = T.load_checkpoint(str(tmp_path))
+    int8_model = T.convert_bitnet_checkpoint_to_int8(state, cfg)
+    model = Transformer.from_checkpoint(args, dic, act="int8")
+    tokens = torch.randint(0, args.vocab_size, (2, 24), generator=torch.Generator().manual_seed(22))
+    print("[case] toy model from a converted checkpoint", flush=True)
+    with torch.inference_mode():
+        got = model.forward(tokens.cuda(), model.make_cache(2, 32), torch.arange(24, device="cuda")).float().cpu()
+        twin = copy.copy(model)
+        twin.tok_embeddings = state["tok_embeddings.weight"].to(torch.bfloat16)
+        twin.norm = state["norm.weight"].to(torch.bfloat16)
+        twin.layers = []
+        names = {"wqkv": "attention.wqkv", "wo": "attention.wo", "w13": "feed_forward.w13", "w2": "feed_forward.w2"}
+        norms = {"attention_norm": "attention_norm", "ffn_norm": "ffn_norm", "attn_sub_norm": "attention.attn_sub_norm",
+                 "ffn_sub_norm": "feed_forward.ffn_sub_norm"}
+        for n, blk in enumerate(model.layers):
+            b = copy.copy(blk)
+            b.fused = False
+            for attr, key in names.items():
+                setattr(b, attr, DenseLinearCPU(getattr(blk, attr), "int8", int8_model[f"layers.{n}.{key}.weight"].numpy()))
+            for attr, key in norms.items():
+                setattr(b, attr, state[f"layers.{n}.{key}.weight"].to(torch.bfloat16))
+            twin.layers.append(b)
+        want = twin.forward(tokens, twin.make_cache(2, 32), torch.arange(24)).float()
+    err, ref = (got - want).abs().max().item(), want.abs().max().item()
+    assert err <= 3e-2 * ref, (err, ref)
+    assert torch.nn.functional.cosine_similarity(got.flatten(), want.flatten(), dim=0).item() > 0.999

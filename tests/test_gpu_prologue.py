@@ -136,8 +136,11 @@ def test_python_wrappers_feed_the_linear(lib):
 
 
 # ------------------------------------------------------------------ attention-side kernels
-@pytest.mark.parametrize("b,t,h,kv,d,s_max", [(1, 1, 20, 5, 128, 64), (2, 24, 4, 2, 64, 32), (3, 5, 20, 5, 128, 40)])
-def test_rope_kv_store(lib, b, t, h, kv, d, s_max):
+@pytest.mark.parametrize("adjacent", [0, 1])
+@pytest.mark.parametrize("b,t,h,kv,d,s_max", [(1, 1, 20, 5, 128, 64), (2, 24, 4, 2, 64, 32), (3, 5, 20, 5, 128, 40),
+                                              (2, 3, 4, 2, 24, 16)])
+def test_rope_kv_store(lib, b, t, h, kv, d, s_max, adjacent):
+    rope = O.rope_adjacent if adjacent else O.rope_rotate_half
     rng = np.random.default_rng(700 + b + t)
     qkv = make_bf16_activations(b * t, (h + 2 * kv) * d, 701 + t)
     pos = np.sort(rng.choice(s_max, t, replace=False)).astype(np.int64)
@@ -148,12 +151,13 @@ def test_rope_kv_store(lib, b, t, h, kv, d, s_max):
     cv = np.full((b, kv, s_max, d), sentinel, np.uint16)
     qd, ckd, cvd = torch.zeros((b, h, t, d), dtype=torch.int16, device="cuda"), _dev(ck), _dev(cv)
     xd, cd, sd, pd = _dev(qkv), _dev(cos), _dev(sin), _dev(pos)      # named: they must outlive the launch
+    print(f"[case] rope_kv_store b={b} t={t} h={h} kv={kv} d={d} adjacent={adjacent}", flush=True)
     lib.ternaspmm_rope_kv_store(_vp(xd), _vp(cd), _vp(sd), _vp(pd), _vp(qd), _vp(ckd), _vp(cvd), b, t, h, kv, d,
-                                s_max, None)
+                                s_max, adjacent, None)
     torch.cuda.synchronize()
     x = qkv.reshape(b, t, h + 2 * kv, d)
-    want_q = O.rope_rotate_half(x[:, :, :h], cos[None, :, None], sin[None, :, None]).transpose(0, 2, 1, 3)
-    want_k = O.rope_rotate_half(x[:, :, h:h + kv], cos[None, :, None], sin[None, :, None]).transpose(0, 2, 1, 3)
+    want_q = rope(x[:, :, :h], cos[None, :, None], sin[None, :, None]).transpose(0, 2, 1, 3)
+    want_k = rope(x[:, :, h:h + kv], cos[None, :, None], sin[None, :, None]).transpose(0, 2, 1, 3)
     want_v = x[:, :, h + kv:].transpose(0, 2, 1, 3)
     got_q = qd.cpu().numpy().view(np.uint16)
     got_k, got_v = ckd.cpu().numpy().view(np.uint16), cvd.cpu().numpy().view(np.uint16)
@@ -296,9 +300,10 @@ def test_fused_gate_prologue_linear(lib, n, f, ws_num):
     assert lib.bitlinear_TernaSpMM_packed_fused_glu(_vp(z), _vp(z), 1e-5, _vp(z), _vp(z), _vp(z), 1, None, None, 2, n, f, None) == 0
 
 
+@pytest.mark.parametrize("adjacent", [0, 1])
 @pytest.mark.parametrize("b,h,kv,d,s_max,n", [(1, 20, 5, 128, 256, 1), (1, 20, 5, 128, 256, 160), (8, 20, 5, 128, 300, 290),
                                               (2, 4, 2, 64, 40, 17), (1, 20, 5, 128, 600, 513)])
-def test_rope_decode_attention_equals_the_two_launches(lib, b, h, kv, d, s_max, n):
+def test_rope_decode_attention_equals_the_two_launches(lib, b, h, kv, d, s_max, n, adjacent):
     """One launch (RoPE + cache write + attention) against ternaspmm_rope_kv_store followed by
     ternaspmm_decode_attention on the same inputs: outputs and both caches bit-identical."""
     rng = np.random.default_rng(720 + n)
@@ -314,14 +319,14 @@ def test_rope_decode_attention_equals_the_two_launches(lib, b, h, kv, d, s_max, 
     ck1, cv1 = _dev(k0), _dev(v0)
     q1 = torch.zeros((b, h, 1, d), dtype=torch.int16, device="cuda")
     o1 = torch.zeros((b, h * d), dtype=torch.int16, device="cuda")
-    lib.ternaspmm_rope_kv_store(_vp(xd), _vp(cd), _vp(sd), _vp(pd), _vp(q1), _vp(ck1), _vp(cv1), b, 1, h, kv, d, s_max, None)
+    lib.ternaspmm_rope_kv_store(_vp(xd), _vp(cd), _vp(sd), _vp(pd), _vp(q1), _vp(ck1), _vp(cv1), b, 1, h, kv, d, s_max, adjacent, None)
     lib.ternaspmm_decode_attention(_vp(q1), _vp(ck1), _vp(cv1), _vp(pd), _vp(o1), b, h, kv, d, s_max, scale, None)
     # one launch
     ck2, cv2 = _dev(k0), _dev(v0)
     o2 = torch.zeros((b, h * d), dtype=torch.int16, device="cuda")
-    print(f"[case] rope + decode attention b={b} h={h} kv={kv} d={d} S={s_max} n={n}", flush=True)
+    print(f"[case] rope + decode attention b={b} h={h} kv={kv} d={d} S={s_max} n={n} adjacent={adjacent}", flush=True)
     lib.ternaspmm_rope_decode_attention(_vp(xd), _vp(cd), _vp(sd), _vp(pd), _vp(ck2), _vp(cv2), _vp(o2), b, h, kv, d, s_max,
-                                        scale, None)
+                                        scale, adjacent, None)
     torch.cuda.synchronize()
     assert torch.equal(ck1, ck2) and torch.equal(cv1, cv2)
     assert torch.equal(o1, o2)

@@ -139,6 +139,19 @@ def test_rope_and_attention_closed_forms():
     xf = O.bf16_bits_to_f32(x)
     want = np.concatenate([-xf[:, 32:], xf[:, :32]], axis=-1)
     assert (O.bf16_bits_to_f32(O.rope_rotate_half(x, zero, one)) == want).all()
+    # adjacent pairing: the same rotation after moving the pairs (2j, 2j+1) to (j, j+D/2); norm of a pair kept
+    rng = np.random.default_rng(86)
+    ang = rng.uniform(-3, 3, (3, 32)).astype(np.float32)
+    cos, sin = np.cos(ang), np.sin(ang)
+    de = np.concatenate([x[:, 0::2], x[:, 1::2]], axis=-1)
+    rot = O.rope_rotate_half(de, cos, sin)
+    back = np.empty_like(rot)
+    back[:, 0::2], back[:, 1::2] = rot[:, :32], rot[:, 32:]
+    assert (O.rope_adjacent(x, cos, sin) == back).all()
+    assert (O.rope_adjacent(x, one, zero) == x).all()
+    sw = np.empty_like(xf)
+    sw[:, 0::2], sw[:, 1::2] = -xf[:, 1::2], xf[:, 0::2]
+    assert (O.bf16_bits_to_f32(O.rope_adjacent(x, zero, one)) == sw).all()
     q = make_bf16_activations(2 * 4, 64, 82).reshape(2, 4, 64)
     k = make_bf16_activations(2 * 2 * 10, 64, 83).reshape(2, 2, 10, 64)
     v = np.broadcast_to(make_bf16_activations(1, 64, 84), (2, 2, 10, 64)).copy()
