@@ -211,6 +211,10 @@ void ternaspmm_rope_decode_attention(const terna_bf16* qkv, const float* cos, co
                                      terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
                                      int D, int S, float scale, int adjacent, terna_stream stream);
 
+/* Greedy sampling (torch.argmax over the logits, generate.py:283, 305): out[b] = index of the largest of
+ * x[b][0 .. V-1] (bf16 [B][V]; out int64 [B]); ties go to the lowest index, NaN never wins.  Only enqueues. */
+void ternaspmm_argmax_bf16(const terna_bf16* x, long long* out, int B, int V, terna_stream stream);
+
 /* Opt-in repack cache for unmodified call sites: with TERNASPMM_REPACK_CACHE=1 in the environment the
  * reference-format entry points above (bitlinear_TernaSpMM*, bitlinear_TernaSpMM_bf16*) keep a device-side P2
  * copy (N*K/4 bytes) of every weight they have seen -- keyed by device, the bitmap / sign / offset pointers and

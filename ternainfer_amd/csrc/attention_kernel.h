@@ -101,8 +101,11 @@ __global__ __launch_bounds__(256) void terna_rope_kv_store_kernel(
     }
 }
 
-// One workgroup per (sequence, head).  q bf16 [B][H][D]; keys / values of kv head h / (H/KV) at
-// slots 0 .. pos[0]; out bf16 [B][H*D].  Dynamic LDS: (S + 2048) floats.
+// One workgroup of NW waves per (sequence, head).  q bf16 [B][H][D]; keys / values of kv head
+// h / (H/KV) at slots 0 .. pos[0]; out bf16 [B][H*D].  Dynamic LDS: decode_attention_lds_bytes().
+// What the waves request up front covers 64 * NW slots of keys (four 16-slot tiles per wave) and
+// 4096 * NW / D slots of values, so with few workgroups on the chip (one per head) more waves mean
+// fewer dependent memory round trips.
 //   pass 1  q K^T on the matrix cores, 16 slots per MFMA tile, four tiles per wave requested up front
 //   pass 2  softmax over the scores in LDS
 //   pass 3  thread (slice, chunk): slots slice, slice+S', ... x 8 dimensions of V, eight rows in
@@ -114,19 +117,27 @@ __global__ __launch_bounds__(256) void terna_rope_kv_store_kernel(
 // -- and the new value row -- in place of cache slot pos[0], and the first workgroup of each kv
 // group writes the new key / value rows into the cache for the steps to come.  ADJACENT selects
 // the pairing of the rotation, as in terna_rope_kv_store_kernel.
-template <int D, bool ROPE, bool ADJACENT = false>
-__global__ __launch_bounds__(256) void terna_decode_attention_kernel(
+constexpr size_t decode_attention_lds_bytes(int D, int NW, int S)
+{
+    return (static_cast<size_t>(S) + (64 * NW / (D / 8)) * D + 64 * NW) * sizeof(float);
+}
+
+template <int D, bool ROPE, bool ADJACENT = false, int NW = 4>
+__global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
     const float* __restrict__ cosv, const float* __restrict__ sinv,
     const long long* __restrict__ pos, uint16_t* __restrict__ out, int H, int KV, int S, float scale)
 {
     static_assert(D == 64 || D == 128, "head dimension");
     constexpr int CH = D / 8;                    // 8-dimension chunks of a row
-    constexpr int SLICES = 256 / CH;
+    constexpr int NT = 64 * NW;
+    constexpr int SLICES = NT / CH;
+    constexpr int GROUPS = NT / D;               // threads per output dimension in the final sum
     extern __shared__ __align__(16) float lds[];
     float* part = lds;                           // [SLICES][D]
-    float* score = lds + SLICES * D;             // [S]
-    __shared__ float red[8];
+    float* part2 = lds + SLICES * D;             // [GROUPS][D]
+    float* score = part2 + GROUPS * D;           // [S]
+    __shared__ float red[2 * NW];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -152,7 +163,7 @@ __global__ __launch_bounds__(256) void terna_decode_attention_kernel(
     u32x4 kr[KT][NJ], vr[VU], qr[NJ];
 #pragma unroll
     for (int t = 0; t < KT; ++t) {
-        const int sk = 16 * (wave + 4 * t) + r16;
+        const int sk = 16 * (wave + NW * t) + r16;
         const uint16_t* kp = kbase + static_cast<size_t>(sk < S ? sk : 0) * D + 8 * kblk;
 #pragma unroll
         for (int jj = 0; jj < NJ; ++jj) kr[t][jj] = *reinterpret_cast<const u32x4*>(kp + 32 * jj);
@@ -275,8 +286,8 @@ __global__ __launch_bounds__(256) void terna_decode_attention_kernel(
     const int tiles = (n + 15) >> 4;
 #pragma unroll
     for (int t = 0; t < KT; ++t)
-        if (wave + 4 * t < tiles) score_tile(wave + 4 * t, kr[t]);
-    for (int tile = wave + 4 * KT; tile < tiles; tile += 4) {     // beyond 256 slots: plain loop
+        if (wave + NW * t < tiles) score_tile(wave + NW * t, kr[t]);
+    for (int tile = wave + NW * KT; tile < tiles; tile += NW) {   // beyond 64 * NW slots: plain loop
         u32x4 k[NJ];
         const int sk = 16 * tile + r16;
         const uint16_t* kp = kbase + static_cast<size_t>(sk < S ? sk : 0) * D + 8 * kblk;
@@ -287,19 +298,23 @@ __global__ __launch_bounds__(256) void terna_decode_attention_kernel(
     mx = wave_max(mx);
     if (lane == 0) red[wave] = mx;
     __syncthreads();
-    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    mx = red[0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) mx = fmaxf(mx, red[w]);
 
     // ---- pass 2: softmax numerators and their sum (each thread revisits the slots it scored)
     float sum = 0.0f;
-    for (int s = tid; s < n; s += 256) {
+    for (int s = tid; s < n; s += NT) {
         const float p = __expf(score[s] - mx);
         score[s] = p;
         sum += p;
     }
     sum = wave_sum(sum);
-    if (lane == 0) red[4 + wave] = sum;
+    if (lane == 0) red[NW + wave] = sum;
     __syncthreads();
-    sum = (red[4] + red[5]) + (red[6] + red[7]);
+    sum = red[NW];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) sum += red[NW + w];
 
     // ---- pass 3: weighted sum of the value rows, VU rows per round (the first round is already here)
     float acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
@@ -329,10 +344,18 @@ __global__ __launch_bounds__(256) void terna_decode_attention_kernel(
 #pragma unroll
     for (int e = 0; e < 8; ++e) part[slice * D + chunk * 8 + e] = acc[e];
     __syncthreads();
+    {                                            // GROUPS threads per dimension, SLICES / GROUPS slices each
+        const int d = tid % D, grp = tid / D;
+        float o = 0.0f;
+#pragma unroll
+        for (int sl = 0; sl < SLICES / GROUPS; ++sl) o += part[(grp * (SLICES / GROUPS) + sl) * D + d];
+        part2[grp * D + d] = o;
+    }
+    __syncthreads();
     if (tid < D) {
         float o = 0.0f;
 #pragma unroll
-        for (int sl = 0; sl < SLICES; ++sl) o += part[sl * D + tid];
+        for (int grp = 0; grp < GROUPS; ++grp) o += part2[grp * D + tid];
         out[(static_cast<size_t>(b) * H + h) * D + tid] = float_to_bf16_bits(o / sum);
     }
 }

@@ -16,6 +16,7 @@
 #include "norm_quant_kernel.h"
 #include "decode_fused_kernel.h"
 #include "attention_kernel.h"
+#include "argmax_kernel.h"
 #include "format_host.h"
 
 using namespace terna;
@@ -375,6 +376,57 @@ __global__ void sleep_kernel(long long ticks)
     while (wall_clock64() - start < ticks) __builtin_amdgcn_s_sleep(8);
 }
 
+// Waves per workgroup of the decode attention: with one workgroup per (sequence, head) and few of them
+// on the chip, wider workgroups request more of the cache up front.  TERNASPMM_ATTN_WAVES=4|8 forces one
+// (tuning aid).  Both entry points use the same rule, so their results stay bit-identical.
+int attention_waves(int B, int H)
+{
+    static const int forced = [] {
+        const char* v = std::getenv("TERNASPMM_ATTN_WAVES");
+        const int w = v ? std::atoi(v) : 0;
+        return (w == 4 || w == 8) ? w : 0;
+    }();
+    if (forced) return forced;
+    return static_cast<long>(B) * H <= 512 ? 8 : 4;
+}
+
+template <int D, bool ROPE, bool ADJ, int NW>
+void launch_attention_as(const uint16_t* q, uint16_t* ck, uint16_t* cv, const float* cos, const float* sin,
+                                const long long* pos, uint16_t* out, int B, int H, int KV, int S, float scale,
+                                hipStream_t st)
+{
+    auto kernel = terna_decode_attention_kernel<D, ROPE, ADJ, NW>;
+    const size_t lds = decode_attention_lds_bytes(D, NW, S);
+    if (lds > 64 * 1024) allow_dynamic_lds(kernel, 160 * 1024, "hipFuncSetAttribute(decode attention)", __LINE__);
+    kernel<<<dim3(B * H), dim3(64 * NW), lds, st>>>(q, ck, cv, cos, sin, pos, out, H, KV, S, scale);
+}
+
+template <bool ROPE, bool ADJ>
+void launch_attention(const uint16_t* q, uint16_t* ck, uint16_t* cv, const float* cos, const float* sin,
+                             const long long* pos, uint16_t* out, int B, int H, int KV, int D, int S, float scale,
+                             hipStream_t st)
+{
+    const int nw = attention_waves(B, H);
+#define TERNA_ATTN(DIM, NWAVES) launch_attention_as<DIM, ROPE, ADJ, NWAVES>(q, ck, cv, cos, sin, pos, out, B, H, KV, S, scale, st)
+    if (D == 128) {
+        if (nw == 8) TERNA_ATTN(128, 8);
+        else TERNA_ATTN(128, 4);
+    } else {
+        if (nw == 8) TERNA_ATTN(64, 8);
+        else TERNA_ATTN(64, 4);
+    }
+#undef TERNA_ATTN
+}
+
+bool attention_args_ok(const char* who, int B, int H, int KV, int D, int S)
+{
+    if (B < 1 || H < 1 || KV < 1 || H % KV != 0 || (D != 64 && D != 128) || S < 1 || S > 8192) {
+        std::fprintf(stderr, "%s: unsupported arguments (H=%d KV=%d D=%d S=%d)\n", who, H, KV, D, S);
+        return false;
+    }
+    return true;
+}
+
 }  // namespace
 
 extern "C" {
@@ -677,18 +729,10 @@ void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, 
                                 const long long* pos, terna_bf16* out, int B, int H, int KV, int D, int S,
                                 float scale, terna_stream stream)
 {
-    if (B < 1 || H < 1 || KV < 1 || H % KV != 0 || (D != 64 && D != 128) || S < 1 || S > 8192) {
-        std::fprintf(stderr, "ternaspmm_decode_attention: unsupported arguments (H=%d KV=%d D=%d S=%d)\n", H, KV, D, S);
-        return;
-    }
-    const size_t lds = (static_cast<size_t>(S) + (256 / (D / 8)) * D) * sizeof(float);
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    uint16_t* ck = const_cast<uint16_t*>(cache_k);      // the kernel writes the caches only in its ROPE variant
-    uint16_t* cv = const_cast<uint16_t*>(cache_v);
-    if (D == 128)
-        terna_decode_attention_kernel<128, false><<<dim3(B * H), dim3(256), lds, st>>>(q, ck, cv, nullptr, nullptr, pos, out, H, KV, S, scale);
-    else
-        terna_decode_attention_kernel<64, false><<<dim3(B * H), dim3(256), lds, st>>>(q, ck, cv, nullptr, nullptr, pos, out, H, KV, S, scale);
+    if (!attention_args_ok("ternaspmm_decode_attention", B, H, KV, D, S)) return;
+    // the kernel writes the caches only in its ROPE variant
+    launch_attention<false, false>(q, const_cast<uint16_t*>(cache_k), const_cast<uint16_t*>(cache_v), nullptr, nullptr, pos,
+                                   out, B, H, KV, D, S, scale, static_cast<hipStream_t>(stream));
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_decode_attention", e, __LINE__);
 }
@@ -697,25 +741,23 @@ void ternaspmm_rope_decode_attention(const terna_bf16* qkv, const float* cos, co
                                      terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
                                      int D, int S, float scale, int adjacent, terna_stream stream)
 {
-    if (B < 1 || H < 1 || KV < 1 || H % KV != 0 || (D != 64 && D != 128) || S < 1 || S > 8192) {
-        std::fprintf(stderr, "ternaspmm_rope_decode_attention: unsupported arguments (H=%d KV=%d D=%d S=%d)\n", H, KV, D, S);
-        return;
-    }
-    const size_t lds = (static_cast<size_t>(S) + (256 / (D / 8)) * D) * sizeof(float);
+    if (!attention_args_ok("ternaspmm_rope_decode_attention", B, H, KV, D, S)) return;
     hipStream_t st = static_cast<hipStream_t>(stream);
-#define TERNA_ROPE_ATTN(DIM, ADJ)                                                                                  \
-    terna_decode_attention_kernel<DIM, true, ADJ><<<dim3(B * H), dim3(256), lds, st>>>(qkv, cache_k, cache_v, cos, sin, \
-                                                                                        pos, out, H, KV, S, scale)
-    if (D == 128) {
-        if (adjacent) TERNA_ROPE_ATTN(128, true);
-        else TERNA_ROPE_ATTN(128, false);
-    } else {
-        if (adjacent) TERNA_ROPE_ATTN(64, true);
-        else TERNA_ROPE_ATTN(64, false);
-    }
-#undef TERNA_ROPE_ATTN
+    if (adjacent) launch_attention<true, true>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, st);
+    else launch_attention<true, false>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, st);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_rope_decode_attention", e, __LINE__);
+}
+
+void ternaspmm_argmax_bf16(const terna_bf16* x, long long* out, int B, int V, terna_stream stream)
+{
+    if (B < 1 || V < 1) {
+        std::fprintf(stderr, "ternaspmm_argmax_bf16: unsupported arguments (B=%d V=%d)\n", B, V);
+        return;
+    }
+    terna_argmax_bf16_kernel<<<dim3(B), dim3(kArgmaxThreads), 0, static_cast<hipStream_t>(stream)>>>(x, out, V);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_argmax_bf16", e, __LINE__);
 }
 
 void ternaspmm_repack_cache_clear(void)

@@ -10,6 +10,7 @@ and streams here; all arithmetic happens in libternaspmm.so.
 from __future__ import annotations
 
 import ctypes
+from typing import Optional
 
 import torch
 from torch import nn
@@ -203,6 +204,19 @@ def relu2_mul_rmsnorm_quant(x13, weight, eps, quant=True):
     y = torch.empty((m, f), dtype=torch.bfloat16, device=x13.device)
     lib.ternaspmm_relu2_mul_rmsnorm_quant(_p(x13), _p(weight), float(eps), _p(y), None, None, m, f, stream)
     return y
+
+
+def argmax_rows(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Greedy sampling: index of the largest logit per row of a bf16 [B, V] tensor -> int64 [B, 1]
+    (torch.argmax(logits, dim=-1), generate.py:283; ties to the lowest index).  `out`, if given, is
+    an int64 tensor of B elements that receives the result in place."""
+    assert logits.dtype == torch.bfloat16 and logits.dim() == 2 and logits.is_contiguous()
+    b, v = logits.shape
+    if out is None:
+        out = torch.empty((b, 1), dtype=torch.int64, device=logits.device)
+    assert out.dtype == torch.int64 and out.numel() == b and out.is_contiguous()
+    _lib.load().ternaspmm_argmax_bf16(_p(logits), _p(out), b, v, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    return out
 
 
 class _CompressedWeight(nn.Module):

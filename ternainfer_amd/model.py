@@ -21,7 +21,7 @@ import torch
 from torch.nn import functional as F
 
 from . import _lib
-from .linear import (relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant, repack_weight, rmsnorm_linear_packed,
+from .linear import (argmax_rows, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant, repack_weight, rmsnorm_linear_packed,
                      rmsnorm_quant)
 
 
@@ -190,7 +190,7 @@ class Block:
         t = x.shape[0] // bsz
         qkv, x = self._norm_linear(self.wqkv, x, self.attention_norm, residual=pending)
         rep = a.n_heads // a.n_kv_heads
-        one_token = self.fused and t == 1 and a.head_dim in (64, 128) and cache_k.shape[2] <= 8192
+        one_token = mask is None           # the caller's rule: fused, one new token, a head size the kernel has
         if one_token:                       # RoPE, cache write and attention over the cache prefix: one launch
             lib = self.wqkv.lib
             stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -244,6 +244,17 @@ class Transformer:
         model.norm = dic["norm.weight"].to(device="cuda", dtype=torch.bfloat16).contiguous()
         return model
 
+    def rope_tables(self, max_seq: int, dev):
+        """cos / sin of every (cache slot, rotary pair): fp32 [max_seq, head_dim / 2], built once per length."""
+        key = (max_seq, str(dev))
+        tables = getattr(self, "_rope_tables", None)
+        if tables is None or tables[0] != key:
+            a = self.args
+            inv = 1.0 / (a.rope_theta ** (torch.arange(0, a.head_dim, 2, device=dev, dtype=torch.float32) / a.head_dim))
+            ang = torch.arange(max_seq, device=dev, dtype=torch.float32)[:, None] * inv[None, :]
+            self._rope_tables = tables = (key, ang.cos().contiguous(), ang.sin().contiguous())
+        return tables[1], tables[2]
+
     def make_cache(self, bsz: int, max_seq: int):
         a = self.args
         shape = (bsz, a.n_kv_heads, max_seq, a.head_dim)
@@ -258,17 +269,23 @@ class Transformer:
         bsz, t = tokens.shape
         max_seq = cache[0][0].shape[2]
         dev = tokens.device
-        inv = 1.0 / (a.rope_theta ** (torch.arange(0, a.head_dim, 2, device=dev, dtype=torch.float32) / a.head_dim))
-        ang = pos_idx.float()[:, None] * inv[None, :]
-        cos, sin = ang.cos().contiguous(), ang.sin().contiguous()            # fp32 [T, head_dim / 2]
-        # causal over cache slots: new token at slot p sees slots <= p
-        mask = torch.arange(max_seq, device=dev)[None, :] <= pos_idx[:, None]
+        cos_all, sin_all = self.rope_tables(max_seq, dev)
+        cos, sin = cos_all.index_select(0, pos_idx), sin_all.index_select(0, pos_idx)     # fp32 [T, head_dim / 2]
+        mask = None
+        one_launch_attention = self.layers[0].fused and t == 1 and a.head_dim in (64, 128) and max_seq <= 8192
+        if not one_launch_attention:
+            # causal over cache slots: new token at slot p sees slots <= p
+            mask = (torch.arange(max_seq, device=dev)[None, :] <= pos_idx[:, None])[None, None]
         x = self.tok_embeddings[tokens.reshape(-1)]
         pending = None
         for layer, (ck, cv) in zip(self.layers, cache):
-            x, pending = layer.forward(x, pending, ck, cv, pos_idx, cos, sin, mask[None, None])
-        x = x + pending
-        x = rms_norm(x.view(bsz, t, a.dim)[:, -1], self.norm, a.norm_eps)
+            x, pending = layer.forward(x, pending, ck, cv, pos_idx, cos, sin, mask)
+        if t > 1:                                                             # only the last new token feeds the head
+            x, pending = x.view(bsz, t, a.dim)[:, -1].contiguous(), pending.view(bsz, t, a.dim)[:, -1].contiguous()
+        if self.layers[0].fused and x.is_cuda:                                # last residual add + final norm: one launch
+            x, _ = rmsnorm_quant(x, self.norm, a.norm_eps, residual=pending, quant=False)
+        else:
+            x = rms_norm(x + pending, self.norm, a.norm_eps)
         return F.linear(x, self.tok_embeddings)                               # tied LM head (model.py:367)
 
 
@@ -282,33 +299,31 @@ def greedy_decode(model: Transformer, prompt: torch.Tensor, gen_tokens: int, use
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
     ev[0].record()
     logits = model.forward(prompt, cache, torch.arange(plen, device="cuda"))
-    tok = logits.argmax(dim=-1, keepdim=True)
+    tok = argmax_rows(logits.contiguous())                                    # int64 [B, 1]
     ev[1].record()
-    pos = torch.full((1,), plen, dtype=torch.int64, device="cuda")
+    counters = torch.tensor([plen, 0], dtype=torch.int64, device="cuda")      # cache slot of the next token, step number
+    pos, step_idx = counters[0:1], counters[1:2]
     out = torch.empty((bsz, gen_tokens), dtype=torch.int64, device="cuda")
-    step_idx = torch.zeros(1, dtype=torch.int64, device="cuda")
 
     def step():
         out.index_copy_(1, step_idx, tok)
-        nxt = model.forward(tok, cache, pos).argmax(dim=-1, keepdim=True)
-        tok.copy_(nxt)
-        pos.add_(1)
-        step_idx.add_(1)
+        argmax_rows(model.forward(tok, cache, pos), out=tok)                  # the forward has read tok by then
+        counters.add_(1)
 
     graph = None
     if use_graph:
         # warm up on a side stream (allocator, lazy inits), then restore the state and capture
-        snap = (tok.clone(), pos.clone(), step_idx.clone())
+        snap = (tok.clone(), counters.clone())
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             step()
         torch.cuda.current_stream().wait_stream(side)
-        tok.copy_(snap[0]); pos.copy_(snap[1]); step_idx.copy_(snap[2])
+        tok.copy_(snap[0]); counters.copy_(snap[1])
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             step()
-        tok.copy_(snap[0]); pos.copy_(snap[1]); step_idx.copy_(snap[2])
+        tok.copy_(snap[0]); counters.copy_(snap[1])
     torch.cuda.synchronize()
     ev[2].record()
     for _ in range(gen_tokens):

@@ -135,6 +135,31 @@ def test_python_wrappers_feed_the_linear(lib):
     assert (out.view(torch.int16).cpu().numpy().view(np.uint16) == want).all()
 
 
+@pytest.mark.parametrize("b,v", [(1, 128256), (8, 128256), (3, 1000), (2, 1003), (1, 5), (4, 8192)])
+def test_argmax_rows(lib, b, v):
+    import ternainfer_amd as T
+    """First index of the row maximum, also with ties, -inf entries, NaNs and rows that are not
+    16-byte aligned (V % 8 != 0)."""
+    rng = np.random.default_rng(900 + v + b)
+    x = O.f32_to_bf16_bits(rng.standard_normal((b, v)).astype(np.float32))       # bf16 rounding makes ties common
+    xf = O.bf16_bits_to_f32(x)
+    if v >= 1000:
+        xf[0, 17] = xf[0, 900] = 9.0                                             # a tie: the lower index wins
+        xf[-1, 3] = -np.inf
+        xf[-1, 11] = np.nan                                                      # never selected
+        x = O.f32_to_bf16_bits(xf)
+        xf = O.bf16_bits_to_f32(x)
+    want = np.array([int(np.flatnonzero(r == np.nanmax(r))[0]) for r in xf], np.int64)
+    xd = _dev(x)
+    od = torch.full((b,), -1, dtype=torch.int64, device="cuda")
+    print(f"[case] argmax b={b} v={v}", flush=True)
+    lib.ternaspmm_argmax_bf16(_vp(xd), _vp(od), b, v, None)
+    torch.cuda.synchronize()
+    assert (od.cpu().numpy() == want).all()
+    got = T.argmax_rows(xd.view(torch.bfloat16))
+    assert got.shape == (b, 1) and (got.cpu().numpy().ravel() == want).all()
+
+
 # ------------------------------------------------------------------ attention-side kernels
 @pytest.mark.parametrize("adjacent", [0, 1])
 @pytest.mark.parametrize("b,t,h,kv,d,s_max", [(1, 1, 20, 5, 128, 64), (2, 24, 4, 2, 64, 32), (3, 5, 20, 5, 128, 40),
