@@ -20,7 +20,12 @@
 //   B  rows' sums: the lanes that share a row (shuffles), then the waves in LDS  -- barrier 1
 //   C  y -> registers, max |y| per row, same reduction                      -- barrier 2
 //   D  per tile: quantise, int8 slab -> wave-private LDS -> operand order, MFMA
-//   E  cross-wave sum of the accumulators + epilogue (wave 0)               -- barrier 3
+//   E  cross-wave sum of the accumulators + epilogue (wave b finishes band b) -- barrier 3
+//
+// NB = bands of W per workgroup.  The prologue is repeated by every workgroup, so a matrix with
+// more bands than the chip has CUs (gate+up: 864) would repeat it once per *round* of workgroups
+// on every CU; with NB bands per workgroup the grid fits one round, the prologue runs once per CU
+// and its result feeds NB accumulators.
 #pragma once
 
 #include "decode_packed_kernel.h"
@@ -60,7 +65,7 @@ template <> struct RowPiece<1> {
 // repeats, costs in proportion to the batch rows that exist, not to the 16 the MFMA tile has.
 enum FusedMode { FUSED_PLAIN, FUSED_RESIDUAL, FUSED_GLU };
 
-template <int WAVES, int TMAX, int MODE, int MP>
+template <int WAVES, int TMAX, int MODE, int MP, int NB = 1>
 __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, uint16_t* __restrict__ sum_out,
     const uint16_t* __restrict__ norm_w, float eps, const uint32_t* __restrict__ packed,
@@ -70,7 +75,8 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
     using XQ = XSlab<int8_t>;
     using Piece = RowPiece<MP>;
     constexpr int LPR = 64 / MP;                     // lanes per row
-    __shared__ i32x4 red[WAVES][64];
+    static_assert(NB <= WAVES, "one finishing wave per band");
+    __shared__ i32x4 red[WAVES][NB][64];
     __shared__ __align__(16) uint8_t slab_all[WAVES][16 * XQ::kPitch];
     __shared__ __align__(16) float stat[2][16][WAVES];
     __shared__ float s_row[16];
@@ -78,24 +84,26 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int band = blockIdx.x;
+    const int band0 = blockIdx.x * NB;               // first of this workgroup's NB bands
     const int ktiles = K >> 6;
     const int i = lane & 15, g = lane >> 4;          // operand coordinates: weight row / batch row i, 16-column group g
     const int row = lane / LPR, cl = (lane % LPR) * MP;   // load coordinates: batch row, first of MP columns
     const bool row_ok = row < M;
-    const bool writer = band == 0;                   // the workgroup that publishes h, q and s
+    const bool writer = blockIdx.x == 0;             // the workgroup that publishes h, q and s
     constexpr bool RES = MODE != FUSED_PLAIN;        // a second operand: the residual, or x3 of the gate
     const size_t pitch = MODE == FUSED_GLU ? 2 * static_cast<size_t>(K) : K;
     const uint16_t* second = MODE == FUSED_GLU ? x + K : residual;
 
     // ---- phase A: request everything
-    uint32_t wword[TMAX];
+    uint32_t wword[NB][TMAX];
     Piece xr[TMAX], rr[TMAX], nw[TMAX];
 #pragma unroll
     for (int t = 0; t < TMAX; ++t) {
         const int j = wave + WAVES * t;
         const bool valid = j < ktiles;
-        wword[t] = valid ? packed[(static_cast<size_t>(band) * ktiles + j) * 64 + i * 4 + g] : 0u;
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+            wword[b][t] = valid ? packed[(static_cast<size_t>(band0 + b) * ktiles + j) * 64 + i * 4 + g] : 0u;
         const size_t off = static_cast<size_t>(row_ok ? row : 0) * pitch + (valid ? j : 0) * 64 + cl;
         if (valid && row_ok) {
             xr[t].load(x + off);
@@ -110,9 +118,10 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
         const int j = wave + WAVES * t;
         nw[t].load(norm_w + (j < ktiles ? j : 0) * 64 + cl);
     }
-    // wave 0 finishes the band: its weight-group scales are requested now, converted at the very end
+    // wave b finishes band b: its weight-group scales are requested now, converted at the very end
     const Epilogue ep{nullptr, ws, nullptr, ws_num, EP_I8_DECODE};
-    EpilogueRaw eraw = load_epilogue_raw_scales(ep, band * 16 + 4 * g, N);
+    const int my_band = band0 + (wave < NB ? wave : 0);
+    EpilogueRaw eraw = load_epilogue_raw_scales(ep, my_band * 16 + 4 * g, N);
     // this wave's LDS slot: rows the batch does not have stay zero
     uint8_t* slab = slab_all[wave];
     for (int o = lane * 16; o < 16 * XQ::kPitch; o += 64 * 16) *reinterpret_cast<u32x4*>(slab + o) = u32x4{0u, 0u, 0u, 0u};
@@ -191,7 +200,9 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
     }
 
     // ---- phase D: quantise a tile, turn it into operand order through the wave's LDS slot, multiply
-    i32x4 acc = {0, 0, 0, 0};
+    i32x4 acc[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) acc[b] = i32x4{0, 0, 0, 0};
 #pragma unroll
     for (int t = 0; t < TMAX; ++t) {
         const int j = wave + WAVES * t;
@@ -224,19 +235,22 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
                 }
             }
             const i32x4 bq = __builtin_bit_cast(i32x4, *reinterpret_cast<const u32x4*>(slab + i * XQ::kPitch + g * 16));
-            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(expand_word_i8(wword[t]), bq, acc, 0, 0, 0);
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+                acc[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(expand_word_i8(wword[b][t]), bq, acc[b], 0, 0, 0);
         }
     }
 
     // ---- phase E: cross-wave sum in wave order + the decode epilogue (lane: batch row i, output rows 4g .. 4g+3)
-    red[wave][lane] = acc;
-    __syncthreads();
-    if (wave == 0) {
-        i32x4 sum = red[0][lane];
 #pragma unroll
-        for (int w = 1; w < WAVES; ++w) sum += red[w][lane];
+    for (int b = 0; b < NB; ++b) red[wave][b][lane] = acc[b];
+    __syncthreads();
+    if (wave < NB) {
+        i32x4 sum = red[0][wave][lane];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) sum += red[w][wave][lane];
         if (i < M) {
-            const int n0 = band * 16 + 4 * g;
+            const int n0 = my_band * 16 + 4 * g;
             EpilogueRegs e = finish_epilogue(ep, eraw);
             e.s = s_row[i];
             uint16_t o[4];

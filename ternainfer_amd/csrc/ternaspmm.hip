@@ -659,30 +659,51 @@ static int launch_decode_fused(int mode, const terna_bf16* x, const terna_bf16* 
 {
     if (!shape_ok(M, N, K) || ws_num < 1 || M > 16) return 0;
     const int ktiles = K / 64;
-    const bool wide = N / 16 <= 256;                  // same split as the unfused small-M kernel
+    const int bands = N / 16;
+    const bool wide = bands <= 256;                  // same split as the unfused small-M kernel
     const uint32_t* p = static_cast<const uint32_t*>(packed);
-    const dim3 grid(N / 16);
-#define TERNA_FUSED(WAVES, TMAX, MODE, MP)                                                                         \
-    terna_decode_fused_kernel<WAVES, TMAX, MODE, MP><<<grid, dim3(WAVES * 64), 0, st>>>(                           \
+    // More bands than CUs: four bands per workgroup, so that the grid is one round and the prologue runs once
+    // per CU.  TERNASPMM_FUSED_BANDS=1 switches that off, TERNASPMM_FUSED_BANDS_WAVES=8 picks the 8-wave
+    // variant of it (tuning aids).
+    static const int forced_nb = [] {
+        const char* v = std::getenv("TERNASPMM_FUSED_BANDS");
+        return v ? std::atoi(v) : 0;
+    }();
+    static const int nb_waves = [] {
+        const char* v = std::getenv("TERNASPMM_FUSED_BANDS_WAVES");
+        return v && std::atoi(v) == 8 ? 8 : 16;
+    }();
+    const bool multi = forced_nb != 1 && bands > 256 && bands % 4 == 0 && mode != FUSED_GLU;
+    const bool multi16 = multi && nb_waves == 16 && ktiles <= 16 * 3;
+    const bool multi8 = multi && !multi16 && ktiles <= 8 * 5;
+    const dim3 grid(multi16 || multi8 ? bands / 4 : bands);
+#define TERNA_FUSED(WAVES, TMAX, MODE, MP, NB)                                                                     \
+    terna_decode_fused_kernel<WAVES, TMAX, MODE, MP, NB><<<grid, dim3(WAVES * 64), 0, st>>>(                       \
         x, residual, sum_out, norm_weight, eps, p, out, ws, ws_num, xq_out, s_out, M, N, K)
-#define TERNA_FUSED_M(WAVES, TMAX, MODE)                                                                           \
+#define TERNA_FUSED_M(WAVES, TMAX, MODE, NB)                                                                       \
     do {                                                                                                           \
-        if (M == 1) TERNA_FUSED(WAVES, TMAX, MODE, 1);                                                             \
-        else if (M <= 8) TERNA_FUSED(WAVES, TMAX, MODE, 8);                                                        \
-        else TERNA_FUSED(WAVES, TMAX, MODE, 16);                                                                   \
+        if (M == 1) TERNA_FUSED(WAVES, TMAX, MODE, 1, NB);                                                         \
+        else if (M <= 8) TERNA_FUSED(WAVES, TMAX, MODE, 8, NB);                                                    \
+        else TERNA_FUSED(WAVES, TMAX, MODE, 16, NB);                                                               \
     } while (0)
     if (mode == FUSED_GLU) {
         // long K (the down projection): only the single-row variant, whose per-lane state is tiny
         if (M != 1 || !wide || ktiles > 16 * 7) return 0;
-        TERNA_FUSED(16, 7, FUSED_GLU, 1);
+        TERNA_FUSED(16, 7, FUSED_GLU, 1, 1);
+    } else if (multi16) {
+        if (mode == FUSED_RESIDUAL) TERNA_FUSED_M(16, 3, FUSED_RESIDUAL, 4);
+        else TERNA_FUSED_M(16, 3, FUSED_PLAIN, 4);
+    } else if (multi8) {
+        if (mode == FUSED_RESIDUAL) TERNA_FUSED_M(8, 5, FUSED_RESIDUAL, 4);
+        else TERNA_FUSED_M(8, 5, FUSED_PLAIN, 4);
     } else if (wide) {
         if (ktiles > 16 * 3) return 0;
-        if (mode == FUSED_RESIDUAL) TERNA_FUSED_M(16, 3, FUSED_RESIDUAL);
-        else TERNA_FUSED_M(16, 3, FUSED_PLAIN);
+        if (mode == FUSED_RESIDUAL) TERNA_FUSED_M(16, 3, FUSED_RESIDUAL, 1);
+        else TERNA_FUSED_M(16, 3, FUSED_PLAIN, 1);
     } else {
         if (ktiles > 8 * 5) return 0;
-        if (mode == FUSED_RESIDUAL) TERNA_FUSED_M(8, 5, FUSED_RESIDUAL);
-        else TERNA_FUSED_M(8, 5, FUSED_PLAIN);
+        if (mode == FUSED_RESIDUAL) TERNA_FUSED_M(8, 5, FUSED_RESIDUAL, 1);
+        else TERNA_FUSED_M(8, 5, FUSED_PLAIN, 1);
     }
 #undef TERNA_FUSED_M
 #undef TERNA_FUSED
