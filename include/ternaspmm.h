@@ -197,19 +197,26 @@ int bitlinear_TernaSpMM_packed_fused_glu(const terna_bf16* x13, const terna_bf16
  *
  * ternaspmm_decode_attention: one new token per sequence.  q bf16 [B][H][D]; head h reads kv head
  * h / (H/KV) at slots 0 .. pos[0]; out bf16 [B][H*D] = softmax(scale * q K^T) V.  D is 64 or 128,
- * S <= 8192.  Both only enqueue. */
+ * S <= 8192.  Both only enqueue.
+ *
+ * `workspace` (may be NULL): device memory of ternaspmm_attention_workspace_bytes(B, H, D) bytes, zero-filled by
+ * the caller once before its first use.  With it the cache prefix of every head is split over up to 8 workgroups
+ * (one CU streams a prefix at a few tens of GB/s, so few heads on the chip are bound by that); each leaves a partial
+ * result in the workspace and the last to arrive merges them in a fixed order.  The kernel leaves the counters at
+ * zero, so the same workspace serves every later call; calls that share one workspace must not overlap. */
+long long ternaspmm_attention_workspace_bytes(int B, int H, int D);
 void ternaspmm_rope_kv_store(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
                              terna_bf16* q_out, terna_bf16* cache_k, terna_bf16* cache_v, int B, int T, int H,
                              int KV, int D, int S, int adjacent, terna_stream stream);
 void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
                                 const long long* pos, terna_bf16* out, int B, int H, int KV, int D, int S,
-                                float scale, terna_stream stream);
+                                float scale, void* workspace, terna_stream stream);
 /* Both of the above in one launch for T = 1: qkv bf16 [B][(H + 2*KV)*D], cos / sin fp32 [D/2] of the new
  * token's position; writes slot pos[0] of the caches and out.  Results are bit-identical to
  * ternaspmm_rope_kv_store followed by ternaspmm_decode_attention. */
 void ternaspmm_rope_decode_attention(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
                                      terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
-                                     int D, int S, float scale, int adjacent, terna_stream stream);
+                                     int D, int S, float scale, int adjacent, void* workspace, terna_stream stream);
 
 /* Greedy sampling (torch.argmax over the logits, generate.py:283, 305): out[b] = index of the largest of
  * x[b][0 .. V-1] (bf16 [B][V]; out int64 [B]); ties go to the lowest index, NaN never wins.  Only enqueues. */

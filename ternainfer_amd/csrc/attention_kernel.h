@@ -117,16 +117,26 @@ __global__ __launch_bounds__(256) void terna_rope_kv_store_kernel(
 // -- and the new value row -- in place of cache slot pos[0], and the first workgroup of each kv
 // group writes the new key / value rows into the cache for the steps to come.  ADJACENT selects
 // the pairing of the rotation, as in terna_rope_kv_store_kernel.
+//
+// Split over the cache (SP = gridDim.y > 1): one CU streams a cache prefix at a few tens of GB/s, so
+// with few heads on the chip the launch is bound by that.  Workgroup (b, h, sp) then takes the
+// 16-slot tiles sp, sp + SP, ... and leaves its unnormalised result, its score maximum and its
+// sum of numerators in `partial` ([B*H][SP][D + 2] floats); the last of a head's SP workgroups
+// to arrive (counted in `arrived`, one int per head, zero before the first launch and zero again
+// after every launch) merges the SP partials in split order -- the result does not depend on
+// which workgroup arrives last -- and writes the output row.
+constexpr int kAttentionMaxSplits = 8;
 constexpr size_t decode_attention_lds_bytes(int D, int NW, int S)
 {
     return (static_cast<size_t>(S) + (64 * NW / (D / 8)) * D + 64 * NW) * sizeof(float);
 }
 
-template <int D, bool ROPE, bool ADJACENT = false, int NW = 4>
+template <int D, bool ROPE, bool ADJACENT = false, int NW = 4, bool SPLIT = false>
 __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
     const float* __restrict__ cosv, const float* __restrict__ sinv,
-    const long long* __restrict__ pos, uint16_t* __restrict__ out, int H, int KV, int S, float scale)
+    const long long* __restrict__ pos, uint16_t* __restrict__ out, int H, int KV, int S, float scale,
+    float* partial, int* arrived, int splits)
 {
     static_assert(D == 64 || D == 128, "head dimension");
     constexpr int CH = D / 8;                    // 8-dimension chunks of a row
@@ -138,7 +148,12 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     float* part2 = lds + SLICES * D;             // [GROUPS][D]
     float* score = part2 + GROUPS * D;           // [S]
     __shared__ float red[2 * NW];
+    __shared__ int last_flag;
 
+    // SP = splits of the cache (= gridDim.y), sp = this workgroup's split; constants in the unsplit kernel
+    const int SP = SPLIT ? splits : 1, sp = SPLIT ? blockIdx.y : 0;
+    // local slot l of this split (16 * local tile + row) -> cache slot
+    auto cache_slot = [&](int l) { return (((l >> 4) * SP + sp) << 4) + (l & 15); };
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int b = blockIdx.x / H, h = blockIdx.x - b * H;
@@ -163,14 +178,14 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     u32x4 kr[KT][NJ], vr[VU], qr[NJ];
 #pragma unroll
     for (int t = 0; t < KT; ++t) {
-        const int sk = 16 * (wave + NW * t) + r16;
+        const int sk = 16 * ((wave + NW * t) * SP + sp) + r16;
         const uint16_t* kp = kbase + static_cast<size_t>(sk < S ? sk : 0) * D + 8 * kblk;
 #pragma unroll
         for (int jj = 0; jj < NJ; ++jj) kr[t][jj] = *reinterpret_cast<const u32x4*>(kp + 32 * jj);
     }
 #pragma unroll
     for (int u = 0; u < VU; ++u) {
-        const int sv = slice + u * SLICES;
+        const int sv = cache_slot(slice + u * SLICES);
         vr[u] = *reinterpret_cast<const u32x4*>(vbase + static_cast<size_t>(sv < S ? sv : 0) * D + chunk * 8);
     }
     u32x4 knew[NJ], vnew;                        // ROPE: the new token's key chunks of this lane, value chunk of this thread
@@ -246,7 +261,7 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
                 knew[jj] = rotate(k_own[jj], k_par[jj], jj, first_half);
             }
         }
-        if (h % (H / KV) == 0) {                 // this kv group's writer: slot pos[0] of both caches
+        if (h % (H / KV) == 0 && sp == 0) {      // this kv group's writer: slot pos[0] of both caches
             const size_t slot_off = ((static_cast<size_t>(b) * KV + kvh) * S + (n - 1)) * D;
             if (wave == 0 && r16 == 0) {
 #pragma unroll
@@ -257,7 +272,8 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     }
 
     float mx = -INFINITY;
-    auto score_tile = [&](int tile, const u32x4 (&kin)[NJ]) {
+    auto score_tile = [&](int ltile, const u32x4 (&kin)[NJ]) {       // ltile: local tile of this split
+        const int tile = ltile * SP + sp;
         u32x4 k[NJ];
 #pragma unroll
         for (int jj = 0; jj < NJ; ++jj) k[jj] = kin[jj];
@@ -277,19 +293,21 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
                 const int sk = 16 * tile + 4 * kblk + v;
                 if (sk < n) {
                     const float d = acc[v] * scale;
-                    score[sk] = d;
+                    score[16 * ltile + 4 * kblk + v] = d;
                     mx = fmaxf(mx, d);
                 }
             }
         }
     };
-    const int tiles = (n + 15) >> 4;
+    const int tiles = (n + 15) >> 4;                                  // tiles with a valid slot, all splits
+    const int ltiles = tiles > sp ? (tiles - sp + SP - 1) / SP : 0;  // ... of this split
+    const int nl = 16 * ltiles;                                       // local slots (the last tile may be partly valid)
 #pragma unroll
     for (int t = 0; t < KT; ++t)
-        if (wave + NW * t < tiles) score_tile(wave + NW * t, kr[t]);
-    for (int tile = wave + NW * KT; tile < tiles; tile += NW) {   // beyond 64 * NW slots: plain loop
+        if (wave + NW * t < ltiles) score_tile(wave + NW * t, kr[t]);
+    for (int tile = wave + NW * KT; tile < ltiles; tile += NW) {      // beyond the tiles requested up front: plain loop
         u32x4 k[NJ];
-        const int sk = 16 * tile + r16;
+        const int sk = 16 * (tile * SP + sp) + r16;
         const uint16_t* kp = kbase + static_cast<size_t>(sk < S ? sk : 0) * D + 8 * kblk;
 #pragma unroll
         for (int jj = 0; jj < NJ; ++jj) k[jj] = *reinterpret_cast<const u32x4*>(kp + 32 * jj);
@@ -304,9 +322,9 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
 
     // ---- pass 2: softmax numerators and their sum (each thread revisits the slots it scored)
     float sum = 0.0f;
-    for (int s = tid; s < n; s += NT) {
-        const float p = __expf(score[s] - mx);
-        score[s] = p;
+    for (int l = tid; l < nl; l += NT) {
+        const float p = cache_slot(l) < n ? __expf(score[l] - mx) : 0.0f;
+        score[l] = p;
         sum += p;
     }
     sum = wave_sum(sum);
@@ -318,27 +336,28 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
 
     // ---- pass 3: weighted sum of the value rows, VU rows per round (the first round is already here)
     float acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-    for (int s0 = slice; s0 < n; s0 += VU * SLICES) {
-        float p[VU];
+    for (int l0 = slice; l0 < nl; l0 += VU * SLICES) {
+        if (l0 != slice) {                       // all VU rows of the round requested before any is used
 #pragma unroll
-        for (int u = 0; u < VU; ++u) {
-            const int s = s0 + u * SLICES;
-            if (s0 != slice) {
-                const int sc = s < n ? s : s0;   // past the end: re-read a valid row with weight 0
-                vr[u] = *reinterpret_cast<const u32x4*>(vbase + static_cast<size_t>(sc) * D + chunk * 8);
-            }
-            p[u] = s < n ? score[s] : 0.0f;
-            if (!(s < n)) vr[u] = u32x4{0u, 0u, 0u, 0u};     // never multiply stale cache contents (could be NaN)
-            if constexpr (ROPE) {
-                if (s == n - 1) vr[u] = vnew;
+            for (int u = 0; u < VU; ++u) {
+                const int l = l0 + u * SLICES;
+                const int s = cache_slot(l);
+                const bool ok = l < nl && s < n; // past the end: re-read slot 0, it gets weight 0 below
+                vr[u] = *reinterpret_cast<const u32x4*>(vbase + static_cast<size_t>(ok ? s : 0) * D + chunk * 8);
             }
         }
 #pragma unroll
         for (int u = 0; u < VU; ++u) {
+            const int l = l0 + u * SLICES;
+            const int s = cache_slot(l);
+            const bool ok = l < nl && s < n;
+            const float p = score[ok ? l : 0];
+            u32x4 row = vr[u];
+            if constexpr (ROPE) row = (s == n - 1) ? vnew : row;
             float vf[8];
-            unpack_bf16x8(vr[u], vf);
+            unpack_bf16x8(row, vf);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[e] = fmaf(p[u], vf[e], acc[e]);
+            for (int e = 0; e < 8; ++e) acc[e] = ok ? fmaf(p, vf[e], acc[e]) : acc[e];   // never use stale cache contents (could be NaN)
         }
     }
 #pragma unroll
@@ -352,12 +371,50 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
         part2[grp * D + d] = o;
     }
     __syncthreads();
+    float o = 0.0f;
     if (tid < D) {
-        float o = 0.0f;
 #pragma unroll
         for (int grp = 0; grp < GROUPS; ++grp) o += part2[grp * D + tid];
-        out[(static_cast<size_t>(b) * H + h) * D + tid] = float_to_bf16_bits(o / sum);
     }
+    uint16_t* orow = out + (static_cast<size_t>(b) * H + h) * D;
+    if (!SPLIT || SP == 1) {
+        if (tid < D) orow[tid] = float_to_bf16_bits(o / sum);
+        return;
+    }
+
+    // ---- split: publish (o, mx, sum), count the arrival; the last workgroup of the head merges.
+    // The partials and the counter are written and read with device-scope relaxed atomics: those go
+    // past the per-XCD L2 to the memory all XCDs share, so no cache write-back or invalidate (what a
+    // device-scope fence would cost every workgroup) is needed.  Order: every thread's partial stores
+    // have completed at the barrier, the arrival is counted after it, and the merging workgroup
+    // reads after it has seen the full count.
+    float* mine = partial + (static_cast<size_t>(blockIdx.x) * SP + sp) * (D + 2);
+    auto publish = [](float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+    auto fetch = [](const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+    if (tid < D) publish(mine + tid, o);
+    if (tid == 0) {
+        publish(mine + D, mx);
+        publish(mine + D + 1, sum);
+    }
+    __syncthreads();                             // waits for this workgroup's stores
+    if (tid == 0)
+        last_flag = __hip_atomic_fetch_add(arrived + blockIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == SP - 1;
+    __syncthreads();
+    if (!last_flag) return;
+    if (tid < D) {
+        const float* head = partial + static_cast<size_t>(blockIdx.x) * SP * (D + 2);
+        float m_all = -INFINITY;
+        for (int j = 0; j < SP; ++j) m_all = fmaxf(m_all, fetch(head + j * (D + 2) + D));
+        float num = 0.0f, den = 0.0f;
+        for (int j = 0; j < SP; ++j) {
+            const float w = __expf(fetch(head + j * (D + 2) + D) - m_all);      // an empty split: exp(-inf) = 0
+            num = fmaf(w, fetch(head + j * (D + 2) + tid), num);
+            den = fmaf(w, fetch(head + j * (D + 2) + D + 1), den);
+        }
+        orow[tid] = float_to_bf16_bits(num / den);
+    }
+    // every split has arrived: ready for the next launch
+    if (tid == 0) __hip_atomic_store(arrived + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 }  // namespace terna

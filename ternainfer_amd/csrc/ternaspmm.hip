@@ -377,8 +377,9 @@ __global__ void sleep_kernel(long long ticks)
 }
 
 // Waves per workgroup of the decode attention: with one workgroup per (sequence, head) and few of them
-// on the chip, wider workgroups request more of the cache up front.  TERNASPMM_ATTN_WAVES=4|8 forces one
-// (tuning aid).  Both entry points use the same rule, so their results stay bit-identical.
+// on the chip, wider workgroups request more of the cache up front (64 slots of keys per wave).
+// TERNASPMM_ATTN_WAVES=4|8 forces one (tuning aid).  Both entry points use the same rule, so their results
+// stay bit-identical.
 int attention_waves(int B, int H)
 {
     static const int forced = [] {
@@ -390,30 +391,60 @@ int attention_waves(int B, int H)
     return static_cast<long>(B) * H <= 512 ? 8 : 4;
 }
 
-template <int D, bool ROPE, bool ADJ, int NW>
-void launch_attention_as(const uint16_t* q, uint16_t* ck, uint16_t* cv, const float* cos, const float* sin,
-                                const long long* pos, uint16_t* out, int B, int H, int KV, int S, float scale,
-                                hipStream_t st)
+// Workspace of the split variant: one arrival counter per head (the caller zeroes them once), then
+// kAttentionMaxSplits partial results of D + 2 floats per head.
+size_t attention_counter_bytes(int B, int H) { return (static_cast<size_t>(B) * H * sizeof(int) + 255) & ~static_cast<size_t>(255); }
+
+// Splits of the cache per head: as many as keep the grid within two workgroups per CU, at most 8; 1 without
+// a workspace, and 1 for caches below 1024 slots, where the merge (three dependent trips to device memory,
+// 4-5 us) costs more than streaming the prefix from one CU.  TERNASPMM_ATTN_SPLITS=1|2|4|8 forces one
+// (tuning aid).
+int attention_splits(int B, int H, int S, const void* workspace)
 {
-    auto kernel = terna_decode_attention_kernel<D, ROPE, ADJ, NW>;
+    if (workspace == nullptr) return 1;
+    static const int forced = [] {
+        const char* v = std::getenv("TERNASPMM_ATTN_SPLITS");
+        const int n = v ? std::atoi(v) : 0;
+        return (n == 1 || n == 2 || n == 4 || n == 8) ? n : 0;
+    }();
+    if (forced) return forced;
+    if (S < 1024) return 1;
+    int sp = 1;
+    while (sp < kAttentionMaxSplits && static_cast<long>(B) * H * sp * 2 <= 512) sp *= 2;
+    return sp;
+}
+
+template <int D, bool ROPE, bool ADJ, int NW, bool SPLIT>
+void launch_attention_as(const uint16_t* q, uint16_t* ck, uint16_t* cv, const float* cos, const float* sin,
+                         const long long* pos, uint16_t* out, int B, int H, int KV, int S, float scale, int splits,
+                         void* workspace, hipStream_t st)
+{
+    auto kernel = terna_decode_attention_kernel<D, ROPE, ADJ, NW, SPLIT>;
     const size_t lds = decode_attention_lds_bytes(D, NW, S);
     if (lds > 64 * 1024) allow_dynamic_lds(kernel, 160 * 1024, "hipFuncSetAttribute(decode attention)", __LINE__);
-    kernel<<<dim3(B * H), dim3(64 * NW), lds, st>>>(q, ck, cv, cos, sin, pos, out, H, KV, S, scale);
+    int* arrived = static_cast<int*>(workspace);
+    float* partial = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + attention_counter_bytes(B, H)) : nullptr;
+    kernel<<<dim3(B * H, splits), dim3(64 * NW), lds, st>>>(q, ck, cv, cos, sin, pos, out, H, KV, S, scale, partial, arrived,
+                                                             splits);
 }
 
 template <bool ROPE, bool ADJ>
 void launch_attention(const uint16_t* q, uint16_t* ck, uint16_t* cv, const float* cos, const float* sin,
                              const long long* pos, uint16_t* out, int B, int H, int KV, int D, int S, float scale,
-                             hipStream_t st)
+                             void* workspace, hipStream_t st)
 {
-    const int nw = attention_waves(B, H);
-#define TERNA_ATTN(DIM, NWAVES) launch_attention_as<DIM, ROPE, ADJ, NWAVES>(q, ck, cv, cos, sin, pos, out, B, H, KV, S, scale, st)
+    const int splits = attention_splits(B, H, S, workspace);
+    const int nw = splits > 1 ? 4 : attention_waves(B, H);       // a split is a short prefix: the narrow workgroup
+#define TERNA_ATTN(DIM, NWAVES, SPLIT) \
+    launch_attention_as<DIM, ROPE, ADJ, NWAVES, SPLIT>(q, ck, cv, cos, sin, pos, out, B, H, KV, S, scale, splits, workspace, st)
     if (D == 128) {
-        if (nw == 8) TERNA_ATTN(128, 8);
-        else TERNA_ATTN(128, 4);
+        if (splits > 1) TERNA_ATTN(128, 4, true);
+        else if (nw == 8) TERNA_ATTN(128, 8, false);
+        else TERNA_ATTN(128, 4, false);
     } else {
-        if (nw == 8) TERNA_ATTN(64, 8);
-        else TERNA_ATTN(64, 4);
+        if (splits > 1) TERNA_ATTN(64, 4, true);
+        else if (nw == 8) TERNA_ATTN(64, 8, false);
+        else TERNA_ATTN(64, 4, false);
     }
 #undef TERNA_ATTN
 }
@@ -746,26 +777,33 @@ void ternaspmm_rope_kv_store(const terna_bf16* qkv, const float* cos, const floa
     if (e != hipSuccess) die("ternaspmm_rope_kv_store", e, __LINE__);
 }
 
+long long ternaspmm_attention_workspace_bytes(int B, int H, int D)
+{
+    if (B < 1 || H < 1 || D < 1) return -1;
+    return static_cast<long long>(attention_counter_bytes(B, H)) +
+           static_cast<long long>(B) * H * kAttentionMaxSplits * (D + 2) * sizeof(float);
+}
+
 void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
                                 const long long* pos, terna_bf16* out, int B, int H, int KV, int D, int S,
-                                float scale, terna_stream stream)
+                                float scale, void* workspace, terna_stream stream)
 {
     if (!attention_args_ok("ternaspmm_decode_attention", B, H, KV, D, S)) return;
     // the kernel writes the caches only in its ROPE variant
     launch_attention<false, false>(q, const_cast<uint16_t*>(cache_k), const_cast<uint16_t*>(cache_v), nullptr, nullptr, pos,
-                                   out, B, H, KV, D, S, scale, static_cast<hipStream_t>(stream));
+                                   out, B, H, KV, D, S, scale, workspace, static_cast<hipStream_t>(stream));
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_decode_attention", e, __LINE__);
 }
 
 void ternaspmm_rope_decode_attention(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
                                      terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
-                                     int D, int S, float scale, int adjacent, terna_stream stream)
+                                     int D, int S, float scale, int adjacent, void* workspace, terna_stream stream)
 {
     if (!attention_args_ok("ternaspmm_rope_decode_attention", B, H, KV, D, S)) return;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (adjacent) launch_attention<true, true>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, st);
-    else launch_attention<true, false>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, st);
+    if (adjacent) launch_attention<true, true>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, workspace, st);
+    else launch_attention<true, false>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, workspace, st);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_rope_decode_attention", e, __LINE__);
 }

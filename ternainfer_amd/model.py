@@ -180,7 +180,7 @@ class Block:
         y, h = rmsnorm_quant(x, weight, eps, residual=residual, quant=False)
         return lin.dense(y), h
 
-    def forward(self, x, pending, cache_k, cache_v, pos_idx, cos, sin, mask):
+    def forward(self, x, pending, cache_k, cache_v, pos_idx, cos, sin, mask, attn_ws=None):
         """x [B*T, dim] (T new tokens per sequence) and `pending`, the previous block's FFN output that
         has not been added to the stream yet (None for the first block): the add is part of this
         block's first fused kernel.  cache_* [B, n_kv, S, hd]; pos_idx int64 [T] cache slots.
@@ -197,7 +197,7 @@ class Block:
             o = torch.empty((bsz, a.n_heads * a.head_dim), dtype=torch.bfloat16, device=x.device)
             lib.ternaspmm_rope_decode_attention(_p(qkv), _p(cos), _p(sin), _p(pos_idx), _p(cache_k), _p(cache_v), _p(o),
                                                 bsz, a.n_heads, a.n_kv_heads, a.head_dim, cache_k.shape[2],
-                                                a.head_dim ** -0.5, int(a.rope_adjacent), stream)
+                                                a.head_dim ** -0.5, int(a.rope_adjacent), _p(attn_ws), stream)
         elif self.fused:
             lib = self.wqkv.lib
             stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -255,6 +255,15 @@ class Transformer:
             self._rope_tables = tables = (key, ang.cos().contiguous(), ang.sin().contiguous())
         return tables[1], tables[2]
 
+    def attention_workspace(self, bsz: int):
+        """Zero-filled scratch of the single-token attention (split over the cache); one per batch size."""
+        ws = getattr(self, "_attn_ws", None)
+        if ws is None or ws[0] != bsz:
+            a = self.args
+            nbytes = _lib.load().ternaspmm_attention_workspace_bytes(bsz, a.n_heads, a.head_dim)
+            self._attn_ws = ws = (bsz, torch.zeros(nbytes, dtype=torch.int8, device="cuda"))
+        return ws[1]
+
     def make_cache(self, bsz: int, max_seq: int):
         a = self.args
         shape = (bsz, a.n_kv_heads, max_seq, a.head_dim)
@@ -278,8 +287,9 @@ class Transformer:
             mask = (torch.arange(max_seq, device=dev)[None, :] <= pos_idx[:, None])[None, None]
         x = self.tok_embeddings[tokens.reshape(-1)]
         pending = None
+        attn_ws = self.attention_workspace(bsz) if one_launch_attention else None     # layers run one after another: shared
         for layer, (ck, cv) in zip(self.layers, cache):
-            x, pending = layer.forward(x, pending, ck, cv, pos_idx, cos, sin, mask)
+            x, pending = layer.forward(x, pending, ck, cv, pos_idx, cos, sin, mask, attn_ws)
         if t > 1:                                                             # only the last new token feeds the head
             x, pending = x.view(bsz, t, a.dim)[:, -1].contiguous(), pending.view(bsz, t, a.dim)[:, -1].contiguous()
         if self.layers[0].fused and x.is_cuda:                                # last residual add + final norm: one launch

@@ -194,21 +194,41 @@ def test_rope_kv_store(lib, b, t, h, kv, d, s_max, adjacent):
 
 
 @pytest.mark.parametrize("b,h,kv,d,s_max,n", [(1, 20, 5, 128, 256, 1), (1, 20, 5, 128, 256, 160), (8, 20, 5, 128, 512, 512),
-                                              (2, 4, 2, 64, 40, 17), (1, 20, 5, 128, 4096, 4000)])
-def test_decode_attention(lib, b, h, kv, d, s_max, n):
+                                              (2, 4, 2, 64, 40, 17), (1, 20, 5, 128, 4096, 4000),
+                                              (2, 4, 2, 64, 1040, 1030), (8, 20, 5, 128, 1024, 1000), (1, 20, 5, 128, 1024, 3)])
+@pytest.mark.parametrize("split", [False, True])
+def test_decode_attention(lib, b, h, kv, d, s_max, n, split):
+    """split: with a workspace and a cache of 1024 slots or more, the prefix of a head is spread over several
+    workgroups and merged by the last one to arrive; two launches in a row on one workspace (the counters must
+    be back at zero)."""
     q = make_bf16_activations(b * h, d, 710 + n).reshape(b, h, d)
     k = make_bf16_activations(b * kv * s_max, d, 711 + n).reshape(b, kv, s_max, d)
     v = make_bf16_activations(b * kv * s_max, d, 712 + n, outlier_frac=0.01).reshape(b, kv, s_max, d)
     pos = np.array([n - 1], np.int64)
     od = torch.zeros((b, h * d), dtype=torch.int16, device="cuda")
     qd, kd, vd, pd = _dev(q), _dev(k), _dev(v), _dev(pos)            # named: they must outlive the launch
-    lib.ternaspmm_decode_attention(_vp(qd), _vp(kd), _vp(vd), _vp(pd), _vp(od), b, h, kv, d, s_max, float(d) ** -0.5, None)
+    ws = _attn_workspace(lib, b, h, d) if split else None
+    print(f"[case] decode attention b={b} h={h} kv={kv} d={d} S={s_max} n={n} split={split}", flush=True)
+    lib.ternaspmm_decode_attention(_vp(qd), _vp(kd), _vp(vd), _vp(pd), _vp(od), b, h, kv, d, s_max, float(d) ** -0.5, _vp(ws), None)
     torch.cuda.synchronize()
     got = O.bf16_bits_to_f32(od.cpu().numpy().view(np.uint16)).reshape(b, h, d).astype(np.float64)
     want = O.attention_one_token(q, k, v, n, float(d) ** -0.5)
     # fp32 softmax and accumulation, bf16 output: relative to the largest output of the head
     tol = 2.0 ** -7 * np.abs(want).max(axis=-1, keepdims=True) + 1e-6
     assert (np.abs(got - want) <= tol).all(), float((np.abs(got - want) / tol).max())
+    if split:
+        counters = ws[:b * h * 4].view(torch.int32)
+        assert int(counters.abs().sum().item()) == 0
+        od2 = torch.zeros_like(od)
+        lib.ternaspmm_decode_attention(_vp(qd), _vp(kd), _vp(vd), _vp(pd), _vp(od2), b, h, kv, d, s_max, float(d) ** -0.5, _vp(ws), None)
+        torch.cuda.synchronize()
+        assert torch.equal(od, od2)                      # merged in split order: the same bits whoever arrives last
+
+
+def _attn_workspace(lib, b, h, d):
+    nbytes = lib.ternaspmm_attention_workspace_bytes(b, h, d)
+    assert nbytes > 0
+    return torch.zeros(nbytes, dtype=torch.int8, device="cuda")
 
 
 # ------------------------------------------------------------------ prologue inside the small-M linear
@@ -325,10 +345,12 @@ def test_fused_gate_prologue_linear(lib, n, f, ws_num):
     assert lib.bitlinear_TernaSpMM_packed_fused_glu(_vp(z), _vp(z), 1e-5, _vp(z), _vp(z), _vp(z), 1, None, None, 2, n, f, None) == 0
 
 
+@pytest.mark.parametrize("split", [False, True])
 @pytest.mark.parametrize("adjacent", [0, 1])
 @pytest.mark.parametrize("b,h,kv,d,s_max,n", [(1, 20, 5, 128, 256, 1), (1, 20, 5, 128, 256, 160), (8, 20, 5, 128, 300, 290),
-                                              (2, 4, 2, 64, 40, 17), (1, 20, 5, 128, 600, 513)])
-def test_rope_decode_attention_equals_the_two_launches(lib, b, h, kv, d, s_max, n, adjacent):
+                                              (2, 4, 2, 64, 40, 17), (1, 20, 5, 128, 600, 513), (1, 20, 5, 128, 2048, 1500),
+                                              (2, 4, 2, 64, 1024, 1)])
+def test_rope_decode_attention_equals_the_two_launches(lib, b, h, kv, d, s_max, n, adjacent, split):
     """One launch (RoPE + cache write + attention) against ternaspmm_rope_kv_store followed by
     ternaspmm_decode_attention on the same inputs: outputs and both caches bit-identical."""
     rng = np.random.default_rng(720 + n)
@@ -340,18 +362,20 @@ def test_rope_decode_attention_equals_the_two_launches(lib, b, h, kv, d, s_max, 
     cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
     xd, cd, sd, pd = _dev(qkv), _dev(cos), _dev(sin), _dev(pos)
     scale = float(d) ** -0.5
+    ws1 = _attn_workspace(lib, b, h, d) if split else None
+    ws2 = _attn_workspace(lib, b, h, d) if split else None
     # two launches
     ck1, cv1 = _dev(k0), _dev(v0)
     q1 = torch.zeros((b, h, 1, d), dtype=torch.int16, device="cuda")
     o1 = torch.zeros((b, h * d), dtype=torch.int16, device="cuda")
     lib.ternaspmm_rope_kv_store(_vp(xd), _vp(cd), _vp(sd), _vp(pd), _vp(q1), _vp(ck1), _vp(cv1), b, 1, h, kv, d, s_max, adjacent, None)
-    lib.ternaspmm_decode_attention(_vp(q1), _vp(ck1), _vp(cv1), _vp(pd), _vp(o1), b, h, kv, d, s_max, scale, None)
+    lib.ternaspmm_decode_attention(_vp(q1), _vp(ck1), _vp(cv1), _vp(pd), _vp(o1), b, h, kv, d, s_max, scale, _vp(ws1), None)
     # one launch
     ck2, cv2 = _dev(k0), _dev(v0)
     o2 = torch.zeros((b, h * d), dtype=torch.int16, device="cuda")
     print(f"[case] rope + decode attention b={b} h={h} kv={kv} d={d} S={s_max} n={n} adjacent={adjacent}", flush=True)
     lib.ternaspmm_rope_decode_attention(_vp(xd), _vp(cd), _vp(sd), _vp(pd), _vp(ck2), _vp(cv2), _vp(o2), b, h, kv, d, s_max,
-                                        scale, adjacent, None)
+                                        scale, adjacent, _vp(ws2), None)
     torch.cuda.synchronize()
     assert torch.equal(ck1, ck2) and torch.equal(cv1, cv2)
     assert torch.equal(o1, o2)
