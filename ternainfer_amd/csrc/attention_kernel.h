@@ -351,13 +351,14 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
             const int l = l0 + u * SLICES;
             const int s = cache_slot(l);
             const bool ok = l < nl && s < n;
-            const float p = score[ok ? l : 0];
+            const float p = ok ? score[ok ? l : 0] : 0.0f;
             u32x4 row = vr[u];
             if constexpr (ROPE) row = (s == n - 1) ? vnew : row;
+            row = ok ? row : u32x4{0u, 0u, 0u, 0u};          // never multiply stale cache contents (could be NaN)
             float vf[8];
             unpack_bf16x8(row, vf);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[e] = ok ? fmaf(p, vf[e], acc[e]) : acc[e];   // never use stale cache contents (could be NaN)
+            for (int e = 0; e < 8; ++e) acc[e] = fmaf(p, vf[e], acc[e]);
         }
     }
 #pragma unroll
