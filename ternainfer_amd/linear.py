@@ -24,8 +24,9 @@ _GLOBAL_WORKSPACE = None
 
 
 def get_global_workspace(device="cuda"):
-    """One int8 scratch buffer shared by every layer (model.py:37-42).  This build's kernels
-    never touch it; it is still passed so the ABI stays the reference's."""
+    """One int8 scratch buffer shared by every layer (model.py:37-42).  The small-M kernels never
+    touch it; a large-M call on the reference format transcodes the weight into its first N*K/4
+    bytes (the 2-bit layout the MFMA kernel reads) instead of the reference's dense N*K copy."""
     global _GLOBAL_WORKSPACE
     if _GLOBAL_WORKSPACE is None:
         _GLOBAL_WORKSPACE = torch.empty(MAX_MATRIX_ELEMENTS, dtype=torch.int8, device=device)
