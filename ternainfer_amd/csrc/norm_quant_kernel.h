@@ -22,18 +22,51 @@ namespace terna {
 constexpr int kNormThreads = 256;
 constexpr int kNormMaxVecs = 4;                       // 8-element vectors per thread: K <= 8192
 
-__device__ __forceinline__ float wave_sum(float v)
+// Reductions over groups of LANES consecutive lanes (LANES = 2 .. 64, a power of two) with the data
+// parallel primitives of the VALU instead of LDS-crossbar shuffles: a ds_bpermute round trip costs
+// on the order of a hundred cycles and a 64-lane butterfly needs six of them in sequence; the
+// quad / half-row / row permutations below are ordinary VALU operands.  Every lane of the wave must
+// be active.  The result is the same in every lane of a group; the order of the additions is
+// fixed (pairs, quads, eights, sixteens, then rows 0+1 and 2+3, then the halves).
+template <int CTRL>
+__device__ __forceinline__ float dpp_permute(float v)
 {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+constexpr int kDppSwapPairs = 0xB1;       // quad_perm [1, 0, 3, 2]: lane ^ 1
+constexpr int kDppSwapHalfQuads = 0x4E;   // quad_perm [2, 3, 0, 1]: lane ^ 2
+constexpr int kDppHalfRowMirror = 0x141;  // lane i <-> 7 - i within 8 lanes
+constexpr int kDppRowMirror = 0x140;      // lane i <-> 15 - i within 16 lanes
+
+template <int LANES, bool IS_MAX>
+__device__ __forceinline__ float group_reduce(float v)
+{
+    static_assert(LANES >= 1 && LANES <= 64 && (LANES & (LANES - 1)) == 0, "group size");
+    auto op = [](float a, float b) { return IS_MAX ? fmaxf(a, b) : a + b; };
+    if constexpr (LANES >= 2) v = op(v, dpp_permute<kDppSwapPairs>(v));
+    if constexpr (LANES >= 4) v = op(v, dpp_permute<kDppSwapHalfQuads>(v));
+    if constexpr (LANES >= 8) v = op(v, dpp_permute<kDppHalfRowMirror>(v));     // quads are uniform by now
+    if constexpr (LANES >= 16) v = op(v, dpp_permute<kDppRowMirror>(v));        // ... and so are the halves of a row
+    if constexpr (LANES == 32) {
+        // rows 0|1 and 2|3: lane ^ 16 through the row's uniform value of the neighbouring row
+        const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+        const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+        const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+        const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+        v = (threadIdx.x & 32) ? op(r2, r3) : op(r0, r1);
+    }
+    if constexpr (LANES == 64) {
+        const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+        const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+        const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+        const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+        v = op(op(r0, r1), op(r2, r3));
+    }
     return v;
 }
-__device__ __forceinline__ float wave_max(float v)
-{
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-    return v;
-}
+
+__device__ __forceinline__ float wave_sum(float v) { return group_reduce<64, false>(v); }
+__device__ __forceinline__ float wave_max(float v) { return group_reduce<64, true>(v); }
 
 __device__ __forceinline__ void unpack_bf16x8(const u32x4& v, float f[8])
 {
