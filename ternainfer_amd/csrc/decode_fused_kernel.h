@@ -123,9 +123,10 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
     const Epilogue ep{nullptr, ws, nullptr, ws_num, EP_I8_DECODE};
     const int my_band = band0 + (wave < NB ? wave : 0);
     EpilogueRaw eraw = load_epilogue_raw_scales(ep, my_band * 16 + 4 * g, N);
-    // this wave's LDS slot: rows the batch does not have stay zero
+    // this wave's LDS slot: rows the batch does not have stay zero (a single row needs no slot, see phase D)
     uint8_t* slab = slab_all[wave];
-    for (int o = lane * 16; o < 16 * XQ::kPitch; o += 64 * 16) *reinterpret_cast<u32x4*>(slab + o) = u32x4{0u, 0u, 0u, 0u};
+    if constexpr (MP != 1)
+        for (int o = lane * 16; o < 16 * XQ::kPitch; o += 64 * 16) *reinterpret_cast<u32x4*>(slab + o) = u32x4{0u, 0u, 0u, 0u};
 
     TERNA_TS(1);
     float ssq = 0.0f;
@@ -220,9 +221,20 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
             uint8_t* dst = slab + row * XQ::kPitch + cl;
             int8_t* gdst = xq_out + static_cast<size_t>(row_ok ? row : 0) * K + j * 64 + cl;
             const bool publish = writer && xq_out != nullptr && row_ok;
+            i32x4 bq;
             if constexpr (MP == 1) {
-                *dst = q[0];
+                // One row: lane c holds the byte of column c.  Four neighbouring bytes into the dword of lane 4d,
+                // the four dwords of 16 columns into lane 16g -- the only lanes whose MFMA operand (batch row 0,
+                // columns 16g .. 16g+15) is not zero.  No LDS.
                 if (publish) *gdst = static_cast<int8_t>(q[0]);
+                const uint32_t b1 = q[0];
+                const uint32_t b2 = b1 | (dpp_permute_u32<kDppSwapPairs>(b1) << 8);          // even lanes: columns c, c+1
+                const uint32_t b4 = b2 | (dpp_permute_u32<kDppSwapHalfQuads>(b2) << 16);     // lanes 4d: columns 4d .. 4d+3
+                const uint32_t d1 = dpp_permute_u32<kDppRowShl4>(b4), d2 = dpp_permute_u32<kDppRowShl8>(b4),
+                               d3 = dpp_permute_u32<kDppRowShl12>(b4);
+                const bool first = i == 0;
+                bq = i32x4{static_cast<int>(first ? b4 : 0u), static_cast<int>(first ? d1 : 0u),
+                           static_cast<int>(first ? d2 : 0u), static_cast<int>(first ? d3 : 0u)};
             } else {
                 uint32_t d[MP / 4];
 #pragma unroll
@@ -235,8 +247,8 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
                     *reinterpret_cast<u32x4*>(dst) = u32x4{d[0], d[1], d[2], d[3]};
                     if (publish) *reinterpret_cast<u32x4*>(gdst) = u32x4{d[0], d[1], d[2], d[3]};
                 }
+                bq = __builtin_bit_cast(i32x4, *reinterpret_cast<const u32x4*>(slab + i * XQ::kPitch + g * 16));
             }
-            const i32x4 bq = __builtin_bit_cast(i32x4, *reinterpret_cast<const u32x4*>(slab + i * XQ::kPitch + g * 16));
 #pragma unroll
             for (int b = 0; b < NB; ++b)
                 acc[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(expand_word_i8(wword[b][t]), bq, acc[b], 0, 0, 0);

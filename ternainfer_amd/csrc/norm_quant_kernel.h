@@ -33,6 +33,14 @@ __device__ __forceinline__ float dpp_permute(float v)
 {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
 }
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_permute_u32(uint32_t v)
+{
+    return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, 0xf, 0xf, true));
+}
+constexpr int kDppRowShl4 = 0x104;        // lane i <- lane i + 4 within 16 lanes (0 past the row)
+constexpr int kDppRowShl8 = 0x108;
+constexpr int kDppRowShl12 = 0x10C;
 constexpr int kDppSwapPairs = 0xB1;       // quad_perm [1, 0, 3, 2]: lane ^ 1
 constexpr int kDppSwapHalfQuads = 0x4E;   // quad_perm [2, 3, 0, 1]: lane ^ 2
 constexpr int kDppHalfRowMirror = 0x141;  // lane i <-> 7 - i within 8 lanes

@@ -691,7 +691,12 @@ static int launch_decode_fused(int mode, const terna_bf16* x, const terna_bf16* 
     if (!shape_ok(M, N, K) || ws_num < 1 || M > 16) return 0;
     const int ktiles = K / 64;
     const int bands = N / 16;
-    const bool wide = bands <= 256;                  // same split as the unfused small-M kernel
+    static const int forced_waves = [] {
+        const char* v = std::getenv("TERNASPMM_FUSED_WAVES");
+        return v ? std::atoi(v) : 0;
+    }();
+    // same split as the unfused small-M kernel; TERNASPMM_FUSED_WAVES=8|16 forces one (tuning aid)
+    const bool wide = forced_waves == 16 ? true : (forced_waves == 8 ? mode == FUSED_GLU : bands <= 256);
     const uint32_t* p = static_cast<const uint32_t*>(packed);
     // More bands than CUs: four bands per workgroup, so that the grid is one round and the prologue runs once
     // per CU.  TERNASPMM_FUSED_BANDS=1 switches that off, TERNASPMM_FUSED_BANDS_WAVES=8 picks the 8-wave
