@@ -46,7 +46,11 @@ __global__ __launch_bounds__(kArgmaxThreads) void terna_argmax_bf16_kernel(const
                 float f[8];
                 unpack_bf16x8(raw[u], f);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) argmax_merge(best, idx, f[e], 8 * v + e);
+                for (int e = 0; e < 8; ++e) {    // a thread's indices ascend: a strict compare keeps the first maximum
+                    const bool better = f[e] > best;
+                    best = better ? f[e] : best;
+                    idx = better ? 8 * v + e : idx;
+                }
             }
         }
     }
