@@ -7,43 +7,49 @@
 // offset fetch, sign window, prefix popcounts, cross-lane gathers and LDS table of the
 // reference-format kernel are all gone.  Every load of a wave is independent of every other, so
 // they are all in flight after one round trip for the kernel arguments.
+//
+// NB = bands per workgroup.  Every workgroup stages the same M x K activations; with more bands than
+// the chip has CUs (gate+up: 864) a CU would pull them from L2 once per round of workgroups -- at
+// M = 8 four times the bytes of a band's weights.  NB bands per workgroup share one staging.
 #pragma once
 
 #include "packed_common.h"
 
 namespace terna {
 
-template <typename Act, int MB>
+template <typename Act, int MB, int NB>
 struct PackedRaw {
-    uint32_t word;                           // 16 weights: row (L & 15), 16-column group (L >> 4)
+    uint32_t word[NB];                       // per band, 16 weights: row (L & 15), 16-column group (L >> 4)
     u32x4    x[MB][XSlab<Act>::kLoads];      // coalesced pieces of the activation slab
 };
 
-template <typename Act, int WAVES, int MB, int DEPTH>
+template <typename Act, int WAVES, int MB, int DEPTH, int NB = 1>
 __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
     const Act* __restrict__ x, const uint32_t* __restrict__ packed, uint16_t* __restrict__ out,
     Epilogue ep, int M, int N, int K)
 {
     using T = ActTraits<Act>;
     using Acc = typename T::Acc;
-    using Raw = PackedRaw<Act, MB>;
+    using Raw = PackedRaw<Act, MB, NB>;
     using XS = XSlab<Act>;
     constexpr int NBUF = DEPTH + 1;
     static_assert(DEPTH >= 1 && DEPTH <= 3, "prefetch distance");
 
-    __shared__ Acc red[WAVES][MB][64];
+    constexpr int UNITS = NB * MB;           // (band, m-block) accumulators per wave
+    __shared__ Acc red[WAVES][UNITS][64];
     __shared__ __align__(16) uint8_t xslab_all[WAVES][MB][16 * XS::kPitch];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     TERNA_TS(0);
-    const int band = blockIdx.x;
+    const int band0 = blockIdx.x * NB;
     const int m_base = blockIdx.y * (16 * MB);
     const int ktiles = K >> 6;
     const int i = lane & 15, g = lane >> 4;
 
-    const uint32_t* wp = packed + (static_cast<size_t>(band) * ktiles + wave) * 64 + i * 4 + g;
+    const uint32_t* wp = packed + (static_cast<size_t>(band0) * ktiles + wave) * 64 + i * 4 + g;
+    const size_t band_pitch = static_cast<size_t>(ktiles) * 64;          // words from one band to the next
     // Coalesced activation pieces of this lane; rows past M are not loaded (their operand is zero
     // and their output column is never stored).
     const Act* xp[MB][XS::kLoads];
@@ -63,7 +69,8 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
     TERNA_TS(2);
 #endif
     auto fetch = [&](int j, Raw& raw) {
-        raw.word = wp[static_cast<size_t>(j) * (WAVES * 64)];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) raw.word[b] = wp[b * band_pitch + static_cast<size_t>(j) * (WAVES * 64)];
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
@@ -73,9 +80,11 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
             }
     };
 
-    Acc acc[MB];
+    Acc acc[NB][MB];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) acc[mb] = Acc{0, 0, 0, 0};
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[b][mb] = Acc{0, 0, 0, 0};
 
     uint8_t* slab = xslab_all[wave][0];
     auto process = [&](const Raw& cur) {
@@ -86,23 +95,33 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
             for (int h = 0; h < XS::kLoads; ++h)
                 *reinterpret_cast<u32x4*>(slab + mb * (16 * XS::kPitch) + XS::write_off(lane, h)) = cur.x[mb][h];
         if constexpr (sizeof(Act) == 2) {
-            const bf16x8 a0 = __builtin_bit_cast(bf16x8, expand_chunk_bf16(cur.word));
-            const bf16x8 a1 = __builtin_bit_cast(bf16x8, expand_chunk_bf16(cur.word >> 4));
+            bf16x8 a0[NB], a1[NB];
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                a0[b] = __builtin_bit_cast(bf16x8, expand_chunk_bf16(cur.word[b]));
+                a1[b] = __builtin_bit_cast(bf16x8, expand_chunk_bf16(cur.word[b] >> 4));
+            }
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
                 const uint8_t* src = slab + mb * (16 * XS::kPitch) + i * XS::kPitch + g * 32;
                 const u32x4 b0 = *reinterpret_cast<const u32x4*>(src);        // columns 16g .. 16g+7
                 const u32x4 b1 = *reinterpret_cast<const u32x4*>(src + 16);   // columns 16g+8 .. 16g+15
-                acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, __builtin_bit_cast(bf16x8, b0), acc[mb], 0, 0, 0);
-                acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, __builtin_bit_cast(bf16x8, b1), acc[mb], 0, 0, 0);
+#pragma unroll
+                for (int b = 0; b < NB; ++b) {
+                    acc[b][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[b], __builtin_bit_cast(bf16x8, b0), acc[b][mb], 0, 0, 0);
+                    acc[b][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[b], __builtin_bit_cast(bf16x8, b1), acc[b][mb], 0, 0, 0);
+                }
             }
         } else {
-            const i32x4 a = expand_word_i8(cur.word);
+            i32x4 a[NB];
+#pragma unroll
+            for (int b = 0; b < NB; ++b) a[b] = expand_word_i8(cur.word[b]);
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
-                const i32x4 b = __builtin_bit_cast(
+                const i32x4 bx = __builtin_bit_cast(
                     i32x4, *reinterpret_cast<const u32x4*>(slab + mb * (16 * XS::kPitch) + i * XS::kPitch + g * 16));
-                acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[mb], 0, 0, 0);
+#pragma unroll
+                for (int b = 0; b < NB; ++b) acc[b][mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[b], bx, acc[b][mb], 0, 0, 0);
             }
         }
     };
@@ -121,14 +140,15 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
     if (DEPTH >= 3 && 2 < cnt) fetch(2, ring2);
     TERNA_TS(1);
 
-    // Wave w finishes m-block w (and w + WAVES, ...): with the data loads in flight, fetch that
-    // block's scale factors so that no global load sits between the last MFMA and the store.
-    const int n0 = band * 16 + 4 * g;
-    EpilogueRaw eraw[(MB + WAVES - 1) / WAVES];
+    // Wave w finishes unit w (and w + WAVES, ...), unit = band * MB + m-block: with the data loads in
+    // flight, fetch that unit's scale factors so that no global load sits between the last MFMA and the store.
+    constexpr int FIN = (UNITS + WAVES - 1) / WAVES;
+    EpilogueRaw eraw[FIN];
 #pragma unroll
-    for (int e = 0; e < (MB + WAVES - 1) / WAVES; ++e) {
-        const int m = m_base + (wave + e * WAVES) * 16 + i;
-        eraw[e] = load_epilogue_raw(ep, m < M ? m : M - 1, n0, N);
+    for (int e = 0; e < FIN; ++e) {
+        const int unit = wave + e * WAVES < UNITS ? wave + e * WAVES : 0;
+        const int m = m_base + (unit % MB) * 16 + i;
+        eraw[e] = load_epilogue_raw(ep, m < M ? m : M - 1, (band0 + unit / MB) * 16 + 4 * g, N);
     }
 
     for (int j0 = 0; j0 < cnt; j0 += NBUF) {
@@ -150,18 +170,21 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
     // Cross-wave sum in wave order, then the fused epilogue (accumulator layout: lane L holds
     // output rows 4*(L>>4) .. +3 of column L & 15).  bf16 weights were +-0.5: undo with an exact x2.
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) red[wave][mb][lane] = acc[mb];
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) red[wave][b * MB + mb][lane] = acc[b][mb];
     TERNA_TS(9);
     __syncthreads();
     TERNA_TS(10);
 #pragma unroll
-    for (int e = 0; e < (MB + WAVES - 1) / WAVES; ++e) {
-        const int mb = wave + e * WAVES;
-        if (mb >= MB) break;
-        Acc sum = red[0][mb][lane];
+    for (int e = 0; e < FIN; ++e) {
+        const int unit = wave + e * WAVES;
+        if (unit >= UNITS) break;
+        Acc sum = red[0][unit][lane];
 #pragma unroll
-        for (int w = 1; w < WAVES; ++w) sum += red[w][mb][lane];
-        const int m = m_base + mb * 16 + i;
+        for (int w = 1; w < WAVES; ++w) sum += red[w][unit][lane];
+        const int m = m_base + (unit % MB) * 16 + i;
+        const int n0 = (band0 + unit / MB) * 16 + 4 * g;
         if (m < M) {
             const EpilogueRegs eregs = finish_epilogue(ep, eraw[e]);
             uint16_t o[4];

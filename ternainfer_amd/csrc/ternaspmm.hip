@@ -146,12 +146,12 @@ void launch_repack(const Weights& w, uint32_t* packed, int N, int K, hipStream_t
                                                               packed, N, K);
 }
 
-template <typename Act, int WAVES, int MB, int DEPTH>
+template <typename Act, int WAVES, int MB, int DEPTH, int NB = 1>
 void launch_decode_packed_as(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N,
                              int K, hipStream_t st)
 {
-    const dim3 grid(N / 16, (M + 16 * MB - 1) / (16 * MB));
-    terna_decode_packed_kernel<Act, WAVES, MB, DEPTH><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, ep, M, N, K);
+    const dim3 grid(N / 16 / NB, (M + 16 * MB - 1) / (16 * MB));
+    terna_decode_packed_kernel<Act, WAVES, MB, DEPTH, NB><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, ep, M, N, K);
 }
 
 template <typename Act>
@@ -164,7 +164,15 @@ void launch_decode_packed(const Act* x, const uint32_t* packed, uint16_t* out, c
         // more than 512 bands (gate+up): per-wave set-up is as expensive as a few band-tiles, so fewer waves
         // with more band-tiles each win (measured 7.4 against 8.2 us)
         const bool narrow = forced ? forced == 4 : (N / 16 > 512);
-        if (narrow) launch_decode_packed_as<Act, 4, 1, 3>(x, packed, out, ep, M, N, K, st);
+        // ... and every workgroup stages the same activations: two bands per workgroup share one staging (N is a
+        // multiple of 64, so the band count is even).  Measured on gate+up, cold: 6.4 us against 7.3 us; four
+        // bands 6.7 us.  TERNASPMM_DECODE_BANDS=1 switches that off (tuning aid).
+        static const bool multi_off = [] {
+            const char* v = std::getenv("TERNASPMM_DECODE_BANDS");
+            return v && std::atoi(v) == 1;
+        }();
+        if (narrow && !forced && !multi_off) launch_decode_packed_as<Act, 8, 1, 2, 2>(x, packed, out, ep, M, N, K, st);
+        else if (narrow) launch_decode_packed_as<Act, 4, 1, 3>(x, packed, out, ep, M, N, K, st);
         else if (wide) launch_decode_packed_as<Act, 16, 1, 3>(x, packed, out, ep, M, N, K, st);
         else launch_decode_packed_as<Act, 8, 1, 2>(x, packed, out, ep, M, N, K, st);
     } else if (M <= 32) {

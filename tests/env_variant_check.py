@@ -1,6 +1,7 @@
 """Run under pytest by tests/test_gpu_parity.py::test_tile_and_path_overrides in a child process whose
 environment pins one of the library's tuning overrides (they are read once per process): large-M
-parity of both families on shapes with ragged M, N tails and odd / even tile counts."""
+parity of both families on shapes with ragged M, N tails and odd / even tile counts, the small-M
+kernels on both layouts, and the decode-step kernels (prologue inside the linear, attention)."""
 import sys
 
 import numpy as np
@@ -41,6 +42,13 @@ def main() -> int:
         gold = co.spmm_bf16(x, w, scale, 1)
         _check_bf16(run_bf16_packed(lib, packed, n, x, scale, 1), gold)
         _check_bf16(run_bf16(lib, fmt, x, scale, 1), gold)
+    # the decode-step kernels behind their overrides: prologue inside the linear, single-token attention
+    from tests import test_gpu_prologue as P
+    for m, n, k, ws_num, res in [(1, 13824, 2560, 2, True), (8, 13824, 2560, 2, True), (1, 2560, 2560, 1, False)]:
+        P.test_fused_prologue_linear(lib, m, n, k, ws_num, res)
+    P.test_decode_attention(lib, 1, 20, 5, 128, 1024, 1000, True)
+    P.test_decode_attention(lib, 2, 4, 2, 64, 300, 290, True)
+    P.test_rope_decode_attention_equals_the_two_launches(lib, 1, 20, 5, 128, 2048, 1500, 1, True)
     torch.cuda.synchronize()
     print("override check ok")
     return 0

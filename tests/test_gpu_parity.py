@@ -516,9 +516,12 @@ def test_kernel_binary_reference_command_line():
                                  {"TERNASPMM_PREFILL_BN": "256"}, {"TERNASPMM_PREFILL_BN": "128"},
                                  {"TERNASPMM_PREFILL_BM": "256"}, {"TERNASPMM_PREFILL_BM": "96"},
                                  {"TERNASPMM_PREFILL_XCD_MAP": "1"}, {"TERNASPMM_PREFILL_XCD_MAP": "1", "TERNASPMM_PREFILL_BM": "128"},
-                                 {"TERNASPMM_DECODE_WAVES": "4"}, {"TERNASPMM_DECODE_WAVES": "8"}, {"TERNASPMM_DECODE_WAVES": "16"}])
+                                 {"TERNASPMM_DECODE_WAVES": "4"}, {"TERNASPMM_DECODE_WAVES": "8"}, {"TERNASPMM_DECODE_WAVES": "16"},
+                                 {"TERNASPMM_DECODE_BANDS": "1"}, {"TERNASPMM_FUSED_BANDS": "1"},
+                                 {"TERNASPMM_FUSED_BANDS_WAVES": "8"}, {"TERNASPMM_FUSED_WAVES": "8"},
+                                 {"TERNASPMM_ATTN_WAVES": "4"}, {"TERNASPMM_ATTN_SPLITS": "2"}, {"TERNASPMM_ATTN_SPLITS": "8"}])
 def test_tile_and_path_overrides(env):
-    """Every large-M tile shape and the register-staged path behind the library's tuning overrides
+    """Every tile shape, launch shape and path behind the library's tuning overrides
     (read once per process, hence a child process): tests/env_variant_check.py must pass under each."""
     import subprocess
     import sys
