@@ -61,12 +61,20 @@ def f32_to_bf16_bits(x):
     return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
 
 
+def make_row_skewed(n, k, seed):
+    """Each output row's zero fraction drawn U[0.2, 0.7]; signs balanced (configs[3])."""
+    rng = np.random.default_rng(seed)
+    p0 = rng.uniform(0.2, 0.7, size=(n, 1))
+    nz = (rng.random((n, k)) >= p0).astype(np.int8)
+    return nz * (1 - 2 * rng.integers(0, 2, size=(n, k), dtype=np.int8))
+
+
 class Matrix:
     """One ternary matrix: host copy, `copies` device copies of the format, activations, output."""
 
-    def __init__(self, name, n, k, m, copies, seed, torch, T):
+    def __init__(self, name, n, k, m, copies, seed, torch, T, w=None):
         self.name, self.n, self.k, self.m = name, n, k, m
-        self.w = make_ternary(n, k, 0.40, seed)
+        self.w = make_ternary(n, k, 0.40, seed) if w is None else w
         vals, off, med, bm = T.compress_weight(torch.from_numpy(self.w))
         self.host_format = (vals.numpy(), off.numpy(), med.numpy(), bm.numpy())
         self.n_sign_words = int(vals.numel())
@@ -203,6 +211,50 @@ def run_model(args, torch):
         "model_build_s": build_s, "first_tokens": toks[0, :8].tolist()}))
 
 
+def run_sweep(args, torch, T, lib):
+    """configs[3]: sparsity / structure sweep at M = 16 on K = N = 2560 and on K = 6912, N = 2560 -- global zero
+    fraction 0.20 / 0.33 / 0.45 / 0.60 and a row-skewed matrix -- on both weight layouts.  The reference format's
+    size, and with it the work of the kernels that read it, follows the number of nonzeros; the 2-bit layout and
+    its kernels do not.  A step is one pass over the ten matrices (cold: --layers copies of each, rotated)."""
+    m = args.m if args.m != 8 else 16
+    copies = min(args.layers, 24)
+    from oracle import terna_oracle as O
+    cases, mats = [], []
+    for n, k in [(2560, 2560), (2560, 6912)]:
+        for kind in ["p20", "p33", "p45", "p60", "skewed"]:
+            seed = 20260400 + len(cases)
+            w = make_row_skewed(n, k, seed) if kind == "skewed" else make_ternary(n, k, int(kind[1:]) / 100.0, seed)
+            cases.append((f"{kind}_{k}x{n}", float((w == 0).mean())))
+            mats.append(Matrix(cases[-1][0], n, k, m, copies, seed, torch, T, w=w))
+    detail, total_bytes, total_us = {}, 0, {"packed": 0.0, "reference": 0.0}
+    for (name, zero_frac), mt in zip(cases, mats):
+        entry = {"zero_fraction": zero_frac, "alg_bytes": mt.alg_bytes}
+        for layout in ("packed", "reference"):
+            g = capture(torch, lambda s, mt=mt, layout=layout: [mt.launch(lib, c, s, layout) for c in range(copies)])
+            us = time_graph(torch, g, max(args.steps // 2, 5), args.warmup) * 1e3 / copies
+            entry[f"{layout}_us"] = us
+            entry[f"{layout}_GBps"] = mt.alg_bytes / us / 1e3
+            total_us[layout] += us
+            # correctness gate of the run: the last launch's output against the fp64 golden
+            gold = O.spmm_bf16_golden(mt.x_bits, mt.w, mt.scale_host, 1)
+            got = O.bf16_bits_to_f32(mt.out.cpu().numpy().view(np.uint16)).astype(np.float64)
+            assert np.abs(got - gold).max() <= 1e-2 * np.abs(gold).max(), (name, layout)
+        detail[name] = entry
+        total_bytes += mt.alg_bytes
+    gbps = total_bytes / total_us[args.layout] / 1e3
+    print(json.dumps({
+        "metric": "TernaSpMM GB/s + %HBM roofline (M=8,K=N=2560); 2B-shape decode tok/s", "value": gbps, "unit": "GB/s",
+        "n_gpus": 1, "steps": max(args.steps // 2, 5), "warmup": args.warmup, "ms_per_step": total_us[args.layout] * 1e-3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"configs[3]: sparsity / structure sweep, M={m}, K=N=2560 and K=6912 N=2560, zero fraction "
+                               f"0.20 / 0.33 / 0.45 / 0.60 and row-skewed U[0.2, 0.7]; {copies} weight copies per matrix, "
+                               f"value = the ten matrices on the {args.layout} layout",
+                   "m": m, "layout": args.layout},
+        "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
+                     "traffic": None},
+        "per_case": detail}))
+
+
 def run_prefill(args, torch, T, lib):
     """configs[2]: the four BitNet-2B matrices at M in {256, 512, 2048}, bf16 activations with 1% of
     the channels scaled x20 (--act int8: the same activations quantised per row to int8, the
@@ -333,9 +385,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--m", type=int, default=8, help="activation rows per call (decode batch)")
     ap.add_argument("--layers", type=int, default=30, help="distinct weight copies per matrix")
-    ap.add_argument("--workload", choices=["decode", "prefill", "model"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "prefill", "model", "sweep"], default="decode",
                     help="decode: the headline small-M HBM-bound pass; prefill: the M>=256 MFMA-bound pass; "
-                         "model: random-init BitNet-2B-shaped decoder, 128-token prompt + 256 greedy tokens")
+                         "model: random-init BitNet-2B-shaped decoder, 128-token prompt + 256 greedy tokens; "
+                         "sweep: the sparsity / structure sweep at M=16")
     ap.add_argument("--batch", type=int, default=1, help="sequences decoded together (model workload)")
     ap.add_argument("--act", choices=["int8", "bf16"], default=None,
                     help="activations into the ternary linears: int8 + per-row scale (the reference's SpBitLinear; "
@@ -370,6 +423,9 @@ def main():
         return
     if args.workload == "model":
         run_model(args, torch)
+        return
+    if args.workload == "sweep":
+        run_sweep(args, torch, T, lib)
         return
 
     mats = [Matrix(name, n, k, args.m, args.layers, 20260200 + 10 * j, torch, T)
