@@ -8,7 +8,7 @@
 // 9 us pair in a decode step -- disappears.  Every workgroup recomputes the same statistics from
 // the same values in the same order, so all bands see identical int8 activations.
 //
-//   h  = x, or bf16(x + residual)            (band 0 also writes h to sum_out: the new stream),
+//   h  = x, or bf16(x + residual)            (workgroup 0 also writes h to sum_out: the new stream),
 //        or bf16(bf16(relu(x1)^2) * x3)      (gated FFN: x = [x1 | x3], 2K columns per row)
 //   y  = bf16(h * rsqrt(mean(h^2) + eps) * norm_w)
 //   s  = bf16(127 / max(max|y|, 1e-5)),  q = clamp(rint(y * s), -128, 127)
@@ -17,9 +17,10 @@
 // Phases of a wave (T = its tiles, at most TMAX):
 //   A  request everything: T weight words, T activation pieces (x, residual), then the norm
 //      weights of its columns; h -> registers (packed bf16), sum of squares per row
-//   B  rows' sums: the lanes that share a row (shuffles), then the waves in LDS  -- barrier 1
+//   B  rows' sums: the lanes that share a row (data-parallel permutes), then the waves in LDS -- barrier 1
 //   C  y -> registers, max |y| per row, same reduction                      -- barrier 2
-//   D  per tile: quantise, int8 slab -> wave-private LDS -> operand order, MFMA
+//   D  per tile: quantise, int8 slab -> wave-private LDS -> operand order (a single row: gathered
+//      with data-parallel permutes, no LDS), MFMA
 //   E  cross-wave sum of the accumulators + epilogue (wave b finishes band b) -- barrier 3
 //
 // NB = bands of W per workgroup.  The prologue is repeated by every workgroup, so a matrix with
