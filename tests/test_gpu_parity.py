@@ -423,6 +423,18 @@ def test_packed_int8_bit_exact(lib, m, n, k, ws_num):
     assert (run_i8_packed(lib, packed, n, xq, s, WS, ws_num, 1) == O.spmm_i8(xq, w, s, WS, ws_num, 1)).all()
 
 
+@pytest.mark.parametrize("m", [1, 8, 16])
+@pytest.mark.parametrize("n,k,ws_num", [(13824, 2560, 2), (8256, 192, 1), (8320, 64, 4)])
+def test_packed_int8_many_bands_bit_exact(lib, m, n, k, ws_num):
+    """More than 512 bands: the small-M kernel takes two bands per workgroup (gate+up and two synthetic
+    shapes with 516 / 520 bands, one to three k-tiles, several weight-scale groups)."""
+    w = make_ternary(n, k, 0.40, 430 + m + n % 97)
+    packed = repack(lib, DeviceFormat(w))
+    xq, s = make_int8_activations(m, k, 431 + m + k)
+    print(f"[case] packed int8, many bands m={m} n={n} k={k}", flush=True)
+    assert (run_i8_packed(lib, packed, n, xq, s, WS, ws_num) == O.spmm_i8(xq, w, s, WS, ws_num, 0)).all()
+
+
 @pytest.mark.parametrize("m", [1, 70, 256])
 @pytest.mark.parametrize("n,k,ws_num", [(64, 64, 1), (192, 448, 1), (3840, 2560, 3), (2560, 6912, 1)])
 def test_packed_int8_mfma_kernel_tile_counts_and_2b_shapes(lib, m, n, k, ws_num):
