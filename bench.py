@@ -189,6 +189,8 @@ def run_model(args, torch):
     t0 = time.perf_counter()
     args.act = args.act or "int8"
     model = Transformer(margs, seed=20260500, act=args.act)
+    if not args.no_prefetch:     # weights of the following launches, pulled through the caches during the attention launch
+        model.enable_prefetch(True, ("wo", "w13", "w2", "next_wqkv") if args.batch <= 2 else ("wo", "w13"))
     torch.cuda.synchronize()
     build_s = time.perf_counter() - t0
     gen = torch.Generator(device="cuda").manual_seed(20260501)
@@ -205,7 +207,8 @@ def run_model(args, torch):
                                f"{args.act} activations into the ternary linears, weights in P2 layout, one HIP graph per "
                                "decode step; norms, gate, activation quantisation, RoPE, cache write and "
                                "single-token attention are library kernels, prefill attention and the bf16 LM head "
-                               "are PyTorch-ROCm ops",
+                               "are PyTorch-ROCm ops" + ("" if args.no_prefetch else "; the idle CUs of the attention launch "
+                                                         "prefetch the weights of the launches that follow"),
                    "batch": args.batch, "act": args.act},
         "prefill_tokens_per_s": args.batch * 128 / prefill_s, "prefill_s": prefill_s, "decode_s": decode_s,
         "model_build_s": build_s, "first_tokens": toks[0, :8].tolist()}))
@@ -396,6 +399,8 @@ def main():
     ap.add_argument("--layout", choices=["packed", "reference"], default="packed",
                     help="packed: weights repacked once at load time to the library's P2 layout (bit-exact); "
                          "reference: kernels read the reference's compressed format directly")
+    ap.add_argument("--no-prefetch", action="store_true",
+                    help="model workload: no weight prefetch by the idle CUs of the attention launch")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-per-shape", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",

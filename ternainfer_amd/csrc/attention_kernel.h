@@ -126,6 +126,47 @@ __global__ __launch_bounds__(256) void terna_rope_kv_store_kernel(
 // after every launch) merges the SP partials in split order -- the result does not depend on
 // which workgroup arrives last -- and writes the output row.
 constexpr int kAttentionMaxSplits = 8;
+// Extra workgroups of the attention launch (blockIdx.x >= heads) that pull up to kAttentionPrefetchRegions regions of
+// device memory through the caches while the heads' workgroups -- one CU each -- do the attention:
+// the weights of the launches that follow.  Unit u of a region goes to a workgroup on XCD (u mod 8),
+// where the consuming workgroup u runs if its dispatch is spread round robin from XCD 0 as well.
+constexpr int kAttentionPrefetchRegions = 4;
+struct AttentionPrefetch {
+    const u32x4* base[kAttentionPrefetchRegions];
+    long long units[kAttentionPrefetchRegions];
+    long long total_vecs[kAttentionPrefetchRegions];
+    int unit_vecs[kAttentionPrefetchRegions];
+    int count;            // regions
+    int workgroups;       // extra workgroups, a multiple of 8 (0: none)
+};
+
+__device__ __forceinline__ void attention_prefetch_role(const AttentionPrefetch& pf, int heads, int nthreads)
+{
+    const int p = blockIdx.x - heads;
+    const int xcd = blockIdx.x & 7;
+    const int per_xcd = pf.workgroups >> 3;
+    // rank of this workgroup among those of its XCD
+    const int rank = (p - ((xcd - (heads & 7) + 8) & 7)) >> 3;
+    uint32_t seen = 0;
+    for (int r = 0; r < pf.count; ++r) {
+        for (long long u = xcd + 8ll * rank; u < pf.units[r]; u += 8ll * per_xcd) {
+            const long long first = u * pf.unit_vecs[r];
+            for (int v0 = threadIdx.x; v0 < pf.unit_vecs[r]; v0 += 4 * nthreads) {
+                u32x4 q[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int vv = v0 + j * nthreads;
+                    const bool ok = vv < pf.unit_vecs[r] && first + vv < pf.total_vecs[r];
+                    q[j] = ok ? pf.base[r][first + vv] : u32x4{0u, 0u, 0u, 0u};
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) seen |= q[j].x & q[j].y & q[j].z & q[j].w;
+            }
+        }
+    }
+    if (seen == 0xffffffffu && pf.count > kAttentionPrefetchRegions) *const_cast<u32x4*>(pf.base[0]) = u32x4{seen, 0u, 0u, 0u};   // never true: keeps the loads
+}
+
 constexpr size_t decode_attention_lds_bytes(int D, int NW, int S)
 {
     return (static_cast<size_t>(S) + (64 * NW / (D / 8)) * D + 64 * NW) * sizeof(float);
@@ -136,7 +177,7 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
     const float* __restrict__ cosv, const float* __restrict__ sinv,
     const long long* __restrict__ pos, uint16_t* __restrict__ out, int H, int KV, int S, float scale,
-    float* partial, int* arrived, int splits)
+    float* partial, int* arrived, int splits, AttentionPrefetch pf, int heads)
 {
     static_assert(D == 64 || D == 128, "head dimension");
     constexpr int CH = D / 8;                    // 8-dimension chunks of a row
@@ -149,6 +190,10 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     float* score = part2 + GROUPS * D;           // [S]
     __shared__ float red[2 * NW];
     __shared__ int last_flag;
+    if (static_cast<int>(blockIdx.x) >= heads) {             // prefetch-only workgroups
+        attention_prefetch_role(pf, heads, 64 * NW);
+        return;
+    }
 
     // SP = splits of the cache (= gridDim.y), sp = this workgroup's split; constants in the unsplit kernel
     const int SP = SPLIT ? splits : 1, sp = SPLIT ? blockIdx.y : 0;

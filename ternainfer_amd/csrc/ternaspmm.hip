@@ -425,26 +425,28 @@ int attention_splits(int B, int H, int S, const void* workspace)
 template <int D, bool ROPE, bool ADJ, int NW, bool SPLIT>
 void launch_attention_as(const uint16_t* q, uint16_t* ck, uint16_t* cv, const float* cos, const float* sin,
                          const long long* pos, uint16_t* out, int B, int H, int KV, int S, float scale, int splits,
-                         void* workspace, hipStream_t st)
+                         void* workspace, const AttentionPrefetch& pf_in, hipStream_t st)
 {
+    AttentionPrefetch pf = pf_in;
+    if (splits > 1) pf.workgroups = 0;                       // the split grid is two-dimensional: no extra workgroups
     auto kernel = terna_decode_attention_kernel<D, ROPE, ADJ, NW, SPLIT>;
     const size_t lds = decode_attention_lds_bytes(D, NW, S);
     if (lds > 64 * 1024) allow_dynamic_lds(kernel, 160 * 1024, "hipFuncSetAttribute(decode attention)", __LINE__);
     int* arrived = static_cast<int*>(workspace);
     float* partial = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + attention_counter_bytes(B, H)) : nullptr;
-    kernel<<<dim3(B * H, splits), dim3(64 * NW), lds, st>>>(q, ck, cv, cos, sin, pos, out, H, KV, S, scale, partial, arrived,
-                                                             splits);
+    kernel<<<dim3(B * H + pf.workgroups, splits), dim3(64 * NW), lds, st>>>(q, ck, cv, cos, sin, pos, out, H, KV, S, scale,
+                                                                           partial, arrived, splits, pf, B * H);
 }
 
 template <bool ROPE, bool ADJ>
 void launch_attention(const uint16_t* q, uint16_t* ck, uint16_t* cv, const float* cos, const float* sin,
                              const long long* pos, uint16_t* out, int B, int H, int KV, int D, int S, float scale,
-                             void* workspace, hipStream_t st)
+                             void* workspace, const AttentionPrefetch& pf, hipStream_t st)
 {
     const int splits = attention_splits(B, H, S, workspace);
     const int nw = splits > 1 ? 4 : attention_waves(B, H);       // a split is a short prefix: the narrow workgroup
 #define TERNA_ATTN(DIM, NWAVES, SPLIT) \
-    launch_attention_as<DIM, ROPE, ADJ, NWAVES, SPLIT>(q, ck, cv, cos, sin, pos, out, B, H, KV, S, scale, splits, workspace, st)
+    launch_attention_as<DIM, ROPE, ADJ, NWAVES, SPLIT>(q, ck, cv, cos, sin, pos, out, B, H, KV, S, scale, splits, workspace, pf, st)
     if (D == 128) {
         if (splits > 1) TERNA_ATTN(128, 4, true);
         else if (nw == 8) TERNA_ATTN(128, 8, false);
@@ -804,7 +806,7 @@ void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, 
     if (!attention_args_ok("ternaspmm_decode_attention", B, H, KV, D, S)) return;
     // the kernel writes the caches only in its ROPE variant
     launch_attention<false, false>(q, const_cast<uint16_t*>(cache_k), const_cast<uint16_t*>(cache_v), nullptr, nullptr, pos,
-                                   out, B, H, KV, D, S, scale, workspace, static_cast<hipStream_t>(stream));
+                                   out, B, H, KV, D, S, scale, workspace, AttentionPrefetch{}, static_cast<hipStream_t>(stream));
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_decode_attention", e, __LINE__);
 }
@@ -815,10 +817,41 @@ void ternaspmm_rope_decode_attention(const terna_bf16* qkv, const float* cos, co
 {
     if (!attention_args_ok("ternaspmm_rope_decode_attention", B, H, KV, D, S)) return;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (adjacent) launch_attention<true, true>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, workspace, st);
-    else launch_attention<true, false>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, workspace, st);
+    if (adjacent) launch_attention<true, true>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, workspace, AttentionPrefetch{}, st);
+    else launch_attention<true, false>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, workspace, AttentionPrefetch{}, st);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_rope_decode_attention", e, __LINE__);
+}
+
+void ternaspmm_rope_decode_attention_prefetch(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
+                                              terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
+                                              int D, int S, float scale, int adjacent, void* workspace,
+                                              const void* const* pf_ptr, const long long* pf_bytes, const long long* pf_unit_bytes,
+                                              int pf_count, terna_stream stream)
+{
+    if (!attention_args_ok("ternaspmm_rope_decode_attention_prefetch", B, H, KV, D, S)) return;
+    AttentionPrefetch pf{};
+    for (int r = 0; r < pf_count && pf.count < kAttentionPrefetchRegions; ++r) {
+        if (pf_ptr[r] == nullptr || (reinterpret_cast<uintptr_t>(pf_ptr[r]) & 15) || pf_unit_bytes[r] < 16 || (pf_unit_bytes[r] & 15) ||
+            pf_unit_bytes[r] > (1ll << 30) || pf_bytes[r] < 16)
+            continue;
+        const int c = pf.count++;
+        pf.base[c] = static_cast<const u32x4*>(pf_ptr[r]);
+        pf.total_vecs[c] = pf_bytes[r] / 16;
+        pf.unit_vecs[c] = static_cast<int>(pf_unit_bytes[r] / 16);
+        pf.units[c] = (pf.total_vecs[c] + pf.unit_vecs[c] - 1) / pf.unit_vecs[c];
+    }
+    // the heads take B*H CUs; the rest of the chip prefetches
+    static const int forced_wgs = [] {
+        const char* v = std::getenv("TERNASPMM_ATTN_PREFETCH_WGS");
+        return v ? std::atoi(v) / 8 * 8 : -1;
+    }();
+    pf.workgroups = pf.count > 0 && B * H < 232 ? (forced_wgs >= 0 ? forced_wgs : (256 - B * H) / 8 * 8) : 0;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (adjacent) launch_attention<true, true>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, workspace, pf, st);
+    else launch_attention<true, false>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, workspace, pf, st);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_rope_decode_attention_prefetch", e, __LINE__);
 }
 
 void ternaspmm_argmax_bf16(const terna_bf16* x, long long* out, int B, int V, terna_stream stream)

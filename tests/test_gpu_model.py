@@ -89,6 +89,10 @@ def test_toy_model_greedy_decode_graph_equals_eager():
     a, _, _ = greedy_decode(model, prompt, 12, use_graph=True)
     b, _, _ = greedy_decode(model, prompt, 12, use_graph=False)
     assert torch.equal(a, b)
+    model.enable_prefetch()                      # idle CUs of the attention launch prefetch the next weights: same tokens
+    c, _, _ = greedy_decode(model, prompt, 12, use_graph=True)
+    model.enable_prefetch(False)
+    assert torch.equal(a, c)
 
 
 def test_converted_checkpoint_loads_and_matches_cpu_golden(tmp_path):

@@ -379,3 +379,37 @@ def test_rope_decode_attention_equals_the_two_launches(lib, b, h, kv, d, s_max, 
     torch.cuda.synchronize()
     assert torch.equal(ck1, ck2) and torch.equal(cv1, cv2)
     assert torch.equal(o1, o2)
+
+
+@pytest.mark.parametrize("b,h,kv,d,s_max,n", [(1, 20, 5, 128, 384, 200), (8, 20, 5, 128, 384, 300), (2, 4, 2, 64, 40, 17)])
+def test_rope_decode_attention_with_prefetch_regions(lib, b, h, kv, d, s_max, n):
+    """The variant with prefetch workgroups: same output and caches as the plain entry point, bit for bit, and the
+    prefetched regions (sizes that are and are not multiples of the unit, a unit larger than the region, a
+    region the call must skip) are left untouched."""
+    qkv = make_bf16_activations(b, (h + 2 * kv) * d, 931 + n)
+    k0 = make_bf16_activations(b * kv * s_max, d, 932 + n).reshape(b, kv, s_max, d)
+    v0 = make_bf16_activations(b * kv * s_max, d, 933 + n).reshape(b, kv, s_max, d)
+    pos = np.array([n - 1], np.int64)
+    ang = (pos[:, None] * (1.0 / 500000.0 ** (np.arange(0, d, 2) / d))[None, :]).astype(np.float32)
+    xd, cd, sd, pd = _dev(qkv), _dev(np.cos(ang).astype(np.float32)), _dev(np.sin(ang).astype(np.float32)), _dev(pos)
+    scale = float(d) ** -0.5
+    ck1, cv1, ck2, cv2 = _dev(k0), _dev(v0), _dev(k0), _dev(v0)
+    o1 = torch.zeros((b, h * d), dtype=torch.int16, device="cuda")
+    o2 = torch.zeros_like(o1)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    regions = [torch.randint(-2 ** 31, 2 ** 31 - 1, (nwords,), dtype=torch.int32, device="cuda", generator=gen)
+               for nwords in (40 * 2560, 3 * 2560 + 36, 64, 4096)]
+    before = [r.clone() for r in regions]
+    units = [10240, 10240, 40960, 27648]
+    count = len(regions) + 1
+    ptrs = (ctypes.c_void_p * count)(*([r.data_ptr() for r in regions] + [None]))           # the last one is skipped
+    sizes = (ctypes.c_longlong * count)(*([r.numel() * 4 for r in regions] + [1024]))
+    unit_arr = (ctypes.c_longlong * count)(*(units + [16]))
+    lib.ternaspmm_rope_decode_attention(_vp(xd), _vp(cd), _vp(sd), _vp(pd), _vp(ck1), _vp(cv1), _vp(o1), b, h, kv, d, s_max,
+                                        scale, 1, None, None)
+    print(f"[case] rope + decode attention with prefetch b={b} h={h} d={d} n={n}", flush=True)
+    lib.ternaspmm_rope_decode_attention_prefetch(_vp(xd), _vp(cd), _vp(sd), _vp(pd), _vp(ck2), _vp(cv2), _vp(o2), b, h, kv, d,
+                                                 s_max, scale, 1, None, ptrs, sizes, unit_arr, count, None)
+    torch.cuda.synchronize()
+    assert torch.equal(o1, o2) and torch.equal(ck1, ck2) and torch.equal(cv1, cv2)
+    assert all(torch.equal(r, r0) for r, r0 in zip(regions, before))
