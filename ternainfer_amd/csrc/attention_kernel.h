@@ -201,6 +201,7 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     auto cache_slot = [&](int l) { return (((l >> 4) * SP + sp) << 4) + (l & 15); };
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
+    TERNA_TS(0);
     const int b = blockIdx.x / H, h = blockIdx.x - b * H;
     const int kvh = h / (H / KV);
     const int n = static_cast<int>(pos[0]) + 1;
@@ -316,6 +317,7 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
         }
     }
 
+    TERNA_TS(1);
     float mx = -INFINITY;
     auto score_tile = [&](int ltile, const u32x4 (&kin)[NJ]) {       // ltile: local tile of this split
         const int tile = ltile * SP + sp;
@@ -358,6 +360,7 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
         for (int jj = 0; jj < NJ; ++jj) k[jj] = *reinterpret_cast<const u32x4*>(kp + 32 * jj);
         score_tile(tile, k);
     }
+    TERNA_TS(2);
     mx = wave_max(mx);
     if (lane == 0) red[wave] = mx;
     __syncthreads();
@@ -372,6 +375,7 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
         score[l] = p;
         sum += p;
     }
+    TERNA_TS(3);
     sum = wave_sum(sum);
     if (lane == 0) red[NW + wave] = sum;
     __syncthreads();
@@ -380,6 +384,7 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     for (int w = 1; w < NW; ++w) sum += red[NW + w];
 
     // ---- pass 3: weighted sum of the value rows, VU rows per round (the first round is already here)
+    TERNA_TS(4);
     float acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
     for (int l0 = slice; l0 < nl; l0 += VU * SLICES) {
         if (l0 != slice) {                       // all VU rows of the round requested before any is used
@@ -406,6 +411,7 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
             for (int e = 0; e < 8; ++e) acc[e] = fmaf(p, vf[e], acc[e]);
         }
     }
+    TERNA_TS(5);
 #pragma unroll
     for (int e = 0; e < 8; ++e) part[slice * D + chunk * 8 + e] = acc[e];
     __syncthreads();
@@ -422,6 +428,7 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
 #pragma unroll
         for (int grp = 0; grp < GROUPS; ++grp) o += part2[grp * D + tid];
     }
+    TERNA_TS(6);
     uint16_t* orow = out + (static_cast<size_t>(b) * H + h) * D;
     if (!SPLIT || SP == 1) {
         if (tid < D) orow[tid] = float_to_bf16_bits(o / sum);

@@ -24,10 +24,6 @@
 
 #include "terna_common.h"
 
-// Phase timestamps for tuning builds; expands to nothing in the shipped library.
-#ifndef TERNA_TS
-#define TERNA_TS(slot)
-#endif
 
 namespace terna {
 
