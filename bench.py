@@ -190,7 +190,7 @@ def run_model(args, torch):
     args.act = args.act or "int8"
     model = Transformer(margs, seed=20260500, act=args.act)
     if not args.no_prefetch:     # weights of the following launches, pulled through the caches during the attention launch
-        model.enable_prefetch(True, ("wo", "w13", "w2", "next_wqkv") if args.batch <= 2 else ("wo", "w13"))
+        model.enable_prefetch(True, ("wo", "w13", "w2", "next_wqkv", "norms") if args.batch <= 2 else ("wo", "w13", "norms"))
     torch.cuda.synchronize()
     build_s = time.perf_counter() - t0
     gen = torch.Generator(device="cuda").manual_seed(20260501)

@@ -130,12 +130,12 @@ constexpr int kAttentionMaxSplits = 8;
 // device memory through the caches while the heads' workgroups -- one CU each -- do the attention:
 // the weights of the launches that follow.  Unit u of a region goes to a workgroup on XCD (u mod 8),
 // where the consuming workgroup u runs if its dispatch is spread round robin from XCD 0 as well.
-constexpr int kAttentionPrefetchRegions = 4;
+constexpr int kAttentionPrefetchRegions = 6;
 struct AttentionPrefetch {
     const u32x4* base[kAttentionPrefetchRegions];
     long long units[kAttentionPrefetchRegions];
     long long total_vecs[kAttentionPrefetchRegions];
-    int unit_vecs[kAttentionPrefetchRegions];
+    int unit_vecs[kAttentionPrefetchRegions];     // 0: a small region that every XCD fetches whole
     int count;            // regions
     int workgroups;       // extra workgroups, a multiple of 8 (0: none)
 };
@@ -149,6 +149,15 @@ __device__ __forceinline__ void attention_prefetch_role(const AttentionPrefetch&
     const int rank = (p - ((xcd - (heads & 7) + 8) & 7)) >> 3;
     uint32_t seen = 0;
     for (int r = 0; r < pf.count; ++r) {
+        if (pf.unit_vecs[r] == 0) {              // read by every workgroup of the consumers: once per XCD
+            if (rank == 0) {
+                for (long long v = threadIdx.x; v < pf.total_vecs[r]; v += nthreads) {
+                    const u32x4 q = pf.base[r][v];
+                    seen |= q.x & q.y & q.z & q.w;
+                }
+            }
+            continue;
+        }
         for (long long u = xcd + 8ll * rank; u < pf.units[r]; u += 8ll * per_xcd) {
             const long long first = u * pf.unit_vecs[r];
             for (int v0 = threadIdx.x; v0 < pf.unit_vecs[r]; v0 += 4 * nthreads) {

@@ -832,14 +832,16 @@ void ternaspmm_rope_decode_attention_prefetch(const terna_bf16* qkv, const float
     if (!attention_args_ok("ternaspmm_rope_decode_attention_prefetch", B, H, KV, D, S)) return;
     AttentionPrefetch pf{};
     for (int r = 0; r < pf_count && pf.count < kAttentionPrefetchRegions; ++r) {
-        if (pf_ptr[r] == nullptr || (reinterpret_cast<uintptr_t>(pf_ptr[r]) & 15) || pf_unit_bytes[r] < 16 || (pf_unit_bytes[r] & 15) ||
-            pf_unit_bytes[r] > (1ll << 30) || pf_bytes[r] < 16)
+        const bool broadcast = pf_unit_bytes[r] == 0;        // every XCD fetches the whole (small) region
+        if (pf_ptr[r] == nullptr || (reinterpret_cast<uintptr_t>(pf_ptr[r]) & 15) || pf_bytes[r] < 16 ||
+            (!broadcast && (pf_unit_bytes[r] < 16 || (pf_unit_bytes[r] & 15) || pf_unit_bytes[r] > (1ll << 30))) ||
+            (broadcast && pf_bytes[r] > (1ll << 20)))
             continue;
         const int c = pf.count++;
         pf.base[c] = static_cast<const u32x4*>(pf_ptr[r]);
         pf.total_vecs[c] = pf_bytes[r] / 16;
-        pf.unit_vecs[c] = static_cast<int>(pf_unit_bytes[r] / 16);
-        pf.units[c] = (pf.total_vecs[c] + pf.unit_vecs[c] - 1) / pf.unit_vecs[c];
+        pf.unit_vecs[c] = broadcast ? 0 : static_cast<int>(pf_unit_bytes[r] / 16);
+        pf.units[c] = broadcast ? 1 : (pf.total_vecs[c] + pf.unit_vecs[c] - 1) / pf.unit_vecs[c];
     }
     // the heads take B*H CUs; the rest of the chip prefetches
     static const int forced_wgs = [] {

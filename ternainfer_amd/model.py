@@ -254,7 +254,25 @@ class Transformer:
         model.norm = dic["norm.weight"].to(device="cuda", dtype=torch.bfloat16).contiguous()
         return model
 
-    def enable_prefetch(self, on: bool = True, which=("wo", "w13", "w2", "next_wqkv")) -> None:
+    def pack_norm_weights(self) -> None:
+        """All norm weights of the model in one buffer, in the order the decode step reads them, so that a block's
+        attention launch can prefetch the ones of the launches that follow as one region."""
+        names = ("attention_norm", "attn_sub_norm", "ffn_norm", "ffn_sub_norm")
+        total = sum(getattr(blk, nm).numel() for blk in self.layers for nm in names)
+        buf = torch.empty(total, dtype=torch.bfloat16, device=self.norm.device)
+        off = 0
+        for blk in self.layers:
+            blk.norm_offsets = {}
+            for nm in names:
+                w = getattr(blk, nm)
+                view = buf[off:off + w.numel()]
+                view.copy_(w)
+                setattr(blk, nm, view)
+                blk.norm_offsets[nm] = off
+                off += w.numel()
+        self.norm_buffer = buf
+
+    def enable_prefetch(self, on: bool = True, which=("wo", "w13", "w2", "next_wqkv", "norms")) -> None:
         """Single-token steps: while a block's attention runs (one workgroup per head), extra workgroups of that
         launch prefetch the weights of its O, gate+up and down projections and of the next block's QKV projection
         (`which` picks among them).  Measured on MI355X: +6 % tokens/s at batch 1 with all four; at batch 8, where
@@ -274,6 +292,14 @@ class Transformer:
             if "next_wqkv" in which and n + 1 < len(self.layers):
                 nxt = self.layers[n + 1].wqkv
                 regions.append((nxt.packed, unit(nxt, 1)))
+            if "norms" in which:
+                if getattr(self, "norm_buffer", None) is None:
+                    self.pack_norm_weights()
+                # attn_sub_norm, ffn_norm, ffn_sub_norm of this block and attention_norm of the next: contiguous
+                first = blk.norm_offsets["attn_sub_norm"]
+                last = self.layers[n + 1].norm_offsets["attn_sub_norm"] if n + 1 < len(self.layers) else self.norm_buffer.numel()
+                first -= first % 8                                        # 16-byte aligned start
+                regions.append((self.norm_buffer[first:last], 0))         # unit 0: every XCD fetches it whole
             count = len(regions)
             ptrs = (ctypes.c_void_p * count)(*[w.data_ptr() for w, _ in regions])
             sizes = (ctypes.c_longlong * count)(*[w.numel() * w.element_size() for w, _ in regions])
