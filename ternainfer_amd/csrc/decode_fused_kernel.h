@@ -97,28 +97,35 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
     const uint16_t* second = MODE == FUSED_GLU ? x + K : residual;
 
     // ---- phase A: request everything
+    // Straight-line code: every load is unconditional on a clamped address and what must be zero is
+    // zeroed by a select afterwards.  Loads inside branches end up with a full wait at every join,
+    // i.e. one memory round trip per tile.
     uint32_t wword[NB][TMAX];
     Piece xr[TMAX], rr[TMAX], nw[TMAX];
+    bool use[TMAX];
 #pragma unroll
     for (int t = 0; t < TMAX; ++t) {
         const int j = wave + WAVES * t;
         const bool valid = j < ktiles;
+        const int jc = valid ? j : 0;
+        use[t] = valid && row_ok;
 #pragma unroll
-        for (int b = 0; b < NB; ++b)
-            wword[b][t] = valid ? packed[(static_cast<size_t>(band0 + b) * ktiles + j) * 64 + i * 4 + g] : 0u;
-        const size_t off = static_cast<size_t>(row_ok ? row : 0) * pitch + (valid ? j : 0) * 64 + cl;
-        if (valid && row_ok) {
-            xr[t].load(x + off);
-            if constexpr (RES) rr[t].load(second + off);
-        } else {
-            xr[t].zero();
-            if constexpr (RES) rr[t].zero();
-        }
+        for (int b = 0; b < NB; ++b) wword[b][t] = packed[(static_cast<size_t>(band0 + b) * ktiles + jc) * 64 + i * 4 + g];
+        const size_t off = static_cast<size_t>(row_ok ? row : 0) * pitch + jc * 64 + cl;
+        xr[t].load(x + off);
+        if constexpr (RES) rr[t].load(second + off);
+        nw[t].load(norm_w + jc * 64 + cl);
     }
 #pragma unroll
     for (int t = 0; t < TMAX; ++t) {
-        const int j = wave + WAVES * t;
-        nw[t].load(norm_w + (j < ktiles ? j : 0) * 64 + cl);
+        if (!use[t]) {
+            xr[t].zero();
+            if constexpr (RES) rr[t].zero();
+        }
+        if (wave + WAVES * t >= ktiles) {
+#pragma unroll
+            for (int b = 0; b < NB; ++b) wword[b][t] = 0u;
+        }
     }
     // wave b finishes band b: its weight-group scales are requested now, converted at the very end
     const Epilogue ep{nullptr, ws, nullptr, ws_num, EP_I8_DECODE};

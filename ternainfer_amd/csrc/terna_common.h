@@ -63,6 +63,22 @@ __device__ __forceinline__ int ws_group_decode(int n, int N, int ws_num)
     return n / (N / ws_num);
 }
 
+// Decode rule for four consecutive columns n0 .. n0+3 with one integer division instead of four: a group is
+// at least 16 columns wide (N >= 64, ws_num <= 4), so at most one group boundary falls inside the four.
+__device__ __forceinline__ void ws_group_decode4(int n0, int N, int ws_num, int g[4])
+{
+    if (ws_num == 3 && N == 3840) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) g[v] = n0 + v < 2560 ? 0 : (n0 + v < 3200 ? 1 : 2);
+        return;
+    }
+    const int q = N / ws_num;                   // uniform
+    g[0] = n0 / q;
+    const int next = (g[0] + 1) * q;            // first column of the next group
+#pragma unroll
+    for (int v = 1; v < 4; ++v) g[v] = g[0] + (n0 + v >= next ? 1 : 0);
+}
+
 // Prefill path: the group of the first column of the 128-wide tile that holds n, clamped
 // (epilogue_visitor_scale_ws.h:135-148).
 __device__ __forceinline__ int ws_group_prefill(int n, int N, int ws_num)
@@ -100,10 +116,11 @@ __device__ __forceinline__ void load_col_scales(const Epilogue& ep, int n0, int 
         w[0] = w[1] = w[2] = w[3] = v;
         return;
     }
+    int gd[4];
+    ws_group_decode4(n0, N, ep.ws_num, gd);
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-        const int g = ep.kind == EP_I8_PREFILL ? ws_group_prefill(n0 + v, N, ep.ws_num)
-                                               : ws_group_decode(n0 + v, N, ep.ws_num);
+        const int g = ep.kind == EP_I8_PREFILL ? ws_group_prefill(n0 + v, N, ep.ws_num) : gd[v];
         w[v] = ep.kind == EP_BF16 ? ep.scale[g] : bf16_bits_to_float(ep.ws[g]);
     }
 }
@@ -134,18 +151,21 @@ __device__ __forceinline__ EpilogueRaw load_epilogue_raw(const Epilogue& ep, int
         if (ep.ws_num == 1) {
             r.w[0] = __float_as_uint(ep.scale[0]);
         } else {
+            int gd[4];
+            ws_group_decode4(n0, N, ep.ws_num, gd);
 #pragma unroll
-            for (int v = 0; v < 4; ++v) r.w[v] = __float_as_uint(ep.scale[ws_group_decode(n0 + v, N, ep.ws_num)]);
+            for (int v = 0; v < 4; ++v) r.w[v] = __float_as_uint(ep.scale[gd[v]]);
         }
     } else {
         r.s = ep.s[m];
         if (ep.ws_num == 1) {
             r.w[0] = ep.ws[0];
         } else {
+            int gd[4];
+            ws_group_decode4(n0, N, ep.ws_num, gd);
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-                const int g = ep.kind == EP_I8_PREFILL ? ws_group_prefill(n0 + v, N, ep.ws_num)
-                                                       : ws_group_decode(n0 + v, N, ep.ws_num);
+                const int g = ep.kind == EP_I8_PREFILL ? ws_group_prefill(n0 + v, N, ep.ws_num) : gd[v];
                 r.w[v] = ep.ws[g];
             }
         }
@@ -162,8 +182,10 @@ __device__ __forceinline__ EpilogueRaw load_epilogue_raw_scales(const Epilogue& 
     if (ep.ws_num == 1) {
         r.w[0] = ep.ws[0];
     } else {
+        int gd[4];
+        ws_group_decode4(n0, N, ep.ws_num, gd);
 #pragma unroll
-        for (int v = 0; v < 4; ++v) r.w[v] = ep.ws[ws_group_decode(n0 + v, N, ep.ws_num)];
+        for (int v = 0; v < 4; ++v) r.w[v] = ep.ws[gd[v]];
     }
     return r;
 }
