@@ -111,17 +111,24 @@ __global__ __launch_bounds__(kNormThreads) void terna_norm_quant_kernel(
 
     // Every global load of the row -- input, second operand, norm weight -- is issued before the
     // first use: with one row per workgroup the kernel's time is its chain of memory round trips.
+    // The loads are unconditional on clamped addresses (a load inside a branch is waited for at
+    // the join, which would serialise them); without a second operand the input is read twice.
     u32x4 raw_x[kNormMaxVecs], raw_b[kNormMaxVecs], raw_w[kNormMaxVecs];
-    const bool has_b = GLU || residual != nullptr;
-    const uint16_t* br = GLU ? xr + K : residual + row * K;
+    const uint16_t* br = GLU ? xr + K : (residual != nullptr ? residual + row * K : xr);
 #pragma unroll
     for (int i = 0; i < kNormMaxVecs; ++i) {
         const int v = tid + i * kNormThreads;
-        if (v < nvec) {
-            raw_x[i] = *reinterpret_cast<const u32x4*>(xr + 8 * v);
-            if (has_b) raw_b[i] = *reinterpret_cast<const u32x4*>(br + 8 * v);
-            raw_w[i] = *reinterpret_cast<const u32x4*>(weight + 8 * v);
-        }
+        const int vc = v < nvec ? v : nvec - 1;
+        raw_x[i] = *reinterpret_cast<const u32x4*>(xr + 8 * vc);
+        raw_b[i] = *reinterpret_cast<const u32x4*>(br + 8 * vc);
+        raw_w[i] = *reinterpret_cast<const u32x4*>(weight + 8 * vc);
+    }
+    // pin the loads here: otherwise they are sunk into the branches below, next to their uses
+#pragma unroll
+    for (int i = 0; i < kNormMaxVecs; ++i) {
+        pin_registers(raw_x[i]);
+        pin_registers(raw_b[i]);
+        pin_registers(raw_w[i]);
     }
 
     float h[kNormMaxVecs][8];

@@ -97,6 +97,13 @@ struct EpilogueRegs {
     float w[4];     // weight-group scale of each column (bf16 family: the fp32 scale)
 };
 
+// Makes the value live in registers at this point of the program: a load that produced it cannot be sunk
+// past here (into a branch, next to its use), and is waited for here.
+__device__ __forceinline__ void pin_registers(u32x4& v)
+{
+    asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w));
+}
+
 // Compile-time loop: the body receives the index as a constant, so register arrays indexed by it
 // never need dynamic addressing.
 template <int I, int N, typename F>
