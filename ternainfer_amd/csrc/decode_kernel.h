@@ -229,33 +229,30 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[mb] = Acc{0, 0, 0, 0};
 
-    // Wave w finishes m-block w (and w + WAVES, ...): fetch that block's scale factors now.
     const int n0 = band * 16 + 4 * g;
-    EpilogueRaw eraw[(MB + WAVES - 1) / WAVES];
-#pragma unroll
-    for (int e = 0; e < (MB + WAVES - 1) / WAVES; ++e) {
-        const int m = m_base + (wave + e * WAVES) * 16 + i;
-        eraw[e] = load_epilogue_raw(ep, m < M ? m : M - 1, n0, N);
-    }
 
     // This wave's band-tiles: gk = wave, wave + WAVES, ...  (cnt of them)
     const int cnt = ktiles > wave ? (ktiles - wave + WAVES - 1) / WAVES : 0;
 
     // Sign-stream start of band-tile number (c0 + lane) of this wave, held one per lane.
-    auto load_bases = [&](int c0) -> int {
+    // (No load sits inside a branch, here or below: the compiler waits for every outstanding load at the
+    // join behind one, which would expose a memory round trip per band-tile.  Indices are clamped instead.)
+    // Two steps, so that the offset-free loads of the first band-tiles can go out between the request and the
+    // first use of the offsets.
+    int base_glob = 0, base_part = 0;
+    auto request_bases = [&](int c0) {
         const int j = c0 + lane;
-        int base = 0;
-        if (j < cnt) {
-            const int tile = gm * ktiles + wave + j * WAVES;
-            base = tile_off[tile];
-            if (med) base += median_off[3 * tile + med - 1];
-        }
-        return base;
+        const int gk = wave + (j < cnt ? j : 0) * WAVES;
+        const int tile = gm * ktiles + (gk < ktiles ? gk : ktiles - 1);
+        base_glob = tile_off[tile];
+        base_part = median_off[3 * tile + (med ? med - 1 : 0)];
     };
+    auto finish_bases = [&](int c0) -> int { return c0 + lane < cnt ? base_glob + (med ? base_part : 0) : 0; };
 
     // Loads that need no offset: the band-tile's bitmaps and the activation slab.
     auto fetch_tile = [&](int j, BandTileRaw<Act, MB>& raw) {
-        const int gk = wave + j * WAVES;
+        const int gk_raw = wave + j * WAVES;
+        const int gk = gk_raw < ktiles ? gk_raw : ktiles - 1;        // past the end: the last one again, never used
         const int tile = gm * ktiles + gk;
         const uint64_t* bmp = bitmap + static_cast<size_t>(tile) * 64 + med * 16;
         raw.bm[0] = bmp[b0];
@@ -267,14 +264,13 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
                 raw.x[mb][h] = x_ok[mb][h] ? *reinterpret_cast<const u32x4*>(xp[mb][h] + gk * 64) : u32x4{0u, 0u, 0u, 0u};
     };
     // The sign window: needs the band-tile's stream offset.
+    // A matrix without nonzeros has no sign words at all: its (unused) window is read from the bitmaps.
+    const uint32_t* sign_src = last_word >= 0 ? sign_words : reinterpret_cast<const uint32_t*>(bitmap);
+    const int last_idx = last_word >= 0 ? last_word : 0;
     auto fetch_signs = [&](int base, BandTileRaw<Act, MB>& raw) {
         raw.sign_base = base;
-        uint32_t win = 0;
-        if (last_word >= 0) {
-            const int wi = (base >> 5) + lane;
-            win = sign_words[wi < last_word ? wi : last_word];
-        }
-        raw.win = win;
+        const int wi = (base >> 5) + lane;
+        raw.win = sign_src[wi < last_idx ? wi : last_idx];
     };
 
     uint8_t* slab = xslab_all[wave][0];
@@ -339,17 +335,27 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
     };
     // Start of a round: offset-free loads go out first so they overlap the offset fetch.
     auto prime = [&]() {
-        if (0 < ccnt) fetch_tile(c0, ring0);
-        if (DEPTH == 2 && 1 < ccnt) fetch_tile(c0 + 1, ring1);
-        if (0 < ccnt) fetch_signs(__builtin_amdgcn_readlane(vbase, 0), ring0);
-        if (DEPTH == 2 && 1 < ccnt) fetch_signs(__builtin_amdgcn_readlane(vbase, 1), ring1);
+        request_bases(c0);
+        fetch_tile(c0, ring0);
+        if constexpr (DEPTH == 2) fetch_tile(c0 + 1, ring1);
+        __builtin_amdgcn_sched_barrier(0);       // nothing that waits for the offsets moves above the requests
+        vbase = finish_bases(c0);
+        fetch_signs(__builtin_amdgcn_readlane(vbase, 0), ring0);
+        if constexpr (DEPTH == 2) fetch_signs(__builtin_amdgcn_readlane(vbase, 1), ring1);
     };
 
     // Offsets come 64 band-tiles at a time (one per lane); K <= 4096 * WAVES needs one round.
     ccnt = cnt < 64 ? cnt : 64;
-    vbase = load_bases(0);
     prime();
     TERNA_TS(1);
+    // Wave w finishes m-block w (and w + WAVES, ...): with the data loads in flight, fetch that block's scale
+    // factors, so that no global load sits between the last MFMA and the store.
+    EpilogueRaw eraw[(MB + WAVES - 1) / WAVES];
+#pragma unroll
+    for (int e = 0; e < (MB + WAVES - 1) / WAVES; ++e) {
+        const int m = m_base + (wave + e * WAVES) * 16 + i;
+        eraw[e] = load_epilogue_raw(ep, m < M ? m : M - 1, n0, N);
+    }
 #pragma unroll
     for (int e = 0; e < 4; ++e) lut[lane + 64 * e] = T::make_lut(lane + 64 * e);
     TERNA_TS(2);
@@ -366,10 +372,7 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
         }
         c0 += 64;
         ccnt = cnt - c0 < 64 ? cnt - c0 : 64;
-        if (ccnt > 0) {
-            vbase = load_bases(c0);
-            prime();
-        }
+        if (ccnt > 0) prime();
     }
 
     // Cross-wave sum in wave order, then the fused epilogue.  The accumulator layout of a
