@@ -354,7 +354,7 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
 #pragma unroll
     for (int e = 0; e < (MB + WAVES - 1) / WAVES; ++e) {
         const int m = m_base + (wave + e * WAVES) * 16 + i;
-        eraw[e] = load_epilogue_raw(ep, m < M ? m : M - 1, n0, N);
+        eraw[e] = load_epilogue_raw_flat<sizeof(Act) == 2>(ep, m < M ? m : M - 1, n0, N);
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e) lut[lane + 64 * e] = T::make_lut(lane + 64 * e);

@@ -146,7 +146,7 @@ __device__ __forceinline__ EpilogueRegs load_epilogue(const Epilogue& ep, int m,
 // them) on the spot.  finish_epilogue() converts once the data is certainly there.
 struct EpilogueRaw {
     uint32_t s;
-    uint32_t w[4];      // one scale per matrix: only w[0] is loaded
+    uint32_t w[4];
 };
 
 __device__ __forceinline__ EpilogueRaw load_epilogue_raw(const Epilogue& ep, int m, int n0, int N)
@@ -180,20 +180,44 @@ __device__ __forceinline__ EpilogueRaw load_epilogue_raw(const Epilogue& ep, int
     return r;
 }
 
+// The same without a load inside a branch (the compiler waits for every outstanding load at the join behind one):
+// the group indices are computed first (arithmetic only) and all five values are loaded unconditionally; with one
+// scale per matrix the four weight-scale loads read the same word.  F32 = the bf16-activation family.  Measured: this
+// form is the faster one where the loads sit in a chain of dependent round trips (reference-format kernel, +4 %), the
+// branching form where they follow a burst of independent loads (P2 kernel, +3 %).
+template <bool F32>
+__device__ __forceinline__ EpilogueRaw load_epilogue_raw_flat(const Epilogue& ep, int m, int n0, int N)
+{
+    EpilogueRaw r;
+    int gd[4] = {0, 0, 0, 0};
+    if (ep.ws_num != 1) ws_group_decode4(n0, N, ep.ws_num, gd);
+    if constexpr (F32) {
+        r.s = 0u;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) r.w[v] = __float_as_uint(ep.scale[gd[v]]);
+    } else {
+        int g[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int gp = ep.ws_num != 1 ? ws_group_prefill(n0 + v, N, ep.ws_num) : 0;
+            g[v] = ep.kind == EP_I8_PREFILL ? gp : gd[v];
+        }
+        r.s = ep.s[m];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) r.w[v] = ep.ws[g[v]];
+    }
+    return r;
+}
+
 // Only the weight-group scales (the caller has the activation scale from elsewhere).
 __device__ __forceinline__ EpilogueRaw load_epilogue_raw_scales(const Epilogue& ep, int n0, int N)
 {
     EpilogueRaw r;
     r.s = 0u;
-    r.w[0] = r.w[1] = r.w[2] = r.w[3] = 0u;
-    if (ep.ws_num == 1) {
-        r.w[0] = ep.ws[0];
-    } else {
-        int gd[4];
-        ws_group_decode4(n0, N, ep.ws_num, gd);
+    int gd[4] = {0, 0, 0, 0};
+    if (ep.ws_num != 1) ws_group_decode4(n0, N, ep.ws_num, gd);
 #pragma unroll
-        for (int v = 0; v < 4; ++v) r.w[v] = ep.ws[gd[v]];
-    }
+    for (int v = 0; v < 4; ++v) r.w[v] = ep.ws[gd[v]];       // unconditional: see load_epilogue_raw
     return r;
 }
 
