@@ -36,7 +36,7 @@ void checkLastCudaError(int line);
 /* kernels/TernaSpMM.cu:25 -- out = bf16( (x_q . W^T) scaled ), int8 activations.
  *   x       int8  [M][K] row-major (quantised activations)
  *   s       bf16  [M]    per-row activation scale (x_q = round(x*s))
- *   ws      bf16  [>=ws_num] weight-group scales, ws_num groups along N
+ *   ws      bf16  [>=ws_num] weight-group scales, ws_num (1 .. 4) groups along N
  *   M <= 64 : epilogue bf16((acc / s[m]) * ws[g])        (Reduction_Kernel.cuh:60)
  *   M  > 64 : epilogue bf16(acc * (ws[g] / s[m])), 0 if s[m]==0, g per 128-column tile
  *                                                        (epilogue_visitor_scale_ws.h:135-205)

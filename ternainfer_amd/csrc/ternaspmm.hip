@@ -41,6 +41,17 @@ bool shape_ok(int M, int N, int K)
     return true;
 }
 
+// weight_scale has four slots (convert/convert_TernaInfer.py:176-194): one to four scale groups per matrix
+bool groups_ok(int ws_num)
+{
+    if (ws_num < 1 || ws_num > 4) {
+        std::printf("TernaSpMM Error: unsupported ws_num=%d (need 1 .. 4)\n", ws_num);
+        std::fflush(stdout);
+        return false;
+    }
+    return true;
+}
+
 struct Weights {
     const uint64_t* bitmap;
     const int* tile_off;
@@ -345,7 +356,7 @@ void run_i8(Route route, int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* m
             uint16_t* out, uint16_t* s, uint16_t* ws, int ws_num, int M, int N, int K, void* workspace,
             hipStream_t st, int line)
 {
-    if (!shape_ok(M, N, K) || ws_num < 1) return;
+    if (!shape_ok(M, N, K) || !groups_ok(ws_num)) return;
     // The reference picks its path, and with it the epilogue arithmetic, by M <= 64
     // (kernels/TernaSpMM.cu:34); the forced entry points pin one of the two.
     const bool decode_rule = route == ROUTE_DECODE || (route == ROUTE_AUTO && M <= 64);
@@ -364,7 +375,7 @@ void run_bf16(Route route, const uint16_t* x, const uint64_t* bitmap, const int*
               const uint16_t* median_off, const uint32_t* sign_words, uint16_t* out, const float* scale,
               int ws_num, int M, int N, int K, void* workspace, hipStream_t st, int line)
 {
-    if (!shape_ok(M, N, K) || ws_num < 1) return;
+    if (!shape_ok(M, N, K) || !groups_ok(ws_num)) return;
     const Epilogue ep{nullptr, nullptr, scale, ws_num, EP_BF16};
     const Weights w{bitmap, tile_off, median_off, sign_words};
     const bool small = route == ROUTE_DECODE || (route == ROUTE_AUTO && M <= 64);
@@ -640,7 +651,7 @@ void ternaspmm_repack(const uint64_t* bitmap, const int* tile_off, const uint16_
 void bitlinear_TernaSpMM_bf16_packed(const terna_bf16* x, const void* packed, terna_bf16* out, const float* scale,
                                      int ws_num, int M, int N, int K, int route, terna_stream stream)
 {
-    if (!shape_ok(M, N, K) || ws_num < 1) return;
+    if (!shape_ok(M, N, K) || !groups_ok(ws_num)) return;
     const Epilogue ep{nullptr, nullptr, scale, ws_num, EP_BF16};
     const uint32_t* p = static_cast<const uint32_t*>(packed);
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -654,7 +665,7 @@ void bitlinear_TernaSpMM_bf16_packed(const terna_bf16* x, const void* packed, te
 void bitlinear_TernaSpMM_packed(const int8_t* x, const void* packed, terna_bf16* out, const terna_bf16* s,
                                 const terna_bf16* ws, int ws_num, int M, int N, int K, int route, terna_stream stream)
 {
-    if (!shape_ok(M, N, K) || ws_num < 1) return;
+    if (!shape_ok(M, N, K) || !groups_ok(ws_num)) return;
     const bool decode_rule = route == 2 || (route != 1 && M <= 64);
     const Epilogue ep{s, ws, nullptr, ws_num, decode_rule ? EP_I8_DECODE : EP_I8_PREFILL};
     const uint32_t* p = static_cast<const uint32_t*>(packed);
@@ -698,7 +709,7 @@ static int launch_decode_fused(int mode, const terna_bf16* x, const terna_bf16* 
                                const terna_bf16* ws, int ws_num, int8_t* xq_out, terna_bf16* s_out, int M, int N,
                                int K, hipStream_t st)
 {
-    if (!shape_ok(M, N, K) || ws_num < 1 || M > 16) return 0;
+    if (!shape_ok(M, N, K) || !groups_ok(ws_num) || M > 16) return 0;
     const int ktiles = K / 64;
     const int bands = N / 16;
     static const int forced_waves = [] {
