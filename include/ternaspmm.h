@@ -234,6 +234,13 @@ void ternaspmm_rope_decode_attention_prefetch(const terna_bf16* qkv, const float
                                               const void* const* pf_ptr, const long long* pf_bytes, const long long* pf_unit_bytes,
                                               int pf_count, terna_stream stream);
 
+/* bf16 LM head of a decode step (F.linear on the tied embedding matrix, model.py:367, 449-455):
+ * logits[m][v] = sum_k x[m][k] * w[v][k], fp32 accumulate, bf16 out.  x bf16 [M][K], M <= 16; w bf16 [V][K];
+ * logits bf16 [M][V]; K a multiple of 32 with M * (2 K + 16) <= 160 KB; x and w 16-byte aligned.  An HBM-bound pass over w.
+ * Only enqueues. */
+void ternaspmm_lm_head_bf16(const terna_bf16* x, const terna_bf16* w, terna_bf16* logits, int M, int V, int K,
+                            terna_stream stream);
+
 /* Greedy sampling (torch.argmax over the logits, generate.py:283, 305): out[b] = index of the largest of
  * x[b][0 .. V-1] (bf16 [B][V]; out int64 [B]); ties go to the lowest index, NaN never wins.  Only enqueues. */
 void ternaspmm_argmax_bf16(const terna_bf16* x, long long* out, int B, int V, terna_stream stream);

@@ -1,0 +1,77 @@
+// bf16 LM head of a decode step: logits[m][v] = sum_k x[m][k] * W[v][k] for M <= 16 rows of
+// activations against the (tied) embedding matrix W [V][K] -- 657 MB for the 2B model, more than
+// all ternary weights of a token together, read once per step: an HBM-bound GEMV
+// (the reference: F.linear on the bf16 output matrix, model.py:367, 449-455).
+//
+// One wave owns 16 consecutive vocabulary rows at a time: v_mfma_f32_16x16x32_bf16 takes them as the
+// A operand straight from memory (lane: row L & 15, 8 consecutive k of chunk L >> 4 -- the 16 bytes
+// the lane loads) and the activations as B from LDS (staged once per workgroup; lanes of the batch
+// rows >= M read row 0 and feed zeros).
+// kLmUnroll loads of a lane are in flight before the first is used; a workgroup walks over row
+// blocks blockIdx.x, blockIdx.x + gridDim.x, ... so that the activations are staged once.
+#pragma once
+
+#include "terna_common.h"
+
+namespace terna {
+
+constexpr int kLmWaves = 4;
+constexpr int kLmUnroll = 16;                    // k-steps of 32 in flight per lane (16 bytes each)
+
+constexpr size_t lm_head_lds_bytes(int M, int K) { return static_cast<size_t>(M) * (K * 2 + 16); }
+
+__global__ __launch_bounds__(kLmWaves * 64) void terna_lm_head_kernel(const uint16_t* __restrict__ x,
+                                                                      const uint16_t* __restrict__ w,
+                                                                      uint16_t* __restrict__ logits, int M, int V, int K)
+{
+    extern __shared__ __align__(16) uint8_t xs[];            // [M][K * 2 + 16]: padded pitch
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int pitch = K * 2 + 16;
+    const int row_vecs = K >> 3;                             // 16-byte pieces per row
+    for (int p = tid; p < M * row_vecs; p += kLmWaves * 64) {
+        const int r = p / row_vecs, c = p - r * row_vecs;
+        *reinterpret_cast<u32x4*>(xs + r * pitch + 16 * c) = *reinterpret_cast<const u32x4*>(x + static_cast<size_t>(r) * K + 8 * c);
+    }
+    __syncthreads();
+
+    const int i = lane & 15, kg = lane >> 4;
+    const int steps = K >> 5;
+    const bool live = i < M;
+    const uint8_t* xrow = xs + (live ? i : 0) * pitch + 16 * kg;   // B operand: batch row i, chunk kg of each step
+    const int blocks = (V + 15) >> 4;
+    for (int blk = blockIdx.x * kLmWaves + wave; blk < blocks; blk += gridDim.x * kLmWaves) {
+        const int row = blk * 16 + i;
+        const uint16_t* wrow = w + static_cast<size_t>(row < V ? row : V - 1) * K + 8 * kg;
+        f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int s0 = 0; s0 < steps; s0 += kLmUnroll) {
+            u32x4 a[kLmUnroll];
+#pragma unroll
+            for (int u = 0; u < kLmUnroll; ++u) {
+                const int s = s0 + u < steps ? s0 + u : steps - 1;           // past the end: re-read, weight zero below
+                a[u] = *reinterpret_cast<const u32x4*>(wrow + 32 * s);
+            }
+#pragma unroll
+            for (int u = 0; u < kLmUnroll; ++u) {
+                const int s = s0 + u;
+                u32x4 b = *reinterpret_cast<const u32x4*>(xrow + 64 * (s < steps ? s : steps - 1));
+                if (s >= steps || !live) b = u32x4{0u, 0u, 0u, 0u};
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[u]), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
+            }
+        }
+        // lane: batch row i (the B column), vocabulary rows blk * 16 + 4 * kg .. + 3
+        const int v0 = blk * 16 + 4 * kg;
+        if (i < M && v0 < V) {
+            uint16_t* dst = logits + static_cast<size_t>(i) * V + v0;
+            if (v0 + 3 < V && (V & 3) == 0) {
+                *reinterpret_cast<u32x2*>(dst) = u32x2{pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3])};
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (v0 + e < V) dst[e] = float_to_bf16_bits(acc[e]);
+            }
+        }
+    }
+}
+
+}  // namespace terna

@@ -17,6 +17,7 @@
 #include "decode_fused_kernel.h"
 #include "attention_kernel.h"
 #include "argmax_kernel.h"
+#include "lm_head_kernel.h"
 #include "format_host.h"
 
 using namespace terna;
@@ -876,6 +877,33 @@ void ternaspmm_argmax_bf16(const terna_bf16* x, long long* out, int B, int V, te
     terna_argmax_bf16_kernel<<<dim3(B), dim3(kArgmaxThreads), 0, static_cast<hipStream_t>(stream)>>>(x, out, V);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_argmax_bf16", e, __LINE__);
+}
+
+void ternaspmm_lm_head_bf16(const terna_bf16* x, const terna_bf16* w, terna_bf16* logits, int M, int V, int K,
+                            terna_stream stream)
+{
+    if (M < 1 || M > 16 || V < 1 || K < 32 || (K & 31) || K > 16384 || (reinterpret_cast<uintptr_t>(x) & 15) ||
+        (reinterpret_cast<uintptr_t>(w) & 15)) {
+        std::fprintf(stderr, "ternaspmm_lm_head_bf16: unsupported arguments (M=%d V=%d K=%d)\n", M, V, K);
+        return;
+    }
+    const size_t lds = lm_head_lds_bytes(M, K);
+    if (lds > 160 * 1024) {
+        std::fprintf(stderr, "ternaspmm_lm_head_bf16: M=%d rows of K=%d do not fit the 160 KB of LDS\n", M, K);
+        return;
+    }
+    if (lds > 64 * 1024) allow_dynamic_lds(terna_lm_head_kernel, 160 * 1024, "hipFuncSetAttribute(lm head)", __LINE__);
+    const int blocks = (V + 15) / 16;
+    const int wgs_needed = (blocks + kLmWaves - 1) / kLmWaves;
+    static const int forced = [] {
+        const char* v = std::getenv("TERNASPMM_LM_HEAD_WGS");
+        return v ? std::atoi(v) : 0;
+    }();
+    const int cap = forced > 0 ? forced : 512;               // two workgroups per CU measure fastest (256: 137 us, 512: 115 us, 1024: 119 us on 657 MB)
+    const int grid = wgs_needed < cap ? wgs_needed : cap;
+    terna_lm_head_kernel<<<dim3(grid), dim3(kLmWaves * 64), lds, static_cast<hipStream_t>(stream)>>>(x, w, logits, M, V, K);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_lm_head_bf16", e, __LINE__);
 }
 
 void ternaspmm_repack_cache_clear(void)

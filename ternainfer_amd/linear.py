@@ -207,6 +207,22 @@ def relu2_mul_rmsnorm_quant(x13, weight, eps, quant=True):
     return y
 
 
+def lm_head(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Logits of a decode step: F.linear(x, weight) for bf16 x [M, K] with M <= 16 and the bf16 output
+    (tied embedding) matrix weight [V, K] (model.py:367, 449-455), as one HBM-bound pass over the matrix."""
+    assert x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.dim() == 2 and weight.dim() == 2
+    assert x.is_contiguous() and weight.is_contiguous() and x.shape[1] == weight.shape[1]
+    m, k = x.shape
+    v = weight.shape[0]
+    if m > 16 or k % 32 or m * (2 * k + 16) > 160 * 1024:
+        raise ValueError(f"lm_head: unsupported shape M={m} K={k}")
+    if out is None:
+        out = torch.empty((m, v), dtype=torch.bfloat16, device=x.device)
+    assert out.dtype == torch.bfloat16 and out.shape == (m, v) and out.is_contiguous()
+    _lib.load().ternaspmm_lm_head_bf16(_p(x), _p(weight), _p(out), m, v, k, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    return out
+
+
 def argmax_rows(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Greedy sampling: index of the largest logit per row of a bf16 [B, V] tensor -> int64 [B, 1]
     (torch.argmax(logits, dim=-1), generate.py:283; ties to the lowest index).  `out`, if given, is

@@ -21,7 +21,7 @@ import torch
 from torch.nn import functional as F
 
 from . import _lib
-from .linear import (argmax_rows, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant, repack_weight, rmsnorm_linear_packed,
+from .linear import (argmax_rows, lm_head, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant, repack_weight, rmsnorm_linear_packed,
                      rmsnorm_quant)
 
 
@@ -358,7 +358,9 @@ class Transformer:
             x, _ = rmsnorm_quant(x, self.norm, a.norm_eps, residual=pending, quant=False)
         else:
             x = rms_norm(x + pending, self.norm, a.norm_eps)
-        return F.linear(x, self.tok_embeddings)                               # tied LM head (model.py:367)
+        if x.is_cuda and bsz <= 16 and a.dim % 32 == 0 and bsz * (2 * a.dim + 16) <= 160 * 1024:
+            return lm_head(x, self.tok_embeddings)                            # tied LM head (model.py:367): one HBM-bound pass
+        return F.linear(x, self.tok_embeddings)
 
 
 @torch.inference_mode()

@@ -160,6 +160,31 @@ def test_argmax_rows(lib, b, v):
     assert got.shape == (b, 1) and (got.cpu().numpy().ravel() == want).all()
 
 
+@pytest.mark.parametrize("m,v,k", [(1, 128256, 2560), (8, 128256, 2560), (16, 4096, 2560), (3, 1003, 64), (2, 50, 32),
+                                   (5, 8200, 6912), (16, 640, 4128)])
+def test_lm_head_against_fp64(lib, m, v, k):
+    """bf16 LM head: within the bf16 GEMM bar of the fp64 product (max|err| <= 1e-2 max|ref|, median <= 1 ULP
+    of the bf16 result), also for V not a multiple of 16 or 4, K that is not a multiple of the unrolled
+    depth, and K whose 16 activation rows need more than 64 KB of LDS."""
+    import ternainfer_amd as T
+    rng = np.random.default_rng(4100 + m + v + k)
+    x = O.f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
+    w = O.f32_to_bf16_bits((rng.standard_normal((v, k)) * 0.05).astype(np.float32))
+    ref = O.bf16_bits_to_f32(x).astype(np.float64) @ O.bf16_bits_to_f32(w).astype(np.float64).T
+    xd, wd = _dev(x), _dev(w)
+    od = torch.zeros((m, v + 8), dtype=torch.int16, device="cuda").view(-1)[: m * v].view(m, v)   # tail stays zero
+    print(f"[case] lm_head m={m} v={v} k={k}", flush=True)
+    lib.ternaspmm_lm_head_bf16(_vp(xd), _vp(wd), _vp(od), m, v, k, None)
+    torch.cuda.synchronize()
+    got = O.bf16_bits_to_f32(od.cpu().numpy().view(np.uint16)).astype(np.float64)
+    err = np.abs(got - ref)
+    assert err.max() <= 1e-2 * np.abs(ref).max()
+    ulp = np.maximum(np.abs(ref), 2.0 ** -126) * 2.0 ** -7
+    assert np.median(err / ulp) <= 1.0
+    got2 = T.lm_head(xd.view(torch.bfloat16), wd.view(torch.bfloat16))
+    assert torch.equal(got2.view(torch.int16), od)
+
+
 # ------------------------------------------------------------------ attention-side kernels
 @pytest.mark.parametrize("adjacent", [0, 1])
 @pytest.mark.parametrize("b,t,h,kv,d,s_max", [(1, 1, 20, 5, 128, 64), (2, 24, 4, 2, 64, 32), (3, 5, 20, 5, 128, 40),
