@@ -40,6 +40,7 @@ __global__ __launch_bounds__(kLmWaves * 64) void terna_lm_head_kernel(const uint
     const bool live = i < M;
     const uint8_t* xrow = xs + (live ? i : 0) * pitch + 16 * kg;   // B operand: batch row i, chunk kg of each step
     const int blocks = (V + 15) >> 4;
+    const bool wide_store = (V & 3) == 0 && (reinterpret_cast<uintptr_t>(logits) & 7) == 0;   // 8-byte stores of four logits
     for (int blk = blockIdx.x * kLmWaves + wave; blk < blocks; blk += gridDim.x * kLmWaves) {
         const int row = blk * 16 + i;
         const uint16_t* wrow = w + static_cast<size_t>(row < V ? row : V - 1) * K + 8 * kg;
@@ -63,7 +64,7 @@ __global__ __launch_bounds__(kLmWaves * 64) void terna_lm_head_kernel(const uint
         const int v0 = blk * 16 + 4 * kg;
         if (i < M && v0 < V) {
             uint16_t* dst = logits + static_cast<size_t>(i) * V + v0;
-            if (v0 + 3 < V && (V & 3) == 0) {
+            if (wide_store) {                                // V % 4 == 0 and v0 % 4 == 0: v0 + 3 < V
                 *reinterpret_cast<u32x2*>(dst) = u32x2{pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3])};
             } else {
 #pragma unroll
