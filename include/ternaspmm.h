@@ -234,6 +234,16 @@ void ternaspmm_rope_decode_attention_prefetch(const terna_bf16* qkv, const float
                                               const void* const* pf_ptr, const long long* pf_bytes, const long long* pf_unit_bytes,
                                               int pf_count, terna_stream stream);
 
+/* The bookkeeping of one greedy decode step in one launch (generate.py:283-305: argmax, tokens[:, pos] = next_token,
+ * the position counters): tok[b] = argmax(logits[b]) as above; if history != NULL and counters[1] < history_len,
+ * history[b][counters[1]] = tok[b]; then counters[0] += 1 and counters[1] += 1 (counters int64 [2] = {cache slot of the
+ * next token, number of tokens in the history}; NULL: step 0, nothing advanced).  Sixteen workgroups share a row.
+ * state: ternaspmm_greedy_step_state_bytes(B) bytes of device memory, 8-byte aligned, zero-filled once by the caller
+ * (every launch leaves its first 8 bytes zero again); launches that share a state must not overlap.  Only enqueues. */
+size_t ternaspmm_greedy_step_state_bytes(int B);
+void ternaspmm_greedy_step_bf16(const terna_bf16* logits, long long* tok, long long* history, int history_len,
+                                long long* counters, void* state, int B, int V, terna_stream stream);
+
 /* bf16 LM head of a decode step (F.linear on the tied embedding matrix, model.py:367, 449-455):
  * logits[m][v] = sum_k x[m][k] * w[v][k], fp32 accumulate, bf16 out.  x bf16 [M][K], M <= 16; w bf16 [V][K];
  * logits bf16 [M][V]; K a multiple of 32 with M * (2 K + 16) <= 160 KB; x and w 16-byte aligned.  An HBM-bound pass over w.

@@ -45,6 +45,8 @@ PROTOTYPES = {
     "bitlinear_TernaSpMM_packed_fused_glu": ([_vp, _vp, ctypes.c_float, _vp, _vp, _vp, _ci, _vp, _vp, _ci, _ci, _ci, _vp],
                                              ctypes.c_int),
     "ternaspmm_rope_decode_attention_prefetch": ([_vp] * 7 + [_ci] * 5 + [ctypes.c_float, _ci, _vp, _vp, _vp, _vp, _ci, _vp], None),
+    "ternaspmm_greedy_step_state_bytes": ([_ci], ctypes.c_size_t),
+    "ternaspmm_greedy_step_bf16": ([_vp, _vp, _vp, _ci, _vp, _vp, _ci, _ci, _vp], None),
     "ternaspmm_lm_head_bf16": ([_vp, _vp, _vp, _ci, _ci, _ci, _vp], None),
     "ternaspmm_argmax_bf16": ([_vp, _vp, _ci, _ci, _vp], None),
     "ternaspmm_rope_kv_store": ([_vp] * 7 + [_ci] * 7 + [_vp], None),

@@ -879,6 +879,22 @@ void ternaspmm_argmax_bf16(const terna_bf16* x, long long* out, int B, int V, te
     if (e != hipSuccess) die("ternaspmm_argmax_bf16", e, __LINE__);
 }
 
+size_t ternaspmm_greedy_step_state_bytes(int B) { return B < 1 ? 0 : greedy_state_bytes(B); }
+
+void ternaspmm_greedy_step_bf16(const terna_bf16* logits, long long* tok, long long* history, int history_len,
+                                long long* counters, void* state, int B, int V, terna_stream stream)
+{
+    if (B < 1 || B > 65535 || V < 1 || !state || (reinterpret_cast<uintptr_t>(state) & 7) || (history && history_len < 1)) {
+        std::fprintf(stderr, "ternaspmm_greedy_step_bf16: unsupported arguments (B=%d V=%d history_len=%d state=%p)\n", B, V,
+                     history_len, state);
+        return;
+    }
+    terna_greedy_step_kernel<<<dim3(kGreedyChunks, B), dim3(kGreedyThreads), 0, static_cast<hipStream_t>(stream)>>>(
+        logits, tok, history, history_len, counters, static_cast<unsigned long long*>(state), B, V);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_greedy_step_bf16", e, __LINE__);
+}
+
 void ternaspmm_lm_head_bf16(const terna_bf16* x, const terna_bf16* w, terna_bf16* logits, int M, int V, int K,
                             terna_stream stream)
 {

@@ -236,6 +236,32 @@ def argmax_rows(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> tor
     return out
 
 
+def greedy_step_state(batch: int, device="cuda") -> torch.Tensor:
+    """Zero-filled scratch of `greedy_step` for `batch` rows; allocate once, launches restore it."""
+    return torch.zeros(_lib.load().ternaspmm_greedy_step_state_bytes(batch) // 8, dtype=torch.int64, device=device)
+
+
+def greedy_step(logits: torch.Tensor, tok: torch.Tensor, history: Optional[torch.Tensor], counters: Optional[torch.Tensor],
+                state: torch.Tensor) -> torch.Tensor:
+    """One launch for the tail of a greedy decode step (generate.py:283-305): tok[b] = argmax(logits[b]);
+    history[b, counters[1]] = tok[b] while there is room; counters += 1 (int64 [2]: next cache slot, tokens stored).
+    `state` comes from `greedy_step_state`."""
+    assert logits.dtype == torch.bfloat16 and logits.dim() == 2 and logits.is_contiguous()
+    b, v = logits.shape
+    assert tok.dtype == torch.int64 and tok.numel() == b and tok.is_contiguous()
+    hist_len = 0
+    if history is not None:
+        assert history.dtype == torch.int64 and history.dim() == 2 and history.shape[0] == b and history.is_contiguous()
+        hist_len = history.shape[1]
+    if counters is not None:
+        assert counters.dtype == torch.int64 and counters.numel() == 2 and counters.is_contiguous()
+    assert state.dtype == torch.int64 and state.numel() * 8 >= _lib.load().ternaspmm_greedy_step_state_bytes(b)
+    _lib.load().ternaspmm_greedy_step_bf16(_p(logits), _p(tok), _p(history) if history is not None else None, hist_len,
+                                           _p(counters) if counters is not None else None, _p(state), b, v,
+                                           ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    return tok
+
+
 class _CompressedWeight(nn.Module):
     """Holds the four format tensors + ``weight_scale`` under the reference's checkpoint keys
     (convert_TernaInfer.py:204-209, model.py:110-116)."""

@@ -21,7 +21,7 @@ import torch
 from torch.nn import functional as F
 
 from . import _lib
-from .linear import (argmax_rows, lm_head, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant, repack_weight, rmsnorm_linear_packed,
+from .linear import (argmax_rows, greedy_step, greedy_step_state, lm_head, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant, repack_weight, rmsnorm_linear_packed,
                      rmsnorm_quant)
 
 
@@ -307,15 +307,16 @@ class Transformer:
             blk.prefetch = (ptrs, sizes, units, count)
 
     def rope_tables(self, max_seq: int, dev):
-        """cos / sin of every (cache slot, rotary pair): fp32 [max_seq, head_dim / 2], built once per length."""
+        """cos / sin of every (cache slot, rotary pair): fp32 [max_seq, 2, head_dim / 2] (cos row, sin row), built
+        once per length; one gather then fetches both rows of a position."""
         key = (max_seq, str(dev))
         tables = getattr(self, "_rope_tables", None)
         if tables is None or tables[0] != key:
             a = self.args
             inv = 1.0 / (a.rope_theta ** (torch.arange(0, a.head_dim, 2, device=dev, dtype=torch.float32) / a.head_dim))
             ang = torch.arange(max_seq, device=dev, dtype=torch.float32)[:, None] * inv[None, :]
-            self._rope_tables = tables = (key, ang.cos().contiguous(), ang.sin().contiguous())
-        return tables[1], tables[2]
+            self._rope_tables = tables = (key, torch.stack([ang.cos(), ang.sin()], dim=1).contiguous())
+        return tables[1]
 
     def attention_workspace(self, bsz: int):
         """Zero-filled scratch of the single-token attention (split over the cache); one per batch size."""
@@ -340,8 +341,8 @@ class Transformer:
         bsz, t = tokens.shape
         max_seq = cache[0][0].shape[2]
         dev = tokens.device
-        cos_all, sin_all = self.rope_tables(max_seq, dev)
-        cos, sin = cos_all.index_select(0, pos_idx), sin_all.index_select(0, pos_idx)     # fp32 [T, head_dim / 2]
+        rows = self.rope_tables(max_seq, dev).index_select(0, pos_idx)         # fp32 [T, 2, head_dim / 2]
+        cos, sin = rows[:, 0].contiguous(), rows[:, 1].contiguous()           # views when T == 1
         mask = None
         one_launch_attention = self.layers[0].fused and t == 1 and a.head_dim in (64, 128) and max_seq <= 8192
         if not one_launch_attention:
@@ -375,14 +376,14 @@ def greedy_decode(model: Transformer, prompt: torch.Tensor, gen_tokens: int, use
     logits = model.forward(prompt, cache, torch.arange(plen, device="cuda"))
     tok = argmax_rows(logits.contiguous())                                    # int64 [B, 1]
     ev[1].record()
-    counters = torch.tensor([plen, 0], dtype=torch.int64, device="cuda")      # cache slot of the next token, step number
-    pos, step_idx = counters[0:1], counters[1:2]
+    counters = torch.tensor([plen, 1], dtype=torch.int64, device="cuda")      # cache slot of the next token, tokens stored
+    pos = counters[0:1]
     out = torch.empty((bsz, gen_tokens), dtype=torch.int64, device="cuda")
+    out[:, 0:1] = tok
+    state = greedy_step_state(bsz)
 
-    def step():
-        out.index_copy_(1, step_idx, tok)
-        argmax_rows(model.forward(tok, cache, pos), out=tok)                  # the forward has read tok by then
-        counters.add_(1)
+    def step():                                                               # the forward has read tok by the time it changes
+        greedy_step(model.forward(tok, cache, pos), tok, out, counters, state)
 
     graph = None
     if use_graph:

@@ -438,3 +438,43 @@ def test_rope_decode_attention_with_prefetch_regions(lib, b, h, kv, d, s_max, n)
     torch.cuda.synchronize()
     assert torch.equal(o1, o2) and torch.equal(ck1, ck2) and torch.equal(cv1, cv2)
     assert all(torch.equal(r, r0) for r, r0 in zip(regions, before))
+
+
+@pytest.mark.parametrize("b,v,hist", [(1, 128256, 4), (8, 128256, 3), (3, 1003, 2), (37, 4096, 5), (2, 64, 1), (300, 520, 2)])
+def test_greedy_step(lib, b, v, hist):
+    """argmax + history append + counters in one launch, several launches in a row on one state: the
+    same tokens as the one-row-per-workgroup argmax (ties, -inf, NaN, unaligned rows), the history
+    filled up to its length and not beyond, counters advanced every time."""
+    import ternainfer_amd as T
+    rng = np.random.default_rng(7000 + b + v)
+    state = T.greedy_step_state(b)
+    tok = torch.full((b, 1), -1, dtype=torch.int64, device="cuda")
+    history = torch.full((b, hist + 1), -7, dtype=torch.int64, device="cuda")[:, :hist].contiguous()
+    counters = torch.tensor([40, 0], dtype=torch.int64, device="cuda")
+    want_hist = np.full((b, hist), -7, np.int64)
+    for launch in range(hist + 2):
+        xf = O.bf16_bits_to_f32(O.f32_to_bf16_bits(rng.standard_normal((b, v)).astype(np.float32)))
+        if v >= 64:
+            xf[0, 17] = xf[0, v - 3] = 9.0                                       # a tie across chunks: the lower index wins
+            xf[-1, 3] = -np.inf
+            xf[-1, 11] = np.nan
+        if launch == 1:
+            xf[0, :] = -np.inf                                                   # nothing ever wins: index 0
+        x = O.f32_to_bf16_bits(xf)
+        xf = O.bf16_bits_to_f32(x)
+        want = np.array([0 if np.all(np.isneginf(r[~np.isnan(r)])) else int(np.flatnonzero(r == np.nanmax(r))[0]) for r in xf], np.int64)
+        xd = _dev(x).view(torch.bfloat16)
+        print(f"[case] greedy_step b={b} v={v} launch={launch}", flush=True)
+        T.greedy_step(xd, tok, history, counters, state)
+        torch.cuda.synchronize()
+        assert (tok.cpu().numpy().ravel() == want).all()
+        assert (T.argmax_rows(xd).cpu().numpy().ravel() == want).all()
+        if launch < hist:
+            want_hist[:, launch] = want
+        assert (history.cpu().numpy() == want_hist).all()
+        assert counters.cpu().tolist() == [41 + launch, 1 + launch]
+        assert int(state[0].item()) == 0
+    # without history and counters: only the tokens
+    T.greedy_step(xd, tok.fill_(-1), None, None, state)
+    torch.cuda.synchronize()
+    assert (tok.cpu().numpy().ravel() == want).all()
