@@ -140,38 +140,68 @@ struct AttentionPrefetch {
     int workgroups;       // extra workgroups, a multiple of 8 (0: none)
 };
 
+// A prefetching workgroup's XCD owns the units u = xcd, xcd + 8, ... of every region (all of a
+// region without units).  These shares, laid end to end, are cut into equal ranges for the XCD's
+// prefetching workgroups, and a thread requests up to kPrefetchBatch of its range's 16-byte
+// vectors before it waits for any: a workgroup's part is one memory round trip, whatever the
+// sizes of the units (unit by unit, with a wait after each, the largest part took six).
+constexpr int kPrefetchBatch = 16;
+
 __device__ __forceinline__ void attention_prefetch_role(const AttentionPrefetch& pf, int heads, int nthreads)
 {
     const int p = blockIdx.x - heads;
-    const int xcd = blockIdx.x & 7;
-    const int per_xcd = pf.workgroups >> 3;
+    const uint32_t xcd = blockIdx.x & 7;
+    const uint32_t per_xcd = pf.workgroups >> 3;
     // rank of this workgroup among those of its XCD
-    const int rank = (p - ((xcd - (heads & 7) + 8) & 7)) >> 3;
+    const uint32_t rank = (p - ((xcd - (heads & 7) + 8) & 7)) >> 3;
+    uint32_t share[kAttentionPrefetchRegions], uv[kAttentionPrefetchRegions], tot[kAttentionPrefetchRegions];
+    float inv[kAttentionPrefetchRegions];
+    uint32_t all = 0;
+#pragma unroll
+    for (int r = 0; r < kAttentionPrefetchRegions; ++r) {
+        const bool on = r < pf.count;
+        uv[r] = on ? static_cast<uint32_t>(pf.unit_vecs[r]) : 0u;
+        tot[r] = on ? static_cast<uint32_t>(pf.total_vecs[r]) : 0u;
+        const uint32_t units = on ? static_cast<uint32_t>(pf.units[r]) : 0u;
+        const uint32_t mine = units > xcd ? (units - xcd + 7) >> 3 : 0u;
+        share[r] = uv[r] == 0 ? tot[r] : mine * uv[r];
+        inv[r] = uv[r] ? 1.0f / static_cast<float>(uv[r]) : 0.0f;
+        all += share[r];
+    }
+    const uint32_t lo = static_cast<uint32_t>(static_cast<unsigned long long>(all) * rank / per_xcd);
+    const uint32_t hi = static_cast<uint32_t>(static_cast<unsigned long long>(all) * (rank + 1) / per_xcd);
     uint32_t seen = 0;
-    for (int r = 0; r < pf.count; ++r) {
-        if (pf.unit_vecs[r] == 0) {              // read by every workgroup of the consumers: once per XCD
-            if (rank == 0) {
-                for (long long v = threadIdx.x; v < pf.total_vecs[r]; v += nthreads) {
-                    const u32x4 q = pf.base[r][v];
-                    seen |= q.x & q.y & q.z & q.w;
-                }
-            }
-            continue;
-        }
-        for (long long u = xcd + 8ll * rank; u < pf.units[r]; u += 8ll * per_xcd) {
-            const long long first = u * pf.unit_vecs[r];
-            for (int v0 = threadIdx.x; v0 < pf.unit_vecs[r]; v0 += 4 * nthreads) {
-                u32x4 q[4];
+    for (uint32_t g0 = lo; g0 < hi; g0 += kPrefetchBatch * nthreads) {
+        u32x4 q[kPrefetchBatch];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int vv = v0 + j * nthreads;
-                    const bool ok = vv < pf.unit_vecs[r] && first + vv < pf.total_vecs[r];
-                    q[j] = ok ? pf.base[r][first + vv] : u32x4{0u, 0u, 0u, 0u};
-                }
+        for (int j = 0; j < kPrefetchBatch; ++j) {
+            const uint32_t g = g0 + j * nthreads + threadIdx.x;
+            // region of g and the offset in this XCD's share of it
+            uint32_t off = g, r_uv = uv[0], r_tot = tot[0];
+            float r_inv = inv[0];
+            const u32x4* r_base = pf.base[0];
+            bool found = off < share[0];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) seen |= q[j].x & q[j].y & q[j].z & q[j].w;
+            for (int r = 1; r < kAttentionPrefetchRegions; ++r) {
+                off -= found ? 0u : share[r - 1];
+                const bool here = !found && off < share[r];
+                r_uv = here ? uv[r] : r_uv;
+                r_tot = here ? tot[r] : r_tot;
+                r_inv = here ? inv[r] : r_inv;
+                r_base = here ? pf.base[r] : r_base;
+                found = found || here;
             }
+            // vector `off` of the share -> unit xcd + 8 (off / uv), vector off % uv of it (shares stay below 2^24 vectors:
+            // the float quotient is off by one at most)
+            uint32_t unit = static_cast<uint32_t>(static_cast<float>(off) * r_inv);
+            unit -= unit * r_uv > off ? 1u : 0u;
+            unit += (unit + 1) * r_uv <= off ? 1u : 0u;
+            const uint32_t v = r_uv ? (xcd + 8 * unit) * r_uv + (off - unit * r_uv) : off;
+            const bool ok = g < hi && found && v < r_tot;
+            q[j] = r_base[ok ? v : 0];           // past the range: the region's first vector again, no branch around the load
         }
+#pragma unroll
+        for (int j = 0; j < kPrefetchBatch; ++j) seen |= q[j].x & q[j].y & q[j].z & q[j].w;
     }
     if (seen == 0xffffffffu && pf.count > kAttentionPrefetchRegions) *const_cast<u32x4*>(pf.base[0]) = u32x4{seen, 0u, 0u, 0u};   // never true: keeps the loads
 }
@@ -221,136 +251,141 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     // tiles per wave, the first VU value rows of this thread's slice, q.  Slots >= n hold stale or
     // unwritten cache lines; they are read (the cache is S slots long) and masked out below.
     //
-    // ---- pass 1: scores on the matrix cores.  A tile is 16 cache slots; v_mfma_f32_16x16x32_bf16
-    // takes the key rows as A (lane: slot L & 15, dimensions 32j + 8(L >> 4) .. +7 -- the 16 bytes
-    // the lane loads) and q as B, the same in all 16 columns, so every column of the result holds
-    // the 16 scores and column 0 (lanes 0, 16, 32, 48: four slots each) writes them.  No shuffles.
+    // ---- pass 1: scores on the matrix cores.  A tile is 16 cache slots; one v_mfma_f32_16x16x32_bf16
+    // takes 16 / R of them, R = D / 32: a key row is R rows of the A operand, 32 dimensions each.
+    // Lane L (row i = L & 15, k-block L >> 4) loads the 16-byte piece (i % R) + R (L >> 4) of slot
+    // i / R, so four consecutive lanes fetch 64 consecutive bytes: the memory pipeline of a CU
+    // handles a load four lanes at a time and takes one step per 64-byte segment these touch, and a
+    // load whose consecutive lanes sit in different key rows (the plain operand layout: row L & 15)
+    // streams at a quarter of the rate (25 against 80 bytes per clock from L2, measured).  The B
+    // operand holds q's matching pieces in column i % R (zero elsewhere), so out[i][i % R] is the
+    // partial score of row i and a slot's score is the sum over its R rows: the accumulator puts
+    // them in R neighbouring lanes (columns 0 .. R-1), one quad permutation or two add them up.
     constexpr int NJ = D / 32;                   // MFMAs (32 dimensions each) per tile
     constexpr int KT = 4;                        // key tiles in flight per wave: slots 0 .. 255
     constexpr int VU = 8;                        // value rows in flight per thread
     const int r16 = lane & 15, kblk = lane >> 4;
     const int chunk = tid % CH, slice = tid / CH;
-    u32x4 kr[KT][NJ], vr[VU], qr[NJ];
+    constexpr int R = D / 32;                    // operand rows per key row
+    constexpr int SPM = 16 / R;                  // slots per MFMA
+    const int rr = r16 % R, sl = r16 / R;
+    const int piece = rr + R * kblk;             // this lane's 16 bytes (8 dimensions) of a key row, and of q
+    u32x4 kr[KT][NJ], vr[VU], qb;
+    auto load_keys = [&](int ltile, u32x4 (&dst)[NJ]) {
 #pragma unroll
-    for (int t = 0; t < KT; ++t) {
-        const int sk = 16 * ((wave + NW * t) * SP + sp) + r16;
-        const uint16_t* kp = kbase + static_cast<size_t>(sk < S ? sk : 0) * D + 8 * kblk;
+        for (int j = 0; j < NJ; ++j) {
+            const int sk = 16 * (ltile * SP + sp) + SPM * j + sl;
+            dst[j] = *reinterpret_cast<const u32x4*>(kbase + static_cast<size_t>(sk < S ? sk : 0) * D + 8 * piece);
+        }
+    };
 #pragma unroll
-        for (int jj = 0; jj < NJ; ++jj) kr[t][jj] = *reinterpret_cast<const u32x4*>(kp + 32 * jj);
-    }
+    for (int t = 0; t < KT; ++t) load_keys(wave + NW * t, kr[t]);
 #pragma unroll
     for (int u = 0; u < VU; ++u) {
         const int sv = cache_slot(slice + u * SLICES);
         vr[u] = *reinterpret_cast<const u32x4*>(vbase + static_cast<size_t>(sv < S ? sv : 0) * D + chunk * 8);
     }
-    u32x4 knew[NJ], vnew;                        // ROPE: the new token's key chunks of this lane, value chunk of this thread
+    u32x4 knew, vnew;                            // ROPE: the new token's key piece of this lane, value chunk of this thread
+    const u32x4 zero4 = {0u, 0u, 0u, 0u};
     if constexpr (!ROPE) {
-#pragma unroll
-        for (int jj = 0; jj < NJ; ++jj)
-            qr[jj] = *reinterpret_cast<const u32x4*>(q + (static_cast<size_t>(b) * H + h) * D + 32 * jj + 8 * kblk);
+        qb = *reinterpret_cast<const u32x4*>(q + (static_cast<size_t>(b) * H + h) * D + 8 * piece);
     } else {
         const uint16_t* row = q + static_cast<size_t>(b) * (H + 2 * KV) * D;
         vnew = *reinterpret_cast<const u32x4*>(row + (H + KV + kvh) * D + 8 * chunk);
+        const int c = piece;                     // chunk c = dimensions 8c .. 8c+7
         if constexpr (ADJACENT) {
-            // chunk c = 4jj + kblk (dimensions 8c .. 8c+7) holds pairs 4c .. 4c+3 whole
-            u32x4 q_own[NJ], k_own[NJ];
-            f32x4 cs[NJ], sn[NJ];
-#pragma unroll
-            for (int jj = 0; jj < NJ; ++jj) {
-                const int c = 4 * jj + kblk;
-                q_own[jj] = *reinterpret_cast<const u32x4*>(row + h * D + 8 * c);
-                k_own[jj] = *reinterpret_cast<const u32x4*>(row + (H + kvh) * D + 8 * c);
-                cs[jj] = *reinterpret_cast<const f32x4*>(cosv + 4 * c);
-                sn[jj] = *reinterpret_cast<const f32x4*>(sinv + 4 * c);
-            }
-            auto rotate = [&](const u32x4& own, int jj) {
+            // a chunk holds the pairs 4c .. 4c+3 whole
+            const u32x4 q_own = *reinterpret_cast<const u32x4*>(row + h * D + 8 * c);
+            const u32x4 k_own = *reinterpret_cast<const u32x4*>(row + (H + kvh) * D + 8 * c);
+            const f32x4 cs = *reinterpret_cast<const f32x4*>(cosv + 4 * c);
+            const f32x4 sn = *reinterpret_cast<const f32x4*>(sinv + 4 * c);
+            auto rotate = [&](const u32x4& own) {
                 float a[8], o[8];
                 unpack_bf16x8(own, a);
 #pragma unroll
                 for (int m = 0; m < 4; ++m) {
 #pragma clang fp contract(off)                   // as terna_rope_kv_store_kernel: every product and sum rounded once
-                    o[2 * m] = a[2 * m] * cs[jj][m] - a[2 * m + 1] * sn[jj][m];
-                    o[2 * m + 1] = a[2 * m + 1] * cs[jj][m] + a[2 * m] * sn[jj][m];
+                    o[2 * m] = a[2 * m] * cs[m] - a[2 * m + 1] * sn[m];
+                    o[2 * m + 1] = a[2 * m + 1] * cs[m] + a[2 * m] * sn[m];
                 }
                 return pack_bf16x8(o);
             };
-#pragma unroll
-            for (int jj = 0; jj < NJ; ++jj) {
-                qr[jj] = rotate(q_own[jj], jj);
-                knew[jj] = rotate(k_own[jj], jj);
-            }
+            qb = rotate(q_own);
+            knew = rotate(k_own);
         } else {
-            // chunk c = 4jj + kblk (dimensions 8c .. 8c+7) and its rotation partner c +- CH/2
-            u32x4 q_own[NJ], q_par[NJ], k_own[NJ], k_par[NJ];
-            f32x4 cs[NJ][2], sn[NJ][2];
-#pragma unroll
-            for (int jj = 0; jj < NJ; ++jj) {
-                const int c = 4 * jj + kblk, cp = (c + CH / 2) % CH, ca = c % (CH / 2);
-                q_own[jj] = *reinterpret_cast<const u32x4*>(row + h * D + 8 * c);
-                q_par[jj] = *reinterpret_cast<const u32x4*>(row + h * D + 8 * cp);
-                k_own[jj] = *reinterpret_cast<const u32x4*>(row + (H + kvh) * D + 8 * c);
-                k_par[jj] = *reinterpret_cast<const u32x4*>(row + (H + kvh) * D + 8 * cp);
-                cs[jj][0] = *reinterpret_cast<const f32x4*>(cosv + 8 * ca);
-                cs[jj][1] = *reinterpret_cast<const f32x4*>(cosv + 8 * ca + 4);
-                sn[jj][0] = *reinterpret_cast<const f32x4*>(sinv + 8 * ca);
-                sn[jj][1] = *reinterpret_cast<const f32x4*>(sinv + 8 * ca + 4);
-            }
-            auto rotate = [&](const u32x4& own, const u32x4& par, int jj, bool first_half) {
+            // the chunk and its rotation partner c +- CH/2
+            const int cp = (c + CH / 2) % CH, ca = c % (CH / 2);
+            const u32x4 q_own = *reinterpret_cast<const u32x4*>(row + h * D + 8 * c);
+            const u32x4 q_par = *reinterpret_cast<const u32x4*>(row + h * D + 8 * cp);
+            const u32x4 k_own = *reinterpret_cast<const u32x4*>(row + (H + kvh) * D + 8 * c);
+            const u32x4 k_par = *reinterpret_cast<const u32x4*>(row + (H + kvh) * D + 8 * cp);
+            f32x4 cs[2], sn[2];
+            cs[0] = *reinterpret_cast<const f32x4*>(cosv + 8 * ca);
+            cs[1] = *reinterpret_cast<const f32x4*>(cosv + 8 * ca + 4);
+            sn[0] = *reinterpret_cast<const f32x4*>(sinv + 8 * ca);
+            sn[1] = *reinterpret_cast<const f32x4*>(sinv + 8 * ca + 4);
+            const bool first_half = c < CH / 2;
+            auto rotate = [&](const u32x4& own, const u32x4& par) {
                 float a[8], p[8], o[8];
                 unpack_bf16x8(own, a);
                 unpack_bf16x8(par, p);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
 #pragma clang fp contract(off)
-                    const float c = cs[jj][e >> 2][e & 3], sv = sn[jj][e >> 2][e & 3];
-                    const float lo = a[e] * c - p[e] * sv;     // own chunk in the first half:  x1 c - x2 s
-                    const float hi = a[e] * c + p[e] * sv;     // own chunk in the second half: x2 c + x1 s
+                    const float cc = cs[e >> 2][e & 3], sv = sn[e >> 2][e & 3];
+                    const float lo = a[e] * cc - p[e] * sv;    // own chunk in the first half:  x1 c - x2 s
+                    const float hi = a[e] * cc + p[e] * sv;    // own chunk in the second half: x2 c + x1 s
                     o[e] = first_half ? lo : hi;
                 }
                 return pack_bf16x8(o);
             };
-#pragma unroll
-            for (int jj = 0; jj < NJ; ++jj) {
-                const bool first_half = 4 * jj + kblk < CH / 2;
-                qr[jj] = rotate(q_own[jj], q_par[jj], jj, first_half);
-                knew[jj] = rotate(k_own[jj], k_par[jj], jj, first_half);
-            }
+            qb = rotate(q_own, q_par);
+            knew = rotate(k_own, k_par);
         }
         if (h % (H / KV) == 0 && sp == 0) {      // this kv group's writer: slot pos[0] of both caches
             const size_t slot_off = ((static_cast<size_t>(b) * KV + kvh) * S + (n - 1)) * D;
-            if (wave == 0 && r16 == 0) {
-#pragma unroll
-                for (int jj = 0; jj < NJ; ++jj) *reinterpret_cast<u32x4*>(cache_k + slot_off + 8 * (4 * jj + kblk)) = knew[jj];
-            }
+            if (wave == 0 && r16 < R) *reinterpret_cast<u32x4*>(cache_k + slot_off + 8 * c) = knew;   // r16 < R: every chunk once
             if (tid < CH) *reinterpret_cast<u32x4*>(cache_v + slot_off + 8 * chunk) = vnew;
         }
     }
+    if (r16 >= R) qb = zero4;                    // B operand: q's pieces in columns 0 .. R-1 only
 
     TERNA_TS(1);
     float mx = -INFINITY;
     auto score_tile = [&](int ltile, const u32x4 (&kin)[NJ]) {       // ltile: local tile of this split
         const int tile = ltile * SP + sp;
-        u32x4 k[NJ];
 #pragma unroll
-        for (int jj = 0; jj < NJ; ++jj) k[jj] = kin[jj];
-        if constexpr (ROPE) {
-            if (16 * tile + r16 == n - 1) {      // the new token's slot: its key row is in registers, not in the cache yet
-#pragma unroll
-                for (int jj = 0; jj < NJ; ++jj) k[jj] = knew[jj];
+        for (int j = 0; j < NJ; ++j) {
+            u32x4 k = kin[j];
+            if constexpr (ROPE) {                // the new token's slot: its key row is in registers, not in the cache yet
+                if (16 * tile + SPM * j + sl == n - 1) k = knew;
             }
-        }
-        f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-        for (int jj = 0; jj < NJ; ++jj)
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, k[jj]), __builtin_bit_cast(bf16x8, qr[jj]), acc, 0, 0, 0);
-        if (r16 == 0) {
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int sk = 16 * tile + 4 * kblk + v;
-                if (sk < n) {
-                    const float d = acc[v] * scale;
-                    score[16 * ltile + 4 * kblk + v] = d;
+            const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+            const f32x4 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, k), __builtin_bit_cast(bf16x8, qb), zero, 0, 0, 0);
+            // lane (column c = r16, rows 4 kblk + v): row i's partial score is out[i][i % R]
+            if constexpr (R == 4) {              // rows 4 kblk + v of slot kblk: column v, lanes 16 kblk + 0 .. 3
+                float x = r16 == 0 ? acc[0] : r16 == 1 ? acc[1] : r16 == 2 ? acc[2] : acc[3];
+                x += dpp_permute<kDppSwapPairs>(x);
+                x += dpp_permute<kDppSwapHalfQuads>(x);
+                const int ls = SPM * j + kblk;   // slot within the tile
+                if (r16 == 0 && 16 * tile + ls < n) {
+                    const float d = x * scale;
+                    score[16 * ltile + ls] = d;
                     mx = fmaxf(mx, d);
+                }
+            } else {                             // R == 2: rows 4 kblk + v of slots 2 kblk + (v >> 1): column v & 1
+                float x0 = r16 == 0 ? acc[0] : acc[1];
+                float x1 = r16 == 0 ? acc[2] : acc[3];
+                x0 += dpp_permute<kDppSwapPairs>(x0);
+                x1 += dpp_permute<kDppSwapPairs>(x1);
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const int ls = SPM * j + 2 * kblk + e;
+                    if (r16 == 0 && 16 * tile + ls < n) {
+                        const float d = (e ? x1 : x0) * scale;
+                        score[16 * ltile + ls] = d;
+                        mx = fmaxf(mx, d);
+                    }
                 }
             }
         }
@@ -363,10 +398,7 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
         if (wave + NW * t < ltiles) score_tile(wave + NW * t, kr[t]);
     for (int tile = wave + NW * KT; tile < ltiles; tile += NW) {      // beyond the tiles requested up front: plain loop
         u32x4 k[NJ];
-        const int sk = 16 * (tile * SP + sp) + r16;
-        const uint16_t* kp = kbase + static_cast<size_t>(sk < S ? sk : 0) * D + 8 * kblk;
-#pragma unroll
-        for (int jj = 0; jj < NJ; ++jj) k[jj] = *reinterpret_cast<const u32x4*>(kp + 32 * jj);
+        load_keys(tile, k);
         score_tile(tile, k);
     }
     TERNA_TS(2);

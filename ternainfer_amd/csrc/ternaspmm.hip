@@ -845,7 +845,7 @@ void ternaspmm_rope_decode_attention_prefetch(const terna_bf16* qkv, const float
     AttentionPrefetch pf{};
     for (int r = 0; r < pf_count && pf.count < kAttentionPrefetchRegions; ++r) {
         const bool broadcast = pf_unit_bytes[r] == 0;        // every XCD fetches the whole (small) region
-        if (pf_ptr[r] == nullptr || (reinterpret_cast<uintptr_t>(pf_ptr[r]) & 15) || pf_bytes[r] < 16 ||
+        if (pf_ptr[r] == nullptr || (reinterpret_cast<uintptr_t>(pf_ptr[r]) & 15) || pf_bytes[r] < 16 || pf_bytes[r] > (1ll << 30) ||
             (!broadcast && (pf_unit_bytes[r] < 16 || (pf_unit_bytes[r] & 15) || pf_unit_bytes[r] > (1ll << 30))) ||
             (broadcast && pf_bytes[r] > (1ll << 20)))
             continue;
