@@ -161,7 +161,8 @@ def test_argmax_rows(lib, b, v):
 
 
 @pytest.mark.parametrize("m,v,k", [(1, 128256, 2560), (8, 128256, 2560), (16, 4096, 2560), (3, 1003, 64), (2, 50, 32),
-                                   (5, 8200, 6912), (16, 640, 4128)])
+                                   (5, 8200, 6912), (16, 640, 4128), (3, 1003, 384), (4, 8200, 6912), (1, 50, 128),
+                                   (4, 128256, 2560), (2, 4098, 2176)])
 def test_lm_head_against_fp64(lib, m, v, k):
     """bf16 LM head: within the bf16 GEMM bar of the fp64 product (max|err| <= 1e-2 max|ref|, median <= 1 ULP
     of the bf16 result), also for V not a multiple of 16 or 4, K that is not a multiple of the unrolled
