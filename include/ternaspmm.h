@@ -220,12 +220,13 @@ void ternaspmm_rope_decode_attention(const terna_bf16* qkv, const float* cos, co
 
 /* ternaspmm_rope_decode_attention with up to six prefetch regions (no counterpart in the reference).  The attention
  * of a decode step occupies one CU per (sequence, head); this variant adds workgroups on the CUs that stay idle, which
- * read pf_bytes[r] bytes at pf_ptr[r] (16-byte aligned device memory) and discard them: the weights of the launches that
+ * read pf_bytes[r] bytes (at most 1 GiB) at pf_ptr[r] (16-byte aligned device memory) and discard them: the weights of the launches that
  * follow then start in the L2s / the last-level cache instead of HBM.  A region is cut into units of pf_unit_bytes[r]
  * (a multiple of 16) that are spread over the XCDs round robin -- for a P2 weight, what one workgroup of the consuming
  * kernel reads: bands per workgroup x K/64 x 256 bytes -- so that a unit lands in the L2 its consumer will use;
  * pf_unit_bytes[r] = 0 marks a small region (at most 1 MiB: norm weights, scales) that every workgroup of the
  * consumers reads and every XCD therefore fetches whole.
+ * A region that breaks one of these rules is skipped.
  * pf_ptr / pf_bytes / pf_unit_bytes are host arrays of pf_count entries, read during the call.  Results are those of
  * ternaspmm_rope_decode_attention; nothing depends on where the prefetched bytes end up. */
 void ternaspmm_rope_decode_attention_prefetch(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
