@@ -216,7 +216,7 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
     const float* __restrict__ cosv, const float* __restrict__ sinv,
     const long long* __restrict__ pos, uint16_t* __restrict__ out, int H, int KV, int S, float scale,
-    float* partial, int* arrived, int splits, AttentionPrefetch pf, int heads)
+    float* partial, int* arrived, int splits, AttentionPrefetch pf, int heads, int groups)
 {
     static_assert(D == 64 || D == 128, "head dimension");
     constexpr int CH = D / 8;                    // 8-dimension chunks of a row
@@ -241,7 +241,22 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     TERNA_TS(0);
-    const int b = blockIdx.x / H, h = blockIdx.x - b * H;
+    // Workgroup -> (sequence, head).  Workgroups go to the 8 XCDs round robin, and the H / KV heads of a kv group read
+    // the same keys and values: with groups > 0 (= B * KV) the heads of group G all sit on XCD G mod 8, so that the
+    // group's cache prefix crosses the fabric once and its other heads hit in that L2 (the grid is padded to whole
+    // rounds of 8 groups; workgroups without a group leave).  groups = 0: heads in launch order.
+    int b, h;
+    if (groups > 0) {
+        const int per = H / KV, q = blockIdx.x >> 3;
+        const int G = 8 * (q / per) + (blockIdx.x & 7);
+        if (G >= groups) return;
+        b = G / KV;
+        h = (G - b * KV) * per + q % per;
+    } else {
+        b = blockIdx.x / H;
+        h = blockIdx.x - b * H;
+    }
+    const int bh = b * H + h;
     const int kvh = h / (H / KV);
     const int n = static_cast<int>(pos[0]) + 1;
     const uint16_t* kbase = cache_k + (static_cast<size_t>(b) * KV + kvh) * S * D;
@@ -482,7 +497,7 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     // device-scope fence would cost every workgroup) is needed.  Order: every thread's partial stores
     // have completed at the barrier, the arrival is counted after it, and the merging workgroup
     // reads after it has seen the full count.
-    float* mine = partial + (static_cast<size_t>(blockIdx.x) * SP + sp) * (D + 2);
+    float* mine = partial + (static_cast<size_t>(bh) * SP + sp) * (D + 2);
     auto publish = [](float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
     auto fetch = [](const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
     if (tid < D) publish(mine + tid, o);
@@ -492,11 +507,11 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     }
     __syncthreads();                             // waits for this workgroup's stores
     if (tid == 0)
-        last_flag = __hip_atomic_fetch_add(arrived + blockIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == SP - 1;
+        last_flag = __hip_atomic_fetch_add(arrived + bh, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == SP - 1;
     __syncthreads();
     if (!last_flag) return;
     if (tid < D) {
-        const float* head = partial + static_cast<size_t>(blockIdx.x) * SP * (D + 2);
+        const float* head = partial + static_cast<size_t>(bh) * SP * (D + 2);
         float m_all = -INFINITY;
         for (int j = 0; j < SP; ++j) m_all = fmaxf(m_all, fetch(head + j * (D + 2) + D));
         float num = 0.0f, den = 0.0f;
@@ -508,7 +523,7 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
         orow[tid] = float_to_bf16_bits(num / den);
     }
     // every split has arrived: ready for the next launch
-    if (tid == 0) __hip_atomic_store(arrived + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) __hip_atomic_store(arrived + bh, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 }  // namespace terna

@@ -411,6 +411,22 @@ int attention_waves(int B, int H)
     return static_cast<long>(B) * H <= 512 ? 8 : 4;
 }
 
+// Workgroups of the attention grid that stand for (sequence, head) pairs: B * H, or -- when kv groups are kept on one
+// XCD each (more than one head per group; TERNASPMM_ATTN_XCD_GROUPS=0 switches it off) -- whole rounds of 8 groups.
+bool attention_groups_on(int H, int KV)
+{
+    static const int on = [] {
+        const char* v = std::getenv("TERNASPMM_ATTN_XCD_GROUPS");
+        return v ? std::atoi(v) : 1;
+    }();
+    return on && H > KV;
+}
+int attention_slots(int B, int H, int KV)
+{
+    if (!attention_groups_on(H, KV)) return B * H;
+    return 8 * (H / KV) * ((B * KV + 7) / 8);
+}
+
 // Workspace of the split variant: one arrival counter per head (the caller zeroes them once), then
 // kAttentionMaxSplits partial results of D + 2 floats per head.
 size_t attention_counter_bytes(int B, int H) { return (static_cast<size_t>(B) * H * sizeof(int) + 255) & ~static_cast<size_t>(255); }
@@ -446,8 +462,10 @@ void launch_attention_as(const uint16_t* q, uint16_t* ck, uint16_t* cv, const fl
     if (lds > 64 * 1024) allow_dynamic_lds(kernel, 160 * 1024, "hipFuncSetAttribute(decode attention)", __LINE__);
     int* arrived = static_cast<int*>(workspace);
     float* partial = workspace ? reinterpret_cast<float*>(static_cast<char*>(workspace) + attention_counter_bytes(B, H)) : nullptr;
-    kernel<<<dim3(B * H + pf.workgroups, splits), dim3(64 * NW), lds, st>>>(q, ck, cv, cos, sin, pos, out, H, KV, S, scale,
-                                                                           partial, arrived, splits, pf, B * H);
+    const int slots = attention_slots(B, H, KV);
+    kernel<<<dim3(slots + pf.workgroups, splits), dim3(64 * NW), lds, st>>>(q, ck, cv, cos, sin, pos, out, H, KV, S, scale,
+                                                                           partial, arrived, splits, pf, slots,
+                                                                           attention_groups_on(H, KV) ? B * KV : 0);
 }
 
 template <bool ROPE, bool ADJ>
@@ -860,7 +878,8 @@ void ternaspmm_rope_decode_attention_prefetch(const terna_bf16* qkv, const float
         const char* v = std::getenv("TERNASPMM_ATTN_PREFETCH_WGS");
         return v ? std::atoi(v) / 8 * 8 : -1;
     }();
-    pf.workgroups = pf.count > 0 && B * H < 232 ? (forced_wgs >= 0 ? forced_wgs : (256 - B * H) / 8 * 8) : 0;
+    const int slots = attention_slots(B, H, KV);
+    pf.workgroups = pf.count > 0 && slots < 232 ? (forced_wgs >= 0 ? forced_wgs : (256 - slots) / 8 * 8) : 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (adjacent) launch_attention<true, true>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, workspace, pf, st);
     else launch_attention<true, false>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, workspace, pf, st);

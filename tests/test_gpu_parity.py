@@ -531,7 +531,8 @@ def test_kernel_binary_reference_command_line():
                                  {"TERNASPMM_DECODE_WAVES": "4"}, {"TERNASPMM_DECODE_WAVES": "8"}, {"TERNASPMM_DECODE_WAVES": "16"},
                                  {"TERNASPMM_DECODE_BANDS": "1"}, {"TERNASPMM_FUSED_BANDS": "1"},
                                  {"TERNASPMM_FUSED_BANDS_WAVES": "8"}, {"TERNASPMM_FUSED_WAVES": "8"},
-                                 {"TERNASPMM_ATTN_WAVES": "4"}, {"TERNASPMM_ATTN_SPLITS": "2"}, {"TERNASPMM_ATTN_SPLITS": "8"}])
+                                 {"TERNASPMM_ATTN_WAVES": "4"}, {"TERNASPMM_ATTN_SPLITS": "2"}, {"TERNASPMM_ATTN_SPLITS": "8"},
+                                 {"TERNASPMM_ATTN_XCD_GROUPS": "0"}])
 def test_tile_and_path_overrides(env):
     """Every tile shape, launch shape and path behind the library's tuning overrides
     (read once per process, hence a child process): tests/env_variant_check.py must pass under each."""
