@@ -110,7 +110,7 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
         const int jc = valid ? j : 0;
         use[t] = valid && row_ok;
 #pragma unroll
-        for (int b = 0; b < NB; ++b) wword[b][t] = packed[(static_cast<size_t>(band0 + b) * ktiles + jc) * 64 + i * 4 + g];
+        for (int b = 0; b < NB; ++b) wword[b][t] = packed[(static_cast<size_t>(band0 + b) * ktiles + jc) * 64 + lane];   // word L; operand order below
         const size_t off = static_cast<size_t>(row_ok ? row : 0) * pitch + jc * 64 + cl;
         xr[t].load(x + off);
         if constexpr (RES) rr[t].load(second + off);
@@ -258,8 +258,12 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
                 bq = __builtin_bit_cast(i32x4, *reinterpret_cast<const u32x4*>(slab + i * XQ::kPitch + g * 16));
             }
 #pragma unroll
-            for (int b = 0; b < NB; ++b)
-                acc[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(expand_word_i8(wword[b][t]), bq, acc[b], 0, 0, 0);
+            for (int b = 0; b < NB; ++b) {
+                // lane L loaded word L of the band-tile (consecutive lanes, consecutive words: the memory pipeline takes
+                // such a load in a quarter of the steps); the operand of lane L is word (L & 15) * 4 + (L >> 4)
+                const uint32_t w = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute((i * 4 + g) * 4, static_cast<int>(wword[b][t])));
+                acc[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(expand_word_i8(w), bq, acc[b], 0, 0, 0);
+            }
         }
     }
 

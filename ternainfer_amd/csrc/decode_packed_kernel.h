@@ -48,7 +48,10 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
     const int ktiles = K >> 6;
     const int i = lane & 15, g = lane >> 4;
 
-    const uint32_t* wp = packed + (static_cast<size_t>(band0) * ktiles + wave) * 64 + i * 4 + g;
+    // lane L loads word L of a band-tile -- consecutive lanes, consecutive words: the memory pipeline takes such a load in a
+    // quarter of the steps of the operand order (word (L & 15) * 4 + (L >> 4)), which one LDS-crossbar permutation restores
+    const uint32_t* wp = packed + (static_cast<size_t>(band0) * ktiles + wave) * 64 + lane;
+    const int operand_src = (i * 4 + g) * 4;
     const size_t band_pitch = static_cast<size_t>(ktiles) * 64;          // words from one band to the next
     // Coalesced activation pieces of this lane; rows past M are not loaded (their operand is zero
     // and their output column is never stored).
@@ -98,8 +101,9 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
             bf16x8 a0[NB], a1[NB];
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
-                a0[b] = __builtin_bit_cast(bf16x8, expand_chunk_bf16(cur.word[b]));
-                a1[b] = __builtin_bit_cast(bf16x8, expand_chunk_bf16(cur.word[b] >> 4));
+                const uint32_t w = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(operand_src, static_cast<int>(cur.word[b])));
+                a0[b] = __builtin_bit_cast(bf16x8, expand_chunk_bf16(w));
+                a1[b] = __builtin_bit_cast(bf16x8, expand_chunk_bf16(w >> 4));
             }
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
@@ -115,7 +119,8 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
         } else {
             i32x4 a[NB];
 #pragma unroll
-            for (int b = 0; b < NB; ++b) a[b] = expand_word_i8(cur.word[b]);
+            for (int b = 0; b < NB; ++b)
+                a[b] = expand_word_i8(static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(operand_src, static_cast<int>(cur.word[b]))));
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
                 const i32x4 bx = __builtin_bit_cast(
