@@ -11,7 +11,7 @@
 // blocks blockIdx.x, blockIdx.x + gridDim.x, ... so that the activations are staged once.
 #pragma once
 
-#include "terna_common.h"
+#include "norm_quant_kernel.h"
 
 namespace terna {
 
@@ -72,6 +72,65 @@ __global__ __launch_bounds__(kLmWaves * 64) void terna_lm_head_kernel(const uint
                     if (v0 + e < V) dst[e] = float_to_bf16_bits(acc[e]);
             }
         }
+    }
+}
+
+// Up to four rows of activations: a vocabulary row becomes four rows of the A operand (row i of A:
+// vocabulary row i / 4, the 16-byte pieces (i % 4) + 4 (L >> 4) of a 128-column step), so that four
+// consecutive lanes load 64 consecutive bytes -- a CU's memory pipeline takes one step per 64-byte
+// segment that consecutive lanes touch, 16 per load here against 64 with one vocabulary row per
+// operand row (above).  Column 4 m + r of B holds batch row m's matching pieces, out[i][4 m + i % 4]
+// is a partial logit, and the four partials of a vocabulary row meet in the four lanes of a quad.
+// UNROLL loads of a lane are in flight; it should divide K / 128.
+template <int UNROLL>
+__global__ __launch_bounds__(kLmWaves * 64) void terna_lm_head_quad_kernel(const uint16_t* __restrict__ x,
+                                                                           const uint16_t* __restrict__ w,
+                                                                           uint16_t* __restrict__ logits, int M, int V, int K)
+{
+    extern __shared__ __align__(16) uint8_t xs[];            // [M][K * 2 + 16]: padded pitch
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int pitch = K * 2 + 16;
+    const int row_vecs = K >> 3;
+    for (int p = tid; p < M * row_vecs; p += kLmWaves * 64) {
+        const int r = p / row_vecs, c = p - r * row_vecs;
+        *reinterpret_cast<u32x4*>(xs + r * pitch + 16 * c) = *reinterpret_cast<const u32x4*>(x + static_cast<size_t>(r) * K + 8 * c);
+    }
+    __syncthreads();
+
+    const int i = lane & 15, kg = lane >> 4;
+    const int piece = (i & 3) + 4 * kg;                      // 16 bytes of a 256-byte step of a row
+    const int steps = K >> 7;
+    const int m = i >> 2;                                    // B column i: batch row i / 4, pieces (i % 4) + 4 kg
+    const bool live = m < M;
+    const uint8_t* xrow = xs + (live ? m : 0) * pitch + 16 * piece;
+    const int blocks = (V + 3) >> 2;
+    for (int blk = blockIdx.x * kLmWaves + wave; blk < blocks; blk += gridDim.x * kLmWaves) {
+        const int row = blk * 4 + (i >> 2);
+        const uint16_t* wrow = w + static_cast<size_t>(row < V ? row : V - 1) * K + 8 * piece;
+        f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int s0 = 0; s0 < steps; s0 += UNROLL) {
+            u32x4 a[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const int s = s0 + u < steps ? s0 + u : steps - 1;
+                a[u] = *reinterpret_cast<const u32x4*>(wrow + 128 * s);
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const int s = s0 + u;
+                u32x4 b = *reinterpret_cast<const u32x4*>(xrow + 256 * (s < steps ? s : steps - 1));
+                if (s >= steps || !live) b = u32x4{0u, 0u, 0u, 0u};
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[u]), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
+            }
+        }
+        // lane (column i, rows 4 kg + v): operand row 4 kg + v is vocabulary row blk * 4 + kg, pieces v (mod 4):
+        // its partial for batch row m is in column 4 m + v
+        float part = (i & 3) == 0 ? acc[0] : (i & 3) == 1 ? acc[1] : (i & 3) == 2 ? acc[2] : acc[3];
+        part += dpp_permute<kDppSwapPairs>(part);
+        part += dpp_permute<kDppSwapHalfQuads>(part);
+        const int v = blk * 4 + kg;
+        if ((i & 3) == 0 && live && v < V) logits[static_cast<size_t>(m) * V + v] = float_to_bf16_bits(part);
     }
 }
 

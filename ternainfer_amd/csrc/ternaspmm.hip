@@ -936,7 +936,24 @@ void ternaspmm_lm_head_bf16(const terna_bf16* x, const terna_bf16* w, terna_bf16
     }();
     const int cap = forced > 0 ? forced : 512;               // two workgroups per CU measure fastest (256: 137 us, 512: 115 us, 1024: 119 us on 657 MB)
     const int grid = wgs_needed < cap ? wgs_needed : cap;
-    terna_lm_head_kernel<<<dim3(grid), dim3(kLmWaves * 64), lds, static_cast<hipStream_t>(stream)>>>(x, w, logits, M, V, K);
+    static const int quad = [] {
+        const char* v = std::getenv("TERNASPMM_LM_HEAD_QUAD");
+        return v ? std::atoi(v) : 1;
+    }();
+    const int ksteps = K / 128;
+    if (quad && M <= 4 && (K & 127) == 0) {
+        const int qwgs = ((V + 3) / 4 + kLmWaves - 1) / kLmWaves;
+        const dim3 qgrid(qwgs < cap ? qwgs : cap);
+        if (ksteps % 10 == 0) {
+            if (lds > 64 * 1024) allow_dynamic_lds(terna_lm_head_quad_kernel<10>, 160 * 1024, "hipFuncSetAttribute(lm head)", __LINE__);
+            terna_lm_head_quad_kernel<10><<<qgrid, dim3(kLmWaves * 64), lds, static_cast<hipStream_t>(stream)>>>(x, w, logits, M, V, K);
+        } else {
+            if (lds > 64 * 1024) allow_dynamic_lds(terna_lm_head_quad_kernel<8>, 160 * 1024, "hipFuncSetAttribute(lm head)", __LINE__);
+            terna_lm_head_quad_kernel<8><<<qgrid, dim3(kLmWaves * 64), lds, static_cast<hipStream_t>(stream)>>>(x, w, logits, M, V, K);
+        }
+    } else {
+        terna_lm_head_kernel<<<dim3(grid), dim3(kLmWaves * 64), lds, static_cast<hipStream_t>(stream)>>>(x, w, logits, M, V, K);
+    }
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_lm_head_bf16", e, __LINE__);
 }

@@ -166,7 +166,8 @@ def test_argmax_rows(lib, b, v):
 def test_lm_head_against_fp64(lib, m, v, k):
     """bf16 LM head: within the bf16 GEMM bar of the fp64 product (max|err| <= 1e-2 max|ref|, median <= 1 ULP
     of the bf16 result), also for V not a multiple of 16 or 4, K that is not a multiple of the unrolled
-    depth, and K whose 16 activation rows need more than 64 KB of LDS."""
+    depth, and K whose 16 activation rows need more than 64 KB of LDS.  Up to four rows with K a multiple of 128
+    take the kernel whose quads of lanes load 64 contiguous bytes, everything else the plain one."""
     import ternainfer_amd as T
     rng = np.random.default_rng(4100 + m + v + k)
     x = O.f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
