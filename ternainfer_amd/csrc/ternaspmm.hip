@@ -735,11 +735,12 @@ static int launch_decode_fused(int mode, const terna_bf16* x, const terna_bf16* 
         const char* v = std::getenv("TERNASPMM_FUSED_WAVES");
         return v ? std::atoi(v) : 0;
     }();
-    // same split as the unfused small-M kernel; TERNASPMM_FUSED_WAVES=8|16 forces one (tuning aid)
-    const bool wide = forced_waves == 16 ? true : (forced_waves == 8 ? mode == FUSED_GLU : bands <= 256);
+    // 8 waves of up to 5 band-tiles where K allows (measured: +2 % tokens/s over 16 waves of 3 once the weight loads
+    // were lane-contiguous), 16 waves for longer K and for the gate variant; TERNASPMM_FUSED_WAVES=8|16 forces one
+    const bool wide = forced_waves == 16 ? true : (forced_waves == 8 ? mode == FUSED_GLU : mode == FUSED_GLU || ktiles > 8 * 5);
     const uint32_t* p = static_cast<const uint32_t*>(packed);
     // More bands than CUs: four bands per workgroup, so that the grid is one round and the prologue runs once
-    // per CU.  TERNASPMM_FUSED_BANDS=1 switches that off, TERNASPMM_FUSED_BANDS_WAVES=8 picks the 8-wave
+    // per CU.  TERNASPMM_FUSED_BANDS=1 switches that off, TERNASPMM_FUSED_BANDS_WAVES=16 picks the 16-wave
     // variant of it (tuning aids).
     static const int forced_nb = [] {
         const char* v = std::getenv("TERNASPMM_FUSED_BANDS");
@@ -747,11 +748,11 @@ static int launch_decode_fused(int mode, const terna_bf16* x, const terna_bf16* 
     }();
     static const int nb_waves = [] {
         const char* v = std::getenv("TERNASPMM_FUSED_BANDS_WAVES");
-        return v && std::atoi(v) == 8 ? 8 : 16;
+        return v && std::atoi(v) == 16 ? 16 : 8;
     }();
     const bool multi = forced_nb != 1 && bands > 256 && bands % 4 == 0 && mode != FUSED_GLU;
-    const bool multi16 = multi && nb_waves == 16 && ktiles <= 16 * 3;
-    const bool multi8 = multi && !multi16 && ktiles <= 8 * 5;
+    const bool multi8 = multi && nb_waves == 8 && ktiles <= 8 * 5;
+    const bool multi16 = multi && !multi8 && ktiles <= 16 * 3;
     const dim3 grid(multi16 || multi8 ? bands / 4 : bands);
 #define TERNA_FUSED(WAVES, TMAX, MODE, MP, NB)                                                                     \
     terna_decode_fused_kernel<WAVES, TMAX, MODE, MP, NB><<<grid, dim3(WAVES * 64), 0, st>>>(                       \

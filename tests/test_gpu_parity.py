@@ -530,7 +530,7 @@ def test_kernel_binary_reference_command_line():
                                  {"TERNASPMM_PREFILL_XCD_MAP": "1"}, {"TERNASPMM_PREFILL_XCD_MAP": "1", "TERNASPMM_PREFILL_BM": "128"},
                                  {"TERNASPMM_DECODE_WAVES": "4"}, {"TERNASPMM_DECODE_WAVES": "8"}, {"TERNASPMM_DECODE_WAVES": "16"},
                                  {"TERNASPMM_DECODE_BANDS": "1"}, {"TERNASPMM_FUSED_BANDS": "1"},
-                                 {"TERNASPMM_FUSED_BANDS_WAVES": "8"}, {"TERNASPMM_FUSED_WAVES": "8"},
+                                 {"TERNASPMM_FUSED_BANDS_WAVES": "16"}, {"TERNASPMM_FUSED_WAVES": "8"}, {"TERNASPMM_FUSED_WAVES": "16"},
                                  {"TERNASPMM_ATTN_WAVES": "4"}, {"TERNASPMM_ATTN_SPLITS": "2"}, {"TERNASPMM_ATTN_SPLITS": "8"},
                                  {"TERNASPMM_ATTN_XCD_GROUPS": "0"}])
 def test_tile_and_path_overrides(env):
