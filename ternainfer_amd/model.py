@@ -174,7 +174,7 @@ class Block:
                 return lin.quantised(*relu2_mul_rmsnorm_quant(x, weight, eps)), None
             return lin.dense(relu2_mul_rmsnorm_quant(x, weight, eps, quant=False)), None
         if self.act == "int8":
-            if x.shape[0] == 1:            # single-row decode step: prologue and linear in one launch
+            if x.shape[0] <= 8:            # decode step: prologue and linear in one launch where that is faster
                 return rmsnorm_linear_packed(x, weight, eps, lin.packed, lin.ws, lin.ws_num, lin.n, residual=residual)
             xq, s, h = rmsnorm_quant(x, weight, eps, residual=residual)
             return lin.quantised(xq, s), h
