@@ -199,6 +199,11 @@ int bitlinear_TernaSpMM_packed_fused_glu(const terna_bf16* x13, const terna_bf16
  * h / (H/KV) at slots 0 .. pos[0]; out bf16 [B][H*D] = softmax(scale * q K^T) V.  D is 64 or 128,
  * S <= 8192.  Both only enqueue.
  *
+ * Precondition on `pos` (device memory, which the host side of the call cannot inspect): 0 <= pos[t] < S.  A
+ * position outside the cache writes no k / v row and the attention runs over the prefix clamped to [1, S]
+ * slots: the result is then meaningless but every access stays inside the caller's buffers.  All sequences of
+ * the batch share the one position: the entry points have no per-sequence prefix lengths.
+ *
  * `workspace` (may be NULL): device memory of ternaspmm_attention_workspace_bytes(B, H, D) bytes, zero-filled by
  * the caller once before its first use.  With it the cache prefix of every head is split over up to 8 workgroups
  * (one CU streams a prefix at a few tens of GB/s, so few heads on the chip are bound by that); each leaves a partial

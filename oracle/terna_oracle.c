@@ -16,6 +16,8 @@
  *   oracle_spmm_i8_*      pinned  (integer matmul is exact; x==1 gives row sums, the
  *                                  construction of the reference's tests/test_kernel.cu:81)
  *   oracle_spmm_bf16      pinned  (plain fp64 matmul)
+ *   oracle_quant_input    pinned  (answers worked by hand: ties to even, scales that are exact,
+ *                                  round down and round up in bf16, the all-zero row)
  *
  * Build: make -C oracle   (gcc -O2 -shared -fPIC)
  */
@@ -307,9 +309,10 @@ void oracle_spmm_bf16(const uint16_t* x, const int8_t* w, const float* scale, in
  * model.py:120-123 (SpBitLinear.quant_input), with the one definition this build
  * fixes for the precision the reference leaves open: compute in fp32,
  * s = bf16_rn(127 / max(|x|, 1e-5)), and that rounded s is used both to quantise
- * and in the epilogue.  x is bf16 storage.  "parity unpinned" beyond the formula:
- * the reference runs this under torch.compile and nothing in it fixes the
- * intermediate precision. */
+ * and in the epilogue.  x is bf16 storage.  (The reference's eager mode multiplies
+ * in the tensor's dtype and its compiled graph in fp32 with the unrounded quotient;
+ * the known answers in tests/test_oracle_linear.py include a row on which the
+ * three differ.) */
 void oracle_quant_input(const uint16_t* x, int M, int K, int8_t* xq, uint16_t* s)
 {
     for (int m = 0; m < M; ++m) {

@@ -19,9 +19,12 @@ Reference files restated (paths relative to the reference checkout):
   convert/convert_TernaInfer.py:159-194      weight ternarisation and scale packing
   model.py:120-123                           activation quantisation
 
-Parity status: every function is pinned by a test in tests/test_oracle_*.py except
-``quant_input``'s intermediate precision, which the reference leaves open
-("parity unpinned" beyond the two-line formula), and ``rmsnorm``, ``rope_rotate_half``,
+Parity status: every function is pinned by a test in tests/test_oracle_*.py --
+``quant_input`` and ``quant_weight_int8`` by answers worked by hand (ties to even, scales
+that are exact / round down / round up in bf16, the clamps; tests/test_oracle_linear.py).
+``quant_input`` fixes one definition where the reference's two execution modes differ
+(eager multiplies in the tensor's dtype, the compiled graph in fp32): fp32 product with
+the bf16-rounded s, the s the epilogue divides by.  Except ``rmsnorm``, ``rope_rotate_half``,
 ``rope_adjacent`` and ``attention_one_token``: the reference takes RMSNorm, rope_padded
 and the attention forward from xformers.ops (model.py:16), a third-party dependency that
 is not part of the reference checkout and not installed here, so "parity unpinned"; the
@@ -218,26 +221,28 @@ def ws_group_prefill(cols: np.ndarray, n: int, ws_num: int) -> np.ndarray:
 
 
 def spmm_i8(x_q: np.ndarray, w: np.ndarray, s_bits: np.ndarray, ws_bits: np.ndarray,
-            ws_num: int, mode: int) -> np.ndarray:
+            ws_num: int, mode: int, cols: np.ndarray | None = None) -> np.ndarray:
     """Integer matmul + reference epilogue -> bf16 storage [M, N].
 
     mode 0: bf16((float(acc)/s)*ws)      Reduction_Kernel.cuh:60
     mode 1: bf16(float(acc)*(ws/s)), coefficient 0 where s == 0   epilogue_visitor_scale_ws.h:188-205
+    `cols`: only these output columns (weight-scale groups still follow the full N) -> [M, len(cols)];
+    keeps the host matmul small at the largest shapes.
     """
     m, _ = x_q.shape
     n = w.shape[0]
+    cols = np.arange(n) if cols is None else np.asarray(cols)
     # integer matmul through fp64 BLAS: exact while |acc| < 2^53 (here |acc| <= 128*K)
-    acc = np.rint(x_q.astype(np.float64) @ w.astype(np.float64).T).astype(np.int64)
+    acc = np.rint(x_q.astype(np.float64) @ w[cols].astype(np.float64).T).astype(np.int64)
     assert np.abs(acc).max(initial=0) < 2 ** 24
     accf = acc.astype(np.float32)
     s = bf16_bits_to_f32(s_bits).reshape(m, 1).astype(np.float32)
-    cols = np.arange(n)
     with np.errstate(divide="ignore", invalid="ignore"):
         if mode == 0:
-            wsv = bf16_bits_to_f32(ws_bits)[ws_group_decode(cols, n, ws_num)].reshape(1, n)
+            wsv = bf16_bits_to_f32(ws_bits)[ws_group_decode(cols, n, ws_num)].reshape(1, -1)
             r = (accf / s).astype(np.float32) * wsv.astype(np.float32)
         else:
-            wsv = bf16_bits_to_f32(ws_bits)[ws_group_prefill(cols, n, ws_num)].reshape(1, n)
+            wsv = bf16_bits_to_f32(ws_bits)[ws_group_prefill(cols, n, ws_num)].reshape(1, -1)
             coeff = np.where(s != 0, (wsv / s).astype(np.float32), np.float32(0)).astype(np.float32)
             r = accf * coeff
     return f32_to_bf16_bits(r.astype(np.float32))
@@ -260,6 +265,17 @@ def quant_input(x_bits: np.ndarray):
     s = bf16_bits_to_f32(s_bits)
     q = np.clip(np.rint((x * s).astype(np.float32)), -128, 127).astype(np.int8)
     return q, s_bits.reshape(-1)
+
+
+def bf16_bitlinear_golden(x_bits: np.ndarray, w_dense_bits: np.ndarray) -> np.ndarray:
+    """model.py:135-153 (BF16BitLinear.forward, the reference's dense golden mode): quant_input, then
+    F.linear(x_q as bf16, W) / s with W = ternary * scale stored dense in bf16 (convert_TernaInfer.py:112-114).
+    Evaluated in float64 -> [M, N]; a composition of quant_input (pinned by known answers) and a float64
+    matmul, so the reference's two bf16 roundings (GEMM output, quotient) show up as tolerance in the caller."""
+    q, s_bits = quant_input(x_bits)
+    w = bf16_bits_to_f32(w_dense_bits).astype(np.float64)
+    s = bf16_bits_to_f32(s_bits).astype(np.float64).reshape(-1, 1)
+    return (q.astype(np.float64) @ w.T) / s
 
 
 # --------------------------------------------------------------------------- glue between two linears

@@ -1,0 +1,221 @@
+// C ABI of the attention-side kernels of a decode step (attention_kernel.h): RoPE + cache write, single-token
+// attention, both in one launch, and the prefetching variant.
+// Declarations: include/ternaspmm.h.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <mutex>
+
+#include "../../include/ternaspmm.h"
+#include "host_util.h"
+#include "attention_kernel.h"
+
+using namespace terna;
+
+namespace {
+
+// Waves per workgroup of the decode attention: with one workgroup per (sequence, head) and few of them
+// on the chip, wider workgroups request more of the cache up front (64 slots of keys per wave).
+// TERNASPMM_ATTN_WAVES=4|8 forces one (tuning aid).  Both entry points use the same rule, so their results
+// stay bit-identical.
+int attention_waves(int B, int H)
+{
+    static const int forced = [] {
+        const char* v = std::getenv("TERNASPMM_ATTN_WAVES");
+        const int w = v ? std::atoi(v) : 0;
+        return (w == 4 || w == 8) ? w : 0;
+    }();
+    if (forced) return forced;
+    return static_cast<long>(B) * H <= 512 ? 8 : 4;
+}
+
+// Workgroups of the attention grid that stand for (sequence, head) pairs: B * H, or -- when kv groups are kept on one
+// XCD each (more than one head per group; TERNASPMM_ATTN_XCD_GROUPS=0 switches it off) -- whole rounds of 8 groups.
+bool attention_groups_on(int H, int KV)
+{
+    static const int on = [] {
+        const char* v = std::getenv("TERNASPMM_ATTN_XCD_GROUPS");
+        return v ? std::atoi(v) : 1;
+    }();
+    return on && H > KV;
+}
+int attention_slots(int B, int H, int KV)
+{
+    if (!attention_groups_on(H, KV)) return B * H;
+    return 8 * (H / KV) * ((B * KV + 7) / 8);
+}
+
+// Workspace of the split variant: one arrival counter per head (the caller zeroes them once), then
+// kAttentionMaxSplits partial results of D + 2 floats per head.
+size_t attention_counter_bytes(int B, int H) { return (static_cast<size_t>(B) * H * sizeof(int) + 255) & ~static_cast<size_t>(255); }
+
+// Splits of the cache per head: as many as keep the grid within two workgroups per CU, at most 8; 1 without
+// a workspace, and 1 for caches below 1024 slots, where the merge (three dependent trips to device memory,
+// 4-5 us) costs more than streaming the prefix from one CU.  TERNASPMM_ATTN_SPLITS=1|2|4|8 forces one
+// (tuning aid).
+// Where the split variant keeps its arrival counters (one int per head, zero between launches) and its partial
+// results: carved out of the caller's workspace, or the library's own static array (the entry point that
+// allocates nothing).
+struct AttentionScratch {
+    int* arrived = nullptr;
+    float* partial = nullptr;
+};
+AttentionScratch attention_scratch_of(void* workspace, int B, int H)
+{
+    if (workspace == nullptr) return {};
+    return {static_cast<int*>(workspace),
+            reinterpret_cast<float*>(static_cast<char*>(workspace) + attention_counter_bytes(B, H))};
+}
+
+int attention_splits(int B, int H, int S, const AttentionScratch& scratch)
+{
+    if (scratch.arrived == nullptr) return 1;
+    static const int forced = [] {
+        const char* v = std::getenv("TERNASPMM_ATTN_SPLITS");
+        const int n = v ? std::atoi(v) : 0;
+        return (n == 1 || n == 2 || n == 4 || n == 8) ? n : 0;
+    }();
+    if (forced) return forced;
+    if (S < 1024) return 1;
+    int sp = 1;
+    while (sp < kAttentionMaxSplits && static_cast<long>(B) * H * sp * 2 <= 512) sp *= 2;
+    return sp;
+}
+
+template <int D, bool ROPE, bool ADJ, int NW, bool SPLIT>
+void launch_attention_as(const uint16_t* q, uint16_t* ck, uint16_t* cv, const float* cos, const float* sin,
+                         const long long* pos, uint16_t* out, int B, int H, int KV, int S, float scale, int splits,
+                         const AttentionScratch& scratch, const AttentionPrefetch& pf_in, hipStream_t st)
+{
+    AttentionPrefetch pf = pf_in;
+    if (splits > 1) pf.workgroups = 0;                       // the split grid is two-dimensional: no extra workgroups
+    auto kernel = terna_decode_attention_kernel<D, ROPE, ADJ, NW, SPLIT>;
+    const size_t lds = decode_attention_lds_bytes(D, NW, S);
+    if (lds > 64 * 1024) allow_dynamic_lds(kernel, 160 * 1024, "hipFuncSetAttribute(decode attention)", __LINE__);
+    const int slots = attention_slots(B, H, KV);
+    kernel<<<dim3(slots + pf.workgroups, splits), dim3(64 * NW), lds, st>>>(q, ck, cv, cos, sin, pos, out, H, KV, S, scale,
+                                                                           scratch.partial, scratch.arrived, splits, pf, slots,
+                                                                           attention_groups_on(H, KV) ? B * KV : 0);
+}
+
+template <bool ROPE, bool ADJ>
+void launch_attention(const uint16_t* q, uint16_t* ck, uint16_t* cv, const float* cos, const float* sin,
+                             const long long* pos, uint16_t* out, int B, int H, int KV, int D, int S, float scale,
+                             const AttentionScratch& scratch, const AttentionPrefetch& pf, hipStream_t st)
+{
+    const int splits = attention_splits(B, H, S, scratch);
+    const int nw = splits > 1 ? 4 : attention_waves(B, H);       // a split is a short prefix: the narrow workgroup
+#define TERNA_ATTN(DIM, NWAVES, SPLIT) \
+    launch_attention_as<DIM, ROPE, ADJ, NWAVES, SPLIT>(q, ck, cv, cos, sin, pos, out, B, H, KV, S, scale, splits, scratch, pf, st)
+    if (D == 128) {
+        if (splits > 1) TERNA_ATTN(128, 4, true);
+        else if (nw == 8) TERNA_ATTN(128, 8, false);
+        else TERNA_ATTN(128, 4, false);
+    } else {
+        if (splits > 1) TERNA_ATTN(64, 4, true);
+        else if (nw == 8) TERNA_ATTN(64, 8, false);
+        else TERNA_ATTN(64, 4, false);
+    }
+#undef TERNA_ATTN
+}
+
+bool attention_args_ok(const char* who, int B, int H, int KV, int D, int S)
+{
+    if (B < 1 || H < 1 || KV < 1 || H % KV != 0 || (D != 64 && D != 128) || S < 1 || S > 8192) {
+        std::fprintf(stderr, "%s: unsupported arguments (H=%d KV=%d D=%d S=%d)\n", who, H, KV, D, S);
+        return false;
+    }
+    return true;
+}
+
+}  // namespace
+
+extern "C" {
+
+void ternaspmm_rope_kv_store(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
+                             terna_bf16* q_out, terna_bf16* cache_k, terna_bf16* cache_v, int B, int T, int H,
+                             int KV, int D, int S, int adjacent, terna_stream stream)
+{
+    if (B < 1 || T < 1 || H < 1 || KV < 1 || D < 2 || (D & 1) || S < 1) {
+        std::fprintf(stderr, "ternaspmm_rope_kv_store: unsupported arguments\n");
+        return;
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (adjacent)
+        terna_rope_kv_store_kernel<true><<<dim3(B * T), dim3(256), 0, st>>>(qkv, cos, sin, pos, q_out, cache_k, cache_v, T, H, KV, D, S);
+    else
+        terna_rope_kv_store_kernel<false><<<dim3(B * T), dim3(256), 0, st>>>(qkv, cos, sin, pos, q_out, cache_k, cache_v, T, H, KV, D, S);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_rope_kv_store", e, __LINE__);
+}
+
+long long ternaspmm_attention_workspace_bytes(int B, int H, int D)
+{
+    if (B < 1 || H < 1 || D < 1) return -1;
+    return static_cast<long long>(attention_counter_bytes(B, H)) +
+           static_cast<long long>(B) * H * kAttentionMaxSplits * (D + 2) * sizeof(float);
+}
+
+void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
+                                const long long* pos, terna_bf16* out, int B, int H, int KV, int D, int S,
+                                float scale, void* workspace, terna_stream stream)
+{
+    if (!attention_args_ok("ternaspmm_decode_attention", B, H, KV, D, S)) return;
+    // the kernel writes the caches only in its ROPE variant
+    launch_attention<false, false>(q, const_cast<uint16_t*>(cache_k), const_cast<uint16_t*>(cache_v), nullptr, nullptr, pos,
+                                   out, B, H, KV, D, S, scale, attention_scratch_of(workspace, B, H), AttentionPrefetch{},
+                                   static_cast<hipStream_t>(stream));
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_decode_attention", e, __LINE__);
+}
+
+void ternaspmm_rope_decode_attention(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
+                                     terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
+                                     int D, int S, float scale, int adjacent, void* workspace, terna_stream stream)
+{
+    if (!attention_args_ok("ternaspmm_rope_decode_attention", B, H, KV, D, S)) return;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const AttentionScratch scratch = attention_scratch_of(workspace, B, H);
+    if (adjacent) launch_attention<true, true>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, scratch, AttentionPrefetch{}, st);
+    else launch_attention<true, false>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, scratch, AttentionPrefetch{}, st);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_rope_decode_attention", e, __LINE__);
+}
+
+void ternaspmm_rope_decode_attention_prefetch(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
+                                              terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
+                                              int D, int S, float scale, int adjacent, void* workspace,
+                                              const void* const* pf_ptr, const long long* pf_bytes, const long long* pf_unit_bytes,
+                                              int pf_count, terna_stream stream)
+{
+    if (!attention_args_ok("ternaspmm_rope_decode_attention_prefetch", B, H, KV, D, S)) return;
+    AttentionPrefetch pf{};
+    for (int r = 0; r < pf_count && pf.count < kAttentionPrefetchRegions; ++r) {
+        const bool broadcast = pf_unit_bytes[r] == 0;        // every XCD fetches the whole (small) region
+        if (pf_ptr[r] == nullptr || (reinterpret_cast<uintptr_t>(pf_ptr[r]) & 15) || pf_bytes[r] < 16 || pf_bytes[r] > (1ll << 30) ||
+            (!broadcast && (pf_unit_bytes[r] < 16 || (pf_unit_bytes[r] & 15) || pf_unit_bytes[r] > (1ll << 30))) ||
+            (broadcast && pf_bytes[r] > (1ll << 20)))
+            continue;
+        const int c = pf.count++;
+        pf.base[c] = static_cast<const u32x4*>(pf_ptr[r]);
+        pf.total_vecs[c] = pf_bytes[r] / 16;
+        pf.unit_vecs[c] = broadcast ? 0 : static_cast<int>(pf_unit_bytes[r] / 16);
+        pf.units[c] = broadcast ? 1 : (pf.total_vecs[c] + pf.unit_vecs[c] - 1) / pf.unit_vecs[c];
+    }
+    // the heads take B*H CUs; the rest of the chip prefetches
+    static const int forced_wgs = [] {
+        const char* v = std::getenv("TERNASPMM_ATTN_PREFETCH_WGS");
+        return v ? std::atoi(v) / 8 * 8 : -1;
+    }();
+    const int slots = attention_slots(B, H, KV);
+    pf.workgroups = pf.count > 0 && slots < 232 ? (forced_wgs >= 0 ? forced_wgs : (256 - slots) / 8 * 8) : 0;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const AttentionScratch scratch = attention_scratch_of(workspace, B, H);
+    if (adjacent) launch_attention<true, true>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, scratch, pf, st);
+    else launch_attention<true, false>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, scratch, pf, st);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_rope_decode_attention_prefetch", e, __LINE__);
+}
+
+}  // extern "C"

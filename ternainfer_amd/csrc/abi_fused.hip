@@ -1,0 +1,128 @@
+// C ABI of the fused prologue of a ternary linear: norm / gate / activation quantisation as kernels of their own
+// (norm_quant_kernel.h) and inside the small-M linear (decode_fused_kernel.h).  Declarations: include/ternaspmm.h.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+
+#include "../../include/ternaspmm.h"
+#include "host_util.h"
+#include "norm_quant_kernel.h"
+#include "decode_fused_kernel.h"
+
+using namespace terna;
+
+extern "C" {
+
+void ternaspmm_rmsnorm_quant(const terna_bf16* x, const terna_bf16* residual, terna_bf16* sum_out,
+                             const terna_bf16* weight, float eps, terna_bf16* y_out, int8_t* xq_out,
+                             terna_bf16* s_out, int M, int K, terna_stream stream)
+{
+    if (M < 1 || K < 8 || (K & 7) || K > 8 * kNormThreads * kNormMaxVecs || (xq_out != nullptr) != (s_out != nullptr)) {
+        std::fprintf(stderr, "ternaspmm_rmsnorm_quant: unsupported arguments (M=%d K=%d)\n", M, K);
+        return;
+    }
+    terna_norm_quant_kernel<false><<<dim3(M), dim3(kNormThreads), 0, static_cast<hipStream_t>(stream)>>>(
+        x, residual, sum_out, weight, eps, y_out, xq_out, s_out, K);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_rmsnorm_quant", e, __LINE__);
+}
+
+void ternaspmm_relu2_mul_rmsnorm_quant(const terna_bf16* x13, const terna_bf16* weight, float eps, terna_bf16* y_out,
+                                       int8_t* xq_out, terna_bf16* s_out, int M, int F, terna_stream stream)
+{
+    if (M < 1 || F < 8 || (F & 7) || F > 8 * kNormThreads * kNormMaxVecs || (xq_out != nullptr) != (s_out != nullptr)) {
+        std::fprintf(stderr, "ternaspmm_relu2_mul_rmsnorm_quant: unsupported arguments (M=%d F=%d)\n", M, F);
+        return;
+    }
+    terna_norm_quant_kernel<true><<<dim3(M), dim3(kNormThreads), 0, static_cast<hipStream_t>(stream)>>>(
+        x13, nullptr, nullptr, weight, eps, y_out, xq_out, s_out, F);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_relu2_mul_rmsnorm_quant", e, __LINE__);
+}
+
+// mode: FUSED_PLAIN / FUSED_RESIDUAL / FUSED_GLU.  Returns 1 when a launch was enqueued.
+static int launch_decode_fused(int mode, const terna_bf16* x, const terna_bf16* residual, terna_bf16* sum_out,
+                               const terna_bf16* norm_weight, float eps, const void* packed, terna_bf16* out,
+                               const terna_bf16* ws, int ws_num, int8_t* xq_out, terna_bf16* s_out, int M, int N,
+                               int K, hipStream_t st)
+{
+    if (!shape_ok(M, N, K) || !groups_ok(ws_num) || M > 16) return 0;
+    const int ktiles = K / 64;
+    const int bands = N / 16;
+    static const int forced_waves = [] {
+        const char* v = std::getenv("TERNASPMM_FUSED_WAVES");
+        return v ? std::atoi(v) : 0;
+    }();
+    // 8 waves of up to 5 band-tiles where K allows (measured: +2 % tokens/s over 16 waves of 3 once the weight loads
+    // were lane-contiguous), 16 waves for longer K and for the gate variant; TERNASPMM_FUSED_WAVES=8|16 forces one
+    const bool wide = forced_waves == 16 ? true : (forced_waves == 8 ? mode == FUSED_GLU : mode == FUSED_GLU || ktiles > 8 * 5);
+    const uint32_t* p = static_cast<const uint32_t*>(packed);
+    // More bands than CUs: four bands per workgroup, so that the grid is one round and the prologue runs once
+    // per CU.  TERNASPMM_FUSED_BANDS=1 switches that off, TERNASPMM_FUSED_BANDS_WAVES=16 picks the 16-wave
+    // variant of it (tuning aids).
+    static const int forced_nb = [] {
+        const char* v = std::getenv("TERNASPMM_FUSED_BANDS");
+        return v ? std::atoi(v) : 0;
+    }();
+    static const int nb_waves = [] {
+        const char* v = std::getenv("TERNASPMM_FUSED_BANDS_WAVES");
+        return v && std::atoi(v) == 16 ? 16 : 8;
+    }();
+    const bool multi = forced_nb != 1 && bands > 256 && bands % 4 == 0 && mode != FUSED_GLU;
+    const bool multi8 = multi && nb_waves == 8 && ktiles <= 8 * 5;
+    const bool multi16 = multi && !multi8 && ktiles <= 16 * 3;
+    const dim3 grid(multi16 || multi8 ? bands / 4 : bands);
+#define TERNA_FUSED(WAVES, TMAX, MODE, MP, NB)                                                                     \
+    terna_decode_fused_kernel<WAVES, TMAX, MODE, MP, NB><<<grid, dim3(WAVES * 64), 0, st>>>(                       \
+        x, residual, sum_out, norm_weight, eps, p, out, ws, ws_num, xq_out, s_out, M, N, K)
+#define TERNA_FUSED_M(WAVES, TMAX, MODE, NB)                                                                       \
+    do {                                                                                                           \
+        if (M == 1) TERNA_FUSED(WAVES, TMAX, MODE, 1, NB);                                                         \
+        else if (M <= 8) TERNA_FUSED(WAVES, TMAX, MODE, 8, NB);                                                    \
+        else TERNA_FUSED(WAVES, TMAX, MODE, 16, NB);                                                               \
+    } while (0)
+    if (mode == FUSED_GLU) {
+        // long K (the down projection): only the single-row variant, whose per-lane state is tiny
+        if (M != 1 || !wide || ktiles > 16 * 7) return 0;
+        TERNA_FUSED(16, 7, FUSED_GLU, 1, 1);
+    } else if (multi16) {
+        if (mode == FUSED_RESIDUAL) TERNA_FUSED_M(16, 3, FUSED_RESIDUAL, 4);
+        else TERNA_FUSED_M(16, 3, FUSED_PLAIN, 4);
+    } else if (multi8) {
+        if (mode == FUSED_RESIDUAL) TERNA_FUSED_M(8, 5, FUSED_RESIDUAL, 4);
+        else TERNA_FUSED_M(8, 5, FUSED_PLAIN, 4);
+    } else if (wide) {
+        if (ktiles > 16 * 3) return 0;
+        if (mode == FUSED_RESIDUAL) TERNA_FUSED_M(16, 3, FUSED_RESIDUAL, 1);
+        else TERNA_FUSED_M(16, 3, FUSED_PLAIN, 1);
+    } else {
+        if (ktiles > 8 * 5) return 0;
+        if (mode == FUSED_RESIDUAL) TERNA_FUSED_M(8, 5, FUSED_RESIDUAL, 1);
+        else TERNA_FUSED_M(8, 5, FUSED_PLAIN, 1);
+    }
+#undef TERNA_FUSED_M
+#undef TERNA_FUSED
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("bitlinear_TernaSpMM_packed_fused", e, __LINE__);
+    return 1;
+}
+
+int bitlinear_TernaSpMM_packed_fused(const terna_bf16* x, const terna_bf16* residual, terna_bf16* sum_out,
+                                     const terna_bf16* norm_weight, float eps, const void* packed, terna_bf16* out,
+                                     const terna_bf16* ws, int ws_num, int8_t* xq_out, terna_bf16* s_out, int M,
+                                     int N, int K, terna_stream stream)
+{
+    return launch_decode_fused(residual ? FUSED_RESIDUAL : FUSED_PLAIN, x, residual, sum_out, norm_weight, eps, packed, out,
+                               ws, ws_num, xq_out, s_out, M, N, K, static_cast<hipStream_t>(stream));
+}
+
+int bitlinear_TernaSpMM_packed_fused_glu(const terna_bf16* x13, const terna_bf16* norm_weight, float eps,
+                                         const void* packed, terna_bf16* out, const terna_bf16* ws, int ws_num,
+                                         int8_t* xq_out, terna_bf16* s_out, int M, int N, int F, terna_stream stream)
+{
+    return launch_decode_fused(FUSED_GLU, x13, nullptr, nullptr, norm_weight, eps, packed, out, ws, ws_num, xq_out, s_out,
+                               M, N, F, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

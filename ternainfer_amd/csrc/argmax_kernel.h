@@ -154,8 +154,10 @@ __global__ __launch_bounds__(kGreedyThreads) void terna_greedy_step_kernel(const
         for (int w = 1; w < kGreedyThreads / 64; ++w) argmax_merge(best, idx, sv[w], si[w]);
         const unsigned long long packed = (static_cast<unsigned long long>(__float_as_uint(best)) << 32) | static_cast<unsigned>(idx);
         __hip_atomic_store(partial + b * kGreedyChunks + chunk, packed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // the arrival below must not overtake this store (another memory channel): wait for its acknowledgement
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
-    __syncthreads();                                         // waits for the store
+    __syncthreads();
     if (tid == 0)
         last_flag = __hip_atomic_fetch_add(arrived, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == B * kGreedyChunks - 1;
     __syncthreads();

@@ -35,6 +35,7 @@ __global__ __launch_bounds__(256) void terna_rope_kv_store_kernel(
     const int slots = H + 2 * KV;
     const uint16_t* src = qkv + static_cast<size_t>(row) * slots * D;
     const long long slot = pos[t];
+    const bool slot_ok = slot >= 0 && slot < S;  // a position outside the cache writes no k / v row (q is still rotated)
     if ((half & 7) == 0) {
         // 8 pairs per thread: 16-byte loads and stores, for the 2B model one pass of 240 threads
         const int per = half >> 3;
@@ -75,6 +76,7 @@ __global__ __launch_bounds__(256) void terna_rope_kv_store_kernel(
             if (hs < H) dst = q_out + ((static_cast<size_t>(b) * H + hs) * T + t) * D;
             else if (hs < H + KV) dst = cache_k + ((static_cast<size_t>(b) * KV + (hs - H)) * S + slot) * D;
             else dst = cache_v + ((static_cast<size_t>(b) * KV + (hs - H - KV)) * S + slot) * D;
+            if (hs >= H && !slot_ok) continue;
             *reinterpret_cast<u32x4*>(dst + off1) = pack_bf16x8(o1);
             *reinterpret_cast<u32x4*>(dst + off2) = pack_bf16x8(o2);
         }
@@ -96,6 +98,7 @@ __global__ __launch_bounds__(256) void terna_rope_kv_store_kernel(
         if (hs < H) dst = q_out + ((static_cast<size_t>(b) * H + hs) * T + t) * D;
         else if (hs < H + KV) dst = cache_k + ((static_cast<size_t>(b) * KV + (hs - H)) * S + slot) * D;
         else dst = cache_v + ((static_cast<size_t>(b) * KV + (hs - H - KV)) * S + slot) * D;
+        if (hs >= H && !slot_ok) continue;
         dst[ia] = float_to_bf16_bits(o1);
         dst[ib] = float_to_bf16_bits(o2);
     }
@@ -240,7 +243,6 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     auto cache_slot = [&](int l) { return (((l >> 4) * SP + sp) << 4) + (l & 15); };
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    TERNA_TS(0);
     // Workgroup -> (sequence, head).  Workgroups go to the 8 XCDs round robin, and the H / KV heads of a kv group read
     // the same keys and values: with groups > 0 (= B * KV) the heads of group G all sit on XCD G mod 8, so that the
     // group's cache prefix crosses the fabric once and its other heads hit in that L2 (the grid is padded to whole
@@ -258,7 +260,12 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     }
     const int bh = b * H + h;
     const int kvh = h / (H / KV);
-    const int n = static_cast<int>(pos[0]) + 1;
+    // Prefix length: slots 0 .. pos[0].  pos comes from device memory the host cannot check, so it is clamped to the
+    // cache -- the LDS score buffer and every cache address are sized by S -- and a position outside [0, S) writes no
+    // cache row below (the attention then runs over the clamped prefix; its result is not meaningful, but in bounds).
+    const long long p0 = pos[0];
+    const bool pos_ok = p0 >= 0 && p0 < S;
+    const int n = p0 < 0 ? 1 : (p0 >= S ? S : static_cast<int>(p0) + 1);
     const uint16_t* kbase = cache_k + (static_cast<size_t>(b) * KV + kvh) * S * D;
     const uint16_t* vbase = cache_v + (static_cast<size_t>(b) * KV + kvh) * S * D;
 
@@ -357,7 +364,7 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
             qb = rotate(q_own, q_par);
             knew = rotate(k_own, k_par);
         }
-        if (h % (H / KV) == 0 && sp == 0) {      // this kv group's writer: slot pos[0] of both caches
+        if (h % (H / KV) == 0 && sp == 0 && pos_ok) {      // this kv group's writer: slot pos[0] of both caches
             const size_t slot_off = ((static_cast<size_t>(b) * KV + kvh) * S + (n - 1)) * D;
             if (wave == 0 && r16 < R) *reinterpret_cast<u32x4*>(cache_k + slot_off + 8 * c) = knew;   // r16 < R: every chunk once
             if (tid < CH) *reinterpret_cast<u32x4*>(cache_v + slot_off + 8 * chunk) = vnew;
@@ -365,7 +372,6 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     }
     if (r16 >= R) qb = zero4;                    // B operand: q's pieces in columns 0 .. R-1 only
 
-    TERNA_TS(1);
     float mx = -INFINITY;
     auto score_tile = [&](int ltile, const u32x4 (&kin)[NJ]) {       // ltile: local tile of this split
         const int tile = ltile * SP + sp;
@@ -416,7 +422,6 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
         load_keys(tile, k);
         score_tile(tile, k);
     }
-    TERNA_TS(2);
     mx = wave_max(mx);
     if (lane == 0) red[wave] = mx;
     __syncthreads();
@@ -431,7 +436,6 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
         score[l] = p;
         sum += p;
     }
-    TERNA_TS(3);
     sum = wave_sum(sum);
     if (lane == 0) red[NW + wave] = sum;
     __syncthreads();
@@ -440,7 +444,6 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     for (int w = 1; w < NW; ++w) sum += red[NW + w];
 
     // ---- pass 3: weighted sum of the value rows, VU rows per round (the first round is already here)
-    TERNA_TS(4);
     float acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
     for (int l0 = slice; l0 < nl; l0 += VU * SLICES) {
         if (l0 != slice) {                       // all VU rows of the round requested before any is used
@@ -467,7 +470,6 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
             for (int e = 0; e < 8; ++e) acc[e] = fmaf(p, vf[e], acc[e]);
         }
     }
-    TERNA_TS(5);
 #pragma unroll
     for (int e = 0; e < 8; ++e) part[slice * D + chunk * 8 + e] = acc[e];
     __syncthreads();
@@ -484,7 +486,6 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
 #pragma unroll
         for (int grp = 0; grp < GROUPS; ++grp) o += part2[grp * D + tid];
     }
-    TERNA_TS(6);
     uint16_t* orow = out + (static_cast<size_t>(b) * H + h) * D;
     if (!SPLIT || SP == 1) {
         if (tid < D) orow[tid] = float_to_bf16_bits(o / sum);
@@ -494,9 +495,11 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     // ---- split: publish (o, mx, sum), count the arrival; the last workgroup of the head merges.
     // The partials and the counter are written and read with device-scope relaxed atomics: those go
     // past the per-XCD L2 to the memory all XCDs share, so no cache write-back or invalidate (what a
-    // device-scope fence would cost every workgroup) is needed.  Order: every thread's partial stores
-    // have completed at the barrier, the arrival is counted after it, and the merging workgroup
-    // reads after it has seen the full count.
+    // device-scope fence would cost every workgroup) is needed.  Order, made explicit: every storing
+    // wave waits until the memory system has acknowledged its own partial stores (vmcnt(0): the
+    // workgroup barrier alone orders instructions, not their completion, and the counter lives in
+    // another memory channel than the partials), then the barrier, then ONE thread counts the arrival;
+    // the merging workgroup issues its loads only after it has seen the full count.
     float* mine = partial + (static_cast<size_t>(bh) * SP + sp) * (D + 2);
     auto publish = [](float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
     auto fetch = [](const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
@@ -505,7 +508,8 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
         publish(mine + D, mx);
         publish(mine + D + 1, sum);
     }
-    __syncthreads();                             // waits for this workgroup's stores
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // this wave's partial stores have reached device memory
+    __syncthreads();                             // ... and so have those of every other wave of the workgroup
     if (tid == 0)
         last_flag = __hip_atomic_fetch_add(arrived + bh, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == SP - 1;
     __syncthreads();

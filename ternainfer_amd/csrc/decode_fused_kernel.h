@@ -85,7 +85,6 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    TERNA_TS(0);
     const int band0 = blockIdx.x * NB;               // first of this workgroup's NB bands
     const int ktiles = K >> 6;
     const int i = lane & 15, g = lane >> 4;          // operand coordinates: weight row / batch row i, 16-column group g
@@ -136,7 +135,6 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
     if constexpr (MP != 1)
         for (int o = lane * 16; o < 16 * XQ::kPitch; o += 64 * 16) *reinterpret_cast<u32x4*>(slab + o) = u32x4{0u, 0u, 0u, 0u};
 
-    TERNA_TS(1);
     float ssq = 0.0f;
 #pragma unroll
     for (int t = 0; t < TMAX; ++t) {
@@ -180,10 +178,8 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
         }
         return r;
     };
-    TERNA_TS(2);
     ssq = row_reduce(ssq, 0, false);
     const float rstd = rsqrtf(ssq / static_cast<float>(K) + eps);
-    TERNA_TS(3);
 
     // ---- phase C: y in place of h, max |y| per row
     float amax = 0.0f;
@@ -200,9 +196,7 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
         }
         xr[t].pack(f);
     }
-    TERNA_TS(4);
     amax = row_reduce(amax, 1, true);
-    TERNA_TS(5);
     const uint16_t s_bits = float_to_bf16_bits(__fdiv_rn(127.0f, fmaxf(amax, 1e-5f)));
     const float s = bf16_bits_to_float(s_bits);
     if (wave == 0 && (lane % LPR) == 0) {
@@ -268,11 +262,9 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
     }
 
     // ---- phase E: cross-wave sum in wave order + the decode epilogue (lane: batch row i, output rows 4g .. 4g+3)
-    TERNA_TS(6);
 #pragma unroll
     for (int b = 0; b < NB; ++b) red[wave][b][lane] = acc[b];
     __syncthreads();
-    TERNA_TS(7);
     if (wave < NB) {
         i32x4 sum = red[0][wave][lane];
 #pragma unroll
@@ -288,7 +280,6 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
             *reinterpret_cast<u32x2*>(out + static_cast<size_t>(i) * N + n0) = pk;
         }
     }
-    TERNA_TS(8);
 }
 
 }  // namespace terna

@@ -200,7 +200,6 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    TERNA_TS(0);
     Lut* lut = lut_all[wave];
 
     const int band = blockIdx.x;            // 16-row band of W
@@ -330,7 +329,6 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
                 fetch_signs(__builtin_amdgcn_readlane(vbase, j + DEPTH), pre);
             }
             process(cur);
-            TERNA_TS(3 + (j < 5 ? j : 5));
         }
     };
     // Start of a round: offset-free loads go out first so they overlap the offset fetch.
@@ -347,7 +345,6 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
     // Offsets come 64 band-tiles at a time (one per lane); K <= 4096 * WAVES needs one round.
     ccnt = cnt < 64 ? cnt : 64;
     prime();
-    TERNA_TS(1);
     // Wave w finishes m-block w (and w + WAVES, ...): with the data loads in flight, fetch that block's scale
     // factors, so that no global load sits between the last MFMA and the store.
     EpilogueRaw eraw[(MB + WAVES - 1) / WAVES];
@@ -358,7 +355,6 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e) lut[lane + 64 * e] = T::make_lut(lane + 64 * e);
-    TERNA_TS(2);
     while (ccnt > 0) {
         for (int j0 = 0; j0 < ccnt; j0 += NBUF) {
             if constexpr (DEPTH == 2) {
@@ -379,9 +375,7 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
     // 16x16 MFMA: lane L holds output rows 4*(L>>4) .. +3 of column L & 15.
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) red[wave][mb][lane] = acc[mb];
-    TERNA_TS(9);
     __syncthreads();
-    TERNA_TS(10);
 #pragma unroll
     for (int e = 0; e < (MB + WAVES - 1) / WAVES; ++e) {
         const int mb = wave + e * WAVES;
@@ -399,7 +393,6 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
             *reinterpret_cast<u32x2*>(out + static_cast<size_t>(m) * N + n0) = packed;
         }
     }
-    TERNA_TS(11);
 }
 
 }  // namespace terna

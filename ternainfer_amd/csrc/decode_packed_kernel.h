@@ -42,7 +42,6 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    TERNA_TS(0);
     const int band0 = blockIdx.x * NB;
     const int m_base = blockIdx.y * (16 * MB);
     const int ktiles = K >> 6;
@@ -67,10 +66,6 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
         }
 
     const int cnt = ktiles > wave ? (ktiles - wave + WAVES - 1) / WAVES : 0;   // this wave's band-tiles
-#ifdef TERNA_TS_ENABLED
-    if (reinterpret_cast<uintptr_t>(wp) == 1 || cnt < -1) return;   // force the kernarg wait before the stamp
-    TERNA_TS(2);
-#endif
     auto fetch = [&](int j, Raw& raw) {
 #pragma unroll
         for (int b = 0; b < NB; ++b) raw.word[b] = wp[b * band_pitch + static_cast<size_t>(j) * (WAVES * 64)];
@@ -137,13 +132,11 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
         if (j < cnt) {
             if (j + DEPTH < cnt) fetch(j + DEPTH, pre);
             process(cur);
-            TERNA_TS(3 + (j < 5 ? j : 5));
         }
     };
     if (0 < cnt) fetch(0, ring0);
     if (DEPTH >= 2 && 1 < cnt) fetch(1, ring1);
     if (DEPTH >= 3 && 2 < cnt) fetch(2, ring2);
-    TERNA_TS(1);
 
     // Wave w finishes unit w (and w + WAVES, ...), unit = band * MB + m-block: with the data loads in
     // flight, fetch that unit's scale factors so that no global load sits between the last MFMA and the store.
@@ -178,9 +171,7 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
     for (int b = 0; b < NB; ++b)
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) red[wave][b * MB + mb][lane] = acc[b][mb];
-    TERNA_TS(9);
     __syncthreads();
-    TERNA_TS(10);
 #pragma unroll
     for (int e = 0; e < FIN; ++e) {
         const int unit = wave + e * WAVES;
@@ -202,7 +193,6 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
             *reinterpret_cast<u32x2*>(out + static_cast<size_t>(m) * N + n0) = pk;
         }
     }
-    TERNA_TS(11);
 }
 
 }  // namespace terna

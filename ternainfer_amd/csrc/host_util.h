@@ -1,0 +1,63 @@
+// Host-side helpers shared by the translation units of libternaspmm.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <mutex>
+#include <unordered_map>
+
+namespace terna {
+
+[[noreturn]] inline void die(const char* what, hipError_t e, int line)
+{
+    std::printf("Last Cuda Error Detected at line: %d, Error: %s (%s).\n", line, hipGetErrorString(e), what);
+    std::fflush(stdout);
+    std::exit(EXIT_FAILURE);
+}
+
+inline bool shape_ok(int M, int N, int K)
+{
+    if (M < 1 || N < 64 || K < 64 || (N % 64) || (K % 64)) {
+        std::printf("TernaSpMM Error: unsupported shape M=%d N=%d K=%d (need M >= 1, N %% 64 == 0, K %% 64 == 0)\n",
+                    M, N, K);
+        std::fflush(stdout);
+        return false;
+    }
+    return true;
+}
+
+// weight_scale has four slots (convert/convert_TernaInfer.py:176-194): one to four scale groups per matrix
+inline bool groups_ok(int ws_num)
+{
+    if (ws_num < 1 || ws_num > 4) {
+        std::printf("TernaSpMM Error: unsupported ws_num=%d (need 1 .. 4)\n", ws_num);
+        std::fflush(stdout);
+        return false;
+    }
+    return true;
+}
+
+// Dynamic-LDS opt-in of one kernel, once per (kernel, device) of the process: the attribute is per device.
+inline void allow_dynamic_lds_ptr(const void* kernel, int bytes, const char* what, int line)
+{
+    static std::mutex mutex;
+    static std::unordered_map<const void*, uint64_t> done;       // kernel -> bit per device ordinal
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
+    std::lock_guard<std::mutex> lock(mutex);
+    uint64_t& mask = done[kernel];
+    if (dev >= 0 && ((mask >> dev) & 1u)) return;
+    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) die(what, e, line);
+    if (dev >= 0) mask |= uint64_t{1} << dev;
+}
+template <typename Kernel>
+void allow_dynamic_lds(Kernel kernel, int bytes, const char* what, int line)
+{
+    allow_dynamic_lds_ptr(reinterpret_cast<const void*>(kernel), bytes, what, line);
+}
+
+}  // namespace terna

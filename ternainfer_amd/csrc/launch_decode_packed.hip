@@ -1,0 +1,56 @@
+// Launchers of the small-M kernel on the P2 layout and of the load-time repack (decode_packed_kernel.h,
+// packed_common.h).
+#include "launchers.h"
+#include "host_util.h"
+#include "decode_packed_kernel.h"
+
+namespace terna {
+
+// ---- P2 layout (load-time repack): see packed_common.h -------------------------------------------
+void launch_repack(const Weights& w, uint32_t* packed, int N, int K, hipStream_t st)
+{
+    terna_repack_kernel<4><<<dim3(N / 16), dim3(256), 0, st>>>(w.bitmap, w.tile_off, w.median_off, w.sign_words,
+                                                              packed, N, K);
+}
+
+template <typename Act, int WAVES, int MB, int DEPTH, int NB = 1>
+void launch_decode_packed_as(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N,
+                             int K, hipStream_t st)
+{
+    const dim3 grid(N / 16 / NB, (M + 16 * MB - 1) / (16 * MB));
+    terna_decode_packed_kernel<Act, WAVES, MB, DEPTH, NB><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, ep, M, N, K);
+}
+
+template <typename Act>
+void launch_decode_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                          hipStream_t st)
+{
+    const int forced = decode_waves_override();
+    const bool wide = forced ? forced == 16 : (N / 16 <= 256);
+    if (M <= 16) {
+        // more than 512 bands (gate+up): per-wave set-up is as expensive as a few band-tiles, so fewer waves
+        // with more band-tiles each win (measured 7.4 against 8.2 us)
+        const bool narrow = forced ? forced == 4 : (N / 16 > 512);
+        // ... and every workgroup stages the same activations: two bands per workgroup share one staging (N is a
+        // multiple of 64, so the band count is even).  Measured on gate+up, cold: 6.4 us against 7.3 us; four
+        // bands 6.7 us.  TERNASPMM_DECODE_BANDS=1 switches that off (tuning aid).
+        static const bool multi_off = [] {
+            const char* v = std::getenv("TERNASPMM_DECODE_BANDS");
+            return v && std::atoi(v) == 1;
+        }();
+        if (narrow && !forced && !multi_off) launch_decode_packed_as<Act, 8, 1, 2, 2>(x, packed, out, ep, M, N, K, st);
+        else if (narrow) launch_decode_packed_as<Act, 4, 1, 3>(x, packed, out, ep, M, N, K, st);
+        else if (wide) launch_decode_packed_as<Act, 16, 1, 3>(x, packed, out, ep, M, N, K, st);
+        else launch_decode_packed_as<Act, 8, 1, 2>(x, packed, out, ep, M, N, K, st);
+    } else if (M <= 32) {
+        if (wide) launch_decode_packed_as<Act, 16, 2, 2>(x, packed, out, ep, M, N, K, st);
+        else launch_decode_packed_as<Act, 8, 2, 2>(x, packed, out, ep, M, N, K, st);
+    } else {
+        launch_decode_packed_as<Act, 8, 4, 1>(x, packed, out, ep, M, N, K, st);
+    }
+}
+
+template void launch_decode_packed<int8_t>(const int8_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
+template void launch_decode_packed<uint16_t>(const uint16_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
+
+}  // namespace terna

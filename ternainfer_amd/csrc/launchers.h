@@ -1,0 +1,54 @@
+// Host-side launchers of the TernaSpMM kernels.  Each kernel family is instantiated in a translation unit
+// of its own (launch_*.hip), so that the library builds in parallel; the C ABI (ternaspmm.hip) only sees
+// these declarations.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "terna_common.h"
+
+namespace terna {
+
+// The four tensors of the reference format.
+struct Weights {
+    const uint64_t* bitmap;
+    const int* tile_off;
+    const uint16_t* median_off;
+    const uint32_t* sign_words;
+};
+
+
+// ---- reference format (launch_reference.hip) -------------------------------------------------------
+// Small-M kernel on the reference format; Act = int8_t | uint16_t (bf16 storage).
+template <typename Act>
+void launch_decode(const Act* x, const Weights& w, uint16_t* out, const Epilogue& ep, int M, int N, int K, hipStream_t st);
+// MFMA-tiled kernel that decodes the reference format on the fly (no workspace needed).
+template <typename Act>
+void launch_prefill(const Act* x, const Weights& w, uint16_t* out, const Epilogue& ep, int M, int N, int K, hipStream_t st);
+// Reference format -> dense bf16 [N][K].
+void launch_decompress(const Weights& w, uint16_t* dense, int N, int K, hipStream_t st);
+
+// ---- P2 layout (launch_decode_packed.hip, launch_prefill_packed_*.hip) ---------------------------------
+void launch_repack(const Weights& w, uint32_t* packed, int N, int K, hipStream_t st);
+template <typename Act>
+void launch_decode_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                          hipStream_t st);
+template <typename Act>
+void launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                           hipStream_t st);
+
+extern template void launch_decode<int8_t>(const int8_t*, const Weights&, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
+extern template void launch_decode<uint16_t>(const uint16_t*, const Weights&, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
+extern template void launch_prefill<int8_t>(const int8_t*, const Weights&, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
+extern template void launch_prefill<uint16_t>(const uint16_t*, const Weights&, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
+extern template void launch_decode_packed<int8_t>(const int8_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
+extern template void launch_decode_packed<uint16_t>(const uint16_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
+extern template void launch_prefill_packed<int8_t>(const int8_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
+extern template void launch_prefill_packed<uint16_t>(const uint16_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
+
+// Tuning override shared by the two small-M launchers: TERNASPMM_DECODE_WAVES=4|8|16 forces one variant.
+int decode_waves_override();
+
+}  // namespace terna

@@ -6,11 +6,6 @@
 
 #include <type_traits>
 
-// Phase timestamps for tuning builds; expands to nothing in the shipped library.
-#ifndef TERNA_TS
-#define TERNA_TS(slot)
-#endif
-
 namespace terna {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;

@@ -263,6 +263,18 @@ def greedy_step(logits: torch.Tensor, tok: torch.Tensor, history: Optional[torch
     return tok
 
 
+def quant_input(input: torch.Tensor):
+    """Per-row int8 quantisation of the activations (model.py:120-123): s = 127 / max(max|x|, 1e-5),
+    x_q = clamp(round(x * s), -128, 127).  One definition for the whole library, the one the norm kernels
+    compute: fp32 arithmetic, s rounded to bf16, and that rounded s both multiplies here and divides in the
+    epilogue.  (The reference's eager mode would multiply in the tensor's dtype, its compiled graph in fp32
+    with the unrounded quotient; the two differ from each other and from this by at most one step.)
+    Returns (x_q int8, s bf16 [..., 1])."""
+    x = input.float()
+    s = (127.0 / x.abs().amax(dim=-1, keepdim=True).clamp_(min=1e-5)).to(torch.bfloat16)
+    return (x * s.float()).round().clamp(-128, 127).to(torch.int8), s
+
+
 class _CompressedWeight(nn.Module):
     """Holds the four format tensors + ``weight_scale`` under the reference's checkpoint keys
     (convert_TernaInfer.py:204-209, model.py:110-116)."""
@@ -297,13 +309,12 @@ class SpBitLinear(_CompressedWeight):
                 requires_grad=False)
 
     def quant_input(self, input):
-        s = 127 / input.abs().max(dim=-1, keepdim=True).values.clamp_(min=1e-5)
-        return (input * s).round().clamp(-128, 127).to(torch.int8), s
+        return quant_input(input)
 
     def forward(self, input):
         input, s = self.quant_input(input)
         if self.weight_packed is not None:
-            return TernaInfer_linear_packed(input, self.weight_packed, s.to(torch.bfloat16), self.weight_scale,
+            return TernaInfer_linear_packed(input, self.weight_packed, s, self.weight_scale,
                                             self.ws_num, self.out_features)
         return TernaInfer_linear(
             input, self.weight_compressed_val, self.weight_TileOffsets_global, self.weight_TileOffsets_median,
@@ -333,8 +344,7 @@ class BF16BitLinear(nn.Module):
         self.weight = torch.nn.Parameter(dic[key + ".weight"].cuda(), requires_grad=False)
 
     def quant_input(self, input):
-        s = 127 / input.abs().max(dim=-1, keepdim=True).values.clamp_(min=1e-5)
-        return (input * s).round().clamp(-128, 127).to(torch.int8), s
+        return quant_input(input)
 
     def forward(self, input):
         input, s = self.quant_input(input)

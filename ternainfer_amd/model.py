@@ -21,8 +21,8 @@ import torch
 from torch.nn import functional as F
 
 from . import _lib
-from .linear import (argmax_rows, greedy_step, greedy_step_state, lm_head, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant, repack_weight, rmsnorm_linear_packed,
-                     rmsnorm_quant)
+from .linear import (argmax_rows, greedy_step, greedy_step_state, lm_head, quant_input, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant,
+                     repack_weight, rmsnorm_linear_packed, rmsnorm_quant)
 
 
 @dataclass
@@ -91,10 +91,8 @@ class TernaryLinear:
         return out
 
     def __call__(self, x: torch.Tensor) -> torch.Tensor:
-        if self.act == "int8":                # model.py:120-133, fp32 inside, the bf16-rounded s used throughout
-            xf = x.float()
-            s = (127 / xf.abs().amax(dim=-1, keepdim=True).clamp_(min=1e-5)).to(torch.bfloat16)
-            xq = (xf * s.float()).round().clamp(-128, 127).to(torch.int8)
+        if self.act == "int8":                # model.py:120-133
+            xq, s = quant_input(x)
             return self.quantised(xq, s.reshape(-1).contiguous())
         return self.dense(x)
 
@@ -334,9 +332,10 @@ class Transformer:
         return [(torch.zeros(shape, dtype=torch.bfloat16, device=dev), torch.zeros(shape, dtype=torch.bfloat16, device=dev))
                 for _ in range(a.n_layers)]
 
-    def forward(self, tokens: torch.Tensor, cache, pos_idx: torch.Tensor) -> torch.Tensor:
+    def forward(self, tokens: torch.Tensor, cache, pos_idx: torch.Tensor, trace=None) -> torch.Tensor:
         """tokens int64 [B, T]; pos_idx int64 [T] = cache slots of the new tokens.  Returns logits [B, vocab]
-        of the last new token."""
+        of the last new token.  `trace`, if given, is called after every block as
+        trace(index, stream_in, pending_in, stream_out, pending_out) (layer-by-layer checks against a golden)."""
         a = self.args
         bsz, t = tokens.shape
         max_seq = cache[0][0].shape[2]
@@ -351,8 +350,11 @@ class Transformer:
         x = self.tok_embeddings[tokens.reshape(-1)]
         pending = None
         attn_ws = self.attention_workspace(bsz) if one_launch_attention else None     # layers run one after another: shared
-        for layer, (ck, cv) in zip(self.layers, cache):
+        for index, (layer, (ck, cv)) in enumerate(zip(self.layers, cache)):
+            x_in, pending_in = x, pending
             x, pending = layer.forward(x, pending, ck, cv, pos_idx, cos, sin, mask, attn_ws)
+            if trace is not None:
+                trace(index, x_in, pending_in, x, pending)
         if t > 1:                                                             # only the last new token feeds the head
             x, pending = x.view(bsz, t, a.dim)[:, -1].contiguous(), pending.view(bsz, t, a.dim)[:, -1].contiguous()
         if self.layers[0].fused and x.is_cuda:                                # last residual add + final norm: one launch

@@ -383,11 +383,48 @@ def test_bf16_prefill_2b_layer_shapes(lib, m, n, k):
     x = make_bf16_activations(m, k, seed_for(3, 30 + m % 97), outlier_frac=0.01)
     scale = np.array([1.37], np.float32)
     got = run_bf16(lib, fmt, x, scale, 1)
-    cols = np.sort(np.random.default_rng(seed_for(3, 99)).permutation(n)[:192])
+    cols = np.sort(np.random.default_rng(seed_for(3, 99) + n + 7 * k + m).permutation(n)[:192])
     ref = O.bf16_bits_to_f32(x).astype(np.float64) @ w[cols].astype(np.float64).T * float(scale[0])
     _check_bf16(got[:, cols], ref)
     neg = run_bf16(lib, fmt, x ^ np.uint16(0x8000), scale, 1)
     _assert_negation_symmetric(got, neg)
+
+
+@pytest.mark.parametrize("n,k,ws_num", [(3840, 2560, 3), (2560, 2560, 1), (13824, 2560, 2), (2560, 6912, 1)])
+@pytest.mark.parametrize("m", [256, 512, 2048])
+def test_int8_reference_entry_points_2b_layer_shapes_large_m(lib, m, n, k, ws_num):
+    """The symbols an unmodified model.py calls (kernels/TernaSpMM.cu:25, :110), on reference-format pointers, at
+    the prefill sizes of the four 2B matrices with their weight-scale group counts: with the call site's workspace
+    (transcode + P2 kernel), without one (fused reference-format kernel), and the forced _prefill entry.  Bit-exact
+    against the integer oracle on a seeded sample of 256 columns that straddles every group boundary; the three
+    routes must also agree with each other on the WHOLE output."""
+    w = make_ternary(n, k, 0.40, seed_for(3, 40 + n % 7))
+    fmt = DeviceFormat(w)
+    xq, s = make_int8_activations(m, k, seed_for(3, 50 + m % 97))
+    s = s.copy()
+    s[m // 3] = 0                                                          # the visitor's s == 0 -> coefficient 0 rule
+    rng = np.random.default_rng(seed_for(3, 60 + n % 7 + m % 5))
+    edges = [c for b in (2560, 3200, n // 2, n - 1, 0) for c in (b - 1, b, b + 127, b + 128) if 0 <= c < n]
+    cols = np.unique(np.concatenate([rng.permutation(n)[:256], np.array(edges)]))
+    want = O.spmm_i8(xq, w, s, WS, ws_num, 1, cols=cols)
+    a = run_i8(lib, fmt, xq, s, WS, ws_num)                                # M > 64: prefill rule, transcode route
+    assert (a[:, cols] == want).all()
+    b = run_i8(lib, fmt, xq, s, WS, ws_num, workspace=False)               # fused reference-format kernel
+    assert (b == a).all()
+    c = run_i8(lib, fmt, xq, s, WS, ws_num, "bitlinear_TernaSpMM_prefill")
+    assert (c == a).all()
+
+
+@pytest.mark.parametrize("n,k", [(3840, 2560), (2560, 2560), (13824, 2560), (2560, 6912)])
+def test_packed_bf16_2b_layer_shapes_m512(lib, n, k):
+    w = make_ternary(n, k, 0.40, seed_for(3, 70 + n % 7))
+    packed = repack(lib, DeviceFormat(w))
+    x = make_bf16_activations(512, k, seed_for(3, 71 + n % 7), outlier_frac=0.01)
+    scale = np.array([0.83], np.float32)
+    got = run_bf16_packed(lib, packed, n, x, scale, 1)
+    cols = np.sort(np.random.default_rng(seed_for(3, 72 + n % 7)).permutation(n)[:192])
+    ref = O.bf16_bits_to_f32(x).astype(np.float64) @ w[cols].astype(np.float64).T * float(scale[0])
+    _check_bf16(got[:, cols], ref)
 
 
 # ------------------------------------------------------------------------------- P2 layout (load-time repack)

@@ -6,6 +6,8 @@
                 epilogue: C (volatile float, one operation at a time) == numpy float32, and the
                 two rounding orders are shown to differ on some element (so a swapped formula fails)
   bf16 family - C fp64 loop == numpy fp64 matmul; linear in the scale; sign flip of W flips the output
+  quantisers  - quant_input and quant_weight_int8 against answers worked by hand (ties to even, exact and
+                inexact scales, the clamps), on both restatements and on the converter's own function
 """
 import ctypes
 
@@ -101,6 +103,101 @@ def test_quant_input_c_equals_numpy(coracle):
     q2, s2 = O.quant_input(x)
     assert (q1 == q2).all() and (s1 == s2).all()
     assert np.abs(q1).max() <= 127 and (np.abs(q1).max(axis=1) >= 126).all()
+
+
+def _row(values, width=16):
+    """One activation row: the given bf16-exact values, zero-padded."""
+    r = np.zeros(width, np.float32)
+    r[:len(values)] = values
+    bits = O.f32_to_bf16_bits(r)
+    assert (O.bf16_bits_to_f32(bits) == r).all(), "test vector must be exact in bf16"
+    return bits
+
+
+# Known answers of quant_input (model.py:120-123) worked by hand.  The definition this build fixes:
+# s = bf16(127 / max(max|x|, 1e-5)); q = clamp(round_half_even(fp32(x * s)), -128, 127), with the
+# ROUNDED s used in the product.  Each row is chosen so that one plausible mistake fails it.
+QUANT_INPUT_KAT = [
+    # max|x| = 127 -> s = 1 exactly, q = round_half_even(x): floor(x + 0.5) or round-half-away fails
+    ([127.0, 0.5, 1.5, 2.5, -2.5, -0.5, 100.5, 101.5, -126.5, 3.5, -1.5],
+     1.0, [127, 0, 2, 2, -2, 0, 100, 102, -126, 4, -2]),
+    # max|x| = 1 -> s = 127 (exact in bf16); 0.5 * 127 = 63.5 is a tie -> 64 (even), -63.5 -> -64
+    ([1.0, -1.0, 0.5, -0.5, 0.25, 0.0078125, 0.00390625],
+     127.0, [127, -127, 64, -64, 32, 1, 0]),                    # 31.75 -> 32, 0.992 -> 1, 0.496 -> 0
+    # max|x| = 0.5 -> s = 254 (exact); max|x| = 4 -> s = 31.75 (exact): a missing or inverted scale fails
+    ([0.5, -0.25, 0.125], 254.0, [127, -64, 32]),               # -63.5 -> -64, 31.75 -> 32
+    ([4.0, 2.0, -1.0, 0.0625], 31.75, [127, 64, -32, 2]),       # 63.5 -> 64, -31.75 -> -32, 1.984 -> 2
+    # max|x| = 129/128: 127 / 1.0078125 = 126.0155 rounds DOWN to s = 126 in bf16.  With the rounded s
+    # 0.75 * 126 = 94.5 is a tie -> 94 and (129/256) * 126 = 63.49 -> 63; the unrounded s would give
+    # 94.51 -> 95 and 63.5 -> 64: a quantiser that multiplies by the fp32 quotient fails here
+    ([1.0078125, 0.75, 0.50390625, -0.75], 126.0, [127, 94, 63, -94]),
+    # max|x| = 255/128: 127 / 1.9921875 = 63.749 rounds UP to s = 63.75; max|x| * s = 127.002 -> 127:
+    # the rounding of s can overshoot 127 by at most 127 * 2^-8 < 0.5, so the clamp never bites
+    ([1.9921875, -1.9921875, 1.0], 63.75, [127, -127, 64]),
+]
+
+
+@pytest.mark.parametrize("values,s_want,q_want", QUANT_INPUT_KAT)
+def test_quant_input_known_answers(coracle, values, s_want, q_want):
+    x = _row(values).reshape(1, -1)
+    for impl in (O.quant_input, coracle.quant_input):
+        q, s = impl(x)
+        assert O.bf16_bits_to_f32(s).tolist() == [s_want]
+        assert q[0, :len(q_want)].tolist() == q_want and not q[0, len(q_want):].any()
+
+
+def test_quant_input_all_zero_row(coracle):
+    """max|x| = 0 is clamped to 1e-5: s = bf16(127 / 1e-5f) = bf16(12 700 000.3) = 1.515625 * 2^23
+    (bits 0x4B42), q = 0."""
+    x = np.zeros((1, 32), np.uint16)
+    for impl in (O.quant_input, coracle.quant_input):
+        q, s = impl(x)
+        assert s.tolist() == [0x4B42] and O.bf16_bits_to_f32(s).tolist() == [1.515625 * 2.0 ** 23]
+        assert not q.any()
+
+
+def test_quant_input_rows_are_independent(coracle):
+    """The scale is per row (dim=-1, keepdim): stacking KAT rows must not change any of them."""
+    width = 16
+    x = np.stack([_row(v, width) for v, _, _ in QUANT_INPUT_KAT])
+    for impl in (O.quant_input, coracle.quant_input):
+        q, s = impl(x)
+        assert O.bf16_bits_to_f32(s).tolist() == [sw for _, sw, _ in QUANT_INPUT_KAT]
+        for r, (_, _, qw) in enumerate(QUANT_INPUT_KAT):
+            assert q[r, :len(qw)].tolist() == qw
+
+
+# Known answers of quant_weight_int8 (convert_TernaInfer.py:159-163): s = 1 / max(mean|W|, 1e-5),
+# W_t = clamp(round_half_even(W * s), -1, 1), scale = 1 / s.
+QUANT_WEIGHT_KAT = [
+    # mean|W| = 1 -> s = 1: ties 0.5 -> 0, 1.5 -> 2 -> clamp 1, 2.5 -> 2 -> 1; floor(x + 0.5) turns 0.5 into 1
+    ([0.5, -0.5, 1.5, -1.5, 0.25, 2.5, 0.75, 0.5], 1.0, [0, 0, 1, -1, 0, 1, 1, 0]),
+    # mean|W| = 0.5 -> s = 2: 0.25 * 2 = 0.5 -> 0, 0.75 * 2 = 1.5 -> 2 -> 1; a max- or rms-based scale fails
+    ([0.25, 0.75, -0.25, -0.75], 0.5, [0, 1, 0, -1]),
+    # mean|W| = 2 -> s = 0.5: 1.0 * 0.5 = 0.5 -> 0, 3 * 0.5 = 1.5 -> 2 -> 1, -3 -> -1, 1.0078125 * 0.5 > 0.5 -> 1
+    ([1.0, 3.0, -3.0, 1.0078125, 2.9921875, -1.0], 2.0, [0, 1, -1, 1, 1, 0]),
+]
+
+
+@pytest.mark.parametrize("values,scale_want,t_want", QUANT_WEIGHT_KAT)
+def test_quant_weight_int8_known_answers(values, scale_want, t_want):
+    import torch
+    import ternainfer_amd as T
+    w = np.array(values, np.float32).reshape(2, -1)
+    assert np.abs(w).mean() == scale_want                       # the vector is built for an exact mean
+    t, scale = O.quant_weight_int8(w)
+    assert t.dtype == np.int8 and t.reshape(-1).tolist() == t_want and float(scale) == scale_want
+    # the converter's own function (the reference's four lines on torch tensors) on the same vector, in fp32
+    # and in bf16 (every value, product and the mean are exact in bf16 here)
+    for dtype in (torch.float32, torch.bfloat16):
+        tt, ss = T.quant_weight_int8(torch.from_numpy(w).to(dtype))
+        assert tt.dtype == torch.int8 and tt.reshape(-1).tolist() == t_want
+        assert ss.dtype == torch.bfloat16 and ss.shape == (1,) and float(ss) == scale_want
+
+
+def test_quant_weight_int8_all_zero():
+    t, scale = O.quant_weight_int8(np.zeros((4, 4), np.float32))
+    assert not t.any() and abs(float(scale) - 1e-5) <= 1e-11   # the clamp of the mean
 
 
 # ------------------------------------------------------------------ glue between two linears
