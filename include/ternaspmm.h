@@ -216,6 +216,18 @@ void ternaspmm_rope_kv_store(const terna_bf16* qkv, const float* cos, const floa
 void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
                                 const long long* pos, terna_bf16* out, int B, int H, int KV, int D, int S,
                                 float scale, void* workspace, terna_stream stream);
+/* ternaspmm_decode_attention for callers that cannot allocate or bring a workspace (code under HIP graph capture
+ * that owns no buffers, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Same arguments, kernels and results as ternaspmm_decode_attention with a workspace, but the split-attention
+ * scratch (arrival counters + partial results) is a static device array inside the library: about 1 MiB per GPU,
+ * held until the process ends.  Limit: B * H <= 256 heads per call (D 64 or 128); beyond that the call prints an
+ * error, does nothing and returns -1 (0 on success).  Calls no hipMalloc / hipFree.  Every call on one GPU shares
+ * that GPU's array: calls that overlap on one GPU (two streams, two threads) race -- serialise them.  The first
+ * call on a device looks the array's address up and enqueues a small clear of the counters on `stream`; make
+ * that first call outside stream capture. */
+int ternaspmm_decode_attention_static(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
+                                      const long long* pos, terna_bf16* out, int B, int H, int KV, int D, int S,
+                                      float scale, terna_stream stream);
 /* Both of the above in one launch for T = 1: qkv bf16 [B][(H + 2*KV)*D], cos / sin fp32 [D/2] of the new
  * token's position; writes slot pos[0] of the caches and out.  Results are bit-identical to
  * ternaspmm_rope_kv_store followed by ternaspmm_decode_attention. */

@@ -1,5 +1,5 @@
 // C ABI of the attention-side kernels of a decode step (attention_kernel.h): RoPE + cache write, single-token
-// attention, both in one launch, and the prefetching variant.
+// attention, both in one launch, the prefetching variant, and the variant that allocates nothing.
 // Declarations: include/ternaspmm.h.
 #include <hip/hip_runtime.h>
 
@@ -14,6 +14,9 @@
 using namespace terna;
 
 namespace {
+
+// one word per thread; the grid covers the buffer exactly
+__global__ void terna_fill_u32_kernel(uint32_t* p, uint32_t v) { p[blockIdx.x * blockDim.x + threadIdx.x] = v; }
 
 // Waves per workgroup of the decode attention: with one workgroup per (sequence, head) and few of them
 // on the chip, wider workgroups request more of the cache up front (64 slots of keys per wave).
@@ -131,6 +134,45 @@ bool attention_args_ok(const char* who, int B, int H, int KV, int D, int S)
 
 }  // namespace
 
+// ---- the entry point that allocates nothing (ternaspmm_decode_attention_static) -------------------------------
+// Its split-attention scratch lives in this file-scope device array instead of a caller workspace: kStaticHeads
+// arrival counters first -- at a fixed place whatever the call's size, so that the zeros every launch leaves behind
+// are the zeros the next one starts from -- then kAttentionMaxSplits partial results of up to 128 + 2 floats per head.
+// Every GPU the library runs on holds its own copy of the array, at its own address, until the process ends.
+constexpr int kStaticHeads = 256;                                       // B * H of one call
+constexpr size_t kStaticCounterBytes = kStaticHeads * sizeof(int);     // 1 KiB, a multiple of 256
+constexpr size_t kStaticScratchBytes =
+    kStaticCounterBytes + static_cast<size_t>(kStaticHeads) * kAttentionMaxSplits * (128 + 2) * sizeof(float);   // ~1.02 MiB
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Device address of `scratch` on the current device (in host code the array's name is only a handle for this lookup).
+// Looked up once per device; the first sight also clears the counters with a fill kernel on the caller's stream.
+static unsigned char* static_scratch(hipStream_t st, int line)
+{
+    static std::mutex mutex;
+    static unsigned char* ptr_of[64] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) die("hipGetDevice", e, line);
+    if (dev < 0 || dev >= 64) {
+        std::fprintf(stderr, "ternaspmm_decode_attention_static: device ordinal %d is outside 0 .. 63\n", dev);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(mutex);
+    if (ptr_of[dev] == nullptr) {
+        unsigned char* ptr = nullptr;
+        e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr) die("hipGetSymbolAddress(scratch)", e, line);
+        static_assert(kStaticCounterBytes % (256 * sizeof(uint32_t)) == 0, "fill grid");
+        terna_fill_u32_kernel<<<dim3(kStaticCounterBytes / (256 * sizeof(uint32_t))), dim3(256), 0, st>>>(
+            reinterpret_cast<uint32_t*>(ptr), 0u);
+        e = hipGetLastError();
+        if (e != hipSuccess) die("scratch clear", e, line);
+        ptr_of[dev] = ptr;
+    }
+    return ptr_of[dev];
+}
+
 extern "C" {
 
 void ternaspmm_rope_kv_store(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
@@ -168,6 +210,28 @@ void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, 
                                    static_cast<hipStream_t>(stream));
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_decode_attention", e, __LINE__);
+}
+
+int ternaspmm_decode_attention_static(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
+                                      const long long* pos, terna_bf16* out, int B, int H, int KV, int D, int S,
+                                      float scale, terna_stream stream)
+{
+    if (!attention_args_ok("ternaspmm_decode_attention_static", B, H, KV, D, S)) return -1;
+    if (static_cast<long>(B) * H > kStaticHeads) {
+        std::fprintf(stderr,
+                     "ternaspmm_decode_attention_static: B * H = %ld heads exceed the %d the library's static scratch holds; "
+                     "use ternaspmm_decode_attention with a workspace\n", static_cast<long>(B) * H, kStaticHeads);
+        return -1;
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    unsigned char* base = static_scratch(st, __LINE__);
+    if (base == nullptr) return -1;
+    const AttentionScratch sc{reinterpret_cast<int*>(base), reinterpret_cast<float*>(base + kStaticCounterBytes)};
+    launch_attention<false, false>(q, const_cast<uint16_t*>(cache_k), const_cast<uint16_t*>(cache_v), nullptr, nullptr, pos,
+                                   out, B, H, KV, D, S, scale, sc, AttentionPrefetch{}, st);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_decode_attention_static", e, __LINE__);
+    return 0;
 }
 
 void ternaspmm_rope_decode_attention(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
