@@ -14,6 +14,14 @@ Prints ONE JSON line.  `value` is algorithmic GB/s: bytes of the reference-forma
 dense matrix -- divided by the measured time.  `roofline` prices the same bytes against the
 8 TB/s HBM peak; `cpu_baseline` times decode-to-dense + torch.matmul on the host cores for one
 layer of the same workload and doubles as the correctness gate of the run.
+
+The default run (`--workload decode`) also measures, in the same process and into the same line,
+the other figures the path is judged on: the literal single-matrix configuration (`config1`),
+the layer set at M = 1 and 16, the unmodified call site (`drop_in_reference_format`), the prefill
+shapes at M = 2048 for both activation types (`prefill_m2048`), the 2B-shaped model's decode
+tokens/s at batch 1 and 8 (`model_decode`) and what the machine gives (`calibration`: cost of a
+graph kernel node, read and copy rate, cost of a device-wide synchronisation).  `--no-extras`
+leaves those out.
 """
 from __future__ import annotations
 
@@ -34,21 +42,21 @@ HBM_PEAK_GBPS = 8000.0
 BF16_MFMA_PEAK_TFLOPS = 2500.0
 INT8_MFMA_PEAK_TOPS = 5000.0
 LAYER_SET = [("wqkv", 3840, 2560), ("wo", 2560, 2560), ("w13", 13824, 2560), ("w2", 2560, 6912)]   # (name, N, K)
+METRIC = "TernaSpMM GB/s + %HBM roofline (M=8,K=N=2560); 2B-shape decode tok/s"
 
-# HBM bytes per launch of the small-M kernel on the default workload (M=8, average over the four
-# matrices), from two rocprofv3 --pmc runs (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each
-# scaled by what the same counter reads for a plain 256 MiB device copy / fill in the same run
-# (FETCH_SIZE reads 131088 for 262144 KiB -> x2.0; WRITE_SIZE reads 262144 -> x1.0).  Per layer:
-# 19209 KiB fetched + 356 KiB written over 4 launches.  None where not collected.
-TRAFFIC_BYTES_PER_LAUNCH = {"packed": (19209.3 + 356.0) * 1024 / 4, "reference": None}
+# HBM bytes per launch of the small-M P2 kernel on the default workload (M=8, average over the four matrices):
+# a counter measurement, not part of this run -- two rocprofv3 --pmc runs of this file (FETCH_SIZE, WRITE_SIZE),
+# scaled by what the same counters read for a 256 MiB copy.  Quoted with its source; null for any other workload.
+TRAFFIC = {"bytes_per_launch": (19209.3 + 356.0) * 1024 / 4,
+           "source": "profiles/decode_packed_kernel_hbm_traffic.md (rocprofv3 --pmc; kernel unchanged since)"}
 
 
 def vp(t):
-    return ctypes.c_void_p(t.data_ptr())
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
 
 
 def make_ternary(n, k, p0, seed):
-    """iid ternary from 16-bit draws: zero iff draw < p0 * 65536 (P(0) = 0.40 to 1e-5), sign = bit 0,
+    """iid ternary from 16-bit draws: zero iff draw < p0 * 65536 (P(0) = p0 to 1e-5), sign = bit 0,
     which is balanced and independent of the zero test."""
     rng = np.random.default_rng(seed)
     b = rng.integers(0, 65536, size=(n, k), dtype=np.uint16)
@@ -70,42 +78,60 @@ def make_row_skewed(n, k, seed):
 
 
 class Matrix:
-    """One ternary matrix: host copy, `copies` device copies of the format, activations, output."""
+    """One ternary matrix: host copy, `copies` device copies of the format (reference layout and P2),
+    and per activation-row count M a bf16 activation block and an output."""
 
-    def __init__(self, name, n, k, m, copies, seed, torch, T, w=None):
+    def __init__(self, name, n, k, m, copies, seed, torch, T, w=None, p0=0.40):
+        self.torch = torch
         self.name, self.n, self.k, self.m = name, n, k, m
-        self.w = make_ternary(n, k, 0.40, seed) if w is None else w
+        self.w = make_ternary(n, k, p0, seed) if w is None else w
         vals, off, med, bm = T.compress_weight(torch.from_numpy(self.w))
         self.host_format = (vals.numpy(), off.numpy(), med.numpy(), bm.numpy())
         self.n_sign_words = int(vals.numel())
         base = [t.cuda() for t in (vals, off, med, bm)]
         self.dev = [base] + [[t.clone() for t in base] for _ in range(copies - 1)]
-        # load-time repack (P2 layout), one buffer per weight copy
         lib = T._lib.load()
-        self.packed = []
+        self.packed = []                     # load-time repack (P2 layout), one buffer per weight copy
         for vals_d, off_d, med_d, bm_d in self.dev:
             buf = torch.empty(lib.ternaspmm_packed_bytes(n, k) // 4, dtype=torch.int32, device="cuda")
             lib.ternaspmm_repack(vp(bm_d), vp(off_d), vp(med_d), vp(vals_d), vp(buf), n, k, None)
             self.packed.append(buf)
         torch.cuda.synchronize()
+        self.seed = seed
         rng = np.random.default_rng(seed + 1)
         self.x_bits = f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
-        self.x = torch.from_numpy(self.x_bits.view(np.int16)).cuda()
         self.scale_host = rng.uniform(0.5, 2.0, 1).astype(np.float32)
         self.scale = torch.from_numpy(self.scale_host).cuda()
-        self.out = torch.zeros((m, n), dtype=torch.int16, device="cuda")
-        # reference-format bytes one call has to move
-        self.alg_bytes = (8 * (n * k // 64) + 4 * self.n_sign_words + 4 * (n * k // 4096 + 1)
-                          + 2 * (3 * n * k // 4096) + 2 * m * k + 4 + 2 * m * n)
+        self.acts = {m: (torch.from_numpy(self.x_bits.view(np.int16)).cuda(), torch.zeros((m, n), dtype=torch.int16, device="cuda"))}
+        self.x, self.out = self.acts[m]
 
-    def launch(self, lib, copy, stream, layout="packed"):
+    def bytes_at(self, m):
+        """Reference-format bytes one call at M = m has to move."""
+        n, k = self.n, self.k
+        return (8 * (n * k // 64) + 4 * self.n_sign_words + 4 * (n * k // 4096 + 1) + 2 * (3 * n * k // 4096)
+                + 2 * m * k + 4 + 2 * m * n)
+
+    @property
+    def alg_bytes(self):
+        return self.bytes_at(self.m)
+
+    def act(self, m):
+        if m not in self.acts:
+            rng = np.random.default_rng(self.seed + 100 + m)
+            x = f32_to_bf16_bits(rng.standard_normal((m, self.k)).astype(np.float32))
+            self.acts[m] = (self.torch.from_numpy(x.view(np.int16)).cuda(),
+                            self.torch.zeros((m, self.n), dtype=self.torch.int16, device="cuda"))
+        return self.acts[m]
+
+    def launch(self, lib, copy, stream, layout="packed", m=None):
+        m = self.m if m is None else m
+        x, out = self.act(m)
         if layout == "packed":
-            lib.bitlinear_TernaSpMM_bf16_packed(vp(self.x), vp(self.packed[copy]), vp(self.out), vp(self.scale),
-                                                1, self.m, self.n, self.k, 0, stream)
+            lib.bitlinear_TernaSpMM_bf16_packed(vp(x), vp(self.packed[copy]), vp(out), vp(self.scale), 1, m, self.n, self.k, 0, stream)
         else:
             vals, off, med, bm = self.dev[copy]
-            lib.bitlinear_TernaSpMM_bf16(vp(self.x), vp(bm), vp(off), vp(med), vp(vals), vp(self.out), vp(self.scale),
-                                         1, self.m, self.n, self.k, 1, None, stream)
+            lib.bitlinear_TernaSpMM_bf16(vp(x), vp(bm), vp(off), vp(med), vp(vals), vp(out), vp(self.scale),
+                                         1, m, self.n, self.k, 1, None, stream)
 
 
 def time_graph(torch, graph, replays, warmup):
@@ -181,39 +207,57 @@ def cpu_baseline(mats, torch):
     }
 
 
-def run_model(args, torch):
-    """configs[4]: 2B-shaped random-init model, prompt of 128 uniform random ids, greedy decode of 256
-    tokens; tokens/s = generated tokens / decode-phase time (as the reference's stats.py:19-27)."""
+# ------------------------------------------------------------------------------------------------ model (configs[4])
+def measure_model(torch, batch, act="int8", prefetch=True, gen_tokens=256, check_tokens=8, model=None):
+    """2B-shaped random-init model, prompt of 128 uniform random ids, greedy decode of `gen_tokens`
+    tokens; tokens/s = generated tokens / decode-phase time (as the reference's stats.py:19-27).
+    Self-check of the run: the captured decode graph must produce the tokens of eager execution
+    for the first `check_tokens` tokens.  Returns (figures, model)."""
     from ternainfer_amd.model import ModelArgs, Transformer, greedy_decode
     margs = ModelArgs()
     t0 = time.perf_counter()
-    args.act = args.act or "int8"
-    model = Transformer(margs, seed=20260500, act=args.act)
-    if not args.no_prefetch:     # weights of the following launches, pulled through the caches during the attention launch
-        model.enable_prefetch(True, ("wo", "w13", "w2", "next_wqkv", "norms") if args.batch <= 2 else ("wo", "w13", "norms"))
+    if model is None:
+        model = Transformer(margs, seed=20260500, act=act)
+    model.enable_prefetch(False)
+    if prefetch:     # weights of the following launches, pulled through the caches during the attention launch
+        model.enable_prefetch(True, ("wo", "w13", "w2", "next_wqkv", "norms") if batch <= 2 else ("wo", "w13", "norms"))
     torch.cuda.synchronize()
     build_s = time.perf_counter() - t0
     gen = torch.Generator(device="cuda").manual_seed(20260501)
-    prompt = torch.randint(0, margs.vocab_size, (args.batch, 128), generator=gen, device="cuda")
-    greedy_decode(model, prompt, 8)                                   # warm-up (code objects, allocator)
-    toks, prefill_s, decode_s = greedy_decode(model, prompt, 256)
-    tps = args.batch * 256 / decode_s
-    print(json.dumps({
-        "metric": "2B-shape decode tok/s", "value": tps, "unit": "tokens/s", "n_gpus": 1, "steps": 256, "warmup": 8,
-        "ms_per_step": decode_s * 1e3 / 256, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": args.act, "data": "synthetic",
+    prompt = torch.randint(0, margs.vocab_size, (batch, 128), generator=gen, device="cuda")
+    warm, _, _ = greedy_decode(model, prompt, check_tokens)                     # warm-up (code objects, allocator)
+    eager, _, _ = greedy_decode(model, prompt, check_tokens, use_graph=False)
+    graph_equals_eager = bool(torch.equal(warm, eager))
+    assert graph_equals_eager, "decode graph and eager execution disagree"
+    toks, prefill_s, decode_s = greedy_decode(model, prompt, gen_tokens)
+    assert torch.equal(toks[:, :check_tokens], eager)
+    return {"batch": batch, "tokens_per_s": batch * gen_tokens / decode_s, "ms_per_step": decode_s * 1e3 / gen_tokens,
+            "prefill_tokens_per_s": batch * 128 / prefill_s, "prefill_ms": prefill_s * 1e3, "decode_s": decode_s,
+            "generated_tokens": gen_tokens, "graph_equals_eager_first_tokens": check_tokens,
+            "first_tokens": toks[0, :8].tolist(), "model_build_s": build_s}, model
+
+
+def run_model(args, torch):
+    act = args.act or "int8"
+    fig, _ = measure_model(torch, args.batch, act, not args.no_prefetch)
+    return {
+        "metric": "2B-shape decode tok/s", "value": fig["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": 256, "warmup": 8,
+        "ms_per_step": fig["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": act, "data": "synthetic",
         "config": {"workload": f"configs[4]: BitNet-b1.58-2B-shaped random-init decoder (30 layers, hidden 2560, 20/5 heads, "
                                f"FFN 6912, vocab 128256), batch {args.batch}, 128-token prompt, 256 greedy tokens, "
-                               f"{args.act} activations into the ternary linears, weights in P2 layout, one HIP graph per "
-                               "decode step; norms, gate, activation quantisation, RoPE, cache write and "
-                               "single-token attention are library kernels, prefill attention and the bf16 LM head "
-                               "are PyTorch-ROCm ops" + ("" if args.no_prefetch else "; the idle CUs of the attention launch "
-                                                         "prefetch the weights of the launches that follow"),
-                   "batch": args.batch, "act": args.act},
-        "prefill_tokens_per_s": args.batch * 128 / prefill_s, "prefill_s": prefill_s, "decode_s": decode_s,
-        "model_build_s": build_s, "first_tokens": toks[0, :8].tolist()}))
+                               f"{act} activations into the ternary linears, weights in P2 layout, one HIP graph per "
+                               "decode step; norms, gate, activation quantisation, RoPE, cache write, single-token "
+                               "attention, the bf16 LM head and greedy sampling are library kernels; the attention of "
+                               "the prompt pass is a PyTorch-ROCm op"
+                               + ("" if args.no_prefetch else "; the idle CUs of the attention launch "
+                                                            "prefetch the weights of the launches that follow"),
+                   "batch": args.batch, "act": act},
+        **{k: fig[k] for k in ("prefill_tokens_per_s", "prefill_ms", "decode_s", "model_build_s", "first_tokens",
+                               "graph_equals_eager_first_tokens")}}
 
 
+# ------------------------------------------------------------------------------------------------ sweep (configs[3])
 def run_sweep(args, torch, T, lib):
     """configs[3]: sparsity / structure sweep at M = 16 on K = N = 2560 and on K = 6912, N = 2560 -- global zero
     fraction 0.20 / 0.33 / 0.45 / 0.60 and a row-skewed matrix -- on both weight layouts.  The reference format's
@@ -245,8 +289,8 @@ def run_sweep(args, torch, T, lib):
         detail[name] = entry
         total_bytes += mt.alg_bytes
     gbps = total_bytes / total_us[args.layout] / 1e3
-    print(json.dumps({
-        "metric": "TernaSpMM GB/s + %HBM roofline (M=8,K=N=2560); 2B-shape decode tok/s", "value": gbps, "unit": "GB/s",
+    return {
+        "metric": METRIC, "value": gbps, "unit": "GB/s",
         "n_gpus": 1, "steps": max(args.steps // 2, 5), "warmup": args.warmup, "ms_per_step": total_us[args.layout] * 1e-3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"configs[3]: sparsity / structure sweep, M={m}, K=N=2560 and K=6912 N=2560, zero fraction "
@@ -255,59 +299,60 @@ def run_sweep(args, torch, T, lib):
                    "m": m, "layout": args.layout},
         "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
                      "traffic": None},
-        "per_case": detail}))
+        "per_case": detail}
 
 
-def run_prefill(args, torch, T, lib):
-    """configs[2]: the four BitNet-2B matrices at M in {256, 512, 2048}, bf16 activations with 1% of
-    the channels scaled x20 (--act int8: the same activations quantised per row to int8, the
-    reference's own prefill input).  A step is one pass over the four matrices at M = --m (default
-    2048 when --workload prefill is given without --m).  Next to every shape the vendor's dense GEMM
-    (torch.matmul / torch._int_mm on already expanded weights) is timed as a yardstick."""
-    m_main = args.m if args.m >= 64 else 2048
-    act = args.act or "bf16"
-    if act == "int8" and args.layout != "packed":
-        sys.exit("bench.py: --workload prefill --act int8 runs on the packed layout")
-    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    rng = np.random.default_rng(20260300)
-    mats = []
-    for j, (name, n, k) in enumerate(LAYER_SET):
-        mt = Matrix(name, n, k, 8, 1, 20260300 + 10 * j, torch, T)
-        xs = {}
-        for m in sorted({256, 512, 2048, m_main}):
-            xf = rng.standard_normal((m, k)).astype(np.float32)
-            ch = rng.permutation(k)[: int(np.ceil(0.01 * k))]
-            xf[:, ch] *= 20.0
-            if act == "bf16":
-                xs[m] = (torch.from_numpy(f32_to_bf16_bits(xf).view(np.int16)).cuda(),
-                         torch.zeros((m, n), dtype=torch.int16, device="cuda"))
-            else:                  # per-row absmax quantisation, as the reference's quant_input (model.py:60-63)
-                sc = 127.0 / np.maximum(np.abs(xf).max(axis=1, keepdims=True), 1e-5)
-                xq = np.clip(np.rint(xf * sc), -128, 127).astype(np.int8)
-                xs[m] = (torch.from_numpy(xq).cuda(), torch.zeros((m, n), dtype=torch.int16, device="cuda"),
-                         torch.from_numpy(f32_to_bf16_bits(sc.astype(np.float32).ravel()).view(np.int16)).cuda())
-        mt.ws = torch.from_numpy(f32_to_bf16_bits(mt.scale_host).view(np.int16)).cuda()
-        mats.append((mt, xs))
+# ------------------------------------------------------------------------------------------------ prefill (configs[2])
+class PrefillSet:
+    """The four BitNet-2B matrices with activations at the given row counts: bf16 with 1% of the channels
+    scaled x20, and the same activations quantised per row to int8 (the reference's own prefill input)."""
 
-    work = torch.empty(13824 * 2560, dtype=torch.int8, device="cuda")      # the reference's global workspace
+    def __init__(self, torch, T, m_values, acts=("bf16", "int8")):
+        self.torch = torch
+        rng = np.random.default_rng(20260300)
+        self.mats = []
+        for j, (name, n, k) in enumerate(LAYER_SET):
+            mt = Matrix(name, n, k, 8, 1, 20260300 + 10 * j, torch, T)
+            xs = {}
+            for m in sorted(set(m_values)):
+                xf = rng.standard_normal((m, k)).astype(np.float32)
+                ch = rng.permutation(k)[: int(np.ceil(0.01 * k))]
+                xf[:, ch] *= 20.0
+                if "bf16" in acts:
+                    xs[("bf16", m)] = (torch.from_numpy(f32_to_bf16_bits(xf).view(np.int16)).cuda(),
+                                       torch.zeros((m, n), dtype=torch.int16, device="cuda"))
+                if "int8" in acts:     # per-row absmax quantisation, as the reference's quant_input (model.py:120-123)
+                    sc = 127.0 / np.maximum(np.abs(xf).max(axis=1, keepdims=True), 1e-5)
+                    xq = np.clip(np.rint(xf * sc), -128, 127).astype(np.int8)
+                    xs[("int8", m)] = (torch.from_numpy(xq).cuda(), torch.zeros((m, n), dtype=torch.int16, device="cuda"),
+                                       torch.from_numpy(f32_to_bf16_bits(sc.astype(np.float32).ravel()).view(np.int16)).cuda())
+            mt.ws = torch.from_numpy(f32_to_bf16_bits(mt.scale_host).view(np.int16)).cuda()
+            self.mats.append((mt, xs))
+        self.work = torch.empty(13824 * 2560, dtype=torch.int8, device="cuda")      # the reference's global workspace
 
-    def launch(mt, xs, m, s):
+    def launch(self, lib, mt, xs, act, m, s, layout="packed", route=0):
         if act == "int8":
-            x, out, srow = xs[m]
-            lib.bitlinear_TernaSpMM_packed(vp(x), vp(mt.packed[0]), vp(out), vp(srow), vp(mt.ws), 1, m, mt.n, mt.k, 0, s)
+            x, out, srow = xs[("int8", m)]
+            if layout == "packed":
+                lib.bitlinear_TernaSpMM_packed_ws(vp(x), vp(mt.packed[0]), vp(out), vp(srow), vp(mt.ws), 1, m, mt.n, mt.k, route,
+                                                  vp(self.work), self.work.numel(), s)
+            else:
+                vals, off, med, bm = mt.dev[0]
+                lib.bitlinear_TernaSpMM(vp(x), vp(bm), vp(off), vp(med), vp(vals), vp(out), vp(srow), vp(mt.ws), 1, m, mt.n, mt.k,
+                                        7, vp(self.work), s)
             return
-        x, out = xs[m]
-        if args.layout == "packed":
-            lib.bitlinear_TernaSpMM_bf16_packed(vp(x), vp(mt.packed[0]), vp(out), vp(mt.scale), 1, m, mt.n, mt.k, 0, s)
+        x, out = xs[("bf16", m)]
+        if layout == "packed":
+            lib.bitlinear_TernaSpMM_bf16_packed_ws(vp(x), vp(mt.packed[0]), vp(out), vp(mt.scale), 1, m, mt.n, mt.k, route,
+                                                   vp(self.work), self.work.numel(), s)
         else:                      # reference-format pointers + workspace: transcode per call, then the P2 kernel
             vals, off, med, bm = mt.dev[0]
             lib.bitlinear_TernaSpMM_bf16(vp(x), vp(bm), vp(off), vp(med), vp(vals), vp(out), vp(mt.scale),
-                                         1, m, mt.n, mt.k, 1, vp(work), s)
+                                         1, m, mt.n, mt.k, 1, vp(self.work), s)
 
-    peak = BF16_MFMA_PEAK_TFLOPS if act == "bf16" else INT8_MFMA_PEAK_TOPS
-
-    def dense_us(m, n, k):
-        """Vendor dense GEMM of the same shape on expanded weights (not part of the product)."""
+    def dense_us(self, act, m, n, k, reps=10):
+        """Vendor dense GEMM of the same shape on expanded weights (a yardstick, not part of the product)."""
+        torch = self.torch
         if act == "bf16":
             a = torch.randn(m, k, device="cuda", dtype=torch.bfloat16)
             b = torch.randn(n, k, device="cuda", dtype=torch.bfloat16).t()
@@ -321,64 +366,208 @@ def run_prefill(args, torch, T, lib):
                 f()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-            for _ in range(10):
+            for _ in range(reps):
                 f()
             e1.record()
             torch.cuda.synchronize()
-            return e0.elapsed_time(e1) * 1e3 / 10
+            return e0.elapsed_time(e1) * 1e3 / reps
         except Exception:                                   # no such vendor kernel in this build
             return None
 
-    per_shape = {}
-    dense_main_us = 0.0
-    for mt, xs in mats:
-        for m in ([] if args.no_per_shape else sorted(xs)):
-            launch(mt, xs, m, stream)
-            torch.cuda.synchronize()
-            g = capture(torch, lambda s, mt=mt, xs=xs, m=m: [launch(mt, xs, m, s) for _ in range(10)])
-            us = time_graph(torch, g, 5, 2) * 1e3 / 10
-            tf = 2.0 * m * mt.n * mt.k / us / 1e6
-            d_us = dense_us(m, mt.n, mt.k)
-            per_shape[f"{mt.name}_{mt.k}x{mt.n}_M{m}"] = {"us": us, "tflops": tf, "frac": tf / peak,
-                                                         "vendor_dense_gemm_us": d_us}
-            if m == m_main and d_us is not None and dense_main_us is not None:
-                dense_main_us += d_us
-            elif m == m_main:
-                dense_main_us = None
+    def shape_us(self, lib, mt, xs, act, m, layout="packed", route=0, reps=10):
+        torch = self.torch
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        self.launch(lib, mt, xs, act, m, stream, layout, route)
+        torch.cuda.synchronize()
+        g = capture(torch, lambda s: [self.launch(lib, mt, xs, act, m, s, layout, route) for _ in range(reps)])
+        return time_graph(torch, g, 5, 2) * 1e3 / reps
 
-    graph = capture(torch, lambda s: [launch(mt, xs, m_main, s) for mt, xs in mats])
-    for _ in range(args.warmup):
-        graph.replay()
-    torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    ev0.record()
-    for _ in range(args.steps):
-        graph.replay()
-    ev1.record()
-    torch.cuda.synchronize()
-    ms = ev0.elapsed_time(ev1) / args.steps
-    flops = sum(2.0 * m_main * mt.n * mt.k for mt, _ in mats)
-    tf = flops / (ms * 1e-3) / 1e12
-    print(json.dumps({
+    def step(self, lib, act, m, steps, warmup, layout="packed"):
+        """One pass over the four matrices at M = m, graph-replayed: (ms per step, flops per step)."""
+        torch = self.torch
+        graph = capture(torch, lambda s: [self.launch(lib, mt, xs, act, m, s, layout) for mt, xs in self.mats])
+        ms = time_graph(torch, graph, steps, warmup)
+        return ms, sum(2.0 * m * mt.n * mt.k for mt, _ in self.mats)
+
+
+def prefill_figures(ps, lib, act, m, steps, warmup, per_shape=True, layout="packed"):
+    peak = BF16_MFMA_PEAK_TFLOPS if act == "bf16" else INT8_MFMA_PEAK_TOPS
+    ms, flops = ps.step(lib, act, m, steps, warmup, layout)
+    rate = flops / (ms * 1e-3) / 1e12
+    out = {"act": act, "m": m, "ms_per_step": ms, "rate": rate, "unit": "TFLOP/s" if act == "bf16" else "TOP/s",
+           "peak": peak, "frac": rate / peak}
+    if per_shape:
+        shapes, dense_total = {}, 0.0
+        for mt, xs in ps.mats:
+            us = ps.shape_us(lib, mt, xs, act, m, layout)
+            d_us = ps.dense_us(act, m, mt.n, mt.k)
+            tf = 2.0 * m * mt.n * mt.k / us / 1e6
+            shapes[f"{mt.name}_{mt.k}x{mt.n}"] = {"us": us, "rate": tf, "frac": tf / peak, "vendor_dense_gemm_us": d_us}
+            dense_total = None if (d_us is None or dense_total is None) else dense_total + d_us
+        out["per_shape"] = shapes
+        out["vendor_dense_gemm"] = None if not dense_total else {
+            "what": "torch.matmul (bf16) / torch._int_mm (int8) on already expanded weights, same four shapes, eager",
+            "ms_per_step": dense_total * 1e-3, "rate": flops / (dense_total * 1e-6) / 1e12}
+    return out
+
+
+def run_prefill(args, torch, T, lib):
+    """configs[2]: the four BitNet-2B matrices at M in {256, 512, 2048}, bf16 activations with 1% of
+    the channels scaled x20 (--act int8: the same activations quantised per row to int8, the
+    reference's own prefill input).  A step is one pass over the four matrices at M = --m (default
+    2048 when --workload prefill is given without --m).  Next to every shape the vendor's dense GEMM
+    (torch.matmul / torch._int_mm on already expanded weights) is timed as a yardstick."""
+    m_main = args.m if args.m >= 64 else 2048
+    act = args.act or "bf16"
+    ms_all = sorted({256, 512, 2048, m_main})
+    ps = PrefillSet(torch, T, [m_main] if args.no_per_shape else ms_all, acts=(act,))
+    fig = prefill_figures(ps, lib, act, m_main, args.steps, args.warmup, per_shape=False, layout=args.layout)
+    per_shape, dense_main = {}, None
+    if not args.no_per_shape:
+        peak = fig["peak"]
+        dense_main = 0.0
+        for mt, xs in ps.mats:
+            for m in ms_all:
+                us = ps.shape_us(lib, mt, xs, act, m, args.layout)
+                d_us = ps.dense_us(act, m, mt.n, mt.k)
+                tf = 2.0 * m * mt.n * mt.k / us / 1e6
+                per_shape[f"{mt.name}_{mt.k}x{mt.n}_M{m}"] = {"us": us, "tflops": tf, "frac": tf / peak, "vendor_dense_gemm_us": d_us}
+                if m == m_main:
+                    dense_main = None if (d_us is None or dense_main is None) else dense_main + d_us
+    flops = sum(2.0 * m_main * mt.n * mt.k for mt, _ in ps.mats)
+    unit = fig["unit"]
+    return {
         "metric": "TernaSpMM prefill TFLOP/s + %bf16 MFMA peak (M=2048, BitNet-2B layer set)" if act == "bf16"
                   else "TernaSpMM prefill TOP/s, int8 activations (M=2048, BitNet-2B layer set)",
-        "value": tf, "unit": "TFLOP/s" if act == "bf16" else "TOP/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16" if act == "bf16" else "int8",
-        "data": "synthetic",
+        "value": fig["rate"], "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": fig["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if act == "bf16" else "int8", "data": "synthetic",
         "config": {"workload": f"configs[2]: four BitNet-b1.58-2B matrices at M={m_main}, P(0)=0.40, {act} activations "
                                "with 1% outlier channels (x20), HIP-graph replay; weight layout: "
                                + ("P2, repacked once at load time" if args.layout == "packed"
                                   else "reference format, transcoded into the workspace on every call"),
                    "m": m_main, "layout": args.layout},
-        "roofline": {"bound": "mfma", "achieved": tf, "peak": peak, "unit": "TFLOP/s" if act == "bf16" else "TOP/s",
-                     "frac": tf / peak, "traffic": None,
+        "roofline": {"bound": "mfma", "achieved": fig["rate"], "peak": fig["peak"], "unit": unit, "frac": fig["frac"], "traffic": None,
                      "kernel": f"terna_prefill_packed_dma_kernel<{act}>", "algorithmic_flops_per_step": flops},
-        "vendor_dense_gemm": None if not dense_main_us else {
+        "vendor_dense_gemm": None if not dense_main else {
             "what": "torch.matmul (bf16) / torch._int_mm (int8) on already expanded weights, same four shapes, eager",
-            "ms_per_step": dense_main_us * 1e-3, "rate": flops / (dense_main_us * 1e-6) / 1e12},
-        "per_shape": per_shape}))
+            "ms_per_step": dense_main * 1e-3, "rate": flops / (dense_main * 1e-6) / 1e12},
+        "per_shape": per_shape}
+
+
+# ------------------------------------------------------------------------------------------------ mid-M policy
+def run_midm(args, torch, T, lib):
+    """Both kernel families (route 2 = small-M dot-product kernel, route 1 = MFMA-tiled kernel) on the four 2B
+    matrices at the batch sizes between decode and prefill, P2 layout, hot (one weight copy: the choice of
+    kernel is about the compute side).  The library's own choice (route 0) is timed beside them."""
+    m_values = [16, 24, 32, 48, 64, 96, 128, 192, 256]
+    act = args.act or "bf16"
+    ps = PrefillSet(torch, T, m_values, acts=(act,))
+    table = {}
+    for mt, xs in ps.mats:
+        for m in m_values:
+            row = {}
+            routes = (("small_m_kernel_us", 2), ("mfma_kernel_us", 1), ("library_choice_us", 0)) if act == "bf16" else \
+                     (("small_m_kernel_us", 4), ("mfma_kernel_us", 8), ("library_choice_us", 0))     # int8: +4 / +8 pick the kernel
+            for label, route in routes:
+                row[label] = ps.shape_us(lib, mt, xs, act, m, "packed", route)
+            row["best"] = "small_m" if row["small_m_kernel_us"] <= row["mfma_kernel_us"] else "mfma"
+            table[f"{mt.name}_{mt.k}x{mt.n}_M{m}"] = row
+    worst = max(r["library_choice_us"] / min(r["small_m_kernel_us"], r["mfma_kernel_us"]) for r in table.values())
+    return {"metric": "TernaSpMM mid-M kernel choice (us per launch)", "value": worst, "unit": "library choice / best, worst case",
+            "n_gpus": 1, "steps": 5, "warmup": 2, "ms_per_step": None, "higher_is_better": False, "scaling": "weak",
+            "vs_baseline": None, "dtype": act, "data": "synthetic",
+            "config": {"workload": f"four BitNet-b1.58-2B matrices at M in {m_values}, {act} activations, P2 layout, hot"},
+            "per_shape": table}
+
+
+# ------------------------------------------------------------------------------------------------ calibration
+def calibration(torch, lib):
+    """What the machine gives, measured by the library's own probe kernels in this run."""
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    out = {}
+    nodes = 1000
+    g = capture(torch, lambda s: [lib.ternaspmm_probe_empty(s) for _ in range(nodes)])
+    out["graph_kernel_node_us"] = time_graph(torch, g, 5, 2) * 1e3 / nodes
+    nbytes = 1 << 30
+    a = torch.empty(nbytes, dtype=torch.int8, device="cuda").fill_(1)
+    b = torch.empty(nbytes, dtype=torch.int8, device="cuda")
+    for name, fn, moved in (("read_GBps", lambda: lib.ternaspmm_probe_read(vp(a), nbytes, None, stream), nbytes),
+                            ("copy_GBps", lambda: lib.ternaspmm_probe_copy(vp(a), vp(b), nbytes, stream), 2 * nbytes)):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(5):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        out[name] = moved * 5 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+    out["read_copy_bytes"] = nbytes
+    del a, b
+    # device-wide synchronisation among co-resident workgroups (one per CU): what a persistent kernel would pay
+    # between two dependent phases, to hold against the cost of a graph kernel node
+    state = torch.zeros(lib.ternaspmm_probe_barrier_state_bytes() // 4, dtype=torch.int32, device="cuda")
+    rounds, tag = 500, 1
+    sync = {}
+    for groups in (32, 64, 128, 256):
+        best = None
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            rc = lib.ternaspmm_probe_barrier(vp(state), groups, rounds, tag, stream)
+            e1.record()
+            torch.cuda.synchronize()
+            tag += rounds
+            if rc != 0:
+                break
+            us = e0.elapsed_time(e1) * 1e3 / rounds
+            best = us if best is None else min(best, us)
+        sync[str(groups)] = best
+    out["device_wide_sync_us_by_workgroups"] = sync
+    out["device_wide_sync_timeouts"] = int(state[512].item())
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ decode (configs[0], [1])
+def layer_set_step(torch, lib, mats, layers, layout, m, steps, warmup):
+    def step(stream):
+        for layer in range(layers):
+            for mt in mats:
+                mt.launch(lib, layer, stream, layout, m)
+    step(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))       # eager pass: code objects, outputs for the gate
+    torch.cuda.synchronize()
+    graph = capture(torch, step)
+    # ---- the timed region: W warm-up replays, then exactly K steps between two synchronised events
+    for _ in range(warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(steps):
+        graph.replay()
+    ev1.record()
+    torch.cuda.synchronize()
+    return ev0.elapsed_time(ev1) / steps
+
+
+def config1_row(torch, T, lib, copies=400):
+    """The literal single-matrix configuration: M = 8, K = N = 2560, P(0) = 0.45, one fp32 scale; cold = `copies`
+    rotating weight copies (more than twice the last-level cache), hot = one copy."""
+    from oracle import terna_oracle as O
+    mt = Matrix("config1", 2560, 2560, 8, copies, 20260100, torch, T, p0=0.45)
+    row = {"alg_bytes": mt.alg_bytes, "copies": copies}
+    for layout in ("packed", "reference"):
+        cold = capture(torch, lambda s: [mt.launch(lib, c, s, layout) for c in range(copies)])
+        hot = capture(torch, lambda s: [mt.launch(lib, 0, s, layout) for _ in range(copies)])
+        cold_us = time_graph(torch, cold, 5, 2) * 1e3 / copies
+        hot_us = time_graph(torch, hot, 5, 2) * 1e3 / copies
+        row[layout] = {"cold_us": cold_us, "cold_GBps": mt.alg_bytes / cold_us / 1e3, "cold_frac": mt.alg_bytes / cold_us / 1e3 / HBM_PEAK_GBPS,
+                       "hot_us": hot_us, "hot_GBps": mt.alg_bytes / hot_us / 1e3}
+        gold = O.spmm_bf16_golden(mt.x_bits, mt.w, mt.scale_host, 1)
+        got = O.bf16_bits_to_f32(mt.out.cpu().numpy().view(np.uint16)).astype(np.float64)
+        assert np.abs(got - gold).max() <= 1e-2 * np.abs(gold).max(), ("config1", layout)
+    return row
 
 
 def main():
@@ -388,10 +577,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--m", type=int, default=8, help="activation rows per call (decode batch)")
     ap.add_argument("--layers", type=int, default=30, help="distinct weight copies per matrix")
-    ap.add_argument("--workload", choices=["decode", "prefill", "model", "sweep"], default="decode",
-                    help="decode: the headline small-M HBM-bound pass; prefill: the M>=256 MFMA-bound pass; "
-                         "model: random-init BitNet-2B-shaped decoder, 128-token prompt + 256 greedy tokens; "
-                         "sweep: the sparsity / structure sweep at M=16")
+    ap.add_argument("--workload", choices=["decode", "prefill", "model", "sweep", "midm"], default="decode",
+                    help="decode: the headline small-M HBM-bound pass (plus, unless --no-extras, every other figure the "
+                         "path is judged on); prefill: the M>=256 MFMA-bound pass; model: random-init BitNet-2B-shaped "
+                         "decoder, 128-token prompt + 256 greedy tokens; sweep: the sparsity / structure sweep at M=16; "
+                         "midm: both kernel families at the batch sizes between decode and prefill")
     ap.add_argument("--batch", type=int, default=1, help="sequences decoded together (model workload)")
     ap.add_argument("--act", choices=["int8", "bf16"], default=None,
                     help="activations into the ternary linears: int8 + per-row scale (the reference's SpBitLinear; "
@@ -403,6 +593,8 @@ def main():
                     help="model workload: no weight prefetch by the idle CUs of the attention launch")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-per-shape", action="store_true")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="decode workload: only the headline step (no config1 / M sweep / prefill / model / calibration sections)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain 256 MiB device copy (calibrates FETCH_SIZE / WRITE_SIZE under rocprofv3 --pmc)")
     args = ap.parse_args()
@@ -423,47 +615,25 @@ def main():
         torch.cuda.synchronize()
         a.copy_(b)                                     # reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
-    if args.workload == "prefill":
-        run_prefill(args, torch, T, lib)
-        return
-    if args.workload == "model":
-        run_model(args, torch)
-        return
-    if args.workload == "sweep":
-        run_sweep(args, torch, T, lib)
+    if args.workload != "decode":
+        runner = {"prefill": lambda: run_prefill(args, torch, T, lib), "model": lambda: run_model(args, torch),
+                  "sweep": lambda: run_sweep(args, torch, T, lib), "midm": lambda: run_midm(args, torch, T, lib)}[args.workload]
+        print(json.dumps(runner()))
         return
 
+    t_start = time.perf_counter()
     mats = [Matrix(name, n, k, args.m, args.layers, 20260200 + 10 * j, torch, T)
             for j, (name, n, k) in enumerate(LAYER_SET)]
     step_bytes = args.layers * sum(mt.alg_bytes for mt in mats)
     launches_per_step = args.layers * len(mats)
 
-    def step(stream, layout=args.layout):
-        for layer in range(args.layers):
-            for mt in mats:
-                mt.launch(lib, layer, stream, layout)
-
-    # eager pass first (loads code objects, fills outputs for the correctness gate)
-    step(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
-    torch.cuda.synchronize()
-    graph = capture(torch, step)
-
-    # ---- the timed region: W warm-up replays, then exactly K steps between two synchronised events
-    for _ in range(args.warmup):
-        graph.replay()
-    torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    ev0.record()
-    for _ in range(args.steps):
-        graph.replay()
-    ev1.record()
-    torch.cuda.synchronize()
-    ms_per_step = ev0.elapsed_time(ev1) / args.steps
+    ms_per_step = layer_set_step(torch, lib, mats, args.layers, args.layout, args.m, args.steps, args.warmup)
     gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
     launch_us = ms_per_step * 1e3 / launches_per_step
+    default_workload = args.m == 8 and args.layers == 30 and args.layout == "packed"
 
     result = {
-        "metric": "TernaSpMM GB/s + %HBM roofline (M=8,K=N=2560); 2B-shape decode tok/s",
+        "metric": METRIC,
         "value": gbps, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
@@ -476,7 +646,8 @@ def main():
                    "algorithmic_bytes_per_step": step_bytes},
         "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": gbps / HBM_PEAK_GBPS,
-                     "traffic": TRAFFIC_BYTES_PER_LAUNCH[args.layout] if args.m == 8 and args.layers == 30 else None,
+                     "traffic": TRAFFIC["bytes_per_launch"] if default_workload else None,
+                     "traffic_source": TRAFFIC["source"] if default_workload else None,
                      "kernel": ("terna_decode_packed_kernel<bf16>" if args.layout == "packed"
                                 else "terna_decode_kernel<bf16>"),
                      "algorithmic_bytes_per_launch": step_bytes / launches_per_step,
@@ -504,6 +675,40 @@ def main():
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(mats, torch)
+
+    if not args.no_extras:
+        # the same layer set through the symbols an unmodified model.py binds (reference-format pointers), and at M = 1 / 16
+        other = "reference" if args.layout == "packed" else "packed"
+        ms_ref = layer_set_step(torch, lib, mats, args.layers, other, args.m, max(args.steps // 2, 5), 2)
+        key = "drop_in_reference_format" if other == "reference" else "packed_layout"
+        result[key] = {"ms_per_step": ms_ref, "GBps": step_bytes / (ms_ref * 1e-3) / 1e9,
+                       "frac": step_bytes / (ms_ref * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                       "what": "the same step through bitlinear_TernaSpMM_bf16 on reference-format pointers (no repack, no cache)"
+                               if other == "reference" else "the same step on the P2 layout"}
+        by_m = {}
+        for m in (1, 16):
+            ms = layer_set_step(torch, lib, mats, args.layers, args.layout, m, max(args.steps // 2, 5), 2)
+            b = args.layers * sum(mt.bytes_at(m) for mt in mats)
+            by_m[str(m)] = {"ms_per_step": ms, "GBps": b / (ms * 1e-3) / 1e9, "frac": b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                            "algorithmic_bytes_per_step": b}
+        result["layer_set_by_m"] = by_m
+        del mats
+        torch.cuda.empty_cache()
+        result["config1"] = config1_row(torch, T, lib)
+        torch.cuda.empty_cache()
+        ps = PrefillSet(torch, T, [2048])
+        result["prefill_m2048"] = {act: prefill_figures(ps, lib, act, 2048, 10, 3) for act in ("bf16", "int8")}
+        del ps
+        torch.cuda.empty_cache()
+        model = None
+        md = {}
+        for batch in (1, 8):
+            md[f"batch{batch}"], model = measure_model(torch, batch, "int8", True, model=model)
+        result["model_decode"] = md
+        del model
+        torch.cuda.empty_cache()
+        result["calibration"] = calibration(torch, lib)
+        result["bench_wall_s"] = time.perf_counter() - t_start
 
     print(json.dumps(result))
 

@@ -138,14 +138,31 @@ int64_t ternaspmm_packed_bytes(int N, int K);
 void ternaspmm_repack(const uint64_t* bitmap, const int* tile_offsets_global, const uint16_t* tile_offsets_median,
                       const uint32_t* sign_words, void* packed, int N, int K, terna_stream stream);
 
-/* bf16-activation linear on a P2 buffer.  route: 0 = pick by M, 1 = MFMA-tiled kernel, 2 = small-M kernel. */
+/* bf16-activation linear on a P2 buffer.  route: 0 = the library picks the kernel (by measurement: the small-M kernel up
+ * to 32 rows for matrices of more than 512 bands, up to 64 - 256 rows otherwise, depending on K, the activation type
+ * and whether scratch memory for split-K is at hand), 1 = MFMA-tiled kernel, 2 = small-M kernel. */
 void bitlinear_TernaSpMM_bf16_packed(const terna_bf16* x, const void* packed, terna_bf16* out, const float* scale,
                                      int ws_num, int M, int N, int K, int route, terna_stream stream);
 
 /* int8-activation linear on a P2 buffer; arguments as bitlinear_TernaSpMM.  route: 0 = the reference's
- * rule (decode epilogue for M <= 64, prefill epilogue above), 1 = prefill epilogue, 2 = decode epilogue. */
+ * rule (decode epilogue for M <= 64, prefill epilogue above), 1 = prefill epilogue, 2 = decode epilogue.  Which kernel
+ * computes the sums is the library's choice (as above) and does not change the result: integer sums are exact. */
 void bitlinear_TernaSpMM_packed(const int8_t* x, const void* packed, terna_bf16* out, const terna_bf16* s,
                                 const terna_bf16* ws, int ws_num, int M, int N, int K, int route, terna_stream stream);
+
+/* The two entry points above with scratch memory the library may use (may be NULL / 0: then they are the calls
+ * above): `workspace` (16-byte aligned, workspace_bytes long) receives split-K partial sums when a large-M call has
+ * few output tiles for the chip -- 4 * M * N bytes per split, up to 8 splits; the call then enqueues two launches
+ * (partial products, then the sum in split order + epilogue; int8 results stay bit-exact).  Nothing has to be
+ * preserved or initialised in it between calls; calls that share it must not overlap.
+ * Kernel override for measurements: bitlinear_TernaSpMM_packed(_ws) also accepts route + 4 (small-M kernel at any M)
+ * and route + 8 (MFMA-tiled kernel at any M); the low two bits keep selecting the epilogue rule. */
+void bitlinear_TernaSpMM_bf16_packed_ws(const terna_bf16* x, const void* packed, terna_bf16* out, const float* scale,
+                                        int ws_num, int M, int N, int K, int route, void* workspace,
+                                        long long workspace_bytes, terna_stream stream);
+void bitlinear_TernaSpMM_packed_ws(const int8_t* x, const void* packed, terna_bf16* out, const terna_bf16* s,
+                                   const terna_bf16* ws, int ws_num, int M, int N, int K, int route, void* workspace,
+                                   long long workspace_bytes, terna_stream stream);
 
 /* ---- Fused prologue of a ternary linear (no counterpart in the reference's library) -----------------
  * One launch replaces the PyTorch / xformers / Inductor kernels the reference runs between two bitlinear
@@ -281,6 +298,26 @@ void ternaspmm_argmax_bf16(const terna_bf16* x, long long* out, int B, int V, te
  * cache trusts the pointers: after freeing or rewriting weight tensors call this function, which releases every
  * cached copy. */
 void ternaspmm_repack_cache_clear(void);
+
+/* ---- Calibration probes (no counterpart in the reference) ------------------------------------------------------
+ * What the machine gives, measured by the same library in the same run as the kernels a benchmark prices:
+ *   ternaspmm_probe_empty    enqueues an empty kernel (one wave): N of them in a captured graph, replayed, give the
+ *                            cost of one graph kernel node -- the floor under every launch of a decode step;
+ *   ternaspmm_probe_read     streams `bytes` (16-byte aligned) through the chip and discards them: the read rate;
+ *                            `sink` (16 bytes, may be NULL) is written practically never;
+ *   ternaspmm_probe_copy     dst <- src, `bytes` each: the read + write rate;
+ *   ternaspmm_probe_barrier  `rounds` device-wide synchronisations among `workgroups` co-resident workgroups (at most
+ *                            one per CU, at most 256) through flags in `state` (ternaspmm_probe_barrier_state_bytes()
+ *                            bytes, 16-byte aligned, zero-filled once; pass first_tag = 1 + the rounds run on it so
+ *                            far): what a persistent kernel would pay between two dependent phases.  Every wait is
+ *                            bounded; uint32 word 512 of `state` counts workgroups that gave up (0 after a good run).
+ *                            Returns 0, or -1 when the arguments are refused.
+ * All only enqueue; time them with events on `stream`. */
+void ternaspmm_probe_empty(terna_stream stream);
+void ternaspmm_probe_read(const void* src, long long bytes, void* sink, terna_stream stream);
+void ternaspmm_probe_copy(const void* src, void* dst, long long bytes, terna_stream stream);
+size_t ternaspmm_probe_barrier_state_bytes(void);
+int ternaspmm_probe_barrier(void* state, int workgroups, int rounds, unsigned first_tag, terna_stream stream);
 
 /* Library version string, e.g. "ternaspmm-gfx950 0.1". */
 const char* ternaspmm_version(void);

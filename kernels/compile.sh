@@ -27,6 +27,7 @@ compile launch_prefill_packed.hip launch_prefill_packed_bf16.o -DTERNA_PREFILL_A
 compile abi_fused.hip abi_fused.o
 compile abi_attention.hip abi_attention.o
 compile abi_head.hip abi_head.o
+compile abi_probe.hip abi_probe.o
 compile format_host.cpp format_host.o
 for p in "${pids[@]}"; do wait "$p"; done
 

@@ -38,6 +38,8 @@ PROTOTYPES = {
     "ternaspmm_repack": ([_vp, _vp, _vp, _vp, _vp, _ci, _ci, _vp], None),
     "bitlinear_TernaSpMM_bf16_packed": ([_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp], None),
     "bitlinear_TernaSpMM_packed": ([_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp], None),
+    "bitlinear_TernaSpMM_bf16_packed_ws": ([_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, ctypes.c_longlong, _vp], None),
+    "bitlinear_TernaSpMM_packed_ws": ([_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, ctypes.c_longlong, _vp], None),
     "ternaspmm_rmsnorm_quant": ([_vp, _vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _ci, _ci, _vp], None),
     "ternaspmm_relu2_mul_rmsnorm_quant": ([_vp, _vp, ctypes.c_float, _vp, _vp, _vp, _ci, _ci, _vp], None),
     "bitlinear_TernaSpMM_packed_fused": ([_vp, _vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _ci, _vp, _vp, _ci, _ci, _ci, _vp],
@@ -54,6 +56,11 @@ PROTOTYPES = {
     "ternaspmm_decode_attention": ([_vp] * 5 + [_ci] * 5 + [ctypes.c_float, _vp, _vp], None),
     "ternaspmm_decode_attention_static": ([_vp] * 5 + [_ci] * 5 + [ctypes.c_float, _vp], ctypes.c_int),
     "ternaspmm_attention_workspace_bytes": ([_ci, _ci, _ci], ctypes.c_longlong),
+    "ternaspmm_probe_empty": ([_vp], None),
+    "ternaspmm_probe_read": ([_vp, ctypes.c_longlong, _vp, _vp], None),
+    "ternaspmm_probe_copy": ([_vp, _vp, ctypes.c_longlong, _vp], None),
+    "ternaspmm_probe_barrier_state_bytes": ([], ctypes.c_size_t),
+    "ternaspmm_probe_barrier": ([_vp, _ci, _ci, ctypes.c_uint, _vp], ctypes.c_int),
     "ternaspmm_repack_cache_clear": ([], None),
     "ternaspmm_version": ([], ctypes.c_char_p),
 }

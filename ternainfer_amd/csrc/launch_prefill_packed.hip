@@ -23,15 +23,48 @@ void launch_prefill_packed_as(const Act* x, const uint32_t* packed, uint16_t* ou
     kernel<<<grid, dim3(256), S::kBytes, st>>>(x, packed, out, ep, M, N, K);
 }
 
+// Split-K: with few output tiles for the chip (small M x N) every workgroup walks all of K alone and most CUs idle.
+// Given scratch memory the K steps are spread over `splits` workgroups per tile, each leaves a plane of raw partial sums
+// ([splits][M][N] fp32 / int32) and a second launch adds the planes in split order and applies the epilogue (the int8
+// family stays bit-exact: integer sums; the bf16 family sums in another order, within its tolerance).
+// Rule, from timings of the four BitNet-2B matrices at M = 128 .. 512 with 1 .. 8 splits (a step is 64 columns of bf16
+// or 128 of int8 activations): a split must keep 13 steps or more; up to 96 tiles three splits (six up to 48 tiles);
+// up to 192 tiles three splits if K gives 48 steps or more, else none (the second launch and the partial planes then
+// cost more than the shorter chains save); above that none.  Measured: down projection at M = 256 / 512, bf16
+// 44.5 -> 22.5 us / 44.8 -> 29.3 us, int8 25.1 -> 17.5 / 25.9 -> 21.8; O projection at M = 256, bf16 18.6 -> 14.8.
+// TERNASPMM_PREFILL_SPLITS=1..8 forces a count (tuning aid).
+int prefill_splits(long tiles, int steps, int M, int N, size_t scratch_bytes)
+{
+    static const int forced = [] {
+        const char* v = std::getenv("TERNASPMM_PREFILL_SPLITS");
+        const int n = v ? std::atoi(v) : 0;
+        return n >= 1 && n <= 8 ? n : 0;
+    }();
+    const long fit = static_cast<long>(scratch_bytes / (static_cast<size_t>(M) * N * 4));
+    long sp = 1;
+    if (forced) sp = forced;
+    else if (tiles <= 48) sp = 6;
+    else if (tiles <= 96) sp = 3;
+    else if (tiles <= 192 && steps >= 48) sp = 3;
+    if (!forced && sp > steps / 13) sp = steps / 13;
+    if (sp > steps) sp = steps;
+    if (sp > fit) sp = fit;
+    return sp < 1 ? 1 : static_cast<int>(sp);
+}
+
 template <typename Act, int MB, int NA>
 void launch_prefill_packed_dma_as(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M,
-                                  int N, int K, hipStream_t st)
+                                  int N, int K, void* scratch, size_t scratch_bytes, hipStream_t st)
 {
     using S = PackedPrefillDmaSmem<MB>;
     auto kernel = terna_prefill_packed_dma_kernel<Act, MB, NA>;
     allow_dynamic_lds(kernel, S::kBytes, "hipFuncSetAttribute(prefill packed dma)", __LINE__);
     constexpr int BN = 128 * NA;
-    const dim3 grid((N + BN - 1) / BN, (M + S::BM - 1) / S::BM);
+    dim3 grid((N + BN - 1) / BN, (M + S::BM - 1) / S::BM);
+    const int steps = sizeof(Act) == 1 ? ((K >> 6) + 1) >> 1 : K >> 6;
+    const bool scratch_ok = scratch != nullptr && (reinterpret_cast<uintptr_t>(scratch) & 15) == 0 && (N & 3) == 0;
+    const int splits = scratch_ok ? prefill_splits(static_cast<long>(grid.x) * grid.y, steps, M, N, scratch_bytes) : 1;
+    grid.z = splits;
     static const int xcd_forced = [] {
         const char* v = std::getenv("TERNASPMM_PREFILL_XCD_MAP");
         return v ? std::atoi(v) : -1;
@@ -41,7 +74,13 @@ void launch_prefill_packed_dma_as(const Act* x, const uint32_t* packed, uint16_t
     // TERNASPMM_PREFILL_XCD_MAP=0|1 forces it off / on (tuning aid).
     const bool big_x = static_cast<size_t>(M) * K * sizeof(Act) > (4u << 20);
     const int xcd_map = (grid.y % 8 == 0) && (xcd_forced < 0 ? big_x : xcd_forced != 0);
-    kernel<<<grid, dim3(256), S::kBytes, st>>>(x, packed, out, ep, M, N, K, xcd_map);
+    kernel<<<grid, dim3(256), S::kBytes, st>>>(x, packed, out, ep, M, N, K, xcd_map, splits, splits > 1 ? scratch : nullptr);
+    if (splits > 1) {
+        using AccT = typename std::conditional<sizeof(Act) == 1, int, float>::type;
+        const long quads = static_cast<long>(M) * (N >> 2);
+        terna_splitk_reduce_kernel<AccT><<<dim3(static_cast<unsigned>((quads + 255) / 256)), dim3(256), 0, st>>>(
+            static_cast<const AccT*>(scratch), out, ep, M, N, splits);
+    }
 }
 
 // The direct-to-LDS kernel addresses both operands as a 64-bit base plus a 32-bit byte offset and
@@ -60,7 +99,7 @@ inline bool prefill_dma_ok(const void* x, size_t act_bytes, int M, int N, int K)
 
 template <typename Act>
 void launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
-                           hipStream_t st)
+                           void* scratch, size_t scratch_bytes, hipStream_t st)
 {
     // Batch rows per workgroup (64 / 128 / 256).  Measured on MI355X the 64-row tile wins at every
     // BitNet-2B shape: it runs four waves per SIMD, and occupancy hides more latency than the taller
@@ -82,10 +121,10 @@ void launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, 
     const long wg256 = static_cast<long>((N + 255) / 256) * ((M + 63) / 64);
     const int bn = forced_bn ? forced_bn : (wg256 <= 640 ? 128 : 256);
     if (prefill_dma_ok(x, sizeof(Act), M, N, K) && (bm == 64 || bm == 128)) {
-        if (bm == 64 && bn == 128) launch_prefill_packed_dma_as<Act, 2, 1>(x, packed, out, ep, M, N, K, st);
-        else if (bm == 128 && forced_bn == 128) launch_prefill_packed_dma_as<Act, 4, 1>(x, packed, out, ep, M, N, K, st);
-        else if (bm == 128) launch_prefill_packed_dma_as<Act, 4, 2>(x, packed, out, ep, M, N, K, st);
-        else launch_prefill_packed_dma_as<Act, 2, 2>(x, packed, out, ep, M, N, K, st);
+        if (bm == 64 && bn == 128) launch_prefill_packed_dma_as<Act, 2, 1>(x, packed, out, ep, M, N, K, scratch, scratch_bytes, st);
+        else if (bm == 128 && forced_bn == 128) launch_prefill_packed_dma_as<Act, 4, 1>(x, packed, out, ep, M, N, K, scratch, scratch_bytes, st);
+        else if (bm == 128) launch_prefill_packed_dma_as<Act, 4, 2>(x, packed, out, ep, M, N, K, scratch, scratch_bytes, st);
+        else launch_prefill_packed_dma_as<Act, 2, 2>(x, packed, out, ep, M, N, K, scratch, scratch_bytes, st);
         return;
     }
     if (bm == 64 && bn == 128) launch_prefill_packed_as<Act, 2, 1>(x, packed, out, ep, M, N, K, st);
@@ -96,6 +135,6 @@ void launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, 
 }
 
 template void launch_prefill_packed<TERNA_PREFILL_ACT>(const TERNA_PREFILL_ACT*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int,
-                                                       hipStream_t);
+                                                       void*, size_t, hipStream_t);
 
 }  // namespace terna

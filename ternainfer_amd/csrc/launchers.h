@@ -35,9 +35,11 @@ void launch_repack(const Weights& w, uint32_t* packed, int N, int K, hipStream_t
 template <typename Act>
 void launch_decode_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
                           hipStream_t st);
+// `scratch` (may be NULL; 16-byte aligned, scratch_bytes long): room for split-K partial sums when the shape has few
+// output tiles for the chip; the call then enqueues two launches.
 template <typename Act>
 void launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
-                           hipStream_t st);
+                           void* scratch, size_t scratch_bytes, hipStream_t st);
 
 extern template void launch_decode<int8_t>(const int8_t*, const Weights&, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
 extern template void launch_decode<uint16_t>(const uint16_t*, const Weights&, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
@@ -45,8 +47,10 @@ extern template void launch_prefill<int8_t>(const int8_t*, const Weights&, uint1
 extern template void launch_prefill<uint16_t>(const uint16_t*, const Weights&, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
 extern template void launch_decode_packed<int8_t>(const int8_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
 extern template void launch_decode_packed<uint16_t>(const uint16_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
-extern template void launch_prefill_packed<int8_t>(const int8_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
-extern template void launch_prefill_packed<uint16_t>(const uint16_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
+extern template void launch_prefill_packed<int8_t>(const int8_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, void*, size_t,
+                                                   hipStream_t);
+extern template void launch_prefill_packed<uint16_t>(const uint16_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, void*, size_t,
+                                                     hipStream_t);
 
 // Tuning override shared by the two small-M launchers: TERNASPMM_DECODE_WAVES=4|8|16 forces one variant.
 int decode_waves_override();

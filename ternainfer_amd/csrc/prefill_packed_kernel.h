@@ -145,6 +145,29 @@ __device__ __forceinline__ void packed_prefill_epilogue(AccV (&acc)[NA][MB], uin
     });
 }
 
+// Raw accumulators of one wave into a [M][N] plane of split-K partial sums (same element order as the epilogue).
+template <int MB, int NA, typename AccV, typename AccT>
+__device__ __forceinline__ void packed_prefill_store_partial(AccV (&acc)[NA][MB], AccT* __restrict__ plane, int M, int N,
+                                                             int n_wave, int m0, int lane)
+{
+    typedef AccT V4 __attribute__((ext_vector_type(4)));
+    const int kb = lane >> 5, l32 = lane & 31;
+    static_for<0, NA>([&](auto ac) {
+        constexpr int a = decltype(ac)::value;
+        static_for<0, MB>([&](auto bc) {
+            constexpr int b = decltype(bc)::value;
+            const int m = m0 + 32 * b + l32;
+            static_for<0, 4>([&](auto vc) {
+                constexpr int vq = decltype(vc)::value;
+                const int n = n_wave + 32 * a + 8 * vq + 4 * kb;
+                if (m < M && n < N)
+                    *reinterpret_cast<V4*>(plane + static_cast<size_t>(m) * N + n) =
+                        V4{acc[a][b][4 * vq], acc[a][b][4 * vq + 1], acc[a][b][4 * vq + 2], acc[a][b][4 * vq + 3]};
+            });
+        });
+    });
+}
+
 template <int MB>
 struct PackedPrefillSmem {
     static constexpr int BM = 32 * MB;
@@ -359,7 +382,7 @@ struct PackedPrefillDmaSmem {
 template <typename Act, int MB, int NA>
 __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) void terna_prefill_packed_dma_kernel(
     const Act* __restrict__ x, const uint32_t* __restrict__ packed, uint16_t* __restrict__ out,
-    Epilogue ep, int M, int N, int K, int xcd_map)
+    Epilogue ep, int M, int N, int K, int xcd_map, int splits, void* __restrict__ partial)
 {
     using S = PackedPrefillDmaSmem<MB>;
     constexpr int BN = 128 * NA, BM = S::BM;
@@ -395,6 +418,10 @@ __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) voi
     // int8 with an odd tile count: in the last step the kb = 1 half has no tile.  Its loads are
     // pulled back onto the kb = 0 half's addresses (in bounds) and its weights are zeroed.
     const bool half_tail = I8 && (ktiles & 1);
+    // Split-K (gridDim.z = splits > 1, partial != NULL): this workgroup walks the steps k_begin .. k_end - 1 only and
+    // leaves its raw accumulators in partial[blockIdx.z][M][N]; terna_splitk_reduce_kernel sums the splits in order.
+    const int k_begin = splits > 1 ? static_cast<int>(static_cast<long>(steps) * blockIdx.z / splits) : 0;
+    const int k_end = splits > 1 ? static_cast<int>(static_cast<long>(steps) * (blockIdx.z + 1) / splits) : steps;
     const int last_band = (N >> 4) - 1;
     const int kb = lane >> 5, l32 = lane & 31;
 
@@ -496,22 +523,22 @@ __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) voi
     BOps b_a, b_b;
     int st_mma = 0;                                          // stage of the step being multiplied
     int st_dma = 2 * S::kStage;                              // stage that the next direct load fills
-    issue_x(0, 0);
-    fetch_w(w0, 0);
-    if (steps > 1) {
-        issue_x(1, S::kStage);
-        fetch_w(w1, 1);
+    issue_x(k_begin, 0);
+    fetch_w(w0, k_begin);
+    if (k_end - k_begin > 1) {
+        issue_x(k_begin + 1, S::kStage);
+        fetch_w(w1, k_begin + 1);
         wait_loads_and_barrier<MB + NA>();
     } else {
         wait_loads_and_barrier<0>();
     }
     load_b(0, 0, b_a);
     auto body = [&](int k, RawW& w) {
-        const bool more1 = k + 1 < steps, more2 = k + 2 < steps;        // uniform
+        const bool more1 = k + 1 < k_end, more2 = k + 2 < k_end;        // uniform
         const int st_next = next_stage(st_mma);
 #pragma unroll
         for (int a = 0; a < NA; ++a) landed(w.w[a]);
-        if (half_tail && !more1 && kb) {
+        if (half_tail && k == steps - 1 && kb) {
 #pragma unroll
             for (int a = 0; a < NA; ++a) w.w[a] = u32x4{0u, 0u, 0u, 0u};
         }
@@ -541,14 +568,45 @@ __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) voi
         st_mma = st_next;
         st_dma = next_stage(st_dma);
     };
-    int k = 0;
-    for (; k + 1 < steps; k += 2) {
+    int k = k_begin;
+    for (; k + 1 < k_end; k += 2) {
         body(k, w0);
         body(k + 1, w1);
     }
-    if (k < steps) body(k, w0);
+    if (k < k_end) body(k, w0);
 
+    if (partial != nullptr) {
+        using AccT = typename std::conditional<I8, int, float>::type;
+        packed_prefill_store_partial<MB, NA>(acc, static_cast<AccT*>(partial) + static_cast<size_t>(blockIdx.z) * M * N, M, N,
+                                             n0 + 32 * NA * wave, m0, lane);
+        return;
+    }
     packed_prefill_epilogue<MB, NA>(acc, out, ep, M, N, n0 + 32 * NA * wave, m0, lane);
+}
+
+// Second launch of a split-K call: out[m][n0 .. n0+3] = epilogue(sum over the splits, in split order, of partial[z][m][n]).
+// AccT = int (int8 family: the sum is exact, so the result is that of the unsplit kernel bit for bit) or float (bf16
+// family: weights were +-0.5, the sum is doubled first, as in the unsplit epilogue).  One thread per four columns.
+template <typename AccT>
+__global__ __launch_bounds__(256) void terna_splitk_reduce_kernel(const AccT* __restrict__ partial, uint16_t* __restrict__ out,
+                                                                  Epilogue ep, int M, int N, int splits)
+{
+    typedef AccT V4 __attribute__((ext_vector_type(4)));
+    const int quads = N >> 2;
+    const long idx = static_cast<long>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= static_cast<long>(M) * quads) return;
+    const int m = static_cast<int>(idx / quads), n0 = static_cast<int>(idx - static_cast<long>(m) * quads) * 4;
+    const size_t at = static_cast<size_t>(m) * N + n0, plane = static_cast<size_t>(M) * N;
+    V4 sum = *reinterpret_cast<const V4*>(partial + at);
+    for (int z = 1; z < splits; ++z) sum += *reinterpret_cast<const V4*>(partial + z * plane + at);
+    const EpilogueRegs e = load_epilogue(ep, m, n0, N);
+    uint16_t o[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        if constexpr (std::is_same<AccT, float>::value) o[v] = apply_epilogue<float>(ep.kind, e, v, sum[v] * 2.0f);
+        else o[v] = apply_epilogue<int>(ep.kind, e, v, sum[v]);
+    }
+    *reinterpret_cast<u32x2*>(out + at) = u32x2{o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16)};
 }
 
 }  // namespace terna

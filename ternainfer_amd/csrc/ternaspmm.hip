@@ -21,6 +21,10 @@ namespace {
 // Large-M call on reference-format pointers: with a 16-byte aligned workspace of N*K/4 bytes the
 // weights are first transcoded to P2 there (one cheap pass) and the P2 kernel does the GEMM;
 // without one the fused reference-format kernel runs.
+//
+// The reference's call site guarantees N*K bytes of workspace on this path (model.py:34-42: the dense int8 copy of the
+// matrix its prefill path writes there); the transcoded weights take the first quarter, and what follows may hold
+// split-K partial sums when the shape has few output tiles for the chip.
 template <typename Act>
 void launch_large_m(const Act* x, const Weights& w, uint16_t* out, const Epilogue& ep, int M, int N, int K,
                     void* workspace, hipStream_t st)
@@ -28,13 +32,34 @@ void launch_large_m(const Act* x, const Weights& w, uint16_t* out, const Epilogu
     if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
         uint32_t* packed = static_cast<uint32_t*>(workspace);
         launch_repack(w, packed, N, K, st);
-        launch_prefill_packed(x, packed, out, ep, M, N, K, st);
+        const size_t p2_bytes = (static_cast<size_t>(N) * K / 4 + 255) & ~static_cast<size_t>(255);
+        launch_prefill_packed(x, packed, out, ep, M, N, K, static_cast<char*>(workspace) + p2_bytes,
+                              static_cast<size_t>(N) * K - p2_bytes, st);
     } else {
         launch_prefill(x, w, out, ep, M, N, K, st);
     }
 }
 
 enum Route { ROUTE_AUTO, ROUTE_DECODE, ROUTE_PREFILL };
+
+// Which P2 kernel runs a call of M rows when the caller leaves the choice to the library: the small-M dot-product
+// kernel or the MFMA-tiled one.  (The epilogue arithmetic of the int8 family follows the reference's M <= 64 rule
+// whatever kernel computes the sums.)
+// By measurement on the four BitNet-2B matrices at M = 16 .. 256 (us per launch, P2 layout, small-M kernel / MFMA-tiled
+// kernel with split-K scratch): the small-M kernel's time grows with every 16 rows, the MFMA-tiled one is flat but
+// pays a fill / drain of 10 us or more.
+//   gate+up (864 bands)  bf16 M=32 11.8 / 16.9   M=48 23.5 / 17.6      int8 M=32  8.4 / 11.3   M=48 12.8 / 12.2
+//   QKV (240 bands)      bf16 M=64  8.1 / 11.6   M=96 13.5 / 12.6      int8 M=128 8.7 / 11.4   M=192 11.6 / 11.5
+//   down (K = 6912)      bf16 M=64 14.0 / 14.1   M=96 24.7 / 15.4      int8 M=64  9.5 / 12.5   M=96 14.6 / 13.3
+// Without scratch the MFMA-tiled kernel cannot split K and walks all of it in every workgroup (QKV bf16 16-17 us flat,
+// down 38-44 us), which moves the cut up.
+bool packed_small_kernel(int M, int N, int K, bool int8, bool has_scratch)
+{
+    if (N / 16 > 512) return M <= 32;
+    if (!has_scratch) return M <= (K > 4096 ? 256 : 128);
+    if (int8 && K <= 4096) return M <= 128;
+    return M <= 64;
+}
 
 // ---- opt-in repack cache behind the reference-format entry points (TERNASPMM_REPACK_CACHE=1).
 // An unmodified call site keeps passing the four format tensors; the first call that sees a weight
@@ -105,8 +130,8 @@ void run_i8(Route route, int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* m
     const Epilogue ep{s, ws, nullptr, ws_num, decode_rule ? EP_I8_DECODE : EP_I8_PREFILL};
     const Weights w{bitmap, tile_off, median_off, sign_words};
     if (const uint32_t* p2 = cached_packed(w, N, K, st)) {
-        if (M <= 64) launch_decode_packed<int8_t>(x, p2, out, ep, M, N, K, st);
-        else launch_prefill_packed<int8_t>(x, p2, out, ep, M, N, K, st);
+        if (packed_small_kernel(M, N, K, true, workspace != nullptr)) launch_decode_packed<int8_t>(x, p2, out, ep, M, N, K, st);
+        else launch_prefill_packed<int8_t>(x, p2, out, ep, M, N, K, workspace, workspace ? static_cast<size_t>(N) * K : 0, st);
     } else if (M <= 64) launch_decode<int8_t>(x, w, out, ep, M, N, K, st);
     else launch_large_m<int8_t>(x, w, out, ep, M, N, K, workspace, st);
     const hipError_t e = hipGetLastError();
@@ -122,8 +147,9 @@ void run_bf16(Route route, const uint16_t* x, const uint64_t* bitmap, const int*
     const Weights w{bitmap, tile_off, median_off, sign_words};
     const bool small = route == ROUTE_DECODE || (route == ROUTE_AUTO && M <= 64);
     if (const uint32_t* p2 = cached_packed(w, N, K, st)) {
-        if (small) launch_decode_packed<uint16_t>(x, p2, out, ep, M, N, K, st);
-        else launch_prefill_packed<uint16_t>(x, p2, out, ep, M, N, K, st);
+        const bool small_p2 = route == ROUTE_DECODE || (route == ROUTE_AUTO && packed_small_kernel(M, N, K, false, workspace != nullptr));
+        if (small_p2) launch_decode_packed<uint16_t>(x, p2, out, ep, M, N, K, st);
+        else launch_prefill_packed<uint16_t>(x, p2, out, ep, M, N, K, workspace, workspace ? static_cast<size_t>(N) * K : 0, st);
     } else if (small) launch_decode<uint16_t>(x, w, out, ep, M, N, K, st);
     else launch_large_m<uint16_t>(x, w, out, ep, M, N, K, workspace, st);
     const hipError_t e = hipGetLastError();
@@ -305,32 +331,48 @@ void ternaspmm_repack(const uint64_t* bitmap, const int* tile_off, const uint16_
     if (e != hipSuccess) die("ternaspmm_repack", e, __LINE__);
 }
 
-void bitlinear_TernaSpMM_bf16_packed(const terna_bf16* x, const void* packed, terna_bf16* out, const float* scale,
-                                     int ws_num, int M, int N, int K, int route, terna_stream stream)
+void bitlinear_TernaSpMM_bf16_packed_ws(const terna_bf16* x, const void* packed, terna_bf16* out, const float* scale,
+                                        int ws_num, int M, int N, int K, int route, void* workspace,
+                                        long long workspace_bytes, terna_stream stream)
 {
     if (!shape_ok(M, N, K) || !groups_ok(ws_num)) return;
     const Epilogue ep{nullptr, nullptr, scale, ws_num, EP_BF16};
     const uint32_t* p = static_cast<const uint32_t*>(packed);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const bool small = route == 2 || (route != 1 && M <= 64);
+    const bool small = route == 2 || (route != 1 && packed_small_kernel(M, N, K, false, workspace != nullptr && workspace_bytes > 0));
     if (small) launch_decode_packed<uint16_t>(x, p, out, ep, M, N, K, st);
-    else launch_prefill_packed<uint16_t>(x, p, out, ep, M, N, K, st);
+    else launch_prefill_packed<uint16_t>(x, p, out, ep, M, N, K, workspace, workspace_bytes > 0 ? static_cast<size_t>(workspace_bytes) : 0, st);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("bitlinear_TernaSpMM_bf16_packed", e, __LINE__);
+}
+
+void bitlinear_TernaSpMM_bf16_packed(const terna_bf16* x, const void* packed, terna_bf16* out, const float* scale,
+                                     int ws_num, int M, int N, int K, int route, terna_stream stream)
+{
+    bitlinear_TernaSpMM_bf16_packed_ws(x, packed, out, scale, ws_num, M, N, K, route, nullptr, 0, stream);
+}
+
+void bitlinear_TernaSpMM_packed_ws(const int8_t* x, const void* packed, terna_bf16* out, const terna_bf16* s,
+                                   const terna_bf16* ws, int ws_num, int M, int N, int K, int route, void* workspace,
+                                   long long workspace_bytes, terna_stream stream)
+{
+    if (!shape_ok(M, N, K) || !groups_ok(ws_num)) return;
+    const int rule = route & 3, kernel = route & 12;
+    const bool decode_rule = rule == 2 || (rule != 1 && M <= 64);
+    const Epilogue ep{s, ws, nullptr, ws_num, decode_rule ? EP_I8_DECODE : EP_I8_PREFILL};
+    const uint32_t* p = static_cast<const uint32_t*>(packed);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool small = kernel == 4 || (kernel != 8 && packed_small_kernel(M, N, K, true, workspace != nullptr && workspace_bytes > 0));
+    if (small) launch_decode_packed<int8_t>(x, p, out, ep, M, N, K, st);
+    else launch_prefill_packed<int8_t>(x, p, out, ep, M, N, K, workspace, workspace_bytes > 0 ? static_cast<size_t>(workspace_bytes) : 0, st);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("bitlinear_TernaSpMM_packed", e, __LINE__);
 }
 
 void bitlinear_TernaSpMM_packed(const int8_t* x, const void* packed, terna_bf16* out, const terna_bf16* s,
                                 const terna_bf16* ws, int ws_num, int M, int N, int K, int route, terna_stream stream)
 {
-    if (!shape_ok(M, N, K) || !groups_ok(ws_num)) return;
-    const bool decode_rule = route == 2 || (route != 1 && M <= 64);
-    const Epilogue ep{s, ws, nullptr, ws_num, decode_rule ? EP_I8_DECODE : EP_I8_PREFILL};
-    const uint32_t* p = static_cast<const uint32_t*>(packed);
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    if (M <= 64) launch_decode_packed<int8_t>(x, p, out, ep, M, N, K, st);
-    else launch_prefill_packed<int8_t>(x, p, out, ep, M, N, K, st);
-    const hipError_t e = hipGetLastError();
-    if (e != hipSuccess) die("bitlinear_TernaSpMM_packed", e, __LINE__);
+    bitlinear_TernaSpMM_packed_ws(x, packed, out, s, ws, ws_num, M, N, K, route, nullptr, 0, stream);
 }
 
 void ternaspmm_repack_cache_clear(void)

@@ -117,8 +117,10 @@ def TernaInfer_linear_packed(input, packed, s, ws, ws_num, out_features):
     M = x.shape[0]
     out = torch.empty((M, out_features), dtype=torch.bfloat16, device=input.device)
     stream = torch.cuda.current_stream()
-    lib.bitlinear_TernaSpMM_packed(_p(x), _p(packed), _p(out), _p(s.reshape(M).contiguous()), _p(ws), ws_num,
-                                   M, out_features, K, 0, ctypes.c_void_p(stream.cuda_stream))
+    work = get_global_workspace(input.device) if M > 64 else None      # large M: room for split-K partial sums
+    lib.bitlinear_TernaSpMM_packed_ws(_p(x), _p(packed), _p(out), _p(s.reshape(M).contiguous()), _p(ws), ws_num,
+                                      M, out_features, K, 0, _p(work) if work is not None else None,
+                                      work.numel() if work is not None else 0, ctypes.c_void_p(stream.cuda_stream))
     return out.reshape(*out_shape)
 
 

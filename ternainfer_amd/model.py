@@ -21,7 +21,7 @@ import torch
 from torch.nn import functional as F
 
 from . import _lib
-from .linear import (argmax_rows, greedy_step, greedy_step_state, lm_head, quant_input, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant,
+from .linear import (argmax_rows, get_global_workspace, greedy_step, greedy_step_state, lm_head, quant_input, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant,
                      repack_weight, rmsnorm_linear_packed, rmsnorm_quant)
 
 
@@ -77,8 +77,9 @@ class TernaryLinear:
         m = xq.shape[0]
         out = torch.empty((m, self.n), dtype=torch.bfloat16, device=xq.device)
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-        self.lib.bitlinear_TernaSpMM_packed(_p(xq), _p(self.packed), _p(out), _p(s), _p(self.ws), self.ws_num,
-                                            m, self.n, self.k, 0, stream)
+        work = get_global_workspace(xq.device) if m > 64 else None              # large M: room for split-K partial sums
+        self.lib.bitlinear_TernaSpMM_packed_ws(_p(xq), _p(self.packed), _p(out), _p(s), _p(self.ws), self.ws_num,
+                                               m, self.n, self.k, 0, _p(work), work.numel() if work is not None else 0, stream)
         return out
 
     def dense(self, x: torch.Tensor) -> torch.Tensor:
@@ -86,8 +87,10 @@ class TernaryLinear:
         m = x.shape[0]
         out = torch.empty((m, self.n), dtype=torch.bfloat16, device=x.device)
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-        self.lib.bitlinear_TernaSpMM_bf16_packed(_p(x.contiguous()), _p(self.packed), _p(out), _p(self.scale_f32),
-                                                 self.ws_num, m, self.n, self.k, 0, stream)
+        work = get_global_workspace(x.device) if m > 64 else None
+        self.lib.bitlinear_TernaSpMM_bf16_packed_ws(_p(x.contiguous()), _p(self.packed), _p(out), _p(self.scale_f32),
+                                                    self.ws_num, m, self.n, self.k, 0, _p(work),
+                                                    work.numel() if work is not None else 0, stream)
         return out
 
     def __call__(self, x: torch.Tensor) -> torch.Tensor:

@@ -27,6 +27,19 @@ def main() -> int:
         x = make_bf16_activations(m, k, 902 + m, outlier_frac=0.01)
         scale = np.array([0.7], np.float32)
         _check_bf16(run_bf16_packed(lib, packed, n, x, scale, 1, 1), co.spmm_bf16(x, w, scale, 1))
+    # split-K of the MFMA-tiled kernel with scratch memory (TERNASPMM_PREFILL_SPLITS forces the split count)
+    from tests.test_gpu_parity import _run_packed_ws
+    for m, n, k in [(100, 256, 2048), (300, 384, 832)]:
+        w = make_ternary(n, k, 0.40, 905 + m + n)
+        packed = repack(lib, DeviceFormat(w))
+        work = torch.empty(8 * m * n * 4, dtype=torch.int8, device="cuda")
+        xq, s = make_int8_activations(m, k, 906 + m)
+        if not (_run_packed_ws(lib, "int8", packed, n, xq, s, WS, 2, 8, work) == O.spmm_i8(xq, w, s, WS, 2, 1)).all():
+            print("int8 split-K mismatch", m, n, k)
+            return 1
+        x = make_bf16_activations(m, k, 907 + m, outlier_frac=0.01)
+        scale = np.array([0.7, 1.1], np.float32)
+        _check_bf16(_run_packed_ws(lib, "bf16", packed, n, x, None, scale, 2, 1, work), co.spmm_bf16(x, w, scale, 2))
     from tests.test_gpu_parity import run_bf16, run_i8
     for m, n, k in [(8, 320, 192), (16, 256, 64), (1, 8256, 128)]:      # small-M kernels, both layouts
         w = make_ternary(n, k, 0.40, 910 + m + n)

@@ -427,6 +427,74 @@ def test_packed_bf16_2b_layer_shapes_m512(lib, n, k):
     _check_bf16(got[:, cols], ref)
 
 
+def _run_packed_ws(lib, act, packed, n, x_or_q, s_bits, scale_or_ws, ws_num, route, work):
+    m, k = x_or_q.shape
+    out = torch.full((m, n), -1, dtype=torch.int16, device="cuda")
+    nbytes = work.numel() if work is not None else 0
+    print(f"[case] packed_ws {act} M={m} N={n} K={k} route={route} workspace={nbytes}", flush=True)
+    if act == "int8":
+        x, sd = torch.from_numpy(x_or_q).cuda(), torch.from_numpy(s_bits.view(np.int16)).cuda()
+        wsd = torch.from_numpy(scale_or_ws.view(np.int16)).cuda()
+        lib.bitlinear_TernaSpMM_packed_ws(vp(x), vp(packed), vp(out), vp(sd), vp(wsd), ws_num, m, n, k, route,
+                                          vp(work) if work is not None else None, nbytes, _stream())
+    else:
+        x, sc = torch.from_numpy(x_or_q.view(np.int16)).cuda(), torch.from_numpy(scale_or_ws).cuda()
+        lib.bitlinear_TernaSpMM_bf16_packed_ws(vp(x), vp(packed), vp(out), vp(sc), ws_num, m, n, k, route,
+                                               vp(work) if work is not None else None, nbytes, _stream())
+    torch.cuda.synchronize()
+    return out.cpu().numpy().view(np.uint16)
+
+
+@pytest.mark.parametrize("m,n,k,ws_num", [(100, 256, 2048, 2), (128, 128, 6400, 1), (300, 384, 1536, 3),
+                                          (256, 2560, 6912, 1), (512, 2560, 6912, 1), (256, 3840, 2560, 3), (192, 2560, 2560, 1)])
+def test_packed_split_k_with_workspace(lib, m, n, k, ws_num):
+    """Few output tiles for the chip + scratch memory: the K steps are spread over several workgroups per tile and a
+    second launch sums the partial planes in split order.  int8: bit-exact against the integer oracle (and hence
+    identical to the unsplit call); bf16: within the family's tolerance.  A workspace too small for one plane, or
+    none, must fall back to the single launch."""
+    w = make_ternary(n, k, 0.40, 460 + m + n % 97)
+    packed = repack(lib, DeviceFormat(w))
+    work = torch.full((8 * m * n * 4 + 64,), 0x55, dtype=torch.int8, device="cuda")[16:]     # 16-byte aligned, poisoned
+    cols = np.sort(np.random.default_rng(461 + m + n).permutation(n)[:256]) if n > 256 else np.arange(n)
+    xq, s = make_int8_activations(m, k, 462 + m)
+    s = s.copy()
+    s[m // 2] = 0
+    want = O.spmm_i8(xq, w, s, WS, ws_num, 1, cols=cols)
+    split = _run_packed_ws(lib, "int8", packed, n, xq, s, WS, ws_num, 8, work)          # MFMA kernel, reference's rule by M
+    assert (split[:, cols] == want).all()
+    plain = _run_packed_ws(lib, "int8", packed, n, xq, s, WS, ws_num, 8, None)
+    assert (plain == split).all()
+    tiny = _run_packed_ws(lib, "int8", packed, n, xq, s, WS, ws_num, 8, work[:m * n * 4 - 16])
+    assert (tiny == split).all()
+    x = make_bf16_activations(m, k, 463 + m, outlier_frac=0.01)
+    scale = np.array([0.7, 1.9, 1.3], np.float32)
+    ref = O.bf16_bits_to_f32(x).astype(np.float64) @ w[cols].astype(np.float64).T * \
+        scale[O.ws_group_decode(cols, n, ws_num)].astype(np.float64)[None, :]
+    _check_bf16(_run_packed_ws(lib, "bf16", packed, n, x, None, scale, ws_num, 1, work)[:, cols], ref)
+    _check_bf16(_run_packed_ws(lib, "bf16", packed, n, x, None, scale, ws_num, 1, None)[:, cols], ref)
+
+
+@pytest.mark.parametrize("with_ws", [False, True])
+@pytest.mark.parametrize("m", [32, 33, 48, 64, 65, 96, 128, 129, 200, 256, 257])
+@pytest.mark.parametrize("n,k,ws_num", [(8256, 192, 1), (3840, 128, 3), (256, 4160, 2)])
+def test_packed_kernel_choice_boundaries(lib, m, n, k, ws_num, with_ws):
+    """The library picks the small-M or the MFMA-tiled kernel by shape (more than 512 bands: up to 32 rows; long K,
+    int8, scratch at hand: other cuts); whatever it picks, int8 results follow the reference's M <= 64 epilogue rule
+    bit for bit and bf16 results stay within tolerance, on both sides of every cut."""
+    w = make_ternary(n, k, 0.40, 470 + n % 89)
+    packed = repack(lib, DeviceFormat(w))
+    work = torch.empty(8 * m * n * 4, dtype=torch.int8, device="cuda") if with_ws else None
+    xq, s = make_int8_activations(m, k, 471 + m)
+    cols = np.sort(np.random.default_rng(472 + n).permutation(n)[:512])
+    got = _run_packed_ws(lib, "int8", packed, n, xq, s, WS, ws_num, 0, work)
+    assert (got[:, cols] == O.spmm_i8(xq, w, s, WS, ws_num, 0 if m <= 64 else 1, cols=cols)).all()
+    x = make_bf16_activations(m, k, 473 + m)
+    scale = np.array([0.7, 1.9, 1.3], np.float32)
+    ref = O.bf16_bits_to_f32(x).astype(np.float64) @ w[cols].astype(np.float64).T * \
+        scale[O.ws_group_decode(cols, n, ws_num)].astype(np.float64)[None, :]
+    _check_bf16(_run_packed_ws(lib, "bf16", packed, n, x, None, scale, ws_num, 0, work)[:, cols], ref)
+
+
 # ------------------------------------------------------------------------------- P2 layout (load-time repack)
 @pytest.mark.parametrize("kind", ["iid40", "skewed", "dense", "empty", "sparse97"])
 def test_repack_is_bit_exact(lib, kind):
@@ -569,7 +637,8 @@ def test_kernel_binary_reference_command_line():
                                  {"TERNASPMM_DECODE_BANDS": "1"}, {"TERNASPMM_FUSED_BANDS": "1"},
                                  {"TERNASPMM_FUSED_BANDS_WAVES": "16"}, {"TERNASPMM_FUSED_WAVES": "8"}, {"TERNASPMM_FUSED_WAVES": "16"},
                                  {"TERNASPMM_ATTN_WAVES": "4"}, {"TERNASPMM_ATTN_SPLITS": "2"}, {"TERNASPMM_ATTN_SPLITS": "8"},
-                                 {"TERNASPMM_ATTN_XCD_GROUPS": "0"}])
+                                 {"TERNASPMM_ATTN_XCD_GROUPS": "0"}, {"TERNASPMM_PREFILL_SPLITS": "1"},
+                                 {"TERNASPMM_PREFILL_SPLITS": "5"}])
 def test_tile_and_path_overrides(env):
     """Every tile shape, launch shape and path behind the library's tuning overrides
     (read once per process, hence a child process): tests/env_variant_check.py must pass under each."""
