@@ -290,14 +290,19 @@ void ternaspmm_lm_head_bf16(const terna_bf16* x, const terna_bf16* w, terna_bf16
  * x[b][0 .. V-1] (bf16 [B][V]; out int64 [B]); ties go to the lowest index, NaN never wins.  Only enqueues. */
 void ternaspmm_argmax_bf16(const terna_bf16* x, long long* out, int B, int V, terna_stream stream);
 
-/* Opt-in repack cache for unmodified call sites: with TERNASPMM_REPACK_CACHE=1 in the environment the
- * reference-format entry points above (bitlinear_TernaSpMM*, bitlinear_TernaSpMM_bf16*) keep a device-side P2
- * copy (N*K/4 bytes) of every weight they have seen -- keyed by device, the bitmap / sign / offset pointers and
- * the shape -- and run the P2 kernels from the second sight on; the first sight allocates, repacks and waits
- * (during stream capture, where nothing may be allocated, it runs the reference-format kernels instead).  The
- * cache trusts the pointers: after freeing or rewriting weight tensors call this function, which releases every
- * cached copy. */
+/* Repack cache for unmodified call sites (on unless TERNASPMM_REPACK_CACHE=0 is in the environment): the
+ * reference-format entry points above (bitlinear_TernaSpMM*, bitlinear_TernaSpMM_bf16*) keep a device-side P2 copy
+ * (N*K/4 bytes) of every weight they have seen -- keyed by device, the bitmap / sign / offset pointers and the shape
+ * -- and run the P2 kernels from the second sight on; the first sight allocates, repacks and waits (during stream
+ * capture, where nothing may be allocated, it runs the reference-format kernels instead: warm up once before
+ * capturing, as generate.py:121-129 does).  Every launch on a cached copy re-checks a fingerprint of the caller's
+ * tensors (2.5 KB sampled from the bitmap and sign arrays + the sign-bit total) against the one recorded with the
+ * copy; when weights were freed or rewritten and other data sits at the same addresses, the next call into the
+ * library prints the reason and exits the process.  Call ternaspmm_repack_cache_clear() after freeing or reloading
+ * weights: it releases every cached copy.  ternaspmm_repack_cache_enable(0 / 1) switches the cache off / on at run
+ * time and returns the previous setting (copies already made are kept until cleared). */
 void ternaspmm_repack_cache_clear(void);
+int ternaspmm_repack_cache_enable(int on);
 
 /* ---- Calibration probes (no counterpart in the reference) ------------------------------------------------------
  * What the machine gives, measured by the same library in the same run as the kernels a benchmark prices:

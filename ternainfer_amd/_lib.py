@@ -62,6 +62,7 @@ PROTOTYPES = {
     "ternaspmm_probe_barrier_state_bytes": ([], ctypes.c_size_t),
     "ternaspmm_probe_barrier": ([_vp, _ci, _ci, ctypes.c_uint, _vp], ctypes.c_int),
     "ternaspmm_repack_cache_clear": ([], None),
+    "ternaspmm_repack_cache_enable": ([_ci], _ci),
     "ternaspmm_version": ([], ctypes.c_char_p),
 }
 

@@ -25,7 +25,7 @@ __global__ void terna_fill_u32_kernel(uint32_t* p, uint32_t v) { p[blockIdx.x * 
 int attention_waves(int B, int H)
 {
     static const int forced = [] {
-        const char* v = std::getenv("TERNASPMM_ATTN_WAVES");
+        const char* v = tuning_env("TERNASPMM_ATTN_WAVES");
         const int w = v ? std::atoi(v) : 0;
         return (w == 4 || w == 8) ? w : 0;
     }();
@@ -38,7 +38,7 @@ int attention_waves(int B, int H)
 bool attention_groups_on(int H, int KV)
 {
     static const int on = [] {
-        const char* v = std::getenv("TERNASPMM_ATTN_XCD_GROUPS");
+        const char* v = tuning_env("TERNASPMM_ATTN_XCD_GROUPS");
         return v ? std::atoi(v) : 1;
     }();
     return on && H > KV;
@@ -75,7 +75,7 @@ int attention_splits(int B, int H, int S, const AttentionScratch& scratch)
 {
     if (scratch.arrived == nullptr) return 1;
     static const int forced = [] {
-        const char* v = std::getenv("TERNASPMM_ATTN_SPLITS");
+        const char* v = tuning_env("TERNASPMM_ATTN_SPLITS");
         const int n = v ? std::atoi(v) : 0;
         return (n == 1 || n == 2 || n == 4 || n == 8) ? n : 0;
     }();
@@ -269,7 +269,7 @@ void ternaspmm_rope_decode_attention_prefetch(const terna_bf16* qkv, const float
     }
     // the heads take B*H CUs; the rest of the chip prefetches
     static const int forced_wgs = [] {
-        const char* v = std::getenv("TERNASPMM_ATTN_PREFETCH_WGS");
+        const char* v = tuning_env("TERNASPMM_ATTN_PREFETCH_WGS");
         return v ? std::atoi(v) / 8 * 8 : -1;
     }();
     const int slots = attention_slots(B, H, KV);

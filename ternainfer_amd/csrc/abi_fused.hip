@@ -51,7 +51,7 @@ static int launch_decode_fused(int mode, const terna_bf16* x, const terna_bf16* 
     const int ktiles = K / 64;
     const int bands = N / 16;
     static const int forced_waves = [] {
-        const char* v = std::getenv("TERNASPMM_FUSED_WAVES");
+        const char* v = tuning_env("TERNASPMM_FUSED_WAVES");
         return v ? std::atoi(v) : 0;
     }();
     // 8 waves of up to 5 band-tiles where K allows (measured: +2 % tokens/s over 16 waves of 3 once the weight loads
@@ -62,11 +62,11 @@ static int launch_decode_fused(int mode, const terna_bf16* x, const terna_bf16* 
     // per CU.  TERNASPMM_FUSED_BANDS=1 switches that off, TERNASPMM_FUSED_BANDS_WAVES=16 picks the 16-wave
     // variant of it (tuning aids).
     static const int forced_nb = [] {
-        const char* v = std::getenv("TERNASPMM_FUSED_BANDS");
+        const char* v = tuning_env("TERNASPMM_FUSED_BANDS");
         return v ? std::atoi(v) : 0;
     }();
     static const int nb_waves = [] {
-        const char* v = std::getenv("TERNASPMM_FUSED_BANDS_WAVES");
+        const char* v = tuning_env("TERNASPMM_FUSED_BANDS_WAVES");
         return v && std::atoi(v) == 16 ? 16 : 8;
     }();
     const bool multi = forced_nb != 1 && bands > 256 && bands % 4 == 0 && mode != FUSED_GLU;

@@ -58,13 +58,13 @@ void ternaspmm_lm_head_bf16(const terna_bf16* x, const terna_bf16* w, terna_bf16
     const int blocks = (V + 15) / 16;
     const int wgs_needed = (blocks + kLmWaves - 1) / kLmWaves;
     static const int forced = [] {
-        const char* v = std::getenv("TERNASPMM_LM_HEAD_WGS");
+        const char* v = tuning_env("TERNASPMM_LM_HEAD_WGS");
         return v ? std::atoi(v) : 0;
     }();
     const int cap = forced > 0 ? forced : 512;               // two workgroups per CU measure fastest (256: 137 us, 512: 115 us, 1024: 119 us on 657 MB)
     const int grid = wgs_needed < cap ? wgs_needed : cap;
     static const int quad = [] {
-        const char* v = std::getenv("TERNASPMM_LM_HEAD_QUAD");
+        const char* v = tuning_env("TERNASPMM_LM_HEAD_QUAD");
         return v ? std::atoi(v) : 1;
     }();
     const int ksteps = K / 128;

@@ -23,11 +23,22 @@ struct PackedRaw {
     u32x4    x[MB][XSlab<Act>::kLoads];      // coalesced pieces of the activation slab
 };
 
-template <typename Act, int WAVES, int MB, int DEPTH, int NB = 1>
+// GUARD: the launch runs on a cached P2 copy and checks it (below).  A variant of its own: the branch at the top costs
+// every workgroup 0.3 us (nothing can start before all arguments are in), which launches on a caller's own P2
+// buffer do not have to pay.
+template <typename Act, int WAVES, int MB, int DEPTH, int NB = 1, bool GUARD = false>
 __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
     const Act* __restrict__ x, const uint32_t* __restrict__ packed, uint16_t* __restrict__ out,
-    Epilogue ep, int M, int N, int K)
+    Epilogue ep, int M, int N, int K, const RepackGuard* __restrict__ guard)
 {
+    // A launch on a cached P2 copy carries one extra workgroup in x -- the one past the last band -- that checks, next to
+    // the others and off their critical path, that the copy still belongs to the caller's tensors.
+    if constexpr (GUARD) {
+        if (static_cast<int>(blockIdx.x) * (16 * NB) >= N) {
+            if (blockIdx.y == 0 && threadIdx.x < 64) repack_guard_role(*guard, threadIdx.x);
+            return;
+        }
+    }
     using T = ActTraits<Act>;
     using Acc = typename T::Acc;
     using Raw = PackedRaw<Act, MB, NB>;

@@ -40,6 +40,18 @@ inline bool groups_ok(int ws_num)
     return true;
 }
 
+// Tuning overrides (TERNASPMM_DECODE_WAVES, TERNASPMM_PREFILL_BM, ...) force one of the kernel variants the library
+// otherwise picks by shape.  They are honoured only when TERNASPMM_TUNING=1 is set as well: a shipped library does not
+// change kernels because a variable of that name happens to be in the environment.
+inline const char* tuning_env(const char* name)
+{
+    static const bool on = [] {
+        const char* v = std::getenv("TERNASPMM_TUNING");
+        return v != nullptr && std::atoi(v) == 1;
+    }();
+    return on ? std::getenv(name) : nullptr;
+}
+
 // Dynamic-LDS opt-in of one kernel, once per (kernel, device) of the process: the attribute is per device.
 inline void allow_dynamic_lds_ptr(const void* kernel, int bytes, const char* what, int line)
 {

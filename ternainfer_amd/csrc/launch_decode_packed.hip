@@ -15,15 +15,18 @@ void launch_repack(const Weights& w, uint32_t* packed, int N, int K, hipStream_t
 
 template <typename Act, int WAVES, int MB, int DEPTH, int NB = 1>
 void launch_decode_packed_as(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N,
-                             int K, hipStream_t st)
+                             int K, const RepackGuard* guard, hipStream_t st)
 {
-    const dim3 grid(N / 16 / NB, (M + 16 * MB - 1) / (16 * MB));
-    terna_decode_packed_kernel<Act, WAVES, MB, DEPTH, NB><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, ep, M, N, K);
+    const dim3 grid(N / 16 / NB + (guard != nullptr ? 1 : 0), (M + 16 * MB - 1) / (16 * MB));
+    if (guard != nullptr)
+        terna_decode_packed_kernel<Act, WAVES, MB, DEPTH, NB, true><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, ep, M, N, K, guard);
+    else
+        terna_decode_packed_kernel<Act, WAVES, MB, DEPTH, NB, false><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, ep, M, N, K, nullptr);
 }
 
 template <typename Act>
 void launch_decode_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
-                          hipStream_t st)
+                          hipStream_t st, const RepackGuard* guard)
 {
     const int forced = decode_waves_override();
     const bool wide = forced ? forced == 16 : (N / 16 <= 256);
@@ -35,22 +38,39 @@ void launch_decode_packed(const Act* x, const uint32_t* packed, uint16_t* out, c
         // multiple of 64, so the band count is even).  Measured on gate+up, cold: 6.4 us against 7.3 us; four
         // bands 6.7 us.  TERNASPMM_DECODE_BANDS=1 switches that off (tuning aid).
         static const bool multi_off = [] {
-            const char* v = std::getenv("TERNASPMM_DECODE_BANDS");
+            const char* v = tuning_env("TERNASPMM_DECODE_BANDS");
             return v && std::atoi(v) == 1;
         }();
-        if (narrow && !forced && !multi_off) launch_decode_packed_as<Act, 8, 1, 2, 2>(x, packed, out, ep, M, N, K, st);
-        else if (narrow) launch_decode_packed_as<Act, 4, 1, 3>(x, packed, out, ep, M, N, K, st);
-        else if (wide) launch_decode_packed_as<Act, 16, 1, 3>(x, packed, out, ep, M, N, K, st);
-        else launch_decode_packed_as<Act, 8, 1, 2>(x, packed, out, ep, M, N, K, st);
+        if (narrow && !forced && !multi_off) launch_decode_packed_as<Act, 8, 1, 2, 2>(x, packed, out, ep, M, N, K, guard, st);
+        else if (narrow) launch_decode_packed_as<Act, 4, 1, 3>(x, packed, out, ep, M, N, K, guard, st);
+        else if (wide) launch_decode_packed_as<Act, 16, 1, 3>(x, packed, out, ep, M, N, K, guard, st);
+        else launch_decode_packed_as<Act, 8, 1, 2>(x, packed, out, ep, M, N, K, guard, st);
     } else if (M <= 32) {
-        if (wide) launch_decode_packed_as<Act, 16, 2, 2>(x, packed, out, ep, M, N, K, st);
-        else launch_decode_packed_as<Act, 8, 2, 2>(x, packed, out, ep, M, N, K, st);
+        if (wide) launch_decode_packed_as<Act, 16, 2, 2>(x, packed, out, ep, M, N, K, guard, st);
+        else launch_decode_packed_as<Act, 8, 2, 2>(x, packed, out, ep, M, N, K, guard, st);
     } else {
-        launch_decode_packed_as<Act, 8, 4, 1>(x, packed, out, ep, M, N, K, st);
+        launch_decode_packed_as<Act, 8, 4, 1>(x, packed, out, ep, M, N, K, guard, st);
     }
 }
 
-template void launch_decode_packed<int8_t>(const int8_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
-template void launch_decode_packed<uint16_t>(const uint16_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
+// one wave each: record the fingerprint of a weight's reference-format tensors / check it as a launch of its own
+__global__ __launch_bounds__(64) void terna_repack_fingerprint_kernel(RepackGuard g, unsigned long long* out)
+{
+    const unsigned long long now = repack_fingerprint(g, threadIdx.x);
+    if (threadIdx.x == 0) *out = now;
+}
+__global__ __launch_bounds__(64) void terna_repack_guard_kernel(const RepackGuard* g) { repack_guard_role(*g, threadIdx.x); }
+
+void launch_repack_fingerprint(const RepackGuard& guard, unsigned long long* out, hipStream_t st)
+{
+    terna_repack_fingerprint_kernel<<<1, 64, 0, st>>>(guard, out);
+}
+
+void launch_repack_guard(const RepackGuard* guard, hipStream_t st) { terna_repack_guard_kernel<<<1, 64, 0, st>>>(guard); }
+
+template void launch_decode_packed<int8_t>(const int8_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t,
+                                           const RepackGuard*);
+template void launch_decode_packed<uint16_t>(const uint16_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t,
+                                             const RepackGuard*);
 
 }  // namespace terna

@@ -36,7 +36,7 @@ void launch_prefill_packed_as(const Act* x, const uint32_t* packed, uint16_t* ou
 int prefill_splits(long tiles, int steps, int M, int N, size_t scratch_bytes)
 {
     static const int forced = [] {
-        const char* v = std::getenv("TERNASPMM_PREFILL_SPLITS");
+        const char* v = tuning_env("TERNASPMM_PREFILL_SPLITS");
         const int n = v ? std::atoi(v) : 0;
         return n >= 1 && n <= 8 ? n : 0;
     }();
@@ -66,7 +66,7 @@ void launch_prefill_packed_dma_as(const Act* x, const uint32_t* packed, uint16_t
     const int splits = scratch_ok ? prefill_splits(static_cast<long>(grid.x) * grid.y, steps, M, N, scratch_bytes) : 1;
     grid.z = splits;
     static const int xcd_forced = [] {
-        const char* v = std::getenv("TERNASPMM_PREFILL_XCD_MAP");
+        const char* v = tuning_env("TERNASPMM_PREFILL_XCD_MAP");
         return v ? std::atoi(v) : -1;
     }();
     // XCD-aware tile order (see the kernel): pays once the activations no longer fit one XCD's 4 MiB L2 --
@@ -88,7 +88,7 @@ void launch_prefill_packed_dma_as(const Act* x, const uint32_t* packed, uint16_t
 inline bool prefill_dma_ok(const void* x, size_t act_bytes, int M, int N, int K)
 {
     static const bool off = [] {
-        const char* v = std::getenv("TERNASPMM_PREFILL_DMA");
+        const char* v = tuning_env("TERNASPMM_PREFILL_DMA");
         return v && std::atoi(v) == 0;
     }();
     return !off && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && static_cast<uint64_t>(M) * K * act_bytes < (1ull << 32) &&
@@ -105,12 +105,12 @@ void launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, 
     // BitNet-2B shape: it runs four waves per SIMD, and occupancy hides more latency than the taller
     // tiles save in weight expansion.  TERNASPMM_PREFILL_BM=64|128|256 forces one (tuning aid).
     static const int forced = [] {
-        const char* v = std::getenv("TERNASPMM_PREFILL_BM");
+        const char* v = tuning_env("TERNASPMM_PREFILL_BM");
         const int bm = v ? std::atoi(v) : 0;
         return (bm == 64 || bm == 96 || bm == 128 || bm == 256) ? bm : 0;
     }();
     static const int forced_bn = [] {
-        const char* v = std::getenv("TERNASPMM_PREFILL_BN");
+        const char* v = tuning_env("TERNASPMM_PREFILL_BN");
         const int bn = v ? std::atoi(v) : 0;
         return (bn == 128 || bn == 256) ? bn : 0;
     }();

@@ -26,7 +26,7 @@ void launch_decode_as(const Act* x, const Weights& w, uint16_t* out, const Epilo
 int decode_waves_override()
 {
     static const int waves = [] {
-        const char* v = std::getenv("TERNASPMM_DECODE_WAVES");
+        const char* v = tuning_env("TERNASPMM_DECODE_WAVES");
         const int w = v ? std::atoi(v) : 0;
         return (w == 4 || w == 8 || w == 16) ? w : 0;
     }();

@@ -32,9 +32,14 @@ void launch_decompress(const Weights& w, uint16_t* dense, int N, int K, hipStrea
 
 // ---- P2 layout (launch_decode_packed.hip, launch_prefill_packed_*.hip) ---------------------------------
 void launch_repack(const Weights& w, uint32_t* packed, int N, int K, hipStream_t st);
+// `guard` (device memory, may be NULL): the launch also checks that `packed` still belongs to the caller's
+// reference-format tensors.
 template <typename Act>
 void launch_decode_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
-                          hipStream_t st);
+                          hipStream_t st, const RepackGuard* guard = nullptr);
+// Fingerprint of the reference-format tensors named by `guard` into *out / the check of it as a launch of its own.
+void launch_repack_fingerprint(const RepackGuard& guard, unsigned long long* out, hipStream_t st);
+void launch_repack_guard(const RepackGuard* guard, hipStream_t st);
 // `scratch` (may be NULL; 16-byte aligned, scratch_bytes long): room for split-K partial sums when the shape has few
 // output tiles for the chip; the call then enqueues two launches.
 template <typename Act>
@@ -45,8 +50,10 @@ extern template void launch_decode<int8_t>(const int8_t*, const Weights&, uint16
 extern template void launch_decode<uint16_t>(const uint16_t*, const Weights&, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
 extern template void launch_prefill<int8_t>(const int8_t*, const Weights&, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
 extern template void launch_prefill<uint16_t>(const uint16_t*, const Weights&, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
-extern template void launch_decode_packed<int8_t>(const int8_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
-extern template void launch_decode_packed<uint16_t>(const uint16_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
+extern template void launch_decode_packed<int8_t>(const int8_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t,
+                                                  const RepackGuard*);
+extern template void launch_decode_packed<uint16_t>(const uint16_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t,
+                                                    const RepackGuard*);
 extern template void launch_prefill_packed<int8_t>(const int8_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, void*, size_t,
                                                    hipStream_t);
 extern template void launch_prefill_packed<uint16_t>(const uint16_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, void*, size_t,

@@ -25,6 +25,18 @@ enum EpilogueKind : int {
     EP_BF16       = 2,  // bf16(acc * scale[g]), fp32 scale             (bf16-activation family)
 };
 
+// What a kernel needs to check that a cached P2 copy still belongs to the reference-format tensors it was made from:
+// the tensors as the caller passes them now, the fingerprint recorded when the copy was made, and a flag in
+// host-visible memory that is raised on a mismatch.  Kernels take a pointer to one in device memory (NULL: no check).
+struct RepackGuard {
+    const uint64_t* bitmap;
+    const int* tile_off;
+    const uint32_t* sign_words;
+    const unsigned long long* expect;
+    uint32_t* stale;
+    int tiles;                       // N * K / 4096
+};
+
 struct Epilogue {
     const uint16_t* s;      // bf16 [M]       (int8 family)
     const uint16_t* ws;     // bf16 [ws_num]  (int8 family)

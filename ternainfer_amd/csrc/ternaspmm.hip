@@ -61,12 +61,17 @@ bool packed_small_kernel(int M, int N, int K, bool int8, bool has_scratch)
     return M <= 64;
 }
 
-// ---- opt-in repack cache behind the reference-format entry points (TERNASPMM_REPACK_CACHE=1).
-// An unmodified call site keeps passing the four format tensors; the first call that sees a weight
-// (identified by device, pointers and shape) allocates N*K/4 bytes, repacks into them and waits for
-// the repack; every later call runs the P2 kernels.  The cache trusts the pointers: a caller that
-// frees or rewrites weights must call ternaspmm_repack_cache_clear().  A first sight during stream
-// capture (where nothing may be allocated) is served by the reference-format kernels instead.
+// ---- repack cache behind the reference-format entry points (on unless TERNASPMM_REPACK_CACHE=0).
+// An unmodified call site keeps passing the four format tensors; the first call that sees a weight (identified by
+// device, pointers and shape) allocates N*K/4 bytes, repacks into them, records a fingerprint of the source tensors
+// and waits; every later call runs the P2 kernels.  A first sight during stream capture (where nothing may be
+// allocated) is served by the reference-format kernels instead.
+// The pointers alone are not trusted: every launch on a cached copy recomputes the fingerprint from the tensors the
+// caller passes (an extra workgroup of the small-M launch, a one-wave launch next to a large-M one) and raises a flag
+// in host-visible memory when it differs from the recorded one -- weights freed or rewritten, other data at the same
+// addresses.  A launch cannot be taken back, so the next call into the library reports the stale copy and ends the
+// process, as every error of this library does (kernels/TernaSpMM.cu:15-22); ternaspmm_repack_cache_clear() after
+// freeing or reloading weights is what avoids it.
 struct RepackKey {
     int device;
     const void* bitmap;
@@ -87,35 +92,79 @@ struct RepackKeyHash {
         return h * 1000003u ^ (static_cast<size_t>(key.n) << 20) ^ static_cast<size_t>(key.k) ^ (static_cast<size_t>(key.device) << 40);
     }
 };
+struct RepackEntry {
+    void* packed;                     // N*K/4 bytes of P2, then (256-byte aligned) the recorded fingerprint and the guard
+    const RepackGuard* guard;         // device memory: what the launches on this copy check
+};
 std::mutex g_repack_mutex;
-std::unordered_map<RepackKey, void*, RepackKeyHash> g_repack_cache;
+std::unordered_map<RepackKey, RepackEntry, RepackKeyHash> g_repack_cache;
+uint32_t* g_repack_stale = nullptr;   // pinned host memory, mapped into every device: set by a guard that found a mismatch
+int g_repack_on = -1;                 // -1: not decided yet (environment), 0 / 1
 
-const uint32_t* cached_packed(const Weights& w, int N, int K, hipStream_t st)
+bool repack_cache_on()
 {
-    static const bool on = [] {
+    if (g_repack_on < 0) {
         const char* v = std::getenv("TERNASPMM_REPACK_CACHE");
-        return v && std::atoi(v) != 0;
-    }();
-    if (!on) return nullptr;
+        g_repack_on = (v == nullptr || std::atoi(v) != 0) ? 1 : 0;
+    }
+    return g_repack_on == 1;
+}
+
+void repack_cache_report_stale(int line)
+{
+    if (g_repack_stale != nullptr && *reinterpret_cast<volatile uint32_t*>(g_repack_stale) != 0) {
+        std::printf("TernaSpMM Error (line %d): a cached repacked weight no longer matches the tensors it was made from -- "
+                    "weights were freed or rewritten without ternaspmm_repack_cache_clear(); results since then are invalid.  "
+                    "Call ternaspmm_repack_cache_clear() after freeing or reloading weights, or set TERNASPMM_REPACK_CACHE=0.\n",
+                    line);
+        std::fflush(stdout);
+        std::exit(EXIT_FAILURE);
+    }
+}
+
+// The cached P2 copy of a weight (made on first sight) and the guard its launches carry, or NULL.
+const uint32_t* cached_packed(const Weights& w, int N, int K, hipStream_t st, const RepackGuard** guard, int line)
+{
+    std::lock_guard<std::mutex> lock(g_repack_mutex);
+    if (!repack_cache_on()) return nullptr;
+    repack_cache_report_stale(line);
     RepackKey key{0, w.bitmap, w.sign_words, w.tile_off, N, K};
     if (hipGetDevice(&key.device) != hipSuccess) return nullptr;
-    std::lock_guard<std::mutex> lock(g_repack_mutex);
     const auto it = g_repack_cache.find(key);
-    if (it != g_repack_cache.end()) return static_cast<const uint32_t*>(it->second);
+    if (it != g_repack_cache.end()) {
+        *guard = it->second.guard;
+        return static_cast<const uint32_t*>(it->second.packed);
+    }
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(st, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
         (void)hipGetLastError();
         return nullptr;
     }
+    if (g_repack_stale == nullptr) {
+        void* flag = nullptr;
+        if (hipHostMalloc(&flag, 256, hipHostMallocMapped | hipHostMallocPortable) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        g_repack_stale = static_cast<uint32_t*>(flag);
+        *g_repack_stale = 0;
+    }
+    const size_t p2_bytes = (static_cast<size_t>(N) * K / 4 + 255) & ~static_cast<size_t>(255);
     void* buf = nullptr;
-    if (hipMalloc(&buf, static_cast<size_t>(N) * K / 4) != hipSuccess) {
+    if (hipMalloc(&buf, p2_bytes + 256) != hipSuccess) {
         (void)hipGetLastError();
         return nullptr;
     }
+    unsigned long long* expect = reinterpret_cast<unsigned long long*>(static_cast<char*>(buf) + p2_bytes);
+    RepackGuard* guard_dev = reinterpret_cast<RepackGuard*>(static_cast<char*>(buf) + p2_bytes + 64);
+    const RepackGuard g{w.bitmap, w.tile_off, w.sign_words, expect, g_repack_stale, N / 64 * (K / 64)};
     launch_repack(w, static_cast<uint32_t*>(buf), N, K, st);
-    const hipError_t e = hipStreamSynchronize(st);       // later calls may come on other streams
+    launch_repack_fingerprint(g, expect, st);
+    hipError_t e = hipMemcpyAsync(guard_dev, &g, sizeof(g), hipMemcpyHostToDevice, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);   // later calls may come on other streams; `g` is on this stack
     if (e != hipSuccess) die("repack cache", e, __LINE__);
-    g_repack_cache.emplace(key, buf);
+    g_repack_cache.emplace(key, RepackEntry{buf, guard_dev});
+    *guard = guard_dev;
     return static_cast<const uint32_t*>(buf);
 }
 
@@ -129,9 +178,14 @@ void run_i8(Route route, int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* m
     const bool decode_rule = route == ROUTE_DECODE || (route == ROUTE_AUTO && M <= 64);
     const Epilogue ep{s, ws, nullptr, ws_num, decode_rule ? EP_I8_DECODE : EP_I8_PREFILL};
     const Weights w{bitmap, tile_off, median_off, sign_words};
-    if (const uint32_t* p2 = cached_packed(w, N, K, st)) {
-        if (packed_small_kernel(M, N, K, true, workspace != nullptr)) launch_decode_packed<int8_t>(x, p2, out, ep, M, N, K, st);
-        else launch_prefill_packed<int8_t>(x, p2, out, ep, M, N, K, workspace, workspace ? static_cast<size_t>(N) * K : 0, st);
+    const RepackGuard* guard = nullptr;
+    if (const uint32_t* p2 = cached_packed(w, N, K, st, &guard, line)) {
+        if (packed_small_kernel(M, N, K, true, workspace != nullptr)) {
+            launch_decode_packed<int8_t>(x, p2, out, ep, M, N, K, st, guard);
+        } else {
+            launch_prefill_packed<int8_t>(x, p2, out, ep, M, N, K, workspace, workspace ? static_cast<size_t>(N) * K : 0, st);
+            launch_repack_guard(guard, st);
+        }
     } else if (M <= 64) launch_decode<int8_t>(x, w, out, ep, M, N, K, st);
     else launch_large_m<int8_t>(x, w, out, ep, M, N, K, workspace, st);
     const hipError_t e = hipGetLastError();
@@ -146,10 +200,15 @@ void run_bf16(Route route, const uint16_t* x, const uint64_t* bitmap, const int*
     const Epilogue ep{nullptr, nullptr, scale, ws_num, EP_BF16};
     const Weights w{bitmap, tile_off, median_off, sign_words};
     const bool small = route == ROUTE_DECODE || (route == ROUTE_AUTO && M <= 64);
-    if (const uint32_t* p2 = cached_packed(w, N, K, st)) {
+    const RepackGuard* guard = nullptr;
+    if (const uint32_t* p2 = cached_packed(w, N, K, st, &guard, line)) {
         const bool small_p2 = route == ROUTE_DECODE || (route == ROUTE_AUTO && packed_small_kernel(M, N, K, false, workspace != nullptr));
-        if (small_p2) launch_decode_packed<uint16_t>(x, p2, out, ep, M, N, K, st);
-        else launch_prefill_packed<uint16_t>(x, p2, out, ep, M, N, K, workspace, workspace ? static_cast<size_t>(N) * K : 0, st);
+        if (small_p2) {
+            launch_decode_packed<uint16_t>(x, p2, out, ep, M, N, K, st, guard);
+        } else {
+            launch_prefill_packed<uint16_t>(x, p2, out, ep, M, N, K, workspace, workspace ? static_cast<size_t>(N) * K : 0, st);
+            launch_repack_guard(guard, st);
+        }
     } else if (small) launch_decode<uint16_t>(x, w, out, ep, M, N, K, st);
     else launch_large_m<uint16_t>(x, w, out, ep, M, N, K, workspace, st);
     const hipError_t e = hipGetLastError();
@@ -378,8 +437,16 @@ void bitlinear_TernaSpMM_packed(const int8_t* x, const void* packed, terna_bf16*
 void ternaspmm_repack_cache_clear(void)
 {
     std::lock_guard<std::mutex> lock(g_repack_mutex);
-    for (auto& kv : g_repack_cache) (void)hipFree(kv.second);
+    for (auto& kv : g_repack_cache) (void)hipFree(kv.second.packed);      // waits for the launches that still read it
     g_repack_cache.clear();
+}
+
+int ternaspmm_repack_cache_enable(int on)
+{
+    std::lock_guard<std::mutex> lock(g_repack_mutex);
+    const int was = repack_cache_on() ? 1 : 0;
+    g_repack_on = on ? 1 : 0;
+    return was;
 }
 
 const char* ternaspmm_version(void) { return "ternaspmm-gfx950 0.1"; }

@@ -1,7 +1,11 @@
 """Run by tests/test_gpu_parity.py::test_repack_cache_behind_reference_entry_points in a child process with
 TERNASPMM_REPACK_CACHE=1: the reference-format entry points must give the same results as without the
 cache, on first sight (allocate + repack), on later sights (P2 kernels), under graph capture, and after
-ternaspmm_repack_cache_clear() when a different weight reuses the same device memory."""
+ternaspmm_repack_cache_clear() when a different weight reuses the same device memory.
+
+With the argument `stale` (a second child process): the weight is rewritten under the same pointers WITHOUT
+ternaspmm_repack_cache_clear(); the launch that follows finds a fingerprint that no longer matches and the call
+after it must end the process with the library's message."""
 import ctypes
 import sys
 
@@ -14,7 +18,32 @@ from tests.test_gpu_parity import WS, _check_bf16, run_bf16, run_i8
 from ternainfer_amd import _lib
 
 
+def stale() -> int:
+    lib = _lib.load()
+    n, k = 320, 192
+    a, b = DeviceFormat(make_ternary(n, k, 0.40, 980)), DeviceFormat(make_ternary(n, k, 0.40, 981))
+    vals = torch.zeros(max(a.vals.numel(), b.vals.numel()), dtype=a.vals.dtype, device="cuda")
+    vals[: a.vals.numel()].copy_(a.vals)
+    a_vals_own, a.vals = a.vals, vals
+    xq, s = make_int8_activations(8, k, 982)
+    for _ in range(2):                           # first sight (copy made), cached sight
+        if not (run_i8(lib, a, xq, s, WS, 1) == O.spmm_i8(xq, a.w, s, WS, 1, 0)).all():
+            print("int8 mismatch before the rewrite")
+            return 0                             # 0: the parent expects a non-zero exit from the library itself
+    a.bm.copy_(b.bm); a.off.copy_(b.off); a.med.copy_(b.med)
+    vals.zero_(); vals[: b.vals.numel()].copy_(b.vals)
+    torch.cuda.synchronize()
+    print("[case] rewritten under the same pointers, no clear", flush=True)
+    run_i8(lib, a, xq, s, WS, 1)                 # this launch raises the flag (its result is the old weight's)
+    torch.cuda.synchronize()
+    run_i8(lib, a, xq, s, WS, 1)                 # ... and this call must not return
+    print("the library did not notice the stale copy")
+    return 0
+
+
 def main() -> int:
+    if len(sys.argv) > 1 and sys.argv[1] == "stale":
+        return stale()
     lib = _lib.load()
     co = O.COracle()
     n, k = 320, 192

@@ -646,7 +646,8 @@ def test_tile_and_path_overrides(env):
     import sys
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     print(f"[case] override {env}", flush=True)
-    r = subprocess.run([sys.executable, "-u", "-m", "tests.env_variant_check"], cwd=root, env={**os.environ, **env},
+    r = subprocess.run([sys.executable, "-u", "-m", "tests.env_variant_check"], cwd=root,
+                       env={**os.environ, "TERNASPMM_TUNING": "1", **env},
                        capture_output=True, text=True, timeout=300)
     assert r.returncode == 0 and "override check ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
 
@@ -659,6 +660,11 @@ def test_repack_cache_behind_reference_entry_points():
     r = subprocess.run([sys.executable, "-u", "-m", "tests.repack_cache_check"], cwd=root,
                        env={**os.environ, "TERNASPMM_REPACK_CACHE": "1"}, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0 and "repack cache check ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+    # a weight rewritten under the same pointers without ternaspmm_repack_cache_clear(): the library ends the process
+    r = subprocess.run([sys.executable, "-u", "-m", "tests.repack_cache_check", "stale"], cwd=root,
+                       env={**os.environ, "TERNASPMM_REPACK_CACHE": "1"}, capture_output=True, text=True, timeout=300)
+    assert r.returncode != 0 and "no longer matches the tensors it was made from" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+    assert "did not notice" not in r.stdout
 
 
 def test_benchmark_entry_point_times_and_leaves_the_result(lib, capfd):
