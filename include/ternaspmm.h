@@ -233,6 +233,15 @@ void ternaspmm_rope_kv_store(const terna_bf16* qkv, const float* cos, const floa
 void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
                                 const long long* pos, terna_bf16* out, int B, int H, int KV, int D, int S,
                                 float scale, void* workspace, terna_stream stream);
+/* Several new tokens per sequence (the prompt pass): q bf16 [B][H][T][D] as ternaspmm_rope_kv_store leaves it, the
+ * caches already holding the new tokens' rows; new token t sees the slots 0 .. pos[t] (int64 [T], shared by the
+ * sequences; clamped to the cache).  out bf16 [B*T][H*D], row b*T + t.  Stands for the same fmha call as
+ * ternaspmm_decode_attention (model.py:231-233) at T > 1; flash-attention style, both products on the matrix cores,
+ * no workspace.  D is 64 or 128, S <= 8192.  Only enqueues. */
+void ternaspmm_prefill_attention(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
+                                 const long long* pos, terna_bf16* out, int B, int T, int H, int KV, int D, int S,
+                                 float scale, terna_stream stream);
+
 /* ternaspmm_decode_attention for callers that cannot allocate or bring a workspace (code under HIP graph capture
  * that owns no buffers, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
  * Same arguments, kernels and results as ternaspmm_decode_attention with a workspace, but the split-attention

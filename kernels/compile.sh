@@ -2,7 +2,9 @@
 # Builds kernels/libternaspmm.so for MI355X (gfx950) and the tests/test_kernel harness.
 # Run from anywhere:  bash kernels/compile.sh
 # One hipcc compile per translation unit, all at once (each kernel family is instantiated in a
-# file of its own), then one link.
+# file of its own), then one link.  -amdgpu-kernarg-preload-count: the first 16 dwords of a kernel's
+# arguments arrive in scalar registers with the wave instead of being fetched by its first instructions
+# (every launch of a decode step starts 0.05 - 0.3 us earlier).
 set -euo pipefail
 here="$(cd "$(dirname "${BASH_SOURCE[0]}")" && pwd)"
 src="$here/../ternainfer_amd/csrc"
@@ -11,6 +13,7 @@ mkdir -p "$obj"
 
 flags=(-std=c++17 -O3 -fPIC --offload-arch=gfx950
        -Xclang -target-feature -Xclang -packed-fp32-ops
+       -mllvm -amdgpu-kernarg-preload-count=16
        -Wall -Wno-unused-function)
 
 pids=()

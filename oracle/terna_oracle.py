@@ -343,6 +343,19 @@ def attention_one_token(q_bits: np.ndarray, k_bits: np.ndarray, v_bits: np.ndarr
     return np.einsum("bhs,bhsd->bhd", p, v)
 
 
+def attention_new_tokens(q_bits: np.ndarray, k_bits: np.ndarray, v_bits: np.ndarray, pos: np.ndarray, scale: float) -> np.ndarray:
+    """The same attention for T new tokens per sequence: q [B, H, T, D], k / v [B, KV, S, D] with the new tokens'
+    rows already in their slots, token t sees the slots 0 .. pos[t] (model.py:231-233 with the causal bias of the
+    prompt pass, generate.py:108-113; absent dependency, parity unpinned).  Each (t) row is attention_one_token
+    over its own prefix -- evaluated that way, so the closed-form checks of attention_one_token carry over.
+    Returns float64 [B, T, H, D]."""
+    b, h, t, d = q_bits.shape
+    out = np.empty((b, t, h, d), dtype=np.float64)
+    for ti in range(t):
+        out[:, ti] = attention_one_token(np.ascontiguousarray(q_bits[:, :, ti]), k_bits, v_bits, int(pos[ti]) + 1, scale)
+    return out
+
+
 def quant_weight_int8(w: np.ndarray):
     """convert_TernaInfer.py:159-163: ternarise by 1/mean(|W|); returns (int8 W, fp32 scale=1/s)."""
     w = np.asarray(w, dtype=np.float32)

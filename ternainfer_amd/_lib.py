@@ -54,6 +54,7 @@ PROTOTYPES = {
     "ternaspmm_rope_kv_store": ([_vp] * 7 + [_ci] * 7 + [_vp], None),
     "ternaspmm_rope_decode_attention": ([_vp] * 7 + [_ci] * 5 + [ctypes.c_float, _ci, _vp, _vp], None),
     "ternaspmm_decode_attention": ([_vp] * 5 + [_ci] * 5 + [ctypes.c_float, _vp, _vp], None),
+    "ternaspmm_prefill_attention": ([_vp] * 5 + [_ci] * 6 + [ctypes.c_float, _vp], None),
     "ternaspmm_decode_attention_static": ([_vp] * 5 + [_ci] * 5 + [ctypes.c_float, _vp], ctypes.c_int),
     "ternaspmm_attention_workspace_bytes": ([_ci, _ci, _ci], ctypes.c_longlong),
     "ternaspmm_probe_empty": ([_vp], None),

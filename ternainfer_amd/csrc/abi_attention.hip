@@ -10,6 +10,7 @@
 #include "../../include/ternaspmm.h"
 #include "host_util.h"
 #include "attention_kernel.h"
+#include "prefill_attention_kernel.h"
 
 using namespace terna;
 
@@ -210,6 +211,22 @@ void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, 
                                    static_cast<hipStream_t>(stream));
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_decode_attention", e, __LINE__);
+}
+
+void ternaspmm_prefill_attention(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
+                                 const long long* pos, terna_bf16* out, int B, int T, int H, int KV, int D, int S,
+                                 float scale, terna_stream stream)
+{
+    if (!attention_args_ok("ternaspmm_prefill_attention", B, H, KV, D, S) || T < 1 || B > 65535 || H > 65535) {
+        if (T < 1 || B > 65535 || H > 65535) std::fprintf(stderr, "ternaspmm_prefill_attention: unsupported arguments (B=%d T=%d H=%d)\n", B, T, H);
+        return;
+    }
+    const dim3 grid((T + 15) / 16, H, B);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (D == 128) terna_prefill_attention_kernel<128><<<grid, dim3(64), 0, st>>>(q, cache_k, cache_v, pos, out, T, H, KV, S, scale);
+    else terna_prefill_attention_kernel<64><<<grid, dim3(64), 0, st>>>(q, cache_k, cache_v, pos, out, T, H, KV, S, scale);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_prefill_attention", e, __LINE__);
 }
 
 int ternaspmm_decode_attention_static(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,

@@ -252,6 +252,31 @@ def test_decode_attention(lib, b, h, kv, d, s_max, n, split):
         assert torch.equal(od, od2)                      # merged in split order: the same bits whoever arrives last
 
 
+@pytest.mark.parametrize("b,h,kv,d,s_max,first,t", [(1, 20, 5, 128, 160, 0, 128), (8, 20, 5, 128, 130, 0, 128), (2, 4, 2, 64, 64, 0, 23),
+                                                   (2, 4, 2, 64, 300, 100, 50), (1, 20, 5, 128, 512, 300, 17), (3, 8, 8, 128, 40, 0, 1)])
+def test_prefill_attention(lib, b, h, kv, d, s_max, first, t):
+    """T new tokens per sequence at the slots first .. first + T - 1, each attending over the cache up to its own
+    slot (the prompt pass; with first > 0 a chunk appended to an existing prefix): against attention_one_token row by
+    row, to the tolerance of the single-token kernel.  Slots past the newest token hold NaN bit patterns: nothing
+    beyond a token's own slot may reach its output."""
+    q = make_bf16_activations(b * h * t, d, 720 + t).reshape(b, h, t, d)
+    k = make_bf16_activations(b * kv * s_max, d, 721 + t).reshape(b, kv, s_max, d)
+    v = make_bf16_activations(b * kv * s_max, d, 722 + t, outlier_frac=0.01).reshape(b, kv, s_max, d)
+    k[:, :, first + t:] = 0x7FC0
+    v[:, :, first + t:] = 0x7FC0
+    pos = np.arange(first, first + t, dtype=np.int64)
+    od = torch.full((b * t, h * d), 0x7FC0, dtype=torch.int16, device="cuda")
+    qd, kd, vd, pd = _dev(q), _dev(k), _dev(v), _dev(pos)
+    print(f"[case] prefill attention b={b} h={h} kv={kv} d={d} S={s_max} first={first} t={t}", flush=True)
+    lib.ternaspmm_prefill_attention(_vp(qd), _vp(kd), _vp(vd), _vp(pd), _vp(od), b, t, h, kv, d, s_max, float(d) ** -0.5, None)
+    torch.cuda.synchronize()
+    got = O.bf16_bits_to_f32(od.cpu().numpy().view(np.uint16)).reshape(b, t, h, d).astype(np.float64)
+    want = O.attention_new_tokens(q, k, v, pos, float(d) ** -0.5)
+    tol = 2.0 ** -7 * np.abs(want).max(axis=-1, keepdims=True) + 1e-6
+    assert np.isfinite(got).all()
+    assert (np.abs(got - want) <= tol).all(), float((np.abs(got - want) / tol).max())
+
+
 def _attn_workspace(lib, b, h, d):
     nbytes = lib.ternaspmm_attention_workspace_bytes(b, h, d)
     assert nbytes > 0
