@@ -20,7 +20,7 @@
 //                  positions works as long as A uses the same one;
 //                  A = V^T: row d, those eight keys -- gathered as eight 2-byte reads from the value block staged
 //                  in LDS (row pitch 2 D + 8 bytes: the four lane groups fall into disjoint banks).
-// fp32 running maximum / sum / output, exp via v_exp_f32, probabilities rounded to bf16 for the second product.
+// fp32 running maximum / sum / output, exp via v_exp_f32, probabilities as a sum of two bf16 terms in the second product.
 #pragma once
 
 #include "norm_quant_kernel.h"
@@ -124,7 +124,14 @@ __global__ __launch_bounds__(64) void terna_prefill_attention_kernel(
         psum += __shfl_xor(psum, 32);
         l_run = l_run * alpha + psum;
         m_run = m_new;
-        const bf16x8 bp = __builtin_bit_cast(bf16x8, pack_bf16x8(p));
+        // probabilities as two bf16 terms (value = hi + lo to 16 bits): a single bf16 rounding of P is a relative error of
+        // 2^-9 per term, which shows when large value channels nearly cancel; the second product runs once per term
+        const u32x4 p_hi = pack_bf16x8(p);
+        float hi_f[8], p_lo_f[8];
+        unpack_bf16x8(p_hi, hi_f);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) p_lo_f[e] = p[e] - hi_f[e];
+        const bf16x8 bp = __builtin_bit_cast(bf16x8, p_hi), bp_lo = __builtin_bit_cast(bf16x8, pack_bf16x8(p_lo_f));
         // ---- value block through LDS (the previous block's reads are done: one wave, program order + the barrier)
         __syncthreads();
 #pragma unroll
@@ -148,7 +155,9 @@ __global__ __launch_bounds__(64) void terna_prefill_attention_kernel(
             }
 #pragma unroll
             for (int v = 0; v < 4; ++v) o[dt][v] *= alpha;
-            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, u32x4{w[0], w[1], w[2], w[3]}), bp, o[dt], 0, 0, 0);
+            const bf16x8 va = __builtin_bit_cast(bf16x8, u32x4{w[0], w[1], w[2], w[3]});
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, bp, o[dt], 0, 0, 0);
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, bp_lo, o[dt], 0, 0, 0);
         }
     }
 

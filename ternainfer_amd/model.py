@@ -117,6 +117,9 @@ def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, adjacent: 
     return torch.cat([x1 * cos - x2 * sin, x2 * cos + x1 * sin], dim=-1).to(x.dtype)
 
 
+KERNEL_ATTENTION = object()    # in place of a mask: several new tokens, attention by ternaspmm_prefill_attention
+
+
 class Block:
     def __init__(self, args: ModelArgs, gen: Optional[torch.Generator], act: str, p_zero: float = 0.40):
         self.args = args
@@ -216,6 +219,10 @@ class Block:
             lib.ternaspmm_rope_kv_store(_p(qkv), _p(cos), _p(sin), _p(pos_idx), _p(q), _p(cache_k), _p(cache_v),
                                         bsz, t, a.n_heads, a.n_kv_heads, a.head_dim, cache_k.shape[2],
                                         int(a.rope_adjacent), stream)
+            if mask is KERNEL_ATTENTION:    # the prompt pass: the library's multi-token attention over the cache
+                o = torch.empty((bsz * t, a.n_heads * a.head_dim), dtype=torch.bfloat16, device=x.device)
+                lib.ternaspmm_prefill_attention(_p(q), _p(cache_k), _p(cache_v), _p(pos_idx), _p(o), bsz, t, a.n_heads,
+                                                a.n_kv_heads, a.head_dim, cache_k.shape[2], a.head_dim ** -0.5, stream)
         else:
             qkv = qkv.view(bsz, t, a.n_heads + 2 * a.n_kv_heads, a.head_dim).transpose(1, 2)
             q, k, v = qkv[:, :a.n_heads], qkv[:, a.n_heads:a.n_heads + a.n_kv_heads], qkv[:, a.n_heads + a.n_kv_heads:]
@@ -223,7 +230,7 @@ class Block:
             k = apply_rope(k, cos[None, None], sin[None, None], a.rope_adjacent)
             cache_k.index_copy_(2, pos_idx, k)
             cache_v.index_copy_(2, pos_idx, v)
-        if not one_token:
+        if not one_token and mask is not KERNEL_ATTENTION:
             kk = cache_k.repeat_interleave(rep, dim=1)
             vv = cache_v.repeat_interleave(rep, dim=1)
             o = F.scaled_dot_product_attention(q, kk, vv, attn_mask=mask)
@@ -346,8 +353,11 @@ class Transformer:
         rows = self.rope_tables(max_seq, dev).index_select(0, pos_idx)         # fp32 [T, 2, head_dim / 2]
         cos, sin = rows[:, 0].contiguous(), rows[:, 1].contiguous()           # views when T == 1
         mask = None
-        one_launch_attention = self.layers[0].fused and t == 1 and a.head_dim in (64, 128) and max_seq <= 8192
-        if not one_launch_attention:
+        kernels_fit = self.layers[0].fused and a.head_dim in (64, 128) and max_seq <= 8192 and tokens.is_cuda
+        one_launch_attention = kernels_fit and t == 1
+        if kernels_fit and t > 1 and getattr(self, "kernel_prefill_attention", True):
+            mask = KERNEL_ATTENTION
+        elif not one_launch_attention:
             # causal over cache slots: new token at slot p sees slots <= p
             mask = (torch.arange(max_seq, device=dev)[None, :] <= pos_idx[:, None])[None, None]
         x = self.tok_embeddings[tokens.reshape(-1)]
@@ -377,8 +387,23 @@ def greedy_decode(model: Transformer, prompt: torch.Tensor, gen_tokens: int, use
     bsz, plen = prompt.shape
     cache = model.make_cache(bsz, plen + gen_tokens)
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
-    ev[0].record()
-    logits = model.forward(prompt, cache, torch.arange(plen, device="cuda"))
+    slots = torch.arange(plen, device="cuda")
+    if use_graph:
+        # the prompt pass as a graph too (generate.py:100-144): warm up on a side stream, capture, replay
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            model.forward(prompt, cache, slots)
+        torch.cuda.current_stream().wait_stream(side)
+        prefill = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(prefill):
+            logits = model.forward(prompt, cache, slots)
+        torch.cuda.synchronize()
+        ev[0].record()
+        prefill.replay()
+    else:
+        ev[0].record()
+        logits = model.forward(prompt, cache, slots)
     tok = argmax_rows(logits.contiguous())                                    # int64 [B, 1]
     ev[1].record()
     counters = torch.tensor([plen, 1], dtype=torch.int64, device="cuda")      # cache slot of the next token, tokens stored

@@ -95,6 +95,42 @@ def test_toy_model_greedy_decode_graph_equals_eager():
     assert torch.equal(a, c)
 
 
+def test_toy_model_prompt_pass_kernel_attention_sdpa_and_graph_replays():
+    """The prompt pass through the library's multi-token attention against the same pass through PyTorch's SDPA, and
+    the captured prompt graph against eager execution on several replays with eager work and synchronisations between
+    them (a captured node that misbehaves from the second replay on would show here)."""
+    from ternainfer_amd.model import ModelArgs, Transformer
+    args = ModelArgs(dim=256, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=1024, ffn_dim=384)
+    model = Transformer(args, seed=13, act="int8")
+    tokens = torch.randint(0, args.vocab_size, (2, 40), generator=torch.Generator().manual_seed(14)).cuda()
+    slots = torch.arange(40, device="cuda")
+    print("[case] toy model prompt pass: kernel attention vs SDPA, graph replays", flush=True)
+    with torch.inference_mode():
+        eager = model.forward(tokens, model.make_cache(2, 48), slots).float()
+        model.kernel_prefill_attention = False
+        sdpa = model.forward(tokens, model.make_cache(2, 48), slots).float()
+        model.kernel_prefill_attention = True
+        assert (eager - sdpa).abs().max().item() <= 3e-2 * sdpa.abs().max().item()
+        assert torch.nn.functional.cosine_similarity(eager.flatten(), sdpa.flatten(), dim=0).item() > 0.999
+        cache = model.make_cache(2, 48)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            model.forward(tokens, cache, slots)
+        torch.cuda.current_stream().wait_stream(side)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            captured = model.forward(tokens, cache, slots)
+        for _ in range(3):
+            captured.zero_()
+            for ck, cv in cache:
+                ck.zero_(); cv.zero_()
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(captured.float(), eager)
+
+
 def test_converted_checkpoint_loads_and_matches_cpu_golden(tmp_path):
     """fp32 state dict -> converter -> three files -> Transformer.from_checkpoint; the CPU golden is built
     from the converter's int8 matrices (not from the packed buffers), so the loader and the repack are
