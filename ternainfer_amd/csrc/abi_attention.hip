@@ -98,9 +98,9 @@ void launch_attention_as(const uint16_t* q, uint16_t* ck, uint16_t* cv, const fl
     const size_t lds = decode_attention_lds_bytes(D, NW, S);
     if (lds > 64 * 1024) allow_dynamic_lds(kernel, 160 * 1024, "hipFuncSetAttribute(decode attention)", __LINE__);
     const int slots = attention_slots(B, H, KV);
-    kernel<<<dim3(slots + pf.workgroups, splits), dim3(64 * NW), lds, st>>>(q, ck, cv, cos, sin, pos, out, H, KV, S, scale,
-                                                                           scratch.partial, scratch.arrived, splits, pf, slots,
-                                                                           attention_groups_on(H, KV) ? B * KV : 0);
+    kernel<<<dim3(slots + pf.workgroups, splits), dim3(64 * NW), lds, st>>>(
+        q, ck, cv, pos, H, KV, S, splits, slots, attention_groups_on(H, KV) ? B * KV : 0, scale, cos, sin, out, scratch.partial,
+        scratch.arrived, pf);
 }
 
 template <bool ROPE, bool ADJ>

@@ -23,7 +23,7 @@ void ternaspmm_rmsnorm_quant(const terna_bf16* x, const terna_bf16* residual, te
         return;
     }
     terna_norm_quant_kernel<false><<<dim3(M), dim3(kNormThreads), 0, static_cast<hipStream_t>(stream)>>>(
-        x, residual, sum_out, weight, eps, y_out, xq_out, s_out, K);
+        x, residual, weight, K, eps, sum_out, y_out, xq_out, s_out);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_rmsnorm_quant", e, __LINE__);
 }
@@ -36,7 +36,7 @@ void ternaspmm_relu2_mul_rmsnorm_quant(const terna_bf16* x13, const terna_bf16* 
         return;
     }
     terna_norm_quant_kernel<true><<<dim3(M), dim3(kNormThreads), 0, static_cast<hipStream_t>(stream)>>>(
-        x13, nullptr, nullptr, weight, eps, y_out, xq_out, s_out, F);
+        x13, nullptr, weight, F, eps, nullptr, y_out, xq_out, s_out);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_relu2_mul_rmsnorm_quant", e, __LINE__);
 }
@@ -75,7 +75,7 @@ static int launch_decode_fused(int mode, const terna_bf16* x, const terna_bf16* 
     const dim3 grid(multi16 || multi8 ? bands / 4 : bands);
 #define TERNA_FUSED(WAVES, TMAX, MODE, MP, NB)                                                                     \
     terna_decode_fused_kernel<WAVES, TMAX, MODE, MP, NB><<<grid, dim3(WAVES * 64), 0, st>>>(                       \
-        x, residual, sum_out, norm_weight, eps, p, out, ws, ws_num, xq_out, s_out, M, N, K)
+        x, residual, norm_weight, p, M, N, K, eps, sum_out, out, ws, ws_num, xq_out, s_out)
 #define TERNA_FUSED_M(WAVES, TMAX, MODE, NB)                                                                       \
     do {                                                                                                           \
         if (M == 1) TERNA_FUSED(WAVES, TMAX, MODE, 1, NB);                                                         \

@@ -216,10 +216,11 @@ constexpr size_t decode_attention_lds_bytes(int D, int NW, int S)
 
 template <int D, bool ROPE, bool ADJACENT = false, int NW = 4, bool SPLIT = false>
 __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
+    // what the first loads depend on comes first: the leading sixteen dwords of the arguments arrive in scalar registers
     const uint16_t* __restrict__ q, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
-    const float* __restrict__ cosv, const float* __restrict__ sinv,
-    const long long* __restrict__ pos, uint16_t* __restrict__ out, int H, int KV, int S, float scale,
-    float* partial, int* arrived, int splits, AttentionPrefetch pf, int heads, int groups)
+    const long long* __restrict__ pos, int H, int KV, int S, int splits, int heads, int groups, float scale,
+    const float* __restrict__ cosv, const float* __restrict__ sinv, uint16_t* __restrict__ out,
+    float* partial, int* arrived, AttentionPrefetch pf)
 {
     static_assert(D == 64 || D == 128, "head dimension");
     constexpr int CH = D / 8;                    // 8-dimension chunks of a row

@@ -68,10 +68,11 @@ enum FusedMode { FUSED_PLAIN, FUSED_RESIDUAL, FUSED_GLU };
 
 template <int WAVES, int TMAX, int MODE, int MP, int NB = 1>
 __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
-    const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, uint16_t* __restrict__ sum_out,
-    const uint16_t* __restrict__ norm_w, float eps, const uint32_t* __restrict__ packed,
+    // what the first loads depend on comes first: the leading sixteen dwords of the arguments arrive in scalar registers
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, const uint16_t* __restrict__ norm_w,
+    const uint32_t* __restrict__ packed, int M, int N, int K, float eps, uint16_t* __restrict__ sum_out,
     uint16_t* __restrict__ out, const uint16_t* __restrict__ ws, int ws_num, int8_t* __restrict__ xq_out,
-    uint16_t* __restrict__ s_out, int M, int N, int K)
+    uint16_t* __restrict__ s_out)
 {
     using XQ = XSlab<int8_t>;
     using Piece = RowPiece<MP>;

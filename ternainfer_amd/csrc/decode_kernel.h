@@ -183,7 +183,7 @@ template <typename Act, int WAVES, int MB, int DEPTH>
 __global__ __launch_bounds__(WAVES * 64) void terna_decode_kernel(
     const Act* __restrict__ x, const uint64_t* __restrict__ bitmap, const int* __restrict__ tile_off,
     const uint16_t* __restrict__ median_off, const uint32_t* __restrict__ sign_words,
-    uint16_t* __restrict__ out, Epilogue ep, int M, int N, int K)
+    uint16_t* __restrict__ out, int M, int N, int K, Epilogue ep)
 {
     using T = ActTraits<Act>;
     using Acc = typename T::Acc;

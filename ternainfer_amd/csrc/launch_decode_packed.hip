@@ -19,9 +19,9 @@ void launch_decode_packed_as(const Act* x, const uint32_t* packed, uint16_t* out
 {
     const dim3 grid(N / 16 / NB + (guard != nullptr ? 1 : 0), (M + 16 * MB - 1) / (16 * MB));
     if (guard != nullptr)
-        terna_decode_packed_kernel<Act, WAVES, MB, DEPTH, NB, true><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, ep, M, N, K, guard);
+        terna_decode_packed_kernel<Act, WAVES, MB, DEPTH, NB, true><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, M, N, K, guard, ep);
     else
-        terna_decode_packed_kernel<Act, WAVES, MB, DEPTH, NB, false><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, ep, M, N, K, nullptr);
+        terna_decode_packed_kernel<Act, WAVES, MB, DEPTH, NB, false><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, M, N, K, nullptr, ep);
 }
 
 template <typename Act>

@@ -15,7 +15,7 @@ void launch_decode_as(const Act* x, const Weights& w, uint16_t* out, const Epilo
 {
     const dim3 grid(N / 16, (M + 16 * MB - 1) / (16 * MB));
     terna_decode_kernel<Act, WAVES, MB, DEPTH><<<grid, dim3(WAVES * 64), 0, st>>>(
-        x, w.bitmap, w.tile_off, w.median_off, w.sign_words, out, ep, M, N, K);
+        x, w.bitmap, w.tile_off, w.median_off, w.sign_words, out, M, N, K, ep);
 }
 
 // Shape of the small-M launch.  With one workgroup per 16-row band, a matrix with few bands

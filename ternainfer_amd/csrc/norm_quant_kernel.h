@@ -98,9 +98,9 @@ __device__ __forceinline__ float round_bf16(float v) { return bf16_bits_to_float
 // GLU = true : x [M][2K] holding x1 | x3; residual / sum_out unused.
 template <bool GLU>
 __global__ __launch_bounds__(kNormThreads) void terna_norm_quant_kernel(
-    const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, uint16_t* __restrict__ sum_out,
-    const uint16_t* __restrict__ weight, float eps, uint16_t* __restrict__ y_out, int8_t* __restrict__ xq_out,
-    uint16_t* __restrict__ s_out, int K)
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, const uint16_t* __restrict__ weight, int K,
+    float eps, uint16_t* __restrict__ sum_out, uint16_t* __restrict__ y_out, int8_t* __restrict__ xq_out,
+    uint16_t* __restrict__ s_out)
 {
     __shared__ float red[2][kNormThreads / 64];
     const int tid = threadIdx.x;
