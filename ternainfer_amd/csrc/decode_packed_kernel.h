@@ -26,19 +26,19 @@ struct PackedRaw {
 // GUARD: the launch runs on a cached P2 copy and checks it (below).  A variant of its own: the branch at the top costs
 // every workgroup 0.3 us (nothing can start before all arguments are in), which launches on a caller's own P2
 // buffer do not have to pay.
-// Argument order: pointers and integers first, the epilogue structure last -- the first sixteen dwords of the arguments
+// Argument order: pointers and integers first, the structures last -- the first sixteen dwords of the arguments
 // arrive preloaded in scalar registers, but only up to the first structure passed by value, and everything the first
 // global loads depend on should be among them.
 template <typename Act, int WAVES, int MB, int DEPTH, int NB = 1, bool GUARD = false>
 __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
     const Act* __restrict__ x, const uint32_t* __restrict__ packed, uint16_t* __restrict__ out,
-    int M, int N, int K, const RepackGuard* __restrict__ guard, Epilogue ep)
+    int M, int N, int K, Epilogue ep, RepackGuard guard)
 {
     // A launch on a cached P2 copy carries one extra workgroup in x -- the one past the last band -- that checks, next to
     // the others and off their critical path, that the copy still belongs to the caller's tensors.
     if constexpr (GUARD) {
         if (static_cast<int>(blockIdx.x) * (16 * NB) >= N) {
-            if (blockIdx.y == 0 && threadIdx.x < 64) repack_guard_role(*guard, threadIdx.x);
+            if (blockIdx.y == 0 && threadIdx.x < 64) repack_guard_role(guard, threadIdx.x);
             return;
         }
     }

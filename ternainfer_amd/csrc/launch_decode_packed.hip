@@ -19,9 +19,9 @@ void launch_decode_packed_as(const Act* x, const uint32_t* packed, uint16_t* out
 {
     const dim3 grid(N / 16 / NB + (guard != nullptr ? 1 : 0), (M + 16 * MB - 1) / (16 * MB));
     if (guard != nullptr)
-        terna_decode_packed_kernel<Act, WAVES, MB, DEPTH, NB, true><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, M, N, K, guard, ep);
+        terna_decode_packed_kernel<Act, WAVES, MB, DEPTH, NB, true><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, M, N, K, ep, *guard);
     else
-        terna_decode_packed_kernel<Act, WAVES, MB, DEPTH, NB, false><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, M, N, K, nullptr, ep);
+        terna_decode_packed_kernel<Act, WAVES, MB, DEPTH, NB, false><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, M, N, K, ep, RepackGuard{});
 }
 
 template <typename Act>
@@ -59,14 +59,14 @@ __global__ __launch_bounds__(64) void terna_repack_fingerprint_kernel(RepackGuar
     const unsigned long long now = repack_fingerprint(g, threadIdx.x);
     if (threadIdx.x == 0) *out = now;
 }
-__global__ __launch_bounds__(64) void terna_repack_guard_kernel(const RepackGuard* g) { repack_guard_role(*g, threadIdx.x); }
+__global__ __launch_bounds__(64) void terna_repack_guard_kernel(RepackGuard g) { repack_guard_role(g, threadIdx.x); }
 
 void launch_repack_fingerprint(const RepackGuard& guard, unsigned long long* out, hipStream_t st)
 {
     terna_repack_fingerprint_kernel<<<1, 64, 0, st>>>(guard, out);
 }
 
-void launch_repack_guard(const RepackGuard* guard, hipStream_t st) { terna_repack_guard_kernel<<<1, 64, 0, st>>>(guard); }
+void launch_repack_guard(const RepackGuard* guard, hipStream_t st) { terna_repack_guard_kernel<<<1, 64, 0, st>>>(*guard); }
 
 template void launch_decode_packed<int8_t>(const int8_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t,
                                            const RepackGuard*);

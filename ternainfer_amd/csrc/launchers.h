@@ -32,8 +32,7 @@ void launch_decompress(const Weights& w, uint16_t* dense, int N, int K, hipStrea
 
 // ---- P2 layout (launch_decode_packed.hip, launch_prefill_packed_*.hip) ---------------------------------
 void launch_repack(const Weights& w, uint32_t* packed, int N, int K, hipStream_t st);
-// `guard` (device memory, may be NULL): the launch also checks that `packed` still belongs to the caller's
-// reference-format tensors.
+// `guard` (may be NULL): the launch also checks that `packed` still belongs to the caller's reference-format tensors.
 template <typename Act>
 void launch_decode_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
                           hipStream_t st, const RepackGuard* guard = nullptr);

@@ -84,7 +84,7 @@ __device__ __forceinline__ unsigned long long repack_fingerprint(const RepackGua
 {
     const long long n_bm = static_cast<long long>(g.tiles) * 64;
     const int total = g.tile_off[g.tiles];
-    const int words = total >> 5;
+    const int words = g.words;
     const unsigned long long b0 = g.bitmap[lane], b1 = g.bitmap[n_bm / 2 - 32 + lane], b2 = g.bitmap[n_bm - 64 + lane];
     unsigned long long s0 = 0, s1 = 0;
     if (words > 0) {
@@ -109,8 +109,9 @@ __device__ __forceinline__ unsigned long long repack_fingerprint(const RepackGua
 // One wave: compare with the recorded fingerprint, raise the host-visible flag on a mismatch.
 __device__ __forceinline__ void repack_guard_role(const RepackGuard& g, int lane)
 {
+    const unsigned long long want = *g.expect;          // requested together with the samples
     const unsigned long long now = repack_fingerprint(g, lane);
-    if (lane == 0 && now != *g.expect) *reinterpret_cast<volatile uint32_t*>(g.stale) = 1u;
+    if (lane == 0 && now != want) *reinterpret_cast<volatile uint32_t*>(g.stale) = 1u;
 }
 
 // Reference format -> P2.  One wave per 16x64 band-tile; lane (i, g) produces word 4*i + g.

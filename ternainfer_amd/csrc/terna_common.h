@@ -27,7 +27,9 @@ enum EpilogueKind : int {
 
 // What a kernel needs to check that a cached P2 copy still belongs to the reference-format tensors it was made from:
 // the tensors as the caller passes them now, the fingerprint recorded when the copy was made, and a flag in
-// host-visible memory that is raised on a mismatch.  Kernels take a pointer to one in device memory (NULL: no check).
+// host-visible memory that is raised on a mismatch.  `words` is the length of the sign stream when the copy was made:
+// the sampled positions follow it, so that every load of the check is independent of every other (one memory round
+// trip; a changed length shows in the sign-bit total, which is part of the fingerprint).
 struct RepackGuard {
     const uint64_t* bitmap;
     const int* tile_off;
@@ -35,6 +37,7 @@ struct RepackGuard {
     const unsigned long long* expect;
     uint32_t* stale;
     int tiles;                       // N * K / 4096
+    int words;                       // sign words of the matrix the copy was made from
 };
 
 struct Epilogue {

@@ -93,8 +93,8 @@ struct RepackKeyHash {
     }
 };
 struct RepackEntry {
-    void* packed;                     // N*K/4 bytes of P2, then (256-byte aligned) the recorded fingerprint and the guard
-    const RepackGuard* guard;         // device memory: what the launches on this copy check
+    void* packed;                     // N*K/4 bytes of P2, then (256-byte aligned) the recorded fingerprint
+    RepackGuard guard;                // what the launches on this copy check (passed to them by value)
 };
 std::mutex g_repack_mutex;
 std::unordered_map<RepackKey, RepackEntry, RepackKeyHash> g_repack_cache;
@@ -123,7 +123,7 @@ void repack_cache_report_stale(int line)
 }
 
 // The cached P2 copy of a weight (made on first sight) and the guard its launches carry, or NULL.
-const uint32_t* cached_packed(const Weights& w, int N, int K, hipStream_t st, const RepackGuard** guard, int line)
+const uint32_t* cached_packed(const Weights& w, int N, int K, hipStream_t st, RepackGuard* guard, int line)
 {
     std::lock_guard<std::mutex> lock(g_repack_mutex);
     if (!repack_cache_on()) return nullptr;
@@ -132,7 +132,7 @@ const uint32_t* cached_packed(const Weights& w, int N, int K, hipStream_t st, co
     if (hipGetDevice(&key.device) != hipSuccess) return nullptr;
     const auto it = g_repack_cache.find(key);
     if (it != g_repack_cache.end()) {
-        *guard = it->second.guard;
+        *guard = it->second.guard;                        // (a copy: the launch takes it by value)
         return static_cast<const uint32_t*>(it->second.packed);
     }
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
@@ -156,15 +156,18 @@ const uint32_t* cached_packed(const Weights& w, int N, int K, hipStream_t st, co
         return nullptr;
     }
     unsigned long long* expect = reinterpret_cast<unsigned long long*>(static_cast<char*>(buf) + p2_bytes);
-    RepackGuard* guard_dev = reinterpret_cast<RepackGuard*>(static_cast<char*>(buf) + p2_bytes + 64);
-    const RepackGuard g{w.bitmap, w.tile_off, w.sign_words, expect, g_repack_stale, N / 64 * (K / 64)};
+    RepackGuard g{w.bitmap, w.tile_off, w.sign_words, expect, g_repack_stale, N / 64 * (K / 64), 0};
+    int total_bits = 0;                                  // the length of the sign stream decides where the check samples it
+    hipError_t e = hipMemcpyAsync(&total_bits, w.tile_off + g.tiles, sizeof(int), hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e != hipSuccess) die("repack cache", e, __LINE__);
+    g.words = total_bits >> 5;
     launch_repack(w, static_cast<uint32_t*>(buf), N, K, st);
     launch_repack_fingerprint(g, expect, st);
-    hipError_t e = hipMemcpyAsync(guard_dev, &g, sizeof(g), hipMemcpyHostToDevice, st);
-    if (e == hipSuccess) e = hipStreamSynchronize(st);   // later calls may come on other streams; `g` is on this stack
+    e = hipStreamSynchronize(st);                        // later calls may come on other streams
     if (e != hipSuccess) die("repack cache", e, __LINE__);
-    g_repack_cache.emplace(key, RepackEntry{buf, guard_dev});
-    *guard = guard_dev;
+    g_repack_cache.emplace(key, RepackEntry{buf, g});
+    *guard = g;
     return static_cast<const uint32_t*>(buf);
 }
 
@@ -178,13 +181,13 @@ void run_i8(Route route, int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* m
     const bool decode_rule = route == ROUTE_DECODE || (route == ROUTE_AUTO && M <= 64);
     const Epilogue ep{s, ws, nullptr, ws_num, decode_rule ? EP_I8_DECODE : EP_I8_PREFILL};
     const Weights w{bitmap, tile_off, median_off, sign_words};
-    const RepackGuard* guard = nullptr;
+    RepackGuard guard{};
     if (const uint32_t* p2 = cached_packed(w, N, K, st, &guard, line)) {
         if (packed_small_kernel(M, N, K, true, workspace != nullptr)) {
-            launch_decode_packed<int8_t>(x, p2, out, ep, M, N, K, st, guard);
+            launch_decode_packed<int8_t>(x, p2, out, ep, M, N, K, st, &guard);
         } else {
             launch_prefill_packed<int8_t>(x, p2, out, ep, M, N, K, workspace, workspace ? static_cast<size_t>(N) * K : 0, st);
-            launch_repack_guard(guard, st);
+            launch_repack_guard(&guard, st);
         }
     } else if (M <= 64) launch_decode<int8_t>(x, w, out, ep, M, N, K, st);
     else launch_large_m<int8_t>(x, w, out, ep, M, N, K, workspace, st);
@@ -200,14 +203,14 @@ void run_bf16(Route route, const uint16_t* x, const uint64_t* bitmap, const int*
     const Epilogue ep{nullptr, nullptr, scale, ws_num, EP_BF16};
     const Weights w{bitmap, tile_off, median_off, sign_words};
     const bool small = route == ROUTE_DECODE || (route == ROUTE_AUTO && M <= 64);
-    const RepackGuard* guard = nullptr;
+    RepackGuard guard{};
     if (const uint32_t* p2 = cached_packed(w, N, K, st, &guard, line)) {
         const bool small_p2 = route == ROUTE_DECODE || (route == ROUTE_AUTO && packed_small_kernel(M, N, K, false, workspace != nullptr));
         if (small_p2) {
-            launch_decode_packed<uint16_t>(x, p2, out, ep, M, N, K, st, guard);
+            launch_decode_packed<uint16_t>(x, p2, out, ep, M, N, K, st, &guard);
         } else {
             launch_prefill_packed<uint16_t>(x, p2, out, ep, M, N, K, workspace, workspace ? static_cast<size_t>(N) * K : 0, st);
-            launch_repack_guard(guard, st);
+            launch_repack_guard(&guard, st);
         }
     } else if (small) launch_decode<uint16_t>(x, w, out, ep, M, N, K, st);
     else launch_large_m<uint16_t>(x, w, out, ep, M, N, K, workspace, st);
