@@ -47,8 +47,8 @@ METRIC = "TernaSpMM GB/s + %HBM roofline (M=8,K=N=2560); 2B-shape decode tok/s"
 # HBM bytes per launch of the small-M P2 kernel on the default workload (M=8, average over the four matrices):
 # a counter measurement, not part of this run -- two rocprofv3 --pmc runs of this file (FETCH_SIZE, WRITE_SIZE),
 # scaled by what the same counters read for a 256 MiB copy.  Quoted with its source; null for any other workload.
-TRAFFIC = {"bytes_per_launch": (19209.3 + 356.0) * 1024 / 4,
-           "source": "profiles/decode_packed_kernel_hbm_traffic.md (rocprofv3 --pmc; kernel unchanged since)"}
+TRAFFIC = {"bytes_per_launch": (19206.6 + 356.0) * 1024 / 4,
+           "source": "profiles/decode_packed_kernel_hbm_traffic.md (two rocprofv3 --pmc runs, FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 by the copy probe)"}
 
 
 def vp(t):
@@ -248,8 +248,8 @@ def run_model(args, torch):
                                f"FFN 6912, vocab 128256), batch {args.batch}, 128-token prompt, 256 greedy tokens, "
                                f"{act} activations into the ternary linears, weights in P2 layout, one HIP graph per "
                                "decode step; norms, gate, activation quantisation, RoPE, cache write, single-token "
-                               "attention, the bf16 LM head and greedy sampling are library kernels; the attention of "
-                               "the prompt pass is a PyTorch-ROCm op"
+                               "attention, the multi-token attention of the prompt pass, the bf16 LM head and greedy "
+                               "sampling are library kernels; the prompt pass is one HIP graph too"
                                + ("" if args.no_prefetch else "; the idle CUs of the attention launch "
                                                             "prefetch the weights of the launches that follow"),
                    "batch": args.batch, "act": act},

@@ -7,9 +7,10 @@ attention and FFN sub-norms, squared-ReLU gating, tied bf16 LM head (model.py:19
 323-335, 367) -- and, like the reference's SpBitLinear (model.py:120-133), quantises activations
 per row to int8 in front of every ternary linear.  The residual adds, the four norms, the gate and
 that quantisation run as the library's fused prologue kernels (one launch in front of each
-linear); RoPE + KV-cache write and single-token attention are library kernels too, multi-token
-(prefill) attention and the LM head are PyTorch-ROCm ops; one decode step is captured in a HIP
-graph, as generate.py:204-224 does.
+linear); RoPE + KV-cache write, single-token attention, the multi-token attention of the prompt
+pass, the LM head of a decode step and greedy sampling are library kernels too (the prompt pass projects
+its last rows through the LM head with a PyTorch-ROCm matmul); the prompt pass and one decode step are
+each captured in a HIP graph, as generate.py:204-224 does for the decode step.
 """
 from __future__ import annotations
 
