@@ -3,8 +3,11 @@
 Provenance: the reference stores no golden vectors for this path and its Python encoder is
 read, not run (its arithmetic is pinned by closed forms and by the replay of the reference
 kernel's consumer in tests/test_oracle_format.py).  These fixtures are therefore written by
-the oracle, once that pinning is green; they freeze the byte-level format against drift in
-either the oracle or the library encoder.
+the oracle, once that pinning is green.  They are DRIFT GUARDS ONLY: they freeze the byte-level
+format and two small linear layers against later changes in the oracle or the library, and
+pin nothing about the oracle itself -- a mistake the oracle had when they were written would
+be frozen with them.  What pins the oracle are the hand-worked and closed-form checks in
+tests/test_oracle_format.py and tests/test_oracle_linear.py.
 """
 import os
 import sys
