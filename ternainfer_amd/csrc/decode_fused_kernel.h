@@ -276,7 +276,7 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
             e.s = s_row[i];
             uint16_t o[4];
 #pragma unroll
-            for (int v = 0; v < 4; ++v) o[v] = apply_epilogue<int>(EP_I8_DECODE, e, v, sum[v]);
+            for (int v = 0; v < 4; ++v) o[v] = apply_epilogue<int>(EP_I8_DECODE, e, v, sum[v] >> kI8WeightShift);
             const u32x2 pk = {o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16)};
             *reinterpret_cast<u32x2*>(out + static_cast<size_t>(i) * N + n0) = pk;
         }

@@ -111,8 +111,8 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 const uint32_t w = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(operand_src, static_cast<int>(cur.word[b])));
-                a0[b] = __builtin_bit_cast(bf16x8, expand_chunk_bf16(w));
-                a1[b] = __builtin_bit_cast(bf16x8, expand_chunk_bf16(w >> 4));
+                a0[b] = __builtin_bit_cast(bf16x8, expand_chunk_bf16(w << 4));
+                a1[b] = __builtin_bit_cast(bf16x8, expand_chunk_bf16(w));
             }
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
@@ -180,7 +180,7 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
     }
 
     // Cross-wave sum in wave order, then the fused epilogue (accumulator layout: lane L holds
-    // output rows 4*(L>>4) .. +3 of column L & 15).  bf16 weights were +-0.5: undo with an exact x2.
+    // output rows 4*(L>>4) .. +3 of column L & 15).  bf16 weights were +-2: undo with an exact x0.5.
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
@@ -200,8 +200,8 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
             uint16_t o[4];
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-                if constexpr (sizeof(Act) == 2) o[v] = apply_epilogue<float>(ep.kind, eregs, v, sum[v] * 2.0f);
-                else o[v] = apply_epilogue<int>(ep.kind, eregs, v, sum[v]);
+                if constexpr (sizeof(Act) == 2) o[v] = apply_epilogue<float>(ep.kind, eregs, v, sum[v] * kBf16WeightUndo);
+                else o[v] = apply_epilogue<int>(ep.kind, eregs, v, sum[v] >> kI8WeightShift);
             }
             const u32x2 pk = {o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16)};
             *reinterpret_cast<u32x2*>(out + static_cast<size_t>(m) * N + n0) = pk;

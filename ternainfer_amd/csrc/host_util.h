@@ -29,6 +29,18 @@ inline bool shape_ok(int M, int N, int K)
     return true;
 }
 
+// int8 activations on the P2 layout: the 32-bit accumulator holds 64 times the sum (packed_common.h), which bounds K
+inline bool i8_depth_ok(int K)
+{
+    constexpr int kMaxK = (1 << 18) - 64;
+    if (K > kMaxK) {
+        std::printf("TernaSpMM Error: unsupported K=%d with int8 activations (need K <= %d)\n", K, kMaxK);
+        std::fflush(stdout);
+        return false;
+    }
+    return true;
+}
+
 // weight_scale has four slots (convert/convert_TernaInfer.py:176-194): one to four scale groups per matrix
 inline bool groups_ok(int ws_num)
 {

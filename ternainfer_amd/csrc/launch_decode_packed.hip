@@ -46,7 +46,9 @@ void launch_decode_packed(const Act* x, const uint32_t* packed, uint16_t* out, c
         else if (wide) launch_decode_packed_as<Act, 16, 1, 3>(x, packed, out, ep, M, N, K, guard, st);
         else launch_decode_packed_as<Act, 8, 1, 2>(x, packed, out, ep, M, N, K, guard, st);
     } else if (M <= 32) {
-        if (wide) launch_decode_packed_as<Act, 16, 2, 2>(x, packed, out, ep, M, N, K, guard, st);
+        // more than 512 bands: two bands per workgroup share the staging of the 32 activation rows, as above
+        if (!forced && N / 16 > 512) launch_decode_packed_as<Act, 4, 2, 2, 2>(x, packed, out, ep, M, N, K, guard, st);
+        else if (wide) launch_decode_packed_as<Act, 16, 2, 2>(x, packed, out, ep, M, N, K, guard, st);
         else launch_decode_packed_as<Act, 8, 2, 2>(x, packed, out, ep, M, N, K, guard, st);
     } else {
         launch_decode_packed_as<Act, 8, 4, 1>(x, packed, out, ep, M, N, K, guard, st);

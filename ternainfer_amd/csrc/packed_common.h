@@ -11,42 +11,42 @@
 //                                 (bit0 = nonzero, bit1 = negative)
 //   column j of the group       : byte j & 3, 2-bit field j >> 2, i.e. bit 8*(j&3) + 2*(j>>2).
 //
-// So `(word >> 2*q) & 0x03030303` is the four 2-bit codes of columns 4q .. 4q+3 in four bytes --
-// exactly a v_perm_b32 selector, and its result is in natural column order: the matching
-// activation operand is a plain contiguous piece of the activation row.  One v_perm against a 4-entry byte table turns it into four int8 weights
-// (0x00 / 0x01 / 0xFF) or four bf16 high bytes (0x00 / 0x3F / 0xBF), and two more v_perm
-// interleave the high bytes with zero low bytes into bf16 pairs.  bf16 weights are therefore
-// +-0.5 (0x3F00 / 0xBF00), not +-1: every product and partial sum is exactly half of what +-1
-// would give, and the epilogue multiplies the accumulator by 2, which is exact.
+// A 2-bit code in the top field of a byte IS the weight in two number formats at once:
+//   as a signed byte        0x40 = +64, 0xC0 = -64, 0x00 = 0                  (int8 operand, times 64)
+//   as a bf16 high byte     0x4000 = +2.0, 0xC000 = -2.0, 0x0000 = 0          (bf16 operand, times 2)
+// and `(word << (6 - 2*q)) & 0xC0C0C0C0` puts the codes of columns 4q .. 4q+3 there, in natural column order -- the
+// matching activation operand is a plain contiguous piece of the activation row.  For int8 that is the whole
+// expansion (seven shift / mask operations per sixteen weights, no table); for bf16 two v_perm_b32 per four weights
+// interleave the high bytes with zero low bytes into bf16 pairs.  The accumulators therefore hold a multiple of the
+// true sum -- 64 times (int32; exact, and it fits for K < 2^31 / (64 * 128) = 262144) or twice (fp32; exact) -- and
+// every consumer undoes it before the epilogue: `>> kI8WeightShift`, respectively `* kBf16WeightUndo`.
 #pragma once
 
 #include "decode_kernel.h"
 
 namespace terna {
 
-constexpr uint32_t kCodeMask = 0x03030303u;
-constexpr uint32_t kTableBf16Hi = 0xBF003F00u;   // code 0 -> 0x00, 1 -> 0x3F, 3 -> 0xBF
-constexpr uint32_t kTableI8 = 0xFF000100u;       // code 0 -> 0x00, 1 -> 0x01, 3 -> 0xFF
+constexpr uint32_t kTopFieldMask = 0xC0C0C0C0u;  // the top field of every byte: an int8 weight times 64 / a bf16 high byte
+constexpr int kI8WeightShift = 6;                // int8 accumulators hold the sum << 6
+constexpr float kBf16WeightUndo = 0.5f;          // bf16-operand accumulators hold twice the sum
 constexpr uint32_t kPair01 = 0x010C000Cu;        // [0, b0, 0, b1]: two bf16 with zero low bytes
 constexpr uint32_t kPair23 = 0x030C020Cu;        // [0, b2, 0, b3]
 
-// Eight bf16 weights (+-0.5 / 0), columns 8h .. 8h+7 of the group, of a packed word `dd` already
-// shifted right by 4h: dword j holds columns 8h + 2j, 8h + 2j + 1.
-__device__ __forceinline__ u32x4 expand_chunk_bf16(uint32_t dd)
+// Eight bf16 weights (+-2 / 0), columns 8h .. 8h+7 of the group, from `t` = the packed word shifted LEFT by 4 - 4h
+// (h = 0: word << 4, h = 1: the word itself): dword j holds columns 8h + 2j, 8h + 2j + 1.
+__device__ __forceinline__ u32x4 expand_chunk_bf16(uint32_t t)
 {
-    const uint32_t hi0 = __builtin_amdgcn_perm(0u, kTableBf16Hi, dd & kCodeMask);
-    const uint32_t hi1 = __builtin_amdgcn_perm(0u, kTableBf16Hi, (dd >> 2) & kCodeMask);
+    const uint32_t hi0 = (t << 2) & kTopFieldMask;     // field 2h of every byte: columns 8h .. 8h+3
+    const uint32_t hi1 = t & kTopFieldMask;            // field 2h + 1: columns 8h+4 .. 8h+7
     return u32x4{__builtin_amdgcn_perm(0u, hi0, kPair01), __builtin_amdgcn_perm(0u, hi0, kPair23),
                  __builtin_amdgcn_perm(0u, hi1, kPair01), __builtin_amdgcn_perm(0u, hi1, kPair23)};
 }
 
-// Sixteen int8 weights (+-1 / 0) of a packed word in column order: dword q holds columns 4q .. 4q+3.
+// Sixteen int8 weights (+-64 / 0) of a packed word in column order: dword q holds columns 4q .. 4q+3.
 __device__ __forceinline__ i32x4 expand_word_i8(uint32_t d)
 {
-    return i32x4{static_cast<int>(__builtin_amdgcn_perm(0u, kTableI8, d & kCodeMask)),
-                 static_cast<int>(__builtin_amdgcn_perm(0u, kTableI8, (d >> 2) & kCodeMask)),
-                 static_cast<int>(__builtin_amdgcn_perm(0u, kTableI8, (d >> 4) & kCodeMask)),
-                 static_cast<int>(__builtin_amdgcn_perm(0u, kTableI8, (d >> 6) & kCodeMask))};
+    return i32x4{static_cast<int>((d << 6) & kTopFieldMask), static_cast<int>((d << 4) & kTopFieldMask),
+                 static_cast<int>((d << 2) & kTopFieldMask), static_cast<int>(d & kTopFieldMask)};
 }
 
 // Repack table: (nonzero nibble, next 4 sign bits of the stream) -> the nibble's four 2-bit codes

@@ -2,7 +2,7 @@
 // operand goes global memory -> registers -> matrix core, expanded by v_perm_b32, and never
 // touches LDS.
 //
-//   out[m][n] = epilogue( 2 * sum_k X[m][k] * Whalf[n][k] ),   Whalf = W / 2 in {-0.5, 0, +0.5}
+//   out[m][n] = epilogue( sum_k X[m][k] * W2[n][k] / 2 ),   W2 = 2 W in {-2, 0, +2}
 //
 // Tiling.  One workgroup (4 waves) owns BN = 128*NA output features x BM = 32*MB batch rows and walks
 // K in steps of 64.  The waves split the output features only: wave w owns rows 32*NA*w .. +32*NA-1 and
@@ -41,7 +41,7 @@ __device__ __forceinline__ void int8x16_to_bf16(const u32x4& v, u32x4& c0, u32x4
 
 // Fused epilogue of one wave's NA x MB accumulator tiles (v_mfma_f32_32x32x16 layout: lane holds
 // column m = L % 32 and rows n = (v&3) + 8(v>>2) + 4(L/32) of each tile).  A float accumulator is
-// half the true sum (weights were +-0.5; x2 is exact); an integer one is the sum itself.
+// twice the true sum (weights were +-2; x0.5 is exact); an integer one is the sum times 64 (weights were +-64; >> 6 is exact).
 template <int MB, int NA, typename AccV>
 __device__ __forceinline__ void packed_prefill_epilogue(AccV (&acc)[NA][MB], uint16_t* __restrict__ out,
                                                         const Epilogue& ep, int M, int N, int n_wave, int m0, int lane)
@@ -50,8 +50,8 @@ __device__ __forceinline__ void packed_prefill_epilogue(AccV (&acc)[NA][MB], uin
     constexpr bool kFloatAcc = std::is_same<AccV, f32x16>::value;
     auto value = [&](auto ac, auto bc, int idx) {
         constexpr int a = decltype(ac)::value, b = decltype(bc)::value;
-        if constexpr (kFloatAcc) return acc[a][b][idx] * 2.0f;
-        else return static_cast<float>(acc[a][b][idx]);
+        if constexpr (kFloatAcc) return acc[a][b][idx] * kBf16WeightUndo;
+        else return static_cast<float>(acc[a][b][idx] >> kI8WeightShift);
     };
     int m_of[MB];
     float s_of[MB];
@@ -266,7 +266,7 @@ __global__ __launch_bounds__(256, MB == 8 ? 1 : (MB == 3 ? 3 : 2)) void terna_pr
     }
 
     const int b_off = kb * PX + l32 * 16;                    // + g*2*PX + b*512
-    const int wshift = 4 * kb;                               // columns 8kb .. 8kb+7 of every word
+    const int wshift = 4 - 4 * kb;                           // columns 8kb .. 8kb+7 of every word (left shift, see expand_chunk_bf16)
 
     struct BOps { bf16x8 b[MB]; };
     auto load_b = [&](int st, int g, BOps& r) {
@@ -285,7 +285,7 @@ __global__ __launch_bounds__(256, MB == 8 ? 1 : (MB == 3 ? 3 : 2)) void terna_pr
             if constexpr (g < 3) load_b(st, g + 1, bnxt);
 #pragma unroll
             for (int a = 0; a < NA; ++a) {
-                const bf16x8 af = __builtin_bit_cast(bf16x8, expand_chunk_bf16(rw.w[a][g] >> wshift));
+                const bf16x8 af = __builtin_bit_cast(bf16x8, expand_chunk_bf16(rw.w[a][g] << wshift));
 #pragma unroll
                 for (int b = 0; b < MB; ++b)
                     acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bcur.b[b], acc[a][b], 0, 0, 0);
@@ -479,7 +479,7 @@ __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) voi
     int b_off[4];
 #pragma unroll
     for (int g = 0; g < 4; ++g) b_off[g] = l32 * 128 + ((((I8 ? 4 * kb + g : 2 * g + kb)) ^ x_swizzle(l32)) * 16);
-    const int wshift = 4 * kb;                               // bf16: columns 8kb .. 8kb+7 of every word
+    const int wshift = 4 - 4 * kb;                           // bf16: columns 8kb .. 8kb+7 of every word (left shift, see expand_chunk_bf16)
 
     struct BOps { u32x4 b[MB]; };
     auto load_b = [&](int st, int g, BOps& r) {
@@ -498,7 +498,7 @@ __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) voi
                 for (int b = 0; b < MB; ++b)
                     acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, __builtin_bit_cast(i32x4, bcur.b[b]), acc[a][b], 0, 0, 0);
             } else {
-                const bf16x8 af = __builtin_bit_cast(bf16x8, expand_chunk_bf16(rw.w[a][g] >> wshift));
+                const bf16x8 af = __builtin_bit_cast(bf16x8, expand_chunk_bf16(rw.w[a][g] << wshift));
 #pragma unroll
                 for (int b = 0; b < MB; ++b)
                     acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, __builtin_bit_cast(bf16x8, bcur.b[b]), acc[a][b], 0, 0, 0);
@@ -586,7 +586,7 @@ __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) voi
 
 // Second launch of a split-K call: out[m][n0 .. n0+3] = epilogue(sum over the splits, in split order, of partial[z][m][n]).
 // AccT = int (int8 family: the sum is exact, so the result is that of the unsplit kernel bit for bit) or float (bf16
-// family: weights were +-0.5, the sum is doubled first, as in the unsplit epilogue).  One thread per four columns.
+// family: weights were +-2, the sum is halved first, as in the unsplit epilogue).  One thread per four columns.
 template <typename AccT>
 __global__ __launch_bounds__(256) void terna_splitk_reduce_kernel(const AccT* __restrict__ partial, uint16_t* __restrict__ out,
                                                                   Epilogue ep, int M, int N, int splits)
@@ -603,8 +603,8 @@ __global__ __launch_bounds__(256) void terna_splitk_reduce_kernel(const AccT* __
     uint16_t o[4];
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-        if constexpr (std::is_same<AccT, float>::value) o[v] = apply_epilogue<float>(ep.kind, e, v, sum[v] * 2.0f);
-        else o[v] = apply_epilogue<int>(ep.kind, e, v, sum[v]);
+        if constexpr (std::is_same<AccT, float>::value) o[v] = apply_epilogue<float>(ep.kind, e, v, sum[v] * kBf16WeightUndo);
+        else o[v] = apply_epilogue<int>(ep.kind, e, v, sum[v] >> kI8WeightShift);   // planes hold the sums << 6, like the accumulators
     }
     *reinterpret_cast<u32x2*>(out + at) = u32x2{o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16)};
 }

@@ -48,16 +48,17 @@ enum Route { ROUTE_AUTO, ROUTE_DECODE, ROUTE_PREFILL };
 // By measurement on the four BitNet-2B matrices at M = 16 .. 256 (us per launch, P2 layout, small-M kernel / MFMA-tiled
 // kernel with split-K scratch): the small-M kernel's time grows with every 16 rows, the MFMA-tiled one is flat but
 // pays a fill / drain of 10 us or more.
-//   gate+up (864 bands)  bf16 M=32 11.8 / 16.9   M=48 23.5 / 17.6      int8 M=32  8.4 / 11.3   M=48 12.8 / 12.2
-//   QKV (240 bands)      bf16 M=64  8.1 / 11.6   M=96 13.5 / 12.6      int8 M=128 8.7 / 11.4   M=192 11.6 / 11.5
-//   down (K = 6912)      bf16 M=64 14.0 / 14.1   M=96 24.7 / 15.4      int8 M=64  9.5 / 12.5   M=96 14.6 / 13.3
+//   gate+up (864 bands)  bf16 M=32  8.7 / 17.4   M=48 23.1 / 18.1      int8 M=32  6.5 / 10.7   M=48 12.4 / 11.6
+//   QKV (240 bands)      bf16 M=64  7.9 / 11.8   M=96 13.2 / 12.7      int8 M=128 8.5 / 10.9   M=192 11.1 / 10.9
+//   O (160 bands)        bf16 M=64  7.6 / 11.4   M=96 12.5 / 12.1      int8 M=192 8.3 / 10.6   M=256 10.6 / 10.8
+//   down (K = 6912)      bf16 M=64 14.2 / 14.4   M=96 24.6 / 15.5      int8 M=64  9.2 / 12.2   M=96 14.2 / 12.8
 // Without scratch the MFMA-tiled kernel cannot split K and walks all of it in every workgroup (QKV bf16 16-17 us flat,
 // down 38-44 us), which moves the cut up.
 bool packed_small_kernel(int M, int N, int K, bool int8, bool has_scratch)
 {
     if (N / 16 > 512) return M <= 32;
     if (!has_scratch) return M <= (K > 4096 ? 256 : 128);
-    if (int8 && K <= 4096) return M <= 128;
+    if (int8 && K <= 4096) return M <= (N / 16 <= 160 ? 192 : 128);
     return M <= 64;
 }
 
@@ -175,7 +176,7 @@ void run_i8(Route route, int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* m
             uint16_t* out, uint16_t* s, uint16_t* ws, int ws_num, int M, int N, int K, void* workspace,
             hipStream_t st, int line)
 {
-    if (!shape_ok(M, N, K) || !groups_ok(ws_num)) return;
+    if (!shape_ok(M, N, K) || !groups_ok(ws_num) || !i8_depth_ok(K)) return;
     // The reference picks its path, and with it the epilogue arithmetic, by M <= 64
     // (kernels/TernaSpMM.cu:34); the forced entry points pin one of the two.
     const bool decode_rule = route == ROUTE_DECODE || (route == ROUTE_AUTO && M <= 64);
@@ -418,7 +419,7 @@ void bitlinear_TernaSpMM_packed_ws(const int8_t* x, const void* packed, terna_bf
                                    const terna_bf16* ws, int ws_num, int M, int N, int K, int route, void* workspace,
                                    long long workspace_bytes, terna_stream stream)
 {
-    if (!shape_ok(M, N, K) || !groups_ok(ws_num)) return;
+    if (!shape_ok(M, N, K) || !groups_ok(ws_num) || !i8_depth_ok(K)) return;
     const int rule = route & 3, kernel = route & 12;
     const bool decode_rule = rule == 2 || (rule != 1 && M <= 64);
     const Epilogue ep{s, ws, nullptr, ws_num, decode_rule ? EP_I8_DECODE : EP_I8_PREFILL};

@@ -57,3 +57,24 @@ def test_encode_sizes_rejects_bad_shapes():
     assert lib.ternaspmm_encode_sizes(64, 100, *ptrs) == -1
     assert lib.ternaspmm_encode_sizes(128, 192, *ptrs) == 0
     assert list(out) == [128 * 192 // 64, 128 * 192 // 4096 + 1, 3 * 128 * 192 // 4096, 128 * 192 // 32]
+
+
+def test_unsupported_shapes_are_refused_before_any_device_work():
+    """A shape the format cannot express, and a K too deep for int8 activations on the P2 layout (its 32-bit
+    accumulator holds 64 times the sum), print a message and return without a launch (the reference's
+    unsupported-batch branch, TernaSpMM_API.cuh:117-120): no pointer is touched, so this runs without a GPU."""
+    import subprocess
+    import sys
+    code = ("from ternainfer_amd import _lib\n"
+            "lib = _lib.load()\n"
+            "lib.bitlinear_TernaSpMM_packed(None, None, None, None, None, 1, 1, 64, 100, 0, None)\n"
+            "lib.bitlinear_TernaSpMM_packed(None, None, None, None, None, 1, 1, 64, 262144, 0, None)\n"
+            "lib.bitlinear_TernaSpMM(None, None, None, None, None, None, None, None, 1, 8, 64, 262144, 1, None, None)\n"
+            "lib.bitlinear_TernaSpMM_bf16_packed(None, None, None, None, 5, 1, 64, 64, 0, None)\n"
+            "print('returned', flush=True)\n")
+    r = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "unsupported shape M=1 N=64 K=100" in r.stdout
+    assert r.stdout.count("unsupported K=262144 with int8 activations (need K <= 262080)") == 2
+    assert "unsupported ws_num=5" in r.stdout
+    assert r.stdout.rstrip().endswith("returned")

@@ -475,11 +475,11 @@ def test_packed_split_k_with_workspace(lib, m, n, k, ws_num):
 
 
 @pytest.mark.parametrize("with_ws", [False, True])
-@pytest.mark.parametrize("m", [32, 33, 48, 64, 65, 96, 128, 129, 200, 256, 257])
-@pytest.mark.parametrize("n,k,ws_num", [(8256, 192, 1), (3840, 128, 3), (256, 4160, 2)])
+@pytest.mark.parametrize("m", [32, 33, 48, 64, 65, 96, 128, 129, 192, 193, 256, 257])
+@pytest.mark.parametrize("n,k,ws_num", [(8256, 192, 1), (3840, 128, 3), (2560, 128, 1), (256, 4160, 2)])
 def test_packed_kernel_choice_boundaries(lib, m, n, k, ws_num, with_ws):
     """The library picks the small-M or the MFMA-tiled kernel by shape (more than 512 bands: up to 32 rows; long K,
-    int8, scratch at hand: other cuts); whatever it picks, int8 results follow the reference's M <= 64 epilogue rule
+    int8, 160 bands or fewer, scratch at hand: other cuts); whatever it picks, int8 results follow the reference's M <= 64 epilogue rule
     bit for bit and bf16 results stay within tolerance, on both sides of every cut."""
     w = make_ternary(n, k, 0.40, 470 + n % 89)
     packed = repack(lib, DeviceFormat(w))
