@@ -218,8 +218,12 @@ int bitlinear_TernaSpMM_packed_fused_glu(const terna_bf16* x13, const terna_bf16
  *
  * Precondition on `pos` (device memory, which the host side of the call cannot inspect): 0 <= pos[t] < S.  A
  * position outside the cache writes no k / v row and the attention runs over the prefix clamped to [1, S]
- * slots: the result is then meaningless but every access stays inside the caller's buffers.  All sequences of
- * the batch share the one position: the entry points have no per-sequence prefix lengths.
+ * slots: the result is then meaningless but every access stays inside the caller's buffers.
+ *
+ * `per_sequence` (every entry point of this group): 0 -- all sequences of the batch share the positions, `pos` is
+ * int64 [T] and cos / sin are fp32 [T][D/2] (T = 1 for the single-token entry points); non-zero -- every sequence has
+ * its own, `pos` is int64 [B][T] and cos / sin are fp32 [B][T][D/2]: sequences with different prefix lengths in one
+ * batch, the kv_seqlen the reference hands to its attention bias (generate.py:253-262, 294).
  *
  * `workspace` (may be NULL): device memory of ternaspmm_attention_workspace_bytes(B, H, D) bytes, zero-filled by
  * the caller once before its first use.  With it the cache prefix of every head is split over up to 8 workgroups
@@ -228,18 +232,18 @@ int bitlinear_TernaSpMM_packed_fused_glu(const terna_bf16* x13, const terna_bf16
  * zero, so the same workspace serves every later call; calls that share one workspace must not overlap. */
 long long ternaspmm_attention_workspace_bytes(int B, int H, int D);
 void ternaspmm_rope_kv_store(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
-                             terna_bf16* q_out, terna_bf16* cache_k, terna_bf16* cache_v, int B, int T, int H,
+                             int per_sequence, terna_bf16* q_out, terna_bf16* cache_k, terna_bf16* cache_v, int B, int T, int H,
                              int KV, int D, int S, int adjacent, terna_stream stream);
 void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
-                                const long long* pos, terna_bf16* out, int B, int H, int KV, int D, int S,
+                                const long long* pos, int per_sequence, terna_bf16* out, int B, int H, int KV, int D, int S,
                                 float scale, void* workspace, terna_stream stream);
 /* Several new tokens per sequence (the prompt pass): q bf16 [B][H][T][D] as ternaspmm_rope_kv_store leaves it, the
- * caches already holding the new tokens' rows; new token t sees the slots 0 .. pos[t] (int64 [T], shared by the
- * sequences; clamped to the cache).  out bf16 [B*T][H*D], row b*T + t.  Stands for the same fmha call as
+ * caches already holding the new tokens' rows; new token t sees the slots 0 .. pos[t] (int64 [T] shared by the
+ * sequences, or [B][T] with `per_sequence`; clamped to the cache).  out bf16 [B*T][H*D], row b*T + t.  Stands for the same fmha call as
  * ternaspmm_decode_attention (model.py:231-233) at T > 1; flash-attention style, both products on the matrix cores,
  * no workspace.  D is 64 or 128, S <= 8192.  Only enqueues. */
 void ternaspmm_prefill_attention(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
-                                 const long long* pos, terna_bf16* out, int B, int T, int H, int KV, int D, int S,
+                                 const long long* pos, int per_sequence, terna_bf16* out, int B, int T, int H, int KV, int D, int S,
                                  float scale, terna_stream stream);
 
 /* ternaspmm_decode_attention for callers that cannot allocate or bring a workspace (code under HIP graph capture
@@ -252,13 +256,13 @@ void ternaspmm_prefill_attention(const terna_bf16* q, const terna_bf16* cache_k,
  * call on a device looks the array's address up and enqueues a small clear of the counters on `stream`; make
  * that first call outside stream capture. */
 int ternaspmm_decode_attention_static(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
-                                      const long long* pos, terna_bf16* out, int B, int H, int KV, int D, int S,
+                                      const long long* pos, int per_sequence, terna_bf16* out, int B, int H, int KV, int D, int S,
                                       float scale, terna_stream stream);
 /* Both of the above in one launch for T = 1: qkv bf16 [B][(H + 2*KV)*D], cos / sin fp32 [D/2] of the new
- * token's position; writes slot pos[0] of the caches and out.  Results are bit-identical to
+ * token's position ([B][D/2] with `per_sequence`); writes slot pos[0] (pos[b]) of the caches and out.  Results are bit-identical to
  * ternaspmm_rope_kv_store followed by ternaspmm_decode_attention. */
 void ternaspmm_rope_decode_attention(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
-                                     terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
+                                     int per_sequence, terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
                                      int D, int S, float scale, int adjacent, void* workspace, terna_stream stream);
 
 /* ternaspmm_rope_decode_attention with up to six prefetch regions (no counterpart in the reference).  The attention
@@ -273,7 +277,7 @@ void ternaspmm_rope_decode_attention(const terna_bf16* qkv, const float* cos, co
  * pf_ptr / pf_bytes / pf_unit_bytes are host arrays of pf_count entries, read during the call.  Results are those of
  * ternaspmm_rope_decode_attention; nothing depends on where the prefetched bytes end up. */
 void ternaspmm_rope_decode_attention_prefetch(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
-                                              terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
+                                              int per_sequence, terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
                                               int D, int S, float scale, int adjacent, void* workspace,
                                               const void* const* pf_ptr, const long long* pf_bytes, const long long* pf_unit_bytes,
                                               int pf_count, terna_stream stream);

@@ -46,16 +46,16 @@ PROTOTYPES = {
                                          ctypes.c_int),
     "bitlinear_TernaSpMM_packed_fused_glu": ([_vp, _vp, ctypes.c_float, _vp, _vp, _vp, _ci, _vp, _vp, _ci, _ci, _ci, _vp],
                                              ctypes.c_int),
-    "ternaspmm_rope_decode_attention_prefetch": ([_vp] * 7 + [_ci] * 5 + [ctypes.c_float, _ci, _vp, _vp, _vp, _vp, _ci, _vp], None),
+    "ternaspmm_rope_decode_attention_prefetch": ([_vp] * 4 + [_ci] + [_vp] * 3 + [_ci] * 5 + [ctypes.c_float, _ci, _vp, _vp, _vp, _vp, _ci, _vp], None),
     "ternaspmm_greedy_step_state_bytes": ([_ci], ctypes.c_size_t),
     "ternaspmm_greedy_step_bf16": ([_vp, _vp, _vp, _ci, _vp, _vp, _ci, _ci, _vp], None),
     "ternaspmm_lm_head_bf16": ([_vp, _vp, _vp, _ci, _ci, _ci, _vp], None),
     "ternaspmm_argmax_bf16": ([_vp, _vp, _ci, _ci, _vp], None),
-    "ternaspmm_rope_kv_store": ([_vp] * 7 + [_ci] * 7 + [_vp], None),
-    "ternaspmm_rope_decode_attention": ([_vp] * 7 + [_ci] * 5 + [ctypes.c_float, _ci, _vp, _vp], None),
-    "ternaspmm_decode_attention": ([_vp] * 5 + [_ci] * 5 + [ctypes.c_float, _vp, _vp], None),
-    "ternaspmm_prefill_attention": ([_vp] * 5 + [_ci] * 6 + [ctypes.c_float, _vp], None),
-    "ternaspmm_decode_attention_static": ([_vp] * 5 + [_ci] * 5 + [ctypes.c_float, _vp], ctypes.c_int),
+    "ternaspmm_rope_kv_store": ([_vp] * 4 + [_ci] + [_vp] * 3 + [_ci] * 7 + [_vp], None),
+    "ternaspmm_rope_decode_attention": ([_vp] * 4 + [_ci] + [_vp] * 3 + [_ci] * 5 + [ctypes.c_float, _ci, _vp, _vp], None),
+    "ternaspmm_decode_attention": ([_vp] * 4 + [_ci, _vp] + [_ci] * 5 + [ctypes.c_float, _vp, _vp], None),
+    "ternaspmm_prefill_attention": ([_vp] * 4 + [_ci, _vp] + [_ci] * 6 + [ctypes.c_float, _vp], None),
+    "ternaspmm_decode_attention_static": ([_vp] * 4 + [_ci, _vp] + [_ci] * 5 + [ctypes.c_float, _vp], ctypes.c_int),
     "ternaspmm_attention_workspace_bytes": ([_ci, _ci, _ci], ctypes.c_longlong),
     "ternaspmm_probe_empty": ([_vp], None),
     "ternaspmm_probe_read": ([_vp, ctypes.c_longlong, _vp, _vp], None),

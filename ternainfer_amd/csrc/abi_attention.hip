@@ -89,7 +89,7 @@ int attention_splits(int B, int H, int S, const AttentionScratch& scratch)
 
 template <int D, bool ROPE, bool ADJ, int NW, bool SPLIT>
 void launch_attention_as(const uint16_t* q, uint16_t* ck, uint16_t* cv, const float* cos, const float* sin,
-                         const long long* pos, uint16_t* out, int B, int H, int KV, int S, float scale, int splits,
+                         const long long* pos, int per_seq, uint16_t* out, int B, int H, int KV, int S, float scale, int splits,
                          const AttentionScratch& scratch, const AttentionPrefetch& pf_in, hipStream_t st)
 {
     AttentionPrefetch pf = pf_in;
@@ -99,19 +99,19 @@ void launch_attention_as(const uint16_t* q, uint16_t* ck, uint16_t* cv, const fl
     if (lds > 64 * 1024) allow_dynamic_lds(kernel, 160 * 1024, "hipFuncSetAttribute(decode attention)", __LINE__);
     const int slots = attention_slots(B, H, KV);
     kernel<<<dim3(slots + pf.workgroups, splits), dim3(64 * NW), lds, st>>>(
-        q, ck, cv, pos, H, KV, S, splits, slots, attention_groups_on(H, KV) ? B * KV : 0, scale, cos, sin, out, scratch.partial,
+        q, ck, cv, pos, H, KV, S, splits, slots, attention_groups_on(H, KV) ? B * KV : 0, per_seq, scale, cos, sin, out, scratch.partial,
         scratch.arrived, pf);
 }
 
 template <bool ROPE, bool ADJ>
 void launch_attention(const uint16_t* q, uint16_t* ck, uint16_t* cv, const float* cos, const float* sin,
-                             const long long* pos, uint16_t* out, int B, int H, int KV, int D, int S, float scale,
+                             const long long* pos, int per_seq, uint16_t* out, int B, int H, int KV, int D, int S, float scale,
                              const AttentionScratch& scratch, const AttentionPrefetch& pf, hipStream_t st)
 {
     const int splits = attention_splits(B, H, S, scratch);
     const int nw = splits > 1 ? 4 : attention_waves(B, H);       // a split is a short prefix: the narrow workgroup
 #define TERNA_ATTN(DIM, NWAVES, SPLIT) \
-    launch_attention_as<DIM, ROPE, ADJ, NWAVES, SPLIT>(q, ck, cv, cos, sin, pos, out, B, H, KV, S, scale, splits, scratch, pf, st)
+    launch_attention_as<DIM, ROPE, ADJ, NWAVES, SPLIT>(q, ck, cv, cos, sin, pos, per_seq, out, B, H, KV, S, scale, splits, scratch, pf, st)
     if (D == 128) {
         if (splits > 1) TERNA_ATTN(128, 4, true);
         else if (nw == 8) TERNA_ATTN(128, 8, false);
@@ -177,7 +177,7 @@ static unsigned char* static_scratch(hipStream_t st, int line)
 extern "C" {
 
 void ternaspmm_rope_kv_store(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
-                             terna_bf16* q_out, terna_bf16* cache_k, terna_bf16* cache_v, int B, int T, int H,
+                             int per_sequence, terna_bf16* q_out, terna_bf16* cache_k, terna_bf16* cache_v, int B, int T, int H,
                              int KV, int D, int S, int adjacent, terna_stream stream)
 {
     if (B < 1 || T < 1 || H < 1 || KV < 1 || D < 2 || (D & 1) || S < 1) {
@@ -186,9 +186,9 @@ void ternaspmm_rope_kv_store(const terna_bf16* qkv, const float* cos, const floa
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (adjacent)
-        terna_rope_kv_store_kernel<true><<<dim3(B * T), dim3(256), 0, st>>>(qkv, cos, sin, pos, q_out, cache_k, cache_v, T, H, KV, D, S);
+        terna_rope_kv_store_kernel<true><<<dim3(B * T), dim3(256), 0, st>>>(qkv, cos, sin, pos, q_out, cache_k, cache_v, T, H, KV, D, S, per_sequence != 0);
     else
-        terna_rope_kv_store_kernel<false><<<dim3(B * T), dim3(256), 0, st>>>(qkv, cos, sin, pos, q_out, cache_k, cache_v, T, H, KV, D, S);
+        terna_rope_kv_store_kernel<false><<<dim3(B * T), dim3(256), 0, st>>>(qkv, cos, sin, pos, q_out, cache_k, cache_v, T, H, KV, D, S, per_sequence != 0);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_rope_kv_store", e, __LINE__);
 }
@@ -201,20 +201,20 @@ long long ternaspmm_attention_workspace_bytes(int B, int H, int D)
 }
 
 void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
-                                const long long* pos, terna_bf16* out, int B, int H, int KV, int D, int S,
+                                const long long* pos, int per_sequence, terna_bf16* out, int B, int H, int KV, int D, int S,
                                 float scale, void* workspace, terna_stream stream)
 {
     if (!attention_args_ok("ternaspmm_decode_attention", B, H, KV, D, S)) return;
     // the kernel writes the caches only in its ROPE variant
     launch_attention<false, false>(q, const_cast<uint16_t*>(cache_k), const_cast<uint16_t*>(cache_v), nullptr, nullptr, pos,
-                                   out, B, H, KV, D, S, scale, attention_scratch_of(workspace, B, H), AttentionPrefetch{},
+                                   per_sequence != 0, out, B, H, KV, D, S, scale, attention_scratch_of(workspace, B, H), AttentionPrefetch{},
                                    static_cast<hipStream_t>(stream));
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_decode_attention", e, __LINE__);
 }
 
 void ternaspmm_prefill_attention(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
-                                 const long long* pos, terna_bf16* out, int B, int T, int H, int KV, int D, int S,
+                                 const long long* pos, int per_sequence, terna_bf16* out, int B, int T, int H, int KV, int D, int S,
                                  float scale, terna_stream stream)
 {
     if (!attention_args_ok("ternaspmm_prefill_attention", B, H, KV, D, S) || T < 1 || B > 65535 || H > 65535) {
@@ -223,14 +223,14 @@ void ternaspmm_prefill_attention(const terna_bf16* q, const terna_bf16* cache_k,
     }
     const dim3 grid((T + 15) / 16, H, B);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (D == 128) terna_prefill_attention_kernel<128><<<grid, dim3(64), 0, st>>>(q, cache_k, cache_v, pos, out, T, H, KV, S, scale);
-    else terna_prefill_attention_kernel<64><<<grid, dim3(64), 0, st>>>(q, cache_k, cache_v, pos, out, T, H, KV, S, scale);
+    if (D == 128) terna_prefill_attention_kernel<128><<<grid, dim3(64), 0, st>>>(q, cache_k, cache_v, pos, out, T, H, KV, S, scale, per_sequence != 0);
+    else terna_prefill_attention_kernel<64><<<grid, dim3(64), 0, st>>>(q, cache_k, cache_v, pos, out, T, H, KV, S, scale, per_sequence != 0);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_prefill_attention", e, __LINE__);
 }
 
 int ternaspmm_decode_attention_static(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
-                                      const long long* pos, terna_bf16* out, int B, int H, int KV, int D, int S,
+                                      const long long* pos, int per_sequence, terna_bf16* out, int B, int H, int KV, int D, int S,
                                       float scale, terna_stream stream)
 {
     if (!attention_args_ok("ternaspmm_decode_attention_static", B, H, KV, D, S)) return -1;
@@ -245,27 +245,27 @@ int ternaspmm_decode_attention_static(const terna_bf16* q, const terna_bf16* cac
     if (base == nullptr) return -1;
     const AttentionScratch sc{reinterpret_cast<int*>(base), reinterpret_cast<float*>(base + kStaticCounterBytes)};
     launch_attention<false, false>(q, const_cast<uint16_t*>(cache_k), const_cast<uint16_t*>(cache_v), nullptr, nullptr, pos,
-                                   out, B, H, KV, D, S, scale, sc, AttentionPrefetch{}, st);
+                                   per_sequence != 0, out, B, H, KV, D, S, scale, sc, AttentionPrefetch{}, st);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_decode_attention_static", e, __LINE__);
     return 0;
 }
 
 void ternaspmm_rope_decode_attention(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
-                                     terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
+                                     int per_sequence, terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
                                      int D, int S, float scale, int adjacent, void* workspace, terna_stream stream)
 {
     if (!attention_args_ok("ternaspmm_rope_decode_attention", B, H, KV, D, S)) return;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const AttentionScratch scratch = attention_scratch_of(workspace, B, H);
-    if (adjacent) launch_attention<true, true>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, scratch, AttentionPrefetch{}, st);
-    else launch_attention<true, false>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, scratch, AttentionPrefetch{}, st);
+    if (adjacent) launch_attention<true, true>(qkv, cache_k, cache_v, cos, sin, pos, per_sequence != 0, out, B, H, KV, D, S, scale, scratch, AttentionPrefetch{}, st);
+    else launch_attention<true, false>(qkv, cache_k, cache_v, cos, sin, pos, per_sequence != 0, out, B, H, KV, D, S, scale, scratch, AttentionPrefetch{}, st);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_rope_decode_attention", e, __LINE__);
 }
 
 void ternaspmm_rope_decode_attention_prefetch(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
-                                              terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
+                                              int per_sequence, terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
                                               int D, int S, float scale, int adjacent, void* workspace,
                                               const void* const* pf_ptr, const long long* pf_bytes, const long long* pf_unit_bytes,
                                               int pf_count, terna_stream stream)
@@ -293,8 +293,8 @@ void ternaspmm_rope_decode_attention_prefetch(const terna_bf16* qkv, const float
     pf.workgroups = pf.count > 0 && slots < 232 ? (forced_wgs >= 0 ? forced_wgs : (256 - slots) / 8 * 8) : 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const AttentionScratch scratch = attention_scratch_of(workspace, B, H);
-    if (adjacent) launch_attention<true, true>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, scratch, pf, st);
-    else launch_attention<true, false>(qkv, cache_k, cache_v, cos, sin, pos, out, B, H, KV, D, S, scale, scratch, pf, st);
+    if (adjacent) launch_attention<true, true>(qkv, cache_k, cache_v, cos, sin, pos, per_sequence != 0, out, B, H, KV, D, S, scale, scratch, pf, st);
+    else launch_attention<true, false>(qkv, cache_k, cache_v, cos, sin, pos, per_sequence != 0, out, B, H, KV, D, S, scale, scratch, pf, st);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_rope_decode_attention_prefetch", e, __LINE__);
 }

@@ -17,8 +17,9 @@
 namespace terna {
 
 // qkv   bf16 [B*T][(H + 2*KV) * D]   row b*T + t: q heads, then k heads, then v heads
-// cosv, sinv  fp32 [T][D/2]          angle of (token t, pair j)
-// pos   int64 [T]                    cache slot of token t (same for every sequence)
+// cosv, sinv  fp32 [T][D/2]          angle of (token t, pair j)        } per_seq != 0: one row per (sequence, token),
+// pos   int64 [T]                    cache slot of token t             } [B][T][D/2] and [B][T] -- sequences of a batch
+//                                                                        with different prefix lengths
 // q_out bf16 [B][H][T][D]
 // cache_k, cache_v  bf16 [B][KV][S][D]
 // Pair j of a head is (a, b) = (x[2j], x[2j + 1]) when ADJACENT, else (x[j], x[j + D/2]):
@@ -27,14 +28,15 @@ template <bool ADJACENT>
 __global__ __launch_bounds__(256) void terna_rope_kv_store_kernel(
     const uint16_t* __restrict__ qkv, const float* __restrict__ cosv, const float* __restrict__ sinv,
     const long long* __restrict__ pos, uint16_t* __restrict__ q_out, uint16_t* __restrict__ cache_k,
-    uint16_t* __restrict__ cache_v, int T, int H, int KV, int D, int S)
+    uint16_t* __restrict__ cache_v, int T, int H, int KV, int D, int S, int per_seq)
 {
     const int row = blockIdx.x;                  // b*T + t
     const int b = row / T, t = row - b * T;
+    const int tr = per_seq ? row : t;            // row of the position / angle tables
     const int half = D >> 1;
     const int slots = H + 2 * KV;
     const uint16_t* src = qkv + static_cast<size_t>(row) * slots * D;
-    const long long slot = pos[t];
+    const long long slot = pos[tr];
     const bool slot_ok = slot >= 0 && slot < S;  // a position outside the cache writes no k / v row (q is still rotated)
     if ((half & 7) == 0) {
         // 8 pairs per thread: 16-byte loads and stores, for the 2B model one pass of 240 threads
@@ -47,8 +49,8 @@ __global__ __launch_bounds__(256) void terna_rope_kv_store_kernel(
             unpack_bf16x8(*reinterpret_cast<const u32x4*>(src + hs * D + off1), x1);
             unpack_bf16x8(*reinterpret_cast<const u32x4*>(src + hs * D + off2), x2);
             if (hs < H + KV) {
-                const f32x4* cp = reinterpret_cast<const f32x4*>(cosv + t * half + j);
-                const f32x4* sp = reinterpret_cast<const f32x4*>(sinv + t * half + j);
+                const f32x4* cp = reinterpret_cast<const f32x4*>(cosv + tr * half + j);
+                const f32x4* sp = reinterpret_cast<const f32x4*>(sinv + tr * half + j);
                 const f32x4 c0 = cp[0], c1 = cp[1], s0 = sp[0], s1 = sp[1];
                 if constexpr (ADJACENT) {
 #pragma unroll
@@ -91,7 +93,7 @@ __global__ __launch_bounds__(256) void terna_rope_kv_store_kernel(
         float o1 = x1, o2 = x2;
         if (hs < H + KV) {
 #pragma clang fp contract(off)
-            const float c = cosv[t * half + j], s = sinv[t * half + j];
+            const float c = cosv[tr * half + j], s = sinv[tr * half + j];
             o1 = x1 * c - x2 * s;
             o2 = x2 * c + x1 * s;
         }
@@ -105,7 +107,8 @@ __global__ __launch_bounds__(256) void terna_rope_kv_store_kernel(
 }
 
 // One workgroup of NW waves per (sequence, head).  q bf16 [B][H][D]; keys / values of kv head
-// h / (H/KV) at slots 0 .. pos[0]; out bf16 [B][H*D].  Dynamic LDS: decode_attention_lds_bytes().
+// h / (H/KV) at slots 0 .. pos[0] (per_seq != 0: sequence b has its own prefix, slots 0 .. pos[b], and with ROPE its
+// own angle row, cosv / sinv [B][D/2]); out bf16 [B][H*D].  Dynamic LDS: decode_attention_lds_bytes().
 // What the waves request up front covers 64 * NW slots of keys (four 16-slot tiles per wave) and
 // 4096 * NW / D slots of values, so with few workgroups on the chip (one per head) more waves mean
 // fewer dependent memory round trips.
@@ -218,8 +221,8 @@ template <int D, bool ROPE, bool ADJACENT = false, int NW = 4, bool SPLIT = fals
 __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     // what the first loads depend on comes first: the leading sixteen dwords of the arguments arrive in scalar registers
     const uint16_t* __restrict__ q, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
-    const long long* __restrict__ pos, int H, int KV, int S, int splits, int heads, int groups, float scale,
-    const float* __restrict__ cosv, const float* __restrict__ sinv, uint16_t* __restrict__ out,
+    const long long* __restrict__ pos, int H, int KV, int S, int splits, int heads, int groups, int per_seq, float scale,
+    const float* __restrict__ cosv_all, const float* __restrict__ sinv_all, uint16_t* __restrict__ out,
     float* partial, int* arrived, AttentionPrefetch pf)
 {
     static_assert(D == 64 || D == 128, "head dimension");
@@ -264,7 +267,10 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     // Prefix length: slots 0 .. pos[0].  pos comes from device memory the host cannot check, so it is clamped to the
     // cache -- the LDS score buffer and every cache address are sized by S -- and a position outside [0, S) writes no
     // cache row below (the attention then runs over the clamped prefix; its result is not meaningful, but in bounds).
-    const long long p0 = pos[0];
+    const int pb = per_seq ? b : 0;              // row of the position / angle tables
+    const long long p0 = pos[pb];
+    const float* cosv = cosv_all + pb * (D / 2);
+    const float* sinv = sinv_all + pb * (D / 2);
     const bool pos_ok = p0 >= 0 && p0 < S;
     const int n = p0 < 0 ? 1 : (p0 >= S ? S : static_cast<int>(p0) + 1);
     const uint16_t* kbase = cache_k + (static_cast<size_t>(b) * KV + kvh) * S * D;

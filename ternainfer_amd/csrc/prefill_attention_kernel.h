@@ -4,6 +4,7 @@
 //   q      bf16 [B][H][T][D]          rotated queries of the T new tokens (ternaspmm_rope_kv_store's q_out)
 //   cache  bf16 [B][KV][S][D]         keys / values; the new tokens' rows are already in their slots
 //   pos    int64 [T]                  cache slot of new token t; it sees the slots 0 .. pos[t]
+//                                     (per_seq != 0: [B][T], sequence b's token t sees 0 .. pos[b][t])
 //   out    bf16 [B*T][H*D]            row b*T + t: softmax(scale * q K^T) V, head h in columns h*D ..
 //
 // One wave per (sequence, head, block of 16 queries), flash-attention style over blocks of 32 cache slots, both
@@ -32,7 +33,7 @@ constexpr int kPrefillAttnKeys = 32;          // cache slots per block
 template <int D>
 __global__ __launch_bounds__(64) void terna_prefill_attention_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ cache_k, const uint16_t* __restrict__ cache_v,
-    const long long* __restrict__ pos, uint16_t* __restrict__ out, int T, int H, int KV, int S, float scale)
+    const long long* __restrict__ pos, uint16_t* __restrict__ out, int T, int H, int KV, int S, float scale, int per_seq)
 {
     static_assert(D == 64 || D == 128, "head size");
     constexpr int DS = D / 32;                // 32-dimension slices of a row (first product)
@@ -46,7 +47,7 @@ __global__ __launch_bounds__(64) void terna_prefill_attention_kernel(
     const int kvh = h / (H / KV);
     const int t = t0 + qi < T ? t0 + qi : T - 1;                     // rows past T repeat the last one and are not stored
     // prefix length of this lane's query, clamped to the cache (pos comes from device memory)
-    long long p64 = pos[t];
+    long long p64 = pos[(per_seq ? b * T : 0) + t];
     p64 = p64 < 0 ? 0 : (p64 >= S ? S - 1 : p64);
     const int my_last = static_cast<int>(p64);                        // last visible slot
     int n_keys = my_last + 1;

@@ -189,11 +189,13 @@ class Block:
     def forward(self, x, pending, cache_k, cache_v, pos_idx, cos, sin, mask, attn_ws=None):
         """x [B*T, dim] (T new tokens per sequence) and `pending`, the previous block's FFN output that
         has not been added to the stream yet (None for the first block): the add is part of this
-        block's first fused kernel.  cache_* [B, n_kv, S, hd]; pos_idx int64 [T] cache slots.
+        block's first fused kernel.  cache_* [B, n_kv, S, hd]; pos_idx int64 [T] cache slots shared by the
+        sequences, or [B, T] with cos / sin [B*T, hd/2]: every sequence at its own positions (generate.py:253-262).
         Returns (stream, pending) for the next block."""
         a = self.args
         bsz = cache_k.shape[0]
         t = x.shape[0] // bsz
+        per_seq = int(pos_idx.dim() == 2)
         qkv, x = self._norm_linear(self.wqkv, x, self.attention_norm, residual=pending)
         rep = a.n_heads // a.n_kv_heads
         one_token = mask is None           # the caller's rule: fused, one new token, a head size the kernel has
@@ -206,31 +208,40 @@ class Block:
                 # weights of the launches that follow through the caches meanwhile
                 ptrs, sizes, units, count = self.prefetch
                 lib.ternaspmm_rope_decode_attention_prefetch(
-                    _p(qkv), _p(cos), _p(sin), _p(pos_idx), _p(cache_k), _p(cache_v), _p(o), bsz, a.n_heads, a.n_kv_heads,
+                    _p(qkv), _p(cos), _p(sin), _p(pos_idx), per_seq, _p(cache_k), _p(cache_v), _p(o), bsz, a.n_heads, a.n_kv_heads,
                     a.head_dim, cache_k.shape[2], a.head_dim ** -0.5, int(a.rope_adjacent), _p(attn_ws), ptrs, sizes, units,
                     count, stream)
             else:
-                lib.ternaspmm_rope_decode_attention(_p(qkv), _p(cos), _p(sin), _p(pos_idx), _p(cache_k), _p(cache_v), _p(o),
+                lib.ternaspmm_rope_decode_attention(_p(qkv), _p(cos), _p(sin), _p(pos_idx), per_seq, _p(cache_k), _p(cache_v), _p(o),
                                                     bsz, a.n_heads, a.n_kv_heads, a.head_dim, cache_k.shape[2],
                                                     a.head_dim ** -0.5, int(a.rope_adjacent), _p(attn_ws), stream)
         elif self.fused:
             lib = self.wqkv.lib
             stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
             q = torch.empty((bsz, a.n_heads, t, a.head_dim), dtype=torch.bfloat16, device=x.device)
-            lib.ternaspmm_rope_kv_store(_p(qkv), _p(cos), _p(sin), _p(pos_idx), _p(q), _p(cache_k), _p(cache_v),
+            lib.ternaspmm_rope_kv_store(_p(qkv), _p(cos), _p(sin), _p(pos_idx), per_seq, _p(q), _p(cache_k), _p(cache_v),
                                         bsz, t, a.n_heads, a.n_kv_heads, a.head_dim, cache_k.shape[2],
                                         int(a.rope_adjacent), stream)
             if mask is KERNEL_ATTENTION:    # the prompt pass: the library's multi-token attention over the cache
                 o = torch.empty((bsz * t, a.n_heads * a.head_dim), dtype=torch.bfloat16, device=x.device)
-                lib.ternaspmm_prefill_attention(_p(q), _p(cache_k), _p(cache_v), _p(pos_idx), _p(o), bsz, t, a.n_heads,
+                lib.ternaspmm_prefill_attention(_p(q), _p(cache_k), _p(cache_v), _p(pos_idx), per_seq, _p(o), bsz, t, a.n_heads,
                                                 a.n_kv_heads, a.head_dim, cache_k.shape[2], a.head_dim ** -0.5, stream)
         else:
             qkv = qkv.view(bsz, t, a.n_heads + 2 * a.n_kv_heads, a.head_dim).transpose(1, 2)
             q, k, v = qkv[:, :a.n_heads], qkv[:, a.n_heads:a.n_heads + a.n_kv_heads], qkv[:, a.n_heads + a.n_kv_heads:]
-            q = apply_rope(q, cos[None, None], sin[None, None], a.rope_adjacent)
-            k = apply_rope(k, cos[None, None], sin[None, None], a.rope_adjacent)
-            cache_k.index_copy_(2, pos_idx, k)
-            cache_v.index_copy_(2, pos_idx, v)
+            if per_seq:
+                cs, sn = cos.view(bsz, 1, t, -1), sin.view(bsz, 1, t, -1)
+            else:
+                cs, sn = cos[None, None], sin[None, None]
+            q = apply_rope(q, cs, sn, a.rope_adjacent)
+            k = apply_rope(k, cs, sn, a.rope_adjacent)
+            if per_seq:
+                for b in range(bsz):
+                    cache_k[b].index_copy_(1, pos_idx[b], k[b])
+                    cache_v[b].index_copy_(1, pos_idx[b], v[b])
+            else:
+                cache_k.index_copy_(2, pos_idx, k)
+                cache_v.index_copy_(2, pos_idx, v)
         if not one_token and mask is not KERNEL_ATTENTION:
             kk = cache_k.repeat_interleave(rep, dim=1)
             vv = cache_v.repeat_interleave(rep, dim=1)
@@ -343,16 +354,18 @@ class Transformer:
         return [(torch.zeros(shape, dtype=torch.bfloat16, device=dev), torch.zeros(shape, dtype=torch.bfloat16, device=dev))
                 for _ in range(a.n_layers)]
 
-    def forward(self, tokens: torch.Tensor, cache, pos_idx: torch.Tensor, trace=None) -> torch.Tensor:
-        """tokens int64 [B, T]; pos_idx int64 [T] = cache slots of the new tokens.  Returns logits [B, vocab]
-        of the last new token.  `trace`, if given, is called after every block as
+    def forward(self, tokens: torch.Tensor, cache, pos_idx: torch.Tensor, trace=None, last_idx=None) -> torch.Tensor:
+        """tokens int64 [B, T]; pos_idx int64 [T] = cache slots of the new tokens, the same for every sequence, or
+        [B, T] = every sequence at its own slots (a batch of different prefix lengths).  Returns logits [B, vocab]
+        of the last new token -- of new token last_idx[b] of sequence b when `last_idx` (int64 [B]) is given: the
+        prompt pass of prompts padded to one length.  `trace`, if given, is called after every block as
         trace(index, stream_in, pending_in, stream_out, pending_out) (layer-by-layer checks against a golden)."""
         a = self.args
         bsz, t = tokens.shape
         max_seq = cache[0][0].shape[2]
         dev = tokens.device
-        rows = self.rope_tables(max_seq, dev).index_select(0, pos_idx)         # fp32 [T, 2, head_dim / 2]
-        cos, sin = rows[:, 0].contiguous(), rows[:, 1].contiguous()           # views when T == 1
+        rows = self.rope_tables(max_seq, dev).index_select(0, pos_idx.reshape(-1))   # fp32 [T | B*T, 2, head_dim / 2]
+        cos, sin = rows[:, 0].contiguous(), rows[:, 1].contiguous()           # views when one row
         mask = None
         kernels_fit = self.layers[0].fused and a.head_dim in (64, 128) and max_seq <= 8192 and tokens.is_cuda
         one_launch_attention = kernels_fit and t == 1
@@ -360,7 +373,8 @@ class Transformer:
             mask = KERNEL_ATTENTION
         elif not one_launch_attention:
             # causal over cache slots: new token at slot p sees slots <= p
-            mask = (torch.arange(max_seq, device=dev)[None, :] <= pos_idx[:, None])[None, None]
+            seen = torch.arange(max_seq, device=dev) <= pos_idx[..., None]    # [T | B, T][S]
+            mask = seen[:, None] if pos_idx.dim() == 2 else seen[None, None]
         x = self.tok_embeddings[tokens.reshape(-1)]
         pending = None
         attn_ws = self.attention_workspace(bsz) if one_launch_attention else None     # layers run one after another: shared
@@ -369,7 +383,10 @@ class Transformer:
             x, pending = layer.forward(x, pending, ck, cv, pos_idx, cos, sin, mask, attn_ws)
             if trace is not None:
                 trace(index, x_in, pending_in, x, pending)
-        if t > 1:                                                             # only the last new token feeds the head
+        if last_idx is not None:                                              # padded prompts: each sequence's own last token
+            pick = torch.arange(bsz, device=dev) * t + last_idx
+            x, pending = x.index_select(0, pick), pending.index_select(0, pick)
+        elif t > 1:                                                           # only the last new token feeds the head
             x, pending = x.view(bsz, t, a.dim)[:, -1].contiguous(), pending.view(bsz, t, a.dim)[:, -1].contiguous()
         if self.layers[0].fused and x.is_cuda:                                # last residual add + final norm: one launch
             x, _ = rmsnorm_quant(x, self.norm, a.norm_eps, residual=pending, quant=False)
@@ -381,14 +398,20 @@ class Transformer:
 
 
 @torch.inference_mode()
-def greedy_decode(model: Transformer, prompt: torch.Tensor, gen_tokens: int, use_graph: bool = True):
+def greedy_decode(model: Transformer, prompt: torch.Tensor, gen_tokens: int, use_graph: bool = True, prompt_lens=None):
     """Prefill `prompt` [B, P], then `gen_tokens` greedy steps.  Returns (tokens [B, gen_tokens],
     prefill seconds, decode seconds).  The decode step (model forward + argmax + position bump) is
-    captured once and replayed, so the host issues one graph launch per token."""
+    captured once and replayed, so the host issues one graph launch per token.
+    `prompt_lens` (int64 [B], each 1 .. P): the prompts have different lengths and are padded to P with any token
+    (generate.py:244-262): sequence b's first generated token comes from its prompt token prompt_lens[b] - 1, and
+    its n-th decode step runs at cache slot prompt_lens[b] + n -- every sequence at its own position."""
     bsz, plen = prompt.shape
     cache = model.make_cache(bsz, plen + gen_tokens)
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
     slots = torch.arange(plen, device="cuda")
+    if prompt_lens is not None:
+        return _greedy_decode_ragged(model, prompt, prompt_lens.to(device="cuda", dtype=torch.int64), gen_tokens, use_graph,
+                                     cache, slots, ev)
     if use_graph:
         # the prompt pass as a graph too (generate.py:100-144): warm up on a side stream, capture, replay
         side = torch.cuda.Stream()
@@ -430,6 +453,50 @@ def greedy_decode(model: Transformer, prompt: torch.Tensor, gen_tokens: int, use
         with torch.cuda.graph(graph):
             step()
         tok.copy_(snap[0]); counters.copy_(snap[1])
+    torch.cuda.synchronize()
+    ev[2].record()
+    for _ in range(gen_tokens):
+        if graph is not None:
+            graph.replay()
+        else:
+            step()
+    ev[3].record()
+    torch.cuda.synchronize()
+    return out, ev[0].elapsed_time(ev[1]) * 1e-3, ev[2].elapsed_time(ev[3]) * 1e-3
+
+
+def _greedy_decode_ragged(model, prompt, prompt_lens, gen_tokens, use_graph, cache, slots, ev):
+    """greedy_decode for prompts of different lengths: the prompt pass runs on the padded prompts (a padding token's
+    cache rows are overwritten by the decode steps before any query can see them), the decode steps carry one cache
+    position per sequence."""
+    bsz = prompt.shape[0]
+    ev[0].record()
+    logits = model.forward(prompt, cache, slots, last_idx=prompt_lens - 1)
+    tok = argmax_rows(logits.contiguous())                                    # int64 [B, 1]
+    ev[1].record()
+    seq_pos = prompt_lens.clone().view(bsz, 1)                                # cache slot of every sequence's next token
+    counters = torch.tensor([0, 1], dtype=torch.int64, device="cuda")         # [1]: tokens stored in the history
+    out = torch.empty((bsz, gen_tokens), dtype=torch.int64, device="cuda")
+    out[:, 0:1] = tok
+    state = greedy_step_state(bsz)
+
+    def step():
+        greedy_step(model.forward(tok, cache, seq_pos), tok, out, counters, state)
+        seq_pos.add_(1)
+
+    graph = None
+    if use_graph:
+        snap = (tok.clone(), counters.clone(), seq_pos.clone())
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        tok.copy_(snap[0]); counters.copy_(snap[1]); seq_pos.copy_(snap[2])
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        tok.copy_(snap[0]); counters.copy_(snap[1]); seq_pos.copy_(snap[2])
     torch.cuda.synchronize()
     ev[2].record()
     for _ in range(gen_tokens):

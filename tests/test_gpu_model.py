@@ -95,6 +95,45 @@ def test_toy_model_greedy_decode_graph_equals_eager():
     assert torch.equal(a, c)
 
 
+@pytest.mark.parametrize("head_dim,prefetch", [(64, False), (128, True)])
+def test_toy_model_prompts_of_different_lengths_in_one_batch(head_dim, prefetch):
+    """Three prompts of different lengths, padded to one length and decoded together with every sequence at its own
+    cache position (generate.py:244-305 hands its attention one kv_seqlen per sequence), against each prompt decoded
+    alone: the same tokens, eager and as a replayed graph; and against the forward without the fused kernels (torch
+    RoPE, per-sequence masks, SDPA) on the first decode step."""
+    from ternainfer_amd.model import ModelArgs, Transformer, greedy_decode
+    args = ModelArgs(dim=4 * head_dim, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=1024, ffn_dim=384)
+    model = Transformer(args, seed=31, act="int8")
+    model.enable_prefetch(prefetch)
+    lens = [5, 12, 9]
+    gen = torch.Generator().manual_seed(32)
+    prompts = [torch.randint(0, args.vocab_size, (1, n), generator=gen).cuda() for n in lens]
+    padded = torch.full((3, max(lens)), 7, dtype=torch.int64, device="cuda")
+    for i, p in enumerate(prompts):
+        padded[i, :lens[i]] = p[0]
+    print(f"[case] toy model, ragged batch head_dim={head_dim} prefetch={prefetch}", flush=True)
+    alone = torch.cat([greedy_decode(model, p, 8, use_graph=False)[0] for p in prompts])
+    together, _, _ = greedy_decode(model, padded, 8, use_graph=False, prompt_lens=torch.tensor(lens))
+    assert torch.equal(alone, together)
+    replayed, _, _ = greedy_decode(model, padded, 8, use_graph=True, prompt_lens=torch.tensor(lens))
+    assert torch.equal(alone, replayed)
+    # one decode step with per-sequence positions: fused kernels against torch ops
+    with torch.inference_mode():
+        outs = []
+        for fused in (True, False):
+            for blk in model.layers:
+                blk.fused = fused
+            cache = model.make_cache(3, 24)
+            model.forward(padded, cache, torch.arange(max(lens), device="cuda"))
+            seq_pos = torch.tensor(lens, device="cuda").view(3, 1)
+            outs.append(model.forward(together[:, :1].contiguous(), cache, seq_pos).float())
+        for blk in model.layers:
+            blk.fused = True
+    err = (outs[0] - outs[1]).abs().max().item()
+    assert err <= 3e-2 * outs[1].abs().max().item()
+    assert torch.nn.functional.cosine_similarity(outs[0].flatten(), outs[1].flatten(), dim=0).item() > 0.999
+
+
 def test_toy_model_prompt_pass_kernel_attention_sdpa_and_graph_replays():
     """The prompt pass through the library's multi-token attention against the same pass through PyTorch's SDPA, and
     the captured prompt graph against eager execution on several replays with eager work and synchronisations between

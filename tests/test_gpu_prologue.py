@@ -204,7 +204,7 @@ def test_rope_kv_store(lib, b, t, h, kv, d, s_max, adjacent):
     qd, ckd, cvd = torch.zeros((b, h, t, d), dtype=torch.int16, device="cuda"), _dev(ck), _dev(cv)
     xd, cd, sd, pd = _dev(qkv), _dev(cos), _dev(sin), _dev(pos)      # named: they must outlive the launch
     print(f"[case] rope_kv_store b={b} t={t} h={h} kv={kv} d={d} adjacent={adjacent}", flush=True)
-    lib.ternaspmm_rope_kv_store(_vp(xd), _vp(cd), _vp(sd), _vp(pd), _vp(qd), _vp(ckd), _vp(cvd), b, t, h, kv, d,
+    lib.ternaspmm_rope_kv_store(_vp(xd), _vp(cd), _vp(sd), _vp(pd), 0, _vp(qd), _vp(ckd), _vp(cvd), b, t, h, kv, d,
                                 s_max, adjacent, None)
     torch.cuda.synchronize()
     x = qkv.reshape(b, t, h + 2 * kv, d)
@@ -236,7 +236,7 @@ def test_decode_attention(lib, b, h, kv, d, s_max, n, split):
     qd, kd, vd, pd = _dev(q), _dev(k), _dev(v), _dev(pos)            # named: they must outlive the launch
     ws = _attn_workspace(lib, b, h, d) if split else None
     print(f"[case] decode attention b={b} h={h} kv={kv} d={d} S={s_max} n={n} split={split}", flush=True)
-    lib.ternaspmm_decode_attention(_vp(qd), _vp(kd), _vp(vd), _vp(pd), _vp(od), b, h, kv, d, s_max, float(d) ** -0.5, _vp(ws), None)
+    lib.ternaspmm_decode_attention(_vp(qd), _vp(kd), _vp(vd), _vp(pd), 0, _vp(od), b, h, kv, d, s_max, float(d) ** -0.5, _vp(ws), None)
     torch.cuda.synchronize()
     got = O.bf16_bits_to_f32(od.cpu().numpy().view(np.uint16)).reshape(b, h, d).astype(np.float64)
     want = O.attention_one_token(q, k, v, n, float(d) ** -0.5)
@@ -247,7 +247,7 @@ def test_decode_attention(lib, b, h, kv, d, s_max, n, split):
         counters = ws[:b * h * 4].view(torch.int32)
         assert int(counters.abs().sum().item()) == 0
         od2 = torch.zeros_like(od)
-        lib.ternaspmm_decode_attention(_vp(qd), _vp(kd), _vp(vd), _vp(pd), _vp(od2), b, h, kv, d, s_max, float(d) ** -0.5, _vp(ws), None)
+        lib.ternaspmm_decode_attention(_vp(qd), _vp(kd), _vp(vd), _vp(pd), 0, _vp(od2), b, h, kv, d, s_max, float(d) ** -0.5, _vp(ws), None)
         torch.cuda.synchronize()
         assert torch.equal(od, od2)                      # merged in split order: the same bits whoever arrives last
 
@@ -268,7 +268,7 @@ def test_prefill_attention(lib, b, h, kv, d, s_max, first, t):
     od = torch.full((b * t, h * d), 0x7FC0, dtype=torch.int16, device="cuda")
     qd, kd, vd, pd = _dev(q), _dev(k), _dev(v), _dev(pos)
     print(f"[case] prefill attention b={b} h={h} kv={kv} d={d} S={s_max} first={first} t={t}", flush=True)
-    lib.ternaspmm_prefill_attention(_vp(qd), _vp(kd), _vp(vd), _vp(pd), _vp(od), b, t, h, kv, d, s_max, float(d) ** -0.5, None)
+    lib.ternaspmm_prefill_attention(_vp(qd), _vp(kd), _vp(vd), _vp(pd), 0, _vp(od), b, t, h, kv, d, s_max, float(d) ** -0.5, None)
     torch.cuda.synchronize()
     got = O.bf16_bits_to_f32(od.cpu().numpy().view(np.uint16)).reshape(b, t, h, d).astype(np.float64)
     want = O.attention_new_tokens(q, k, v, pos, float(d) ** -0.5)
@@ -420,13 +420,13 @@ def test_rope_decode_attention_equals_the_two_launches(lib, b, h, kv, d, s_max, 
     ck1, cv1 = _dev(k0), _dev(v0)
     q1 = torch.zeros((b, h, 1, d), dtype=torch.int16, device="cuda")
     o1 = torch.zeros((b, h * d), dtype=torch.int16, device="cuda")
-    lib.ternaspmm_rope_kv_store(_vp(xd), _vp(cd), _vp(sd), _vp(pd), _vp(q1), _vp(ck1), _vp(cv1), b, 1, h, kv, d, s_max, adjacent, None)
-    lib.ternaspmm_decode_attention(_vp(q1), _vp(ck1), _vp(cv1), _vp(pd), _vp(o1), b, h, kv, d, s_max, scale, _vp(ws1), None)
+    lib.ternaspmm_rope_kv_store(_vp(xd), _vp(cd), _vp(sd), _vp(pd), 0, _vp(q1), _vp(ck1), _vp(cv1), b, 1, h, kv, d, s_max, adjacent, None)
+    lib.ternaspmm_decode_attention(_vp(q1), _vp(ck1), _vp(cv1), _vp(pd), 0, _vp(o1), b, h, kv, d, s_max, scale, _vp(ws1), None)
     # one launch
     ck2, cv2 = _dev(k0), _dev(v0)
     o2 = torch.zeros((b, h * d), dtype=torch.int16, device="cuda")
     print(f"[case] rope + decode attention b={b} h={h} kv={kv} d={d} S={s_max} n={n} adjacent={adjacent}", flush=True)
-    lib.ternaspmm_rope_decode_attention(_vp(xd), _vp(cd), _vp(sd), _vp(pd), _vp(ck2), _vp(cv2), _vp(o2), b, h, kv, d, s_max,
+    lib.ternaspmm_rope_decode_attention(_vp(xd), _vp(cd), _vp(sd), _vp(pd), 0, _vp(ck2), _vp(cv2), _vp(o2), b, h, kv, d, s_max,
                                         scale, adjacent, _vp(ws2), None)
     torch.cuda.synchronize()
     assert torch.equal(ck1, ck2) and torch.equal(cv1, cv2)
@@ -457,10 +457,10 @@ def test_rope_decode_attention_with_prefetch_regions(lib, b, h, kv, d, s_max, n)
     ptrs = (ctypes.c_void_p * count)(*([r.data_ptr() for r in regions] + [None]))           # the last one is skipped
     sizes = (ctypes.c_longlong * count)(*([r.numel() * 4 for r in regions] + [1024]))
     unit_arr = (ctypes.c_longlong * count)(*(units + [16]))
-    lib.ternaspmm_rope_decode_attention(_vp(xd), _vp(cd), _vp(sd), _vp(pd), _vp(ck1), _vp(cv1), _vp(o1), b, h, kv, d, s_max,
+    lib.ternaspmm_rope_decode_attention(_vp(xd), _vp(cd), _vp(sd), _vp(pd), 0, _vp(ck1), _vp(cv1), _vp(o1), b, h, kv, d, s_max,
                                         scale, 1, None, None)
     print(f"[case] rope + decode attention with prefetch b={b} h={h} d={d} n={n}", flush=True)
-    lib.ternaspmm_rope_decode_attention_prefetch(_vp(xd), _vp(cd), _vp(sd), _vp(pd), _vp(ck2), _vp(cv2), _vp(o2), b, h, kv, d,
+    lib.ternaspmm_rope_decode_attention_prefetch(_vp(xd), _vp(cd), _vp(sd), _vp(pd), 0, _vp(ck2), _vp(cv2), _vp(o2), b, h, kv, d,
                                                  s_max, scale, 1, None, ptrs, sizes, unit_arr, count, None)
     torch.cuda.synchronize()
     assert torch.equal(o1, o2) and torch.equal(ck1, ck2) and torch.equal(cv1, cv2)
@@ -505,3 +505,145 @@ def test_greedy_step(lib, b, v, hist):
     T.greedy_step(xd, tok.fill_(-1), None, None, state)
     torch.cuda.synchronize()
     assert (tok.cpu().numpy().ravel() == want).all()
+
+
+# ------------------------------------------------------------------ per-sequence positions (per_sequence = 1)
+def _angles(pos, d):
+    ang = (pos.reshape(-1)[:, None] * (1.0 / 500000.0 ** (np.arange(0, d, 2) / d))[None, :]).astype(np.float32)
+    return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+
+
+@pytest.mark.parametrize("adjacent", [0, 1])
+@pytest.mark.parametrize("b,t,h,kv,d,s_max", [(3, 1, 20, 5, 128, 64), (2, 7, 4, 2, 64, 40), (4, 3, 4, 2, 24, 16)])
+def test_rope_kv_store_per_sequence(lib, b, t, h, kv, d, s_max, adjacent):
+    """Every sequence at its own cache slots and angles (pos [B][T], cos / sin [B][T][D/2]): sequence by sequence
+    against the rotation of the oracle, rows of other slots untouched."""
+    rope = O.rope_adjacent if adjacent else O.rope_rotate_half
+    rng = np.random.default_rng(1700 + b + t)
+    qkv = make_bf16_activations(b * t, (h + 2 * kv) * d, 1701 + t)
+    pos = np.stack([np.sort(rng.choice(s_max, t, replace=False)) for _ in range(b)]).astype(np.int64)      # [B][T]
+    cos, sin = _angles(pos, d)                                                                               # [B*T][D/2]
+    sentinel = 0x7FC1
+    ck = np.full((b, kv, s_max, d), sentinel, np.uint16)
+    cv = np.full((b, kv, s_max, d), sentinel, np.uint16)
+    qd, ckd, cvd = torch.zeros((b, h, t, d), dtype=torch.int16, device="cuda"), _dev(ck), _dev(cv)
+    xd, cd, sd, pd = _dev(qkv), _dev(cos), _dev(sin), _dev(pos)
+    print(f"[case] rope_kv_store per sequence b={b} t={t} h={h} kv={kv} d={d} adjacent={adjacent}", flush=True)
+    lib.ternaspmm_rope_kv_store(_vp(xd), _vp(cd), _vp(sd), _vp(pd), 1, _vp(qd), _vp(ckd), _vp(cvd), b, t, h, kv, d,
+                                s_max, adjacent, None)
+    torch.cuda.synchronize()
+    x = qkv.reshape(b, t, h + 2 * kv, d)
+    c4, s4 = cos.reshape(b, t, 1, d // 2), sin.reshape(b, t, 1, d // 2)
+    want_q = rope(x[:, :, :h], c4, s4).transpose(0, 2, 1, 3)
+    want_k = rope(x[:, :, h:h + kv], c4, s4).transpose(0, 2, 1, 3)
+    want_v = x[:, :, h + kv:].transpose(0, 2, 1, 3)
+    got_q = qd.cpu().numpy().view(np.uint16)
+    got_k, got_v = ckd.cpu().numpy().view(np.uint16), cvd.cpu().numpy().view(np.uint16)
+    assert (got_q == want_q).all()
+    for i in range(b):
+        assert (got_k[i][:, pos[i]] == want_k[i]).all() and (got_v[i][:, pos[i]] == want_v[i]).all()
+        untouched = np.setdiff1d(np.arange(s_max), pos[i])
+        assert (got_k[i][:, untouched] == sentinel).all() and (got_v[i][:, untouched] == sentinel).all()
+
+
+@pytest.mark.parametrize("split", [False, True])
+@pytest.mark.parametrize("b,h,kv,d,s_max,lens", [(3, 20, 5, 128, 256, (1, 160, 77)), (8, 20, 5, 128, 1024, (1000, 3, 512, 17, 1024, 64, 65, 700)),
+                                                 (2, 4, 2, 64, 1040, (1030, 12))])
+def test_decode_attention_per_sequence(lib, b, h, kv, d, s_max, lens, split):
+    """Sequences of different prefix lengths in one call (pos [B]): every sequence against the oracle at its own
+    length, and bit-identical to a call of its own with the shared-position form."""
+    q = make_bf16_activations(b * h, d, 1710 + b).reshape(b, h, d)
+    k = make_bf16_activations(b * kv * s_max, d, 1711 + b).reshape(b, kv, s_max, d)
+    v = make_bf16_activations(b * kv * s_max, d, 1712 + b, outlier_frac=0.01).reshape(b, kv, s_max, d)
+    pos = np.array(lens, np.int64) - 1
+    od = torch.zeros((b, h * d), dtype=torch.int16, device="cuda")
+    qd, kd, vd, pd = _dev(q), _dev(k), _dev(v), _dev(pos)
+    ws = _attn_workspace(lib, b, h, d) if split else None
+    print(f"[case] decode attention per sequence b={b} h={h} d={d} S={s_max} lens={lens} split={split}", flush=True)
+    lib.ternaspmm_decode_attention(_vp(qd), _vp(kd), _vp(vd), _vp(pd), 1, _vp(od), b, h, kv, d, s_max, float(d) ** -0.5, _vp(ws), None)
+    torch.cuda.synchronize()
+    got = O.bf16_bits_to_f32(od.cpu().numpy().view(np.uint16)).reshape(b, h, d).astype(np.float64)
+    for i in range(b):
+        want = O.attention_one_token(q[i:i + 1], k[i:i + 1], v[i:i + 1], lens[i], float(d) ** -0.5)[0]
+        tol = 2.0 ** -7 * np.abs(want).max(axis=-1, keepdims=True) + 1e-6
+        assert (np.abs(got[i] - want) <= tol).all(), (i, float((np.abs(got[i] - want) / tol).max()))
+    # the same sequences one at a time, shared-position form: the same bits (a head's work does not depend on the batch)
+    ws1 = _attn_workspace(lib, 1, h, d) if split else None
+    for i in range(b):
+        o1 = torch.zeros((1, h * d), dtype=torch.int16, device="cuda")
+        p1 = _dev(pos[i:i + 1])
+        lib.ternaspmm_decode_attention(_vp(qd[i:i + 1]), _vp(kd[i:i + 1]), _vp(vd[i:i + 1]), _vp(p1), 0, _vp(o1), 1, h, kv, d, s_max,
+                                       float(d) ** -0.5, _vp(ws1), None)
+        torch.cuda.synchronize()
+        if not split:                                    # with a workspace the split count depends on B: other summation order
+            assert torch.equal(o1[0], od[i])
+    if split:
+        assert int(ws[:b * h * 4].view(torch.int32).abs().sum().item()) == 0
+
+
+@pytest.mark.parametrize("b,h,kv,d,s_max,firsts,t", [(3, 20, 5, 128, 200, (0, 60, 17), 40), (2, 4, 2, 64, 300, (100, 0), 50),
+                                                    (4, 8, 8, 128, 64, (5, 0, 33, 20), 1)])
+def test_prefill_attention_per_sequence(lib, b, h, kv, d, s_max, firsts, t):
+    """T new tokens per sequence, sequence b at the slots firsts[b] .. firsts[b] + T - 1 (pos [B][T]); slots past each
+    sequence's newest token hold NaN bit patterns."""
+    q = make_bf16_activations(b * h * t, d, 1720 + t).reshape(b, h, t, d)
+    k = make_bf16_activations(b * kv * s_max, d, 1721 + t).reshape(b, kv, s_max, d)
+    v = make_bf16_activations(b * kv * s_max, d, 1722 + t, outlier_frac=0.01).reshape(b, kv, s_max, d)
+    for i in range(b):
+        k[i, :, firsts[i] + t:] = 0x7FC0
+        v[i, :, firsts[i] + t:] = 0x7FC0
+    pos = np.stack([np.arange(f, f + t) for f in firsts]).astype(np.int64)
+    od = torch.full((b * t, h * d), 0x7FC0, dtype=torch.int16, device="cuda")
+    qd, kd, vd, pd = _dev(q), _dev(k), _dev(v), _dev(pos)
+    print(f"[case] prefill attention per sequence b={b} h={h} d={d} S={s_max} firsts={firsts} t={t}", flush=True)
+    lib.ternaspmm_prefill_attention(_vp(qd), _vp(kd), _vp(vd), _vp(pd), 1, _vp(od), b, t, h, kv, d, s_max, float(d) ** -0.5, None)
+    torch.cuda.synchronize()
+    got = O.bf16_bits_to_f32(od.cpu().numpy().view(np.uint16)).reshape(b, t, h, d).astype(np.float64)
+    assert np.isfinite(got).all()
+    for i in range(b):
+        want = O.attention_new_tokens(q[i:i + 1], k[i:i + 1], v[i:i + 1], pos[i], float(d) ** -0.5)[0]
+        tol = 2.0 ** -7 * np.abs(want).max(axis=-1, keepdims=True) + 1e-6
+        assert (np.abs(got[i] - want) <= tol).all(), (i, float((np.abs(got[i] - want) / tol).max()))
+
+
+@pytest.mark.parametrize("prefetch", [False, True])
+@pytest.mark.parametrize("adjacent", [0, 1])
+@pytest.mark.parametrize("b,h,kv,d,s_max,lens", [(3, 20, 5, 128, 300, (290, 1, 45)), (2, 4, 2, 64, 40, (17, 40)),
+                                                 (8, 20, 5, 128, 384, (200, 201, 1, 384, 100, 7, 300, 64))])
+def test_rope_decode_attention_per_sequence(lib, b, h, kv, d, s_max, lens, adjacent, prefetch):
+    """One launch with per-sequence positions against ternaspmm_rope_kv_store + ternaspmm_decode_attention with the
+    same positions (outputs and both caches bit-identical), and against one shared-position call per sequence."""
+    qkv = make_bf16_activations(b, (h + 2 * kv) * d, 1731 + b)
+    k0 = make_bf16_activations(b * kv * s_max, d, 1732 + b).reshape(b, kv, s_max, d)
+    v0 = make_bf16_activations(b * kv * s_max, d, 1733 + b, outlier_frac=0.01).reshape(b, kv, s_max, d)
+    pos = np.array(lens, np.int64) - 1
+    cos, sin = _angles(pos, d)                                                    # [B][D/2]
+    xd, cd, sd, pd = _dev(qkv), _dev(cos), _dev(sin), _dev(pos)
+    scale = float(d) ** -0.5
+    ck1, cv1, ck2, cv2 = _dev(k0), _dev(v0), _dev(k0), _dev(v0)
+    q1 = torch.zeros((b, h, 1, d), dtype=torch.int16, device="cuda")
+    o1 = torch.zeros((b, h * d), dtype=torch.int16, device="cuda")
+    o2 = torch.zeros_like(o1)
+    lib.ternaspmm_rope_kv_store(_vp(xd), _vp(cd), _vp(sd), _vp(pd), 1, _vp(q1), _vp(ck1), _vp(cv1), b, 1, h, kv, d, s_max, adjacent, None)
+    lib.ternaspmm_decode_attention(_vp(q1), _vp(ck1), _vp(cv1), _vp(pd), 1, _vp(o1), b, h, kv, d, s_max, scale, None, None)
+    print(f"[case] rope + decode attention per sequence b={b} h={h} d={d} lens={lens} adjacent={adjacent} prefetch={prefetch}", flush=True)
+    if prefetch:
+        region = torch.zeros(40 * 2560, dtype=torch.int32, device="cuda")
+        ptrs = (ctypes.c_void_p * 1)(region.data_ptr())
+        sizes = (ctypes.c_longlong * 1)(region.numel() * 4)
+        units = (ctypes.c_longlong * 1)(10240)
+        lib.ternaspmm_rope_decode_attention_prefetch(_vp(xd), _vp(cd), _vp(sd), _vp(pd), 1, _vp(ck2), _vp(cv2), _vp(o2), b, h, kv, d,
+                                                     s_max, scale, adjacent, None, ptrs, sizes, units, 1, None)
+    else:
+        lib.ternaspmm_rope_decode_attention(_vp(xd), _vp(cd), _vp(sd), _vp(pd), 1, _vp(ck2), _vp(cv2), _vp(o2), b, h, kv, d, s_max,
+                                            scale, adjacent, None, None)
+    torch.cuda.synchronize()
+    assert torch.equal(ck1, ck2) and torch.equal(cv1, cv2) and torch.equal(o1, o2)
+    for i in range(b):                                   # sequence i alone, shared-position form
+        ck3, cv3 = _dev(k0[i:i + 1]), _dev(v0[i:i + 1])
+        o3 = torch.zeros((1, h * d), dtype=torch.int16, device="cuda")
+        c3, s3, p3 = _dev(cos[i:i + 1]), _dev(sin[i:i + 1]), _dev(pos[i:i + 1])
+        lib.ternaspmm_rope_decode_attention(_vp(xd[i:i + 1]), _vp(c3), _vp(s3), _vp(p3), 0, _vp(ck3), _vp(cv3), _vp(o3), 1, h, kv, d,
+                                            s_max, scale, adjacent, None, None)
+        torch.cuda.synchronize()
+        assert torch.equal(o3[0], o2[i]) and torch.equal(ck3[0], ck2[i]) and torch.equal(cv3[0], cv2[i])

@@ -30,10 +30,10 @@ def _case(lib, b, h, kv, d, s_max, n, seed):
     scale = float(d) ** -0.5
     ws = torch.zeros(lib.ternaspmm_attention_workspace_bytes(b, h, d), dtype=torch.int8, device="cuda")
     want = torch.zeros((b, h * d), dtype=torch.int16, device="cuda")
-    lib.ternaspmm_decode_attention(_vp(qd), _vp(kd), _vp(vd), _vp(pd), _vp(want), b, h, kv, d, s_max, scale, _vp(ws), None)
+    lib.ternaspmm_decode_attention(_vp(qd), _vp(kd), _vp(vd), _vp(pd), 0, _vp(want), b, h, kv, d, s_max, scale, _vp(ws), None)
     got = torch.full((b, h * d), -1, dtype=torch.int16, device="cuda")
     print(f"[case] decode attention, static scratch: b={b} h={h} kv={kv} d={d} S={s_max} n={n}", flush=True)
-    rc = lib.ternaspmm_decode_attention_static(_vp(qd), _vp(kd), _vp(vd), _vp(pd), _vp(got), b, h, kv, d, s_max, scale, None)
+    rc = lib.ternaspmm_decode_attention_static(_vp(qd), _vp(kd), _vp(vd), _vp(pd), 0, _vp(got), b, h, kv, d, s_max, scale, None)
     torch.cuda.synchronize()
     assert rc == 0
     assert torch.equal(got, want), f"static-scratch output differs (b={b} h={h} S={s_max} n={n})"
@@ -57,7 +57,7 @@ def test_static_scratch_entry_point_rejects_what_does_not_fit(capfd):
     lib = _lib.load()
     out = torch.zeros(16, dtype=torch.int16, device="cuda")
     # 13 * 20 = 260 heads > 256: refused before any pointer is touched
-    assert lib.ternaspmm_decode_attention_static(None, None, None, None, _vp(out), 13, 20, 5, 128, 1024, 0.1, None) == -1
+    assert lib.ternaspmm_decode_attention_static(None, None, None, None, 0, _vp(out), 13, 20, 5, 128, 1024, 0.1, None) == -1
     assert "exceed" in capfd.readouterr().err
-    assert lib.ternaspmm_decode_attention_static(None, None, None, None, _vp(out), 1, 20, 5, 96, 1024, 0.1, None) == -1
+    assert lib.ternaspmm_decode_attention_static(None, None, None, None, 0, _vp(out), 1, 20, 5, 96, 1024, 0.1, None) == -1
     torch.cuda.synchronize()
