@@ -43,10 +43,11 @@ __device__ __forceinline__ u32x4 expand_chunk_bf16(uint32_t t)
 }
 
 // Sixteen int8 weights (+-64 / 0) of a packed word in column order: dword q holds columns 4q .. 4q+3.
-__device__ __forceinline__ i32x4 expand_word_i8(uint32_t d)
+// `mask`: kTopFieldMask, or 0 for a lane whose word stands for columns that do not exist (all weights zero).
+__device__ __forceinline__ i32x4 expand_word_i8(uint32_t d, uint32_t mask = kTopFieldMask)
 {
-    return i32x4{static_cast<int>((d << 6) & kTopFieldMask), static_cast<int>((d << 4) & kTopFieldMask),
-                 static_cast<int>((d << 2) & kTopFieldMask), static_cast<int>(d & kTopFieldMask)};
+    return i32x4{static_cast<int>((d << 6) & mask), static_cast<int>((d << 4) & mask),
+                 static_cast<int>((d << 2) & mask), static_cast<int>(d & mask)};
 }
 
 // Repack table: (nonzero nibble, next 4 sign bits of the stream) -> the nibble's four 2-bit codes

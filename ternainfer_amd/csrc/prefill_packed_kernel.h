@@ -488,12 +488,13 @@ __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) voi
         for (int b = 0; b < MB; ++b) r.b[b] = *reinterpret_cast<const u32x4*>(stage + b_off[g] + b * 4096);
     };
     // One 16-column group: expand the NA weight operands and issue NA*MB MFMAs against `bcur`.
+    uint32_t wmask = kTopFieldMask;                          // int8: 0 in the lanes without a tile (odd tile count, last step)
     auto mma_group = [&](const RawW& rw, auto gc, const BOps& bcur) {
         constexpr int g = decltype(gc)::value;
 #pragma unroll
         for (int a = 0; a < NA; ++a) {
             if constexpr (I8) {
-                const i32x4 af = expand_word_i8(rw.w[a][g]);
+                const i32x4 af = expand_word_i8(rw.w[a][g], wmask);
 #pragma unroll
                 for (int b = 0; b < MB; ++b)
                     acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, __builtin_bit_cast(i32x4, bcur.b[b]), acc[a][b], 0, 0, 0);
@@ -538,10 +539,7 @@ __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) voi
         const int st_next = next_stage(st_mma);
 #pragma unroll
         for (int a = 0; a < NA; ++a) landed(w.w[a]);
-        if (half_tail && k == steps - 1 && kb) {
-#pragma unroll
-            for (int a = 0; a < NA; ++a) w.w[a] = u32x4{0u, 0u, 0u, 0u};
-        }
+        wmask = (half_tail && k == steps - 1 && kb) ? 0u : kTopFieldMask;   // its loads were pulled onto the kb = 0 half's addresses
         __builtin_amdgcn_sched_barrier(0);
         load_b(st_mma, 1, b_b);
         mma_group(w, std::integral_constant<int, 0>{}, b_a);
