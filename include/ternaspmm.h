@@ -282,6 +282,25 @@ void ternaspmm_rope_decode_attention_prefetch(const terna_bf16* qkv, const float
                                               const void* const* pf_ptr, const long long* pf_bytes, const long long* pf_unit_bytes,
                                               int pf_count, terna_stream stream);
 
+/* The single-token attention split over the cache WITHOUT the merge (no counterpart in the reference): as
+ * ternaspmm_rope_decode_attention_prefetch, but the cache prefix of every head is spread over `splits` (1, 2, 4 or 8)
+ * workgroups that leave their partial results -- unnormalised sums, score maxima, sums of numerators, fp32 -- in
+ * `partial` (ternaspmm_attention_partial_bytes(B, H, D) bytes of device memory, no initialisation needed) and end;
+ * the consumer of the attention output merges them in the next launch: ternaspmm_attention_merge (out bf16 [B][H*D],
+ * the bits of the in-launch merge at the same split count) or bitlinear_TernaSpMM_packed_fused_attn, which merges
+ * inside the O projection's prologue.  The launch boundary takes the place of the arrival counter and of the merging
+ * workgroup's dependent reads, which cost the in-launch merge 5 - 6 us whatever the prefix length.
+ * ternaspmm_attention_partial_splits(B, H, S): the split count the library recommends (a power of two; 1 when the
+ * heads fill the chip anyway).  pf_ptr may be NULL with pf_count = 0. */
+long long ternaspmm_attention_partial_bytes(int B, int H, int D);
+int ternaspmm_attention_partial_splits(int B, int H, int S);
+void ternaspmm_rope_decode_attention_partial(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
+                                             int per_sequence, terna_bf16* cache_k, terna_bf16* cache_v, float* partial, int splits,
+                                             int B, int H, int KV, int D, int S, float scale, int adjacent,
+                                             const void* const* pf_ptr, const long long* pf_bytes, const long long* pf_unit_bytes,
+                                             int pf_count, terna_stream stream);
+void ternaspmm_attention_merge(const float* partial, int splits, terna_bf16* out, int B, int H, int D, terna_stream stream);
+
 /* The bookkeeping of one greedy decode step in one launch (generate.py:283-305: argmax, tokens[:, pos] = next_token,
  * the position counters): tok[b] = argmax(logits[b]) as above; if history != NULL and counters[1] < history_len,
  * history[b][counters[1]] = tok[b]; then counters[0] += 1 and counters[1] += 1 (counters int64 [2] = {cache slot of the

@@ -51,6 +51,10 @@ PROTOTYPES = {
     "ternaspmm_greedy_step_bf16": ([_vp, _vp, _vp, _ci, _vp, _vp, _ci, _ci, _vp], None),
     "ternaspmm_lm_head_bf16": ([_vp, _vp, _vp, _ci, _ci, _ci, _vp], None),
     "ternaspmm_argmax_bf16": ([_vp, _vp, _ci, _ci, _vp], None),
+    "ternaspmm_attention_partial_bytes": ([_ci] * 3, ctypes.c_longlong),
+    "ternaspmm_attention_partial_splits": ([_ci] * 3, ctypes.c_int),
+    "ternaspmm_rope_decode_attention_partial": ([_vp] * 4 + [_ci] + [_vp] * 3 + [_ci] * 6 + [ctypes.c_float, _ci, _vp, _vp, _vp, _ci, _vp], None),
+    "ternaspmm_attention_merge": ([_vp, _ci, _vp, _ci, _ci, _ci, _vp], None),
     "ternaspmm_rope_kv_store": ([_vp] * 4 + [_ci] + [_vp] * 3 + [_ci] * 7 + [_vp], None),
     "ternaspmm_rope_decode_attention": ([_vp] * 4 + [_ci] + [_vp] * 3 + [_ci] * 5 + [ctypes.c_float, _ci, _vp, _vp], None),
     "ternaspmm_decode_attention": ([_vp] * 4 + [_ci, _vp] + [_ci] * 5 + [ctypes.c_float, _vp, _vp], None),

@@ -103,6 +103,24 @@ void launch_attention_as(const uint16_t* q, uint16_t* ck, uint16_t* cv, const fl
         scratch.arrived, pf);
 }
 
+// The split with the merge left to the next launch (DEFER): one-dimensional grid of (sequence, head, split) workgroups,
+// padded to whole rounds of 8 (group, split) pairs when kv groups are kept on one XCD each, then the prefetching ones.
+template <int D, bool ADJ>
+void launch_attention_deferred(const uint16_t* qkv, uint16_t* ck, uint16_t* cv, const float* cos, const float* sin,
+                               const long long* pos, int per_seq, float* partial, int splits, int B, int H, int KV, int S,
+                               float scale, const AttentionPrefetch& pf_in, hipStream_t st)
+{
+    constexpr int NW = 4;                                     // a split is a short prefix: the narrow workgroup
+    AttentionPrefetch pf = pf_in;
+    auto kernel = terna_decode_attention_kernel<D, true, ADJ, NW, true, true>;
+    const size_t lds = decode_attention_lds_bytes(D, NW, S);
+    if (lds > 64 * 1024) allow_dynamic_lds(kernel, 160 * 1024, "hipFuncSetAttribute(decode attention, deferred merge)", __LINE__);
+    const bool grouped = attention_groups_on(H, KV);
+    const int slots = grouped ? 8 * (H / KV) * ((B * KV * splits + 7) / 8) : B * H * splits;
+    kernel<<<dim3(slots + pf.workgroups), dim3(64 * NW), lds, st>>>(
+        qkv, ck, cv, pos, H, KV, S, splits, slots, grouped ? B * KV : 0, per_seq, scale, cos, sin, nullptr, partial, nullptr, pf);
+}
+
 template <bool ROPE, bool ADJ>
 void launch_attention(const uint16_t* q, uint16_t* ck, uint16_t* cv, const float* cos, const float* sin,
                              const long long* pos, int per_seq, uint16_t* out, int B, int H, int KV, int D, int S, float scale,
@@ -131,6 +149,35 @@ bool attention_args_ok(const char* who, int B, int H, int KV, int D, int S)
         return false;
     }
     return true;
+}
+
+// The regions of a prefetching launch from the caller's host arrays; a region that breaks a rule is skipped.
+AttentionPrefetch prefetch_regions(const void* const* pf_ptr, const long long* pf_bytes, const long long* pf_unit_bytes, int pf_count)
+{
+    AttentionPrefetch pf{};
+    for (int r = 0; r < pf_count && pf.count < kAttentionPrefetchRegions; ++r) {
+        const bool broadcast = pf_unit_bytes[r] == 0;        // every XCD fetches the whole (small) region
+        if (pf_ptr[r] == nullptr || (reinterpret_cast<uintptr_t>(pf_ptr[r]) & 15) || pf_bytes[r] < 16 || pf_bytes[r] > (1ll << 30) ||
+            (!broadcast && (pf_unit_bytes[r] < 16 || (pf_unit_bytes[r] & 15) || pf_unit_bytes[r] > (1ll << 30))) ||
+            (broadcast && pf_bytes[r] > (1ll << 20)))
+            continue;
+        const int c = pf.count++;
+        pf.base[c] = static_cast<const u32x4*>(pf_ptr[r]);
+        pf.total_vecs[c] = pf_bytes[r] / 16;
+        pf.unit_vecs[c] = broadcast ? 0 : static_cast<int>(pf_unit_bytes[r] / 16);
+        pf.units[c] = broadcast ? 1 : (pf.total_vecs[c] + pf.unit_vecs[c] - 1) / pf.unit_vecs[c];
+    }
+    return pf;
+}
+
+// The attention takes `slots` workgroups; the rest of the chip prefetches (none when few CUs are left).
+int prefetch_workgroups(const AttentionPrefetch& pf, int slots)
+{
+    static const int forced_wgs = [] {
+        const char* v = tuning_env("TERNASPMM_ATTN_PREFETCH_WGS");
+        return v ? std::atoi(v) / 8 * 8 : -1;
+    }();
+    return pf.count > 0 && slots < 232 ? (forced_wgs >= 0 ? forced_wgs : (256 - slots) / 8 * 8) : 0;
 }
 
 }  // namespace
@@ -271,32 +318,76 @@ void ternaspmm_rope_decode_attention_prefetch(const terna_bf16* qkv, const float
                                               int pf_count, terna_stream stream)
 {
     if (!attention_args_ok("ternaspmm_rope_decode_attention_prefetch", B, H, KV, D, S)) return;
-    AttentionPrefetch pf{};
-    for (int r = 0; r < pf_count && pf.count < kAttentionPrefetchRegions; ++r) {
-        const bool broadcast = pf_unit_bytes[r] == 0;        // every XCD fetches the whole (small) region
-        if (pf_ptr[r] == nullptr || (reinterpret_cast<uintptr_t>(pf_ptr[r]) & 15) || pf_bytes[r] < 16 || pf_bytes[r] > (1ll << 30) ||
-            (!broadcast && (pf_unit_bytes[r] < 16 || (pf_unit_bytes[r] & 15) || pf_unit_bytes[r] > (1ll << 30))) ||
-            (broadcast && pf_bytes[r] > (1ll << 20)))
-            continue;
-        const int c = pf.count++;
-        pf.base[c] = static_cast<const u32x4*>(pf_ptr[r]);
-        pf.total_vecs[c] = pf_bytes[r] / 16;
-        pf.unit_vecs[c] = broadcast ? 0 : static_cast<int>(pf_unit_bytes[r] / 16);
-        pf.units[c] = broadcast ? 1 : (pf.total_vecs[c] + pf.unit_vecs[c] - 1) / pf.unit_vecs[c];
-    }
-    // the heads take B*H CUs; the rest of the chip prefetches
-    static const int forced_wgs = [] {
-        const char* v = tuning_env("TERNASPMM_ATTN_PREFETCH_WGS");
-        return v ? std::atoi(v) / 8 * 8 : -1;
-    }();
+    AttentionPrefetch pf = prefetch_regions(pf_ptr, pf_bytes, pf_unit_bytes, pf_count);
     const int slots = attention_slots(B, H, KV);
-    pf.workgroups = pf.count > 0 && slots < 232 ? (forced_wgs >= 0 ? forced_wgs : (256 - slots) / 8 * 8) : 0;
+    pf.workgroups = prefetch_workgroups(pf, slots);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const AttentionScratch scratch = attention_scratch_of(workspace, B, H);
     if (adjacent) launch_attention<true, true>(qkv, cache_k, cache_v, cos, sin, pos, per_sequence != 0, out, B, H, KV, D, S, scale, scratch, pf, st);
     else launch_attention<true, false>(qkv, cache_k, cache_v, cos, sin, pos, per_sequence != 0, out, B, H, KV, D, S, scale, scratch, pf, st);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_rope_decode_attention_prefetch", e, __LINE__);
+}
+
+long long ternaspmm_attention_partial_bytes(int B, int H, int D)
+{
+    if (B < 1 || H < 1 || D < 1) return -1;
+    return static_cast<long long>(sizeof(float)) *
+           (static_cast<long long>(attention_stat_floats(static_cast<size_t>(B) * H)) + static_cast<long long>(B) * H * kAttentionMaxSplits * D);
+}
+
+int ternaspmm_attention_partial_splits(int B, int H, int S)
+{
+    if (B < 1 || H < 1 || S < 1) return -1;
+    // as many splits as keep the (sequence, head, split) workgroups within half of the chip's CUs: the launch is bound
+    // by what ONE CU streams, and the consumer of the partial results reads splits x the bytes of a merged row
+    int sp = 1;
+    while (sp < kAttentionMaxSplits && static_cast<long>(B) * H * sp * 2 <= 128 && 16 * sp * 2 <= S) sp *= 2;
+    return sp;
+}
+
+void ternaspmm_rope_decode_attention_partial(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
+                                             int per_sequence, terna_bf16* cache_k, terna_bf16* cache_v, float* partial, int splits,
+                                             int B, int H, int KV, int D, int S, float scale, int adjacent,
+                                             const void* const* pf_ptr, const long long* pf_bytes, const long long* pf_unit_bytes,
+                                             int pf_count, terna_stream stream)
+{
+    if (!attention_args_ok("ternaspmm_rope_decode_attention_partial", B, H, KV, D, S)) return;
+    if (splits < 1 || splits > kAttentionMaxSplits || (splits & (splits - 1)) || partial == nullptr ||
+        static_cast<long>(B) * H * splits > 65536) {
+        std::fprintf(stderr, "ternaspmm_rope_decode_attention_partial: unsupported splits=%d (1, 2, 4 or 8) or no partial buffer\n", splits);
+        return;
+    }
+    AttentionPrefetch pf = prefetch_regions(pf_ptr, pf_bytes, pf_unit_bytes, pf_count);
+    const bool grouped = attention_groups_on(H, KV);
+    const int slots = grouped ? 8 * (H / KV) * ((B * KV * splits + 7) / 8) : B * H * splits;
+    pf.workgroups = prefetch_workgroups(pf, slots);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define TERNA_DEFER(DIM, ADJ) \
+    launch_attention_deferred<DIM, ADJ>(qkv, cache_k, cache_v, cos, sin, pos, per_sequence != 0, partial, splits, B, H, KV, S, scale, pf, st)
+    if (D == 128) {
+        if (adjacent) TERNA_DEFER(128, true);
+        else TERNA_DEFER(128, false);
+    } else {
+        if (adjacent) TERNA_DEFER(64, true);
+        else TERNA_DEFER(64, false);
+    }
+#undef TERNA_DEFER
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_rope_decode_attention_partial", e, __LINE__);
+}
+
+void ternaspmm_attention_merge(const float* partial, int splits, terna_bf16* out, int B, int H, int D, terna_stream stream)
+{
+    if (B < 1 || H < 1 || (D != 64 && D != 128) || splits < 1 || splits > kAttentionMaxSplits) {
+        std::fprintf(stderr, "ternaspmm_attention_merge: unsupported arguments (H=%d D=%d splits=%d)\n", H, D, splits);
+        return;
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (D == 128) terna_attention_merge_kernel<128><<<dim3(B * H), dim3(128), 0, st>>>(partial, out, B * H, splits);
+    else terna_attention_merge_kernel<64><<<dim3(B * H), dim3(64), 0, st>>>(partial, out, B * H, splits);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_attention_merge", e, __LINE__);
 }
 
 }  // extern "C"

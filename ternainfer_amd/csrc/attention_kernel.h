@@ -132,6 +132,42 @@ __global__ __launch_bounds__(256) void terna_rope_kv_store_kernel(
 // after every launch) merges the SP partials in split order -- the result does not depend on
 // which workgroup arrives last -- and writes the output row.
 constexpr int kAttentionMaxSplits = 8;
+//
+// DEFER = true: the split without the hand-off.  The grid is one-dimensional (so that the prefetching workgroups fit
+// behind it): workgroup -> (sequence, head, split), the splits of a kv group's heads spread over the XCDs like the
+// groups themselves.  Every workgroup leaves its partial result with plain stores and ends; whoever consumes the
+// attention output in the NEXT launch merges the splits (attention_merge below: the arithmetic of the in-launch
+// merge, so the same bits) -- the launch boundary is the synchronisation, which takes the 5 - 6 us of the
+// arrival counter and the merging workgroup's dependent reads out of the step.  Layout of `partial` then:
+//   floats [B*H][2][kAttentionMaxSplits]   score maximum / sum of numerators of every split (attention_stat_floats)
+//   floats [B*H][SP][D]                    unnormalised results
+constexpr int kAttentionStatFloats = 2 * kAttentionMaxSplits;          // per head
+__device__ __host__ inline size_t attention_stat_floats(size_t heads) { return heads * kAttentionStatFloats; }
+
+// Output dimension d of head bh from its SP partial results, in split order.
+__device__ __forceinline__ float attention_merge(const float* __restrict__ stat, const float* __restrict__ o_head, int SP, int D, int d)
+{
+    float m_all = -INFINITY;
+    for (int j = 0; j < SP; ++j) m_all = fmaxf(m_all, stat[j]);
+    float num = 0.0f, den = 0.0f;
+    for (int j = 0; j < SP; ++j) {
+        const float w = __expf(stat[j] - m_all);                       // an empty split: exp(-inf) = 0
+        num = fmaf(w, o_head[j * D + d], num);
+        den = fmaf(w, stat[kAttentionMaxSplits + j], den);
+    }
+    return num / den;
+}
+
+// out bf16 [B*H][D] from the partial results of a DEFER launch: one workgroup of D threads per head.
+template <int D>
+__global__ __launch_bounds__(D) void terna_attention_merge_kernel(const float* __restrict__ partial, uint16_t* __restrict__ out,
+                                                                  int heads, int SP)
+{
+    const int bh = blockIdx.x;
+    const float* stat = partial + static_cast<size_t>(bh) * kAttentionStatFloats;
+    const float* o_head = partial + attention_stat_floats(heads) + static_cast<size_t>(bh) * SP * D;
+    out[static_cast<size_t>(bh) * D + threadIdx.x] = float_to_bf16_bits(attention_merge(stat, o_head, SP, D, threadIdx.x));
+}
 // Extra workgroups of the attention launch (blockIdx.x >= heads) that pull up to kAttentionPrefetchRegions regions of
 // device memory through the caches while the heads' workgroups -- one CU each -- do the attention:
 // the weights of the launches that follow.  Unit u of a region goes to a workgroup on XCD (u mod 8),
@@ -217,7 +253,7 @@ constexpr size_t decode_attention_lds_bytes(int D, int NW, int S)
     return (static_cast<size_t>(S) + (64 * NW / (D / 8)) * D + 64 * NW) * sizeof(float);
 }
 
-template <int D, bool ROPE, bool ADJACENT = false, int NW = 4, bool SPLIT = false>
+template <int D, bool ROPE, bool ADJACENT = false, int NW = 4, bool SPLIT = false, bool DEFER = false>
 __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     // what the first loads depend on comes first: the leading sixteen dwords of the arguments arrive in scalar registers
     const uint16_t* __restrict__ q, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
@@ -241,27 +277,40 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
         return;
     }
 
-    // SP = splits of the cache (= gridDim.y), sp = this workgroup's split; constants in the unsplit kernel
-    const int SP = SPLIT ? splits : 1, sp = SPLIT ? blockIdx.y : 0;
-    // local slot l of this split (16 * local tile + row) -> cache slot
-    auto cache_slot = [&](int l) { return (((l >> 4) * SP + sp) << 4) + (l & 15); };
+    static_assert(!DEFER || SPLIT, "the deferred merge is a variant of the split kernel");
+    // SP = splits of the cache (= gridDim.y, or folded into blockIdx.x when DEFER), sp = this workgroup's split;
+    // constants in the unsplit kernel
+    const int SP = SPLIT ? splits : 1;
+    int sp = SPLIT && !DEFER ? blockIdx.y : 0;
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     // Workgroup -> (sequence, head).  Workgroups go to the 8 XCDs round robin, and the H / KV heads of a kv group read
     // the same keys and values: with groups > 0 (= B * KV) the heads of group G all sit on XCD G mod 8, so that the
     // group's cache prefix crosses the fabric once and its other heads hit in that L2 (the grid is padded to whole
     // rounds of 8 groups; workgroups without a group leave).  groups = 0: heads in launch order.
+    // DEFER: the same with (group, split) pairs in place of groups -- the heads of a group read the same tiles of a split.
     int b, h;
     if (groups > 0) {
         const int per = H / KV, q = blockIdx.x >> 3;
-        const int G = 8 * (q / per) + (blockIdx.x & 7);
-        if (G >= groups) return;
+        int G = 8 * (q / per) + (blockIdx.x & 7);
+        if (G >= (DEFER ? groups * SP : groups)) return;
+        if constexpr (DEFER) {
+            sp = G % SP;
+            G /= SP;
+        }
         b = G / KV;
         h = (G - b * KV) * per + q % per;
     } else {
-        b = blockIdx.x / H;
-        h = blockIdx.x - b * H;
+        int u = blockIdx.x;
+        if constexpr (DEFER) {
+            sp = u % SP;
+            u /= SP;
+        }
+        b = u / H;
+        h = u - b * H;
     }
+    // local slot l of this split (16 * local tile + row) -> cache slot
+    auto cache_slot = [&](int l) { return (((l >> 4) * SP + sp) << 4) + (l & 15); };
     const int bh = b * H + h;
     const int kvh = h / (H / KV);
     // Prefix length: slots 0 .. pos[0].  pos comes from device memory the host cannot check, so it is clamped to the
@@ -494,7 +543,7 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
         for (int grp = 0; grp < GROUPS; ++grp) o += part2[grp * D + tid];
     }
     uint16_t* orow = out + (static_cast<size_t>(b) * H + h) * D;
-    if (!SPLIT || SP == 1) {
+    if ((!SPLIT || SP == 1) && !DEFER) {        // (DEFER has no output row: `out` is NULL there, also with one split)
         if (tid < D) orow[tid] = float_to_bf16_bits(o / sum);
         return;
     }
@@ -507,6 +556,17 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     // workgroup barrier alone orders instructions, not their completion, and the counter lives in
     // another memory channel than the partials), then the barrier, then ONE thread counts the arrival;
     // the merging workgroup issues its loads only after it has seen the full count.
+    if constexpr (DEFER) {
+        const int heads_total = groups > 0 ? groups * (H / KV) : heads / SP;           // B * H
+        float* stat = partial + static_cast<size_t>(bh) * kAttentionStatFloats;
+        float* o_out = partial + attention_stat_floats(static_cast<size_t>(heads_total)) + (static_cast<size_t>(bh) * SP + sp) * D;
+        if (tid < D) o_out[tid] = o;
+        if (tid == 0) {
+            stat[sp] = mx;
+            stat[kAttentionMaxSplits + sp] = sum;
+        }
+        return;
+    }
     float* mine = partial + (static_cast<size_t>(bh) * SP + sp) * (D + 2);
     auto publish = [](float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
     auto fetch = [](const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };

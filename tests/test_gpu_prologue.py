@@ -647,3 +647,84 @@ def test_rope_decode_attention_per_sequence(lib, b, h, kv, d, s_max, lens, adjac
                                             s_max, scale, adjacent, None, None)
         torch.cuda.synchronize()
         assert torch.equal(o3[0], o2[i]) and torch.equal(ck3[0], ck2[i]) and torch.equal(cv3[0], cv2[i])
+
+
+# ------------------------------------------------------------------ split attention with the merge left to the next launch
+def _partial_buffer(lib, b, h, d):
+    nbytes = lib.ternaspmm_attention_partial_bytes(b, h, d)
+    assert nbytes > 0
+    return torch.full((nbytes // 4,), float("nan"), dtype=torch.float32, device="cuda")       # needs no initialisation
+
+
+@pytest.mark.parametrize("per_seq", [0, 1])
+@pytest.mark.parametrize("splits", [1, 2, 4, 8])
+@pytest.mark.parametrize("b,h,kv,d,s_max,n", [(1, 20, 5, 128, 384, 200), (1, 20, 5, 128, 4096, 4000), (2, 4, 2, 64, 300, 17),
+                                              (3, 8, 8, 128, 64, 1), (1, 20, 5, 128, 2048, 1029)])
+def test_rope_decode_attention_partial_and_merge(lib, b, h, kv, d, s_max, n, splits, per_seq):
+    """The split attention that leaves the merge to the next launch + the merge kernel: caches bit-identical to
+    ternaspmm_rope_decode_attention, output within the attention tolerance of the oracle (splits change the order
+    of the sums); a prefix shorter than the splits leaves empty splits, which the merge must weigh with zero; and
+    with a prefetch region the launch gives the same bits."""
+    lens = [max(1, n - 7 * i) for i in range(b)] if per_seq else [n] * b
+    qkv = make_bf16_activations(b, (h + 2 * kv) * d, 1801 + n)
+    k0 = make_bf16_activations(b * kv * s_max, d, 1802 + n).reshape(b, kv, s_max, d)
+    v0 = make_bf16_activations(b * kv * s_max, d, 1803 + n, outlier_frac=0.01).reshape(b, kv, s_max, d)
+    pos = (np.array(lens, np.int64) - 1) if per_seq else np.array([n - 1], np.int64)
+    cos, sin = _angles(pos, d)
+    xd, cd, sd, pd = _dev(qkv), _dev(cos), _dev(sin), _dev(pos)
+    scale = float(d) ** -0.5
+    ck1, cv1, ck2, cv2, ck3, cv3 = _dev(k0), _dev(v0), _dev(k0), _dev(v0), _dev(k0), _dev(v0)
+    o1 = torch.zeros((b, h * d), dtype=torch.int16, device="cuda")
+    o2, o3 = torch.zeros_like(o1), torch.zeros_like(o1)
+    lib.ternaspmm_rope_decode_attention(_vp(xd), _vp(cd), _vp(sd), _vp(pd), per_seq, _vp(ck1), _vp(cv1), _vp(o1), b, h, kv, d, s_max,
+                                        scale, 1, None, None)
+    part = _partial_buffer(lib, b, h, d)
+    print(f"[case] attention partial + merge b={b} h={h} d={d} S={s_max} n={n} splits={splits} per_seq={per_seq}", flush=True)
+    lib.ternaspmm_rope_decode_attention_partial(_vp(xd), _vp(cd), _vp(sd), _vp(pd), per_seq, _vp(ck2), _vp(cv2), _vp(part), splits,
+                                                b, h, kv, d, s_max, scale, 1, None, None, None, 0, None)
+    lib.ternaspmm_attention_merge(_vp(part), splits, _vp(o2), b, h, d, None)
+    torch.cuda.synchronize()
+    assert torch.equal(ck1, ck2) and torch.equal(cv1, cv2)
+    got = O.bf16_bits_to_f32(o2.cpu().numpy().view(np.uint16)).reshape(b, h, d).astype(np.float64)
+    unsplit = O.bf16_bits_to_f32(o1.cpu().numpy().view(np.uint16)).reshape(b, h, d).astype(np.float64)
+    tol = 2.0 ** -7 * np.abs(unsplit).max(axis=-1, keepdims=True) + 1e-6
+    assert np.isfinite(got).all()
+    assert (np.abs(got - unsplit) <= 2 * tol).all(), float((np.abs(got - unsplit) / tol).max())
+    # the same launch with prefetching workgroups
+    region = torch.zeros(40 * 2560, dtype=torch.int32, device="cuda")
+    ptrs = (ctypes.c_void_p * 1)(region.data_ptr())
+    sizes = (ctypes.c_longlong * 1)(region.numel() * 4)
+    units = (ctypes.c_longlong * 1)(10240)
+    part3 = _partial_buffer(lib, b, h, d)
+    lib.ternaspmm_rope_decode_attention_partial(_vp(xd), _vp(cd), _vp(sd), _vp(pd), per_seq, _vp(ck3), _vp(cv3), _vp(part3), splits,
+                                                b, h, kv, d, s_max, scale, 1, ptrs, sizes, units, 1, None)
+    lib.ternaspmm_attention_merge(_vp(part3), splits, _vp(o3), b, h, d, None)
+    torch.cuda.synchronize()
+    assert torch.equal(o2, o3) and torch.equal(ck2, ck3) and torch.equal(cv2, cv3)
+
+
+def test_attention_partial_against_the_oracle(lib):
+    """Every sequence against attention_one_token at its own length, 8 splits over a 2B-shaped cache."""
+    b, h, kv, d, s_max, lens = 2, 20, 5, 128, 1024, (1000, 333)
+    qkv = make_bf16_activations(b, (h + 2 * kv) * d, 1811)
+    k0 = make_bf16_activations(b * kv * s_max, d, 1812).reshape(b, kv, s_max, d)
+    v0 = make_bf16_activations(b * kv * s_max, d, 1813, outlier_frac=0.01).reshape(b, kv, s_max, d)
+    pos = np.array(lens, np.int64) - 1
+    cos, sin = _angles(pos, d)
+    xd, cd, sd, pd, ck, cv = _dev(qkv), _dev(cos), _dev(sin), _dev(pos), _dev(k0), _dev(v0)
+    part = _partial_buffer(lib, b, h, d)
+    out = torch.zeros((b, h * d), dtype=torch.int16, device="cuda")
+    lib.ternaspmm_rope_decode_attention_partial(_vp(xd), _vp(cd), _vp(sd), _vp(pd), 1, _vp(ck), _vp(cv), _vp(part), 8,
+                                                b, h, kv, d, s_max, float(d) ** -0.5, 1, None, None, None, 0, None)
+    lib.ternaspmm_attention_merge(_vp(part), 8, _vp(out), b, h, d, None)
+    torch.cuda.synchronize()
+    got = O.bf16_bits_to_f32(out.cpu().numpy().view(np.uint16)).reshape(b, h, d).astype(np.float64)
+    kc, vc = ck.cpu().numpy().view(np.uint16), cv.cpu().numpy().view(np.uint16)
+    x = qkv.reshape(b, h + 2 * kv, d)
+    for i in range(b):
+        q = O.rope_adjacent(x[i:i + 1, :h], cos[i][None, None], sin[i][None, None])
+        want = O.attention_one_token(q, kc[i:i + 1], vc[i:i + 1], lens[i], float(d) ** -0.5)[0]
+        tol = 2.0 ** -7 * np.abs(want).max(axis=-1, keepdims=True) + 1e-6
+        assert (np.abs(got[i] - want) <= tol).all(), (i, float((np.abs(got[i] - want) / tol).max()))
+    assert lib.ternaspmm_attention_partial_splits(1, 20, 384) in (1, 2, 4, 8)
+    assert lib.ternaspmm_attention_partial_splits(8, 20, 384) == 1
