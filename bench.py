@@ -250,8 +250,10 @@ def run_model(args, torch):
                                "decode step; norms, gate, activation quantisation, RoPE, cache write, single-token "
                                "attention, the multi-token attention of the prompt pass, the bf16 LM head and greedy "
                                "sampling are library kernels; the prompt pass is one HIP graph too"
-                               + ("" if args.no_prefetch else "; the idle CUs of the attention launch "
-                                                            "prefetch the weights of the launches that follow"),
+                               + ("; one sequence: the attention is split over several workgroups per head and the O "
+                                  "projection's prologue merges the partial results" if args.batch == 1 else
+                                  ("" if args.no_prefetch else "; the idle CUs of the attention launch "
+                                                               "prefetch the weights of the launches that follow")),
                    "batch": args.batch, "act": act},
         **{k: fig[k] for k in ("prefill_tokens_per_s", "prefill_ms", "decode_s", "model_build_s", "first_tokens",
                                "graph_equals_eager_first_tokens")}}

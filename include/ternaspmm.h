@@ -198,6 +198,14 @@ int bitlinear_TernaSpMM_packed_fused(const terna_bf16* x, const terna_bf16* resi
 /* Gated-FFN variant: h = bf16(bf16(relu(x1)^2) * x3) from x13 (bf16 [M][2F], as ternaspmm_relu2_mul_rmsnorm_quant),
  * norm and quantisation over F columns, then the [N][F] ternary linear.  Supported: M = 1, N <= 4096, F <= 7168;
  * returns 0 otherwise (caller: ternaspmm_relu2_mul_rmsnorm_quant + bitlinear_TernaSpMM_packed). */
+/* The O projection of a single-row decode step with the attention's deferred merge inside: as
+ * bitlinear_TernaSpMM_packed_fused without a residual, but the activation row is formed from the partial results a
+ * ternaspmm_rope_decode_attention_partial launch left (`partial`, `splits`; K = heads * head_dim) -- bit-identical to
+ * ternaspmm_attention_merge followed by bitlinear_TernaSpMM_packed_fused.  M must be 1 (one sequence); returns 0
+ * without doing anything for shapes outside what it supports (the caller then runs that pair). */
+int bitlinear_TernaSpMM_packed_fused_attn(const float* partial, int splits, int head_dim, const terna_bf16* norm_weight, float eps,
+                                          const void* packed, terna_bf16* out, const terna_bf16* ws, int ws_num,
+                                          int8_t* xq_out, terna_bf16* s_out, int M, int N, int K, terna_stream stream);
 int bitlinear_TernaSpMM_packed_fused_glu(const terna_bf16* x13, const terna_bf16* norm_weight, float eps,
                                          const void* packed, terna_bf16* out, const terna_bf16* ws, int ws_num,
                                          int8_t* xq_out, terna_bf16* s_out, int M, int N, int F, terna_stream stream);

@@ -44,6 +44,8 @@ PROTOTYPES = {
     "ternaspmm_relu2_mul_rmsnorm_quant": ([_vp, _vp, ctypes.c_float, _vp, _vp, _vp, _ci, _ci, _vp], None),
     "bitlinear_TernaSpMM_packed_fused": ([_vp, _vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _ci, _vp, _vp, _ci, _ci, _ci, _vp],
                                          ctypes.c_int),
+    "bitlinear_TernaSpMM_packed_fused_attn": ([_vp, _ci, _ci, _vp, ctypes.c_float, _vp, _vp, _vp, _ci, _vp, _vp, _ci, _ci, _ci, _vp],
+                                              ctypes.c_int),
     "bitlinear_TernaSpMM_packed_fused_glu": ([_vp, _vp, ctypes.c_float, _vp, _vp, _vp, _ci, _vp, _vp, _ci, _ci, _ci, _vp],
                                              ctypes.c_int),
     "ternaspmm_rope_decode_attention_prefetch": ([_vp] * 4 + [_ci] + [_vp] * 3 + [_ci] * 5 + [ctypes.c_float, _ci, _vp, _vp, _vp, _vp, _ci, _vp], None),

@@ -339,10 +339,13 @@ long long ternaspmm_attention_partial_bytes(int B, int H, int D)
 int ternaspmm_attention_partial_splits(int B, int H, int S)
 {
     if (B < 1 || H < 1 || S < 1) return -1;
-    // as many splits as keep the (sequence, head, split) workgroups within half of the chip's CUs: the launch is bound
-    // by what ONE CU streams, and the consumer of the partial results reads splits x the bytes of a merged row
+    // The launch is bound by what ONE CU streams, so a split should not get more than about 512 slots -- but the consumer
+    // of the partial results reads splits x the bytes of a merged row (measured on the 2B shapes, one sequence: four splits
+    // cost the O projection 0.9 us, eight 1.7 us): four splits up to 1024 slots, eight beyond, fewer when the
+    // (sequence, head, split) workgroups would not fit the chip or a split would get less than two tiles.
+    const int want = S > 1024 ? kAttentionMaxSplits : 4;
     int sp = 1;
-    while (sp < kAttentionMaxSplits && static_cast<long>(B) * H * sp * 2 <= 128 && 16 * sp * 2 <= S) sp *= 2;
+    while (sp < want && static_cast<long>(B) * H * sp * 2 <= 256 && 32 * sp * 2 <= S) sp *= 2;
     return sp;
 }
 

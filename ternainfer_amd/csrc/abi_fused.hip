@@ -117,6 +117,38 @@ int bitlinear_TernaSpMM_packed_fused(const terna_bf16* x, const terna_bf16* resi
                                ws, ws_num, xq_out, s_out, M, N, K, static_cast<hipStream_t>(stream));
 }
 
+int bitlinear_TernaSpMM_packed_fused_attn(const float* partial, int splits, int head_dim, const terna_bf16* norm_weight, float eps,
+                                          const void* packed, terna_bf16* out, const terna_bf16* ws, int ws_num,
+                                          int8_t* xq_out, terna_bf16* s_out, int M, int N, int K, terna_stream stream)
+{
+    if (!shape_ok(M, N, K) || !groups_ok(ws_num)) return 0;
+    const int ktiles = K / 64;
+    if (M != 1 || (head_dim != 64 && head_dim != 128) || K % head_dim != 0 || (splits != 1 && splits != 2 && splits != 4 && splits != 8) ||
+        partial == nullptr || N / 16 > 65535 || ktiles > 8 * 5)
+        return 0;
+    const dim3 grid(N / 16);
+    const uint16_t* x = reinterpret_cast<const uint16_t*>(partial);
+    const uint32_t* p = static_cast<const uint32_t*>(packed);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define TERNA_FUSED_ATTN(SP, HD)                                                                                   \
+    terna_decode_fused_kernel<8, 5, FUSED_ATTN, 1, 1, SP, HD><<<grid, dim3(8 * 64), 0, st>>>(                      \
+        x, nullptr, norm_weight, p, M, N, K, eps, nullptr, out, ws, ws_num, xq_out, s_out)
+#define TERNA_FUSED_ATTN_HD(HD)                                                                                    \
+    do {                                                                                                           \
+        if (splits == 1) TERNA_FUSED_ATTN(1, HD);                                                                  \
+        else if (splits == 2) TERNA_FUSED_ATTN(2, HD);                                                             \
+        else if (splits == 4) TERNA_FUSED_ATTN(4, HD);                                                             \
+        else TERNA_FUSED_ATTN(8, HD);                                                                              \
+    } while (0)
+    if (head_dim == 128) TERNA_FUSED_ATTN_HD(128);
+    else TERNA_FUSED_ATTN_HD(64);
+#undef TERNA_FUSED_ATTN_HD
+#undef TERNA_FUSED_ATTN
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("bitlinear_TernaSpMM_packed_fused_attn", e, __LINE__);
+    return 1;
+}
+
 int bitlinear_TernaSpMM_packed_fused_glu(const terna_bf16* x13, const terna_bf16* norm_weight, float eps,
                                          const void* packed, terna_bf16* out, const terna_bf16* ws, int ws_num,
                                          int8_t* xq_out, terna_bf16* s_out, int M, int N, int F, terna_stream stream)

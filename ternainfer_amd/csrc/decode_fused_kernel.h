@@ -9,7 +9,10 @@
 // the same values in the same order, so all bands see identical int8 activations.
 //
 //   h  = x, or bf16(x + residual)            (workgroup 0 also writes h to sum_out: the new stream),
-//        or bf16(bf16(relu(x1)^2) * x3)      (gated FFN: x = [x1 | x3], 2K columns per row)
+//        or bf16(bf16(relu(x1)^2) * x3)      (gated FFN: x = [x1 | x3], 2K columns per row),
+//        or the single-token attention's output row merged from the partial results of its splits
+//        (FUSED_ATTN, one row: `x` is then the fp32 buffer a deferred-merge attention launch left, see
+//        attention_kernel.h; the merge arithmetic is attention_merge's, so the row has the bits the merge kernel gives)
 //   y  = bf16(h * rsqrt(mean(h^2) + eps) * norm_w)
 //   s  = bf16(127 / max(max|y|, 1e-5)),  q = clamp(rint(y * s), -128, 127)
 //   out[m][n] = bf16((sum_k q[m][k] W[n][k] / s[m]) * ws[group(n)])      (decode epilogue)
@@ -31,6 +34,7 @@
 
 #include "decode_packed_kernel.h"
 #include "norm_quant_kernel.h"
+#include "attention_kernel.h"
 
 namespace terna {
 
@@ -64,9 +68,11 @@ template <> struct RowPiece<1> {
 // MP = rows a wave's 64 lanes cover at once (M <= MP): 64/MP lanes walk along a row, MP columns
 // each, so a lane handles MP elements per tile -- the prologue arithmetic, which every workgroup
 // repeats, costs in proportion to the batch rows that exist, not to the 16 the MFMA tile has.
-enum FusedMode { FUSED_PLAIN, FUSED_RESIDUAL, FUSED_GLU };
+enum FusedMode { FUSED_PLAIN, FUSED_RESIDUAL, FUSED_GLU, FUSED_ATTN };
 
-template <int WAVES, int TMAX, int MODE, int MP, int NB = 1>
+// ASP / AHD (FUSED_ATTN only): splits and head size of the attention whose partial results the row is merged from --
+// compile-time, so that a head's statistics are two scalar loads and no address needs a division.
+template <int WAVES, int TMAX, int MODE, int MP, int NB = 1, int ASP = 1, int AHD = 64>
 __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
     // what the first loads depend on comes first: the leading sixteen dwords of the arguments arrive in scalar registers
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, const uint16_t* __restrict__ norm_w,
@@ -74,6 +80,8 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ ws, int ws_num, int8_t* __restrict__ xq_out,
     uint16_t* __restrict__ s_out)
 {
+    static_assert(MODE != FUSED_ATTN || MP == 1, "the attention merge feeds a single row");
+    static_assert(AHD % 64 == 0 && ASP >= 1 && ASP <= kAttentionMaxSplits, "a 64-column tile lies inside one head");
     using XQ = XSlab<int8_t>;
     using Piece = RowPiece<MP>;
     constexpr int LPR = 64 / MP;                     // lanes per row
@@ -92,7 +100,7 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
     const int row = lane / LPR, cl = (lane % LPR) * MP;   // load coordinates: batch row, first of MP columns
     const bool row_ok = row < M;
     const bool writer = blockIdx.x == 0;             // the workgroup that publishes h, q and s
-    constexpr bool RES = MODE != FUSED_PLAIN;        // a second operand: the residual, or x3 of the gate
+    constexpr bool RES = MODE == FUSED_RESIDUAL || MODE == FUSED_GLU;   // a second operand: the residual, or x3 of the gate
     const size_t pitch = MODE == FUSED_GLU ? 2 * static_cast<size_t>(K) : K;
     const uint16_t* second = MODE == FUSED_GLU ? x + K : residual;
 
@@ -102,6 +110,9 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
     // i.e. one memory round trip per tile.
     uint32_t wword[NB][TMAX];
     Piece xr[TMAX], rr[TMAX], nw[TMAX];
+    constexpr int AT = MODE == FUSED_ATTN ? TMAX : 1;
+    f32x4 ast[AT][4];                                // FUSED_ATTN: score maxima and sums of numerators of the tile's head
+    float ao[AT][ASP];                               //             unnormalised result of every split, this lane's dimension
     bool use[TMAX];
 #pragma unroll
     for (int t = 0; t < TMAX; ++t) {
@@ -112,9 +123,46 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
 #pragma unroll
         for (int b = 0; b < NB; ++b) wword[b][t] = packed[(static_cast<size_t>(band0 + b) * ktiles + jc) * 64 + lane];   // word L; operand order below
         const size_t off = static_cast<size_t>(row_ok ? row : 0) * pitch + jc * 64 + cl;
-        xr[t].load(x + off);
+        if constexpr (MODE == FUSED_ATTN) {
+            // column jc * 64 + lane of the one row = dimension d of head `head` (a tile lies inside one head);
+            // the head's statistics are the same for the whole wave, its unnormalised results one float per lane and split
+            const float* part = reinterpret_cast<const float*>(x);
+            const int head = (jc * 64) / AHD;                           // wave-uniform
+            const int d = jc * 64 - head * AHD + lane;
+            const f32x4* stat = reinterpret_cast<const f32x4*>(part + static_cast<size_t>(head) * kAttentionStatFloats);
+            const float* o_head = part + attention_stat_floats(static_cast<size_t>(K / AHD)) + static_cast<size_t>(head) * (ASP * AHD);
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) ast[t][q4] = stat[q4];      // maxima 0 .. 7, sums 0 .. 7
+#pragma unroll
+            for (int jj = 0; jj < ASP; ++jj) ao[t][jj] = o_head[jj * AHD + d];
+        } else {
+            xr[t].load(x + off);
+        }
         if constexpr (RES) rr[t].load(second + off);
         nw[t].load(norm_w + jc * 64 + cl);
+    }
+    if constexpr (MODE == FUSED_ATTN) {
+#pragma unroll
+        for (int t = 0; t < TMAX; ++t) {             // attention_merge, on the values requested above
+            float am[kAttentionMaxSplits], al[kAttentionMaxSplits];
+#pragma unroll
+            for (int jj = 0; jj < kAttentionMaxSplits; ++jj) {
+                am[jj] = ast[t][jj >> 2][jj & 3];
+                al[jj] = ast[t][2 + (jj >> 2)][jj & 3];
+            }
+            float m_all = -INFINITY;
+#pragma unroll
+            for (int jj = 0; jj < ASP; ++jj) m_all = fmaxf(m_all, am[jj]);
+            float num = 0.0f, den = 0.0f;
+#pragma unroll
+            for (int jj = 0; jj < ASP; ++jj) {
+                const float w = __expf(am[jj] - m_all);
+                num = fmaf(w, ao[t][jj], num);
+                den = fmaf(w, al[jj], den);
+            }
+            const float merged[1] = {num / den};
+            xr[t].pack(merged);
+        }
     }
 #pragma unroll
     for (int t = 0; t < TMAX; ++t) {

@@ -22,7 +22,7 @@ import torch
 from torch.nn import functional as F
 
 from . import _lib
-from .linear import (argmax_rows, get_global_workspace, greedy_step, greedy_step_state, lm_head, quant_input, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant,
+from .linear import (argmax_rows, attention_merge_rmsnorm_linear_packed, get_global_workspace, greedy_step, greedy_step_state, lm_head, quant_input, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant,
                      repack_weight, rmsnorm_linear_packed, rmsnorm_quant)
 
 
@@ -199,7 +199,20 @@ class Block:
         qkv, x = self._norm_linear(self.wqkv, x, self.attention_norm, residual=pending)
         rep = a.n_heads // a.n_kv_heads
         one_token = mask is None           # the caller's rule: fused, one new token, a head size the kernel has
-        if one_token:                       # RoPE, cache write and attention over the cache prefix: one launch
+        deferred = one_token and isinstance(attn_ws, tuple)
+        if deferred:
+            # one sequence: the cache prefix of every head split over several workgroups that leave partial results;
+            # the O projection's prologue merges them (the launch boundary is the synchronisation)
+            lib = self.wqkv.lib
+            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            # (no prefetch regions here: this launch is shorter than the prefetch of the following weights would be --
+            # measured with them 1005 - 1125 us per step against 960 without and 971 for the unsplit launch that prefetches)
+            partial, splits = attn_ws
+            lib.ternaspmm_rope_decode_attention_partial(
+                _p(qkv), _p(cos), _p(sin), _p(pos_idx), per_seq, _p(cache_k), _p(cache_v), _p(partial), splits, bsz, a.n_heads,
+                a.n_kv_heads, a.head_dim, cache_k.shape[2], a.head_dim ** -0.5, int(a.rope_adjacent), None, None, None, 0,
+                stream)
+        elif one_token:                     # RoPE, cache write and attention over the cache prefix: one launch
             lib = self.wqkv.lib
             stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
             o = torch.empty((bsz, a.n_heads * a.head_dim), dtype=torch.bfloat16, device=x.device)
@@ -247,7 +260,11 @@ class Block:
             vv = cache_v.repeat_interleave(rep, dim=1)
             o = F.scaled_dot_product_attention(q, kk, vv, attn_mask=mask)
             o = o.transpose(1, 2).reshape(bsz * t, a.n_heads * a.head_dim)
-        attn, _ = self._norm_linear(self.wo, o.contiguous(), self.attn_sub_norm)
+        if deferred:
+            attn = attention_merge_rmsnorm_linear_packed(partial, splits, a.n_heads, a.head_dim, self.attn_sub_norm, a.norm_eps,
+                                                         self.wo.packed, self.wo.ws, self.wo.ws_num, self.wo.n)
+        else:
+            attn, _ = self._norm_linear(self.wo, o.contiguous(), self.attn_sub_norm)
         x13, x = self._norm_linear(self.w13, x, self.ffn_norm, residual=attn)
         ffn, _ = self._norm_linear(self.w2, x13, self.ffn_sub_norm, glu=True)
         return x, ffn
@@ -338,6 +355,22 @@ class Transformer:
             self._rope_tables = tables = (key, torch.stack([ang.cos(), ang.sin()], dim=1).contiguous())
         return tables[1]
 
+    def attention_partial(self, max_seq: int):
+        """(buffer, splits) for the single-sequence decode step whose attention leaves the merge of its splits to the O
+        projection, or None when that form does not apply (one split recommended; `deferred_attention_merge` False)."""
+        if not getattr(self, "deferred_attention_merge", True):
+            return None
+        a = self.args
+        lib = _lib.load()
+        splits = getattr(self, "attention_splits", None) or lib.ternaspmm_attention_partial_splits(1, a.n_heads, max_seq)
+        if splits <= 1:
+            return None
+        buf = getattr(self, "_attn_partial", None)
+        if buf is None:
+            nbytes = lib.ternaspmm_attention_partial_bytes(1, a.n_heads, a.head_dim)
+            self._attn_partial = buf = torch.empty(nbytes // 4, dtype=torch.float32, device="cuda")
+        return buf, splits
+
     def attention_workspace(self, bsz: int):
         """Zero-filled scratch of the single-token attention (split over the cache); one per batch size."""
         ws = getattr(self, "_attn_ws", None)
@@ -378,6 +411,8 @@ class Transformer:
         x = self.tok_embeddings[tokens.reshape(-1)]
         pending = None
         attn_ws = self.attention_workspace(bsz) if one_launch_attention else None     # layers run one after another: shared
+        if one_launch_attention and bsz == 1 and self.layers[0].act == "int8":
+            attn_ws = self.attention_partial(max_seq) or attn_ws
         for index, (layer, (ck, cv)) in enumerate(zip(self.layers, cache)):
             x_in, pending_in = x, pending
             x, pending = layer.forward(x, pending, ck, cv, pos_idx, cos, sin, mask, attn_ws)

@@ -134,6 +134,36 @@ def test_toy_model_prompts_of_different_lengths_in_one_batch(head_dim, prefetch)
     assert torch.nn.functional.cosine_similarity(outs[0].flatten(), outs[1].flatten(), dim=0).item() > 0.999
 
 
+@pytest.mark.parametrize("head_dim,splits", [(64, 2), (128, 4), (128, 8)])
+def test_toy_model_attention_merge_deferred_to_the_o_projection(head_dim, splits):
+    """One sequence: the decode step whose attention leaves the merge of its splits to the O projection's prologue
+    against the step with the attention in one piece -- logits within the tolerance of the two summation orders,
+    the greedy tokens of a replayed graph equal to eager execution."""
+    from ternainfer_amd.model import ModelArgs, Transformer, greedy_decode
+    args = ModelArgs(dim=4 * head_dim, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=1024, ffn_dim=384)
+    model = Transformer(args, seed=41, act="int8")
+    prompt = torch.randint(0, args.vocab_size, (1, 150), generator=torch.Generator().manual_seed(42)).cuda()
+    print(f"[case] toy model, deferred attention merge head_dim={head_dim} splits={splits}", flush=True)
+    outs = []
+    with torch.inference_mode():
+        for deferred in (True, False):
+            model.deferred_attention_merge = deferred
+            model.attention_splits = splits
+            cache = model.make_cache(1, 200)
+            model.forward(prompt, cache, torch.arange(150, device="cuda"))
+            outs.append(model.forward(prompt[:, -1:].contiguous(), cache, torch.tensor([150], device="cuda")).float())
+    err = (outs[0] - outs[1]).abs().max().item()
+    assert err <= 3e-2 * outs[1].abs().max().item(), err
+    assert torch.nn.functional.cosine_similarity(outs[0].flatten(), outs[1].flatten(), dim=0).item() > 0.9995
+    model.deferred_attention_merge = True
+    a, _, _ = greedy_decode(model, prompt, 10, use_graph=True)
+    b, _, _ = greedy_decode(model, prompt, 10, use_graph=False)
+    assert torch.equal(a, b)
+    model.enable_prefetch()
+    c, _, _ = greedy_decode(model, prompt, 10, use_graph=True)
+    assert torch.equal(a, c)
+
+
 def test_toy_model_prompt_pass_kernel_attention_sdpa_and_graph_replays():
     """The prompt pass through the library's multi-token attention against the same pass through PyTorch's SDPA, and
     the captured prompt graph against eager execution on several replays with eager work and synchronisations between

@@ -728,3 +728,47 @@ def test_attention_partial_against_the_oracle(lib):
         assert (np.abs(got[i] - want) <= tol).all(), (i, float((np.abs(got[i] - want) / tol).max()))
     assert lib.ternaspmm_attention_partial_splits(1, 20, 384) in (1, 2, 4, 8)
     assert lib.ternaspmm_attention_partial_splits(8, 20, 384) == 1
+
+
+@pytest.mark.parametrize("splits", [1, 2, 4, 8])
+@pytest.mark.parametrize("h,kv,d,n_out,s_max,n", [(20, 5, 128, 2560, 384, 300), (4, 2, 64, 320, 64, 5), (16, 8, 128, 1024, 1024, 1000)])
+def test_fused_attention_merge_projection(lib, h, kv, d, n_out, s_max, n, splits):
+    """bitlinear_TernaSpMM_packed_fused_attn (merge of the attention's partial results + sub-norm + quantisation +
+    the O projection in one launch) against ternaspmm_attention_merge followed by bitlinear_TernaSpMM_packed_fused:
+    output, published activations and scale bit-identical."""
+    from tests.test_gpu_parity import repack
+    from tests._util import DeviceFormat, make_ternary
+    k_in = h * d
+    w = make_ternary(n_out, k_in, 0.40, 1900 + h)
+    packed = repack(lib, DeviceFormat(w))
+    qkv = make_bf16_activations(1, (h + 2 * kv) * d, 1901 + n)
+    k0 = make_bf16_activations(kv * s_max, d, 1902 + n).reshape(1, kv, s_max, d)
+    v0 = make_bf16_activations(kv * s_max, d, 1903 + n, outlier_frac=0.01).reshape(1, kv, s_max, d)
+    pos = np.array([n - 1], np.int64)
+    cos, sin = _angles(pos, d)
+    xd, cd, sd, pd, ck, cv = _dev(qkv), _dev(cos), _dev(sin), _dev(pos), _dev(k0), _dev(v0)
+    part = _partial_buffer(lib, 1, h, d)
+    lib.ternaspmm_rope_decode_attention_partial(_vp(xd), _vp(cd), _vp(sd), _vp(pd), 0, _vp(ck), _vp(cv), _vp(part), splits,
+                                                1, h, kv, d, s_max, float(d) ** -0.5, 1, None, None, None, 0, None)
+    norm_w = _dev(make_bf16_activations(1, k_in, 1904).reshape(-1))
+    ws = _dev(O.f32_to_bf16_bits(np.array([0.75, 0, 0, 0], np.float32)))
+    # the pair
+    attn = torch.zeros((1, k_in), dtype=torch.int16, device="cuda")
+    out1 = torch.zeros((1, n_out), dtype=torch.int16, device="cuda")
+    xq1, s1 = torch.zeros((1, k_in), dtype=torch.int8, device="cuda"), torch.zeros(1, dtype=torch.int16, device="cuda")
+    lib.ternaspmm_attention_merge(_vp(part), splits, _vp(attn), 1, h, d, None)
+    assert lib.bitlinear_TernaSpMM_packed_fused(_vp(attn), None, None, _vp(norm_w), 1e-5, _vp(packed), _vp(out1), _vp(ws), 1,
+                                                _vp(xq1), _vp(s1), 1, n_out, k_in, None) == 1
+    # one launch
+    out2 = torch.zeros_like(out1)
+    xq2, s2 = torch.zeros_like(xq1), torch.zeros_like(s1)
+    print(f"[case] fused attention merge + O projection h={h} d={d} N={n_out} n={n} splits={splits}", flush=True)
+    assert lib.bitlinear_TernaSpMM_packed_fused_attn(_vp(part), splits, d, _vp(norm_w), 1e-5, _vp(packed), _vp(out2), _vp(ws), 1,
+                                                     _vp(xq2), _vp(s2), 1, n_out, k_in, None) == 1
+    torch.cuda.synchronize()
+    assert torch.equal(xq1, xq2) and torch.equal(s1, s2)
+    assert torch.equal(out1, out2)
+    assert int(xq2.abs().max().item()) >= 126                   # a real quantised row, not zeros
+    # outside its range: two rows
+    assert lib.bitlinear_TernaSpMM_packed_fused_attn(_vp(part), splits, d, _vp(norm_w), 1e-5, _vp(packed), _vp(out2), _vp(ws), 1,
+                                                     None, None, 2, n_out, k_in, None) == 0
