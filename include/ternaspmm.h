@@ -188,15 +188,16 @@ void ternaspmm_relu2_mul_rmsnorm_quant(const terna_bf16* x13, const terna_bf16* 
  * (NULL = not written).  sum_out must not alias x or residual (every workgroup reads both).  Supported: M <= 16
  * and K <= 3072 (K <= 2560 when N > 4096); returns 1 when the launch was enqueued, 0 when the shape is outside
  * that range and nothing was done -- the caller then runs ternaspmm_rmsnorm_quant + bitlinear_TernaSpMM_packed.
- * Every workgroup repeats the prologue arithmetic, so the single launch pays for M = 1 (measured on MI355X:
- * 5.2-5.6 us against 7.2-7.5 us for the pair) and is no faster than the pair from M = 8 on. */
+ * Every workgroup repeats the prologue arithmetic (variants for 1, 2, 4, 8 and 16 rows: the lanes of a wave are spread
+ * over the rows that exist), so the single launch pays for M = 1 (measured on MI355X: 5.2-5.6 us against 7.2-7.5 us
+ * for the pair), still pays for M <= 4 and is no faster than the pair from M = 8 on. */
 int bitlinear_TernaSpMM_packed_fused(const terna_bf16* x, const terna_bf16* residual, terna_bf16* sum_out,
                                      const terna_bf16* norm_weight, float eps, const void* packed, terna_bf16* out,
                                      const terna_bf16* ws, int ws_num, int8_t* xq_out, terna_bf16* s_out, int M,
                                      int N, int K, terna_stream stream);
 
 /* Gated-FFN variant: h = bf16(bf16(relu(x1)^2) * x3) from x13 (bf16 [M][2F], as ternaspmm_relu2_mul_rmsnorm_quant),
- * norm and quantisation over F columns, then the [N][F] ternary linear.  Supported: M = 1, N <= 4096, F <= 7168;
+ * norm and quantisation over F columns, then the [N][F] ternary linear.  Supported: M <= 4, N <= 4096, F <= 7168;
  * returns 0 otherwise (caller: ternaspmm_relu2_mul_rmsnorm_quant + bitlinear_TernaSpMM_packed). */
 /* The O projection of a single-row decode step with the attention's deferred merge inside: as
  * bitlinear_TernaSpMM_packed_fused without a residual, but the activation row is formed from the partial results a

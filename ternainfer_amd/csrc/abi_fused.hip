@@ -79,13 +79,17 @@ static int launch_decode_fused(int mode, const terna_bf16* x, const terna_bf16* 
 #define TERNA_FUSED_M(WAVES, TMAX, MODE, NB)                                                                       \
     do {                                                                                                           \
         if (M == 1) TERNA_FUSED(WAVES, TMAX, MODE, 1, NB);                                                         \
+        else if (M == 2) TERNA_FUSED(WAVES, TMAX, MODE, 2, NB);                                                    \
+        else if (M <= 4) TERNA_FUSED(WAVES, TMAX, MODE, 4, NB);                                                    \
         else if (M <= 8) TERNA_FUSED(WAVES, TMAX, MODE, 8, NB);                                                    \
         else TERNA_FUSED(WAVES, TMAX, MODE, 16, NB);                                                               \
     } while (0)
     if (mode == FUSED_GLU) {
-        // long K (the down projection): only the single-row variant, whose per-lane state is tiny
-        if (M != 1 || !wide || ktiles > 16 * 7) return 0;
-        TERNA_FUSED(16, 7, FUSED_GLU, 1, 1);
+        // long K (the down projection): the variants for up to four rows, whose per-lane state is small
+        if (M > 4 || !wide || ktiles > 16 * 7) return 0;
+        if (M == 1) TERNA_FUSED(16, 7, FUSED_GLU, 1, 1);
+        else if (M == 2) TERNA_FUSED(16, 7, FUSED_GLU, 2, 1);
+        else TERNA_FUSED(16, 7, FUSED_GLU, 4, 1);
     } else if (multi16) {
         if (mode == FUSED_RESIDUAL) TERNA_FUSED_M(16, 3, FUSED_RESIDUAL, 4);
         else TERNA_FUSED_M(16, 3, FUSED_PLAIN, 4);

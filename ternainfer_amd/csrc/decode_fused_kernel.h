@@ -56,6 +56,26 @@ template <> struct RowPiece<8> {
     __device__ void unpack(float f[8]) const { unpack_bf16x8(v, f); }
     __device__ void pack(const float f[8]) { v = pack_bf16x8(f); }
 };
+template <> struct RowPiece<4> {
+    u32x2 v;
+    __device__ void load(const uint16_t* p) { v = *reinterpret_cast<const u32x2*>(p); }
+    __device__ void store(uint16_t* p) const { *reinterpret_cast<u32x2*>(p) = v; }
+    __device__ void zero() { v = u32x2{0u, 0u}; }
+    __device__ void unpack(float f[4]) const
+    {
+        f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+        f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+    }
+    __device__ void pack(const float f[4]) { v = u32x2{pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3])}; }
+};
+template <> struct RowPiece<2> {
+    uint32_t v;
+    __device__ void load(const uint16_t* p) { v = *reinterpret_cast<const uint32_t*>(p); }
+    __device__ void store(uint16_t* p) const { *reinterpret_cast<uint32_t*>(p) = v; }
+    __device__ void zero() { v = 0u; }
+    __device__ void unpack(float f[2]) const { f[0] = __uint_as_float(v << 16); f[1] = __uint_as_float(v & 0xffff0000u); }
+    __device__ void pack(const float f[2]) { v = pack_bf16x2(f[0], f[1]); }
+};
 template <> struct RowPiece<1> {
     uint16_t v;
     __device__ void load(const uint16_t* p) { v = *p; }
@@ -287,11 +307,22 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
                 bq = i32x4{static_cast<int>(first ? b4 : 0u), static_cast<int>(first ? d1 : 0u),
                            static_cast<int>(first ? d2 : 0u), static_cast<int>(first ? d3 : 0u)};
             } else {
-                uint32_t d[MP / 4];
+                constexpr int ND = MP >= 4 ? MP / 4 : 1;
+                uint32_t d[ND];
+                if constexpr (MP >= 4) {
 #pragma unroll
-                for (int e = 0; e < MP / 4; ++e)
-                    d[e] = q[4 * e] | (q[4 * e + 1] << 8) | (q[4 * e + 2] << 16) | (static_cast<uint32_t>(q[4 * e + 3]) << 24);
-                if constexpr (MP == 8) {
+                    for (int e = 0; e < ND; ++e)
+                        d[e] = q[4 * e] | (q[4 * e + 1] << 8) | (q[4 * e + 2] << 16) | (static_cast<uint32_t>(q[4 * e + 3]) << 24);
+                } else {
+                    d[0] = q[0] | (q[1] << 8);
+                }
+                if constexpr (MP == 2) {
+                    *reinterpret_cast<uint16_t*>(dst) = static_cast<uint16_t>(d[0]);
+                    if (publish) *reinterpret_cast<uint16_t*>(gdst) = static_cast<uint16_t>(d[0]);
+                } else if constexpr (MP == 4) {
+                    *reinterpret_cast<uint32_t*>(dst) = d[0];
+                    if (publish) *reinterpret_cast<uint32_t*>(gdst) = d[0];
+                } else if constexpr (MP == 8) {
                     *reinterpret_cast<u32x2*>(dst) = u32x2{d[0], d[1]};
                     if (publish) *reinterpret_cast<u32x2*>(gdst) = u32x2{d[0], d[1]};
                 } else {

@@ -154,8 +154,9 @@ def rmsnorm_quant(x, weight, eps, residual=None, quant=True):
 def rmsnorm_linear_packed(x, norm_weight, eps, packed, ws, ws_num, out_features, residual=None):
     """[residual add] -> RMSNorm -> quant_input -> int8 TernaSpMM on a P2 weight.  One launch where that is
     faster and the library supports the shape -- every workgroup of the fused kernel repeats the prologue
-    arithmetic, which pays at M = 1 (4.0-6.6 us against 6.6-8.8 us on MI355X) and, without a residual, up
-    to M = 8 (6.3 against 6.9 us; with one it is 7.7 against 7.2) -- else rmsnorm_quant + TernaInfer_linear_packed.
+    arithmetic, which pays at M = 1 (4.0-6.6 us against 6.6-8.8 us on MI355X), up to M = 4 with the 2- and 4-row
+    variants and, without a residual, up to M = 8 (6.3 against 6.9 us; with one it is 7.7 against 7.2) -- else
+    rmsnorm_quant + TernaInfer_linear_packed.
     x, residual: bf16 [M, K].  Returns (out bf16 [M, out_features], h = x + residual)."""
     m, k = x.shape
     x = x.contiguous()
@@ -166,7 +167,7 @@ def rmsnorm_linear_packed(x, norm_weight, eps, packed, ws, ws_num, out_features,
         h = torch.empty_like(x)
     out = torch.empty((m, out_features), dtype=torch.bfloat16, device=x.device)
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    one_launch = m == 1 or (m <= 8 and residual is None)
+    one_launch = m <= 4 or (m <= 8 and residual is None)
     done = one_launch and lib.bitlinear_TernaSpMM_packed_fused(
         _p(x), _p(residual) if residual is not None else None, _p(h) if residual is not None else None,
         _p(norm_weight), float(eps), _p(packed), _p(out), _p(ws), ws_num, None, None, m, out_features, k, stream)
@@ -194,15 +195,15 @@ def attention_merge_rmsnorm_linear_packed(partial, splits, heads, head_dim, norm
 
 
 def relu2_mul_rmsnorm_linear_packed(x13, norm_weight, eps, packed, ws, ws_num, out_features):
-    """squared_relu(x1) * x3 -> RMSNorm -> quant_input -> int8 TernaSpMM on a P2 weight: one launch for a single
-    row where the library supports the shape, else relu2_mul_rmsnorm_quant + TernaInfer_linear_packed.
+    """squared_relu(x1) * x3 -> RMSNorm -> quant_input -> int8 TernaSpMM on a P2 weight: one launch for up to four
+    rows where the library supports the shape, else relu2_mul_rmsnorm_quant + TernaInfer_linear_packed.
     x13: bf16 [M, 2F].  Returns out bf16 [M, out_features]."""
     m, f2 = x13.shape
     x13 = x13.contiguous()
     lib = _lib.load()
     out = torch.empty((m, out_features), dtype=torch.bfloat16, device=x13.device)
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    if m == 1 and lib.bitlinear_TernaSpMM_packed_fused_glu(_p(x13), _p(norm_weight), float(eps), _p(packed), _p(out), _p(ws),
+    if m <= 4 and lib.bitlinear_TernaSpMM_packed_fused_glu(_p(x13), _p(norm_weight), float(eps), _p(packed), _p(out), _p(ws),
                                                          ws_num, None, None, m, out_features, f2 // 2, stream):
         return out
     xq, s = relu2_mul_rmsnorm_quant(x13, norm_weight, eps)

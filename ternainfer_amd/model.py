@@ -174,7 +174,7 @@ class Block:
             return lin(rms_norm(h, weight, eps)), h
         if glu:
             if self.act == "int8":
-                if x.shape[0] == 1:
+                if x.shape[0] <= 4:
                     return relu2_mul_rmsnorm_linear_packed(x, weight, eps, lin.packed, lin.ws, lin.ws_num, lin.n), None
                 return lin.quantised(*relu2_mul_rmsnorm_quant(x, weight, eps)), None
             return lin.dense(relu2_mul_rmsnorm_quant(x, weight, eps, quant=False)), None

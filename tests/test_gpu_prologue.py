@@ -289,7 +289,7 @@ def _bf16_key(b):
     return np.where(b & 0x8000, -(b & 0x7FFF), b & 0x7FFF)
 
 
-@pytest.mark.parametrize("m", [1, 2, 8, 11, 16])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 8, 11, 16])
 @pytest.mark.parametrize("n,k,ws_num,res", [(3840, 2560, 3, True), (2560, 2560, 1, False), (13824, 2560, 2, True),
                                             (256, 192, 1, True), (320, 64, 2, False), (4160, 128, 1, False)])
 def test_fused_prologue_linear(lib, m, n, k, ws_num, res):
@@ -366,24 +366,25 @@ def test_rmsnorm_linear_wrapper_matches_two_launch_sequence(lib):
         assert err <= 2e-2 * out2.float().abs().max().item()
 
 
+@pytest.mark.parametrize("m", [1, 2, 3, 4])
 @pytest.mark.parametrize("n,f,ws_num", [(2560, 6912, 1), (256, 192, 2), (320, 7168, 1)])
-def test_fused_gate_prologue_linear(lib, n, f, ws_num):
-    """Single row: squared_relu(x1) * x3 -> norm -> quantise -> matmul in one launch; same bars as above."""
+def test_fused_gate_prologue_linear(lib, n, f, ws_num, m):
+    """Up to four rows: squared_relu(x1) * x3 -> norm -> quantise -> matmul in one launch; same bars as above."""
     from tests._util import DeviceFormat, make_ternary
     w = make_ternary(n, f, 0.40, 870 + n)
     fmt = DeviceFormat(w)
     packed = torch.empty(n * f // 16, dtype=torch.int32, device="cuda")
     lib.ternaspmm_repack(_vp(fmt.bm), _vp(fmt.off), _vp(fmt.med), _vp(fmt.vals), _vp(packed), n, f, None)
-    x13 = make_bf16_activations(1, 2 * f, 871 + f, outlier_frac=0.01)
+    x13 = make_bf16_activations(m, 2 * f, 871 + f + m, outlier_frac=0.01)
     g = _weight(f, 872)
     ws = O.f32_to_bf16_bits(np.array([1.25, 0.75, 0.0, 0.0], np.float32))
     xd, gd, wsd = _dev(x13), _dev(g), _dev(ws)
-    od = torch.zeros((1, n), dtype=torch.int16, device="cuda")
-    qd = torch.zeros((1, f), dtype=torch.int8, device="cuda")
-    sd = torch.zeros(1, dtype=torch.int16, device="cuda")
-    print(f"[case] fused gate prologue linear n={n} f={f}", flush=True)
+    od = torch.zeros((m, n), dtype=torch.int16, device="cuda")
+    qd = torch.zeros((m, f), dtype=torch.int8, device="cuda")
+    sd = torch.zeros(m, dtype=torch.int16, device="cuda")
+    print(f"[case] fused gate prologue linear m={m} n={n} f={f}", flush=True)
     assert lib.bitlinear_TernaSpMM_packed_fused_glu(_vp(xd), _vp(gd), 1e-5, _vp(packed), _vp(od), _vp(wsd), ws_num, _vp(qd),
-                                                    _vp(sd), 1, n, f, None) == 1
+                                                    _vp(sd), m, n, f, None) == 1
     torch.cuda.synchronize()
     q, s = qd.cpu().numpy(), sd.cpu().numpy().view(np.uint16)
     y64 = O.rmsnorm(O.relu2_mul(x13), g, 1e-5)
@@ -394,7 +395,7 @@ def test_fused_gate_prologue_linear(lib, n, f, ws_num):
     assert dq.max() <= 1 and (dq != 0).mean() < 0.02
     assert (od.cpu().numpy().view(np.uint16) == O.spmm_i8(q, w, s, ws, ws_num, 0)).all()
     z = torch.zeros(64, dtype=torch.int32, device="cuda")
-    assert lib.bitlinear_TernaSpMM_packed_fused_glu(_vp(z), _vp(z), 1e-5, _vp(z), _vp(z), _vp(z), 1, None, None, 2, n, f, None) == 0
+    assert lib.bitlinear_TernaSpMM_packed_fused_glu(_vp(z), _vp(z), 1e-5, _vp(z), _vp(z), _vp(z), 1, None, None, 5, n, f, None) == 0
 
 
 @pytest.mark.parametrize("split", [False, True])
