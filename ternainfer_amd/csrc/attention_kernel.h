@@ -313,15 +313,12 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     auto cache_slot = [&](int l) { return (((l >> 4) * SP + sp) << 4) + (l & 15); };
     const int bh = b * H + h;
     const int kvh = h / (H / KV);
-    // Prefix length: slots 0 .. pos[0].  pos comes from device memory the host cannot check, so it is clamped to the
-    // cache -- the LDS score buffer and every cache address are sized by S -- and a position outside [0, S) writes no
-    // cache row below (the attention then runs over the clamped prefix; its result is not meaningful, but in bounds).
     const int pb = per_seq ? b : 0;              // row of the position / angle tables
+    // (the position is requested here and first looked at after every other request of the launch has been issued: none
+    // of their addresses depends on it, and waiting for it first put one memory round trip in front of all the others)
     const long long p0 = pos[pb];
     const float* cosv = cosv_all + pb * (D / 2);
     const float* sinv = sinv_all + pb * (D / 2);
-    const bool pos_ok = p0 >= 0 && p0 < S;
-    const int n = p0 < 0 ? 1 : (p0 >= S ? S : static_cast<int>(p0) + 1);
     const uint16_t* kbase = cache_k + (static_cast<size_t>(b) * KV + kvh) * S * D;
     const uint16_t* vbase = cache_v + (static_cast<size_t>(b) * KV + kvh) * S * D;
 
@@ -356,6 +353,34 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
             dst[j] = *reinterpret_cast<const u32x4*>(kbase + static_cast<size_t>(sk < S ? sk : 0) * D + 8 * piece);
         }
     };
+    // Order of the requests: the new token's own row pieces and angles first (ROPE) -- loads return in order, so
+    // the rotation can run while the cache rows are still on their way -- then the keys, then the values.
+    u32x4 knew, vnew;                            // ROPE: the new token's key piece of this lane, value chunk of this thread
+    u32x4 q_own, k_own, q_par, k_par;            // raw pieces of the new token's q / k rows (q_par, k_par: rotate-half partners)
+    f32x4 cs[2], sn[2];
+    const u32x4 zero4 = {0u, 0u, 0u, 0u};
+    const int c = piece;                         // chunk c = dimensions 8c .. 8c+7
+    const int cp = (c + CH / 2) % CH, ca = c % (CH / 2);      // rotate-half: the partner chunk, the angle chunk
+    if constexpr (!ROPE) {
+        qb = *reinterpret_cast<const u32x4*>(q + (static_cast<size_t>(b) * H + h) * D + 8 * piece);
+    } else {
+        const uint16_t* row = q + static_cast<size_t>(b) * (H + 2 * KV) * D;
+        q_own = *reinterpret_cast<const u32x4*>(row + h * D + 8 * c);
+        k_own = *reinterpret_cast<const u32x4*>(row + (H + kvh) * D + 8 * c);
+        vnew = *reinterpret_cast<const u32x4*>(row + (H + KV + kvh) * D + 8 * chunk);
+        if constexpr (ADJACENT) {                // a chunk holds the pairs 4c .. 4c+3 whole
+            cs[0] = *reinterpret_cast<const f32x4*>(cosv + 4 * c);
+            sn[0] = *reinterpret_cast<const f32x4*>(sinv + 4 * c);
+        } else {                                 // the chunk and its rotation partner c +- CH/2
+            q_par = *reinterpret_cast<const u32x4*>(row + h * D + 8 * cp);
+            k_par = *reinterpret_cast<const u32x4*>(row + (H + kvh) * D + 8 * cp);
+            cs[0] = *reinterpret_cast<const f32x4*>(cosv + 8 * ca);
+            cs[1] = *reinterpret_cast<const f32x4*>(cosv + 8 * ca + 4);
+            sn[0] = *reinterpret_cast<const f32x4*>(sinv + 8 * ca);
+            sn[1] = *reinterpret_cast<const f32x4*>(sinv + 8 * ca + 4);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);           // the requests above stay above the ones below
 #pragma unroll
     for (int t = 0; t < KT; ++t) load_keys(wave + NW * t, kr[t]);
 #pragma unroll
@@ -363,45 +388,28 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
         const int sv = cache_slot(slice + u * SLICES);
         vr[u] = *reinterpret_cast<const u32x4*>(vbase + static_cast<size_t>(sv < S ? sv : 0) * D + chunk * 8);
     }
-    u32x4 knew, vnew;                            // ROPE: the new token's key piece of this lane, value chunk of this thread
-    const u32x4 zero4 = {0u, 0u, 0u, 0u};
-    if constexpr (!ROPE) {
-        qb = *reinterpret_cast<const u32x4*>(q + (static_cast<size_t>(b) * H + h) * D + 8 * piece);
-    } else {
-        const uint16_t* row = q + static_cast<size_t>(b) * (H + 2 * KV) * D;
-        vnew = *reinterpret_cast<const u32x4*>(row + (H + KV + kvh) * D + 8 * chunk);
-        const int c = piece;                     // chunk c = dimensions 8c .. 8c+7
+    __builtin_amdgcn_sched_barrier(0);           // everything is requested; only now the position is looked at
+    // Prefix length: slots 0 .. pos.  It comes from device memory the host cannot check, so it is clamped to the
+    // cache -- the LDS score buffer and every cache address are sized by S -- and a position outside [0, S) writes no
+    // cache row below (the attention then runs over the clamped prefix; its result is not meaningful, but in bounds).
+    const bool pos_ok = p0 >= 0 && p0 < S;
+    const int n = p0 < 0 ? 1 : (p0 >= S ? S : static_cast<int>(p0) + 1);
+    if constexpr (ROPE) {
         if constexpr (ADJACENT) {
-            // a chunk holds the pairs 4c .. 4c+3 whole
-            const u32x4 q_own = *reinterpret_cast<const u32x4*>(row + h * D + 8 * c);
-            const u32x4 k_own = *reinterpret_cast<const u32x4*>(row + (H + kvh) * D + 8 * c);
-            const f32x4 cs = *reinterpret_cast<const f32x4*>(cosv + 4 * c);
-            const f32x4 sn = *reinterpret_cast<const f32x4*>(sinv + 4 * c);
             auto rotate = [&](const u32x4& own) {
                 float a[8], o[8];
                 unpack_bf16x8(own, a);
 #pragma unroll
                 for (int m = 0; m < 4; ++m) {
 #pragma clang fp contract(off)                   // as terna_rope_kv_store_kernel: every product and sum rounded once
-                    o[2 * m] = a[2 * m] * cs[m] - a[2 * m + 1] * sn[m];
-                    o[2 * m + 1] = a[2 * m + 1] * cs[m] + a[2 * m] * sn[m];
+                    o[2 * m] = a[2 * m] * cs[0][m] - a[2 * m + 1] * sn[0][m];
+                    o[2 * m + 1] = a[2 * m + 1] * cs[0][m] + a[2 * m] * sn[0][m];
                 }
                 return pack_bf16x8(o);
             };
             qb = rotate(q_own);
             knew = rotate(k_own);
         } else {
-            // the chunk and its rotation partner c +- CH/2
-            const int cp = (c + CH / 2) % CH, ca = c % (CH / 2);
-            const u32x4 q_own = *reinterpret_cast<const u32x4*>(row + h * D + 8 * c);
-            const u32x4 q_par = *reinterpret_cast<const u32x4*>(row + h * D + 8 * cp);
-            const u32x4 k_own = *reinterpret_cast<const u32x4*>(row + (H + kvh) * D + 8 * c);
-            const u32x4 k_par = *reinterpret_cast<const u32x4*>(row + (H + kvh) * D + 8 * cp);
-            f32x4 cs[2], sn[2];
-            cs[0] = *reinterpret_cast<const f32x4*>(cosv + 8 * ca);
-            cs[1] = *reinterpret_cast<const f32x4*>(cosv + 8 * ca + 4);
-            sn[0] = *reinterpret_cast<const f32x4*>(sinv + 8 * ca);
-            sn[1] = *reinterpret_cast<const f32x4*>(sinv + 8 * ca + 4);
             const bool first_half = c < CH / 2;
             auto rotate = [&](const u32x4& own, const u32x4& par) {
                 float a[8], p[8], o[8];
@@ -420,7 +428,7 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
             qb = rotate(q_own, q_par);
             knew = rotate(k_own, k_par);
         }
-        if (h % (H / KV) == 0 && sp == 0 && pos_ok) {      // this kv group's writer: slot pos[0] of both caches
+        if (h % (H / KV) == 0 && sp == 0 && pos_ok) {      // this kv group's writer: slot pos of both caches
             const size_t slot_off = ((static_cast<size_t>(b) * KV + kvh) * S + (n - 1)) * D;
             if (wave == 0 && r16 < R) *reinterpret_cast<u32x4*>(cache_k + slot_off + 8 * c) = knew;   // r16 < R: every chunk once
             if (tid < CH) *reinterpret_cast<u32x4*>(cache_v + slot_off + 8 * chunk) = vnew;
