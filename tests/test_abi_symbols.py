@@ -78,3 +78,20 @@ def test_unsupported_shapes_are_refused_before_any_device_work():
     assert r.stdout.count("unsupported K=262144 with int8 activations (need K <= 262080)") == 2
     assert "unsupported ws_num=5" in r.stdout
     assert r.stdout.rstrip().endswith("returned")
+
+
+def test_host_side_size_and_policy_functions():
+    """Functions that only compute on the host: buffer sizes and the recommended split count of the attention."""
+    from ternainfer_amd import _lib
+    lib = _lib.load()
+    assert lib.ternaspmm_packed_bytes(2560, 6912) == 2560 * 6912 // 4
+    assert lib.ternaspmm_packed_bytes(2560, 100) < 0
+    assert lib.ternaspmm_attention_partial_bytes(1, 20, 128) == 4 * (20 * 16 + 20 * 8 * 128)
+    assert lib.ternaspmm_attention_partial_bytes(0, 20, 128) == -1
+    assert lib.ternaspmm_attention_partial_splits(1, 20, 384) == 4       # up to 1024 slots: four splits
+    assert lib.ternaspmm_attention_partial_splits(1, 20, 4096) == 8      # beyond: eight
+    assert lib.ternaspmm_attention_partial_splits(8, 20, 384) == 1       # the heads fill the chip anyway
+    assert lib.ternaspmm_attention_partial_splits(1, 20, 32) == 1        # a split must keep two tiles
+    assert lib.ternaspmm_attention_partial_splits(1, 20, 64) == 2
+    assert lib.ternaspmm_attention_partial_splits(1, 20, 128) == 4
+    assert lib.ternaspmm_attention_workspace_bytes(1, 20, 128) > 0
