@@ -19,7 +19,7 @@ The default run (`--workload decode`) also measures, in the same process and int
 the other figures the path is judged on: the literal single-matrix configuration (`config1`),
 the layer set at M = 1 and 16, the unmodified call site (`drop_in_reference_format`), the prefill
 shapes at M = 2048 for both activation types (`prefill_m2048`), the 2B-shaped model's decode
-tokens/s at batch 1 and 8 (`model_decode`) and what the machine gives (`calibration`: cost of a
+tokens/s at batch 1 and 8 and, for one sequence, far into a 2048-slot context (`model_decode`) and what the machine gives (`calibration`: cost of a
 graph kernel node, read and copy rate, cost of a device-wide synchronisation).  `--no-extras`
 leaves those out.
 """
@@ -208,8 +208,8 @@ def cpu_baseline(mats, torch):
 
 
 # ------------------------------------------------------------------------------------------------ model (configs[4])
-def measure_model(torch, batch, act="int8", prefetch=True, gen_tokens=256, check_tokens=8, model=None):
-    """2B-shaped random-init model, prompt of 128 uniform random ids, greedy decode of `gen_tokens`
+def measure_model(torch, batch, act="int8", prefetch=True, gen_tokens=256, check_tokens=8, model=None, prompt_tokens=128):
+    """2B-shaped random-init model, prompt of `prompt_tokens` (128) uniform random ids, greedy decode of `gen_tokens`
     tokens; tokens/s = generated tokens / decode-phase time (as the reference's stats.py:19-27).
     Self-check of the run: the captured decode graph must produce the tokens of eager execution
     for the first `check_tokens` tokens.  Returns (figures, model)."""
@@ -224,7 +224,7 @@ def measure_model(torch, batch, act="int8", prefetch=True, gen_tokens=256, check
     torch.cuda.synchronize()
     build_s = time.perf_counter() - t0
     gen = torch.Generator(device="cuda").manual_seed(20260501)
-    prompt = torch.randint(0, margs.vocab_size, (batch, 128), generator=gen, device="cuda")
+    prompt = torch.randint(0, margs.vocab_size, (batch, prompt_tokens), generator=gen, device="cuda")
     warm, _, _ = greedy_decode(model, prompt, check_tokens)                     # warm-up (code objects, allocator)
     eager, _, _ = greedy_decode(model, prompt, check_tokens, use_graph=False)
     graph_equals_eager = bool(torch.equal(warm, eager))
@@ -232,7 +232,8 @@ def measure_model(torch, batch, act="int8", prefetch=True, gen_tokens=256, check
     toks, prefill_s, decode_s = greedy_decode(model, prompt, gen_tokens)
     assert torch.equal(toks[:, :check_tokens], eager)
     return {"batch": batch, "tokens_per_s": batch * gen_tokens / decode_s, "ms_per_step": decode_s * 1e3 / gen_tokens,
-            "prefill_tokens_per_s": batch * 128 / prefill_s, "prefill_ms": prefill_s * 1e3, "decode_s": decode_s,
+            "prefill_tokens_per_s": batch * prompt_tokens / prefill_s, "prefill_ms": prefill_s * 1e3, "decode_s": decode_s,
+            "prompt_tokens": prompt_tokens,
             "generated_tokens": gen_tokens, "graph_equals_eager_first_tokens": check_tokens,
             "first_tokens": toks[0, :8].tolist(), "model_build_s": build_s}, model
 
@@ -718,6 +719,8 @@ def main():
         md = {}
         for batch in (1, 8):
             md[f"batch{batch}"], model = measure_model(torch, batch, "int8", True, model=model)
+        # the same model far into a long context: one sequence, 1920-token prompt, 128 tokens (cache of 2048 slots)
+        md["batch1_context2048"], model = measure_model(torch, 1, "int8", True, gen_tokens=128, model=model, prompt_tokens=1920)
         result["model_decode"] = md
         del model
         torch.cuda.empty_cache()
