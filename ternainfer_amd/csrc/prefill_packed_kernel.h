@@ -39,13 +39,35 @@ __device__ __forceinline__ void int8x16_to_bf16(const u32x4& v, u32x4& c0, u32x4
     c1 = u32x4{o[4], o[5], o[6], o[7]};
 }
 
+// A wave's finished 32 batch rows x 32*NA features on their way to memory.  In the accumulator layout a lane holds
+// four consecutive features of ONE batch row, so a direct store writes 8 bytes into each of 32 rows that lie N * 2
+// bytes apart: 64 lanes, 32 memory segments, and the memory pipeline takes one step per segment.  Through this LDS
+// tile the same block leaves as whole rows -- 16 bytes per lane, 4*NA consecutive lanes per row of 64*NA contiguous
+// bytes -- in an eighth of the store instructions' pipeline steps (gate+up at M = 2048, same box: int8 76 -> 69 us, and
+// 64 us with streaming stores; bf16 120 -> 117 us).
+// Rows are 64*NA bytes with no padding; the 16-byte piece c of row r sits at position c ^ swizzle(r) so that both the
+// 8-byte writes of 32 consecutive rows and the 16-byte reads of 4*NA-lane rows spread over all banks.
+template <int NA>
+struct OutTile {
+    static constexpr int kRowBytes = 64 * NA;
+    static constexpr int kBytes = 32 * kRowBytes;            // per wave
+    static constexpr int kPieces = 4 * NA;                   // 16-byte pieces per row
+    static constexpr int kRowsPerRead = 64 / kPieces;        // rows that one 64-lane, 16-byte read covers
+    static constexpr int kReads = 32 / kRowsPerRead;
+    __device__ static constexpr int swizzle(int row) { return (row >> (NA == 2 ? 1 : 2)) & (kPieces - 1); }
+};
+
 // Fused epilogue of one wave's NA x MB accumulator tiles (v_mfma_f32_32x32x16 layout: lane holds
 // column m = L % 32 and rows n = (v&3) + 8(v>>2) + 4(L/32) of each tile).  A float accumulator is
 // twice the true sum (weights were +-2; x0.5 is exact); an integer one is the sum times 64 (weights were +-64; >> 6 is exact).
+// `tile`: this wave's OutTile<NA>::kBytes of LDS (results leave as whole rows; needs out and N * 2 to be multiples of
+// 16 bytes), or nullptr (every lane stores its 8-byte pieces itself).
 template <int MB, int NA, typename AccV>
 __device__ __forceinline__ void packed_prefill_epilogue(AccV (&acc)[NA][MB], uint16_t* __restrict__ out,
-                                                        const Epilogue& ep, int M, int N, int n_wave, int m0, int lane)
+                                                        const Epilogue& ep, int M, int N, int n_wave, int m0, int lane,
+                                                        uint8_t* tile = nullptr)
 {
+    using OT = OutTile<NA>;
     const int kb = lane >> 5, l32 = lane & 31;
     constexpr bool kFloatAcc = std::is_same<AccV, f32x16>::value;
     auto value = [&](auto ac, auto bc, int idx) {
@@ -60,9 +82,34 @@ __device__ __forceinline__ void packed_prefill_epilogue(AccV (&acc)[NA][MB], uin
         m_of[b] = m0 + 32 * b + l32;
         s_of[b] = ep.kind == EP_BF16 ? 1.0f : bf16_bits_to_float(ep.s[m_of[b] < M ? m_of[b] : M - 1]);
     });
-    auto store4 = [&](int b_m, int n, float r0, float r1, float r2, float r3) {
-        if (b_m < M && n < N)
-            *reinterpret_cast<u32x2*>(out + static_cast<size_t>(b_m) * N + n) = u32x2{pack_bf16x2(r0, r1), pack_bf16x2(r2, r3)};
+    // features 32a + 8vq + 4kb .. +3 of batch row 32b + l32
+    const int tile_put = l32 * OT::kRowBytes + 8 * kb, tile_swz = OT::swizzle(l32);
+    auto store4 = [&](int a, int b, int vq, float r0, float r1, float r2, float r3) {
+        const u32x2 v = {pack_bf16x2(r0, r1), pack_bf16x2(r2, r3)};
+        if (tile != nullptr) {
+            *reinterpret_cast<u32x2*>(tile + tile_put + (((4 * a + vq) ^ tile_swz) << 4)) = v;
+        } else {
+            const int n = n_wave + 32 * a + 8 * vq + 4 * kb;
+            if (m_of[b] < M && n < N) *reinterpret_cast<u32x2*>(out + static_cast<size_t>(m_of[b]) * N + n) = v;
+        }
+    };
+    // after the last store4 of batch block b: its 32 rows leave the tile as rows
+    auto flush = [&](int b) {
+        if (tile == nullptr) return;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        const int piece = lane & (OT::kPieces - 1);
+        const int n = n_wave + 8 * piece;
+#pragma unroll
+        for (int i = 0; i < OT::kReads; ++i) {
+            const int row = i * OT::kRowsPerRead + lane / OT::kPieces;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(tile + row * OT::kRowBytes + ((piece ^ OT::swizzle(row)) << 4));
+            const int m = m0 + 32 * b + row;
+            // written once and read by a later launch: a streaming store keeps it from displacing the operands in L2
+            if (m < M && n < N) __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(out + static_cast<size_t>(m) * N + n));
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
     };
 
     // One weight-group scale per 32-feature tile whenever the group boundaries fall on multiples of
@@ -81,57 +128,46 @@ __device__ __forceinline__ void packed_prefill_epilogue(AccV (&acc)[NA][MB], uin
                                                                        : ws_group_decode(n_a, N, ep.ws_num));
             w_of[a] = ep.kind == EP_BF16 ? ep.scale[g] : bf16_bits_to_float(ep.ws[g]);
         });
-        // Two separate loops under a uniform branch: written as a select, the compiler evaluates the
+        // Separate loops under a uniform branch: written as a select, the compiler evaluates the
         // IEEE division of the decode rule for every element of every kind.
         auto tiles = [&](auto&& element) {
-            static_for<0, NA>([&](auto ac) {
-                constexpr int a = decltype(ac)::value;
-                static_for<0, MB>([&](auto bc) {
-                    constexpr int b = decltype(bc)::value;
+            static_for<0, MB>([&](auto bc) {
+                constexpr int b = decltype(bc)::value;
+                static_for<0, NA>([&](auto ac) {
+                    constexpr int a = decltype(ac)::value;
                     static_for<0, 4>([&](auto vc) {
                         constexpr int vq = decltype(vc)::value;
                         float r[4];
 #pragma unroll
-                        for (int v = 0; v < 4; ++v) r[v] = element(w_of[a], s_of[b], value(ac, bc, 4 * vq + v));
-                        store4(m_of[b], n_wave + 32 * a + 8 * vq + 4 * kb, r[0], r[1], r[2], r[3]);
+                        for (int v = 0; v < 4; ++v) r[v] = element(ac, bc, value(ac, bc, 4 * vq + v));
+                        store4(a, b, vq, r[0], r[1], r[2], r[3]);
                     });
                 });
+                flush(b);
             });
         };
         if (ep.kind == EP_I8_DECODE) {
-            tiles([](float w, float sm, float x) { return __fmul_rn(__fdiv_rn(x, sm), w); });
+            tiles([&](auto ac, auto bc, float x) { return __fmul_rn(__fdiv_rn(x, s_of[decltype(bc)::value]), w_of[decltype(ac)::value]); });
         } else if (ep.kind == EP_I8_PREFILL) {
             float coeff[NA][MB];
 #pragma unroll
             for (int a = 0; a < NA; ++a)
 #pragma unroll
                 for (int b = 0; b < MB; ++b) coeff[a][b] = s_of[b] != 0.0f ? __fdiv_rn(w_of[a], s_of[b]) : 0.0f;
-            static_for<0, NA>([&](auto ac) {
-                constexpr int a = decltype(ac)::value;
-                static_for<0, MB>([&](auto bc) {
-                    constexpr int b = decltype(bc)::value;
-                    static_for<0, 4>([&](auto vc) {
-                        constexpr int vq = decltype(vc)::value;
-                        float r[4];
-#pragma unroll
-                        for (int v = 0; v < 4; ++v) r[v] = __fmul_rn(value(ac, bc, 4 * vq + v), coeff[a][b]);
-                        store4(m_of[b], n_wave + 32 * a + 8 * vq + 4 * kb, r[0], r[1], r[2], r[3]);
-                    });
-                });
-            });
+            tiles([&](auto ac, auto bc, float x) { return __fmul_rn(x, coeff[decltype(ac)::value][decltype(bc)::value]); });
         } else {
-            tiles([](float w, float, float x) { return __fmul_rn(x, w); });
+            tiles([&](auto ac, auto, float x) { return __fmul_rn(x, w_of[decltype(ac)::value]); });
         }
         return;
     }
     // group boundaries inside a tile: per-column scales
-    static_for<0, 4 * NA>([&](auto tc) {
-        constexpr int a = decltype(tc)::value >> 2, vq = decltype(tc)::value & 3;
-        const int n = n_wave + 32 * a + 8 * vq + 4 * kb;
-        float wv[4];
-        load_col_scales(ep, n < N ? n : N - 4, N, wv);
-        static_for<0, MB>([&](auto bc) {
-            constexpr int b = decltype(bc)::value;
+    static_for<0, MB>([&](auto bc) {
+        constexpr int b = decltype(bc)::value;
+        static_for<0, 4 * NA>([&](auto tc) {
+            constexpr int a = decltype(tc)::value >> 2, vq = decltype(tc)::value & 3;
+            const int n = n_wave + 32 * a + 8 * vq + 4 * kb;
+            float wv[4];
+            load_col_scales(ep, n < N ? n : N - 4, N, wv);
             EpilogueRegs eb;
             eb.s = s_of[b];
 #pragma unroll
@@ -140,8 +176,9 @@ __device__ __forceinline__ void packed_prefill_epilogue(AccV (&acc)[NA][MB], uin
 #pragma unroll
             for (int v = 0; v < 4; ++v)
                 r[v] = bf16_bits_to_float(apply_epilogue<float>(ep.kind, eb, v, value(std::integral_constant<int, a>{}, bc, 4 * vq + v)));
-            store4(m_of[b], n, r[0], r[1], r[2], r[3]);
+            store4(a, b, vq, r[0], r[1], r[2], r[3]);
         });
+        flush(b);
     });
 }
 
@@ -579,7 +616,13 @@ __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) voi
                                              n0 + 32 * NA * wave, m0, lane);
         return;
     }
-    packed_prefill_epilogue<MB, NA>(acc, out, ep, M, N, n0 + 32 * NA * wave, m0, lane);
+    // results leave as whole rows through a per-wave LDS tile whenever 16-byte stores can address the output; the tiles
+    // take the place of the activation stages once every wave is done reading those
+    static_assert(4 * OutTile<NA>::kBytes <= S::kBytes, "output tiles fit in the activation stages");
+    const bool rows_ok = ((reinterpret_cast<uintptr_t>(out) | (static_cast<uintptr_t>(N) * 2)) & 15) == 0;
+    __syncthreads();
+    packed_prefill_epilogue<MB, NA>(acc, out, ep, M, N, n0 + 32 * NA * wave, m0, lane,
+                                    rows_ok ? smem + wave * OutTile<NA>::kBytes : nullptr);
 }
 
 // Second launch of a split-K call: out[m][n0 .. n0+3] = epilogue(sum over the splits, in split order, of partial[z][m][n]).
