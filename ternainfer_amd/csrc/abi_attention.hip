@@ -1,5 +1,6 @@
 // C ABI of the attention-side kernels of a decode step (attention_kernel.h): RoPE + cache write, single-token
-// attention, both in one launch, the prefetching variant, and the variant that allocates nothing.
+// attention, both in one launch, the prefetching variant, and the variant that allocates nothing.  The multi-token
+// attention of a prompt pass: abi_prefill_attention.hip.
 // Declarations: include/ternaspmm.h.
 #include <hip/hip_runtime.h>
 
@@ -10,7 +11,6 @@
 #include "../../include/ternaspmm.h"
 #include "host_util.h"
 #include "attention_kernel.h"
-#include "prefill_attention_kernel.h"
 
 using namespace terna;
 
@@ -142,15 +142,6 @@ void launch_attention(const uint16_t* q, uint16_t* ck, uint16_t* cv, const float
 #undef TERNA_ATTN
 }
 
-bool attention_args_ok(const char* who, int B, int H, int KV, int D, int S)
-{
-    if (B < 1 || H < 1 || KV < 1 || H % KV != 0 || (D != 64 && D != 128) || S < 1 || S > 8192) {
-        std::fprintf(stderr, "%s: unsupported arguments (H=%d KV=%d D=%d S=%d)\n", who, H, KV, D, S);
-        return false;
-    }
-    return true;
-}
-
 // The regions of a prefetching launch from the caller's host arrays; a region that breaks a rule is skipped.
 AttentionPrefetch prefetch_regions(const void* const* pf_ptr, const long long* pf_bytes, const long long* pf_unit_bytes, int pf_count)
 {
@@ -258,22 +249,6 @@ void ternaspmm_decode_attention(const terna_bf16* q, const terna_bf16* cache_k, 
                                    static_cast<hipStream_t>(stream));
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_decode_attention", e, __LINE__);
-}
-
-void ternaspmm_prefill_attention(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
-                                 const long long* pos, int per_sequence, terna_bf16* out, int B, int T, int H, int KV, int D, int S,
-                                 float scale, terna_stream stream)
-{
-    if (!attention_args_ok("ternaspmm_prefill_attention", B, H, KV, D, S) || T < 1 || B > 65535 || H > 65535) {
-        if (T < 1 || B > 65535 || H > 65535) std::fprintf(stderr, "ternaspmm_prefill_attention: unsupported arguments (B=%d T=%d H=%d)\n", B, T, H);
-        return;
-    }
-    const dim3 grid((T + 15) / 16, H, B);
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    if (D == 128) terna_prefill_attention_kernel<128><<<grid, dim3(64), 0, st>>>(q, cache_k, cache_v, pos, out, T, H, KV, S, scale, per_sequence != 0);
-    else terna_prefill_attention_kernel<64><<<grid, dim3(64), 0, st>>>(q, cache_k, cache_v, pos, out, T, H, KV, S, scale, per_sequence != 0);
-    const hipError_t e = hipGetLastError();
-    if (e != hipSuccess) die("ternaspmm_prefill_attention", e, __LINE__);
 }
 
 int ternaspmm_decode_attention_static(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,

@@ -84,4 +84,14 @@ void allow_dynamic_lds(Kernel kernel, int bytes, const char* what, int line)
     allow_dynamic_lds_ptr(reinterpret_cast<const void*>(kernel), bytes, what, line);
 }
 
+// Shapes the attention entry points accept (head sizes 64 and 128, whole kv groups, caches of up to 8192 slots).
+inline bool attention_args_ok(const char* who, int B, int H, int KV, int D, int S)
+{
+    if (B < 1 || H < 1 || KV < 1 || H % KV != 0 || (D != 64 && D != 128) || S < 1 || S > 8192) {
+        std::fprintf(stderr, "%s: unsupported arguments (H=%d KV=%d D=%d S=%d)\n", who, H, KV, D, S);
+        return false;
+    }
+    return true;
+}
+
 }  // namespace terna

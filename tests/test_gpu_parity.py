@@ -589,6 +589,43 @@ def test_large_m_with_workspace_matches_without(lib):
     _check_bf16(run_bf16(lib, fmt, x, scale, 1, workspace=False), ref)
 
 
+@pytest.mark.parametrize("n", [384, 192])
+def test_large_m_output_store_paths_agree(lib, n):
+    """The MFMA-tiled kernels write whole rows (16 bytes per lane, through an LDS tile) when the output pointer
+    and row pitch are multiples of 16 bytes and 8-byte pieces otherwise: an output buffer shifted by 8 bytes must
+    receive the same bits, for both families, with ragged M and a feature count that leaves the last tile partly
+    outside N, and nothing outside the [M][N] block may be written."""
+    k, m = 320, 200
+    w = make_ternary(n, k, 0.40, 461 + n)
+    packed = repack(lib, DeviceFormat(w))
+    x = make_bf16_activations(m, k, 462, outlier_frac=0.01)
+    xq, s = make_int8_activations(m, k, 463)
+    scale = np.array([1.25], np.float32)
+    want_bf = run_bf16_packed(lib, packed, n, x, scale, 1, route=1)
+    want_i8 = run_i8_packed(lib, packed, n, xq, s, WS, 1, route=9)     # MFMA-tiled kernel, prefill epilogue
+    xd = torch.from_numpy(x.view(np.int16)).cuda()
+    xqd = torch.from_numpy(xq).cuda()
+    sd = torch.from_numpy(s.view(np.int16)).cuda()
+    wsd = torch.from_numpy(WS.view(np.int16)).cuda()
+    scd = torch.from_numpy(scale).cuda()
+    for shift in (4, 8):       # elements: 8 bytes (pieces), 16 bytes (rows again)
+        buf = torch.full((m * n + 64,), -1, dtype=torch.int16, device="cuda")
+        out = buf[shift:shift + m * n]
+        print(f"[case] bitlinear_TernaSpMM_bf16_packed M={m} N={n} K={k}, output shifted by {2 * shift} bytes", flush=True)
+        lib.bitlinear_TernaSpMM_bf16_packed(vp(xd), vp(packed), vp(out), vp(scd), 1, m, n, k, 1, _stream())
+        torch.cuda.synchronize()
+        got = buf.cpu().numpy().view(np.uint16)
+        assert (got[shift:shift + m * n].reshape(m, n) == want_bf).all()
+        assert (got[:shift] == 0xFFFF).all() and (got[shift + m * n:] == 0xFFFF).all()
+        buf.fill_(-1)
+        print(f"[case] bitlinear_TernaSpMM_packed M={m} N={n} K={k}, output shifted by {2 * shift} bytes", flush=True)
+        lib.bitlinear_TernaSpMM_packed(vp(xqd), vp(packed), vp(out), vp(sd), vp(wsd), 1, m, n, k, 9, _stream())
+        torch.cuda.synchronize()
+        got = buf.cpu().numpy().view(np.uint16)
+        assert (got[shift:shift + m * n].reshape(m, n) == want_i8).all()
+        assert (got[:shift] == 0xFFFF).all() and (got[shift + m * n:] == 0xFFFF).all()
+
+
 def test_spbitlinear_module_reference_and_repacked_agree(lib, coracle):
     """The call-site mirror: SpBitLinear from a reference-format checkpoint dict, with and without
     the load-time repack, against the oracle on the module's own quantised activations."""

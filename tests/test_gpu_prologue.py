@@ -252,13 +252,14 @@ def test_decode_attention(lib, b, h, kv, d, s_max, n, split):
         assert torch.equal(od, od2)                      # merged in split order: the same bits whoever arrives last
 
 
-@pytest.mark.parametrize("b,h,kv,d,s_max,first,t", [(1, 20, 5, 128, 160, 0, 128), (8, 20, 5, 128, 130, 0, 128), (2, 4, 2, 64, 64, 0, 23),
-                                                   (2, 4, 2, 64, 300, 100, 50), (1, 20, 5, 128, 512, 300, 17), (3, 8, 8, 128, 40, 0, 1)])
-def test_prefill_attention(lib, b, h, kv, d, s_max, first, t):
-    """T new tokens per sequence at the slots first .. first + T - 1, each attending over the cache up to its own
-    slot (the prompt pass; with first > 0 a chunk appended to an existing prefix): against attention_one_token row by
-    row, to the tolerance of the single-token kernel.  Slots past the newest token hold NaN bit patterns: nothing
-    beyond a token's own slot may reach its output."""
+PREFILL_ATTENTION_CASES = [(1, 20, 5, 128, 160, 0, 128), (8, 20, 5, 128, 130, 0, 128), (2, 4, 2, 64, 64, 0, 23),
+                           (2, 4, 2, 64, 300, 100, 50), (1, 20, 5, 128, 512, 300, 17), (3, 8, 8, 128, 40, 0, 1),
+                           (1, 16, 2, 128, 200, 90, 70), (2, 8, 2, 64, 150, 0, 150), (1, 16, 2, 64, 96, 3, 40), (2, 3, 3, 64, 70, 0, 33),
+                           (1, 6, 2, 128, 100, 0, 37), (1, 20, 5, 128, 1100, 0, 1090)]
+
+
+def prefill_attention_case(lib, b, h, kv, d, s_max, first, t, check=True):
+    """Runs one case of ternaspmm_prefill_attention, checks it against the oracle and returns the output bits."""
     q = make_bf16_activations(b * h * t, d, 720 + t).reshape(b, h, t, d)
     k = make_bf16_activations(b * kv * s_max, d, 721 + t).reshape(b, kv, s_max, d)
     v = make_bf16_activations(b * kv * s_max, d, 722 + t, outlier_frac=0.01).reshape(b, kv, s_max, d)
@@ -270,11 +271,45 @@ def test_prefill_attention(lib, b, h, kv, d, s_max, first, t):
     print(f"[case] prefill attention b={b} h={h} kv={kv} d={d} S={s_max} first={first} t={t}", flush=True)
     lib.ternaspmm_prefill_attention(_vp(qd), _vp(kd), _vp(vd), _vp(pd), 0, _vp(od), b, t, h, kv, d, s_max, float(d) ** -0.5, None)
     torch.cuda.synchronize()
-    got = O.bf16_bits_to_f32(od.cpu().numpy().view(np.uint16)).reshape(b, t, h, d).astype(np.float64)
-    want = O.attention_new_tokens(q, k, v, pos, float(d) ** -0.5)
-    tol = 2.0 ** -7 * np.abs(want).max(axis=-1, keepdims=True) + 1e-6
-    assert np.isfinite(got).all()
-    assert (np.abs(got - want) <= tol).all(), float((np.abs(got - want) / tol).max())
+    bits = od.cpu().numpy().view(np.uint16)
+    if check:
+        got = O.bf16_bits_to_f32(bits).reshape(b, t, h, d).astype(np.float64)
+        want = O.attention_new_tokens(q, k, v, pos, float(d) ** -0.5)
+        tol = 2.0 ** -7 * np.abs(want).max(axis=-1, keepdims=True) + 1e-6
+        assert np.isfinite(got).all()
+        assert (np.abs(got - want) <= tol).all(), float((np.abs(got - want) / tol).max())
+    return bits
+
+
+@pytest.mark.parametrize("b,h,kv,d,s_max,first,t", PREFILL_ATTENTION_CASES)
+def test_prefill_attention(lib, b, h, kv, d, s_max, first, t):
+    """T new tokens per sequence at the slots first .. first + T - 1, each attending over the cache up to its own
+    slot (the prompt pass; with first > 0 a chunk appended to an existing prefix): against attention_one_token row by
+    row, to the tolerance of the single-token kernel.  Slots past the newest token hold NaN bit patterns: nothing
+    beyond a token's own slot may reach its output.  The cases cover 1, 2, 4 and 8 query heads per kv head (one
+    workgroup per kv head), 3 (one wave per head), both head sizes, ragged last query blocks and a prefix of more than
+    a thousand slots."""
+    prefill_attention_case(lib, b, h, kv, d, s_max, first, t)
+
+
+def test_prefill_attention_kernels_give_the_same_bits(lib):
+    """The grouped kernel (query heads of a kv head in one workgroup, keys / values through LDS) against the one-wave
+    kernel, which a child process selects through the tuning override: same arithmetic in the same order, so the
+    outputs must agree bit for bit."""
+    import hashlib
+    import os
+    import subprocess
+    import sys
+    cases = [c for c in PREFILL_ATTENTION_CASES if c[1] // c[2] in (1, 2, 4, 8)][:8]
+    mine = [hashlib.sha1(prefill_attention_case(lib, *c, check=False).tobytes()).hexdigest() for c in cases]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = ("import hashlib\nfrom ternainfer_amd import _lib\nfrom tests import test_gpu_prologue as P\nlib = _lib.load()\n"
+            f"for c in {cases!r}:\n    print('bits', hashlib.sha1(P.prefill_attention_case(lib, *c, check=False).tobytes()).hexdigest(), flush=True)\n")
+    r = subprocess.run([sys.executable, "-u", "-c", code], cwd=root, capture_output=True, text=True, timeout=300,
+                       env={**os.environ, "TERNASPMM_TUNING": "1", "TERNASPMM_PREFILL_ATTN_GROUP": "0"})
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    theirs = [line.split()[1] for line in r.stdout.splitlines() if line.startswith("bits ")]
+    assert theirs == mine, (theirs, mine)
 
 
 def _attn_workspace(lib, b, h, d):
