@@ -240,13 +240,14 @@ def measure_model(torch, batch, act="int8", prefetch=True, gen_tokens=256, check
 
 def run_model(args, torch):
     act = args.act or "int8"
-    fig, _ = measure_model(torch, args.batch, act, not args.no_prefetch)
+    gen = 256 if args.prompt_tokens <= 128 else 128
+    fig, _ = measure_model(torch, args.batch, act, not args.no_prefetch, gen_tokens=gen, prompt_tokens=args.prompt_tokens)
     return {
-        "metric": "2B-shape decode tok/s", "value": fig["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": 256, "warmup": 8,
+        "metric": "2B-shape decode tok/s", "value": fig["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": gen, "warmup": 8,
         "ms_per_step": fig["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": act, "data": "synthetic",
         "config": {"workload": f"configs[4]: BitNet-b1.58-2B-shaped random-init decoder (30 layers, hidden 2560, 20/5 heads, "
-                               f"FFN 6912, vocab 128256), batch {args.batch}, 128-token prompt, 256 greedy tokens, "
+                               f"FFN 6912, vocab 128256), batch {args.batch}, {args.prompt_tokens}-token prompt, {gen} greedy tokens, "
                                f"{act} activations into the ternary linears, weights in P2 layout, one HIP graph per "
                                "decode step; norms, gate, activation quantisation, RoPE, cache write, single-token "
                                "attention, the multi-token attention of the prompt pass, the bf16 LM head and greedy "
@@ -586,6 +587,9 @@ def main():
                          "decoder, 128-token prompt + 256 greedy tokens; sweep: the sparsity / structure sweep at M=16; "
                          "midm: both kernel families at the batch sizes between decode and prefill")
     ap.add_argument("--batch", type=int, default=1, help="sequences decoded together (model workload)")
+    ap.add_argument("--prompt-tokens", type=int, default=128,
+                    help="prompt length of the model workload (configs[4]: 128, then 256 generated tokens; longer prompts: 128 "
+                         "generated tokens; the attention kernels take caches of up to 8192 slots)")
     ap.add_argument("--act", choices=["int8", "bf16"], default=None,
                     help="activations into the ternary linears: int8 + per-row scale (the reference's SpBitLinear; "
                          "default of the model workload) or bf16 (default of the prefill workload)")
