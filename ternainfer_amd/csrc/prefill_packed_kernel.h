@@ -183,24 +183,41 @@ __device__ __forceinline__ void packed_prefill_epilogue(AccV (&acc)[NA][MB], uin
 }
 
 // Raw accumulators of one wave into a [M][N] plane of split-K partial sums (same element order as the epilogue).
+// `tile`: 4 KiB of LDS of this wave's own.  One 32 x 32 accumulator tile at a time goes through it and leaves as whole
+// rows of 128 bytes (16 bytes per lane, 8 consecutive lanes per row), for the reason given at OutTile; the plane's rows
+// are 16-byte aligned whenever split-K runs (N is a multiple of 4 and the scratch memory is aligned).  Piece p (16 bytes)
+// of row r sits at position p ^ ((r >> 1) & 7): writes and reads are bank-conflict free.
+constexpr int kPartialTileBytes = 32 * 128;
 template <int MB, int NA, typename AccV, typename AccT>
 __device__ __forceinline__ void packed_prefill_store_partial(AccV (&acc)[NA][MB], AccT* __restrict__ plane, int M, int N,
-                                                             int n_wave, int m0, int lane)
+                                                             int n_wave, int m0, int lane, uint8_t* tile)
 {
     typedef AccT V4 __attribute__((ext_vector_type(4)));
+    static_assert(sizeof(AccT) == 4, "partial sums are 32-bit");
     const int kb = lane >> 5, l32 = lane & 31;
+    const int put = l32 * 128, put_swz = (l32 >> 1) & 7;
+    const int piece = lane & 7;
     static_for<0, NA>([&](auto ac) {
         constexpr int a = decltype(ac)::value;
         static_for<0, MB>([&](auto bc) {
             constexpr int b = decltype(bc)::value;
-            const int m = m0 + 32 * b + l32;
             static_for<0, 4>([&](auto vc) {
-                constexpr int vq = decltype(vc)::value;
-                const int n = n_wave + 32 * a + 8 * vq + 4 * kb;
-                if (m < M && n < N)
-                    *reinterpret_cast<V4*>(plane + static_cast<size_t>(m) * N + n) =
-                        V4{acc[a][b][4 * vq], acc[a][b][4 * vq + 1], acc[a][b][4 * vq + 2], acc[a][b][4 * vq + 3]};
+                constexpr int vq = decltype(vc)::value;          // features 8 vq + 4 kb .. +3 of row l32: piece 2 vq + kb
+                *reinterpret_cast<V4*>(tile + put + (((2 * vq + kb) ^ put_swz) << 4)) =
+                    V4{acc[a][b][4 * vq], acc[a][b][4 * vq + 1], acc[a][b][4 * vq + 2], acc[a][b][4 * vq + 3]};
             });
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            const int n = n_wave + 32 * a + 4 * piece;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int row = 8 * i + (lane >> 3);
+                const V4 v = *reinterpret_cast<const V4*>(tile + row * 128 + ((piece ^ ((row >> 1) & 7)) << 4));
+                const int m = m0 + 32 * b + row;
+                if (m < M && n < N) __builtin_nontemporal_store(v, reinterpret_cast<V4*>(plane + static_cast<size_t>(m) * N + n));
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
         });
     });
 }
@@ -610,17 +627,18 @@ __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) voi
     }
     if (k < k_end) body(k, w0);
 
+    // Results (or split-K partial sums) leave as whole rows through a per-wave LDS tile; the tiles take the place of the
+    // activation stages once every wave is done reading those.
+    static_assert(4 * OutTile<NA>::kBytes <= S::kBytes && 4 * kPartialTileBytes <= S::kBytes, "output tiles fit in the activation stages");
+    __syncthreads();
     if (partial != nullptr) {
         using AccT = typename std::conditional<I8, int, float>::type;
         packed_prefill_store_partial<MB, NA>(acc, static_cast<AccT*>(partial) + static_cast<size_t>(blockIdx.z) * M * N, M, N,
-                                             n0 + 32 * NA * wave, m0, lane);
+                                             n0 + 32 * NA * wave, m0, lane, smem + wave * kPartialTileBytes);
         return;
     }
-    // results leave as whole rows through a per-wave LDS tile whenever 16-byte stores can address the output; the tiles
-    // take the place of the activation stages once every wave is done reading those
-    static_assert(4 * OutTile<NA>::kBytes <= S::kBytes, "output tiles fit in the activation stages");
+    // ... for the final results whenever 16-byte stores can address the output
     const bool rows_ok = ((reinterpret_cast<uintptr_t>(out) | (static_cast<uintptr_t>(N) * 2)) & 15) == 0;
-    __syncthreads();
     packed_prefill_epilogue<MB, NA>(acc, out, ep, M, N, n0 + 32 * NA * wave, m0, lane,
                                     rows_ok ? smem + wave * OutTile<NA>::kBytes : nullptr);
 }
