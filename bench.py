@@ -17,7 +17,8 @@ layer of the same workload and doubles as the correctness gate of the run.
 
 The default run (`--workload decode`) also measures, in the same process and into the same line,
 the other figures the path is judged on: the literal single-matrix configuration (`config1`),
-the layer set at M = 1 and 16, the unmodified call site (`drop_in_reference_format`), the prefill
+the layer set at M = 1 and 16, the same launches without the dependence between them (`launches_overlapped`,
+evidence only), the unmodified call site (`drop_in_reference_format`), the prefill
 shapes at M = 2048 for both activation types (`prefill_m2048`), the 2B-shaped model's decode
 tokens/s at batch 1 and 8 and, for one sequence, far into a 2048-slot context (`model_decode`) and what the machine gives (`calibration`: cost of a
 graph kernel node, read and copy rate, cost of a device-wide synchronisation).  `--no-extras`
@@ -555,6 +556,30 @@ def layer_set_step(torch, lib, mats, layers, layout, m, steps, warmup):
     return ev0.elapsed_time(ev1) / steps
 
 
+def overlapped_layer_set(torch, lib, mats, layers, layout, m, steps, warmup):
+    """The launches of the layer-set step with the dependence between them taken away: one stream per matrix shape inside
+    the captured graph (fork at the start of a step, join at its end), every stream running its 30 launches back to back.
+    A decoder cannot run like this -- each of its launches consumes the previous one's output -- so this is no throughput
+    figure of the path; it shows what the same kernels on the same bytes reach once the per-launch latency chains
+    overlap, i.e. how much of the distance to the HBM roofline is launch latency and how much is the kernels."""
+    side = torch.cuda.Stream()
+    branches = [torch.cuda.Stream() for _ in mats]
+    side.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            for br, mt in zip(branches, mats):
+                br.wait_stream(side)
+                with torch.cuda.stream(br):
+                    handle = ctypes.c_void_p(br.cuda_stream)
+                    for layer in range(layers):
+                        mt.launch(lib, layer, handle, layout, m)
+            for br in branches:
+                side.wait_stream(br)
+    torch.cuda.current_stream().wait_stream(side)
+    return time_graph(torch, g, steps, warmup)
+
+
 def config1_row(torch, T, lib, copies=400):
     """The literal single-matrix configuration: M = 8, K = N = 2560, P(0) = 0.45, one fp32 scale; cold = `copies`
     rotating weight copies (more than twice the last-level cache), hot = one copy."""
@@ -711,6 +736,11 @@ def main():
             by_m[str(m)] = {"ms_per_step": ms, "GBps": b / (ms * 1e-3) / 1e9, "frac": b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                             "algorithmic_bytes_per_step": b}
         result["layer_set_by_m"] = by_m
+        ms = overlapped_layer_set(torch, lib, mats, args.layers, args.layout, args.m, half, 2)
+        result["launches_overlapped"] = as_figures(
+            ms, "NOT a figure of the path: the same launches with the dependence between them removed (one stream per matrix shape "
+                "inside the graph, four chains of 30 launches side by side) -- what the kernels reach on these bytes when the "
+                "per-launch latency chains overlap; a decoder's launches depend on each other and cannot run like this")
         del mats
         torch.cuda.empty_cache()
         result["config1"] = config1_row(torch, T, lib)
