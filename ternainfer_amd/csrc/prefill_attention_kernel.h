@@ -199,8 +199,9 @@ __global__ __launch_bounds__(64) void terna_prefill_attention_kernel(
 // ------------------------------------------------------------------------------------------------
 // The same computation with the query heads of a kv head in one workgroup (grouped-query attention: H / KV = G heads
 // read the same keys and values).  Wave w is head kvh * G + w over the same block of 16 queries; a block of 32 cache
-// slots is fetched ONCE per workgroup, coalesced (16 bytes per lane, consecutive lanes on consecutive addresses),
-// three blocks ahead of the one being multiplied, and shared through LDS (two buffers, one barrier per block):
+// slots (64 with four or more heads per workgroup: two softmax steps per block) is fetched ONCE per workgroup,
+// coalesced (16 bytes per lane, consecutive lanes on consecutive addresses), two blocks ahead of the one being
+// multiplied, and shared through LDS (two buffers, one barrier per block):
 //   * rows of a tile are 2 D + 16 bytes apart, so that the 16 rows a 16-byte operand read of the first product
 //     touches (A = 16 keys x 32 dims) fall into different banks, and every operand address of a round is one
 //     per-lane base plus a constant;
@@ -238,12 +239,14 @@ __global__ __launch_bounds__(64 * G) void terna_prefill_attention_group_kernel(
     static_assert(G == 1 || G == 2 || G == 4 || G == 8, "query heads per kv head");
     constexpr int DS = D / 32;                 // 32-dimension slices of a row (first product)
     constexpr int DT = D / 16;                 // 16-dimension tiles of the output (second product)
-    constexpr int KB = kPrefillAttnKeys;       // cache slots per block
+    constexpr int KB = kPrefillAttnKeys;       // cache slots per softmax step (as in the one-wave kernel)
+    constexpr int SUB = G >= 4 ? 2 : 1;        // softmax steps per round: fetch, move to LDS and barrier once per LB slots
+    constexpr int LB = SUB * KB;               // cache slots per block in LDS
     constexpr int ROW = 2 * D;                 // bytes of a key / value row in the cache
     constexpr int PITCH = ROW + 16;            // ... and in LDS
     constexpr int PPR = D / 8;                 // 16-byte pieces per row
-    constexpr int TILE = KB * PITCH;           // bytes of a key (or value) tile in LDS
-    constexpr int PIECES = 2 * KB * PPR;       // pieces of a block: keys, then values
+    constexpr int TILE = LB * PITCH;           // bytes of a key (or value) tile in LDS
+    constexpr int PIECES = 2 * LB * PPR;       // pieces of a block: keys, then values
     constexpr int PT = PIECES / (64 * G);      // pieces per thread
     static_assert(PIECES % (64 * G) == 0 && PT >= 1, "a block divides over the workgroup");
     __shared__ __align__(16) uint8_t tiles[2][2 * TILE];
@@ -282,7 +285,7 @@ __global__ __launch_bounds__(64 * G) void terna_prefill_attention_group_kernel(
 #pragma unroll
     for (int u = 0; u < PT; ++u) {
         const int idx = tid + 64 * G * u;
-        const int which = __builtin_amdgcn_readfirstlane(idx / (KB * PPR)), rem = idx % (KB * PPR);
+        const int which = __builtin_amdgcn_readfirstlane(idx / (LB * PPR)), rem = idx % (LB * PPR);
         const int row = rem / PPR, piece = rem % PPR;
         pc_row[u] = row;
         pc_val[u] = which != 0;
@@ -291,16 +294,16 @@ __global__ __launch_bounds__(64 * G) void terna_prefill_attention_group_kernel(
         pc_off[u] = row * ROW + piece * 16;
         pc_lds[u] = which * TILE + row * PITCH + piece * 16;
     }
-    // Blocks travel global memory -> registers -> LDS; a block is requested three rounds before it is multiplied (a
-    // round is far shorter than a trip to memory) and moved into the free LDS buffer one round before.  The requests are
-    // issued and awaited by hand: the load counter is in order, so "the block requested two rounds ago has landed" is
-    // one s_waitcnt vmcnt(n) with n = the loads issued since -- written as ordinary loads, the compiler waits for
+    // Blocks travel global memory -> registers -> LDS; a block is requested two rounds before it is multiplied (one
+    // round is shorter than a trip to memory) and moved into the free LDS buffer one round before.  The requests are
+    // issued and awaited by hand: the load counter is in order, so "the block requested in the previous round has landed"
+    // is one s_waitcnt vmcnt(n) with n = the loads issued since -- written as ordinary loads, the compiler waits for
     // everything at every round.
     struct Stage { u32x4 v[PT]; };
     // the block's first row goes into the (scalar) base address, so that a whole block costs no address arithmetic per
     // lane; only the last block of a prefix can reach past it, and there the row is pulled back in range
     auto fetch = [&](int k0, Stage& st) {
-        if (k0 + KB <= n_keys) {                   // uniform
+        if (k0 + LB <= n_keys) {                   // uniform
 #pragma unroll
             for (int u = 0; u < PT; ++u) attn_load_b128_nowait(st.v[u], pc_base[u] + static_cast<size_t>(k0) * D, pc_off[u]);
         } else {
@@ -313,14 +316,13 @@ __global__ __launch_bounds__(64 * G) void terna_prefill_attention_group_kernel(
     };
     // Value slots past the block's largest prefix were never written (they may hold anything, NaN included, and 0 * NaN
     // would poison the product): the in-range row read in their place is zeroed.  Keys only need to be in range: their
-    // scores are masked.  `younger`: how many fetch() calls were issued after the one that filled `st` (0, 1 or 2).
-    auto commit = [&](Stage& st, int k0, int buf, int younger) {
-        if (younger == 2) attn_wait_loads<2 * PT>();
-        else if (younger == 1) attn_wait_loads<PT>();
+    // scores are masked.  `younger`: whether a fetch() was issued after the one that filled `st`.
+    auto commit = [&](Stage& st, int k0, int buf, bool younger) {
+        if (younger) attn_wait_loads<PT>();
         else attn_wait_loads<0>();
 #pragma unroll
         for (int u = 0; u < PT; ++u) attn_landed(st.v[u]);
-        if (k0 + KB <= n_keys) {                   // uniform
+        if (k0 + LB <= n_keys) {                   // uniform
 #pragma unroll
             for (int u = 0; u < PT; ++u) *reinterpret_cast<u32x4*>(&tiles[buf][pc_lds[u]]) = st.v[u];
         } else {
@@ -349,18 +351,17 @@ __global__ __launch_bounds__(64 * G) void terna_prefill_attention_group_kernel(
     // loop would count those requests as its own and drain them every time round
 #pragma unroll
     for (int ds = 0; ds < DS; ++ds) asm volatile("" : "+v"(bq[ds]));
-    Stage st0, st1, st2;
+    Stage st0, st1;
     fetch(0, st0);
-    if (KB < n_keys) fetch(KB, st1);
-    if (2 * KB < n_keys) fetch(2 * KB, st2);
-    commit(st0, 0, 0, (KB < n_keys) + (2 * KB < n_keys));
+    if (LB < n_keys) fetch(LB, st1);
+    commit(st0, 0, 0, LB < n_keys);
     __syncthreads();
     int buf = 0;
 
-    // the block at k0 out of LDS buffer `buf`; MASKED: some query of the workgroup does not see all of it
-    auto multiply = [&](int k0, auto masked) {
+    // the KB slots at k0, which start at `tile` in the key tile of the current LDS buffer; MASKED: some query of the
+    // workgroup does not see all of them
+    auto multiply = [&](int k0, const uint8_t* tile, auto masked) {
         constexpr bool MASKED = decltype(masked)::value;
-        const uint8_t* tile = tiles[buf];
         // ---- scores, transposed: lane = (query qi, keys 4g + v of tile j)
         f32x4 s[2];
 #pragma unroll
@@ -422,26 +423,29 @@ __global__ __launch_bounds__(64 * G) void terna_prefill_attention_group_kernel(
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, bp_lo, o[dt], 0, 0, 0);
         }
     };
-    // one round: the block at k0 is multiplied; `refill` (whose block is in LDS already) takes the block three ahead,
-    // `next` (requested two rounds ago) goes into the other buffer, which every wave stopped reading before the barrier
-    // that ended the previous round.  All conditions are uniform over the workgroup.
+    // one round: the block at k0 is multiplied, KB slots at a time; `refill` (whose block is in LDS already) takes the
+    // block two ahead, `next` (requested in the previous round) goes into the other buffer, which every wave stopped
+    // reading before the barrier that ended the previous round.  All conditions are uniform over the workgroup.
     auto round = [&](int k0, Stage& refill, Stage& next) {
-        if (k0 + 3 * KB < n_keys) fetch(k0 + 3 * KB, refill);
-        if (k0 + KB <= n_full) multiply(k0, std::false_type{});
-        else multiply(k0, std::true_type{});
-        if (k0 + KB < n_keys) commit(next, k0 + KB, buf ^ 1, (k0 + 2 * KB < n_keys) + (k0 + 3 * KB < n_keys));
+        if (k0 + 2 * LB < n_keys) fetch(k0 + 2 * LB, refill);
+#pragma unroll
+        for (int sub = 0; sub < SUB; ++sub) {
+            const int ks = k0 + sub * KB;
+            if (sub > 0 && ks >= n_keys) break;
+            const uint8_t* tile = tiles[buf] + sub * KB * PITCH;
+            if (ks + KB <= n_full) multiply(ks, tile, std::false_type{});
+            else multiply(ks, tile, std::true_type{});
+        }
+        if (k0 + LB < n_keys) commit(next, k0 + LB, buf ^ 1, k0 + 2 * LB < n_keys);
         __syncthreads();
         buf ^= 1;
     };
     for (int k0 = 0; k0 < n_keys;) {
         round(k0, st0, st1);
-        k0 += KB;
+        k0 += LB;
         if (k0 >= n_keys) break;
-        round(k0, st1, st2);
-        k0 += KB;
-        if (k0 >= n_keys) break;
-        round(k0, st2, st0);
-        k0 += KB;
+        round(k0, st1, st0);
+        k0 += LB;
     }
 
     l_run = key_groups_reduce<false>(l_run);
