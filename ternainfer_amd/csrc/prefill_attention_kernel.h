@@ -213,8 +213,8 @@ __global__ __launch_bounds__(64) void terna_prefill_attention_kernel(
 //     reads (one per 16-key score tile) are the eight keys of the operand, in the position order the probabilities
 //     already have.  The one-wave kernel above gathers the same operand with eight 2-byte reads.
 //   * blocks that every query of the workgroup sees whole run without the causal compares; the running output is
-//     rescaled only in rounds where some lane's maximum moved (x 1.0 changes nothing, and the accumulators would have
-//     to leave the matrix core's registers for it).
+//     rescaled only in rounds where some lane's maximum moved (x 1.0 changes nothing: 32 multiplications saved in
+//     most rounds once the maxima have settled).
 // Arithmetic, order of the sums and therefore the bits of the result are those of the one-wave kernel.
 // Workgroups are numbered from the last query block down: under a causal mask those have the most keys to walk.
 typedef short s16x4 __attribute__((ext_vector_type(4)));
