@@ -12,6 +12,10 @@
  *     fully overwritten; nothing is allocated, freed or synchronised on the call path;
  *   - W is [N][K] ternary in the compressed format (bitmap / TileOffsets_global /
  *     TileOffsets_median / sign words), N % 64 == 0 and K % 64 == 0;
+ *   - alignment: `out` at least 8 bytes (the kernels store four bf16 at a time); x, the scales and the format's
+ *     arrays as their element types require.  16-byte aligned x and out (any torch / hipMalloc allocation) select
+ *     the faster variants of the large-M kernels -- activations loaded straight into LDS, results stored as whole
+ *     rows -- other pointers take slower variants with the same results;
  *   - calls only enqueue work on `stream` and are safe under stream capture;
  *   - on a HIP runtime error the library prints the error and exits the process, as the
  *     reference does (kernels/TernaSpMM.cu:15-22).
