@@ -15,7 +15,7 @@
  *   - alignment: `out` at least 8 bytes (the kernels store four bf16 at a time); x, the scales and the format's
  *     arrays as their element types require.  16-byte aligned x and out (any torch / hipMalloc allocation) select
  *     the faster variants of the large-M kernels -- activations loaded straight into LDS, results stored as whole
- *     rows -- other pointers take slower variants with the same results;
+ *     rows -- other pointers take slower variants (same bits for the int8 family, same tolerance for bf16);
  *   - calls only enqueue work on `stream` and are safe under stream capture;
  *   - on a HIP runtime error the library prints the error and exits the process, as the
  *     reference does (kernels/TernaSpMM.cu:15-22).
