@@ -318,9 +318,13 @@ int ternaspmm_attention_partial_splits(int B, int H, int S)
     // of the partial results reads splits x the bytes of a merged row (measured on the 2B shapes, one sequence: four splits
     // cost the O projection 0.9 us, eight 1.7 us): four splits up to 1024 slots, eight beyond, fewer when the
     // (sequence, head, split) workgroups would not fit the chip or a split would get less than two tiles.
+    // Long caches of several sequences (more heads than the chip has CUs): an unsplit workgroup walks up to S slots alone
+    // while a split costs a merge pass, so split there as well, up to about four workgroups per CU (measured, 8 sequences
+    // of the 2B shape at slot 1500 of 2048: unsplit 25.5 us, four splits 18.2 us + 2.2 us for the merge launch).
     const int want = S > 1024 ? kAttentionMaxSplits : 4;
+    const long fill = S > 1024 ? 1024 : 256;
     int sp = 1;
-    while (sp < want && static_cast<long>(B) * H * sp * 2 <= 256 && 32 * sp * 2 <= S) sp *= 2;
+    while (sp < want && static_cast<long>(B) * H * sp * 2 <= fill && 32 * sp * 2 <= S) sp *= 2;
     return sp;
 }
 

@@ -177,20 +177,26 @@ def rmsnorm_linear_packed(x, norm_weight, eps, packed, ws, ws_num, out_features,
     return TernaInfer_linear_packed(xq, packed, s, ws, ws_num, out_features), h
 
 
-def attention_merge_rmsnorm_linear_packed(partial, splits, heads, head_dim, norm_weight, eps, packed, ws, ws_num, out_features):
-    """The O projection of a single-sequence decode step fed by the partial results of a split attention launch
-    (ternaspmm_rope_decode_attention_partial): merge -> RMSNorm -> quant_input -> int8 TernaSpMM in one launch where the
-    library supports the shape, else ternaspmm_attention_merge + rmsnorm_linear_packed (the same bits).
-    partial: fp32 device buffer; returns out bf16 [1, out_features]."""
+def attention_merge_rmsnorm_linear_packed(partial, splits, heads, head_dim, norm_weight, eps, packed, ws, ws_num, out_features,
+                                          sequences=1):
+    """The O projection of a decode step fed by the partial results of a split attention launch
+    (ternaspmm_rope_decode_attention_partial over `sequences` sequences): for one sequence merge -> RMSNorm -> quant_input
+    -> int8 TernaSpMM in one launch where the library supports the shape, else ternaspmm_attention_merge +
+    rmsnorm_linear_packed (the same bits).  partial: fp32 device buffer of ternaspmm_attention_partial_bytes(sequences, ...);
+    returns out bf16 [sequences, out_features]."""
     lib = _lib.load()
     k = heads * head_dim
-    out = torch.empty((1, out_features), dtype=torch.bfloat16, device=partial.device)
+    need = lib.ternaspmm_attention_partial_bytes(sequences, heads, head_dim)
+    if sequences < 1 or need < 0 or partial.numel() * partial.element_size() < need:
+        raise ValueError(f"partial buffer of {partial.numel() * partial.element_size()} bytes does not hold {sequences} sequences")
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    if lib.bitlinear_TernaSpMM_packed_fused_attn(_p(partial), splits, head_dim, _p(norm_weight), float(eps), _p(packed), _p(out),
-                                                 _p(ws), ws_num, None, None, 1, out_features, k, stream):
-        return out
-    o = torch.empty((1, k), dtype=torch.bfloat16, device=partial.device)
-    lib.ternaspmm_attention_merge(_p(partial), splits, _p(o), 1, heads, head_dim, stream)
+    if sequences == 1:
+        out = torch.empty((1, out_features), dtype=torch.bfloat16, device=partial.device)
+        if lib.bitlinear_TernaSpMM_packed_fused_attn(_p(partial), splits, head_dim, _p(norm_weight), float(eps), _p(packed), _p(out),
+                                                     _p(ws), ws_num, None, None, 1, out_features, k, stream):
+            return out
+    o = torch.empty((sequences, k), dtype=torch.bfloat16, device=partial.device)
+    lib.ternaspmm_attention_merge(_p(partial), splits, _p(o), sequences, heads, head_dim, stream)
     return rmsnorm_linear_packed(o, norm_weight, eps, packed, ws, ws_num, out_features)[0]
 
 

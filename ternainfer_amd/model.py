@@ -201,8 +201,8 @@ class Block:
         one_token = mask is None           # the caller's rule: fused, one new token, a head size the kernel has
         deferred = one_token and isinstance(attn_ws, tuple)
         if deferred:
-            # one sequence: the cache prefix of every head split over several workgroups that leave partial results;
-            # the O projection's prologue merges them (the launch boundary is the synchronisation)
+            # the cache prefix of every head split over several workgroups that leave partial results; the O
+            # projection's prologue merges them (one sequence; else a merge launch): the launch boundary is the synchronisation
             lib = self.wqkv.lib
             stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
             # (no prefetch regions here: this launch is shorter than the prefetch of the following weights would be --
@@ -262,7 +262,8 @@ class Block:
             o = o.transpose(1, 2).reshape(bsz * t, a.n_heads * a.head_dim)
         if deferred:
             attn = attention_merge_rmsnorm_linear_packed(partial, splits, a.n_heads, a.head_dim, self.attn_sub_norm, a.norm_eps,
-                                                         self.wo.packed, self.wo.ws, self.wo.ws_num, self.wo.n)
+                                                         self.wo.packed, self.wo.ws, self.wo.ws_num, self.wo.n, sequences=bsz)
+            assert attn.shape[0] == bsz
         else:
             attn, _ = self._norm_linear(self.wo, o.contiguous(), self.attn_sub_norm)
         x13, x = self._norm_linear(self.w13, x, self.ffn_norm, residual=attn)
@@ -355,21 +356,22 @@ class Transformer:
             self._rope_tables = tables = (key, torch.stack([ang.cos(), ang.sin()], dim=1).contiguous())
         return tables[1]
 
-    def attention_partial(self, max_seq: int):
-        """(buffer, splits) for the single-sequence decode step whose attention leaves the merge of its splits to the O
-        projection, or None when that form does not apply (one split recommended; `deferred_attention_merge` False)."""
+    def attention_partial(self, bsz: int, max_seq: int):
+        """(buffer, splits) for the decode step whose attention leaves the merge of its splits to the consumer of its
+        output (one sequence: the O projection's prologue; more: a merge launch), or None when that form does not apply
+        (one split recommended; `deferred_attention_merge` False)."""
         if not getattr(self, "deferred_attention_merge", True):
             return None
         a = self.args
         lib = _lib.load()
-        splits = getattr(self, "attention_splits", None) or lib.ternaspmm_attention_partial_splits(1, a.n_heads, max_seq)
+        splits = getattr(self, "attention_splits", None) or lib.ternaspmm_attention_partial_splits(bsz, a.n_heads, max_seq)
         if splits <= 1:
             return None
-        buf = getattr(self, "_attn_partial", None)
-        if buf is None:
-            nbytes = lib.ternaspmm_attention_partial_bytes(1, a.n_heads, a.head_dim)
-            self._attn_partial = buf = torch.empty(nbytes // 4, dtype=torch.float32, device="cuda")
-        return buf, splits
+        held = getattr(self, "_attn_partial", None)
+        if held is None or held[0] != bsz:
+            nbytes = lib.ternaspmm_attention_partial_bytes(bsz, a.n_heads, a.head_dim)
+            self._attn_partial = held = (bsz, torch.empty(nbytes // 4, dtype=torch.float32, device="cuda"))
+        return held[1], splits
 
     def attention_workspace(self, bsz: int):
         """Zero-filled scratch of the single-token attention (split over the cache); one per batch size."""
@@ -411,8 +413,11 @@ class Transformer:
         x = self.tok_embeddings[tokens.reshape(-1)]
         pending = None
         attn_ws = self.attention_workspace(bsz) if one_launch_attention else None     # layers run one after another: shared
-        if one_launch_attention and bsz == 1 and self.layers[0].act == "int8":
-            attn_ws = self.attention_partial(max_seq) or attn_ws
+        # split attention whose merge is left to its consumer: always for one sequence (the O projection's prologue merges);
+        # for more only with long caches, where the shorter attention launch pays for the merge launch (8 sequences at slot
+        # 1500: 1943 -> 1713 us per step; at slot 255 of 384 the pair of launches is 1.5 us slower than the unsplit one)
+        if one_launch_attention and self.layers[0].act == "int8" and (bsz == 1 or max_seq > 1024):
+            attn_ws = self.attention_partial(bsz, max_seq) or attn_ws
         for index, (layer, (ck, cv)) in enumerate(zip(self.layers, cache)):
             x_in, pending_in = x, pending
             x, pending = layer.forward(x, pending, ck, cv, pos_idx, cos, sin, mask, attn_ws)

@@ -91,6 +91,8 @@ def test_host_side_size_and_policy_functions():
     assert lib.ternaspmm_attention_partial_splits(1, 20, 384) == 4       # up to 1024 slots: four splits
     assert lib.ternaspmm_attention_partial_splits(1, 20, 4096) == 8      # beyond: eight
     assert lib.ternaspmm_attention_partial_splits(8, 20, 384) == 1       # the heads fill the chip anyway
+    assert lib.ternaspmm_attention_partial_splits(8, 20, 2048) == 4      # ... but a long cache is split all the same
+    assert lib.ternaspmm_attention_partial_splits(64, 20, 2048) == 1     # up to about eight workgroups per CU
     assert lib.ternaspmm_attention_partial_splits(1, 20, 32) == 1        # a split must keep two tiles
     assert lib.ternaspmm_attention_partial_splits(1, 20, 64) == 2
     assert lib.ternaspmm_attention_partial_splits(1, 20, 128) == 4

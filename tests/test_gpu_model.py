@@ -164,6 +164,35 @@ def test_toy_model_attention_merge_deferred_to_the_o_projection(head_dim, splits
     assert torch.equal(a, c)
 
 
+def test_toy_model_several_sequences_long_cache_deferred_merge():
+    """Several sequences with a cache of more than 1024 slots: the harness splits the single-token attention and leaves
+    the merge to a launch of its own in front of the O projection (ternaspmm_attention_merge).  Logits against the step
+    with the attention in one piece; greedy tokens of a replayed graph against eager execution; every row of the batch
+    must come out (the O projection sees one row per sequence)."""
+    from ternainfer_amd.model import ModelArgs, Transformer, greedy_decode
+    args = ModelArgs(dim=512, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=1024, ffn_dim=384)
+    model = Transformer(args, seed=43, act="int8")
+    bsz, plen, cache_slots = 3, 1040, 1100
+    prompt = torch.randint(0, args.vocab_size, (bsz, plen), generator=torch.Generator().manual_seed(44)).cuda()
+    print("[case] toy model, 3 sequences, 1100-slot cache, deferred attention merge", flush=True)
+    assert model.attention_partial(bsz, cache_slots) is not None          # the path under test is the one that runs
+    outs = []
+    with torch.inference_mode():
+        for deferred in (True, False):
+            model.deferred_attention_merge = deferred
+            cache = model.make_cache(bsz, cache_slots)
+            model.forward(prompt, cache, torch.arange(plen, device="cuda"))
+            outs.append(model.forward(prompt[:, -1:].contiguous(), cache, torch.tensor([plen], device="cuda")).float())
+    assert outs[0].shape == outs[1].shape and outs[0].shape[0] == bsz
+    err = (outs[0] - outs[1]).abs().max().item()
+    assert err <= 3e-2 * outs[1].abs().max().item(), err
+    assert torch.nn.functional.cosine_similarity(outs[0].flatten(), outs[1].flatten(), dim=0).item() > 0.9995
+    model.deferred_attention_merge = True
+    a, _, _ = greedy_decode(model, prompt, 70, use_graph=True)            # plen + 70 > 1024 slots
+    b, _, _ = greedy_decode(model, prompt, 70, use_graph=False)
+    assert torch.equal(a, b)
+
+
 def test_toy_model_prompt_pass_kernel_attention_sdpa_and_graph_replays():
     """The prompt pass through the library's multi-token attention against the same pass through PyTorch's SDPA, and
     the captured prompt graph against eager execution on several replays with eager work and synchronisations between
