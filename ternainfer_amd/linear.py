@@ -106,6 +106,16 @@ def repack_weight(compressed_val, TileOffsets_global, TileOffsets_median, bitmap
     return packed
 
 
+def _check_rows(who, x, k=None, **others):
+    """The kernels take pointers and sizes on trust: a tensor with the wrong number of elements would be read or written
+    past its end on the GPU.  Raise here instead."""
+    if x.dim() != 2 or (k is not None and x.shape[1] != k):
+        raise ValueError(f"{who}: expected a [M, {k if k is not None else 'K'}] tensor, got {tuple(x.shape)}")
+    for name, (t, numel) in others.items():
+        if t is not None and t.numel() != numel:
+            raise ValueError(f"{who}: {name} has {t.numel()} elements, expected {numel}")
+
+
 def TernaInfer_linear_packed(input, packed, s, ws, ws_num, out_features):
     """int8 activations x P2-layout ternary weight -> bf16; the reference's epilogue rule by M
     (decode arithmetic for M <= 64, prefill arithmetic above).  No row padding needed."""
@@ -115,6 +125,9 @@ def TernaInfer_linear_packed(input, packed, s, ws, ws_num, out_features):
     K = input.shape[-1]
     x = input.reshape(-1, K).contiguous()
     M = x.shape[0]
+    _check_rows("TernaInfer_linear_packed", x, s=(s, M))
+    if packed.numel() * packed.element_size() < out_features * K // 4 or ws.numel() < ws_num:
+        raise ValueError("TernaInfer_linear_packed: packed weight or weight scales too small for this shape")
     out = torch.empty((M, out_features), dtype=torch.bfloat16, device=input.device)
     stream = torch.cuda.current_stream()
     work = get_global_workspace(input.device) if M > 64 else None      # large M: room for split-K partial sums
@@ -130,6 +143,7 @@ def rmsnorm_quant(x, weight, eps, residual=None, quant=True):
     Returns (xq int8 [M, K], s bf16 [M], h) when quant else (y bf16 [M, K], h); h is the bf16 sum
     x + residual (x itself when residual is None)."""
     m, k = x.shape
+    _check_rows("rmsnorm_quant", x, residual=(residual, m * k), weight=(weight, k))
     x = x.contiguous()
     lib = _lib.load()
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -159,6 +173,9 @@ def rmsnorm_linear_packed(x, norm_weight, eps, packed, ws, ws_num, out_features,
     rmsnorm_quant + TernaInfer_linear_packed.
     x, residual: bf16 [M, K].  Returns (out bf16 [M, out_features], h = x + residual)."""
     m, k = x.shape
+    _check_rows("rmsnorm_linear_packed", x, residual=(residual, m * k), norm_weight=(norm_weight, k))
+    if packed.numel() * packed.element_size() < out_features * k // 4 or ws.numel() < ws_num:
+        raise ValueError("rmsnorm_linear_packed: packed weight or weight scales too small for this shape")
     x = x.contiguous()
     lib = _lib.load()
     h = x
@@ -205,6 +222,9 @@ def relu2_mul_rmsnorm_linear_packed(x13, norm_weight, eps, packed, ws, ws_num, o
     rows where the library supports the shape, else relu2_mul_rmsnorm_quant + TernaInfer_linear_packed.
     x13: bf16 [M, 2F].  Returns out bf16 [M, out_features]."""
     m, f2 = x13.shape
+    _check_rows("relu2_mul_rmsnorm_linear_packed", x13, norm_weight=(norm_weight, f2 // 2))
+    if f2 % 2 or packed.numel() * packed.element_size() < out_features * (f2 // 2) // 4 or ws.numel() < ws_num:
+        raise ValueError("relu2_mul_rmsnorm_linear_packed: packed weight or weight scales too small for this shape")
     x13 = x13.contiguous()
     lib = _lib.load()
     out = torch.empty((m, out_features), dtype=torch.bfloat16, device=x13.device)
@@ -221,6 +241,7 @@ def relu2_mul_rmsnorm_quant(x13, weight, eps, quant=True):
     x13: bf16 [M, 2F].  Returns (xq int8 [M, F], s bf16 [M]) when quant else y bf16 [M, F]."""
     m, f2 = x13.shape
     f = f2 // 2
+    _check_rows("relu2_mul_rmsnorm_quant", x13, weight=(weight, f))
     x13 = x13.contiguous()
     lib = _lib.load()
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)

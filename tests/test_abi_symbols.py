@@ -97,3 +97,31 @@ def test_host_side_size_and_policy_functions():
     assert lib.ternaspmm_attention_partial_splits(1, 20, 64) == 2
     assert lib.ternaspmm_attention_partial_splits(1, 20, 128) == 4
     assert lib.ternaspmm_attention_workspace_bytes(1, 20, 128) > 0
+
+
+def test_python_wrappers_refuse_mismatched_tensors_on_the_host():
+    """The library takes pointers and sizes on trust; the Python wrappers check element counts first, so that a
+    tensor with too few rows raises here instead of being read or written past its end on the GPU.  (CPU tensors:
+    the checks run before anything touches a device.)"""
+    import torch
+    from ternainfer_amd import linear as L
+    x = torch.zeros(8, 2560, dtype=torch.bfloat16)
+    one_row = torch.zeros(1, 2560, dtype=torch.bfloat16)
+    w = torch.zeros(2560, dtype=torch.bfloat16)
+    ws = torch.zeros(4, dtype=torch.bfloat16)
+    packed = torch.zeros(2560 * 2560 // 4, dtype=torch.int8)
+    with pytest.raises(ValueError, match="residual"):
+        L.rmsnorm_quant(x, w, 1e-5, residual=one_row)
+    with pytest.raises(ValueError, match="residual"):
+        L.rmsnorm_linear_packed(x, w, 1e-5, packed, ws, 1, 2560, residual=one_row)
+    with pytest.raises(ValueError, match="norm_weight"):
+        L.rmsnorm_linear_packed(x, w[:100], 1e-5, packed, ws, 1, 2560)
+    with pytest.raises(ValueError, match="too small"):
+        L.rmsnorm_linear_packed(x, w, 1e-5, packed[:1000], ws, 1, 2560)
+    with pytest.raises(ValueError, match="s has"):
+        L.TernaInfer_linear_packed(torch.zeros(8, 2560, dtype=torch.int8), packed, torch.zeros(1, dtype=torch.bfloat16), ws, 1, 2560)
+    with pytest.raises(ValueError, match="weight"):
+        L.relu2_mul_rmsnorm_quant(torch.zeros(2, 2 * 6912, dtype=torch.bfloat16), w, 1e-5)
+    with pytest.raises(ValueError, match="does not hold"):
+        L.attention_merge_rmsnorm_linear_packed(torch.zeros(1000, dtype=torch.float32), 4, 20, 128, w, 1e-5, packed, ws, 1, 2560,
+                                                sequences=8)
