@@ -9,7 +9,13 @@
  *
  * Conventions shared by every compute entry point:
  *   - all pointers are device memory owned by the caller; `out` [M][N] row-major bf16 is
- *     fully overwritten; nothing is allocated, freed or synchronised on the call path;
+ *     fully overwritten.  Nothing is allocated, freed or synchronised on the call path -- with ONE exception, which
+ *     is on by default: the repack cache behind the entry points that take the reference format (the section
+ *     "Repack cache" below).  The first call that sees a weight allocates N*K/4 + 256 bytes of device memory
+ *     (hipMalloc), runs two small launches and waits for the stream twice (hipStreamSynchronize); when the cache's
+ *     byte limit is reached or a stale copy is dropped, a call may also hipFree (which waits for the device).  Later
+ *     calls on that weight, every call during stream capture, and every call with TERNASPMM_REPACK_CACHE=0 in the
+ *     environment (or after ternaspmm_repack_cache_enable(0)) only enqueue, as the reference does;
  *   - W is [N][K] ternary in the compressed format (bitmap / TileOffsets_global /
  *     TileOffsets_median / sign words), N % 64 == 0 and K % 64 == 0;
  *   - alignment: `out` at least 8 bytes (the kernels store four bf16 at a time); x, the scales and the format's
@@ -44,9 +50,17 @@ void checkLastCudaError(int line);
  *   M <= 64 : epilogue bf16((acc / s[m]) * ws[g])        (Reduction_Kernel.cuh:60)
  *   M  > 64 : epilogue bf16(acc * (ws[g] / s[m])), 0 if s[m]==0, g per 128-column tile
  *                                                        (epilogue_visitor_scale_ws.h:135-205)
- *   SPLIT_K is accepted for compatibility (split-K partials are reduced on chip).  `workspace`
- *   is used only for M > 64: if it is non-NULL and 16-byte aligned, N*K/4 bytes of it receive a
- *   transcoded copy of the weights for the duration of the call; pass NULL to keep it untouched. */
+ *   `workspace` / SPLIT_K: the library writes at most what the reference itself writes there, so a buffer sized for
+ *   the reference is large enough (model.py:34-42, tests/test_kernel.cu:331):
+ *     - a call the reference serves by its decode path (M <= 64 here, any M on _decode):
+ *       4 * M * N * SPLIT_K bytes, the reference's int32 partial planes (TernaSpMM_API.cuh:66-136);
+ *     - a call it serves by its prefill path (M > 64 here, any M on _prefill): N * K bytes, the reference's dense
+ *       int8 copy of the matrix (SpMM_Kernel.cuh:263-269, TernaSpMM_API.cuh:279-282).
+ *   What for: split-K partial sums of the MFMA-tiled kernel (at most SPLIT_K planes of 4 * M * N bytes on the
+ *   decode path) and, without a cached copy of the weight, a per-call transcode of the weights into its first
+ *   N*K/4 bytes.  It is used only when it is non-NULL and 16-byte aligned; pass NULL to keep it untouched (the
+ *   kernels then do without).  Small calls (the usual decode shapes) never touch it.  Nothing has to be preserved
+ *   in it between calls; calls that share it must not overlap. */
 void bitlinear_TernaSpMM(int8_t* x, uint64_t* bitmap, int* tile_offsets_global,
                          uint16_t* tile_offsets_median, uint32_t* sign_words,
                          terna_bf16* out, terna_bf16* s, terna_bf16* ws, int ws_num,
@@ -94,8 +108,10 @@ void gpu_sleep(double us, terna_stream stream);
  *   x bf16 [M][K], any M >= 1 (no padding rows needed); scale fp32 [ws_num];
  *   group rule of the decode path (Reduction_Kernel.cuh:46-54).
  * The plain symbol picks a kernel by M; _decode / _prefill force the small-M dot-product
- * kernel or the MFMA-tiled kernel.  workspace may be NULL; if given (16-byte aligned, N*K/4
- * bytes) the MFMA-tiled path transcodes the weights into it first, which is faster. */
+ * kernel or the MFMA-tiled kernel.  workspace may be NULL; if given (16-byte aligned) it is used under the same
+ * rule and within the same sizes as bitlinear_TernaSpMM's: 4 * M * N * SPLIT_K bytes for M <= 64 (and on _decode),
+ * N * K bytes for M > 64 (and on _prefill) -- split-K partial sums, and the per-call transcode of a weight the cache
+ * holds no copy of. */
 void bitlinear_TernaSpMM_bf16(const terna_bf16* x, const uint64_t* bitmap, const int* tile_offsets_global,
                               const uint16_t* tile_offsets_median, const uint32_t* sign_words,
                               terna_bf16* out, const float* scale, int ws_num,
@@ -131,9 +147,9 @@ void ternaspmm_decompress_bf16(const uint64_t* bitmap, const int* tile_offsets_g
  * The reference format stays the on-disk and interchange format.  P2 is a device-side layout
  * this library can derive from it, bit-exactly, once at load time; its kernels need no offset
  * arrays and no sign-stream arithmetic.  Callers that keep to the reference entry points never
- * see it, except that the large-M path (M > 64) transcodes into `workspace` when one is given:
- * it needs N*K/4 bytes there, within the N*K bytes the reference's call site guarantees
- * (model.py:34-42). */
+ * see it, except through the repack cache (below) and in that a large-M call on a weight without a cached copy
+ * transcodes into `workspace` when one is given: N*K/4 bytes there, within the N*K bytes the reference's call site
+ * guarantees (model.py:34-42). */
 
 /* Bytes of a P2 buffer for an [N][K] matrix, or -1 if N or K is not a multiple of 64. */
 int64_t ternaspmm_packed_bytes(int N, int K);
@@ -180,6 +196,21 @@ void bitlinear_TernaSpMM_packed_ws(const int8_t* x, const void* packed, terna_bf
 void ternaspmm_rmsnorm_quant(const terna_bf16* x, const terna_bf16* residual, terna_bf16* sum_out,
                              const terna_bf16* weight, float eps, terna_bf16* y_out, int8_t* xq_out,
                              terna_bf16* s_out, int M, int K, terna_stream stream);
+
+/* Which of the reference's evaluations of SpBitLinear.quant_input (model.py:120-123) the prologue kernels above and
+ * below reproduce -- its two lines leave the intermediate precision to PyTorch, and the ways of running them differ on a
+ * few percent of the int8 activations (by one step):
+ *   0  s = bf16(127 / max(max|y|, 1e-5)) and q = rint(fp32(y * s)) with that ROUNDED s: quantiser and epilogue use one
+ *      number (default);
+ *   1  the method as shipped, under @torch.compile (one fused fp32 kernel, no intermediate rounding to bf16; `127 / t`
+ *      on a tensor is t.reciprocal() * 127): q = rint(fp32(y * t)) with the UNROUNDED
+ *      t = fp32(fp32(1 / max(max|y|, 1e-5)) * 127), s = bf16(t);
+ *   2  the same lines in eager mode on bf16 tensors, every op rounded to bf16:
+ *      s = bf16(bf16(1 / max(max|y|, bf16(1e-5))) * 127), q = rint(bf16(y * s)).
+ * ternaspmm_quant_mode(mode) selects one for every later call of the process (a launch recorded in a graph keeps the
+ * mode it was captured with) and returns the previous mode; any other value only queries.  Initial value:
+ * TERNASPMM_QUANT_MODE in the environment, else 0.  The epilogue always divides by the published bf16 s. */
+int ternaspmm_quant_mode(int mode);
 
 /* Same with h = bf16(bf16(relu(x1)^2) * x3), x1 = x13[m][0:F], x3 = x13[m][F:2F] (x13 is the gate/up
  * linear's output, bf16 [M][2F]); the norm and the quantisation run over F columns. */
@@ -335,19 +366,49 @@ void ternaspmm_lm_head_bf16(const terna_bf16* x, const terna_bf16* w, terna_bf16
  * x[b][0 .. V-1] (bf16 [B][V]; out int64 [B]); ties go to the lowest index, NaN never wins.  Only enqueues. */
 void ternaspmm_argmax_bf16(const terna_bf16* x, long long* out, int B, int V, terna_stream stream);
 
-/* Repack cache for unmodified call sites (on unless TERNASPMM_REPACK_CACHE=0 is in the environment): the
- * reference-format entry points above (bitlinear_TernaSpMM*, bitlinear_TernaSpMM_bf16*) keep a device-side P2 copy
- * (N*K/4 bytes) of every weight they have seen -- keyed by device, the bitmap / sign / offset pointers and the shape
- * -- and run the P2 kernels from the second sight on; the first sight allocates, repacks and waits (during stream
- * capture, where nothing may be allocated, it runs the reference-format kernels instead: warm up once before
- * capturing, as generate.py:121-129 does).  Every launch on a cached copy re-checks a fingerprint of the caller's
- * tensors (2.5 KB sampled from the bitmap and sign arrays + the sign-bit total) against the one recorded with the
- * copy; when weights were freed or rewritten and other data sits at the same addresses, the next call into the
- * library prints the reason and exits the process.  Call ternaspmm_repack_cache_clear() after freeing or reloading
- * weights: it releases every cached copy.  ternaspmm_repack_cache_enable(0 / 1) switches the cache off / on at run
- * time and returns the previous setting (copies already made are kept until cleared). */
+/* ---- Repack cache for unmodified call sites (on unless TERNASPMM_REPACK_CACHE=0 is in the environment) ----------
+ * The reference-format entry points above (bitlinear_TernaSpMM*, bitlinear_TernaSpMM_bf16*) keep a device-side P2
+ * copy of every weight they have seen -- keyed by device, the bitmap / sign / offset pointers and the shape -- and run
+ * the P2 kernels from the second sight on.
+ *   Cost in memory: N*K/4 + 256 bytes per weight seen (520 MB for the 120 matrices of a BitNet-2B model), up to a
+ *     limit: by default an eighth of the device's memory, TERNASPMM_REPACK_CACHE_LIMIT_MB in the environment or
+ *     ternaspmm_repack_cache_limit() change it.  At the limit the least recently used copies are released; a weight
+ *     whose copy does not fit is served by the reference-format kernels.
+ *   Cost in behaviour: the first sight of a weight allocates, repacks and waits for the stream (see the conventions
+ *     at the top).  During stream capture nothing is allocated, released or waited for: a weight first seen there is
+ *     served by the reference-format kernels -- warm up once before capturing, as generate.py:121-129 does.  A copy
+ *     that a capture has used is never released behind the graph's back (not at the limit, not when it turns stale);
+ *     only ternaspmm_repack_cache_clear() releases it: destroy such graphs before calling that.
+ *   Stale copies: every launch on a cached copy re-checks a fingerprint of the caller's tensors (2.5 KB sampled from
+ *     the bitmap and sign arrays + the sign-bit total) against the one recorded with the copy.  When weights were
+ *     freed or replaced and other data sits at the same addresses, that launch reports it; the launch itself has
+ *     already used the old copy and its output is invalid.  The next call into the library (outside capture) drops
+ *     the copy, prints a warning (the first eight times) and continues: the weight gets a fresh copy at its next
+ *     sight.  TERNASPMM_REPACK_CACHE_STRICT=1 makes that next call print an error and exit the process instead.  The
+ *     check samples: it finds a replaced tensor, not a few weights edited in place.  Call
+ *     ternaspmm_repack_cache_clear() after freeing, reloading or editing weights and the window never opens.
+ * ternaspmm_repack_cache_clear(): releases every copy (waits for the device).
+ * ternaspmm_repack_cache_enable(0 / 1): switches the cache off / on at run time, returns the previous setting (copies
+ *   already made are kept until cleared).
+ * ternaspmm_repack_cache_limit(bytes): sets the limit (bytes >= 0; a negative value only queries) and returns the
+ *   previous one (-1: none set yet).  Copies beyond a lowered limit go at the next first sight.
+ * ternaspmm_repack_cache_stats(out): out[0] copies held, [1] their bytes, [2] copies dropped as stale so far,
+ *   [3] copies released at the limit so far, [4] bytes parked for captured graphs, [5] the limit (-1: none yet). */
 void ternaspmm_repack_cache_clear(void);
 int ternaspmm_repack_cache_enable(int on);
+long long ternaspmm_repack_cache_limit(long long bytes);
+void ternaspmm_repack_cache_stats(long long out[6]);
+
+/* Host only, enqueues nothing: what a call of the reference-format entry points would do.  int8_activations:
+ * 1 = bitlinear_TernaSpMM*, 0 = bitlinear_TernaSpMM_bf16*; route 0 / 1 / 2 = plain / _prefill / _decode symbol;
+ * `workspace` as the call would pass it (only its alignment matters); cached: whether the weight has a cached P2
+ * copy.  Returns the kernel: 0 small-M kernel on the reference format, 1 MFMA-tiled kernel decoding the reference
+ * format on the fly, 2 per-call transcode into the workspace + MFMA-tiled P2 kernel, 3 small-M kernel on the cached
+ * copy, 4 MFMA-tiled kernel on the cached copy; -1 for an unsupported shape.  *workspace_bytes_used (may be NULL):
+ * the highest byte offset of `workspace` the call would write, 0 when it stays untouched -- never more than the
+ * sizes documented at bitlinear_TernaSpMM. */
+int ternaspmm_plan_reference_call(int int8_activations, int route, int M, int N, int K, int SPLIT_K,
+                                  const void* workspace, int cached, long long* workspace_bytes_used);
 
 /* ---- Calibration probes (no counterpart in the reference) ------------------------------------------------------
  * What the machine gives, measured by the same library in the same run as the kernels a benchmark prices:

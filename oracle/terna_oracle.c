@@ -17,7 +17,8 @@
  *                                  construction of the reference's tests/test_kernel.cu:81)
  *   oracle_spmm_bf16      pinned  (plain fp64 matmul)
  *   oracle_quant_input    pinned  (answers worked by hand: ties to even, scales that are exact,
- *                                  round down and round up in bf16, the all-zero row)
+ *   oracle_quant_input_mode        round down and round up in bf16, the all-zero row; one row on which the three
+ *                                  modes give three different integers)
  *
  * Build: make -C oracle   (gcc -O2 -shared -fPIC)
  */
@@ -313,23 +314,47 @@ void oracle_spmm_bf16(const uint16_t* x, const int8_t* w, const float* scale, in
  * in the tensor's dtype and its compiled graph in fp32 with the unrounded quotient;
  * the known answers in tests/test_oracle_linear.py include a row on which the
  * three differ.) */
-void oracle_quant_input(const uint16_t* x, int M, int K, int8_t* xq, uint16_t* s)
+/* mode 0: the definition above.
+ * `127 / tensor` in the reference's line is Tensor.__rtruediv__, which PyTorch evaluates as tensor.reciprocal() * 127:
+ * mode 1: the method as the reference ships it, under @torch.compile -- one fused fp32 kernel with no intermediate
+ *   rounding to bf16: the multiplier is t = fl32(fl32(1 / max(|x|, 1e-5)) * 127), UNROUNDED (product rounded to
+ *   fp32, then to the nearest integer, ties to even); the returned s is bf16_rn(t).
+ * mode 2: the same two lines in eager mode on a bf16 tensor -- every op rounds its result to bf16: the clamp floor
+ *   is bf16_rn(1e-5), s = bf16_rn(bf16_rn(1 / max) * 127), the product x * s is rounded to bf16 before round(). */
+void oracle_quant_input_mode(const uint16_t* x, int M, int K, int mode, int8_t* xq, uint16_t* s)
 {
+    const float floor_v = mode == 2 ? bf16_to_f32(f32_to_bf16_rn(1e-5f)) : 1e-5f;
     for (int m = 0; m < M; ++m) {
         float amax = 0.0f;
         for (int k = 0; k < K; ++k) {
             float v = fabsf(bf16_to_f32(x[(size_t)m * K + k]));
             if (v > amax) amax = v;
         }
-        if (amax < 1e-5f) amax = 1e-5f;
-        uint16_t sb = f32_to_bf16_rn(127.0f / amax);
-        float sf = bf16_to_f32(sb);
+        if (amax < floor_v) amax = floor_v;
+        volatile float t;                                          /* volatile: rounded to fp32, no wider intermediate */
+        if (mode == 0) {
+            t = 127.0f / amax;
+        } else {
+            volatile float r = 1.0f / amax;
+            if (mode == 2) r = bf16_to_f32(f32_to_bf16_rn(r));
+            t = r * 127.0f;
+        }
+        uint16_t sb = f32_to_bf16_rn(t);
+        float mul = mode == 1 ? t : bf16_to_f32(sb);
         s[m] = sb;
         for (int k = 0; k < K; ++k) {
-            float q = nearbyintf(bf16_to_f32(x[(size_t)m * K + k]) * sf);
+            volatile float p = bf16_to_f32(x[(size_t)m * K + k]) * mul;
+            float pr = p;
+            if (mode == 2) pr = bf16_to_f32(f32_to_bf16_rn(pr));
+            float q = nearbyintf(pr);
             if (q > 127.0f) q = 127.0f;
             if (q < -128.0f) q = -128.0f;
             xq[(size_t)m * K + k] = (int8_t)q;
         }
     }
+}
+
+void oracle_quant_input(const uint16_t* x, int M, int K, int8_t* xq, uint16_t* s)
+{
+    oracle_quant_input_mode(x, M, K, 0, xq, s);
 }

@@ -257,13 +257,35 @@ def spmm_bf16_golden(x_bits: np.ndarray, w: np.ndarray, scale: np.ndarray, ws_nu
     return acc * sc.reshape(1, n)
 
 
-def quant_input(x_bits: np.ndarray):
-    """model.py:120-123 with fp32 compute and s rounded to bf16 (see terna_oracle.c)."""
+QUANT_ROUNDED, QUANT_COMPILED, QUANT_EAGER = 0, 1, 2
+
+
+def quant_input(x_bits: np.ndarray, mode: int = QUANT_ROUNDED):
+    """model.py:120-123.  The reference's two lines leave the intermediate precision to PyTorch; `mode` says which
+    evaluation is restated (see terna_oracle.c):
+      QUANT_ROUNDED   fp32 compute, s = bf16(127 / max) and that rounded s multiplies (this build's default);
+      QUANT_COMPILED  the @torch.compile'd method: fp32 compute without intermediate roundings to bf16.  `127 / t` on a
+                      tensor is Tensor.__rtruediv__ = t.reciprocal() * 127, so the multiplier is fl32(fl32(1 / max) * 127),
+                      unrounded; the returned s is its bf16 rounding;
+      QUANT_EAGER     eager mode on a bf16 tensor, every op rounded to bf16: the clamp floor bf16(1e-5),
+                      s = bf16(bf16(1 / max) * 127), and the product bf16(x * s) before round()."""
     x = bf16_bits_to_f32(x_bits)
-    amax = np.maximum(np.abs(x).max(axis=-1, keepdims=True), np.float32(1e-5)).astype(np.float32)
-    s_bits = f32_to_bf16_bits((np.float32(127.0) / amax).astype(np.float32))
-    s = bf16_bits_to_f32(s_bits)
-    q = np.clip(np.rint((x * s).astype(np.float32)), -128, 127).astype(np.int8)
+    rb = lambda v: bf16_bits_to_f32(f32_to_bf16_bits(np.asarray(v, dtype=np.float32)))
+    floor = rb(np.float32(1e-5)) if mode == QUANT_EAGER else np.float32(1e-5)
+    amax = np.maximum(np.abs(x).max(axis=-1, keepdims=True), floor).astype(np.float32)
+    if mode == QUANT_ROUNDED:
+        t = (np.float32(127.0) / amax).astype(np.float32)
+    else:
+        r = (np.float32(1.0) / amax).astype(np.float32)
+        if mode == QUANT_EAGER:
+            r = rb(r)
+        t = (r * np.float32(127.0)).astype(np.float32)
+    s_bits = f32_to_bf16_bits(t)
+    mul = t if mode == QUANT_COMPILED else bf16_bits_to_f32(s_bits)
+    prod = (x * mul).astype(np.float32)
+    if mode == QUANT_EAGER:
+        prod = rb(prod)
+    q = np.clip(np.rint(prod), -128, 127).astype(np.int8)
     return q, s_bits.reshape(-1)
 
 
@@ -394,6 +416,7 @@ class COracle:
         L.oracle_spmm_i8.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
         L.oracle_spmm_bf16.argtypes = [vp, vp, vp, ci, ci, ci, ci, vp]
         L.oracle_quant_input.argtypes = [vp, ci, ci, vp, vp]
+        L.oracle_quant_input_mode.argtypes = [vp, ci, ci, ci, vp, vp]
         L.oracle_f32_to_bf16.argtypes = [ctypes.c_float]
         L.oracle_f32_to_bf16.restype = ctypes.c_uint16
 
@@ -462,10 +485,10 @@ class COracle:
                                   ws_num, m, n, k, self._p(out))
         return out
 
-    def quant_input(self, x_bits):
+    def quant_input(self, x_bits, mode: int = QUANT_ROUNDED):
         m, k = x_bits.shape
         xq = np.empty((m, k), dtype=np.int8)
         s = np.empty(m, dtype=np.uint16)
-        self.lib.oracle_quant_input(self._p(np.ascontiguousarray(x_bits, dtype=np.uint16)), m, k,
-                                    self._p(xq), self._p(s))
+        self.lib.oracle_quant_input_mode(self._p(np.ascontiguousarray(x_bits, dtype=np.uint16)), m, k, mode,
+                                         self._p(xq), self._p(s))
         return xq, s

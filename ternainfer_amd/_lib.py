@@ -70,6 +70,10 @@ PROTOTYPES = {
     "ternaspmm_probe_barrier": ([_vp, _ci, _ci, ctypes.c_uint, _vp], ctypes.c_int),
     "ternaspmm_repack_cache_clear": ([], None),
     "ternaspmm_repack_cache_enable": ([_ci], _ci),
+    "ternaspmm_repack_cache_limit": ([ctypes.c_longlong], ctypes.c_longlong),
+    "ternaspmm_repack_cache_stats": ([_vp], None),
+    "ternaspmm_plan_reference_call": ([_ci] * 6 + [_vp, _ci, _vp], _ci),
+    "ternaspmm_quant_mode": ([_ci], _ci),
     "ternaspmm_version": ([], ctypes.c_char_p),
 }
 

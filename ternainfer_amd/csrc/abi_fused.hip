@@ -23,7 +23,7 @@ void ternaspmm_rmsnorm_quant(const terna_bf16* x, const terna_bf16* residual, te
         return;
     }
     terna_norm_quant_kernel<false><<<dim3(M), dim3(kNormThreads), 0, static_cast<hipStream_t>(stream)>>>(
-        x, residual, weight, K, eps, sum_out, y_out, xq_out, s_out);
+        x, residual, weight, K, eps, sum_out, y_out, xq_out, s_out, quant_mode());
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_rmsnorm_quant", e, __LINE__);
 }
@@ -36,7 +36,7 @@ void ternaspmm_relu2_mul_rmsnorm_quant(const terna_bf16* x13, const terna_bf16* 
         return;
     }
     terna_norm_quant_kernel<true><<<dim3(M), dim3(kNormThreads), 0, static_cast<hipStream_t>(stream)>>>(
-        x13, nullptr, weight, F, eps, nullptr, y_out, xq_out, s_out);
+        x13, nullptr, weight, F, eps, nullptr, y_out, xq_out, s_out, quant_mode());
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_relu2_mul_rmsnorm_quant", e, __LINE__);
 }
@@ -73,9 +73,10 @@ static int launch_decode_fused(int mode, const terna_bf16* x, const terna_bf16* 
     const bool multi8 = multi && nb_waves == 8 && ktiles <= 8 * 5;
     const bool multi16 = multi && !multi8 && ktiles <= 16 * 3;
     const dim3 grid(multi16 || multi8 ? bands / 4 : bands);
+    const int qmode = quant_mode();
 #define TERNA_FUSED(WAVES, TMAX, MODE, MP, NB)                                                                     \
     terna_decode_fused_kernel<WAVES, TMAX, MODE, MP, NB><<<grid, dim3(WAVES * 64), 0, st>>>(                       \
-        x, residual, norm_weight, p, M, N, K, eps, sum_out, out, ws, ws_num, xq_out, s_out)
+        x, residual, norm_weight, p, M, N, K, eps, sum_out, out, ws, ws_num, xq_out, s_out, qmode)
 #define TERNA_FUSED_M(WAVES, TMAX, MODE, NB)                                                                       \
     do {                                                                                                           \
         if (M == 1) TERNA_FUSED(WAVES, TMAX, MODE, 1, NB);                                                         \
@@ -134,9 +135,10 @@ int bitlinear_TernaSpMM_packed_fused_attn(const float* partial, int splits, int 
     const uint16_t* x = reinterpret_cast<const uint16_t*>(partial);
     const uint32_t* p = static_cast<const uint32_t*>(packed);
     hipStream_t st = static_cast<hipStream_t>(stream);
+    const int qmode = quant_mode();
 #define TERNA_FUSED_ATTN(SP, HD)                                                                                   \
     terna_decode_fused_kernel<8, 5, FUSED_ATTN, 1, 1, SP, HD><<<grid, dim3(8 * 64), 0, st>>>(                      \
-        x, nullptr, norm_weight, p, M, N, K, eps, nullptr, out, ws, ws_num, xq_out, s_out)
+        x, nullptr, norm_weight, p, M, N, K, eps, nullptr, out, ws, ws_num, xq_out, s_out, qmode)
 #define TERNA_FUSED_ATTN_HD(HD)                                                                                    \
     do {                                                                                                           \
         if (splits == 1) TERNA_FUSED_ATTN(1, HD);                                                                  \

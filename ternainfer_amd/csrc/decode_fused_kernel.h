@@ -98,7 +98,7 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, const uint16_t* __restrict__ norm_w,
     const uint32_t* __restrict__ packed, int M, int N, int K, float eps, uint16_t* __restrict__ sum_out,
     uint16_t* __restrict__ out, const uint16_t* __restrict__ ws, int ws_num, int8_t* __restrict__ xq_out,
-    uint16_t* __restrict__ s_out)
+    uint16_t* __restrict__ s_out, int quant_mode)
 {
     static_assert(MODE != FUSED_ATTN || MP == 1, "the attention merge feeds a single row");
     static_assert(AHD % 64 == 0 && ASP >= 1 && ASP <= kAttentionMaxSplits, "a 64-column tile lies inside one head");
@@ -266,10 +266,10 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
         xr[t].pack(f);
     }
     amax = row_reduce(amax, 1, true);
-    const uint16_t s_bits = float_to_bf16_bits(__fdiv_rn(127.0f, fmaxf(amax, 1e-5f)));
-    const float s = bf16_bits_to_float(s_bits);
+    uint16_t s_bits;
+    const float s = quant_scale(amax, quant_mode, &s_bits);      // what multiplies; the epilogue divides by the bf16 value
     if (wave == 0 && (lane % LPR) == 0) {
-        s_row[row] = s;
+        s_row[row] = bf16_bits_to_float(s_bits);
         if (writer && s_out != nullptr && row_ok) s_out[row] = s_bits;
     }
 
@@ -286,7 +286,7 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
             uint8_t q[MP];
 #pragma unroll
             for (int e = 0; e < MP; ++e) {
-                const float r = __builtin_amdgcn_fmed3f(rintf(__fmul_rn(f[e], s)), -128.0f, 127.0f);
+                const float r = quant_value(f[e], s, quant_mode);
                 q[e] = static_cast<uint8_t>(static_cast<int>(r) & 0xff);
             }
             uint8_t* dst = slab + row * XQ::kPitch + cl;

@@ -84,6 +84,10 @@ void allow_dynamic_lds(Kernel kernel, int bytes, const char* what, int line)
     allow_dynamic_lds_ptr(reinterpret_cast<const void*>(kernel), bytes, what, line);
 }
 
+// The process-wide quant_input mode (QuantMode in terna_common.h; ternaspmm_quant_mode sets it, TERNASPMM_QUANT_MODE in
+// the environment gives the initial value).  Defined in ternaspmm.hip.
+int quant_mode();
+
 // Shapes the attention entry points accept (head sizes 64 and 128, whole kv groups, caches of up to 8192 slots).
 inline bool attention_args_ok(const char* who, int B, int H, int KV, int D, int S)
 {

@@ -54,17 +54,13 @@ int prefill_splits(long tiles, int steps, int M, int N, size_t scratch_bytes)
 
 template <typename Act, int MB, int NA>
 void launch_prefill_packed_dma_as(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M,
-                                  int N, int K, void* scratch, size_t scratch_bytes, hipStream_t st)
+                                  int N, int K, const PrefillPlan& plan, void* scratch, hipStream_t st)
 {
     using S = PackedPrefillDmaSmem<MB>;
     auto kernel = terna_prefill_packed_dma_kernel<Act, MB, NA>;
     allow_dynamic_lds(kernel, S::kBytes, "hipFuncSetAttribute(prefill packed dma)", __LINE__);
-    constexpr int BN = 128 * NA;
-    dim3 grid((N + BN - 1) / BN, (M + S::BM - 1) / S::BM);
-    const int steps = sizeof(Act) == 1 ? ((K >> 6) + 1) >> 1 : K >> 6;
-    const bool scratch_ok = scratch != nullptr && (reinterpret_cast<uintptr_t>(scratch) & 15) == 0 && (N & 3) == 0;
-    const int splits = scratch_ok ? prefill_splits(static_cast<long>(grid.x) * grid.y, steps, M, N, scratch_bytes) : 1;
-    grid.z = splits;
+    const dim3 grid(plan.grid_x, plan.grid_y, plan.splits);
+    const int splits = plan.splits;
     static const int xcd_forced = [] {
         const char* v = tuning_env("TERNASPMM_PREFILL_XCD_MAP");
         return v ? std::atoi(v) : -1;
@@ -98,8 +94,7 @@ inline bool prefill_dma_ok(const void* x, size_t act_bytes, int M, int N, int K)
 }  // namespace
 
 template <typename Act>
-void launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
-                           void* scratch, size_t scratch_bytes, hipStream_t st)
+PrefillPlan plan_prefill_packed(const void* x, int M, int N, int K, const void* scratch, size_t scratch_bytes)
 {
     // Batch rows per workgroup (64 / 128 / 256).  Measured on MI355X the 64-row tile wins at every
     // BitNet-2B shape: it runs four waves per SIMD, and occupancy hides more latency than the taller
@@ -114,27 +109,50 @@ void launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, 
         const int bn = v ? std::atoi(v) : 0;
         return (bn == 128 || bn == 256) ? bn : 0;
     }();
-    const int bm = forced ? forced : 64;
+    PrefillPlan plan{};
+    plan.bm = forced ? forced : 64;
     // 256-feature tiles expand every weight once per 64 batch rows with two MFMAs per operand read;
     // when they would leave most of the 1024 workgroup slots of the chip empty, 128-feature tiles
     // double the workgroup count instead.  TERNASPMM_PREFILL_BN=128|256 forces one (tuning aid).
     const long wg256 = static_cast<long>((N + 255) / 256) * ((M + 63) / 64);
-    const int bn = forced_bn ? forced_bn : (wg256 <= 640 ? 128 : 256);
-    if (prefill_dma_ok(x, sizeof(Act), M, N, K) && (bm == 64 || bm == 128)) {
-        if (bm == 64 && bn == 128) launch_prefill_packed_dma_as<Act, 2, 1>(x, packed, out, ep, M, N, K, scratch, scratch_bytes, st);
-        else if (bm == 128 && forced_bn == 128) launch_prefill_packed_dma_as<Act, 4, 1>(x, packed, out, ep, M, N, K, scratch, scratch_bytes, st);
-        else if (bm == 128) launch_prefill_packed_dma_as<Act, 4, 2>(x, packed, out, ep, M, N, K, scratch, scratch_bytes, st);
-        else launch_prefill_packed_dma_as<Act, 2, 2>(x, packed, out, ep, M, N, K, scratch, scratch_bytes, st);
+    plan.bn = forced_bn ? forced_bn : (wg256 <= 640 ? 128 : 256);
+    plan.direct_lds = prefill_dma_ok(x, sizeof(Act), M, N, K) && (plan.bm == 64 || plan.bm == 128);
+    if (plan.direct_lds) {
+        if (plan.bm == 128 && forced_bn != 128) plan.bn = 256;
+    } else if (!(plan.bm == 64 && plan.bn == 128)) {
+        plan.bn = 256;                       // the register-staged kernel has 256-feature tiles except at 64 x 128
+    }
+    plan.grid_x = static_cast<unsigned>((N + plan.bn - 1) / plan.bn);
+    plan.grid_y = static_cast<unsigned>((M + plan.bm - 1) / plan.bm);
+    plan.steps = sizeof(Act) == 1 ? ((K >> 6) + 1) >> 1 : K >> 6;
+    plan.splits = 1;
+    const bool scratch_ok = plan.direct_lds && scratch != nullptr && (reinterpret_cast<uintptr_t>(scratch) & 15) == 0 && (N & 3) == 0;
+    if (scratch_ok) plan.splits = prefill_splits(static_cast<long>(plan.grid_x) * plan.grid_y, plan.steps, M, N, scratch_bytes);
+    plan.scratch_used = plan.splits > 1 ? static_cast<size_t>(plan.splits) * M * N * 4 : 0;
+    return plan;
+}
+
+template <typename Act>
+void launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                           void* scratch, size_t scratch_bytes, hipStream_t st)
+{
+    const PrefillPlan plan = plan_prefill_packed<Act>(x, M, N, K, scratch, scratch_bytes);
+    if (plan.direct_lds) {
+        if (plan.bm == 64 && plan.bn == 128) launch_prefill_packed_dma_as<Act, 2, 1>(x, packed, out, ep, M, N, K, plan, scratch, st);
+        else if (plan.bm == 128 && plan.bn == 128) launch_prefill_packed_dma_as<Act, 4, 1>(x, packed, out, ep, M, N, K, plan, scratch, st);
+        else if (plan.bm == 128) launch_prefill_packed_dma_as<Act, 4, 2>(x, packed, out, ep, M, N, K, plan, scratch, st);
+        else launch_prefill_packed_dma_as<Act, 2, 2>(x, packed, out, ep, M, N, K, plan, scratch, st);
         return;
     }
-    if (bm == 64 && bn == 128) launch_prefill_packed_as<Act, 2, 1>(x, packed, out, ep, M, N, K, st);
-    else if (bm == 256) launch_prefill_packed_as<Act, 8>(x, packed, out, ep, M, N, K, st);
-    else if (bm == 96) launch_prefill_packed_as<Act, 3>(x, packed, out, ep, M, N, K, st);
-    else if (bm == 128) launch_prefill_packed_as<Act, 4>(x, packed, out, ep, M, N, K, st);
+    if (plan.bm == 64 && plan.bn == 128) launch_prefill_packed_as<Act, 2, 1>(x, packed, out, ep, M, N, K, st);
+    else if (plan.bm == 256) launch_prefill_packed_as<Act, 8>(x, packed, out, ep, M, N, K, st);
+    else if (plan.bm == 96) launch_prefill_packed_as<Act, 3>(x, packed, out, ep, M, N, K, st);
+    else if (plan.bm == 128) launch_prefill_packed_as<Act, 4>(x, packed, out, ep, M, N, K, st);
     else launch_prefill_packed_as<Act, 2>(x, packed, out, ep, M, N, K, st);
 }
 
 template void launch_prefill_packed<TERNA_PREFILL_ACT>(const TERNA_PREFILL_ACT*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int,
                                                        void*, size_t, hipStream_t);
+template PrefillPlan plan_prefill_packed<TERNA_PREFILL_ACT>(const void*, int, int, int, const void*, size_t);
 
 }  // namespace terna

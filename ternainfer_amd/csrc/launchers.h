@@ -44,6 +44,19 @@ void launch_repack_guard(const RepackGuard* guard, hipStream_t st);
 template <typename Act>
 void launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
                            void* scratch, size_t scratch_bytes, hipStream_t st);
+// What launch_prefill_packed does with a call (host arithmetic only, nothing is enqueued): the output tile, the
+// grid, the split-K count and how many bytes of `scratch` the partial planes take (0 without a split; never more than
+// scratch_bytes).
+struct PrefillPlan {
+    int bm, bn;                 // batch rows x output features per workgroup
+    unsigned grid_x, grid_y;
+    int steps;                  // K steps of one workgroup without a split
+    int splits;
+    bool direct_lds;            // activations loaded straight into LDS (16-byte aligned x, operands below 4 GiB)
+    size_t scratch_used;        // splits * M * N * 4 when splits > 1
+};
+template <typename Act>
+PrefillPlan plan_prefill_packed(const void* x, int M, int N, int K, const void* scratch, size_t scratch_bytes);
 
 extern template void launch_decode<int8_t>(const int8_t*, const Weights&, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
 extern template void launch_decode<uint16_t>(const uint16_t*, const Weights&, uint16_t*, const Epilogue&, int, int, int, hipStream_t);
@@ -57,6 +70,9 @@ extern template void launch_prefill_packed<int8_t>(const int8_t*, const uint32_t
                                                    hipStream_t);
 extern template void launch_prefill_packed<uint16_t>(const uint16_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, void*, size_t,
                                                      hipStream_t);
+
+extern template PrefillPlan plan_prefill_packed<int8_t>(const void*, int, int, int, const void*, size_t);
+extern template PrefillPlan plan_prefill_packed<uint16_t>(const void*, int, int, int, const void*, size_t);
 
 // Tuning override shared by the two small-M launchers: TERNASPMM_DECODE_WAVES=4|8|16 forces one variant.
 int decode_waves_override();

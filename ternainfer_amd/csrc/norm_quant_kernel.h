@@ -9,7 +9,8 @@
 //      = bf16(x + residual)                  (residual add; h is also written back as the new stream)
 //      = bf16(bf16(relu(x1)^2) * x3)         (gated FFN; x1 = row[0:F], x3 = row[F:2F])
 //   y  = bf16(h * rsqrt(mean(h^2) + eps) * weight)          fp32 inside, one rounding at the end
-//   s  = bf16(127 / max(max|y|, 1e-5));  q = clamp(rint(y * s), -128, 127)   (fp32 inside)
+//   s  = bf16(127 / max(max|y|, 1e-5));  q = clamp(rint(y * s), -128, 127)   (fp32 inside; `quant_mode` selects
+//        which of the reference's ways of evaluating these two lines is reproduced: QuantMode in terna_common.h)
 //
 // The row stays in registers between the three passes; HBM sees each input element once and each
 // output element once.  Rows are independent, so the grid is M workgroups of 256 threads.
@@ -100,7 +101,7 @@ template <bool GLU>
 __global__ __launch_bounds__(kNormThreads) void terna_norm_quant_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, const uint16_t* __restrict__ weight, int K,
     float eps, uint16_t* __restrict__ sum_out, uint16_t* __restrict__ y_out, int8_t* __restrict__ xq_out,
-    uint16_t* __restrict__ s_out)
+    uint16_t* __restrict__ s_out, int quant_mode)
 {
     __shared__ float red[2][kNormThreads / 64];
     const int tid = threadIdx.x;
@@ -184,8 +185,8 @@ __global__ __launch_bounds__(kNormThreads) void terna_norm_quant_kernel(
     if (lane == 0) red[1][wave] = amax;
     __syncthreads();
     amax = fmaxf(fmaxf(red[1][0], red[1][1]), fmaxf(red[1][2], red[1][3]));
-    const uint16_t s_bits = float_to_bf16_bits(__fdiv_rn(127.0f, fmaxf(amax, 1e-5f)));
-    const float s = bf16_bits_to_float(s_bits);
+    uint16_t s_bits;
+    const float s = quant_scale(amax, quant_mode, &s_bits);
     if (tid == 0) s_out[row] = s_bits;
 #pragma unroll
     for (int i = 0; i < kNormMaxVecs; ++i) {
@@ -194,8 +195,7 @@ __global__ __launch_bounds__(kNormThreads) void terna_norm_quant_kernel(
             uint32_t q[2] = {0u, 0u};
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                float r = rintf(__fmul_rn(h[i][j], s));
-                r = fminf(fmaxf(r, -128.0f), 127.0f);
+                const float r = quant_value(h[i][j], s, quant_mode);
                 q[j >> 2] |= (static_cast<uint32_t>(static_cast<int>(r)) & 0xffu) << (8 * (j & 3));
             }
             *reinterpret_cast<u32x2*>(xq_out + row * K + 8 * v) = u32x2{q[0], q[1]};

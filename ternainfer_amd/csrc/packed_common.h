@@ -72,7 +72,8 @@ __device__ __forceinline__ uint32_t make_lut_code(int e)
 // Fingerprint of a matrix in the reference format, computed by one wave: the total sign-bit count
 // (tile_off[tiles]) and 64 words each from the start, the middle and the end of the bitmap array and from the start
 // and the end of the sign stream, mixed per lane and folded over the wave.  A weight that was freed and replaced by
-// another one at the same addresses differs in these 2.5 KB with all but negligible probability.
+// another one at the same addresses differs in these 2.5 KB with all but negligible probability.  (Weights edited in
+// place at a few positions are NOT what this detects.)
 __device__ __forceinline__ unsigned long long fingerprint_mix(unsigned long long x)
 {
     x ^= x >> 30;
@@ -81,14 +82,17 @@ __device__ __forceinline__ unsigned long long fingerprint_mix(unsigned long long
     x *= 0x94d049bb133111ebull;
     return x ^ (x >> 31);
 }
+// `total` = tile_off[tiles] as it reads now.  The sign stream is sampled only when that equals the recorded length --
+// the positions follow the length, and a stream that is shorter now must not be read past its end; a different length
+// alone makes the fingerprint differ (the total is mixed in last).
 __device__ __forceinline__ unsigned long long repack_fingerprint(const RepackGuard& g, int lane)
 {
     const long long n_bm = static_cast<long long>(g.tiles) * 64;
     const int total = g.tile_off[g.tiles];
-    const int words = g.words;
     const unsigned long long b0 = g.bitmap[lane], b1 = g.bitmap[n_bm / 2 - 32 + lane], b2 = g.bitmap[n_bm - 64 + lane];
+    const int words = g.total_bits >> 5;
     unsigned long long s0 = 0, s1 = 0;
-    if (words > 0) {
+    if (total == g.total_bits && words > 0) {
         const int hi = words - 1;
         int tail = words - 64 + lane;
         tail = tail < 0 ? 0 : tail;
@@ -107,12 +111,16 @@ __device__ __forceinline__ unsigned long long repack_fingerprint(const RepackGua
     }
     return fingerprint_mix(((static_cast<unsigned long long>(hi32) << 32) | lo) ^ static_cast<unsigned long long>(static_cast<uint32_t>(total)));
 }
-// One wave: compare with the recorded fingerprint, raise the host-visible flag on a mismatch.
+// One wave: compare with the recorded fingerprint; on a mismatch report the copy's id in the host-visible words.
 __device__ __forceinline__ void repack_guard_role(const RepackGuard& g, int lane)
 {
     const unsigned long long want = *g.expect;          // requested together with the samples
     const unsigned long long now = repack_fingerprint(g, lane);
-    if (lane == 0 && now != want) *reinterpret_cast<volatile uint32_t*>(g.stale) = 1u;
+    if (lane == 0 && now != want) {
+        volatile uint32_t* flags = g.stale;
+        flags[1 + g.id % 1023u] = g.id;
+        flags[0] = 1u;
+    }
 }
 
 // Reference format -> P2.  One wave per 16x64 band-tile; lane (i, g) produces word 4*i + g.

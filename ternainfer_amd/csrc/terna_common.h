@@ -26,10 +26,11 @@ enum EpilogueKind : int {
 };
 
 // What a kernel needs to check that a cached P2 copy still belongs to the reference-format tensors it was made from:
-// the tensors as the caller passes them now, the fingerprint recorded when the copy was made, and a flag in
-// host-visible memory that is raised on a mismatch.  `words` is the length of the sign stream when the copy was made:
-// the sampled positions follow it, so that every load of the check is independent of every other (one memory round
-// trip; a changed length shows in the sign-bit total, which is part of the fingerprint).
+// the tensors as the caller passes them now, the fingerprint recorded when the copy was made, the copy's id and the
+// host-visible words in which a mismatch is reported (word 0: any report; word 1 + id % 1023: the id).
+// `total_bits` is the length of the sign stream when the copy was made: the check compares it with the length the
+// caller's offset array states now before it samples the stream, so no sample lies past the end of a shorter stream
+// that has taken the old one's place.
 struct RepackGuard {
     const uint64_t* bitmap;
     const int* tile_off;
@@ -37,8 +38,22 @@ struct RepackGuard {
     const unsigned long long* expect;
     uint32_t* stale;
     int tiles;                       // N * K / 4096
-    int words;                       // sign words of the matrix the copy was made from
+    int total_bits;                  // sign bits (padded per tile) of the matrix the copy was made from
+    uint32_t id;
 };
+
+// How quant_input (model.py:120-123) is evaluated.  The reference's two lines leave the intermediate precision to
+// PyTorch, and its two ways of running them differ.  (`127 / tensor` there is Tensor.__rtruediv__, which PyTorch
+// evaluates as tensor.reciprocal() * 127.)
+//   QUANT_ROUNDED   s = bf16(127 / max(max|x|, 1e-5)); q = rint(fp32(x * s)) with that ROUNDED s -- the quantiser and
+//                   the epilogue's division then use the same number (this library's default);
+//   QUANT_COMPILED  what the @torch.compile'd method computes (one fused fp32 kernel, no intermediate rounding to
+//                   bf16): q = rint(fp32(x * t)) with the UNROUNDED t = fp32(fp32(1 / max(max|x|, 1e-5)) * 127); the
+//                   returned s is bf16(t);
+//   QUANT_EAGER     what the same lines give without torch.compile on bf16 tensors: every op rounds to bf16 --
+//                   s = bf16(bf16(1 / max(max|x|, bf16(1e-5))) * 127), q = rint(bf16(x * s)).
+// In every mode the s that is published (and that the epilogue divides by) is the bf16 value.
+enum QuantMode : int { QUANT_ROUNDED = 0, QUANT_COMPILED = 1, QUANT_EAGER = 2 };
 
 struct Epilogue {
     const uint16_t* s;      // bf16 [M]       (int8 family)
@@ -64,6 +79,32 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
     typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
     typedef float f32x2_t __attribute__((ext_vector_type(2)));
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
+}
+
+// The per-row scale of quant_input from the row's max |x|: `s_bits` is what is published, the return value what
+// multiplies the activations.
+__device__ __forceinline__ float quant_scale(float amax, int mode, uint16_t* s_bits)
+{
+    const float floor_v = mode == QUANT_EAGER ? 1.0013580322265625e-05f /* bf16(1e-5) */ : 1e-5f;
+    const float a = fmaxf(amax, floor_v);
+    float t;
+    if (mode == QUANT_ROUNDED) {
+        t = __fdiv_rn(127.0f, a);
+    } else {
+        float r = __fdiv_rn(1.0f, a);
+        if (mode == QUANT_EAGER) r = bf16_bits_to_float(float_to_bf16_bits(r));
+        t = __fmul_rn(r, 127.0f);
+    }
+    *s_bits = float_to_bf16_bits(t);
+    return mode == QUANT_COMPILED ? t : bf16_bits_to_float(*s_bits);
+}
+// One activation: clamp(rint(x * s_mul)), the product rounded to bf16 first in QUANT_EAGER.  Returned as a float in
+// [-128, 127].
+__device__ __forceinline__ float quant_value(float x, float s_mul, int mode)
+{
+    float p = __fmul_rn(x, s_mul);
+    if (mode == QUANT_EAGER) p = bf16_bits_to_float(float_to_bf16_bits(p));
+    return __builtin_amdgcn_fmed3f(rintf(p), -128.0f, 127.0f);
 }
 
 // Weight-scale group of output column n on the decode path (Reduction_Kernel.cuh:46-54).

@@ -4,6 +4,7 @@
 // kernels of a decode step have their entry points in abi_fused.hip, abi_attention.hip and abi_head.hip.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <mutex>
@@ -13,32 +14,28 @@
 #include "format_host.h"
 #include "host_util.h"
 #include "launchers.h"
+#include "repack_cache.h"
 
 using namespace terna;
 
+namespace terna {
 namespace {
-
-// Large-M call on reference-format pointers: with a 16-byte aligned workspace of N*K/4 bytes the
-// weights are first transcoded to P2 there (one cheap pass) and the P2 kernel does the GEMM;
-// without one the fused reference-format kernel runs.
-//
-// The reference's call site guarantees N*K bytes of workspace on this path (model.py:34-42: the dense int8 copy of the
-// matrix its prefill path writes there); the transcoded weights take the first quarter, and what follows may hold
-// split-K partial sums when the shape has few output tiles for the chip.
-template <typename Act>
-void launch_large_m(const Act* x, const Weights& w, uint16_t* out, const Epilogue& ep, int M, int N, int K,
-                    void* workspace, hipStream_t st)
-{
-    if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
-        uint32_t* packed = static_cast<uint32_t*>(workspace);
-        launch_repack(w, packed, N, K, st);
-        const size_t p2_bytes = (static_cast<size_t>(N) * K / 4 + 255) & ~static_cast<size_t>(255);
-        launch_prefill_packed(x, packed, out, ep, M, N, K, static_cast<char*>(workspace) + p2_bytes,
-                              static_cast<size_t>(N) * K - p2_bytes, st);
-    } else {
-        launch_prefill(x, w, out, ep, M, N, K, st);
-    }
+std::atomic<int> g_quant_mode{-1};     // -1: not decided yet (environment)
 }
+int quant_mode()
+{
+    int m = g_quant_mode.load(std::memory_order_relaxed);
+    if (m < 0) {
+        const char* v = std::getenv("TERNASPMM_QUANT_MODE");
+        m = v != nullptr ? std::atoi(v) : 0;
+        if (m < QUANT_ROUNDED || m > QUANT_EAGER) m = QUANT_ROUNDED;
+        g_quant_mode.store(m, std::memory_order_relaxed);
+    }
+    return m;
+}
+}  // namespace terna
+
+namespace {
 
 enum Route { ROUTE_AUTO, ROUTE_DECODE, ROUTE_PREFILL };
 
@@ -62,45 +59,84 @@ bool packed_small_kernel(int M, int N, int K, bool int8, bool has_scratch)
     return M <= 64;
 }
 
+// Scratch for split-K is worth counting on when it holds two planes of partial sums or more.
+bool scratch_for_split(const void* scratch, size_t bytes, int M, int N)
+{
+    return scratch != nullptr && (reinterpret_cast<uintptr_t>(scratch) & 15) == 0 && bytes >= static_cast<size_t>(8) * M * N;
+}
+
+// What a call on reference-format pointers does, decided on the host before anything is enqueued (also what
+// ternaspmm_plan_reference_call reports).  The caller's workspace is used within the bytes the reference itself would
+// write there and never beyond (reference_workspace_bytes): with a cached P2 copy all of them may hold split-K planes;
+// without one a large-M call puts its per-call P2 transcode (N*K/4 bytes) first and the planes behind it.
+enum CallKernel {
+    CALL_REF_SMALL = 0,        // small-M kernel on the reference format
+    CALL_REF_FUSED_LARGE = 1,  // MFMA-tiled kernel that decodes the reference format on the fly (no workspace)
+    CALL_TRANSCODE_LARGE = 2,  // transcode into the workspace, then the MFMA-tiled P2 kernel
+    CALL_P2_SMALL = 3,         // small-M kernel on the cached P2 copy
+    CALL_P2_LARGE = 4,         // MFMA-tiled kernel on the cached P2 copy
+};
+struct CallPlan {
+    CallKernel kernel;
+    size_t p2_bytes;           // bytes of the workspace that receive transcoded weights (CALL_TRANSCODE_LARGE)
+    size_t scratch_offset;     // where split-K planes may start
+    size_t scratch_bytes;      // ... and how many bytes they may take
+};
+CallPlan plan_call(bool int8, Route route, int M, int N, int K, int split_k, const void* workspace, bool cached)
+{
+    const bool ref_prefill_path = route == ROUTE_PREFILL || (route == ROUTE_AUTO && M > 64);
+    const bool aligned = workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0;
+    const size_t avail = aligned ? reference_workspace_bytes(ref_prefill_path, M, N, K, split_k) : 0;
+    CallPlan plan{CALL_REF_SMALL, 0, 0, 0};
+    if (cached) {
+        bool small;
+        if (int8) small = packed_small_kernel(M, N, K, true, scratch_for_split(workspace, avail, M, N));   // integer sums: any kernel, same bits
+        else small = route == ROUTE_DECODE || (route == ROUTE_AUTO && packed_small_kernel(M, N, K, false, scratch_for_split(workspace, avail, M, N)));
+        plan.kernel = small ? CALL_P2_SMALL : CALL_P2_LARGE;
+        if (!small) plan.scratch_bytes = avail;
+        return plan;
+    }
+    const bool small = int8 ? M <= 64 : (route == ROUTE_DECODE || (route == ROUTE_AUTO && M <= 64));
+    if (small) return plan;
+    const size_t p2_bytes = (static_cast<size_t>(N) * K / 4 + 255) & ~static_cast<size_t>(255);
+    if (aligned && avail >= p2_bytes) {
+        plan.kernel = CALL_TRANSCODE_LARGE;
+        plan.p2_bytes = static_cast<size_t>(N) * K / 4;
+        plan.scratch_offset = p2_bytes;
+        plan.scratch_bytes = avail - p2_bytes;
+    } else {
+        plan.kernel = CALL_REF_FUSED_LARGE;
+    }
+    return plan;
+}
+
 // ---- repack cache behind the reference-format entry points (on unless TERNASPMM_REPACK_CACHE=0).
 // An unmodified call site keeps passing the four format tensors; the first call that sees a weight (identified by
 // device, pointers and shape) allocates N*K/4 bytes, repacks into them, records a fingerprint of the source tensors
 // and waits; every later call runs the P2 kernels.  A first sight during stream capture (where nothing may be
-// allocated) is served by the reference-format kernels instead.
+// allocated) is served by the reference-format kernels instead.  The bookkeeping -- least recently used copies go
+// when a byte limit is reached, copies a captured graph may hold are never released behind its back -- is
+// repack_cache.h.
 // The pointers alone are not trusted: every launch on a cached copy recomputes the fingerprint from the tensors the
-// caller passes (an extra workgroup of the small-M launch, a one-wave launch next to a large-M one) and raises a flag
-// in host-visible memory when it differs from the recorded one -- weights freed or rewritten, other data at the same
-// addresses.  A launch cannot be taken back, so the next call into the library reports the stale copy and ends the
-// process, as every error of this library does (kernels/TernaSpMM.cu:15-22); ternaspmm_repack_cache_clear() after
-// freeing or reloading weights is what avoids it.
-struct RepackKey {
-    int device;
-    const void* bitmap;
-    const void* signs;
-    const void* offsets;
-    int n, k;
-    bool operator==(const RepackKey& o) const
-    {
-        return device == o.device && bitmap == o.bitmap && signs == o.signs && offsets == o.offsets && n == o.n && k == o.k;
-    }
-};
-struct RepackKeyHash {
-    size_t operator()(const RepackKey& key) const
-    {
-        size_t h = std::hash<const void*>()(key.bitmap);
-        h = h * 1000003u ^ std::hash<const void*>()(key.signs);
-        h = h * 1000003u ^ std::hash<const void*>()(key.offsets);
-        return h * 1000003u ^ (static_cast<size_t>(key.n) << 20) ^ static_cast<size_t>(key.k) ^ (static_cast<size_t>(key.device) << 40);
-    }
-};
-struct RepackEntry {
-    void* packed;                     // N*K/4 bytes of P2, then (256-byte aligned) the recorded fingerprint
+// caller passes (an extra workgroup of the small-M launch, a one-wave launch next to a large-M one) and, when it differs
+// from the recorded one -- weights freed or rewritten, other data at the same addresses -- reports the copy's id in
+// host-visible memory.  A launch cannot be taken back: the ONE launch that found the mismatch has used the old copy.
+// The next call into the library drops that copy, says so, and goes on (the weight gets a fresh copy at its next
+// sight); with TERNASPMM_REPACK_CACHE_STRICT=1 it ends the process instead, as every error of this library does
+// (kernels/TernaSpMM.cu:15-22).  ternaspmm_repack_cache_clear() after freeing or reloading weights avoids the window.
+struct RepackLaunch {
+    const uint32_t* packed;           // N*K/4 bytes of P2, then (256-byte aligned) the recorded fingerprint
     RepackGuard guard;                // what the launches on this copy check (passed to them by value)
 };
+constexpr uint32_t kStaleSlots = 1023;     // host-visible words 1 .. 1023: id of a stale copy at [1 + id % 1023]; word 0: any
+void release_device(void* p) { (void)hipFree(p); }     // waits for the launches that still read it
 std::mutex g_repack_mutex;
-std::unordered_map<RepackKey, RepackEntry, RepackKeyHash> g_repack_cache;
-uint32_t* g_repack_stale = nullptr;   // pinned host memory, mapped into every device: set by a guard that found a mismatch
+RepackCachePolicy<RepackLaunch> g_repack_cache(release_device, ~static_cast<size_t>(0));
+bool g_repack_limit_set = false;      // the default limit (an eighth of the device's memory) is fixed at the first copy
+uint32_t* g_repack_stale = nullptr;   // pinned host memory, mapped into every device
 int g_repack_on = -1;                 // -1: not decided yet (environment), 0 / 1
+int g_repack_strict = -1;
+uint64_t g_repack_warned = 0;
 
 bool repack_cache_on()
 {
@@ -111,69 +147,125 @@ bool repack_cache_on()
     return g_repack_on == 1;
 }
 
-void repack_cache_report_stale(int line)
+// Copies the device-side checks have reported stale since the last look: dropped here (not during stream capture:
+// releasing memory waits for the device).
+void repack_cache_collect_stale(int line)
 {
-    if (g_repack_stale != nullptr && *reinterpret_cast<volatile uint32_t*>(g_repack_stale) != 0) {
-        std::printf("TernaSpMM Error (line %d): a cached repacked weight no longer matches the tensors it was made from -- "
-                    "weights were freed or rewritten without ternaspmm_repack_cache_clear(); results since then are invalid.  "
-                    "Call ternaspmm_repack_cache_clear() after freeing or reloading weights, or set TERNASPMM_REPACK_CACHE=0.\n",
-                    line);
-        std::fflush(stdout);
-        std::exit(EXIT_FAILURE);
+    volatile uint32_t* flags = g_repack_stale;
+    if (flags == nullptr || flags[0] == 0) return;
+    flags[0] = 0;                                        // before the scan: a report that arrives meanwhile raises it again
+    for (uint32_t slot = 1; slot <= kStaleSlots; ++slot) {
+        const uint32_t id = flags[slot];
+        if (id == 0) continue;
+        flags[slot] = 0;
+        if (!g_repack_cache.retire(id)) continue;
+        if (g_repack_strict < 0) {
+            const char* v = std::getenv("TERNASPMM_REPACK_CACHE_STRICT");
+            g_repack_strict = (v != nullptr && std::atoi(v) != 0) ? 1 : 0;
+        }
+        if (g_repack_strict == 1 || g_repack_warned++ < 8) {
+            std::printf("TernaSpMM %s (line %d): a cached repacked weight no longer matched the tensors it was made from -- "
+                        "weights were freed or rewritten without ternaspmm_repack_cache_clear().  The copy was dropped; the one "
+                        "launch that found the mismatch had already used it and its output is invalid.\n",
+                        g_repack_strict == 1 ? "Error" : "Warning", line);
+            std::fflush(stdout);
+        }
+        if (g_repack_strict == 1) std::exit(EXIT_FAILURE);
     }
 }
 
-// The cached P2 copy of a weight (made on first sight) and the guard its launches carry, or NULL.
-const uint32_t* cached_packed(const Weights& w, int N, int K, hipStream_t st, RepackGuard* guard, int line)
+// The cached P2 copy of a weight (made on first sight) and the guard its launches carry; false: no copy, the
+// reference-format kernels serve the call.
+bool cached_packed(const Weights& w, int N, int K, hipStream_t st, RepackLaunch* launch, int line)
 {
     std::lock_guard<std::mutex> lock(g_repack_mutex);
-    if (!repack_cache_on()) return nullptr;
-    repack_cache_report_stale(line);
-    RepackKey key{0, w.bitmap, w.sign_words, w.tile_off, N, K};
-    if (hipGetDevice(&key.device) != hipSuccess) return nullptr;
-    const auto it = g_repack_cache.find(key);
-    if (it != g_repack_cache.end()) {
-        *guard = it->second.guard;                        // (a copy: the launch takes it by value)
-        return static_cast<const uint32_t*>(it->second.packed);
-    }
+    if (!repack_cache_on()) return false;
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(st, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+    if (hipStreamIsCapturing(st, &capturing) != hipSuccess) {
         (void)hipGetLastError();
-        return nullptr;
+        return false;
     }
+    const bool capture = capturing != hipStreamCaptureStatusNone;
+    if (!capture) repack_cache_collect_stale(line);
+    RepackKey key{0, w.bitmap, w.sign_words, w.tile_off, N, K};
+    if (hipGetDevice(&key.device) != hipSuccess) return false;
+    if (auto* slot = g_repack_cache.find(key)) {
+        if (capture) slot->pinned = true;                 // the graph being captured will hold this copy's address
+        *launch = slot->payload;                          // (a copy: the launch takes the guard by value)
+        return true;
+    }
+    if (capture) return false;
     if (g_repack_stale == nullptr) {
         void* flag = nullptr;
-        if (hipHostMalloc(&flag, 256, hipHostMallocMapped | hipHostMallocPortable) != hipSuccess) {
+        if (hipHostMalloc(&flag, (kStaleSlots + 1) * sizeof(uint32_t), hipHostMallocMapped | hipHostMallocPortable) != hipSuccess) {
             (void)hipGetLastError();
-            return nullptr;
+            return false;
         }
         g_repack_stale = static_cast<uint32_t*>(flag);
-        *g_repack_stale = 0;
+        for (uint32_t i = 0; i <= kStaleSlots; ++i) g_repack_stale[i] = 0;
+    }
+    if (!g_repack_limit_set) {
+        g_repack_limit_set = true;
+        size_t limit = 0;
+        if (const char* v = std::getenv("TERNASPMM_REPACK_CACHE_LIMIT_MB")) {
+            limit = static_cast<size_t>(std::strtoull(v, nullptr, 10)) << 20;
+        } else {
+            size_t free_b = 0, total_b = 0;
+            if (hipMemGetInfo(&free_b, &total_b) == hipSuccess) limit = total_b / 8;
+            else (void)hipGetLastError();
+        }
+        if (limit > 0) g_repack_cache.set_limit(limit);
     }
     const size_t p2_bytes = (static_cast<size_t>(N) * K / 4 + 255) & ~static_cast<size_t>(255);
+    if (!g_repack_cache.make_room(p2_bytes + 256)) return false;
     void* buf = nullptr;
     if (hipMalloc(&buf, p2_bytes + 256) != hipSuccess) {
         (void)hipGetLastError();
-        return nullptr;
+        return false;
     }
     unsigned long long* expect = reinterpret_cast<unsigned long long*>(static_cast<char*>(buf) + p2_bytes);
-    RepackGuard g{w.bitmap, w.tile_off, w.sign_words, expect, g_repack_stale, N / 64 * (K / 64), 0};
-    int total_bits = 0;                                  // the length of the sign stream decides where the check samples it
-    hipError_t e = hipMemcpyAsync(&total_bits, w.tile_off + g.tiles, sizeof(int), hipMemcpyDeviceToHost, st);
+    RepackGuard g{w.bitmap, w.tile_off, w.sign_words, expect, g_repack_stale, N / 64 * (K / 64), 0, g_repack_cache.next_id()};
+    // the length of the sign stream decides where the check samples it
+    hipError_t e = hipMemcpyAsync(&g.total_bits, w.tile_off + g.tiles, sizeof(int), hipMemcpyDeviceToHost, st);
     if (e == hipSuccess) e = hipStreamSynchronize(st);
     if (e != hipSuccess) die("repack cache", e, __LINE__);
-    g.words = total_bits >> 5;
     launch_repack(w, static_cast<uint32_t*>(buf), N, K, st);
     launch_repack_fingerprint(g, expect, st);
     e = hipStreamSynchronize(st);                        // later calls may come on other streams
     if (e != hipSuccess) die("repack cache", e, __LINE__);
-    g_repack_cache.emplace(key, RepackEntry{buf, g});
-    *guard = g;
-    return static_cast<const uint32_t*>(buf);
+    *launch = RepackLaunch{static_cast<const uint32_t*>(buf), g};
+    g_repack_cache.insert(key, buf, p2_bytes + 256, *launch);
+    return true;
+}
+
+template <typename Act>
+void run_planned(const CallPlan& plan, const Act* x, const Weights& w, const RepackLaunch& cached, uint16_t* out,
+                 const Epilogue& ep, int M, int N, int K, void* workspace, hipStream_t st)
+{
+    char* scratch = plan.scratch_bytes ? static_cast<char*>(workspace) + plan.scratch_offset : nullptr;
+    switch (plan.kernel) {
+    case CALL_P2_SMALL:
+        launch_decode_packed<Act>(x, cached.packed, out, ep, M, N, K, st, &cached.guard);
+        break;
+    case CALL_P2_LARGE:
+        launch_prefill_packed<Act>(x, cached.packed, out, ep, M, N, K, scratch, plan.scratch_bytes, st);
+        launch_repack_guard(&cached.guard, st);
+        break;
+    case CALL_REF_SMALL:
+        launch_decode<Act>(x, w, out, ep, M, N, K, st);
+        break;
+    case CALL_TRANSCODE_LARGE:
+        launch_repack(w, static_cast<uint32_t*>(workspace), N, K, st);
+        launch_prefill_packed<Act>(x, static_cast<const uint32_t*>(workspace), out, ep, M, N, K, scratch, plan.scratch_bytes, st);
+        break;
+    case CALL_REF_FUSED_LARGE:
+        launch_prefill<Act>(x, w, out, ep, M, N, K, st);
+        break;
+    }
 }
 
 void run_i8(Route route, int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* median_off, uint32_t* sign_words,
-            uint16_t* out, uint16_t* s, uint16_t* ws, int ws_num, int M, int N, int K, void* workspace,
+            uint16_t* out, uint16_t* s, uint16_t* ws, int ws_num, int M, int N, int K, int split_k, void* workspace,
             hipStream_t st, int line)
 {
     if (!shape_ok(M, N, K) || !groups_ok(ws_num) || !i8_depth_ok(K)) return;
@@ -182,39 +274,23 @@ void run_i8(Route route, int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* m
     const bool decode_rule = route == ROUTE_DECODE || (route == ROUTE_AUTO && M <= 64);
     const Epilogue ep{s, ws, nullptr, ws_num, decode_rule ? EP_I8_DECODE : EP_I8_PREFILL};
     const Weights w{bitmap, tile_off, median_off, sign_words};
-    RepackGuard guard{};
-    if (const uint32_t* p2 = cached_packed(w, N, K, st, &guard, line)) {
-        if (packed_small_kernel(M, N, K, true, workspace != nullptr)) {
-            launch_decode_packed<int8_t>(x, p2, out, ep, M, N, K, st, &guard);
-        } else {
-            launch_prefill_packed<int8_t>(x, p2, out, ep, M, N, K, workspace, workspace ? static_cast<size_t>(N) * K : 0, st);
-            launch_repack_guard(&guard, st);
-        }
-    } else if (M <= 64) launch_decode<int8_t>(x, w, out, ep, M, N, K, st);
-    else launch_large_m<int8_t>(x, w, out, ep, M, N, K, workspace, st);
+    RepackLaunch cached{};
+    const bool have = cached_packed(w, N, K, st, &cached, line);
+    run_planned<int8_t>(plan_call(true, route, M, N, K, split_k, workspace, have), x, w, cached, out, ep, M, N, K, workspace, st);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("bitlinear_TernaSpMM", e, line);
 }
 
 void run_bf16(Route route, const uint16_t* x, const uint64_t* bitmap, const int* tile_off,
               const uint16_t* median_off, const uint32_t* sign_words, uint16_t* out, const float* scale,
-              int ws_num, int M, int N, int K, void* workspace, hipStream_t st, int line)
+              int ws_num, int M, int N, int K, int split_k, void* workspace, hipStream_t st, int line)
 {
     if (!shape_ok(M, N, K) || !groups_ok(ws_num)) return;
     const Epilogue ep{nullptr, nullptr, scale, ws_num, EP_BF16};
     const Weights w{bitmap, tile_off, median_off, sign_words};
-    const bool small = route == ROUTE_DECODE || (route == ROUTE_AUTO && M <= 64);
-    RepackGuard guard{};
-    if (const uint32_t* p2 = cached_packed(w, N, K, st, &guard, line)) {
-        const bool small_p2 = route == ROUTE_DECODE || (route == ROUTE_AUTO && packed_small_kernel(M, N, K, false, workspace != nullptr));
-        if (small_p2) {
-            launch_decode_packed<uint16_t>(x, p2, out, ep, M, N, K, st, &guard);
-        } else {
-            launch_prefill_packed<uint16_t>(x, p2, out, ep, M, N, K, workspace, workspace ? static_cast<size_t>(N) * K : 0, st);
-            launch_repack_guard(&guard, st);
-        }
-    } else if (small) launch_decode<uint16_t>(x, w, out, ep, M, N, K, st);
-    else launch_large_m<uint16_t>(x, w, out, ep, M, N, K, workspace, st);
+    RepackLaunch cached{};
+    const bool have = cached_packed(w, N, K, st, &cached, line);
+    run_planned<uint16_t>(plan_call(false, route, M, N, K, split_k, workspace, have), x, w, cached, out, ep, M, N, K, workspace, st);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("bitlinear_TernaSpMM_bf16", e, line);
 }
@@ -238,25 +314,25 @@ void checkLastCudaError(int line)
 
 void bitlinear_TernaSpMM(int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* median_off, uint32_t* sign_words,
                          terna_bf16* out, terna_bf16* s, terna_bf16* ws, int ws_num, int M, int N, int K,
-                         int /*SPLIT_K*/, int32_t* workspace, terna_stream stream)
+                         int SPLIT_K, int32_t* workspace, terna_stream stream)
 {
-    run_i8(ROUTE_AUTO, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K, workspace,
+    run_i8(ROUTE_AUTO, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K, SPLIT_K, workspace,
            static_cast<hipStream_t>(stream), __LINE__);
 }
 
 void bitlinear_TernaSpMM_decode(int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* median_off,
                                 uint32_t* sign_words, terna_bf16* out, terna_bf16* s, terna_bf16* ws, int ws_num,
-                                int M, int N, int K, int /*SPLIT_K*/, int32_t* workspace, terna_stream stream)
+                                int M, int N, int K, int SPLIT_K, int32_t* workspace, terna_stream stream)
 {
-    run_i8(ROUTE_DECODE, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K, workspace,
+    run_i8(ROUTE_DECODE, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K, SPLIT_K, workspace,
            static_cast<hipStream_t>(stream), __LINE__);
 }
 
 void bitlinear_TernaSpMM_prefill(int8_t* x, uint64_t* bitmap, int* tile_off, uint16_t* median_off,
                                  uint32_t* sign_words, terna_bf16* out, terna_bf16* s, terna_bf16* ws, int ws_num,
-                                 int M, int N, int K, int /*SPLIT_K*/, int32_t* workspace, terna_stream stream)
+                                 int M, int N, int K, int SPLIT_K, int32_t* workspace, terna_stream stream)
 {
-    run_i8(ROUTE_PREFILL, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K, workspace,
+    run_i8(ROUTE_PREFILL, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K, SPLIT_K, workspace,
            static_cast<hipStream_t>(stream), __LINE__);
 }
 
@@ -267,10 +343,9 @@ void bitlinear_TernaSpMM_benchmark(int mode, int warmup_iters, int bench_iters, 
 {
     // mode 0 = auto, 1 = prefill, 2 = decode (kernels/TernaSpMM.cu:165-173)
     const Route route = mode == 1 ? ROUTE_PREFILL : (mode == 2 ? ROUTE_DECODE : ROUTE_AUTO);
-    (void)SPLIT_K;
     hipStream_t st = static_cast<hipStream_t>(stream);
     for (int it = 0; it < warmup_iters; ++it)
-        run_i8(route, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K, workspace, st, __LINE__);
+        run_i8(route, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K, SPLIT_K, workspace, st, __LINE__);
     hipError_t e = hipStreamSynchronize(st);
     if (e != hipSuccess) die("benchmark warm-up", e, __LINE__);
 
@@ -279,7 +354,7 @@ void bitlinear_TernaSpMM_benchmark(int mode, int warmup_iters, int bench_iters, 
     if ((e = hipEventCreate(&stop)) != hipSuccess) die("hipEventCreate", e, __LINE__);
     (void)hipEventRecord(start, st);
     for (int it = 0; it < bench_iters; ++it)
-        run_i8(route, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K, workspace, st, __LINE__);
+        run_i8(route, x, bitmap, tile_off, median_off, sign_words, out, s, ws, ws_num, M, N, K, SPLIT_K, workspace, st, __LINE__);
     (void)hipEventRecord(stop, st);
     if ((e = hipEventSynchronize(stop)) != hipSuccess) die("benchmark loop", e, __LINE__);
     float total_ms = 0.0f;
@@ -332,28 +407,28 @@ void gpu_sleep(double us, terna_stream stream)
 
 void bitlinear_TernaSpMM_bf16(const terna_bf16* x, const uint64_t* bitmap, const int* tile_off,
                               const uint16_t* median_off, const uint32_t* sign_words, terna_bf16* out,
-                              const float* scale, int ws_num, int M, int N, int K, int /*SPLIT_K*/,
+                              const float* scale, int ws_num, int M, int N, int K, int SPLIT_K,
                               void* workspace, terna_stream stream)
 {
-    run_bf16(ROUTE_AUTO, x, bitmap, tile_off, median_off, sign_words, out, scale, ws_num, M, N, K, workspace,
+    run_bf16(ROUTE_AUTO, x, bitmap, tile_off, median_off, sign_words, out, scale, ws_num, M, N, K, SPLIT_K, workspace,
              static_cast<hipStream_t>(stream), __LINE__);
 }
 
 void bitlinear_TernaSpMM_bf16_decode(const terna_bf16* x, const uint64_t* bitmap, const int* tile_off,
                                      const uint16_t* median_off, const uint32_t* sign_words, terna_bf16* out,
-                                     const float* scale, int ws_num, int M, int N, int K, int /*SPLIT_K*/,
+                                     const float* scale, int ws_num, int M, int N, int K, int SPLIT_K,
                                      void* workspace, terna_stream stream)
 {
-    run_bf16(ROUTE_DECODE, x, bitmap, tile_off, median_off, sign_words, out, scale, ws_num, M, N, K, workspace,
+    run_bf16(ROUTE_DECODE, x, bitmap, tile_off, median_off, sign_words, out, scale, ws_num, M, N, K, SPLIT_K, workspace,
              static_cast<hipStream_t>(stream), __LINE__);
 }
 
 void bitlinear_TernaSpMM_bf16_prefill(const terna_bf16* x, const uint64_t* bitmap, const int* tile_off,
                                       const uint16_t* median_off, const uint32_t* sign_words, terna_bf16* out,
-                                      const float* scale, int ws_num, int M, int N, int K, int /*SPLIT_K*/,
+                                      const float* scale, int ws_num, int M, int N, int K, int SPLIT_K,
                                       void* workspace, terna_stream stream)
 {
-    run_bf16(ROUTE_PREFILL, x, bitmap, tile_off, median_off, sign_words, out, scale, ws_num, M, N, K, workspace,
+    run_bf16(ROUTE_PREFILL, x, bitmap, tile_off, median_off, sign_words, out, scale, ws_num, M, N, K, SPLIT_K, workspace,
              static_cast<hipStream_t>(stream), __LINE__);
 }
 
@@ -441,8 +516,9 @@ void bitlinear_TernaSpMM_packed(const int8_t* x, const void* packed, terna_bf16*
 void ternaspmm_repack_cache_clear(void)
 {
     std::lock_guard<std::mutex> lock(g_repack_mutex);
-    for (auto& kv : g_repack_cache) (void)hipFree(kv.second.packed);      // waits for the launches that still read it
-    g_repack_cache.clear();
+    g_repack_cache.clear();                               // hipFree waits for the launches that still read a copy
+    if (g_repack_stale != nullptr)
+        for (uint32_t i = 0; i <= kStaleSlots; ++i) g_repack_stale[i] = 0;
 }
 
 int ternaspmm_repack_cache_enable(int on)
@@ -450,6 +526,53 @@ int ternaspmm_repack_cache_enable(int on)
     std::lock_guard<std::mutex> lock(g_repack_mutex);
     const int was = repack_cache_on() ? 1 : 0;
     g_repack_on = on ? 1 : 0;
+    return was;
+}
+
+long long ternaspmm_repack_cache_limit(long long bytes)
+{
+    std::lock_guard<std::mutex> lock(g_repack_mutex);
+    const size_t was = g_repack_cache.limit();
+    if (bytes >= 0) {
+        g_repack_cache.set_limit(static_cast<size_t>(bytes));
+        g_repack_limit_set = true;
+    }
+    return was > static_cast<size_t>(INT64_MAX) ? -1 : static_cast<long long>(was);
+}
+
+void ternaspmm_repack_cache_stats(long long out[6])
+{
+    std::lock_guard<std::mutex> lock(g_repack_mutex);
+    out[0] = static_cast<long long>(g_repack_cache.entries());
+    out[1] = static_cast<long long>(g_repack_cache.used());
+    out[2] = static_cast<long long>(g_repack_cache.retired());
+    out[3] = static_cast<long long>(g_repack_cache.evicted());
+    out[4] = static_cast<long long>(g_repack_cache.parked_bytes());
+    out[5] = g_repack_cache.limit() > static_cast<size_t>(INT64_MAX) ? -1 : static_cast<long long>(g_repack_cache.limit());
+}
+
+int ternaspmm_plan_reference_call(int int8_activations, int route, int M, int N, int K, int SPLIT_K, const void* workspace,
+                                  int cached, long long* workspace_bytes_used)
+{
+    if (M < 1 || N < 64 || K < 64 || (N % 64) || (K % 64) || route < 0 || route > 2) return -1;
+    const Route r = route == 1 ? ROUTE_PREFILL : (route == 2 ? ROUTE_DECODE : ROUTE_AUTO);
+    const CallPlan plan = plan_call(int8_activations != 0, r, M, N, K, SPLIT_K, workspace, cached != 0);
+    size_t used = plan.p2_bytes;
+    if (plan.kernel == CALL_P2_LARGE || plan.kernel == CALL_TRANSCODE_LARGE) {
+        const void* scratch = plan.scratch_bytes ? static_cast<const char*>(workspace) + plan.scratch_offset : nullptr;
+        const void* x_aligned = reinterpret_cast<const void*>(uintptr_t{256});          // any 16-byte aligned address: the common case
+        const PrefillPlan pp = int8_activations ? plan_prefill_packed<int8_t>(x_aligned, M, N, K, scratch, plan.scratch_bytes)
+                                                : plan_prefill_packed<uint16_t>(x_aligned, M, N, K, scratch, plan.scratch_bytes);
+        if (pp.scratch_used) used = plan.scratch_offset + pp.scratch_used;
+    }
+    if (workspace_bytes_used) *workspace_bytes_used = static_cast<long long>(used);
+    return static_cast<int>(plan.kernel);
+}
+
+int ternaspmm_quant_mode(int mode)
+{
+    const int was = quant_mode();
+    if (mode >= QUANT_ROUNDED && mode <= QUANT_EAGER) g_quant_mode.store(mode, std::memory_order_relaxed);
     return was;
 }
 

@@ -310,15 +310,33 @@ def greedy_step(logits: torch.Tensor, tok: torch.Tensor, history: Optional[torch
     return tok
 
 
-def quant_input(input: torch.Tensor):
+QUANT_ROUNDED, QUANT_COMPILED, QUANT_EAGER = 0, 1, 2
+
+
+def quant_input(input: torch.Tensor, mode: Optional[int] = None):
     """Per-row int8 quantisation of the activations (model.py:120-123): s = 127 / max(max|x|, 1e-5),
-    x_q = clamp(round(x * s), -128, 127).  One definition for the whole library, the one the norm kernels
-    compute: fp32 arithmetic, s rounded to bf16, and that rounded s both multiplies here and divides in the
-    epilogue.  (The reference's eager mode would multiply in the tensor's dtype, its compiled graph in fp32
-    with the unrounded quotient; the two differ from each other and from this by at most one step.)
+    x_q = clamp(round(x * s), -128, 127).  The reference's two lines leave the intermediate precision to PyTorch;
+    `mode` (default: the library's current ternaspmm_quant_mode, which the prologue kernels follow too) says which
+    evaluation is reproduced:
+      QUANT_ROUNDED   fp32 arithmetic, s rounded to bf16, and that rounded s both multiplies here and divides in the
+                      epilogue (the library's default);
+      QUANT_COMPILED  the method as the reference ships it, under @torch.compile: fp32 arithmetic, the UNROUNDED
+                      quotient multiplies, the returned s is its bf16 rounding;
+      QUANT_EAGER     the same lines without torch.compile on a bf16 tensor: every op rounds to bf16.
+    The three differ from each other on a few percent of the elements, by one step (two at most).
     Returns (x_q int8, s bf16 [..., 1])."""
+    if mode is None:
+        mode = _lib.load().ternaspmm_quant_mode(-1)
+    if mode == QUANT_EAGER:                       # the reference's two lines as they stand, on the bf16 tensor
+        x = input.to(torch.bfloat16)
+        s = 127 / x.abs().max(dim=-1, keepdim=True).values.clamp_(min=1e-5)
+        return (x * s).round().clamp(-128, 127).to(torch.int8), s
     x = input.float()
-    s = (127.0 / x.abs().amax(dim=-1, keepdim=True).clamp_(min=1e-5)).to(torch.bfloat16)
+    amax = x.abs().amax(dim=-1, keepdim=True).clamp_(min=1e-5)
+    if mode == QUANT_COMPILED:                    # `127 / t` is t.reciprocal() * 127; nothing is rounded to bf16 on the way
+        t = amax.reciprocal() * 127.0
+        return (x * t).round().clamp(-128, 127).to(torch.int8), t.to(torch.bfloat16)
+    s = (127.0 / amax).to(torch.bfloat16)
     return (x * s.float()).round().clamp(-128, 127).to(torch.int8), s
 
 

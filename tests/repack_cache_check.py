@@ -4,8 +4,13 @@ cache, on first sight (allocate + repack), on later sights (P2 kernels), under g
 ternaspmm_repack_cache_clear() when a different weight reuses the same device memory.
 
 With the argument `stale` (a second child process): the weight is rewritten under the same pointers WITHOUT
-ternaspmm_repack_cache_clear(); the launch that follows finds a fingerprint that no longer matches and the call
-after it must end the process with the library's message."""
+ternaspmm_repack_cache_clear(); the launch that follows finds a fingerprint that no longer matches, the call after it
+drops the copy with a warning and every call from then on serves the new weight (with TERNASPMM_REPACK_CACHE_STRICT=1
+that call ends the process with the library's message instead).  The replacement has a SHORTER sign stream than the
+original: the check must not sample past its end.
+
+With the argument `limit`: a byte limit that holds two of three weights -- the least recently used copy goes, results
+stay right, and a limit below one copy serves every call from the reference format."""
 import ctypes
 import sys
 
@@ -18,32 +23,73 @@ from tests.test_gpu_parity import WS, _check_bf16, run_bf16, run_i8
 from ternainfer_amd import _lib
 
 
+def _stats(lib):
+    out = (ctypes.c_longlong * 6)()
+    lib.ternaspmm_repack_cache_stats(out)
+    return list(out)
+
+
 def stale() -> int:
     lib = _lib.load()
     n, k = 320, 192
-    a, b = DeviceFormat(make_ternary(n, k, 0.40, 980)), DeviceFormat(make_ternary(n, k, 0.40, 981))
-    vals = torch.zeros(max(a.vals.numel(), b.vals.numel()), dtype=a.vals.dtype, device="cuda")
-    vals[: a.vals.numel()].copy_(a.vals)
-    a_vals_own, a.vals = a.vals, vals
+    # the replacement is sparser: its sign stream is shorter than the one the copy's check was set up for
+    a, b = DeviceFormat(make_ternary(n, k, 0.30, 980)), DeviceFormat(make_ternary(n, k, 0.70, 981))
+    assert b.vals.numel() < a.vals.numel()
     xq, s = make_int8_activations(8, k, 982)
     for _ in range(2):                           # first sight (copy made), cached sight
         if not (run_i8(lib, a, xq, s, WS, 1) == O.spmm_i8(xq, a.w, s, WS, 1, 0)).all():
             print("int8 mismatch before the rewrite")
-            return 0                             # 0: the parent expects a non-zero exit from the library itself
+            return 1
+    assert _stats(lib)[0] == 1
     a.bm.copy_(b.bm); a.off.copy_(b.off); a.med.copy_(b.med)
-    vals.zero_(); vals[: b.vals.numel()].copy_(b.vals)
+    a.vals.zero_(); a.vals[: b.vals.numel()].copy_(b.vals)
     torch.cuda.synchronize()
     print("[case] rewritten under the same pointers, no clear", flush=True)
-    run_i8(lib, a, xq, s, WS, 1)                 # this launch raises the flag (its result is the old weight's)
+    run_i8(lib, a, xq, s, WS, 1)                 # this launch reports the stale copy (its result is the old weight's)
     torch.cuda.synchronize()
-    run_i8(lib, a, xq, s, WS, 1)                 # ... and this call must not return
-    print("the library did not notice the stale copy")
+    want = O.spmm_i8(xq, b.w, s, WS, 1, 0)
+    for sight in range(3):                       # dropped + rebuilt (first sight again), then cached sights
+        if not (run_i8(lib, a, xq, s, WS, 1) == want).all():
+            print("the new weight is not served correctly after the stale copy was dropped", sight)
+            return 1
+    st = _stats(lib)
+    assert st[0] == 1 and st[2] == 1, st
+    print("stale copy dropped and rebuilt ok")
+    return 0
+
+
+def limit() -> int:
+    lib = _lib.load()
+    n, k = 320, 192
+    one = n * k // 4 + 256
+    assert lib.ternaspmm_repack_cache_limit(2 * one + 100) == -1
+    fmts = [DeviceFormat(make_ternary(n, k, 0.40, 990 + j)) for j in range(3)]
+    xq, s = make_int8_activations(8, k, 995)
+    for order in ([0, 1, 2], [0, 1, 2], [2, 1, 0]):
+        for j in order:
+            for _ in range(2):
+                if not (run_i8(lib, fmts[j], xq, s, WS, 1) == O.spmm_i8(xq, fmts[j].w, s, WS, 1, 0)).all():
+                    print("int8 mismatch under the byte limit", order, j)
+                    return 1
+            st = _stats(lib)
+            assert st[0] <= 2 and st[1] <= 2 * one + 100, st
+    assert _stats(lib)[3] >= 3, _stats(lib)      # copies were released at the limit
+    lib.ternaspmm_repack_cache_clear()
+    lib.ternaspmm_repack_cache_limit(one - 1)    # nothing fits: every call is served from the reference format
+    for j in range(3):
+        if not (run_i8(lib, fmts[j], xq, s, WS, 1) == O.spmm_i8(xq, fmts[j].w, s, WS, 1, 0)).all():
+            print("int8 mismatch without room for a copy", j)
+            return 1
+    assert _stats(lib)[0] == 0
+    print("cache limit check ok")
     return 0
 
 
 def main() -> int:
     if len(sys.argv) > 1 and sys.argv[1] == "stale":
         return stale()
+    if len(sys.argv) > 1 and sys.argv[1] == "limit":
+        return limit()
     lib = _lib.load()
     co = O.COracle()
     n, k = 320, 192

@@ -29,9 +29,26 @@ def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
+_CANARY = 1 << 20
+
+
+class _Workspace:
+    """Exactly the bytes the reference itself would write for this call -- SPLIT_K int32 planes of M x N on its decode
+    path (tests/test_kernel.cu:331), a dense int8 N x K matrix on its prefill path (model.py:34-42) -- followed by a
+    canary region that must come back untouched."""
+
+    def __init__(self, entry, m, n, k, split_k):
+        prefill_path = entry.endswith("_prefill") or (not entry.endswith("_decode") and m > 64)
+        self.bytes = n * k if prefill_path else 4 * m * n * split_k
+        self.buf = torch.full((self.bytes + _CANARY,), 0x5A, dtype=torch.int8, device="cuda")
+
+    def check(self):
+        assert bool((self.buf[self.bytes:] == 0x5A).all()), "the call wrote past the workspace the reference guarantees"
+
+
 def _workspace(m, n, k):
-    """What the reference's call site guarantees (model.py:34-42): room for 7 int32 split-K partials
-    and for N*K bytes.  The large-M path transcodes the weights into its first N*K/4 bytes."""
+    """Room for both of the reference's uses of its workspace (model.py:34-42): callers that do not go through run_i8 /
+    run_bf16."""
     return torch.empty(max(4 * m * n * 7, n * k) + 256, dtype=torch.int8, device="cuda")
 
 
@@ -41,24 +58,28 @@ def run_i8(lib, fmt, xq, s_bits, ws_bits, ws_num, entry="bitlinear_TernaSpMM", w
     s = torch.from_numpy(s_bits.view(np.int16)).cuda()
     ws = torch.from_numpy(ws_bits.view(np.int16)).cuda()
     out = torch.full((m, fmt.n), -1, dtype=torch.int16, device="cuda")      # poison: must be overwritten
-    work = _workspace(m, fmt.n, k) if workspace else None
+    work = _Workspace(entry, m, fmt.n, k, 7) if workspace else None
     print(f"[case] {entry} M={m} N={fmt.n} K={k} ws_num={ws_num} workspace={workspace}", flush=True)
     getattr(lib, entry)(vp(x), vp(fmt.bm), vp(fmt.off), vp(fmt.med), vp(fmt.vals), vp(out), vp(s), vp(ws),
-                        ws_num, m, fmt.n, k, 7, vp(work) if workspace else None, _stream())
+                        ws_num, m, fmt.n, k, 7, vp(work.buf) if workspace else None, _stream())
     torch.cuda.synchronize()
+    if workspace:
+        work.check()
     return out.cpu().numpy().view(np.uint16)
 
 
-def run_bf16(lib, fmt, x_bits, scale, ws_num, entry="bitlinear_TernaSpMM_bf16", workspace=False):
+def run_bf16(lib, fmt, x_bits, scale, ws_num, entry="bitlinear_TernaSpMM_bf16", workspace=False, split_k=1):
     m, k = x_bits.shape
     x = torch.from_numpy(x_bits.view(np.int16)).cuda()
     sc = torch.from_numpy(scale).cuda()
     out = torch.full((m, fmt.n), -1, dtype=torch.int16, device="cuda")
-    work = _workspace(m, fmt.n, k) if workspace else None
+    work = _Workspace(entry, m, fmt.n, k, split_k) if workspace else None
     print(f"[case] {entry} M={m} N={fmt.n} K={k} ws_num={ws_num} workspace={workspace}", flush=True)
     getattr(lib, entry)(vp(x), vp(fmt.bm), vp(fmt.off), vp(fmt.med), vp(fmt.vals), vp(out), vp(sc), ws_num,
-                        m, fmt.n, k, 1, vp(work) if workspace else None, _stream())
+                        m, fmt.n, k, split_k, vp(work.buf) if workspace else None, _stream())
     torch.cuda.synchronize()
+    if workspace:
+        work.check()
     return out.cpu().numpy().view(np.uint16)
 
 
@@ -697,11 +718,22 @@ def test_repack_cache_behind_reference_entry_points():
     r = subprocess.run([sys.executable, "-u", "-m", "tests.repack_cache_check"], cwd=root,
                        env={**os.environ, "TERNASPMM_REPACK_CACHE": "1"}, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0 and "repack cache check ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
-    # a weight rewritten under the same pointers without ternaspmm_repack_cache_clear(): the library ends the process
+    # a weight rewritten under the same pointers without ternaspmm_repack_cache_clear(): the launch that follows reports
+    # the stale copy, the next call drops it with a warning and serves the new weight correctly ...
     r = subprocess.run([sys.executable, "-u", "-m", "tests.repack_cache_check", "stale"], cwd=root,
                        env={**os.environ, "TERNASPMM_REPACK_CACHE": "1"}, capture_output=True, text=True, timeout=300)
-    assert r.returncode != 0 and "no longer matches the tensors it was made from" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
-    assert "did not notice" not in r.stdout
+    assert r.returncode == 0 and "stale copy dropped and rebuilt ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+    assert "no longer matched the tensors it was made from" in r.stdout and "Warning" in r.stdout
+    # ... or, with TERNASPMM_REPACK_CACHE_STRICT=1, ends the process as every error of the library does
+    r = subprocess.run([sys.executable, "-u", "-m", "tests.repack_cache_check", "stale"], cwd=root,
+                       env={**os.environ, "TERNASPMM_REPACK_CACHE": "1", "TERNASPMM_REPACK_CACHE_STRICT": "1"},
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode != 0 and "no longer matched the tensors it was made from" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+    assert "stale copy dropped" not in r.stdout
+    # the byte limit: least recently used copies go, a weight that does not fit is served without a copy
+    r = subprocess.run([sys.executable, "-u", "-m", "tests.repack_cache_check", "limit"], cwd=root,
+                       env={**os.environ, "TERNASPMM_REPACK_CACHE": "1"}, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "cache limit check ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
 
 
 def test_benchmark_entry_point_times_and_leaves_the_result(lib, capfd):

@@ -373,6 +373,57 @@ def test_fused_prologue_linear(lib, m, n, k, ws_num, res):
     assert torch.equal(od, od2)
 
 
+@pytest.mark.parametrize("mode", [O.QUANT_COMPILED, O.QUANT_EAGER])
+def test_quant_modes_of_the_prologue_kernels(lib, mode):
+    """ternaspmm_quant_mode: the reference's other evaluations of quant_input (model.py:120-123; the @torch.compile'd
+    method as shipped, and eager mode on bf16 tensors).  The norm kernels' (q, s) must be the oracle's for that mode
+    on the kernel's own norm output, bit for bit; the fused linear's must be that mode's for a norm output within one
+    bf16 step, with the matmul on them bit-exact; and the mode must really change the integers."""
+    from tests._util import DeviceFormat, make_ternary
+    assert lib.ternaspmm_quant_mode(-1) == O.QUANT_ROUNDED
+    x = make_bf16_activations(37, 2560, 640, outlier_frac=0.01)
+    x13 = make_bf16_activations(9, 2 * 6912, 641, outlier_frac=0.01)
+    w, wf = _weight(2560, 642), _weight(6912, 643)
+    _, _, q0, _ = _run(lib, x, w, 1e-5)
+    n, k, m = 2560, 2560, 8
+    wt = make_ternary(n, k, 0.40, 644)
+    fmt = DeviceFormat(wt)
+    packed = torch.empty(n * k // 16, dtype=torch.int32, device="cuda")
+    lib.ternaspmm_repack(_vp(fmt.bm), _vp(fmt.off), _vp(fmt.med), _vp(fmt.vals), _vp(packed), n, k, None)
+    ws = O.f32_to_bf16_bits(np.array([1.25, 0.0, 0.0, 0.0], np.float32))
+    assert lib.ternaspmm_quant_mode(mode) == O.QUANT_ROUNDED
+    try:
+        print(f"[case] quant mode {mode}: norm kernels", flush=True)
+        _, y, q, s = _run(lib, x, w, 1e-5)
+        want_q, want_s = O.quant_input(y, mode)
+        assert (s == want_s).all() and (q == want_q).all()
+        assert 0.005 < (q != q0).mean() < 0.2                       # not the default rule's integers
+        _, y, q, s = _run(lib, x13, wf, 1e-5, glu=True)
+        want_q, want_s = O.quant_input(y, mode)
+        assert (s == want_s).all() and (q == want_q).all()
+        for mm in (1, m):
+            print(f"[case] quant mode {mode}: fused prologue linear m={mm}", flush=True)
+            xs = x[:mm]
+            xd, gd, wsd = _dev(xs), _dev(w), _dev(ws)
+            od = torch.zeros((mm, n), dtype=torch.int16, device="cuda")
+            qd = torch.zeros((mm, k), dtype=torch.int8, device="cuda")
+            sd = torch.zeros(mm, dtype=torch.int16, device="cuda")
+            assert lib.bitlinear_TernaSpMM_packed_fused(_vp(xd), None, None, _vp(gd), 1e-5, _vp(packed), _vp(od), _vp(wsd), 1,
+                                                        _vp(qd), _vp(sd), mm, n, k, None) == 1
+            torch.cuda.synchronize()
+            qk, sk = qd.cpu().numpy(), sd.cpu().numpy().view(np.uint16)
+            q_ref, s_ref = O.quant_input(O.rmsnorm(xs, w, 1e-5), mode)
+            assert np.abs(_bf16_key(sk) - _bf16_key(s_ref)).max() <= 1
+            same_s = sk == s_ref                                     # rows whose scale agrees: the integers may differ only where y does
+            dq = np.abs(qk.astype(np.int32) - q_ref.astype(np.int32))[same_s]
+            assert dq.size and dq.max() <= 1 and (dq != 0).mean() < 0.02
+            assert (od.cpu().numpy().view(np.uint16) == O.spmm_i8(qk, wt, sk, ws, 1, 0)).all()
+    finally:
+        lib.ternaspmm_quant_mode(O.QUANT_ROUNDED)
+    _, _, q1, _ = _run(lib, x, w, 1e-5)
+    assert (q1 == q0).all()
+
+
 def test_fused_prologue_linear_declines_what_it_cannot_do(lib):
     z = torch.zeros(64, dtype=torch.int32, device="cuda")
     for m, n, k in [(17, 256, 192), (8, 2560, 6912), (8, 13824, 3136)]:

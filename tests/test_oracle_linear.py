@@ -114,36 +114,95 @@ def _row(values, width=16):
     return bits
 
 
-# Known answers of quant_input (model.py:120-123) worked by hand.  The definition this build fixes:
-# s = bf16(127 / max(max|x|, 1e-5)); q = clamp(round_half_even(fp32(x * s)), -128, 127), with the
-# ROUNDED s used in the product.  Each row is chosen so that one plausible mistake fails it.
+# Known answers of quant_input (model.py:120-123) worked by hand, for the three evaluations the reference's two lines
+# admit (oracle: quant_input(x, mode)):
+#   rounded  (this build's default) s = bf16(127 / max(max|x|, 1e-5)); q = clamp(round_half_even(fp32(x * s))), with
+#            the ROUNDED s in the product;
+#   compiled (the method as shipped, under @torch.compile) fp32 throughout: `127 / t` on a tensor is t.reciprocal() * 127,
+#            so the multiplier is fl32(fl32(1 / max) * 127), UNROUNDED; s = its bf16;
+#   eager    (no torch.compile, bf16 tensor) every op rounded to bf16: s = bf16(bf16(1 / max) * 127), product bf16(x * s).
+# Each row is chosen so that one plausible mistake fails it.
+# (values, s, q rounded, q compiled, q eager[, s eager]); None = as rounded.
 QUANT_INPUT_KAT = [
     # max|x| = 127 -> s = 1 exactly, q = round_half_even(x): floor(x + 0.5) or round-half-away fails
     ([127.0, 0.5, 1.5, 2.5, -2.5, -0.5, 100.5, 101.5, -126.5, 3.5, -1.5],
-     1.0, [127, 0, 2, 2, -2, 0, 100, 102, -126, 4, -2]),
+     1.0, [127, 0, 2, 2, -2, 0, 100, 102, -126, 4, -2], None, None),
     # max|x| = 1 -> s = 127 (exact in bf16); 0.5 * 127 = 63.5 is a tie -> 64 (even), -63.5 -> -64
     ([1.0, -1.0, 0.5, -0.5, 0.25, 0.0078125, 0.00390625],
-     127.0, [127, -127, 64, -64, 32, 1, 0]),                    # 31.75 -> 32, 0.992 -> 1, 0.496 -> 0
+     127.0, [127, -127, 64, -64, 32, 1, 0], None, None),        # 31.75 -> 32, 0.992 -> 1, 0.496 -> 0
     # max|x| = 0.5 -> s = 254 (exact); max|x| = 4 -> s = 31.75 (exact): a missing or inverted scale fails
-    ([0.5, -0.25, 0.125], 254.0, [127, -64, 32]),               # -63.5 -> -64, 31.75 -> 32
-    ([4.0, 2.0, -1.0, 0.0625], 31.75, [127, 64, -32, 2]),       # 63.5 -> 64, -31.75 -> -32, 1.984 -> 2
-    # max|x| = 129/128: 127 / 1.0078125 = 126.0155 rounds DOWN to s = 126 in bf16.  With the rounded s
-    # 0.75 * 126 = 94.5 is a tie -> 94 and (129/256) * 126 = 63.49 -> 63; the unrounded s would give
-    # 94.51 -> 95 and 63.5 -> 64: a quantiser that multiplies by the fp32 quotient fails here
-    ([1.0078125, 0.75, 0.50390625, -0.75], 126.0, [127, 94, 63, -94]),
+    ([0.5, -0.25, 0.125], 254.0, [127, -64, 32], None, None),   # -63.5 -> -64, 31.75 -> 32
+    ([4.0, 2.0, -1.0, 0.0625], 31.75, [127, 64, -32, 2], None, None),   # 63.5 -> 64, -31.75 -> -32, 1.984 -> 2
+    # max|x| = 129/128: 127 / (129/128) = 16256/129 = 126.01550..., s = 126 in bf16 (rounds DOWN).
+    #   rounded : 0.75 * 126 = 94.5, a tie -> 94;  (129/256) * 126 = 63.49 -> 63
+    #   compiled: fl32(128/129) = 2080895/2097152, times 127 -> t = 1032319/8192 = 126.0155029 (just below 16256/129);
+    #             0.75 * t = 94.5116 -> 95;  (129/256) * t = 63.4999995, which is nearer to 63.5 than to the fp32
+    #             number below it (63.5 - 2^-18) -> the fp32 product IS 63.5, a tie -> 64.  (An implementation that
+    #             keeps the product in double gets 63.)
+    #   eager   : bf16(128/129) = 0.9921875, times 127 = 126.008 -> s = 126; 0.75 * 126 = 94.5 is exact in bf16 -> 94;
+    #             63.49 rounds to 63.5 in bf16 (step 0.25) -> 64
+    ([1.0078125, 0.75, 0.50390625, -0.75], 126.0, [127, 94, 63, -94], [127, 95, 64, -95], [127, 94, 64, -94]),
     # max|x| = 255/128: 127 / 1.9921875 = 63.749 rounds UP to s = 63.75; max|x| * s = 127.002 -> 127:
-    # the rounding of s can overshoot 127 by at most 127 * 2^-8 < 0.5, so the clamp never bites
-    ([1.9921875, -1.9921875, 1.0], 63.75, [127, -127, 64]),
+    # the rounding of s can overshoot 127 by at most 127 * 2^-8 < 0.5, so the clamp never bites -- in fp32.  Eager mode
+    # rounds the reciprocal first: 1 / 1.9921875 = 0.50196 -> bf16 0.50390625 (the upper neighbour, by 2e-5), times 127 =
+    # 63.996 -> s = 64; then 1.9921875 * 64 = 127.5 exactly, a tie -> 128 -> clamped to 127, and -127.5 -> -128 stays
+    ([1.9921875, -1.9921875, 1.0], 63.75, [127, -127, 64], None, [127, -128, 64], 64.0),
+    # max|x| = 1 -> s = 127; x = 135/512: x * s = 33.486 -> 33 in fp32, but bf16 (step 0.25 between 32 and 64) rounds the
+    # product to 33.5 first, a tie -> 34: only the eager evaluation rounds the product
+    ([1.0, 0.263671875], 127.0, [127, 33], None, [127, 34]),
 ]
+KAT_MODES = [(O.QUANT_ROUNDED, 2), (O.QUANT_COMPILED, 3), (O.QUANT_EAGER, 4)]
 
 
-@pytest.mark.parametrize("values,s_want,q_want", QUANT_INPUT_KAT)
-def test_quant_input_known_answers(coracle, values, s_want, q_want):
+@pytest.mark.parametrize("row", QUANT_INPUT_KAT)
+def test_quant_input_known_answers(coracle, row):
+    values, s_want = row[0], row[1]
     x = _row(values).reshape(1, -1)
-    for impl in (O.quant_input, coracle.quant_input):
-        q, s = impl(x)
-        assert O.bf16_bits_to_f32(s).tolist() == [s_want]
-        assert q[0, :len(q_want)].tolist() == q_want and not q[0, len(q_want):].any()
+    for mode, col in KAT_MODES:
+        q_want = row[col] if row[col] is not None else row[2]
+        s_want = row[5] if mode == O.QUANT_EAGER and len(row) > 5 else row[1]
+        for impl in (O.quant_input, coracle.quant_input):
+            q, s = impl(x, mode)
+            assert O.bf16_bits_to_f32(s).tolist() == [s_want]
+            assert q[0, :len(q_want)].tolist() == q_want and not q[0, len(q_want):].any(), (mode, q[0].tolist())
+    assert (O.quant_input(x)[0] == O.quant_input(x, O.QUANT_ROUNDED)[0]).all()      # the default is the rounded rule
+
+
+def test_quant_input_call_site_function_known_answers():
+    """ternainfer_amd.linear.quant_input -- what SpBitLinear / BF16BitLinear of this build call, written with torch ops
+    as the reference's method is -- on the same rows, in the three modes (CPU tensors)."""
+    import torch
+    from ternainfer_amd import linear as L
+    for row in QUANT_INPUT_KAT:
+        x = torch.from_numpy(O.bf16_bits_to_f32(_row(row[0]).reshape(1, -1))).to(torch.bfloat16)
+        for mode, col in KAT_MODES:
+            q_want = row[col] if row[col] is not None else row[2]
+            s_want = row[5] if mode == O.QUANT_EAGER and len(row) > 5 else row[1]
+            q, s = L.quant_input(x, mode)
+            assert q.dtype == torch.int8 and s.dtype == torch.bfloat16 and s.shape == (1, 1)
+            assert float(s) == s_want and q[0, :len(q_want)].tolist() == q_want, (mode, q[0].tolist())
+
+
+def test_quant_input_modes_on_random_rows(coracle):
+    """The three evaluations agree with each other on most elements and never differ by more than two steps; the two
+    restatements agree bit for bit in every mode; and the torch statement of the reference's own two lines, run
+    eagerly on the bf16 tensor, IS the eager mode."""
+    import torch
+    x = make_bf16_activations(16, 2560, 77)
+    got = {}
+    for mode, _ in KAT_MODES:
+        q1, s1 = O.quant_input(x, mode)
+        q2, s2 = coracle.quant_input(x, mode)
+        assert (q1 == q2).all() and (s1 == s2).all()
+        got[mode] = q1.astype(np.int32)
+    for a in got:
+        for b in got:
+            d = np.abs(got[a] - got[b])
+            assert d.max() <= 2 and (a == b or 0.01 < (d != 0).mean() < 0.15), (a, b, d.max(), (d != 0).mean())
+    xt = torch.from_numpy(O.bf16_bits_to_f32(x)).to(torch.bfloat16)
+    s = 127 / xt.abs().max(dim=-1, keepdim=True).values.clamp_(min=1e-5)            # model.py:122-123, verbatim semantics
+    q = (xt * s).round().clamp(-128, 127).to(torch.int8)
+    assert (q.numpy() == got[O.QUANT_EAGER]).all()
 
 
 def test_quant_input_all_zero_row(coracle):
@@ -159,12 +218,12 @@ def test_quant_input_all_zero_row(coracle):
 def test_quant_input_rows_are_independent(coracle):
     """The scale is per row (dim=-1, keepdim): stacking KAT rows must not change any of them."""
     width = 16
-    x = np.stack([_row(v, width) for v, _, _ in QUANT_INPUT_KAT])
+    x = np.stack([_row(row[0], width) for row in QUANT_INPUT_KAT])
     for impl in (O.quant_input, coracle.quant_input):
         q, s = impl(x)
-        assert O.bf16_bits_to_f32(s).tolist() == [sw for _, sw, _ in QUANT_INPUT_KAT]
-        for r, (_, _, qw) in enumerate(QUANT_INPUT_KAT):
-            assert q[r, :len(qw)].tolist() == qw
+        assert O.bf16_bits_to_f32(s).tolist() == [row[1] for row in QUANT_INPUT_KAT]
+        for r, row in enumerate(QUANT_INPUT_KAT):
+            assert q[r, :len(row[2])].tolist() == row[2]
 
 
 # Known answers of quant_weight_int8 (convert_TernaInfer.py:159-163): s = 1 / max(mean|W|, 1e-5),
