@@ -319,3 +319,86 @@ def test_rope_and_attention_closed_forms():
     v2 = make_bf16_activations(5, 64, 85).reshape(1, 1, 5, 64)
     assert np.allclose(O.attention_one_token(q2, k2, v2, 5, 1.0)[0, 0], O.bf16_bits_to_f32(v2[0, 0, 3]), atol=1e-9)
     assert not np.allclose(O.attention_one_token(q2, k2, v2, 3, 1.0)[0, 0], O.bf16_bits_to_f32(v2[0, 0, 3]), atol=1e-3)
+
+
+# ------------------------------------------------------------------ the glue functions against library routines
+def test_attention_against_torch_sdpa():
+    """attention_one_token / attention_new_tokens against torch.nn.functional.scaled_dot_product_attention in float64,
+    at the 2B head layout (20 query heads on 5 kv heads, head size 128) with a scale that is not the default and
+    values that differ per kv head: a wrong softmax scale, a wrong head -> kv-head mapping (h % KV instead of
+    h // (H / KV)) or an off-by-one in the causal prefix each fail here."""
+    import torch
+    from torch.nn import functional as F
+    b, h, kv, d, s_max, n = 2, 20, 5, 128, 48, 37
+    scale = 0.0713
+    q = make_bf16_activations(b * h, d, 301).reshape(b, h, d)
+    k = make_bf16_activations(b * kv * s_max, d, 302).reshape(b, kv, s_max, d)
+    v = make_bf16_activations(b * kv * s_max, d, 303).reshape(b, kv, s_max, d)
+    t64 = lambda a: torch.from_numpy(O.bf16_bits_to_f32(a).astype(np.float64))
+    rep = h // kv
+    kk, vv = t64(k)[:, :, :n].repeat_interleave(rep, dim=1), t64(v)[:, :, :n].repeat_interleave(rep, dim=1)
+    want = F.scaled_dot_product_attention(t64(q)[:, :, None], kk, vv, scale=scale)[:, :, 0].numpy()
+    got = O.attention_one_token(q, k, v, n, scale)
+    assert np.abs(got - want).max() < 1e-12
+    wrong_scale = F.scaled_dot_product_attention(t64(q)[:, :, None], kk, vv)[:, :, 0].numpy()      # d ** -0.5
+    assert np.abs(got - wrong_scale).max() > 1e-2
+    kk_mod = t64(k)[:, :, :n].repeat(1, rep, 1, 1)                                                  # head h -> kv head h % KV
+    vv_mod = t64(v)[:, :, :n].repeat(1, rep, 1, 1)
+    wrong_map = F.scaled_dot_product_attention(t64(q)[:, :, None], kk_mod, vv_mod, scale=scale)[:, :, 0].numpy()
+    assert np.abs(got - wrong_map).max() > 1e-2
+
+    # several new tokens at slots first .. first + T - 1 of a cache that already holds `first` rows
+    t_new, first = 9, 20
+    qn = make_bf16_activations(b * h * t_new, d, 304).reshape(b, h, t_new, d)
+    pos = np.arange(first, first + t_new)
+    seen = torch.arange(s_max)[None, :] <= torch.from_numpy(pos)[:, None]                          # [T, S]
+    kk, vv = t64(k).repeat_interleave(rep, dim=1), t64(v).repeat_interleave(rep, dim=1)
+    want = F.scaled_dot_product_attention(t64(qn), kk, vv, attn_mask=seen[None, None], scale=scale).transpose(1, 2).numpy()
+    got = O.attention_new_tokens(qn, k, v, pos, scale)                                             # [B, T, H, D]
+    assert got.shape == want.shape and np.abs(got - want).max() < 1e-12
+    off_by_one = torch.arange(s_max)[None, :] < torch.from_numpy(pos)[:, None]
+    wrong = F.scaled_dot_product_attention(t64(qn), kk, vv, attn_mask=off_by_one[None, None], scale=scale).transpose(1, 2).numpy()
+    assert np.abs(got - wrong).max() > 1e-2
+
+
+def test_rmsnorm_against_torch_rms_norm():
+    """rmsnorm against torch.nn.functional.rms_norm evaluated in float64 and rounded once to bf16: identical bits."""
+    import torch
+    from torch.nn import functional as F
+    x = make_bf16_activations(7, 2560, 311, outlier_frac=0.01)
+    w = O.f32_to_bf16_bits(np.random.default_rng(312).uniform(0.5, 1.5, 2560).astype(np.float32))
+    for eps in (1e-5, 1e-2):
+        ref = F.rms_norm(torch.from_numpy(O.bf16_bits_to_f32(x).astype(np.float64)), (2560,),
+                         torch.from_numpy(O.bf16_bits_to_f32(w).astype(np.float64)), eps)
+        want = O.f32_to_bf16_bits(ref.numpy().astype(np.float32))
+        assert (O.rmsnorm(x, w, eps) == want).all()
+    assert (O.rmsnorm(x, w, 1e-5) != O.rmsnorm(x, w, 1e-2)).any()          # eps takes part
+
+
+def test_rope_against_complex_multiplication():
+    """Both pairings are the complex product (x1 + i x2) * exp(i angle) per pair, rounded once to bf16: compared with
+    numpy's complex128 product (the oracle's fp32 products and sums stay within one bf16 step of it, and agree on
+    all but a sliver of the elements); a conjugated angle or swapped cos / sin fails by far more."""
+    rng = np.random.default_rng(321)
+    x = make_bf16_activations(6, 128, 322)
+    ang = rng.uniform(-np.pi, np.pi, (6, 64))
+    cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    xf = O.bf16_bits_to_f32(x).astype(np.float64)
+    rot = np.exp(1j * np.arctan2(sin.astype(np.float64), cos.astype(np.float64)))
+
+    def key(bits):
+        bits = bits.astype(np.int32)
+        return np.where(bits & 0x8000, -(bits & 0x7FFF), bits & 0x7FFF)
+
+    z = (xf[:, 0::2] + 1j * xf[:, 1::2]) * rot
+    want = np.empty_like(xf)
+    want[:, 0::2], want[:, 1::2] = z.real, z.imag
+    d = np.abs(key(O.rope_adjacent(x, cos, sin)) - key(O.f32_to_bf16_bits(want.astype(np.float32))))
+    assert d.max() <= 1 and (d != 0).mean() < 0.01
+    conj = np.abs(key(O.rope_adjacent(x, cos, -sin)) - key(O.f32_to_bf16_bits(want.astype(np.float32))))
+    swapped = np.abs(key(O.rope_adjacent(x, sin, cos)) - key(O.f32_to_bf16_bits(want.astype(np.float32))))
+    assert conj.max() > 64 and swapped.max() > 64
+    z = (xf[:, :64] + 1j * xf[:, 64:]) * rot
+    want = np.concatenate([z.real, z.imag], axis=-1)
+    d = np.abs(key(O.rope_rotate_half(x, cos, sin)) - key(O.f32_to_bf16_bits(want.astype(np.float32))))
+    assert d.max() <= 1 and (d != 0).mean() < 0.01
