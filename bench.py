@@ -209,7 +209,7 @@ def cpu_baseline(mats, torch):
 
 
 # ------------------------------------------------------------------------------------------------ model (configs[4])
-def measure_model(torch, batch, act="int8", prefetch=True, gen_tokens=256, check_tokens=8, model=None, prompt_tokens=128):
+def measure_model(torch, batch, act="int8", prefetch=True, gen_tokens=256, check_tokens=8, model=None, prompt_tokens=128, chain=True):
     """2B-shaped random-init model, prompt of `prompt_tokens` (128) uniform random ids, greedy decode of `gen_tokens`
     tokens; tokens/s = generated tokens / decode-phase time (as the reference's stats.py:19-27).
     Self-check of the run: the captured decode graph must produce the tokens of eager execution
@@ -219,6 +219,7 @@ def measure_model(torch, batch, act="int8", prefetch=True, gen_tokens=256, check
     t0 = time.perf_counter()
     if model is None:
         model = Transformer(margs, seed=20260500, act=act)
+    model.chain = chain
     model.enable_prefetch(False)
     if prefetch:     # weights of the following launches, pulled through the caches during the attention launch
         model.enable_prefetch(True, ("wo", "w13", "w2", "next_wqkv", "norms") if batch <= 2 else ("wo", "w13", "norms"))
@@ -242,7 +243,8 @@ def measure_model(torch, batch, act="int8", prefetch=True, gen_tokens=256, check
 def run_model(args, torch):
     act = args.act or "int8"
     gen = 256 if args.prompt_tokens <= 128 else 128
-    fig, _ = measure_model(torch, args.batch, act, not args.no_prefetch, gen_tokens=gen, prompt_tokens=args.prompt_tokens)
+    fig, _ = measure_model(torch, args.batch, act, not args.no_prefetch, gen_tokens=gen, prompt_tokens=args.prompt_tokens,
+                           chain=not args.no_chain)
     return {
         "metric": "2B-shape decode tok/s", "value": fig["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": gen, "warmup": 8,
         "ms_per_step": fig["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -623,6 +625,8 @@ def main():
                          "reference: kernels read the reference's compressed format directly")
     ap.add_argument("--no-prefetch", action="store_true",
                     help="model workload: no weight prefetch by the idle CUs of the attention launch")
+    ap.add_argument("--no-chain", action="store_true",
+                    help="model workload: the decode step without producer-side norm statistics (every linear re-derives them)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-per-shape", action="store_true")
     ap.add_argument("--no-extras", action="store_true",

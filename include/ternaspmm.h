@@ -246,6 +246,68 @@ int bitlinear_TernaSpMM_packed_fused_glu(const terna_bf16* x13, const terna_bf16
                                          const void* packed, terna_bf16* out, const terna_bf16* ws, int ws_num,
                                          int8_t* xq_out, terna_bf16* s_out, int M, int N, int F, terna_stream stream);
 
+/* ---- Chained small-M linears: producer-side norm statistics (no counterpart in the reference's library) ----------
+ * The prologue above re-derives, in every workgroup, the two row statistics of the norm and of quant_input -- the sum
+ * of h^2 and max |y| -- with two workgroup-wide reductions over K.  In a decode step the launch that PRODUCES h can
+ * leave them instead: per row and per 16 (or more) columns a partial (sum of h^2, max |h * w|), w = the weights of
+ * the norm that will read h (both are exact: products of two bf16 values).  The consumer adds / maximises the partials
+ * of a row in a fixed order and continues element-wise:
+ *     rstd = rsqrt(sum / K + eps);   y = bf16((h * w) * rstd);   max |y| = bf16(max|h * w| * rstd)   (exactly)
+ * then s and xq as in ternaspmm_rmsnorm_quant (ternaspmm_quant_mode applies).  The norm output stays within one bf16
+ * step of the float64 evaluation; (xq, s) can be published as before and the matmul on them is exact.
+ *
+ * ternaspmm_fused_linear: one launch = prologue -> ternary matmul on a P2 weight -> epilogue, M <= 8 rows.
+ *   prologue  TERNASPMM_PROLOGUE_NORM       x = h bf16 [M][K]; statistics taken inside (as bitlinear_TernaSpMM_packed_fused)
+ *             TERNASPMM_PROLOGUE_ATTENTION  x = the partial results of ternaspmm_rope_decode_attention_partial
+ *                                           (attention_splits, head_dim; M = 1), merged inside, statistics taken inside
+ *             TERNASPMM_PROLOGUE_STATS      x = h bf16 [M][K] with its partials stats_in fp32 [M][stats_count][2]
+ *                                           (stats_count <= 448), as a producing epilogue or ternaspmm_row_stats left them
+ *   epilogue  TERNASPMM_EPILOGUE_STORE      out bf16 [M][N] = the linear's output (decode rule, Reduction_Kernel.cuh:60)
+ *             TERNASPMM_EPILOGUE_RESIDUAL   out bf16 [M][N] = bf16(residual + output): the residual stream after this
+ *                                           linear (model.py:330, :334); stats_out fp32 [M][N/16][2] = its partials under
+ *                                           next_norm_weight (bf16 [N]); raw_out (optional) also receives the output itself
+ *             TERNASPMM_EPILOGUE_GATE       `packed` is a gate+up matrix whose bands were interleaved by
+ *                                           ternaspmm_interleave_gate_up, ws = [scale of w1, scale of w3] (ws_num = 2);
+ *                                           out bf16 [M][N/2] = bf16(bf16(relu(x1)^2) * x3) (model.py:279-280);
+ *                                           stats_out fp32 [M][N/32][2] under next_norm_weight (bf16 [N/2], ffn_sub_norm)
+ * Returns the number of partials per row written to stats_out (0 for TERNASPMM_EPILOGUE_STORE), or -1 when the
+ * combination or the shape is not supported and nothing was enqueued (supported: K <= 2560 for every combination,
+ * K <= 7168 for TERNASPMM_PROLOGUE_STATS with STORE / RESIDUAL; GATE needs PROLOGUE_STATS; PROLOGUE_NORM here only with
+ * EPILOGUE_RESIDUAL).  out must not alias x or residual.  Only enqueues. */
+enum { TERNASPMM_PROLOGUE_NORM = 0, TERNASPMM_PROLOGUE_ATTENTION = 1, TERNASPMM_PROLOGUE_STATS = 2 };
+enum { TERNASPMM_EPILOGUE_STORE = 0, TERNASPMM_EPILOGUE_RESIDUAL = 1, TERNASPMM_EPILOGUE_GATE = 2 };
+typedef struct ternaspmm_fused_linear_desc {
+    int prologue, epilogue;
+    int M, N, K;
+    int ws_num;
+    float eps;
+    int stats_count;                  /* PROLOGUE_STATS */
+    int attention_splits, head_dim;   /* PROLOGUE_ATTENTION */
+    const void* x;
+    const float* stats_in;
+    const terna_bf16* norm_weight;    /* bf16 [K] */
+    const void* packed;
+    const terna_bf16* ws;
+    terna_bf16* out;
+    const terna_bf16* residual;       /* EPILOGUE_RESIDUAL: bf16 [M][N] */
+    const terna_bf16* next_norm_weight;
+    float* stats_out;
+    terna_bf16* raw_out;              /* EPILOGUE_RESIDUAL, optional */
+    int8_t* xq_out;                   /* optional pair: the quantised activations as published by the first workgroup */
+    terna_bf16* s_out;
+} ternaspmm_fused_linear_desc;
+int ternaspmm_fused_linear(const ternaspmm_fused_linear_desc* desc, terna_stream stream);
+
+/* Partials of a row block no producing epilogue wrote (the embedding rows in front of the first block): per row and per
+ * 512 columns (sum of h^2, max |h * norm_weight|) -> stats_out fp32 [M][ternaspmm_row_stats_count(K)][2].  Returns that
+ * count, or -1 (K not a multiple of 8).  Only enqueues. */
+int ternaspmm_row_stats_count(int K);
+int ternaspmm_row_stats(const terna_bf16* h, const terna_bf16* norm_weight, float* stats_out, int M, int K, terna_stream stream);
+
+/* Load time: band permutation of a P2 gate+up matrix [w1; w3] ([N][K], N = 2F) for TERNASPMM_EPILOGUE_GATE -- band 2j <-
+ * rows 16j .. 16j+15 of w1, band 2j+1 <- the same rows of w3.  packed_out: N*K/4 bytes, not `packed`.  Returns 0 / -1. */
+int ternaspmm_interleave_gate_up(const void* packed, void* packed_out, int N, int K, terna_stream stream);
+
 /* ---- Attention-side kernels of a decode step (no counterpart in the reference's library) -----------
  * They stand where the reference calls xformers' rope_padded (model.py:218-229) and
  * fmha.memory_efficient_attention_forward (model.py:231-233).
@@ -297,8 +359,8 @@ void ternaspmm_prefill_attention(const terna_bf16* q, const terna_bf16* cache_k,
  * held until the process ends.  Limit: B * H <= 256 heads per call (D 64 or 128); beyond that the call prints an
  * error, does nothing and returns -1 (0 on success).  Calls no hipMalloc / hipFree.  Every call on one GPU shares
  * that GPU's array: calls that overlap on one GPU (two streams, two threads) race -- serialise them.  The first
- * call on a device looks the array's address up and enqueues a small clear of the counters on `stream`; make
- * that first call outside stream capture. */
+ * call on a device looks the array's address up and enqueues a small clear of the counters on `stream`: it must
+ * be made outside stream capture -- under capture that first call records nothing, prints an error and returns -1. */
 int ternaspmm_decode_attention_static(const terna_bf16* q, const terna_bf16* cache_k, const terna_bf16* cache_v,
                                       const long long* pos, int per_sequence, terna_bf16* out, int B, int H, int KV, int D, int S,
                                       float scale, terna_stream stream);

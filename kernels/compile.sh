@@ -28,6 +28,7 @@ compile launch_decode_packed.hip launch_decode_packed.o
 compile launch_prefill_packed.hip launch_prefill_packed_i8.o -DTERNA_PREFILL_ACT=int8_t
 compile launch_prefill_packed.hip launch_prefill_packed_bf16.o -DTERNA_PREFILL_ACT=uint16_t
 compile abi_fused.hip abi_fused.o
+compile abi_chain.hip abi_chain.o
 compile abi_attention.hip abi_attention.o
 # accumulators of the prompt-pass attention in ordinary vector registers (they are rescaled between matrix instructions)
 compile abi_prefill_attention.hip abi_prefill_attention.o -mllvm -amdgpu-mfma-vgpr-form

@@ -6,6 +6,6 @@ from .convert_utils import (  # noqa: F401
     reorder_weight, save_checkpoint)
 from .linear import (  # noqa: F401
     BF16BitLinear, SpBitLinear, argmax_rows, greedy_step, greedy_step_state, lm_head, SpBitLinearBF16, TernaInfer_linear, TernaInfer_linear_bf16,
-    TernaInfer_linear_packed, get_global_workspace, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant, repack_weight, rmsnorm_linear_packed, rmsnorm_quant)
+    TernaInfer_linear_packed, fused_linear, get_global_workspace, interleave_gate_up, row_stats, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant, repack_weight, rmsnorm_linear_packed, rmsnorm_quant)
 
 __version__ = "0.1"

@@ -74,6 +74,10 @@ PROTOTYPES = {
     "ternaspmm_repack_cache_stats": ([_vp], None),
     "ternaspmm_plan_reference_call": ([_ci] * 6 + [_vp, _ci, _vp], _ci),
     "ternaspmm_quant_mode": ([_ci], _ci),
+    "ternaspmm_fused_linear": ([_vp, _vp], _ci),
+    "ternaspmm_row_stats_count": ([_ci], _ci),
+    "ternaspmm_row_stats": ([_vp, _vp, _vp, _ci, _ci, _vp], _ci),
+    "ternaspmm_interleave_gate_up": ([_vp, _vp, _ci, _ci, _vp], _ci),
     "ternaspmm_version": ([], ctypes.c_char_p),
 }
 

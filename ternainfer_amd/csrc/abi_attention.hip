@@ -199,6 +199,15 @@ static unsigned char* static_scratch(hipStream_t st, int line)
     }
     std::lock_guard<std::mutex> lock(mutex);
     if (ptr_of[dev] == nullptr) {
+        // the first call on a device clears the counters with a launch on the caller's stream: recorded into a graph
+        // it would run at replay time only, and calls made before the first replay would find the array as it was
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(st, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            std::fprintf(stderr, "ternaspmm_decode_attention_static: the first call on a device must be made outside stream "
+                                 "capture (it sets the library's scratch array up); nothing was recorded\n");
+            return nullptr;
+        }
         unsigned char* ptr = nullptr;
         e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch));
         if (e != hipSuccess || ptr == nullptr) die("hipGetSymbolAddress(scratch)", e, line);

@@ -1,0 +1,213 @@
+// C ABI of the chained small-M linears of a decode step: every launch is the consumer of the row statistics its
+// producer left and the producer of the statistics its consumer needs (decode_fused_kernel.h: FUSED_STATS prologue,
+// FEPI_RESIDUAL / FEPI_GLU epilogues).  Declarations: include/ternaspmm.h.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+
+#include "../../include/ternaspmm.h"
+#include "host_util.h"
+#include "decode_fused_kernel.h"
+
+using namespace terna;
+
+namespace {
+
+// Row statistics of a bf16 matrix h [M][K] under the weights of the norm that will read it: per row and per 512 columns
+// (sum of h^2, max |h * norm_w|), in the form the FUSED_STATS prologue adds up -- for a row block that no producing
+// epilogue wrote (the embedding rows in front of the first block).  One workgroup of 256 threads per row.
+__global__ __launch_bounds__(256) void terna_row_stats_kernel(const uint16_t* __restrict__ h, const uint16_t* __restrict__ norm_w,
+                                                               float2* __restrict__ stats_out, int K, int count)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const size_t row = blockIdx.x;
+    for (int p = wave; p < count; p += 4) {
+        const int c = p * 512 + lane * 8;
+        float ssq = 0.0f, pmax = 0.0f;
+        if (c < K) {                                    // K is a multiple of 8
+            float f[8], w[8];
+            unpack_bf16x8(*reinterpret_cast<const u32x4*>(h + row * K + c), f);
+            unpack_bf16x8(*reinterpret_cast<const u32x4*>(norm_w + c), w);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                ssq = fmaf(f[e], f[e], ssq);
+                pmax = fmaxf(pmax, fabsf(__fmul_rn(f[e], w[e])));
+            }
+        }
+        ssq = wave_sum(ssq);
+        pmax = wave_max(pmax);
+        if (lane == 0) stats_out[row * count + p] = float2{ssq, pmax};
+    }
+}
+
+// Band permutation of a P2 gate+up matrix ([w1; w3], N = 2F rows) for the FEPI_GLU epilogue: band 2j <- band j (rows
+// 16j .. of w1), band 2j + 1 <- band F/16 + j (the same rows of w3).  One workgroup per destination band.
+__global__ __launch_bounds__(256) void terna_interleave_gate_up_kernel(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst,
+                                                                        int N, int K)
+{
+    const int half_bands = N / 32;
+    const int dst_band = blockIdx.x;
+    const int src_band = (dst_band & 1) * half_bands + (dst_band >> 1);
+    const size_t words = static_cast<size_t>(K >> 6) * 64;
+    const u32x4* s4 = reinterpret_cast<const u32x4*>(src + src_band * words);
+    u32x4* d4 = reinterpret_cast<u32x4*>(dst + dst_band * words);
+    for (size_t q = threadIdx.x; q < words / 4; q += 256) d4[q] = s4[q];
+}
+
+// One launch of terna_decode_fused_kernel<WAVES, TMAX, MODE, MP, NB, ASP, AHD, EPI> with MP picked by M (1, 2, 4, 8).
+struct ChainArgs {
+    const uint16_t* x;
+    const uint16_t* residual;
+    const uint16_t* norm_w;
+    const uint32_t* packed;
+    int M, N, K;
+    float eps;
+    uint16_t* sum_out;
+    uint16_t* out;
+    const uint16_t* ws;
+    int ws_num;
+    int8_t* xq_out;
+    uint16_t* s_out;
+    int qmode;
+    FusedExtra ex;
+    dim3 grid;
+    hipStream_t st;
+};
+
+template <int WAVES, int TMAX, int MODE, int MP, int NB, int ASP, int AHD, int EPI>
+void launch_one(const ChainArgs& a)
+{
+    terna_decode_fused_kernel<WAVES, TMAX, MODE, MP, NB, ASP, AHD, EPI><<<a.grid, dim3(WAVES * 64), 0, a.st>>>(
+        a.x, a.residual, a.norm_w, a.packed, a.M, a.N, a.K, a.eps, a.sum_out, a.out, a.ws, a.ws_num, a.xq_out, a.s_out, a.qmode,
+        a.ex);
+}
+
+template <int WAVES, int TMAX, int MODE, int NB, int EPI>
+void launch_by_rows(const ChainArgs& a)
+{
+    if (a.M == 1) launch_one<WAVES, TMAX, MODE, 1, NB, 1, 64, EPI>(a);
+    else if (a.M == 2) launch_one<WAVES, TMAX, MODE, 2, NB, 1, 64, EPI>(a);
+    else if (a.M <= 4) launch_one<WAVES, TMAX, MODE, 4, NB, 1, 64, EPI>(a);
+    else launch_one<WAVES, TMAX, MODE, 8, NB, 1, 64, EPI>(a);
+}
+
+template <int EPI>
+void launch_attn(const ChainArgs& a, int splits, int head_dim)
+{
+#define TERNA_CHAIN_ATTN(SP, HD) launch_one<8, 5, FUSED_ATTN, 1, 1, SP, HD, EPI>(a)
+    if (head_dim == 128) {
+        if (splits == 1) TERNA_CHAIN_ATTN(1, 128);
+        else if (splits == 2) TERNA_CHAIN_ATTN(2, 128);
+        else if (splits == 4) TERNA_CHAIN_ATTN(4, 128);
+        else TERNA_CHAIN_ATTN(8, 128);
+    } else {
+        if (splits == 1) TERNA_CHAIN_ATTN(1, 64);
+        else if (splits == 2) TERNA_CHAIN_ATTN(2, 64);
+        else if (splits == 4) TERNA_CHAIN_ATTN(4, 64);
+        else TERNA_CHAIN_ATTN(8, 64);
+    }
+#undef TERNA_CHAIN_ATTN
+}
+
+}  // namespace
+
+extern "C" {
+
+int ternaspmm_row_stats_count(int K) { return K < 8 || (K & 7) ? -1 : (K + 511) / 512; }
+
+int ternaspmm_row_stats(const terna_bf16* h, const terna_bf16* norm_weight, float* stats_out, int M, int K, terna_stream stream)
+{
+    const int count = ternaspmm_row_stats_count(K);
+    if (M < 1 || count < 1 || count > kStatsMaxPartials) {
+        std::fprintf(stderr, "ternaspmm_row_stats: unsupported arguments (M=%d K=%d)\n", M, K);
+        return -1;
+    }
+    terna_row_stats_kernel<<<dim3(M), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(h, norm_weight, reinterpret_cast<float2*>(stats_out), K, count);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_row_stats", e, __LINE__);
+    return count;
+}
+
+int ternaspmm_interleave_gate_up(const void* packed, void* packed_out, int N, int K, terna_stream stream)
+{
+    if (N < 64 || K < 64 || (N % 64) || (K % 64) || packed == packed_out) return -1;
+    terna_interleave_gate_up_kernel<<<dim3(N / 16), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<const uint32_t*>(packed), static_cast<uint32_t*>(packed_out), N, K);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_interleave_gate_up", e, __LINE__);
+    return 0;
+}
+
+int ternaspmm_fused_linear(const ternaspmm_fused_linear_desc* d, terna_stream stream)
+{
+    if (d == nullptr) return -1;
+    const int M = d->M, N = d->N, K = d->K;
+    if (!shape_ok(M, N, K) || !groups_ok(d->ws_num) || M > 8) return -1;
+    const int pro = d->prologue, epi = d->epilogue;
+    const int ktiles = K / 64, bands = N / 16;
+    if (pro != TERNASPMM_PROLOGUE_NORM && pro != TERNASPMM_PROLOGUE_ATTENTION && pro != TERNASPMM_PROLOGUE_STATS) return -1;
+    if (epi != TERNASPMM_EPILOGUE_STORE && epi != TERNASPMM_EPILOGUE_RESIDUAL && epi != TERNASPMM_EPILOGUE_GATE) return -1;
+    if (d->x == nullptr || d->norm_weight == nullptr || d->packed == nullptr || d->ws == nullptr || d->out == nullptr) return -1;
+    if ((d->xq_out != nullptr) != (d->s_out != nullptr)) return -1;
+    if (pro == TERNASPMM_PROLOGUE_STATS && (d->stats_in == nullptr || d->stats_count < 1 || d->stats_count > kStatsMaxPartials)) return -1;
+    if (epi != TERNASPMM_EPILOGUE_STORE && (d->next_norm_weight == nullptr || d->stats_out == nullptr)) return -1;
+    if (epi == TERNASPMM_EPILOGUE_RESIDUAL && d->residual == nullptr) return -1;
+    if (epi == TERNASPMM_EPILOGUE_GATE && (d->ws_num != 2 || bands % 4 != 0)) return -1;
+    const int out_partials = epi == TERNASPMM_EPILOGUE_RESIDUAL ? bands : (epi == TERNASPMM_EPILOGUE_GATE ? bands / 2 : 0);
+    if (out_partials > kStatsMaxPartials) return -1;
+
+    ChainArgs a{};
+    a.x = static_cast<const uint16_t*>(d->x);
+    a.norm_w = d->norm_weight;
+    a.packed = static_cast<const uint32_t*>(d->packed);
+    a.M = M; a.N = N; a.K = K;
+    a.eps = d->eps;
+    a.out = d->out;
+    a.ws = d->ws;
+    a.ws_num = d->ws_num;
+    a.xq_out = d->xq_out;
+    a.s_out = d->s_out;
+    a.qmode = quant_mode();
+    a.ex = FusedExtra{reinterpret_cast<const float2*>(d->stats_in), d->stats_count, d->residual, d->next_norm_weight,
+                      reinterpret_cast<float2*>(d->stats_out), d->raw_out};
+    a.st = static_cast<hipStream_t>(stream);
+
+    if (pro == TERNASPMM_PROLOGUE_ATTENTION) {
+        // the O projection of a single-row step with the deferred attention merge inside (x = the partial results)
+        const int hd = d->head_dim, sp = d->attention_splits;
+        if (M != 1 || (hd != 64 && hd != 128) || K % hd != 0 || (sp != 1 && sp != 2 && sp != 4 && sp != 8) || ktiles > 8 * 5 ||
+            bands > 65535 || epi == TERNASPMM_EPILOGUE_GATE)
+            return -1;
+        a.grid = dim3(bands);
+        if (epi == TERNASPMM_EPILOGUE_RESIDUAL) launch_attn<FEPI_RESIDUAL>(a, sp, hd);
+        else launch_attn<FEPI_PLAIN>(a, sp, hd);
+    } else if (epi == TERNASPMM_EPILOGUE_GATE) {
+        // gate+up, bands interleaved: four bands (two gate / up pairs) per workgroup
+        if (pro != TERNASPMM_PROLOGUE_STATS || ktiles > 8 * 5) return -1;
+        a.grid = dim3(bands / 4);
+        launch_by_rows<8, 5, FUSED_STATS, 4, FEPI_GLU>(a);
+    } else if (pro == TERNASPMM_PROLOGUE_STATS) {
+        const bool res = epi == TERNASPMM_EPILOGUE_RESIDUAL;
+        a.grid = dim3(bands);
+        if (ktiles <= 8 * 5) {
+            if (res) launch_by_rows<8, 5, FUSED_STATS, 1, FEPI_RESIDUAL>(a);
+            else launch_by_rows<8, 5, FUSED_STATS, 1, FEPI_PLAIN>(a);
+        } else if (ktiles <= 16 * 7) {
+            if (res) launch_by_rows<16, 7, FUSED_STATS, 1, FEPI_RESIDUAL>(a);
+            else launch_by_rows<16, 7, FUSED_STATS, 1, FEPI_PLAIN>(a);
+        } else {
+            return -1;
+        }
+    } else {
+        // the norm's statistics taken inside (two workgroup-wide reductions), producing epilogue
+        if (epi != TERNASPMM_EPILOGUE_RESIDUAL || ktiles > 8 * 5) return -1;     // (with a plain store: bitlinear_TernaSpMM_packed_fused)
+        a.grid = dim3(bands);
+        launch_by_rows<8, 5, FUSED_PLAIN, 1, FEPI_RESIDUAL>(a);
+    }
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_fused_linear", e, __LINE__);
+    return out_partials;
+}
+
+}  // extern "C"

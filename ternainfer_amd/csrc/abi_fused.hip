@@ -76,7 +76,7 @@ static int launch_decode_fused(int mode, const terna_bf16* x, const terna_bf16* 
     const int qmode = quant_mode();
 #define TERNA_FUSED(WAVES, TMAX, MODE, MP, NB)                                                                     \
     terna_decode_fused_kernel<WAVES, TMAX, MODE, MP, NB><<<grid, dim3(WAVES * 64), 0, st>>>(                       \
-        x, residual, norm_weight, p, M, N, K, eps, sum_out, out, ws, ws_num, xq_out, s_out, qmode)
+        x, residual, norm_weight, p, M, N, K, eps, sum_out, out, ws, ws_num, xq_out, s_out, qmode, FusedExtra{})
 #define TERNA_FUSED_M(WAVES, TMAX, MODE, NB)                                                                       \
     do {                                                                                                           \
         if (M == 1) TERNA_FUSED(WAVES, TMAX, MODE, 1, NB);                                                         \
@@ -138,7 +138,7 @@ int bitlinear_TernaSpMM_packed_fused_attn(const float* partial, int splits, int 
     const int qmode = quant_mode();
 #define TERNA_FUSED_ATTN(SP, HD)                                                                                   \
     terna_decode_fused_kernel<8, 5, FUSED_ATTN, 1, 1, SP, HD><<<grid, dim3(8 * 64), 0, st>>>(                      \
-        x, nullptr, norm_weight, p, M, N, K, eps, nullptr, out, ws, ws_num, xq_out, s_out, qmode)
+        x, nullptr, norm_weight, p, M, N, K, eps, nullptr, out, ws, ws_num, xq_out, s_out, qmode, FusedExtra{})
 #define TERNA_FUSED_ATTN_HD(HD)                                                                                    \
     do {                                                                                                           \
         if (splits == 1) TERNA_FUSED_ATTN(1, HD);                                                                  \

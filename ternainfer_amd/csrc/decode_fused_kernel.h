@@ -26,6 +26,21 @@
 //      with data-parallel permutes, no LDS), MFMA
 //   E  cross-wave sum of the accumulators + epilogue (wave b finishes band b) -- barrier 3
 //
+// FUSED_STATS: the row statistics come from the PRODUCER of h instead.  The launch that wrote h also left, per row and
+// per 16 (or more) columns, the partial sums of h^2 and the partial maxima of |h * norm_w| (both exact products of two
+// bf16 values); here one wave per row adds / maximises the partials in a fixed order -- the same order in every
+// workgroup, so all bands see identical int8 activations -- and the rest is element-wise:
+//   y = bf16((h * norm_w) * rstd)        max|y| = bf16(max|h * norm_w| * rstd) exactly: both roundings are monotone
+// One barrier instead of two, no second pass over the row, and the row need not stay in registers.
+//
+// Epilogues (EPI): FEPI_PLAIN stores bf16 out[m][n].  The other two make this launch the producer for the next one:
+//   FEPI_RESIDUAL  h' = bf16(residual[m][n] + out[m][n]) is stored (the new residual stream, model.py:330, :334) with
+//                  the statistics of h' under the NEXT norm's weights, one partial per row and 16-row band;
+//   FEPI_GLU       the bands of W alternate between the gate and the up matrix (band 2j = rows 16j.. of w1, band
+//                  2j+1 = the same rows of w3; a load-time permutation), so the workgroup holds matching x1 / x3 and
+//                  stores inner = bf16(bf16(relu(x1)^2) * x3) (model.py:279-280) -- N/2 columns instead of N -- with
+//                  its statistics under the ffn_sub_norm weights.
+//
 // NB = bands of W per workgroup.  The prologue is repeated by every workgroup, so a matrix with
 // more bands than the chip has CUs (gate+up: 864) would repeat it once per *round* of workgroups
 // on every CU; with NB bands per workgroup the grid fits one round, the prologue runs once per CU
@@ -88,19 +103,34 @@ template <> struct RowPiece<1> {
 // MP = rows a wave's 64 lanes cover at once (M <= MP): 64/MP lanes walk along a row, MP columns
 // each, so a lane handles MP elements per tile -- the prologue arithmetic, which every workgroup
 // repeats, costs in proportion to the batch rows that exist, not to the 16 the MFMA tile has.
-enum FusedMode { FUSED_PLAIN, FUSED_RESIDUAL, FUSED_GLU, FUSED_ATTN };
+enum FusedMode { FUSED_PLAIN, FUSED_RESIDUAL, FUSED_GLU, FUSED_ATTN, FUSED_STATS };
+enum FusedEpilogue { FEPI_PLAIN, FEPI_RESIDUAL, FEPI_GLU };
+
+constexpr int kStatsMaxPartials = 448;           // partials per row a consumer adds up: 7 per lane of one wave
+
+// What the newer prologue / epilogues need beyond the original argument list (passed by value, last).
+struct FusedExtra {
+    const float2* stats_in;          // FUSED_STATS: [M][stats_count] (sum of h^2, max |h * norm_w|)
+    int stats_count;
+    const uint16_t* epi_residual;    // FEPI_RESIDUAL: bf16 [M][N], the stream the output is added to
+    const uint16_t* epi_next_w;      // FEPI_RESIDUAL / FEPI_GLU: weights of the norm that follows (bf16 [N] / [N/2])
+    float2* stats_out;               // [M][N/16] / [M][N/32]
+    uint16_t* raw_out;               // FEPI_RESIDUAL, optional: the linear's own output bf16 [M][N] as well
+};
 
 // ASP / AHD (FUSED_ATTN only): splits and head size of the attention whose partial results the row is merged from --
 // compile-time, so that a head's statistics are two scalar loads and no address needs a division.
-template <int WAVES, int TMAX, int MODE, int MP, int NB = 1, int ASP = 1, int AHD = 64>
+template <int WAVES, int TMAX, int MODE, int MP, int NB = 1, int ASP = 1, int AHD = 64, int EPI = FEPI_PLAIN>
 __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
     // what the first loads depend on comes first: the leading sixteen dwords of the arguments arrive in scalar registers
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, const uint16_t* __restrict__ norm_w,
     const uint32_t* __restrict__ packed, int M, int N, int K, float eps, uint16_t* __restrict__ sum_out,
     uint16_t* __restrict__ out, const uint16_t* __restrict__ ws, int ws_num, int8_t* __restrict__ xq_out,
-    uint16_t* __restrict__ s_out, int quant_mode)
+    uint16_t* __restrict__ s_out, int quant_mode, FusedExtra ex)
 {
     static_assert(MODE != FUSED_ATTN || MP == 1, "the attention merge feeds a single row");
+    static_assert(MODE != FUSED_STATS || MP <= WAVES, "one reducing wave per row");
+    static_assert(EPI != FEPI_GLU || NB % 2 == 0, "gate and up bands come in pairs");
     static_assert(AHD % 64 == 0 && ASP >= 1 && ASP <= kAttentionMaxSplits, "a 64-column tile lies inside one head");
     using XQ = XSlab<int8_t>;
     using Piece = RowPiece<MP>;
@@ -197,8 +227,49 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
     }
     // wave b finishes band b: its weight-group scales are requested now, converted at the very end
     const Epilogue ep{nullptr, ws, nullptr, ws_num, EP_I8_DECODE};
+    constexpr int NFIN = EPI == FEPI_GLU ? NB / 2 : NB;            // finishing waves (a gate / up pair shares one)
+    const bool finisher = wave < NFIN;
     const int my_band = band0 + (wave < NB ? wave : 0);
-    EpilogueRaw eraw = load_epilogue_raw_scales(ep, my_band * 16 + 4 * g, N);
+    EpilogueRaw eraw;
+    if constexpr (EPI == FEPI_GLU) {
+        eraw.s = 0u;
+        eraw.w[0] = ws[0];                                         // gate rows (w1) and up rows (w3): one scale each
+        eraw.w[1] = ws[1];
+        eraw.w[2] = eraw.w[3] = 0u;
+    } else {
+        eraw = load_epilogue_raw_scales(ep, my_band * 16 + 4 * g, N);
+    }
+    // What the producing epilogues read besides the accumulators -- four stream values and four weights of the next
+    // norm per lane -- is requested here as well, by the finishing waves (the others read one address: no traffic).
+    u32x2 eres = {0u, 0u}, enw = {0u, 0u};
+    const int out_cols = EPI == FEPI_GLU ? N / 2 : N;
+    const int epi_col = EPI == FEPI_GLU ? (static_cast<int>(blockIdx.x) * NFIN + (finisher ? wave : 0)) * 16 + 4 * g : my_band * 16 + 4 * g;
+    if constexpr (EPI != FEPI_PLAIN) {
+        const size_t noff = finisher ? static_cast<size_t>(epi_col) : 0;
+        enw = *reinterpret_cast<const u32x2*>(ex.epi_next_w + noff);
+        if constexpr (EPI == FEPI_RESIDUAL) {
+            const size_t roff = finisher ? static_cast<size_t>(i < M ? i : 0) * N + epi_col : 0;
+            eres = *reinterpret_cast<const u32x2*>(ex.epi_residual + roff);
+        }
+    }
+    // FUSED_STATS: wave r adds up the partials of row r (the other waves read one address: no traffic)
+    constexpr int PT = MODE == FUSED_STATS ? kStatsMaxPartials / 64 : 1;
+    float2 part[PT];
+    if constexpr (MODE == FUSED_STATS) {
+        const bool reducer = wave < M;
+        const float2* sp = ex.stats_in + (reducer ? static_cast<size_t>(wave) * ex.stats_count : 0);
+#pragma unroll
+        for (int t = 0; t < PT; ++t) {
+            const int idx = lane + 64 * t;
+            part[t] = sp[reducer && idx < ex.stats_count ? idx : 0];
+        }
+    }
+    // Requested here, used at the very end: without this the compiler moves the two loads next to their use, behind
+    // the last barrier, and the launch ends with one more dependent trip to memory.
+    if constexpr (EPI != FEPI_PLAIN) {
+        pin_registers(enw);
+        pin_registers(eres);
+    }
     // this wave's LDS slot: rows the batch does not have stay zero (a single row needs no slot, see phase D)
     uint8_t* slab = slab_all[wave];
     if constexpr (MP != 1)
@@ -206,7 +277,7 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
 
     float ssq = 0.0f;
 #pragma unroll
-    for (int t = 0; t < TMAX; ++t) {
+    for (int t = 0; t < (MODE == FUSED_STATS ? 0 : TMAX); ++t) {
         const int j = wave + WAVES * t;
         float f[MP];
         xr[t].unpack(f);
@@ -247,8 +318,38 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
         }
         return r;
     };
+    float rstd, s;
+    uint16_t s_bits = 0;
+    if constexpr (MODE == FUSED_STATS) {
+        // ---- phases B + C from the producer's partials: one wave per row, a fixed order, one barrier
+        if (wave < M) {
+            float sum = 0.0f, pmax = 0.0f;
+#pragma unroll
+            for (int t = 0; t < PT; ++t) {
+                if (lane + 64 * t < ex.stats_count) {
+                    sum += part[t].x;
+                    pmax = fmaxf(pmax, part[t].y);
+                }
+            }
+            sum = wave_sum(sum);
+            pmax = wave_max(pmax);
+            if (lane == 0) {
+                const float r = rsqrtf(sum / static_cast<float>(K) + eps);
+                const float amax_y = fabsf(round_bf16(__fmul_rn(pmax, r)));      // = max |y| of the row, exactly
+                uint16_t sb;
+                const float s_mul = quant_scale(amax_y, quant_mode, &sb);
+                stat[0][wave][0] = r;
+                stat[1][wave][0] = s_mul;
+                s_row[wave] = bf16_bits_to_float(sb);
+                if (writer && s_out != nullptr) s_out[wave] = sb;
+            }
+        }
+        __syncthreads();
+        rstd = stat[0][row_ok ? row : 0][0];
+        s = stat[1][row_ok ? row : 0][0];
+    } else {
     ssq = row_reduce(ssq, 0, false);
-    const float rstd = rsqrtf(ssq / static_cast<float>(K) + eps);
+    rstd = rsqrtf(ssq / static_cast<float>(K) + eps);
 
     // ---- phase C: y in place of h, max |y| per row
     float amax = 0.0f;
@@ -260,17 +361,17 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
         const bool valid = wave + WAVES * t < ktiles;
 #pragma unroll
         for (int e = 0; e < MP; ++e) {
-            f[e] = round_bf16(f[e] * rstd * w[e]);
+            f[e] = round_bf16(__fmul_rn(__fmul_rn(f[e], w[e]), rstd));
             if (valid) amax = fmaxf(amax, fabsf(f[e]));
         }
         xr[t].pack(f);
     }
     amax = row_reduce(amax, 1, true);
-    uint16_t s_bits;
-    const float s = quant_scale(amax, quant_mode, &s_bits);      // what multiplies; the epilogue divides by the bf16 value
+    s = quant_scale(amax, quant_mode, &s_bits);      // what multiplies; the epilogue divides by the bf16 value
     if (wave == 0 && (lane % LPR) == 0) {
         s_row[row] = bf16_bits_to_float(s_bits);
         if (writer && s_out != nullptr && row_ok) s_out[row] = s_bits;
+    }
     }
 
     // ---- phase D: quantise a tile, turn it into operand order through the wave's LDS slot, multiply
@@ -283,11 +384,31 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
         if (j < ktiles) {
             float f[MP];
             xr[t].unpack(f);
-            uint8_t q[MP];
+            if constexpr (MODE == FUSED_STATS) {                  // the norm, element-wise: rstd came from the partials
+                float w[MP];
+                nw[t].unpack(w);
 #pragma unroll
-            for (int e = 0; e < MP; ++e) {
-                const float r = quant_value(f[e], s, quant_mode);
-                q[e] = static_cast<uint8_t>(static_cast<int>(r) & 0xff);
+                for (int e = 0; e < MP; ++e) f[e] = round_bf16(__fmul_rn(__fmul_rn(f[e], w[e]), rstd));
+            }
+            // int8 bytes, packed four to a dword: clamp(rint(y * s)) + 128 is an integer in [0, 255] that one
+            // conversion drops into its byte; the xor takes the 128 out again (two's complement)
+            constexpr int ND = MP >= 4 ? MP / 4 : 1;
+            constexpr uint32_t kBias = MP >= 4 ? 0x80808080u : (MP == 2 ? 0x8080u : 0x80u);
+            uint32_t d[ND];
+            const bool eager = quant_mode == QUANT_EAGER;                    // uniform: one branch per tile, not per element
+#pragma unroll
+            for (int e4 = 0; e4 < ND; ++e4) {
+                uint32_t wd = 0u;
+                if (eager) {
+#pragma unroll
+                    for (int e = 4 * e4; e < 4 * e4 + 4 && e < MP; ++e)
+                        wd = __builtin_amdgcn_cvt_pk_u8_f32(quant_value(f[e], s, QUANT_EAGER) + 128.0f, e & 3, wd);
+                } else {
+#pragma unroll
+                    for (int e = 4 * e4; e < 4 * e4 + 4 && e < MP; ++e)
+                        wd = __builtin_amdgcn_cvt_pk_u8_f32(quant_value(f[e], s, QUANT_ROUNDED) + 128.0f, e & 3, wd);
+                }
+                d[e4] = wd ^ kBias;
             }
             uint8_t* dst = slab + row * XQ::kPitch + cl;
             int8_t* gdst = xq_out + static_cast<size_t>(row_ok ? row : 0) * K + j * 64 + cl;
@@ -297,8 +418,8 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
                 // One row: lane c holds the byte of column c.  Four neighbouring bytes into the dword of lane 4d,
                 // the four dwords of 16 columns into lane 16g -- the only lanes whose MFMA operand (batch row 0,
                 // columns 16g .. 16g+15) is not zero.  No LDS.
-                if (publish) *gdst = static_cast<int8_t>(q[0]);
-                const uint32_t b1 = q[0];
+                if (publish) *gdst = static_cast<int8_t>(d[0]);
+                const uint32_t b1 = d[0];
                 const uint32_t b2 = b1 | (dpp_permute_u32<kDppSwapPairs>(b1) << 8);          // even lanes: columns c, c+1
                 const uint32_t b4 = b2 | (dpp_permute_u32<kDppSwapHalfQuads>(b2) << 16);     // lanes 4d: columns 4d .. 4d+3
                 const uint32_t d1 = dpp_permute_u32<kDppRowShl4>(b4), d2 = dpp_permute_u32<kDppRowShl8>(b4),
@@ -307,15 +428,6 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
                 bq = i32x4{static_cast<int>(first ? b4 : 0u), static_cast<int>(first ? d1 : 0u),
                            static_cast<int>(first ? d2 : 0u), static_cast<int>(first ? d3 : 0u)};
             } else {
-                constexpr int ND = MP >= 4 ? MP / 4 : 1;
-                uint32_t d[ND];
-                if constexpr (MP >= 4) {
-#pragma unroll
-                    for (int e = 0; e < ND; ++e)
-                        d[e] = q[4 * e] | (q[4 * e + 1] << 8) | (q[4 * e + 2] << 16) | (static_cast<uint32_t>(q[4 * e + 3]) << 24);
-                } else {
-                    d[0] = q[0] | (q[1] << 8);
-                }
                 if constexpr (MP == 2) {
                     *reinterpret_cast<uint16_t*>(dst) = static_cast<uint16_t>(d[0]);
                     if (publish) *reinterpret_cast<uint16_t*>(gdst) = static_cast<uint16_t>(d[0]);
@@ -345,19 +457,73 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_fused_kernel(
 #pragma unroll
     for (int b = 0; b < NB; ++b) red[wave][b][lane] = acc[b];
     __syncthreads();
-    if (wave < NB) {
-        i32x4 sum = red[0][wave][lane];
+    if (finisher) {
+        EpilogueRegs e = finish_epilogue(ep, eraw);
+        e.s = s_row[i < M ? i : 0];
+        if constexpr (EPI == FEPI_GLU) {
+            // gate band 2 * wave and up band 2 * wave + 1: x1, x3 of the same sixteen features
+            i32x4 sum1 = red[0][2 * wave][lane], sum3 = red[0][2 * wave + 1][lane];
 #pragma unroll
-        for (int w = 1; w < WAVES; ++w) sum += red[w][wave][lane];
-        if (i < M) {
-            const int n0 = my_band * 16 + 4 * g;
-            EpilogueRegs e = finish_epilogue(ep, eraw);
-            e.s = s_row[i];
+            for (int w = 1; w < WAVES; ++w) {
+                sum1 += red[w][2 * wave][lane];
+                sum3 += red[w][2 * wave + 1][lane];
+            }
+            const float w1 = __uint_as_float(eraw.w[0] << 16), w3 = __uint_as_float(eraw.w[1] << 16);
+            float nwv[4], hv[4];
+            nwv[0] = __uint_as_float(enw.x << 16); nwv[1] = __uint_as_float(enw.x & 0xffff0000u);
+            nwv[2] = __uint_as_float(enw.y << 16); nwv[3] = __uint_as_float(enw.y & 0xffff0000u);
+            float ssq_o = 0.0f, pmax_o = 0.0f;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                e.w[v] = w1;
+                const float x1 = bf16_bits_to_float(apply_epilogue<int>(EP_I8_DECODE, e, v, sum1[v] >> kI8WeightShift));
+                e.w[v] = w3;
+                const float x3 = bf16_bits_to_float(apply_epilogue<int>(EP_I8_DECODE, e, v, sum3[v] >> kI8WeightShift));
+                const float p = fmaxf(x1, 0.0f);
+                hv[v] = i < M ? round_bf16(round_bf16(p * p) * x3) : 0.0f;
+                ssq_o = fmaf(hv[v], hv[v], ssq_o);
+                pmax_o = fmaxf(pmax_o, fabsf(__fmul_rn(hv[v], nwv[v])));
+            }
+            // the four lanes (g = 0 .. 3) of a batch row hold the band's sixteen features between them
+            ssq_o = cross_row_reduce<false>(ssq_o);
+            pmax_o = cross_row_reduce<true>(pmax_o);
+            if (i < M) {
+                *reinterpret_cast<u32x2*>(out + static_cast<size_t>(i) * out_cols + epi_col) =
+                    u32x2{pack_bf16x2(hv[0], hv[1]), pack_bf16x2(hv[2], hv[3])};
+                if (g == 0) ex.stats_out[static_cast<size_t>(i) * (out_cols / 16) + epi_col / 16] = float2{ssq_o, pmax_o};
+            }
+        } else {
+            i32x4 sum = red[0][wave][lane];
+#pragma unroll
+            for (int w = 1; w < WAVES; ++w) sum += red[w][wave][lane];
             uint16_t o[4];
 #pragma unroll
             for (int v = 0; v < 4; ++v) o[v] = apply_epilogue<int>(EP_I8_DECODE, e, v, sum[v] >> kI8WeightShift);
             const u32x2 pk = {o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16)};
-            *reinterpret_cast<u32x2*>(out + static_cast<size_t>(i) * N + n0) = pk;
+            if constexpr (EPI == FEPI_PLAIN) {
+                if (i < M) *reinterpret_cast<u32x2*>(out + static_cast<size_t>(i) * N + epi_col) = pk;
+            } else {
+                float rv[4], nwv[4], hv[4];
+                rv[0] = __uint_as_float(eres.x << 16); rv[1] = __uint_as_float(eres.x & 0xffff0000u);
+                rv[2] = __uint_as_float(eres.y << 16); rv[3] = __uint_as_float(eres.y & 0xffff0000u);
+                nwv[0] = __uint_as_float(enw.x << 16); nwv[1] = __uint_as_float(enw.x & 0xffff0000u);
+                nwv[2] = __uint_as_float(enw.y << 16); nwv[3] = __uint_as_float(enw.y & 0xffff0000u);
+                float ssq_o = 0.0f, pmax_o = 0.0f;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    hv[v] = i < M ? round_bf16(rv[v] + bf16_bits_to_float(o[v])) : 0.0f;
+                    ssq_o = fmaf(hv[v], hv[v], ssq_o);
+                    pmax_o = fmaxf(pmax_o, fabsf(__fmul_rn(hv[v], nwv[v])));
+                }
+                ssq_o = cross_row_reduce<false>(ssq_o);
+                pmax_o = cross_row_reduce<true>(pmax_o);
+                if (i < M) {
+                    *reinterpret_cast<u32x2*>(out + static_cast<size_t>(i) * N + epi_col) =
+                        u32x2{pack_bf16x2(hv[0], hv[1]), pack_bf16x2(hv[2], hv[3])};
+                    if (ex.raw_out != nullptr) *reinterpret_cast<u32x2*>(ex.raw_out + static_cast<size_t>(i) * N + epi_col) = pk;
+                    if (g == 0) ex.stats_out[static_cast<size_t>(i) * (N / 16) + epi_col / 16] = float2{ssq_o, pmax_o};
+                }
+            }
         }
     }
 }

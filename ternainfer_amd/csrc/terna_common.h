@@ -155,6 +155,27 @@ __device__ __forceinline__ void pin_registers(u32x4& v)
     asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w));
 }
 
+__device__ __forceinline__ void pin_registers(u32x2& v) { asm volatile("" : "+v"(v.x), "+v"(v.y)); }
+__device__ __forceinline__ void pin_registers(float2& v) { asm volatile("" : "+v"(v.x), "+v"(v.y)); }
+
+// max / sum over the four lanes L, L ^ 16, L ^ 32, L ^ 48 with the row-swap permutations of the VALU (gfx950):
+// v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even rows of its second,
+// v_permlane32_swap the upper half of the first with the lower half of the second; applied to two copies of v, every
+// lane ends up holding its own value and its partner's.  No LDS round trip; the order of the additions is the same in
+// all four lanes.  (asm statements: through the builtins the compiler took the two results of a swap for equal.)
+template <bool IS_MAX>
+__device__ __forceinline__ float cross_row_reduce(float v)
+{
+    auto op = [](float a, float b) { return IS_MAX ? fmaxf(a, b) : a + b; };
+    float a = v, b = v;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+    v = op(a, b);
+    a = v;
+    b = v;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+    return op(a, b);
+}
+
 // Compile-time loop: the body receives the index as a constant, so register arrays indexed by it
 // never need dynamic addressing.
 template <int I, int N, typename F>

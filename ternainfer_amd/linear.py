@@ -255,6 +255,95 @@ def relu2_mul_rmsnorm_quant(x13, weight, eps, quant=True):
     return y
 
 
+class FusedLinearDesc(ctypes.Structure):
+    """ternaspmm_fused_linear_desc of include/ternaspmm.h."""
+    _fields_ = [(n, ctypes.c_int) for n in ("prologue", "epilogue", "M", "N", "K", "ws_num")] + [("eps", ctypes.c_float)] + \
+               [(n, ctypes.c_int) for n in ("stats_count", "attention_splits", "head_dim")] + \
+               [(n, ctypes.c_void_p) for n in ("x", "stats_in", "norm_weight", "packed", "ws", "out", "residual",
+                                               "next_norm_weight", "stats_out", "raw_out", "xq_out", "s_out")]
+
+
+PROLOGUE_NORM, PROLOGUE_ATTENTION, PROLOGUE_STATS = 0, 1, 2
+EPILOGUE_STORE, EPILOGUE_RESIDUAL, EPILOGUE_GATE = 0, 1, 2
+
+
+def row_stats(h, norm_weight):
+    """Partials of the norm statistics of h bf16 [M, K] under `norm_weight` (ternaspmm_row_stats): fp32 [M, count, 2]."""
+    m, k = h.shape
+    _check_rows("row_stats", h, norm_weight=(norm_weight, k))
+    lib = _lib.load()
+    count = lib.ternaspmm_row_stats_count(k)
+    if count < 1:
+        raise ValueError(f"row_stats: unsupported K={k}")
+    out = torch.empty((m, count, 2), dtype=torch.float32, device=h.device)
+    lib.ternaspmm_row_stats(_p(h.contiguous()), _p(norm_weight), _p(out), m, k, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    return out
+
+
+def interleave_gate_up(packed, out_features, in_features):
+    """Load time: the band order TERNASPMM_EPILOGUE_GATE reads (ternaspmm_interleave_gate_up) of a P2 gate+up matrix."""
+    out = torch.empty_like(packed)
+    if _lib.load().ternaspmm_interleave_gate_up(_p(packed), _p(out), out_features, in_features,
+                                               ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) != 0:
+        raise ValueError(f"interleave_gate_up: unsupported shape {out_features}x{in_features}")
+    return out
+
+
+def fused_linear(x, norm_weight, eps, packed, ws, ws_num, out_features, in_features, *, stats=None, attention=None,
+                 epilogue=EPILOGUE_STORE, residual=None, next_norm_weight=None, want_raw=False, publish=False):
+    """One launch of ternaspmm_fused_linear (include/ternaspmm.h): prologue -> ternary matmul on a P2 weight -> epilogue.
+    x: h bf16 [M, K], with `stats` (fp32 [M, count, 2]) when its producer left the norm statistics; or, with
+    `attention` = (splits, head_dim), the fp32 partial results of a split attention launch (one sequence).
+    Returns (out, stats_out, raw, xq, s) -- stats_out for the producing epilogues, raw with `want_raw`, (xq, s) with
+    `publish`, None otherwise -- or None when the library does not support the combination (nothing was enqueued)."""
+    lib = _lib.load()
+    k, n = in_features, out_features
+    if attention is not None:
+        m, pro = 1, PROLOGUE_ATTENTION
+    else:
+        m = x.shape[0]
+        _check_rows("fused_linear", x, k, norm_weight=(norm_weight, k))
+        x = x.contiguous()
+        pro = PROLOGUE_STATS if stats is not None else PROLOGUE_NORM
+    if packed.numel() * packed.element_size() < n * k // 4 or ws.numel() < ws_num:
+        raise ValueError("fused_linear: packed weight or weight scales too small for this shape")
+    dev = packed.device
+    out_cols = n // 2 if epilogue == EPILOGUE_GATE else n
+    d = FusedLinearDesc()
+    d.prologue, d.epilogue, d.M, d.N, d.K, d.ws_num, d.eps = pro, epilogue, m, n, k, ws_num, float(eps)
+    d.x, d.norm_weight, d.packed, d.ws = x.data_ptr(), norm_weight.data_ptr(), packed.data_ptr(), ws.data_ptr()
+    if stats is not None:
+        if stats.dtype != torch.float32 or stats.dim() != 3 or stats.shape[0] != m or stats.shape[2] != 2 or not stats.is_contiguous():
+            raise ValueError("fused_linear: stats must be a contiguous fp32 [M, count, 2] tensor")
+        d.stats_in, d.stats_count = stats.data_ptr(), stats.shape[1]
+    if attention is not None:
+        d.attention_splits, d.head_dim = attention
+    out = torch.empty((m, out_cols), dtype=torch.bfloat16, device=dev)
+    d.out = out.data_ptr()
+    stats_out = raw = xq = s = None
+    if epilogue != EPILOGUE_STORE:
+        if next_norm_weight is None or next_norm_weight.numel() != out_cols:
+            raise ValueError("fused_linear: a producing epilogue needs the next norm's weights")
+        stats_out = torch.empty((m, out_cols // 16, 2), dtype=torch.float32, device=dev)
+        d.next_norm_weight, d.stats_out = next_norm_weight.data_ptr(), stats_out.data_ptr()
+    if epilogue == EPILOGUE_RESIDUAL:
+        if residual is None or residual.numel() != m * n or residual.dtype != torch.bfloat16:
+            raise ValueError("fused_linear: the residual epilogue needs a bf16 [M, N] stream")
+        residual = residual.contiguous()
+        d.residual = residual.data_ptr()
+        if want_raw:
+            raw = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+            d.raw_out = raw.data_ptr()
+    if publish:
+        xq = torch.empty((m, k), dtype=torch.int8, device=dev)
+        s = torch.empty(m, dtype=torch.bfloat16, device=dev)
+        d.xq_out, d.s_out = xq.data_ptr(), s.data_ptr()
+    rc = lib.ternaspmm_fused_linear(ctypes.byref(d), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    if rc < 0:
+        return None
+    return out, stats_out, raw, xq, s
+
+
 def lm_head(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Logits of a decode step: F.linear(x, weight) for bf16 x [M, K] with M <= 16 and the bf16 output
     (tied embedding) matrix weight [V, K] (model.py:367, 449-455), as one HBM-bound pass over the matrix."""

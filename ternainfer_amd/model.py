@@ -22,7 +22,8 @@ import torch
 from torch.nn import functional as F
 
 from . import _lib
-from .linear import (argmax_rows, attention_merge_rmsnorm_linear_packed, get_global_workspace, greedy_step, greedy_step_state, lm_head, quant_input, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant,
+from .linear import (EPILOGUE_GATE, EPILOGUE_RESIDUAL, argmax_rows, attention_merge_rmsnorm_linear_packed, fused_linear, get_global_workspace, greedy_step,
+                     greedy_step_state, interleave_gate_up, lm_head, quant_input, row_stats, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant,
                      repack_weight, rmsnorm_linear_packed, rmsnorm_quant)
 
 
@@ -127,6 +128,8 @@ class Block:
         self.act = act
         self.fused = True          # norms / gate / activation quantisation through the fused prologue kernels
         self.prefetch = None       # (pointers, sizes, unit sizes, count): see Transformer.enable_prefetch
+        self.capture = None        # a list: forward_chain appends (name, xq, s, raw output) of each of its four linears
+        self.w13_interleaved = None
         if gen is None:            # filled in by from_checkpoint
             return
         d, hd = args.dim, args.head_dim
@@ -162,8 +165,9 @@ class Block:
         blk.attn_sub_norm, blk.ffn_sub_norm = norm("attention.attn_sub_norm"), norm("feed_forward.ffn_sub_norm")
         return blk
 
-    def _norm_linear(self, lin, x, weight, residual=None, glu=False):
-        """[x + residual | relu(x1)^2 * x3] -> RMSNorm -> lin.  Returns (lin output, x + residual)."""
+    def _norm_linear(self, lin, x, weight, residual=None, glu=False, name=None):
+        """[x + residual | relu(x1)^2 * x3] -> RMSNorm -> lin.  Returns (lin output, x + residual).  With `capture` set the
+        quantised activations go through memory (norm kernel + linear, never the one-launch form) and are recorded."""
         eps = self.args.norm_eps
         if not self.fused:
             if glu:
@@ -172,19 +176,102 @@ class Block:
             else:
                 h = x if residual is None else x + residual
             return lin(rms_norm(h, weight, eps)), h
+        cap = self.capture if self.act == "int8" else None
         if glu:
             if self.act == "int8":
-                if x.shape[0] <= 4:
+                if x.shape[0] <= 4 and cap is None:
                     return relu2_mul_rmsnorm_linear_packed(x, weight, eps, lin.packed, lin.ws, lin.ws_num, lin.n), None
-                return lin.quantised(*relu2_mul_rmsnorm_quant(x, weight, eps)), None
+                xq, s = relu2_mul_rmsnorm_quant(x, weight, eps)
+                out = lin.quantised(xq, s)
+                if cap is not None:
+                    cap.append((name, xq, s, out))
+                return out, None
             return lin.dense(relu2_mul_rmsnorm_quant(x, weight, eps, quant=False)), None
         if self.act == "int8":
-            if x.shape[0] <= 8:            # decode step: prologue and linear in one launch where that is faster
+            if x.shape[0] <= 8 and cap is None:   # decode step: prologue and linear in one launch where that is faster
                 return rmsnorm_linear_packed(x, weight, eps, lin.packed, lin.ws, lin.ws_num, lin.n, residual=residual)
             xq, s, h = rmsnorm_quant(x, weight, eps, residual=residual)
-            return lin.quantised(xq, s), h
+            out = lin.quantised(xq, s)
+            if cap is not None:
+                cap.append((name, xq, s, out))
+            return out, h
         y, h = rmsnorm_quant(x, weight, eps, residual=residual, quant=False)
         return lin.dense(y), h
+
+    def gate_up_interleaved(self):
+        """The gate+up matrix with the bands of w1 and w3 interleaved (made once): what the gate epilogue reads."""
+        if self.w13_interleaved is None:
+            self.w13_interleaved = interleave_gate_up(self.w13.packed, self.w13.n, self.w13.k)
+        return self.w13_interleaved
+
+    def forward_chain(self, x, stats, cache_k, cache_v, pos_idx, cos, sin, attn_ws, next_norm):
+        """One new token per sequence (up to 8 sequences), the linears chained through producer-side norm statistics:
+        `x` is the residual stream INCLUDING the previous block's FFN output and `stats` its partials under this block's
+        attention_norm (None: the first block, which takes them inside).  Every linear's epilogue leaves what the next
+        launch needs: the O projection adds the stream and leaves the ffn_norm partials, gate+up leaves
+        relu(x1)^2 * x3 with the ffn_sub_norm partials, the down projection adds the stream again and leaves the
+        partials under `next_norm` (the next block's attention_norm).  Returns (stream, partials)."""
+        a = self.args
+        bsz = cache_k.shape[0]
+        lib = self.wqkv.lib
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        per_seq = int(pos_idx.dim() == 2)
+        cap = self.capture
+        pub = cap is not None
+
+        def note(name, r):
+            if pub:
+                cap.append((name, r[3], r[4], r[2] if r[2] is not None else r[0]))
+
+        if stats is None and not pub:
+            qkv, _ = rmsnorm_linear_packed(x, self.attention_norm, a.norm_eps, self.wqkv.packed, self.wqkv.ws, self.wqkv.ws_num, self.wqkv.n)
+        else:
+            if stats is None:                       # (recording: the first block's statistics as a launch of their own)
+                stats = row_stats(x, self.attention_norm)
+            r = fused_linear(x, self.attention_norm, a.norm_eps, self.wqkv.packed, self.wqkv.ws, self.wqkv.ws_num, self.wqkv.n, self.wqkv.k,
+                             stats=stats, publish=pub)
+            note("wqkv", r)
+            qkv = r[0]
+        deferred = isinstance(attn_ws, tuple)
+        o_kw = dict(epilogue=EPILOGUE_RESIDUAL, residual=x, next_norm_weight=self.ffn_norm, want_raw=pub, publish=pub)
+        if deferred:
+            partial, splits = attn_ws
+            lib.ternaspmm_rope_decode_attention_partial(
+                _p(qkv), _p(cos), _p(sin), _p(pos_idx), per_seq, _p(cache_k), _p(cache_v), _p(partial), splits, bsz, a.n_heads,
+                a.n_kv_heads, a.head_dim, cache_k.shape[2], a.head_dim ** -0.5, int(a.rope_adjacent), None, None, None, 0, stream)
+            r = None
+            if bsz == 1:
+                r = fused_linear(partial, self.attn_sub_norm, a.norm_eps, self.wo.packed, self.wo.ws, self.wo.ws_num, self.wo.n, self.wo.k,
+                                 attention=(splits, a.head_dim), **o_kw)
+            if r is None:
+                o = torch.empty((bsz, a.n_heads * a.head_dim), dtype=torch.bfloat16, device=x.device)
+                lib.ternaspmm_attention_merge(_p(partial), splits, _p(o), bsz, a.n_heads, a.head_dim, stream)
+                r = fused_linear(o, self.attn_sub_norm, a.norm_eps, self.wo.packed, self.wo.ws, self.wo.ws_num, self.wo.n, self.wo.k, **o_kw)
+        else:
+            o = torch.empty((bsz, a.n_heads * a.head_dim), dtype=torch.bfloat16, device=x.device)
+            if self.prefetch is not None:
+                ptrs, sizes, units, count = self.prefetch
+                lib.ternaspmm_rope_decode_attention_prefetch(
+                    _p(qkv), _p(cos), _p(sin), _p(pos_idx), per_seq, _p(cache_k), _p(cache_v), _p(o), bsz, a.n_heads, a.n_kv_heads,
+                    a.head_dim, cache_k.shape[2], a.head_dim ** -0.5, int(a.rope_adjacent), _p(attn_ws), ptrs, sizes, units,
+                    count, stream)
+            else:
+                lib.ternaspmm_rope_decode_attention(_p(qkv), _p(cos), _p(sin), _p(pos_idx), per_seq, _p(cache_k), _p(cache_v), _p(o),
+                                                    bsz, a.n_heads, a.n_kv_heads, a.head_dim, cache_k.shape[2],
+                                                    a.head_dim ** -0.5, int(a.rope_adjacent), _p(attn_ws), stream)
+            if pub:
+                cap.append(("attention", None, None, o))
+            r = fused_linear(o, self.attn_sub_norm, a.norm_eps, self.wo.packed, self.wo.ws, self.wo.ws_num, self.wo.n, self.wo.k, **o_kw)
+        note("wo", r)
+        h, h_stats = r[0], r[1]
+        r = fused_linear(h, self.ffn_norm, a.norm_eps, self.gate_up_interleaved(), self.w13.ws, self.w13.ws_num, self.w13.n, self.w13.k,
+                         stats=h_stats, epilogue=EPILOGUE_GATE, next_norm_weight=self.ffn_sub_norm, publish=pub)
+        note("w13", r)
+        inner, inner_stats = r[0], r[1]
+        r = fused_linear(inner, self.ffn_sub_norm, a.norm_eps, self.w2.packed, self.w2.ws, self.w2.ws_num, self.w2.n, self.w2.k,
+                         stats=inner_stats, epilogue=EPILOGUE_RESIDUAL, residual=h, next_norm_weight=next_norm, want_raw=pub, publish=pub)
+        note("w2", r)
+        return r[0], r[1]
 
     def forward(self, x, pending, cache_k, cache_v, pos_idx, cos, sin, mask, attn_ws=None):
         """x [B*T, dim] (T new tokens per sequence) and `pending`, the previous block's FFN output that
@@ -196,7 +283,7 @@ class Block:
         bsz = cache_k.shape[0]
         t = x.shape[0] // bsz
         per_seq = int(pos_idx.dim() == 2)
-        qkv, x = self._norm_linear(self.wqkv, x, self.attention_norm, residual=pending)
+        qkv, x = self._norm_linear(self.wqkv, x, self.attention_norm, residual=pending, name="wqkv")
         rep = a.n_heads // a.n_kv_heads
         one_token = mask is None           # the caller's rule: fused, one new token, a head size the kernel has
         deferred = one_token and isinstance(attn_ws, tuple)
@@ -265,9 +352,11 @@ class Block:
                                                          self.wo.packed, self.wo.ws, self.wo.ws_num, self.wo.n, sequences=bsz)
             assert attn.shape[0] == bsz
         else:
-            attn, _ = self._norm_linear(self.wo, o.contiguous(), self.attn_sub_norm)
-        x13, x = self._norm_linear(self.w13, x, self.ffn_norm, residual=attn)
-        ffn, _ = self._norm_linear(self.w2, x13, self.ffn_sub_norm, glu=True)
+            if self.capture is not None:
+                self.capture.append(("attention", None, None, o))
+            attn, _ = self._norm_linear(self.wo, o.contiguous(), self.attn_sub_norm, name="wo")
+        x13, x = self._norm_linear(self.w13, x, self.ffn_norm, residual=attn, name="w13")
+        ffn, _ = self._norm_linear(self.w2, x13, self.ffn_sub_norm, glu=True, name="w2")
         return x, ffn
 
 
@@ -344,6 +433,13 @@ class Transformer:
             units = (ctypes.c_longlong * count)(*[u for _, u in regions])
             blk.prefetch = (ptrs, sizes, units, count)
 
+    def chain_supported(self) -> bool:
+        """Shapes ternaspmm_fused_linear takes for every linear of a block (see include/ternaspmm.h)."""
+        a = self.args
+        qd = a.n_heads * a.head_dim
+        return (a.dim % 64 == 0 and qd % 64 == 0 and a.ffn_dim % 64 == 0 and a.dim <= 2560 and qd <= 2560 and a.ffn_dim <= 7168
+                and a.dim // 16 <= 448 and a.ffn_dim // 16 <= 448)
+
     def rope_tables(self, max_seq: int, dev):
         """cos / sin of every (cache slot, rotary pair): fp32 [max_seq, 2, head_dim / 2] (cos row, sin row), built
         once per length; one gather then fetches both rows of a position."""
@@ -367,20 +463,22 @@ class Transformer:
         splits = getattr(self, "attention_splits", None) or lib.ternaspmm_attention_partial_splits(bsz, a.n_heads, max_seq)
         if splits <= 1:
             return None
-        held = getattr(self, "_attn_partial", None)
-        if held is None or held[0] != bsz:
+        # one buffer per batch size, kept while the model lives: a captured decode graph holds the raw pointer
+        held = self.__dict__.setdefault("_attn_partial", {})
+        if bsz not in held:
             nbytes = lib.ternaspmm_attention_partial_bytes(bsz, a.n_heads, a.head_dim)
-            self._attn_partial = held = (bsz, torch.empty(nbytes // 4, dtype=torch.float32, device="cuda"))
-        return held[1], splits
+            held[bsz] = torch.empty(nbytes // 4, dtype=torch.float32, device="cuda")
+        return held[bsz], splits
 
     def attention_workspace(self, bsz: int):
-        """Zero-filled scratch of the single-token attention (split over the cache); one per batch size."""
-        ws = getattr(self, "_attn_ws", None)
-        if ws is None or ws[0] != bsz:
+        """Zero-filled scratch of the single-token attention (split over the cache); one per batch size, kept while
+        the model lives (a captured decode graph holds the raw pointer)."""
+        held = self.__dict__.setdefault("_attn_ws", {})
+        if bsz not in held:
             a = self.args
             nbytes = _lib.load().ternaspmm_attention_workspace_bytes(bsz, a.n_heads, a.head_dim)
-            self._attn_ws = ws = (bsz, torch.zeros(nbytes, dtype=torch.int8, device="cuda"))
-        return ws[1]
+            held[bsz] = torch.zeros(nbytes, dtype=torch.int8, device="cuda")
+        return held[bsz]
 
     def make_cache(self, bsz: int, max_seq: int):
         a = self.args
@@ -418,9 +516,16 @@ class Transformer:
         # 1500: 1943 -> 1713 us per step; at slot 255 of 384 the pair of launches is 1.5 us slower than the unsplit one)
         if one_launch_attention and self.layers[0].act == "int8" and (bsz == 1 or max_seq > 1024):
             attn_ws = self.attention_partial(bsz, max_seq) or attn_ws
+        # one new token for up to 8 sequences: the linears chained through producer-side norm statistics (forward_chain)
+        chain = one_launch_attention and self.layers[0].act == "int8" and bsz <= 8 and getattr(self, "chain", True) and self.chain_supported()
+        stats = None
         for index, (layer, (ck, cv)) in enumerate(zip(self.layers, cache)):
             x_in, pending_in = x, pending
-            x, pending = layer.forward(x, pending, ck, cv, pos_idx, cos, sin, mask, attn_ws)
+            if chain:
+                nxt = self.layers[index + 1].attention_norm if index + 1 < len(self.layers) else self.norm
+                x, stats = layer.forward_chain(x, stats, ck, cv, pos_idx, cos, sin, attn_ws, nxt)
+            else:
+                x, pending = layer.forward(x, pending, ck, cv, pos_idx, cos, sin, mask, attn_ws)
             if trace is not None:
                 trace(index, x_in, pending_in, x, pending)
         if last_idx is not None:                                              # padded prompts: each sequence's own last token
@@ -429,7 +534,7 @@ class Transformer:
         elif t > 1:                                                           # only the last new token feeds the head
             x, pending = x.view(bsz, t, a.dim)[:, -1].contiguous(), pending.view(bsz, t, a.dim)[:, -1].contiguous()
         if self.layers[0].fused and x.is_cuda:                                # last residual add + final norm: one launch
-            x, _ = rmsnorm_quant(x, self.norm, a.norm_eps, residual=pending, quant=False)
+            x, _ = rmsnorm_quant(x, self.norm, a.norm_eps, residual=pending, quant=False)     # (chain: pending is None, the stream has it)
         else:
             x = rms_norm(x + pending, self.norm, a.norm_eps)
         if x.is_cuda and bsz <= 16 and a.dim % 32 == 0 and bsz * (2 * a.dim + 16) <= 160 * 1024:

@@ -397,7 +397,7 @@ def test_quant_modes_of_the_prologue_kernels(lib, mode):
         _, y, q, s = _run(lib, x, w, 1e-5)
         want_q, want_s = O.quant_input(y, mode)
         assert (s == want_s).all() and (q == want_q).all()
-        assert 0.005 < (q != q0).mean() < 0.2                       # not the default rule's integers
+        assert 0 < (q != q0).mean() < 0.2                           # not the default rule's integers
         _, y, q, s = _run(lib, x13, wf, 1e-5, glu=True)
         want_q, want_s = O.quant_input(y, mode)
         assert (s == want_s).all() and (q == want_q).all()
