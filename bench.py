@@ -49,7 +49,8 @@ METRIC = "TernaSpMM GB/s + %HBM roofline (M=8,K=N=2560); 2B-shape decode tok/s"
 # a counter measurement, not part of this run -- two rocprofv3 --pmc runs of this file (FETCH_SIZE, WRITE_SIZE),
 # scaled by what the same counters read for a 256 MiB copy.  Quoted with its source; null for any other workload.
 TRAFFIC = {"bytes_per_launch": (19206.6 + 356.0) * 1024 / 4,
-           "source": "profiles/decode_packed_kernel_hbm_traffic.md (two rocprofv3 --pmc runs, FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 by the copy probe)"}
+           "source": "profiles/decode_packed_kernel_hbm_traffic.md (two rocprofv3 --pmc runs, FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 by the copy probe)",
+           "measured_at": "the tree of commit 772a0ab; csrc/decode_packed_kernel.h and launch_decode_packed.hip are unchanged since"}
 
 
 def vp(t):
@@ -133,6 +134,25 @@ class Matrix:
             vals, off, med, bm = self.dev[copy]
             lib.bitlinear_TernaSpMM_bf16(vp(x), vp(bm), vp(off), vp(med), vp(vals), vp(out), vp(self.scale),
                                          1, m, self.n, self.k, 1, None, stream)
+
+
+def golden_gate(mats, what):
+    """The correctness gate of a timed leg, on the outputs its launches left: every matrix against the float64
+    evaluation of X (bf16) x W^T (the host's ternary matrix) x scale, max |err| <= 1e-2 max |ref| and a median error of
+    at most one bf16 step.  numpy only.  Returns max err / max |ref| per matrix."""
+    ratios = {}
+    for mat in mats:
+        x = (mat.x_bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+        golden = x @ mat.w.astype(np.float64).T * float(mat.scale_host[0])
+        bits = mat.out.cpu().numpy().view(np.uint16)
+        got = (bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+        max_ref, max_err = np.abs(golden).max(), np.abs(got - golden).max()
+        assert max_err <= 1e-2 * max_ref, f"{what}, {mat.name}: max_err {max_err} vs max_ref {max_ref}"
+        want = f32_to_bf16_bits(golden.astype(np.float32)).astype(np.int32)
+        key = lambda u: np.where(u & 0x8000, -(u & 0x7FFF), u & 0x7FFF)
+        assert np.median(np.abs(key(bits.astype(np.int32)) - key(want))) <= 1, f"{what}, {mat.name}: median error above one bf16 step"
+        ratios[mat.name] = float(max_err / max_ref)
+    return ratios
 
 
 def time_graph(torch, graph, replays, warmup):
@@ -381,13 +401,13 @@ class PrefillSet:
         except Exception:                                   # no such vendor kernel in this build
             return None
 
-    def shape_us(self, lib, mt, xs, act, m, layout="packed", route=0, reps=10):
+    def shape_us(self, lib, mt, xs, act, m, layout="packed", route=0, reps=10, replays=5, warmup=2):
         torch = self.torch
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
         self.launch(lib, mt, xs, act, m, stream, layout, route)
         torch.cuda.synchronize()
         g = capture(torch, lambda s: [self.launch(lib, mt, xs, act, m, s, layout, route) for _ in range(reps)])
-        return time_graph(torch, g, 5, 2) * 1e3 / reps
+        return time_graph(torch, g, replays, warmup) * 1e3 / reps
 
     def step(self, lib, act, m, steps, warmup, layout="packed"):
         """One pass over the four matrices at M = m, graph-replayed: (ms per step, flops per step)."""
@@ -395,6 +415,37 @@ class PrefillSet:
         graph = capture(torch, lambda s: [self.launch(lib, mt, xs, act, m, s, layout) for mt, xs in self.mats])
         ms = time_graph(torch, graph, steps, warmup)
         return ms, sum(2.0 * m * mt.n * mt.k for mt, _ in self.mats)
+
+    def dense_step(self, act, m, steps, warmup):
+        """The vendor's dense GEMM on the same four shapes in the SAME protocol: one graph of the four calls (operands
+        and outputs allocated beforehand), replayed `steps` times after `warmup`.  ms per step, or None."""
+        torch = self.torch
+        try:
+            ops = []
+            for mt, _ in self.mats:
+                if act == "bf16":
+                    a = torch.randn(m, mt.k, device="cuda", dtype=torch.bfloat16)
+                    b = torch.randn(mt.n, mt.k, device="cuda", dtype=torch.bfloat16).t()
+                    o = torch.empty(m, mt.n, device="cuda", dtype=torch.bfloat16)
+                    ops.append((torch.matmul, a, b, o))
+                else:
+                    a = torch.randint(-127, 128, (m, mt.k), device="cuda", dtype=torch.int8)
+                    b = torch.randint(-1, 2, (mt.n, mt.k), device="cuda", dtype=torch.int8).t()
+                    o = torch.empty(m, mt.n, device="cuda", dtype=torch.int32)
+                    ops.append((torch._int_mm, a, b, o))
+            run = lambda: [f(a, b, out=o) for f, a, b, o in ops]
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                run()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                run()
+            return time_graph(torch, g, steps, warmup)
+        except Exception:                                   # no such vendor kernel in this build
+            return None
 
 
 def prefill_figures(ps, lib, act, m, steps, warmup, per_shape=True, layout="packed"):
@@ -404,17 +455,27 @@ def prefill_figures(ps, lib, act, m, steps, warmup, per_shape=True, layout="pack
     out = {"act": act, "m": m, "ms_per_step": ms, "rate": rate, "unit": "TFLOP/s" if act == "bf16" else "TOP/s",
            "peak": peak, "frac": rate / peak}
     if per_shape:
-        shapes, dense_total = {}, 0.0
+        shapes, dense_total, own_total = {}, 0.0, 0.0
         for mt, xs in ps.mats:
-            us = ps.shape_us(lib, mt, xs, act, m, layout)
-            d_us = ps.dense_us(act, m, mt.n, mt.k)
+            us = ps.shape_us(lib, mt, xs, act, m, layout, replays=10, warmup=3)           # 100 timed launches per shape
+            d_us = ps.dense_us(act, m, mt.n, mt.k, reps=30)
             tf = 2.0 * m * mt.n * mt.k / us / 1e6
             shapes[f"{mt.name}_{mt.k}x{mt.n}"] = {"us": us, "rate": tf, "frac": tf / peak, "vendor_dense_gemm_us": d_us}
             dense_total = None if (d_us is None or dense_total is None) else dense_total + d_us
+            own_total += us
         out["per_shape"] = shapes
-        out["vendor_dense_gemm"] = None if not dense_total else {
-            "what": "torch.matmul (bf16) / torch._int_mm (int8) on already expanded weights, same four shapes, eager",
-            "ms_per_step": dense_total * 1e-3, "rate": flops / (dense_total * 1e-6) / 1e12}
+        # the step (a graph of the four launches, one after the other) and the sum of the four shapes timed alone,
+        # side by side: the clock under matrix load moves the former more than the latter
+        out["per_shape_sum"] = {"ms": own_total * 1e-3, "rate": flops / (own_total * 1e-6) / 1e12,
+                                "frac": flops / (own_total * 1e-6) / 1e12 / peak}
+        d_ms = ps.dense_step(act, m, steps, warmup)
+        out["vendor_dense_gemm"] = None if (not dense_total and d_ms is None) else {
+            "what": "torch.matmul (bf16) / torch._int_mm (int8) on already expanded weights, same four shapes: "
+                    "ms_per_step = one graph of the four calls, timed exactly as this kernel's step; per_shape_sum_ms = "
+                    "the four shapes timed alone (eager, 30 calls each)",
+            "ms_per_step": d_ms, "rate": None if d_ms is None else flops / (d_ms * 1e-3) / 1e12,
+            "per_shape_sum_ms": None if not dense_total else dense_total * 1e-3,
+            "per_shape_sum_rate": None if not dense_total else flops / (dense_total * 1e-6) / 1e12}
     return out
 
 
@@ -512,6 +573,21 @@ def calibration(torch, lib):
         out[name] = moved * 5 / (e0.elapsed_time(e1) * 1e-3) / 1e9
     out["read_copy_bytes"] = nbytes
     del a, b
+    # the rate of the library's own largest stream: the bf16 LM head of the 2B shape, 128256 x 2560, one row of activations
+    from ternainfer_amd.linear import lm_head
+    w = torch.randn((128256, 2560), device="cuda", dtype=torch.bfloat16)
+    x = torch.randn((1, 2560), device="cuda", dtype=torch.bfloat16)
+    lg = torch.empty((1, 128256), device="cuda", dtype=torch.bfloat16)
+    lm_head(x, w, lg)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(20):
+        lm_head(x, w, lg)
+    e1.record()
+    torch.cuda.synchronize()
+    out["lm_head_stream_GBps"] = w.numel() * 2 * 20 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+    del w, x, lg
     # device-wide synchronisation among co-resident workgroups (one per CU): what a persistent kernel would pay
     # between two dependent phases, to hold against the cost of a graph kernel node
     state = torch.zeros(lib.ternaspmm_probe_barrier_state_bytes() // 4, dtype=torch.int32, device="cuda")
@@ -688,6 +764,7 @@ def main():
                      "frac": gbps / HBM_PEAK_GBPS,
                      "traffic": TRAFFIC["bytes_per_launch"] if default_workload else None,
                      "traffic_source": TRAFFIC["source"] if default_workload else None,
+                     "traffic_measured_at": TRAFFIC["measured_at"] if default_workload else None,
                      "kernel": ("terna_decode_packed_kernel<bf16>" if args.layout == "packed"
                                 else "terna_decode_kernel<bf16>"),
                      "algorithmic_bytes_per_launch": step_bytes / launches_per_step,
@@ -727,10 +804,17 @@ def main():
             "the same step through bitlinear_TernaSpMM_bf16 on reference-format pointers, repack cache off: the kernels that "
             "read the reference format directly")
         lib.ternaspmm_repack_cache_enable(1)
+        for mt in mats:
+            mt.out.fill_(-1)                             # poison: the leg's own launches must produce the checked outputs
         result["drop_in_reference_format"] = as_figures(
             layer_set_step(torch, lib, mats, args.layers, "reference", args.m, half, 2),
             "the same step through bitlinear_TernaSpMM_bf16 on reference-format pointers as an unmodified call site issues it "
             "(library defaults: every weight repacked once on first sight, every launch re-checks the copy's fingerprint)")
+        result["drop_in_reference_format"]["parity_max_err_over_max_ref"] = golden_gate(mats, "drop-in leg")
+        stats = (ctypes.c_longlong * 6)()
+        lib.ternaspmm_repack_cache_stats(stats)
+        result["drop_in_reference_format"]["repack_cache"] = {"copies": stats[0], "bytes": stats[1], "dropped_as_stale": stats[2]}
+        assert stats[0] == args.layers * len(mats) and stats[2] == 0
         lib.ternaspmm_repack_cache_enable(0)
         lib.ternaspmm_repack_cache_clear()
         by_m = {}
@@ -750,7 +834,7 @@ def main():
         result["config1"] = config1_row(torch, T, lib)
         torch.cuda.empty_cache()
         ps = PrefillSet(torch, T, [2048])
-        result["prefill_m2048"] = {act: prefill_figures(ps, lib, act, 2048, 10, 3) for act in ("bf16", "int8")}
+        result["prefill_m2048"] = {act: prefill_figures(ps, lib, act, 2048, 50, 10) for act in ("bf16", "int8")}
         del ps
         torch.cuda.empty_cache()
         model = None

@@ -17,39 +17,49 @@ namespace {
 __global__ void terna_probe_empty_kernel() {}
 
 constexpr int kProbeThreads = 256;
-constexpr int kProbeUnroll = 8;              // 16-byte vectors in flight per thread
+constexpr int kProbeUnroll = 16;             // 16-byte vectors in flight per thread
+constexpr long long kProbeTile = static_cast<long long>(kProbeThreads) * kProbeUnroll;     // vectors per tile: 64 KB, contiguous
 
-// Grid-stride read of `vecs` 16-byte vectors; the sum is written only if it takes a value it never takes.
+// Streaming read of `vecs` 16-byte vectors.  A workgroup takes contiguous 64 KB tiles (tile t, t + grid, ...): every
+// load of a wave is one contiguous kilobyte and the sixteen loads a thread has in flight stay inside one tile -- the
+// access pattern of the streaming kernels here (a lane walks along a weight row), and the one that reaches the rate
+// those kernels reach; vectors a grid apart (8 MB strides, sixteen distant regions per workgroup at a time) measured
+// 20 % lower.  Non-temporal loads: nothing is read twice.  The sum is written only if it takes a value it never takes.
 __global__ __launch_bounds__(kProbeThreads) void terna_probe_read_kernel(const u32x4* __restrict__ src, long long vecs,
                                                                        u32x4* __restrict__ sink)
 {
-    const long long stride = static_cast<long long>(gridDim.x) * kProbeThreads;
     u32x4 acc = {0u, 0u, 0u, 0u};
-    long long i = static_cast<long long>(blockIdx.x) * kProbeThreads + threadIdx.x;
-    for (; i + (kProbeUnroll - 1) * stride < vecs; i += kProbeUnroll * stride) {
+    const long long tiles = vecs / kProbeTile;
+    for (long long t = blockIdx.x; t < tiles; t += gridDim.x) {
+        const u32x4* p = src + t * kProbeTile + threadIdx.x;
         u32x4 v[kProbeUnroll];
 #pragma unroll
-        for (int u = 0; u < kProbeUnroll; ++u) v[u] = src[i + u * stride];
+        for (int u = 0; u < kProbeUnroll; ++u) v[u] = __builtin_nontemporal_load(p + u * kProbeThreads);
 #pragma unroll
         for (int u = 0; u < kProbeUnroll; ++u) acc ^= v[u];
     }
-    for (; i < vecs; i += stride) acc ^= src[i];
+    for (long long i = tiles * kProbeTile + static_cast<long long>(blockIdx.x) * kProbeThreads + threadIdx.x; i < vecs;
+         i += static_cast<long long>(gridDim.x) * kProbeThreads)
+        acc ^= src[i];
     if ((acc.x & acc.y & acc.z & acc.w) == 0xFFFFFFFFu && sink != nullptr) sink[0] = acc;   // practically never: keeps the loads alive
 }
 
 __global__ __launch_bounds__(kProbeThreads) void terna_probe_copy_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst,
                                                                        long long vecs)
 {
-    const long long stride = static_cast<long long>(gridDim.x) * kProbeThreads;
-    long long i = static_cast<long long>(blockIdx.x) * kProbeThreads + threadIdx.x;
-    for (; i + (kProbeUnroll - 1) * stride < vecs; i += kProbeUnroll * stride) {
+    const long long tiles = vecs / kProbeTile;
+    for (long long t = blockIdx.x; t < tiles; t += gridDim.x) {
+        const u32x4* p = src + t * kProbeTile + threadIdx.x;
+        u32x4* q = dst + t * kProbeTile + threadIdx.x;
         u32x4 v[kProbeUnroll];
 #pragma unroll
-        for (int u = 0; u < kProbeUnroll; ++u) v[u] = src[i + u * stride];
+        for (int u = 0; u < kProbeUnroll; ++u) v[u] = __builtin_nontemporal_load(p + u * kProbeThreads);
 #pragma unroll
-        for (int u = 0; u < kProbeUnroll; ++u) dst[i + u * stride] = v[u];
+        for (int u = 0; u < kProbeUnroll; ++u) __builtin_nontemporal_store(v[u], q + u * kProbeThreads);
     }
-    for (; i < vecs; i += stride) dst[i] = src[i];
+    for (long long i = tiles * kProbeTile + static_cast<long long>(blockIdx.x) * kProbeThreads + threadIdx.x; i < vecs;
+         i += static_cast<long long>(gridDim.x) * kProbeThreads)
+        dst[i] = src[i];
 }
 
 // `rounds` device-wide synchronisations among the workgroups of the grid (all co-resident: the host caps the grid
