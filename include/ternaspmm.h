@@ -262,6 +262,9 @@ int bitlinear_TernaSpMM_packed_fused_glu(const terna_bf16* x13, const terna_bf16
  *                                           (attention_splits, head_dim; M = 1), merged inside, statistics taken inside
  *             TERNASPMM_PROLOGUE_STATS      x = h bf16 [M][K] with its partials stats_in fp32 [M][stats_count][2]
  *                                           (stats_count <= 448), as a producing epilogue or ternaspmm_row_stats left them
+ *             TERNASPMM_PROLOGUE_QUANTISED  x = int8 [M][K] with its scales s_in bf16 [M] (ternaspmm_quant_from_stats,
+ *                                           ternaspmm_rmsnorm_quant): no prologue; M <= 16, any K the int8 kernels take,
+ *                                           only with TERNASPMM_EPILOGUE_RESIDUAL
  *   epilogue  TERNASPMM_EPILOGUE_STORE      out bf16 [M][N] = the linear's output (decode rule, Reduction_Kernel.cuh:60)
  *             TERNASPMM_EPILOGUE_RESIDUAL   out bf16 [M][N] = bf16(residual + output): the residual stream after this
  *                                           linear (model.py:330, :334); stats_out fp32 [M][N/16][2] = its partials under
@@ -274,7 +277,7 @@ int bitlinear_TernaSpMM_packed_fused_glu(const terna_bf16* x13, const terna_bf16
  * combination or the shape is not supported and nothing was enqueued (supported: K <= 2560 for every combination,
  * K <= 7168 for TERNASPMM_PROLOGUE_STATS with STORE / RESIDUAL; GATE needs PROLOGUE_STATS; PROLOGUE_NORM here only with
  * EPILOGUE_RESIDUAL).  out must not alias x or residual.  Only enqueues. */
-enum { TERNASPMM_PROLOGUE_NORM = 0, TERNASPMM_PROLOGUE_ATTENTION = 1, TERNASPMM_PROLOGUE_STATS = 2 };
+enum { TERNASPMM_PROLOGUE_NORM = 0, TERNASPMM_PROLOGUE_ATTENTION = 1, TERNASPMM_PROLOGUE_STATS = 2, TERNASPMM_PROLOGUE_QUANTISED = 3 };
 enum { TERNASPMM_EPILOGUE_STORE = 0, TERNASPMM_EPILOGUE_RESIDUAL = 1, TERNASPMM_EPILOGUE_GATE = 2 };
 typedef struct ternaspmm_fused_linear_desc {
     int prologue, epilogue;
@@ -295,8 +298,16 @@ typedef struct ternaspmm_fused_linear_desc {
     terna_bf16* raw_out;              /* EPILOGUE_RESIDUAL, optional */
     int8_t* xq_out;                   /* optional pair: the quantised activations as published by the first workgroup */
     terna_bf16* s_out;
+    const terna_bf16* s_in;           /* PROLOGUE_QUANTISED: bf16 [M], the scales that go with x = int8 [M][K] */
 } ternaspmm_fused_linear_desc;
 int ternaspmm_fused_linear(const ternaspmm_fused_linear_desc* desc, terna_stream stream);
+
+/* Norm + quant_input of h bf16 [M][K] as a launch of its own, from partials a producer left: xq_out int8 [M][K], s_out bf16 [M]
+ * -- the values the TERNASPMM_PROLOGUE_STATS prologue forms inside its launch (same order of additions), for row counts at
+ * which every consuming workgroup repeating the element-wise work costs more than one more launch (measured on MI355X: the
+ * down projection, K = 6912, from five rows on).  Returns 0 / -1.  Only enqueues. */
+int ternaspmm_quant_from_stats(const terna_bf16* h, const float* stats, int stats_count, const terna_bf16* norm_weight, float eps,
+                               int8_t* xq_out, terna_bf16* s_out, int M, int K, terna_stream stream);
 
 /* Partials of a row block no producing epilogue wrote (the embedding rows in front of the first block): per row and per
  * 512 columns (sum of h^2, max |h * norm_weight|) -> stats_out fp32 [M][ternaspmm_row_stats_count(K)][2].  Returns that
@@ -476,8 +487,13 @@ int ternaspmm_plan_reference_call(int int8_activations, int route, int M, int N,
  * What the machine gives, measured by the same library in the same run as the kernels a benchmark prices:
  *   ternaspmm_probe_empty    enqueues an empty kernel (one wave): N of them in a captured graph, replayed, give the
  *                            cost of one graph kernel node -- the floor under every launch of a decode step;
+ *   ternaspmm_probe_empty_shape  the same with a launch shape: `workgroups` of `threads` (a multiple of 64, at most 1024)
+ *                            with `lds_bytes` (at most 64 KB) of LDS each and an empty body -- the floor under a
+ *                            kernel of that shape (dispatch of its waves, LDS allocation, end of kernel).  0 / -1;
  *   ternaspmm_probe_read     streams `bytes` (16-byte aligned) through the chip and discards them: the read rate;
  *                            `sink` (16 bytes, may be NULL) is written practically never;
+ *   ternaspmm_probe_read_grid  the same stream read by a given number of workgroups (1 .. 4096): the rate ONE CU sustains
+ *                            (64 KB in flight per workgroup) and how it adds up.  0 / -1;
  *   ternaspmm_probe_copy     dst <- src, `bytes` each: the read + write rate;
  *   ternaspmm_probe_barrier  `rounds` device-wide synchronisations among `workgroups` co-resident workgroups (at most
  *                            one per CU, at most 256) through flags in `state` (ternaspmm_probe_barrier_state_bytes()
@@ -487,7 +503,9 @@ int ternaspmm_plan_reference_call(int int8_activations, int route, int M, int N,
  *                            Returns 0, or -1 when the arguments are refused.
  * All only enqueue; time them with events on `stream`. */
 void ternaspmm_probe_empty(terna_stream stream);
+int ternaspmm_probe_empty_shape(int workgroups, int threads, int lds_bytes, terna_stream stream);
 void ternaspmm_probe_read(const void* src, long long bytes, void* sink, terna_stream stream);
+int ternaspmm_probe_read_grid(const void* src, long long bytes, void* sink, int workgroups, terna_stream stream);
 void ternaspmm_probe_copy(const void* src, void* dst, long long bytes, terna_stream stream);
 size_t ternaspmm_probe_barrier_state_bytes(void);
 int ternaspmm_probe_barrier(void* state, int workgroups, int rounds, unsigned first_tag, terna_stream stream);

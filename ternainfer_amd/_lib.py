@@ -64,7 +64,9 @@ PROTOTYPES = {
     "ternaspmm_decode_attention_static": ([_vp] * 4 + [_ci, _vp] + [_ci] * 5 + [ctypes.c_float, _vp], ctypes.c_int),
     "ternaspmm_attention_workspace_bytes": ([_ci, _ci, _ci], ctypes.c_longlong),
     "ternaspmm_probe_empty": ([_vp], None),
+    "ternaspmm_probe_empty_shape": ([_ci, _ci, _ci, _vp], _ci),
     "ternaspmm_probe_read": ([_vp, ctypes.c_longlong, _vp, _vp], None),
+    "ternaspmm_probe_read_grid": ([_vp, ctypes.c_longlong, _vp, _ci, _vp], _ci),
     "ternaspmm_probe_copy": ([_vp, _vp, ctypes.c_longlong, _vp], None),
     "ternaspmm_probe_barrier_state_bytes": ([], ctypes.c_size_t),
     "ternaspmm_probe_barrier": ([_vp, _ci, _ci, ctypes.c_uint, _vp], ctypes.c_int),
@@ -75,6 +77,7 @@ PROTOTYPES = {
     "ternaspmm_plan_reference_call": ([_ci] * 6 + [_vp, _ci, _vp], _ci),
     "ternaspmm_quant_mode": ([_ci], _ci),
     "ternaspmm_fused_linear": ([_vp, _vp], _ci),
+    "ternaspmm_quant_from_stats": ([_vp, _vp, _ci, _vp, ctypes.c_float, _vp, _vp, _ci, _ci, _vp], _ci),
     "ternaspmm_row_stats_count": ([_ci], _ci),
     "ternaspmm_row_stats": ([_vp, _vp, _vp, _ci, _ci, _vp], _ci),
     "ternaspmm_interleave_gate_up": ([_vp, _vp, _ci, _ci, _vp], _ci),

@@ -9,6 +9,7 @@
 #include "../../include/ternaspmm.h"
 #include "host_util.h"
 #include "decode_fused_kernel.h"
+#include "launchers.h"
 
 using namespace terna;
 
@@ -53,6 +54,54 @@ __global__ __launch_bounds__(256) void terna_interleave_gate_up_kernel(const uin
     const u32x4* s4 = reinterpret_cast<const u32x4*>(src + src_band * words);
     u32x4* d4 = reinterpret_cast<u32x4*>(dst + dst_band * words);
     for (size_t q = threadIdx.x; q < words / 4; q += 256) d4[q] = s4[q];
+}
+
+// Norm + quantisation of h [M][K] as a launch of its own, from the producer's partials (no reduction over the row here):
+// for row counts at which every consuming workgroup repeating the element-wise work costs more than this launch.
+// Grid (M, ceil(K / 2048)); every wave adds up the partials of its row in the same fixed order as the FUSED_STATS
+// prologue, so the (xq, s) written here are the ones that prologue would have formed.
+__global__ __launch_bounds__(256) void terna_quant_stats_kernel(const uint16_t* __restrict__ h, const float2* __restrict__ stats, int count,
+                                                                 const uint16_t* __restrict__ norm_w, int K, float eps,
+                                                                 int8_t* __restrict__ xq_out, uint16_t* __restrict__ s_out, int quant_mode)
+{
+    const int lane = threadIdx.x & 63;
+    const size_t row = blockIdx.x;
+    const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
+    const bool in = c < K;                                       // K is a multiple of 8
+    const u32x4 hv = *reinterpret_cast<const u32x4*>(h + row * K + (in ? c : 0));
+    const u32x4 wv = *reinterpret_cast<const u32x4*>(norm_w + (in ? c : 0));
+    constexpr int PT = kStatsMaxPartials / 64;
+    float2 part[PT];
+#pragma unroll
+    for (int t = 0; t < PT; ++t) {
+        const int idx = lane + 64 * t;
+        part[t] = stats[row * count + (idx < count ? idx : 0)];
+    }
+    float sum = 0.0f, pmax = 0.0f;
+#pragma unroll
+    for (int t = 0; t < PT; ++t) {
+        if (lane + 64 * t < count) {
+            sum += part[t].x;
+            pmax = fmaxf(pmax, part[t].y);
+        }
+    }
+    sum = wave_sum(sum);
+    pmax = wave_max(pmax);
+    const float rstd = rsqrtf(sum / static_cast<float>(K) + eps);
+    uint16_t sb;
+    const float s = quant_scale(fabsf(round_bf16(__fmul_rn(pmax, rstd))), quant_mode, &sb);
+    if (blockIdx.y == 0 && threadIdx.x == 0) s_out[row] = sb;
+    if (!in) return;
+    float f[8], w[8];
+    unpack_bf16x8(hv, f);
+    unpack_bf16x8(wv, w);
+    uint32_t d[2] = {0u, 0u};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const float y = round_bf16(__fmul_rn(__fmul_rn(f[e], w[e]), rstd));
+        d[e >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(quant_value(y, s, quant_mode) + 128.0f, e & 3, d[e >> 2]);
+    }
+    *reinterpret_cast<u32x2*>(xq_out + row * K + c) = u32x2{d[0] ^ 0x80808080u, d[1] ^ 0x80808080u};
 }
 
 // One launch of terna_decode_fused_kernel<WAVES, TMAX, MODE, MP, NB, ASP, AHD, EPI> with MP picked by M (1, 2, 4, 8).
@@ -139,12 +188,41 @@ int ternaspmm_interleave_gate_up(const void* packed, void* packed_out, int N, in
     return 0;
 }
 
+int ternaspmm_quant_from_stats(const terna_bf16* h, const float* stats, int stats_count, const terna_bf16* norm_weight, float eps,
+                               int8_t* xq_out, terna_bf16* s_out, int M, int K, terna_stream stream)
+{
+    if (M < 1 || K < 8 || (K & 7) || stats_count < 1 || stats_count > kStatsMaxPartials || h == nullptr || stats == nullptr ||
+        norm_weight == nullptr || xq_out == nullptr || s_out == nullptr) {
+        std::fprintf(stderr, "ternaspmm_quant_from_stats: unsupported arguments (M=%d K=%d partials=%d)\n", M, K, stats_count);
+        return -1;
+    }
+    terna_quant_stats_kernel<<<dim3(M, (K + 2047) / 2048), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+        h, reinterpret_cast<const float2*>(stats), stats_count, norm_weight, K, eps, xq_out, s_out, quant_mode());
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_quant_from_stats", e, __LINE__);
+    return 0;
+}
+
 int ternaspmm_fused_linear(const ternaspmm_fused_linear_desc* d, terna_stream stream)
 {
     if (d == nullptr) return -1;
     const int M = d->M, N = d->N, K = d->K;
-    if (!shape_ok(M, N, K) || !groups_ok(d->ws_num) || M > 8) return -1;
     const int pro = d->prologue, epi = d->epilogue;
+    if (pro == TERNASPMM_PROLOGUE_QUANTISED) {
+        // activations already quantised (ternaspmm_quant_from_stats, ternaspmm_rmsnorm_quant): the small-M kernel of
+        // bitlinear_TernaSpMM_packed with the producing epilogue
+        if (!shape_ok(M, N, K) || !groups_ok(d->ws_num) || !i8_depth_ok(K) || M > 16 || epi != TERNASPMM_EPILOGUE_RESIDUAL ||
+            d->x == nullptr || d->s_in == nullptr || d->packed == nullptr || d->ws == nullptr || d->out == nullptr ||
+            d->residual == nullptr || d->next_norm_weight == nullptr || d->stats_out == nullptr || N / 16 > kStatsMaxPartials)
+            return -1;
+        const Epilogue ep{d->s_in, d->ws, nullptr, d->ws_num, EP_I8_DECODE};
+        launch_decode_packed_producer(static_cast<const int8_t*>(d->x), static_cast<const uint32_t*>(d->packed), d->out, ep, M, N, K,
+                                      d->residual, d->next_norm_weight, d->stats_out, d->raw_out, static_cast<hipStream_t>(stream));
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) die("ternaspmm_fused_linear", e, __LINE__);
+        return N / 16;
+    }
+    if (!shape_ok(M, N, K) || !groups_ok(d->ws_num) || M > 8) return -1;
     const int ktiles = K / 64, bands = N / 16;
     if (pro != TERNASPMM_PROLOGUE_NORM && pro != TERNASPMM_PROLOGUE_ATTENTION && pro != TERNASPMM_PROLOGUE_STATS) return -1;
     if (epi != TERNASPMM_EPILOGUE_STORE && epi != TERNASPMM_EPILOGUE_RESIDUAL && epi != TERNASPMM_EPILOGUE_GATE) return -1;

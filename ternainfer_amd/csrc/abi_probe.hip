@@ -16,6 +16,14 @@ namespace {
 
 __global__ void terna_probe_empty_kernel() {}
 
+// An empty body behind a launch of a given shape: what the dispatch of that many waves, the LDS allocation and the end
+// of the kernel cost before any work.  One lane touches the LDS so that the allocation is not optimised away.
+__global__ void terna_probe_empty_shape_kernel(int never)
+{
+    extern __shared__ uint32_t probe_lds[];
+    if (never) probe_lds[threadIdx.x] = 1u;
+}
+
 constexpr int kProbeThreads = 256;
 constexpr int kProbeUnroll = 16;             // 16-byte vectors in flight per thread
 constexpr long long kProbeTile = static_cast<long long>(kProbeThreads) * kProbeUnroll;     // vectors per tile: 64 KB, contiguous
@@ -124,6 +132,16 @@ void ternaspmm_probe_empty(terna_stream stream)
     if (e != hipSuccess) die("ternaspmm_probe_empty", e, __LINE__);
 }
 
+int ternaspmm_probe_empty_shape(int workgroups, int threads, int lds_bytes, terna_stream stream)
+{
+    if (workgroups < 1 || workgroups > (1 << 20) || threads < 64 || threads > 1024 || (threads & 63) || lds_bytes < 0 || lds_bytes > 64 * 1024)
+        return -1;
+    terna_probe_empty_shape_kernel<<<dim3(workgroups), dim3(threads), lds_bytes, static_cast<hipStream_t>(stream)>>>(0);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_probe_empty_shape", e, __LINE__);
+    return 0;
+}
+
 void ternaspmm_probe_read(const void* src, long long bytes, void* sink, terna_stream stream)
 {
     if (src == nullptr || bytes < 16 || (reinterpret_cast<uintptr_t>(src) & 15)) {
@@ -135,6 +153,16 @@ void ternaspmm_probe_read(const void* src, long long bytes, void* sink, terna_st
         static_cast<const u32x4*>(src), vecs, static_cast<u32x4*>(sink));
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_probe_read", e, __LINE__);
+}
+
+int ternaspmm_probe_read_grid(const void* src, long long bytes, void* sink, int workgroups, terna_stream stream)
+{
+    if (src == nullptr || bytes < 16 || (reinterpret_cast<uintptr_t>(src) & 15) || workgroups < 1 || workgroups > 4096) return -1;
+    terna_probe_read_kernel<<<workgroups, kProbeThreads, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<const u32x4*>(src), bytes / 16, static_cast<u32x4*>(sink));
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_probe_read_grid", e, __LINE__);
+    return 0;
 }
 
 void ternaspmm_probe_copy(const void* src, void* dst, long long bytes, terna_stream stream)

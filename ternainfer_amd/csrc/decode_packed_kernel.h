@@ -29,11 +29,23 @@ struct PackedRaw {
 // Argument order: pointers and integers first, the structures last -- the first sixteen dwords of the arguments
 // arrive preloaded in scalar registers, but only up to the first structure passed by value, and everything the first
 // global loads depend on should be among them.
-template <typename Act, int WAVES, int MB, int DEPTH, int NB = 1, bool GUARD = false>
+// RES: the launch is also the producer for the next one (int8 activations, one m-block): instead of its own output
+// it stores h' = bf16(residual[m][n] + out[m][n]), the residual stream after this linear (model.py:330, :334), and leaves
+// per row and 16-row band the partial (sum of h'^2, max |h' * next_w|) that the consumer's norm and quantisation need
+// (decode_fused_kernel.h has the consumer).
+struct PackedProducer {
+    const uint16_t* residual;        // bf16 [M][N]
+    const uint16_t* next_w;          // bf16 [N]: weights of the norm that follows
+    float2* stats_out;               // [M][N/16]
+    uint16_t* raw_out;               // optional: the linear's own output as well
+};
+
+template <typename Act, int WAVES, int MB, int DEPTH, int NB = 1, bool GUARD = false, bool RES = false>
 __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
     const Act* __restrict__ x, const uint32_t* __restrict__ packed, uint16_t* __restrict__ out,
-    int M, int N, int K, Epilogue ep, RepackGuard guard)
+    int M, int N, int K, Epilogue ep, RepackGuard guard, PackedProducer prod)
 {
+    static_assert(!RES || (MB == 1 && sizeof(Act) == 1), "the producing epilogue: int8 activations, up to 16 rows");
     // A launch on a cached P2 copy carries one extra workgroup in x -- the one past the last band -- that checks, next to
     // the others and off their critical path, that the copy still belongs to the caller's tensors.
     if constexpr (GUARD) {
@@ -162,6 +174,20 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
         const int m = m_base + (unit % MB) * 16 + i;
         eraw[e] = load_epilogue_raw(ep, m < M ? m : M - 1, (band0 + unit / MB) * 16 + 4 * g, N);
     }
+    // the producing epilogue's own operands -- four stream values, four weights of the next norm -- by the finishing
+    // waves (the others read one address: no traffic); requested with everything else, used at the very end
+    u32x2 eres[FIN], enw[FIN];
+    if constexpr (RES) {
+#pragma unroll
+        for (int e = 0; e < FIN; ++e) {
+            const int unit = wave + e * WAVES;
+            const bool fin = unit < UNITS;
+            const int n0 = (band0 + (fin ? unit : 0)) * 16 + 4 * g;
+            const int m = m_base + i;
+            enw[e] = *reinterpret_cast<const u32x2*>(prod.next_w + (fin ? n0 : 0));
+            eres[e] = *reinterpret_cast<const u32x2*>(prod.residual + (fin ? static_cast<size_t>(m < M ? m : 0) * N + n0 : 0));
+        }
+    }
 
     for (int j0 = 0; j0 < cnt; j0 += NBUF) {
         if constexpr (DEPTH == 3) {
@@ -195,7 +221,31 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
         for (int w = 1; w < WAVES; ++w) sum += red[w][unit][lane];
         const int m = m_base + (unit % MB) * 16 + i;
         const int n0 = (band0 + unit / MB) * 16 + 4 * g;
-        if (m < M) {
+        if constexpr (RES) {
+            // every lane takes part in the cross-lane sums; rows the batch does not have contribute zeros
+            const EpilogueRegs eregs = finish_epilogue(ep, eraw[e]);
+            uint16_t o[4];
+            float hv[4], ssq_o = 0.0f, pmax_o = 0.0f;
+            const uint32_t rbits[2] = {eres[e].x, eres[e].y}, wbits[2] = {enw[e].x, enw[e].y};
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                o[v] = apply_epilogue<int>(ep.kind, eregs, v, sum[v] >> kI8WeightShift);
+                const float rv = (v & 1) ? __uint_as_float(rbits[v >> 1] & 0xffff0000u) : __uint_as_float(rbits[v >> 1] << 16);
+                const float wv = (v & 1) ? __uint_as_float(wbits[v >> 1] & 0xffff0000u) : __uint_as_float(wbits[v >> 1] << 16);
+                hv[v] = m < M ? bf16_bits_to_float(float_to_bf16_bits(rv + bf16_bits_to_float(o[v]))) : 0.0f;
+                ssq_o = fmaf(hv[v], hv[v], ssq_o);
+                pmax_o = fmaxf(pmax_o, fabsf(__fmul_rn(hv[v], wv)));
+            }
+            ssq_o = cross_row_reduce<false>(ssq_o);              // the four lanes (g = 0 .. 3) of a batch row: the band's sixteen features
+            pmax_o = cross_row_reduce<true>(pmax_o);
+            if (m < M) {
+                *reinterpret_cast<u32x2*>(out + static_cast<size_t>(m) * N + n0) = u32x2{pack_bf16x2(hv[0], hv[1]), pack_bf16x2(hv[2], hv[3])};
+                if (prod.raw_out != nullptr)
+                    *reinterpret_cast<u32x2*>(prod.raw_out + static_cast<size_t>(m) * N + n0) =
+                        u32x2{o[0] | (static_cast<uint32_t>(o[1]) << 16), o[2] | (static_cast<uint32_t>(o[3]) << 16)};
+                if (g == 0) prod.stats_out[static_cast<size_t>(m) * (N / 16) + n0 / 16] = float2{ssq_o, pmax_o};
+            }
+        } else if (m < M) {
             const EpilogueRegs eregs = finish_epilogue(ep, eraw[e]);
             uint16_t o[4];
 #pragma unroll

@@ -19,9 +19,9 @@ void launch_decode_packed_as(const Act* x, const uint32_t* packed, uint16_t* out
 {
     const dim3 grid(N / 16 / NB + (guard != nullptr ? 1 : 0), (M + 16 * MB - 1) / (16 * MB));
     if (guard != nullptr)
-        terna_decode_packed_kernel<Act, WAVES, MB, DEPTH, NB, true><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, M, N, K, ep, *guard);
+        terna_decode_packed_kernel<Act, WAVES, MB, DEPTH, NB, true><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, M, N, K, ep, *guard, PackedProducer{});
     else
-        terna_decode_packed_kernel<Act, WAVES, MB, DEPTH, NB, false><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, M, N, K, ep, RepackGuard{});
+        terna_decode_packed_kernel<Act, WAVES, MB, DEPTH, NB, false><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, M, N, K, ep, RepackGuard{}, PackedProducer{});
 }
 
 template <typename Act>
@@ -53,6 +53,18 @@ void launch_decode_packed(const Act* x, const uint32_t* packed, uint16_t* out, c
     } else {
         launch_decode_packed_as<Act, 8, 4, 1>(x, packed, out, ep, M, N, K, guard, st);
     }
+}
+
+// The small-M int8 launch as a producer (residual add + the next norm's partial statistics in the epilogue): M <= 16.
+void launch_decode_packed_producer(const int8_t* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                                   const uint16_t* residual, const uint16_t* next_w, float* stats_out, uint16_t* raw_out, hipStream_t st)
+{
+    const PackedProducer prod{residual, next_w, reinterpret_cast<float2*>(stats_out), raw_out};
+    const dim3 grid(N / 16, 1);
+    if (N / 16 <= 256)
+        terna_decode_packed_kernel<int8_t, 16, 1, 3, 1, false, true><<<grid, dim3(16 * 64), 0, st>>>(x, packed, out, M, N, K, ep, RepackGuard{}, prod);
+    else
+        terna_decode_packed_kernel<int8_t, 8, 1, 2, 1, false, true><<<grid, dim3(8 * 64), 0, st>>>(x, packed, out, M, N, K, ep, RepackGuard{}, prod);
 }
 
 // one wave each: record the fingerprint of a weight's reference-format tensors / check it as a launch of its own

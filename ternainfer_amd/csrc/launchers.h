@@ -36,6 +36,10 @@ void launch_repack(const Weights& w, uint32_t* packed, int N, int K, hipStream_t
 template <typename Act>
 void launch_decode_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
                           hipStream_t st, const RepackGuard* guard = nullptr);
+// The small-M int8 launch with the producing epilogue (M <= 16): out = bf16(residual + output), stats_out [M][N/16][2] under
+// next_w; raw_out (optional) the output itself.
+void launch_decode_packed_producer(const int8_t* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                                   const uint16_t* residual, const uint16_t* next_w, float* stats_out, uint16_t* raw_out, hipStream_t st);
 // Fingerprint of the reference-format tensors named by `guard` into *out / the check of it as a launch of its own.
 void launch_repack_fingerprint(const RepackGuard& guard, unsigned long long* out, hipStream_t st);
 void launch_repack_guard(const RepackGuard* guard, hipStream_t st);

@@ -260,10 +260,10 @@ class FusedLinearDesc(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int) for n in ("prologue", "epilogue", "M", "N", "K", "ws_num")] + [("eps", ctypes.c_float)] + \
                [(n, ctypes.c_int) for n in ("stats_count", "attention_splits", "head_dim")] + \
                [(n, ctypes.c_void_p) for n in ("x", "stats_in", "norm_weight", "packed", "ws", "out", "residual",
-                                               "next_norm_weight", "stats_out", "raw_out", "xq_out", "s_out")]
+                                               "next_norm_weight", "stats_out", "raw_out", "xq_out", "s_out", "s_in")]
 
 
-PROLOGUE_NORM, PROLOGUE_ATTENTION, PROLOGUE_STATS = 0, 1, 2
+PROLOGUE_NORM, PROLOGUE_ATTENTION, PROLOGUE_STATS, PROLOGUE_QUANTISED = 0, 1, 2, 3
 EPILOGUE_STORE, EPILOGUE_RESIDUAL, EPILOGUE_GATE = 0, 1, 2
 
 
@@ -280,6 +280,21 @@ def row_stats(h, norm_weight):
     return out
 
 
+def quant_from_stats(h, stats, norm_weight, eps):
+    """Norm + quant_input of h bf16 [M, K] from the partials its producer left (ternaspmm_quant_from_stats):
+    (xq int8 [M, K], s bf16 [M])."""
+    m, k = h.shape
+    _check_rows("quant_from_stats", h, norm_weight=(norm_weight, k))
+    if stats.dtype != torch.float32 or stats.dim() != 3 or stats.shape[0] != m or stats.shape[2] != 2 or not stats.is_contiguous():
+        raise ValueError("quant_from_stats: stats must be a contiguous fp32 [M, count, 2] tensor")
+    xq = torch.empty((m, k), dtype=torch.int8, device=h.device)
+    s = torch.empty(m, dtype=torch.bfloat16, device=h.device)
+    if _lib.load().ternaspmm_quant_from_stats(_p(h.contiguous()), _p(stats), stats.shape[1], _p(norm_weight), float(eps), _p(xq), _p(s),
+                                             m, k, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) != 0:
+        raise ValueError(f"quant_from_stats: unsupported shape M={m} K={k}")
+    return xq, s
+
+
 def interleave_gate_up(packed, out_features, in_features):
     """Load time: the band order TERNASPMM_EPILOGUE_GATE reads (ternaspmm_interleave_gate_up) of a P2 gate+up matrix."""
     out = torch.empty_like(packed)
@@ -289,17 +304,24 @@ def interleave_gate_up(packed, out_features, in_features):
     return out
 
 
-def fused_linear(x, norm_weight, eps, packed, ws, ws_num, out_features, in_features, *, stats=None, attention=None,
+def fused_linear(x, norm_weight, eps, packed, ws, ws_num, out_features, in_features, *, stats=None, attention=None, quantised=None,
                  epilogue=EPILOGUE_STORE, residual=None, next_norm_weight=None, want_raw=False, publish=False):
     """One launch of ternaspmm_fused_linear (include/ternaspmm.h): prologue -> ternary matmul on a P2 weight -> epilogue.
     x: h bf16 [M, K], with `stats` (fp32 [M, count, 2]) when its producer left the norm statistics; or, with
-    `attention` = (splits, head_dim), the fp32 partial results of a split attention launch (one sequence).
+    `attention` = (splits, head_dim), the fp32 partial results of a split attention launch (one sequence); or, with
+    `quantised` = s (bf16 [M]), int8 activations that are quantised already (norm_weight is then not used).
     Returns (out, stats_out, raw, xq, s) -- stats_out for the producing epilogues, raw with `want_raw`, (xq, s) with
     `publish`, None otherwise -- or None when the library does not support the combination (nothing was enqueued)."""
     lib = _lib.load()
     k, n = in_features, out_features
     if attention is not None:
         m, pro = 1, PROLOGUE_ATTENTION
+    elif quantised is not None:
+        m, pro = x.shape[0], PROLOGUE_QUANTISED
+        _check_rows("fused_linear", x, k, s=(quantised, m))
+        if x.dtype != torch.int8 or quantised.dtype != torch.bfloat16:
+            raise ValueError("fused_linear: quantised activations are int8 with bf16 scales")
+        x = x.contiguous()
     else:
         m = x.shape[0]
         _check_rows("fused_linear", x, k, norm_weight=(norm_weight, k))
@@ -311,7 +333,11 @@ def fused_linear(x, norm_weight, eps, packed, ws, ws_num, out_features, in_featu
     out_cols = n // 2 if epilogue == EPILOGUE_GATE else n
     d = FusedLinearDesc()
     d.prologue, d.epilogue, d.M, d.N, d.K, d.ws_num, d.eps = pro, epilogue, m, n, k, ws_num, float(eps)
-    d.x, d.norm_weight, d.packed, d.ws = x.data_ptr(), norm_weight.data_ptr(), packed.data_ptr(), ws.data_ptr()
+    d.x, d.packed, d.ws = x.data_ptr(), packed.data_ptr(), ws.data_ptr()
+    d.norm_weight = norm_weight.data_ptr() if norm_weight is not None else None
+    if quantised is not None:
+        quantised = quantised.contiguous()
+        d.s_in = quantised.data_ptr()
     if stats is not None:
         if stats.dtype != torch.float32 or stats.dim() != 3 or stats.shape[0] != m or stats.shape[2] != 2 or not stats.is_contiguous():
             raise ValueError("fused_linear: stats must be a contiguous fp32 [M, count, 2] tensor")

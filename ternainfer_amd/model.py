@@ -23,7 +23,7 @@ from torch.nn import functional as F
 
 from . import _lib
 from .linear import (EPILOGUE_GATE, EPILOGUE_RESIDUAL, argmax_rows, attention_merge_rmsnorm_linear_packed, fused_linear, get_global_workspace, greedy_step,
-                     greedy_step_state, interleave_gate_up, lm_head, quant_input, row_stats, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant,
+                     greedy_step_state, interleave_gate_up, lm_head, quant_from_stats, quant_input, row_stats, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant,
                      repack_weight, rmsnorm_linear_packed, rmsnorm_quant)
 
 
@@ -268,8 +268,16 @@ class Block:
                          stats=h_stats, epilogue=EPILOGUE_GATE, next_norm_weight=self.ffn_sub_norm, publish=pub)
         note("w13", r)
         inner, inner_stats = r[0], r[1]
-        r = fused_linear(inner, self.ffn_sub_norm, a.norm_eps, self.w2.packed, self.w2.ws, self.w2.ws_num, self.w2.n, self.w2.k,
-                         stats=inner_stats, epilogue=EPILOGUE_RESIDUAL, residual=h, next_norm_weight=next_norm, want_raw=pub, publish=pub)
+        if bsz > 4:
+            # K = 6912: from five rows on every workgroup repeating the norm + quantisation of the whole block costs more than
+            # one launch that does it once (measured at 8 rows: 10.7 us in one launch, 2.7 + 5.3 us in two)
+            xq, s = quant_from_stats(inner, inner_stats, self.ffn_sub_norm, a.norm_eps)
+            r = fused_linear(xq, None, a.norm_eps, self.w2.packed, self.w2.ws, self.w2.ws_num, self.w2.n, self.w2.k, quantised=s,
+                             epilogue=EPILOGUE_RESIDUAL, residual=h, next_norm_weight=next_norm, want_raw=pub)
+            r = (r[0], r[1], r[2], xq, s)
+        else:
+            r = fused_linear(inner, self.ffn_sub_norm, a.norm_eps, self.w2.packed, self.w2.ws, self.w2.ws_num, self.w2.n, self.w2.k,
+                             stats=inner_stats, epilogue=EPILOGUE_RESIDUAL, residual=h, next_norm_weight=next_norm, want_raw=pub, publish=pub)
         note("w2", r)
         return r[0], r[1]
 

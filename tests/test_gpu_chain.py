@@ -196,6 +196,41 @@ def test_norm_and_attention_prologues_with_the_residual_epilogue():
     _check_stats(st.cpu().numpy(), h_next, nxt, 16)
 
 
+@pytest.mark.parametrize("m", [1, 5, 8, 16])
+@pytest.mark.parametrize("n,k", [(2560, 6912), (2560, 2560), (8256, 192)])
+def test_quantise_launch_and_quantised_prologue(m, n, k):
+    """The norm + quantisation as a launch of its own from the producer's partials, and the small-M linear on its output
+    with the producing epilogue: (xq, s) must be the bits the statistics-fed prologue forms inside its launch (up to 8
+    rows, where both exist), the linear exact on them, the stream and its partials as for the other producers."""
+    w = make_ternary(n, k, 0.40, 1260 + m + n)
+    packed = _packed(w)
+    h = make_bf16_activations(m, k, 1261 + m + k, outlier_frac=0.01)
+    g, nxt = _weight(k, 1262 + k), _weight(n, 1263 + n)
+    res = make_bf16_activations(m, n, 1264 + m + n)
+    ws = _bf(WS)
+    stats = L.row_stats(_bf(h), _bf(g))
+    print(f"[case] quantise launch + quantised prologue: m={m} n={n} k={k}", flush=True)
+    xq, s = L.quant_from_stats(_bf(h), stats, _bf(g), 1e-5)
+    torch.cuda.synchronize()
+    q, sb = xq.cpu().numpy(), _bits(s)
+    _check_quantiser(h, g, q, sb)
+    if m <= 8 and n <= 2560:
+        r = L.fused_linear(_bf(h), _bf(g), 1e-5, packed, ws, 1, n, k, stats=stats, publish=True)
+        assert torch.equal(r[3], xq) and torch.equal(r[4], s)
+    r = L.fused_linear(xq, None, 1e-5, packed, ws, 1, n, k, quantised=s, epilogue=L.EPILOGUE_RESIDUAL, residual=_bf(res),
+                       next_norm_weight=_bf(nxt), want_raw=True)
+    if n // 16 > 448:
+        assert r is None                                   # more partials per row than a consumer adds up
+        return
+    out, st, raw, _, _ = r
+    torch.cuda.synchronize()
+    want = O.spmm_i8(q, w, sb, WS, 1, 0)
+    assert (_bits(raw) == want).all()
+    h_next = O.residual_add(res, want)
+    assert (_bits(out) == h_next).all()
+    _check_stats(st.cpu().numpy(), h_next, nxt, 16)
+
+
 def test_unsupported_combinations_are_declined():
     n, k = 256, 192
     packed = _packed(make_ternary(n, k, 0.4, 1250))
