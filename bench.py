@@ -48,9 +48,10 @@ METRIC = "TernaSpMM GB/s + %HBM roofline (M=8,K=N=2560); 2B-shape decode tok/s"
 # HBM bytes per launch of the small-M P2 kernel on the default workload (M=8, average over the four matrices):
 # a counter measurement, not part of this run -- two rocprofv3 --pmc runs of this file (FETCH_SIZE, WRITE_SIZE),
 # scaled by what the same counters read for a 256 MiB copy.  Quoted with its source; null for any other workload.
-TRAFFIC = {"bytes_per_launch": (19206.6 + 356.0) * 1024 / 4,
+TRAFFIC = {"bytes_per_launch": (19175.4 + 356.0) * 1024 / 4,
            "source": "profiles/decode_packed_kernel_hbm_traffic.md (two rocprofv3 --pmc runs, FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 by the copy probe)",
-           "measured_at": "the tree of commit 772a0ab; csrc/decode_packed_kernel.h and launch_decode_packed.hip are unchanged since"}
+           "measured_at": "the tree of the commit 'Chain at 5-8 rows: norm + quantisation of the down projection's input as one launch ...' "
+                          "(the last change to csrc/decode_packed_kernel.h and launch_decode_packed.hip)"}
 
 
 def vp(t):
