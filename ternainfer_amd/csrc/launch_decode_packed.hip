@@ -3,6 +3,7 @@
 #include "launchers.h"
 #include "host_util.h"
 #include "decode_packed_kernel.h"
+#include "decode_flat_kernel.h"
 
 namespace terna {
 
@@ -24,11 +25,44 @@ void launch_decode_packed_as(const Act* x, const uint32_t* packed, uint16_t* out
         terna_decode_packed_kernel<Act, WAVES, MB, DEPTH, NB, false><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, M, N, K, ep, RepackGuard{}, PackedProducer{});
 }
 
+template <typename Act, int WAVES, int TMAX, int NB>
+void launch_decode_flat_as(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                           const RepackGuard* guard, hipStream_t st)
+{
+    const dim3 grid(N / 16 / NB + (guard != nullptr ? 1 : 0));
+    if (guard != nullptr)
+        terna_decode_flat_kernel<Act, WAVES, TMAX, NB, true><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, M, N, K, ep, *guard);
+    else
+        terna_decode_flat_kernel<Act, WAVES, TMAX, NB, false><<<grid, dim3(WAVES * 64), 0, st>>>(x, packed, out, M, N, K, ep, RepackGuard{});
+}
+
+// Up to 16 rows and a K whose tiles one workgroup holds in flight: the straight-line kernel (decode_flat_kernel.h).
+// Returns false where it does not apply.  TERNASPMM_DECODE_FLAT=0 switches it off (tuning aid).
+template <typename Act>
+static bool try_decode_flat(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                            hipStream_t st, const RepackGuard* guard)
+{
+    static const bool off = [] {
+        const char* v = tuning_env("TERNASPMM_DECODE_FLAT");
+        return v && std::atoi(v) == 0;
+    }();
+    const int ktiles = K / 64, bands = N / 16;
+    if (off || M > 16 || static_cast<long long>(N) * K / 4 >= (1ll << 31)) return false;      // byte offsets are 32-bit
+    if (bands > 512 && bands % 2 == 0 && ktiles <= 8 * 5) launch_decode_flat_as<Act, 8, 5, 2>(x, packed, out, ep, M, N, K, guard, st);
+    else if (bands > 256 && ktiles <= 8 * 5) launch_decode_flat_as<Act, 8, 5, 1>(x, packed, out, ep, M, N, K, guard, st);
+    else if (bands > 256) return false;
+    else if (ktiles <= 16 * 3) launch_decode_flat_as<Act, 16, 3, 1>(x, packed, out, ep, M, N, K, guard, st);
+    else if (ktiles <= 16 * 7) launch_decode_flat_as<Act, 16, 7, 1>(x, packed, out, ep, M, N, K, guard, st);
+    else return false;
+    return true;
+}
+
 template <typename Act>
 void launch_decode_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
                           hipStream_t st, const RepackGuard* guard)
 {
     const int forced = decode_waves_override();
+    if (!forced && try_decode_flat(x, packed, out, ep, M, N, K, st, guard)) return;
     const bool wide = forced ? forced == 16 : (N / 16 <= 256);
     if (M <= 16) {
         // more than 512 bands (gate+up): per-wave set-up is as expensive as a few band-tiles, so fewer waves
