@@ -4,6 +4,7 @@
 #include "host_util.h"
 #include "decode_packed_kernel.h"
 #include "decode_flat_kernel.h"
+#include "decode_chunk_kernel.h"
 
 namespace terna {
 
@@ -57,11 +58,68 @@ static bool try_decode_flat(const Act* x, const uint32_t* packed, uint16_t* out,
     return true;
 }
 
+template <typename Act, int CT, int MR>
+void launch_decode_chunk_as(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                            const RepackGuard* guard, hipStream_t st)
+{
+    const dim3 grid(N / 16 + (guard != nullptr ? 1 : 0));
+    if (guard != nullptr)
+        terna_decode_chunk_kernel<Act, CT, MR, true><<<grid, dim3(kChunkWaves * 64), 0, st>>>(x, packed, out, M, N, K, ep, *guard);
+    else
+        terna_decode_chunk_kernel<Act, CT, MR, false><<<grid, dim3(kChunkWaves * 64), 0, st>>>(x, packed, out, M, N, K, ep, RepackGuard{});
+}
+
+template <typename Act, int MR>
+void launch_decode_chunk4_as(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                             const RepackGuard* guard, hipStream_t st)
+{
+    const dim3 grid(N / 64 + (guard != nullptr ? 1 : 0));
+    if (guard != nullptr)
+        terna_decode_chunk4_kernel<Act, MR, true><<<grid, dim3(kChunkWaves * 64), 0, st>>>(x, packed, out, M, N, K, ep, *guard);
+    else
+        terna_decode_chunk4_kernel<Act, MR, false><<<grid, dim3(kChunkWaves * 64), 0, st>>>(x, packed, out, M, N, K, ep, RepackGuard{});
+}
+
+// Up to 16 rows, up to 32 chunks of four tiles (K <= 8192): the kernel with four band-tiles per load (decode_chunk_kernel.h).
+// Returns false where it does not apply.  TERNASPMM_DECODE_CHUNK=0 switches it off, =2 gives every band a workgroup of
+// its own whatever the band count, =3 leaves matrices of more than 256 bands to the other kernels (tuning aids).
+template <typename Act>
+static bool try_decode_chunk(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                             hipStream_t st, const RepackGuard* guard)
+{
+    static const int mode = [] {
+        const char* v = tuning_env("TERNASPMM_DECODE_CHUNK");
+        return v ? std::atoi(v) : 1;
+    }();
+    const int ktiles = K / 64, bands = N / 16, chunks = (ktiles + 3) / 4;
+    if (mode == 0 || M > 16 || chunks > 2 * kChunkWaves) return false;
+    if (static_cast<long long>(N) * K / 4 >= (1ll << 31)) return false;      // byte offsets are 32-bit
+    if (bands > 256 && mode != 2) {
+        // four bands per workgroup: one round of workgroups up to 1024 bands (the bf16 slabs of 16 rows do not fit LDS)
+        if (mode == 3 || bands % 4 != 0 || chunks > kChunkWaves || (sizeof(Act) == 2 && M > 8)) return false;
+        if (M <= 4) launch_decode_chunk4_as<Act, 4>(x, packed, out, ep, M, N, K, guard, st);
+        else if (M <= 8) launch_decode_chunk4_as<Act, 8>(x, packed, out, ep, M, N, K, guard, st);
+        else if constexpr (sizeof(Act) == 1) launch_decode_chunk4_as<Act, 16>(x, packed, out, ep, M, N, K, guard, st);
+        return true;
+    }
+#define TERNA_CHUNK(CT)                                                                                   \
+    do {                                                                                                  \
+        if (M <= 4) launch_decode_chunk_as<Act, CT, 4>(x, packed, out, ep, M, N, K, guard, st);            \
+        else if (M <= 8) launch_decode_chunk_as<Act, CT, 8>(x, packed, out, ep, M, N, K, guard, st);       \
+        else launch_decode_chunk_as<Act, CT, 16>(x, packed, out, ep, M, N, K, guard, st);                  \
+    } while (0)
+    if (chunks <= kChunkWaves) TERNA_CHUNK(1);
+    else TERNA_CHUNK(2);
+#undef TERNA_CHUNK
+    return true;
+}
+
 template <typename Act>
 void launch_decode_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
                           hipStream_t st, const RepackGuard* guard)
 {
     const int forced = decode_waves_override();
+    if (!forced && try_decode_chunk(x, packed, out, ep, M, N, K, st, guard)) return;
     if (!forced && try_decode_flat(x, packed, out, ep, M, N, K, st, guard)) return;
     const bool wide = forced ? forced == 16 : (N / 16 <= 256);
     if (M <= 16) {
