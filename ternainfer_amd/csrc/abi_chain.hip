@@ -9,6 +9,7 @@
 #include "../../include/ternaspmm.h"
 #include "host_util.h"
 #include "decode_fused_kernel.h"
+#include "chain_chunk_kernel.h"
 #include "launchers.h"
 
 using namespace terna;
@@ -159,6 +160,43 @@ void launch_attn(const ChainArgs& a, int splits, int head_dim)
 #undef TERNA_CHAIN_ATTN
 }
 
+// The statistics-given prologue in the wide-load form (chain_chunk_kernel.h): M waves add up the partials, the other
+// 16 - M share `units` units of work, up to three each.  Returns false where that does not cover the matrix.
+template <int NBANDS, int EPI>
+bool launch_chunk_by_rows(const ChainArgs& a, int units)
+{
+    const ChainIo io{a.out, a.ws, a.xq_out, a.s_out, a.ex.epi_residual, a.ex.epi_next_w, a.ex.stats_out, a.ex.raw_out};
+    const int workers = kChunkWaves - a.M;
+    const int ct = (units + workers - 1) / workers;
+    if (ct > 3) return false;
+#define TERNA_CHAIN_CHUNK(CT, MR)                                                                                       \
+    terna_chain_chunk_kernel<NBANDS, CT, MR, EPI><<<a.grid, dim3(kChunkWaves * 64), 0, a.st>>>(                            \
+        a.x, a.norm_w, a.packed, a.ex.stats_in, a.M, a.N, a.K, a.ex.stats_count, a.eps, a.ws_num, a.qmode, io)
+#define TERNA_CHAIN_CHUNK_CT(MR)                                                                                        \
+    do {                                                                                                                \
+        if (ct == 1) TERNA_CHAIN_CHUNK(1, MR);                                                                          \
+        else if (ct == 2) TERNA_CHAIN_CHUNK(2, MR);                                                                     \
+        else TERNA_CHAIN_CHUNK(3, MR);                                                                                  \
+    } while (0)
+    if (a.M == 1) TERNA_CHAIN_CHUNK_CT(1);
+    else if (a.M == 2) TERNA_CHAIN_CHUNK_CT(2);
+    else if (a.M <= 4) TERNA_CHAIN_CHUNK_CT(4);
+    else TERNA_CHAIN_CHUNK_CT(8);
+#undef TERNA_CHAIN_CHUNK_CT
+#undef TERNA_CHAIN_CHUNK
+    return true;
+}
+
+// TERNASPMM_CHAIN_CHUNK=0 keeps the per-tile kernels (tuning aid).
+bool chain_chunk_enabled()
+{
+    static const bool on = [] {
+        const char* v = tuning_env("TERNASPMM_CHAIN_CHUNK");
+        return !(v && std::atoi(v) == 0);
+    }();
+    return on;
+}
+
 }  // namespace
 
 extern "C" {
@@ -264,11 +302,16 @@ int ternaspmm_fused_linear(const ternaspmm_fused_linear_desc* d, terna_stream st
         // gate+up, bands interleaved: four bands (two gate / up pairs) per workgroup
         if (pro != TERNASPMM_PROLOGUE_STATS || ktiles > 8 * 5) return -1;
         a.grid = dim3(bands / 4);
-        launch_by_rows<8, 5, FUSED_STATS, 4, FEPI_GLU>(a);
+        const bool wide = chain_chunk_enabled() && static_cast<long long>(N) * K / 4 < (1ll << 31);
+        if (!(wide && launch_chunk_by_rows<4, CEPI_GATE>(a, 2 * ((ktiles + 3) / 4)))) launch_by_rows<8, 5, FUSED_STATS, 4, FEPI_GLU>(a);
     } else if (pro == TERNASPMM_PROLOGUE_STATS) {
         const bool res = epi == TERNASPMM_EPILOGUE_RESIDUAL;
         a.grid = dim3(bands);
-        if (ktiles <= 8 * 5) {
+        const int chunks = (ktiles + 3) / 4;
+        const bool wide = chain_chunk_enabled() && static_cast<long long>(N) * K / 4 < (1ll << 31);
+        if (wide && (res ? launch_chunk_by_rows<1, CEPI_RESIDUAL>(a, chunks) : launch_chunk_by_rows<1, CEPI_STORE>(a, chunks))) {
+            // launched
+        } else if (ktiles <= 8 * 5) {
             if (res) launch_by_rows<8, 5, FUSED_STATS, 1, FEPI_RESIDUAL>(a);
             else launch_by_rows<8, 5, FUSED_STATS, 1, FEPI_PLAIN>(a);
         } else if (ktiles <= 16 * 7) {

@@ -71,17 +71,22 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_decode_chunk_kernel(
     uint32_t es = 0u, ew = 0u;
 
     Acc acc = Acc{0, 0, 0, 0};
-    if (wave * 4 < ktiles) {
-        // ---- (1) the weights, at once.  Tiles past K (the tail of a partial last chunk, a chunk slot this wave does not
-        // have) come back as zeros
+    // ---- (1) the weights, at once.  Tiles past K (the tail of a partial last chunk, a chunk slot this wave does not
+    // have) come back as zeros; a wave without any chunk issues nothing
+    const bool has_work = wave * 4 < ktiles;
+    u32x4 wq[CT];
+    if (has_work) {
         const __amdgpu_buffer_rsrc_t rw = make_raw_buffer(packed, static_cast<uint32_t>(N >> 4) * static_cast<uint32_t>(ktiles) * 256u);
-        u32x4 wq[CT];
 #pragma unroll
         for (int t = 0; t < CT; ++t) {
             const int tile0 = (wave + WAVES * t) * 4;
             wq[t] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, tile0 + g < ktiles ? lane * 16 : kBufferOutOfRange,
                                                                                    (band * ktiles + tile0) * 256, 0));
         }
+    }
+    // (A workgroup barrier here, so that every wave's weight requests precede anybody's activation requests, was measured:
+    // slower -- the activations then arrive last and everything waits for them.)
+    if (has_work) {
         // ---- (2) the activations of the wave's chunks
         const int rowbytes = K * SZ;
         const __amdgpu_buffer_rsrc_t rx = make_raw_buffer(x, static_cast<uint32_t>(M) * rowbytes);

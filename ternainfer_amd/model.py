@@ -524,8 +524,10 @@ class Transformer:
         # 1500: 1943 -> 1713 us per step; at slot 255 of 384 the pair of launches is 1.5 us slower than the unsplit one)
         if one_launch_attention and self.layers[0].act == "int8" and (bsz == 1 or max_seq > 1024):
             attn_ws = self.attention_partial(bsz, max_seq) or attn_ws
-        # one new token for up to 8 sequences: the linears chained through producer-side norm statistics (forward_chain)
-        chain = one_launch_attention and self.layers[0].act == "int8" and bsz <= 8 and getattr(self, "chain", True) and self.chain_supported()
+        # one new token for up to 4 sequences: the linears chained through producer-side norm statistics (forward_chain).
+        # Every workgroup of a chained linear normalises and quantises the whole activation matrix again; from five rows
+        # on a norm + quantisation launch of its own and the plain small-M kernel are faster (measured at 6 and 8 rows).
+        chain = one_launch_attention and self.layers[0].act == "int8" and bsz <= 4 and getattr(self, "chain", True) and self.chain_supported()
         stats = None
         for index, (layer, (ck, cv)) in enumerate(zip(self.layers, cache)):
             x_in, pending_in = x, pending
