@@ -241,6 +241,11 @@ def measure_model(torch, batch, act="int8", prefetch=True, gen_tokens=256, check
     if model is None:
         model = Transformer(margs, seed=20260500, act=act)
     model.chain = chain
+    if os.environ.get("TERNA_BENCH_CHAIN_ROWS"):           # measurement aids
+        model.chain_rows = int(os.environ["TERNA_BENCH_CHAIN_ROWS"])
+    if os.environ.get("TERNA_BENCH_CHAIN_DOWN_ROWS"):
+        for blk in model.layers:
+            blk.chain_down_rows = int(os.environ["TERNA_BENCH_CHAIN_DOWN_ROWS"])
     model.enable_prefetch(False)
     if prefetch:     # weights of the following launches, pulled through the caches during the attention launch
         model.enable_prefetch(True, ("wo", "w13", "w2", "next_wqkv", "norms") if batch <= 2 else ("wo", "w13", "norms"))

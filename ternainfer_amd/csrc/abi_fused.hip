@@ -22,8 +22,22 @@ void ternaspmm_rmsnorm_quant(const terna_bf16* x, const terna_bf16* residual, te
         std::fprintf(stderr, "ternaspmm_rmsnorm_quant: unsupported arguments (M=%d K=%d)\n", M, K);
         return;
     }
-    terna_norm_quant_kernel<false><<<dim3(M), dim3(kNormThreads), 0, static_cast<hipStream_t>(stream)>>>(
-        x, residual, weight, K, eps, sum_out, y_out, xq_out, s_out, quant_mode());
+    // as many 8-element vectors per thread as the row needs (1, 2 or 4), the residual's loads only where there is one
+    const int nv = (K / 8 + kNormThreads - 1) / kNormThreads;
+    const dim3 grid(M), block(kNormThreads);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int qm = quant_mode();
+#define TERNA_NORM(NV, SECOND) terna_norm_quant_kernel<false, NV, SECOND><<<grid, block, 0, st>>>(x, residual, weight, K, eps, sum_out, y_out, xq_out, s_out, qm)
+    if (residual != nullptr) {
+        if (nv <= 1) TERNA_NORM(1, true);
+        else if (nv <= 2) TERNA_NORM(2, true);
+        else TERNA_NORM(4, true);
+    } else {
+        if (nv <= 1) TERNA_NORM(1, false);
+        else if (nv <= 2) TERNA_NORM(2, false);
+        else TERNA_NORM(4, false);
+    }
+#undef TERNA_NORM
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_rmsnorm_quant", e, __LINE__);
 }
@@ -35,8 +49,15 @@ void ternaspmm_relu2_mul_rmsnorm_quant(const terna_bf16* x13, const terna_bf16* 
         std::fprintf(stderr, "ternaspmm_relu2_mul_rmsnorm_quant: unsupported arguments (M=%d F=%d)\n", M, F);
         return;
     }
-    terna_norm_quant_kernel<true><<<dim3(M), dim3(kNormThreads), 0, static_cast<hipStream_t>(stream)>>>(
-        x13, nullptr, weight, F, eps, nullptr, y_out, xq_out, s_out, quant_mode());
+    const int nv = (F / 8 + kNormThreads - 1) / kNormThreads;
+    const dim3 grid(M), block(kNormThreads);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int qm = quant_mode();
+#define TERNA_NORM(NV) terna_norm_quant_kernel<true, NV, true><<<grid, block, 0, st>>>(x13, nullptr, weight, F, eps, nullptr, y_out, xq_out, s_out, qm)
+    if (nv <= 1) TERNA_NORM(1);
+    else if (nv <= 2) TERNA_NORM(2);
+    else TERNA_NORM(4);
+#undef TERNA_NORM
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_relu2_mul_rmsnorm_quant", e, __LINE__);
 }

@@ -97,12 +97,14 @@ __device__ __forceinline__ float round_bf16(float v) { return bf16_bits_to_float
 
 // GLU = false: x [M][K], optional residual [M][K] and sum_out [M][K].
 // GLU = true : x [M][2K] holding x1 | x3; residual / sum_out unused.
-template <bool GLU>
+// NV = 8-element vectors per thread (K <= 2048 NV); SECOND = there is a second operand (the residual, or x3).
+template <bool GLU, int NV = kNormMaxVecs, bool SECOND = true>
 __global__ __launch_bounds__(kNormThreads) void terna_norm_quant_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, const uint16_t* __restrict__ weight, int K,
     float eps, uint16_t* __restrict__ sum_out, uint16_t* __restrict__ y_out, int8_t* __restrict__ xq_out,
     uint16_t* __restrict__ s_out, int quant_mode)
 {
+    static_assert(!GLU || SECOND, "the gate has two operands");
     __shared__ float red[2][kNormThreads / 64];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -111,31 +113,32 @@ __global__ __launch_bounds__(kNormThreads) void terna_norm_quant_kernel(
     const uint16_t* xr = x + row * static_cast<size_t>(GLU ? 2 * K : K);
 
     // Every global load of the row -- input, second operand, norm weight -- is issued before the
-    // first use: with one row per workgroup the kernel's time is its chain of memory round trips.
+    // first use: with one row per workgroup the kernel's time is its chain of memory round trips, and the address
+    // unit takes a wave's load in a dozen cycles whatever it fetches: no more loads than the row needs.
     // The loads are unconditional on clamped addresses (a load inside a branch is waited for at
-    // the join, which would serialise them); without a second operand the input is read twice.
-    u32x4 raw_x[kNormMaxVecs], raw_b[kNormMaxVecs], raw_w[kNormMaxVecs];
-    const uint16_t* br = GLU ? xr + K : (residual != nullptr ? residual + row * K : xr);
+    // the join, which would serialise them).
+    u32x4 raw_x[NV], raw_b[NV], raw_w[NV];
+    const uint16_t* br = GLU ? xr + K : (SECOND ? residual + row * K : xr);
 #pragma unroll
-    for (int i = 0; i < kNormMaxVecs; ++i) {
+    for (int i = 0; i < NV; ++i) {
         const int v = tid + i * kNormThreads;
         const int vc = v < nvec ? v : nvec - 1;
         raw_x[i] = *reinterpret_cast<const u32x4*>(xr + 8 * vc);
-        raw_b[i] = *reinterpret_cast<const u32x4*>(br + 8 * vc);
+        if constexpr (SECOND) raw_b[i] = *reinterpret_cast<const u32x4*>(br + 8 * vc);
         raw_w[i] = *reinterpret_cast<const u32x4*>(weight + 8 * vc);
     }
     // pin the loads here: otherwise they are sunk into the branches below, next to their uses
 #pragma unroll
-    for (int i = 0; i < kNormMaxVecs; ++i) {
+    for (int i = 0; i < NV; ++i) {
         pin_registers(raw_x[i]);
-        pin_registers(raw_b[i]);
+        if constexpr (SECOND) pin_registers(raw_b[i]);
         pin_registers(raw_w[i]);
     }
 
-    float h[kNormMaxVecs][8];
+    float h[NV][8];
     float ssq = 0.0f;
 #pragma unroll
-    for (int i = 0; i < kNormMaxVecs; ++i) {
+    for (int i = 0; i < NV; ++i) {
         const int v = tid + i * kNormThreads;
         if (v < nvec) {
             unpack_bf16x8(raw_x[i], h[i]);
@@ -147,7 +150,7 @@ __global__ __launch_bounds__(kNormThreads) void terna_norm_quant_kernel(
                     const float r = fmaxf(h[i][j], 0.0f);
                     h[i][j] = round_bf16(round_bf16(r * r) * g[j]);
                 }
-            } else if (residual != nullptr) {
+            } else if constexpr (SECOND) {
                 float r[8];
                 unpack_bf16x8(raw_b[i], r);
 #pragma unroll
@@ -166,7 +169,7 @@ __global__ __launch_bounds__(kNormThreads) void terna_norm_quant_kernel(
 
     float amax = 0.0f;
 #pragma unroll
-    for (int i = 0; i < kNormMaxVecs; ++i) {
+    for (int i = 0; i < NV; ++i) {
         const int v = tid + i * kNormThreads;
         if (v < nvec) {
             float w[8];
@@ -189,7 +192,7 @@ __global__ __launch_bounds__(kNormThreads) void terna_norm_quant_kernel(
     const float s = quant_scale(amax, quant_mode, &s_bits);
     if (tid == 0) s_out[row] = s_bits;
 #pragma unroll
-    for (int i = 0; i < kNormMaxVecs; ++i) {
+    for (int i = 0; i < NV; ++i) {
         const int v = tid + i * kNormThreads;
         if (v < nvec) {
             uint32_t q[2] = {0u, 0u};

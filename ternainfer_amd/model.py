@@ -123,6 +123,8 @@ KERNEL_ATTENTION = object()    # in place of a mask: several new tokens, attenti
 
 
 class Block:
+    chain_down_rows = 4            # forward_chain: up to this many rows the down projection normalises + quantises in its own launch
+
     def __init__(self, args: ModelArgs, gen: Optional[torch.Generator], act: str, p_zero: float = 0.40):
         self.args = args
         self.act = act
@@ -268,7 +270,7 @@ class Block:
                          stats=h_stats, epilogue=EPILOGUE_GATE, next_norm_weight=self.ffn_sub_norm, publish=pub)
         note("w13", r)
         inner, inner_stats = r[0], r[1]
-        if bsz > 4:
+        if bsz > self.chain_down_rows:
             # K = 6912: from five rows on every workgroup repeating the norm + quantisation of the whole block costs more than
             # one launch that does it once (measured at 8 rows: 10.7 us in one launch, 2.7 + 5.3 us in two)
             xq, s = quant_from_stats(inner, inner_stats, self.ffn_sub_norm, a.norm_eps)
@@ -370,6 +372,12 @@ class Block:
 
 class Transformer:
     """Random-init decoder; `act` selects int8-quantised (reference semantics) or bf16 activations."""
+
+    # Up to this many sequences a one-token step chains its linears (Block.forward_chain).  Every workgroup of a chained
+    # linear normalises and quantises the whole activation matrix again, and one of its waves per row only adds up
+    # partials; from five rows on a norm + quantisation launch of its own and the plain small-M kernel are faster
+    # (measured at 6 and 8 rows).
+    chain_rows = 4
 
     def __init__(self, args: ModelArgs, seed: int = 0, act: str = "int8", p_zero: float = 0.40):
         gen = torch.Generator(device="cuda").manual_seed(seed)
@@ -524,10 +532,8 @@ class Transformer:
         # 1500: 1943 -> 1713 us per step; at slot 255 of 384 the pair of launches is 1.5 us slower than the unsplit one)
         if one_launch_attention and self.layers[0].act == "int8" and (bsz == 1 or max_seq > 1024):
             attn_ws = self.attention_partial(bsz, max_seq) or attn_ws
-        # one new token for up to 4 sequences: the linears chained through producer-side norm statistics (forward_chain).
-        # Every workgroup of a chained linear normalises and quantises the whole activation matrix again; from five rows
-        # on a norm + quantisation launch of its own and the plain small-M kernel are faster (measured at 6 and 8 rows).
-        chain = one_launch_attention and self.layers[0].act == "int8" and bsz <= 4 and getattr(self, "chain", True) and self.chain_supported()
+        # one new token for a few sequences: the linears chained through producer-side norm statistics (forward_chain)
+        chain = one_launch_attention and self.layers[0].act == "int8" and bsz <= self.chain_rows and getattr(self, "chain", True) and self.chain_supported()
         stats = None
         for index, (layer, (ck, cv)) in enumerate(zip(self.layers, cache)):
             x_in, pending_in = x, pending
