@@ -187,6 +187,53 @@ bool launch_chunk_by_rows(const ChainArgs& a, int units)
     return true;
 }
 
+// The statistics-inside prologues in the wide-load form (terna_chain_norm_kernel): plain rows ...
+template <int EPI>
+bool launch_norm_chunk_by_rows(const ChainArgs& a, int chunks)
+{
+    const ChainIo io{a.out, a.ws, a.xq_out, a.s_out, a.ex.epi_residual, a.ex.epi_next_w, a.ex.stats_out, a.ex.raw_out};
+    if (chunks > 2 * kChunkWaves) return false;
+#define TERNA_CHAIN_NORM(CT, MR)                                                                                        \
+    terna_chain_norm_kernel<CPRO_NORM, CT, MR, EPI><<<a.grid, dim3(kChunkWaves * 64), 0, a.st>>>(                         \
+        a.x, a.norm_w, a.packed, a.M, a.N, a.K, a.eps, a.ws_num, a.qmode, io)
+#define TERNA_CHAIN_NORM_CT(MR)                                                                                         \
+    do {                                                                                                                \
+        if (chunks <= kChunkWaves) TERNA_CHAIN_NORM(1, MR);                                                             \
+        else TERNA_CHAIN_NORM(2, MR);                                                                                   \
+    } while (0)
+    if (a.M == 1) TERNA_CHAIN_NORM_CT(1);
+    else if (a.M == 2) TERNA_CHAIN_NORM_CT(2);
+    else if (a.M <= 4) TERNA_CHAIN_NORM_CT(4);
+    else TERNA_CHAIN_NORM_CT(8);
+#undef TERNA_CHAIN_NORM_CT
+#undef TERNA_CHAIN_NORM
+    return true;
+}
+
+// ... and the single row merged from a deferred attention's partial results (K <= 4096)
+template <int EPI>
+bool launch_attn_chunk(const ChainArgs& a, int splits, int head_dim, int chunks)
+{
+    const ChainIo io{a.out, a.ws, a.xq_out, a.s_out, a.ex.epi_residual, a.ex.epi_next_w, a.ex.stats_out, a.ex.raw_out};
+    if (chunks > kChunkWaves || a.M != 1) return false;
+#define TERNA_CHAIN_ATTN(SP, HD)                                                                                        \
+    terna_chain_norm_kernel<CPRO_ATTN, 1, 1, EPI, SP, HD><<<a.grid, dim3(kChunkWaves * 64), 0, a.st>>>(                   \
+        a.x, a.norm_w, a.packed, a.M, a.N, a.K, a.eps, a.ws_num, a.qmode, io)
+    if (head_dim == 128) {
+        if (splits == 1) TERNA_CHAIN_ATTN(1, 128);
+        else if (splits == 2) TERNA_CHAIN_ATTN(2, 128);
+        else if (splits == 4) TERNA_CHAIN_ATTN(4, 128);
+        else TERNA_CHAIN_ATTN(8, 128);
+    } else {
+        if (splits == 1) TERNA_CHAIN_ATTN(1, 64);
+        else if (splits == 2) TERNA_CHAIN_ATTN(2, 64);
+        else if (splits == 4) TERNA_CHAIN_ATTN(4, 64);
+        else TERNA_CHAIN_ATTN(8, 64);
+    }
+#undef TERNA_CHAIN_ATTN
+    return true;
+}
+
 // TERNASPMM_CHAIN_CHUNK=0 keeps the per-tile kernels (tuning aid).
 bool chain_chunk_enabled()
 {
@@ -296,8 +343,13 @@ int ternaspmm_fused_linear(const ternaspmm_fused_linear_desc* d, terna_stream st
             bands > 65535 || epi == TERNASPMM_EPILOGUE_GATE)
             return -1;
         a.grid = dim3(bands);
-        if (epi == TERNASPMM_EPILOGUE_RESIDUAL) launch_attn<FEPI_RESIDUAL>(a, sp, hd);
-        else launch_attn<FEPI_PLAIN>(a, sp, hd);
+        const bool wide = chain_chunk_enabled() && static_cast<long long>(N) * K / 4 < (1ll << 31);
+        const int chunks = (ktiles + 3) / 4;
+        if (epi == TERNASPMM_EPILOGUE_RESIDUAL) {
+            if (!(wide && launch_attn_chunk<CEPI_RESIDUAL>(a, sp, hd, chunks))) launch_attn<FEPI_RESIDUAL>(a, sp, hd);
+        } else {
+            if (!(wide && launch_attn_chunk<CEPI_STORE>(a, sp, hd, chunks))) launch_attn<FEPI_PLAIN>(a, sp, hd);
+        }
     } else if (epi == TERNASPMM_EPILOGUE_GATE) {
         // gate+up, bands interleaved: four bands (two gate / up pairs) per workgroup
         if (pro != TERNASPMM_PROLOGUE_STATS || ktiles > 8 * 5) return -1;
@@ -324,7 +376,8 @@ int ternaspmm_fused_linear(const ternaspmm_fused_linear_desc* d, terna_stream st
         // the norm's statistics taken inside (two workgroup-wide reductions), producing epilogue
         if (epi != TERNASPMM_EPILOGUE_RESIDUAL || ktiles > 8 * 5) return -1;     // (with a plain store: bitlinear_TernaSpMM_packed_fused)
         a.grid = dim3(bands);
-        launch_by_rows<8, 5, FUSED_PLAIN, 1, FEPI_RESIDUAL>(a);
+        const bool wide = chain_chunk_enabled() && static_cast<long long>(N) * K / 4 < (1ll << 31);
+        if (!(wide && launch_norm_chunk_by_rows<CEPI_RESIDUAL>(a, (ktiles + 3) / 4))) launch_by_rows<8, 5, FUSED_PLAIN, 1, FEPI_RESIDUAL>(a);
     }
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_fused_linear", e, __LINE__);

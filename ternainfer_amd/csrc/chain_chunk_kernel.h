@@ -364,4 +364,279 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_chain_chunk_kernel(
     }
 }
 
+// The same linear with the norm's statistics taken INSIDE (no producer left them): the O projection behind the attention.
+//   CPRO_NORM  x is bf16 [M][K]
+//   CPRO_ATTN  one row: x is the fp32 buffer a deferred-merge attention launch left (attention_kernel.h) -- per head the
+//              score maxima and sums of its ASP splits, then the splits' unnormalised results; a lane merges its four
+//              columns with attention_merge's arithmetic, so the row has the bits the merge kernel would give
+// One band per workgroup, every wave works (unit = chunk, wave w takes chunks w, w + 16, ...).  The prologue is a chain
+// of its own here -- values, partial statistics per wave, barrier, totals, norm, quantisation -- so everything it reads
+// (cache resident) is requested by ALL waves first, then a barrier, then the weights: the vector cache returns data in
+// the order of the requests of the whole CU, and what is requested behind a weight load arrives with the weights.  The
+// chain then runs under the weights' round trip.  Sums of squares: per lane in column order, the lanes of a row pairwise
+// (group_reduce), the waves pairwise -- the same in every workgroup.
+enum ChainPrologue { CPRO_NORM, CPRO_ATTN };
+
+template <int PRO, int CT, int MR, int EPI, int ASP = 1, int AHD = 128>
+__global__ __launch_bounds__(kChunkWaves * 64) void terna_chain_norm_kernel(
+    const void* __restrict__ xin, const uint16_t* __restrict__ norm_w, const uint32_t* __restrict__ packed,
+    int M, int N, int K, float eps, int ws_num, int quant_mode, ChainIo io)
+{
+    static_assert(EPI == CEPI_STORE || EPI == CEPI_RESIDUAL, "one band per workgroup");
+    static_assert(MR == 1 || MR == 2 || MR == 4 || MR == 8, "rows of the slab");
+    static_assert(PRO != CPRO_ATTN || MR == 1, "the attention merge feeds a single row");
+    static_assert(AHD % 4 == 0 && 256 % AHD == 0 && ASP >= 1 && ASP <= kAttentionMaxSplits, "a lane's four columns lie inside one head");
+    constexpr int WAVES = kChunkWaves;
+    constexpr int NE = MR == 1 ? 4 : 8;
+    constexpr int LPR = 256 / NE;
+    constexpr int RPL = 64 / LPR;
+    constexpr int XL = MR / RPL;
+    constexpr int FW = (MR + 3) / 4;
+    constexpr int PASSES = (MR + 3) / 4;         // four rows' totals per pass over the waves' partials
+
+    __shared__ int red[WAVES][256];
+    __shared__ __align__(16) uint8_t slab_all[WAVES][(MR + 1) * kChainSlabPitch];
+    __shared__ float2 part_s[8][WAVES];          // per row and wave: (sum of squares, max |value * norm weight|)
+    __shared__ float stat_w[WAVES][8][2];        // per wave, its own copy: rstd and the multiplier of every row
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int band = blockIdx.x;
+    const int ktiles = K >> 6;
+    const int chunks = (ktiles + 3) >> 2;
+    const int i = lane & 15, g = lane >> 4;
+    const bool writer = blockIdx.x == 0;
+    int uchunk[CT];
+    bool uok[CT];
+#pragma unroll
+    for (int t = 0; t < CT; ++t) {
+        uchunk[t] = wave + WAVES * t;
+        uok[t] = uchunk[t] < chunks;
+    }
+    const bool has_work = uok[0];
+    const bool finisher = wave < FW;
+    const int fin_m = 4 * wave + (lane >> 4);
+    const int fin_n = band * 16 + (lane & 15);
+    uint32_t ew = 0u, eres = 0u, enw = 0u;
+    const int xrow0 = lane / LPR, xcol = (lane % LPR) * NE;
+    uint8_t* slab = slab_all[wave];
+
+    // ---- (1) everything the prologue reads, all waves; barrier; (2) the weights
+    uint32_t xr[CT][XL][NE / 2], nw[CT][NE / 2];
+    constexpr int SQ = PRO == CPRO_ATTN ? (ASP > 4 ? 4 : 2) : 1;                 // statistic quads of a head that matter
+    f32x4 ast[PRO == CPRO_ATTN ? CT : 1][SQ], ao[PRO == CPRO_ATTN ? CT : 1][ASP];
+    if (has_work) {
+        const __amdgpu_buffer_rsrc_t rn = make_raw_buffer(norm_w, static_cast<uint32_t>(K) * 2u);
+#pragma unroll
+        for (int t = 0; t < CT; ++t) {
+            const int col0 = uchunk[t] * 256;
+            const bool col_ok = uok[t] && col0 + xcol < K;
+            if constexpr (PRO == CPRO_ATTN) {
+                const int heads = K / AHD;
+                const __amdgpu_buffer_rsrc_t rp = make_raw_buffer(xin, static_cast<uint32_t>(heads) * (kAttentionStatFloats + ASP * AHD) * 4u);
+                const int c = col0 + xcol;
+                const int head = c / AHD, d = c % AHD;             // AHD is a power of two times ... a constant: shifts
+#pragma unroll
+                for (int q4 = 0; q4 < SQ; ++q4) {
+                    const int quad = SQ == 2 ? 2 * q4 : q4;        // maxima 0-3 (4-7), sums 0-3 (4-7)
+                    ast[t][q4] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rp, col_ok ? (head * kAttentionStatFloats + 4 * quad) * 4 : kBufferOutOfRange, 0, 0));
+                }
+#pragma unroll
+                for (int jj = 0; jj < ASP; ++jj)
+                    ao[t][jj] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                        rp, col_ok ? (heads * kAttentionStatFloats + (head * ASP + jj) * AHD + d) * 4 : kBufferOutOfRange, 0, 0));
+            } else {
+                const __amdgpu_buffer_rsrc_t rx = make_raw_buffer(xin, static_cast<uint32_t>(M) * K * 2u);
+#pragma unroll
+                for (int q = 0; q < XL; ++q) {
+                    const int row = xrow0 + RPL * q;
+                    const int voff = row < M && col_ok ? (row * K + xcol) * 2 : kBufferOutOfRange;
+                    if constexpr (NE == 8) {
+                        const u32x4 v = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rx, voff, col0 * 2, 0));
+                        xr[t][q][0] = v.x; xr[t][q][1] = v.y; xr[t][q][2] = v.z; xr[t][q][3] = v.w;
+                    } else {
+                        const u32x2 v = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rx, voff, col0 * 2, 0));
+                        xr[t][q][0] = v.x; xr[t][q][1] = v.y;
+                    }
+                }
+            }
+            const int woff = col_ok ? xcol * 2 : kBufferOutOfRange;
+            if constexpr (NE == 8) {
+                const u32x4 v = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rn, woff, col0 * 2, 0));
+                nw[t][0] = v.x; nw[t][1] = v.y; nw[t][2] = v.z; nw[t][3] = v.w;
+            } else {
+                const u32x2 v = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rn, woff, col0 * 2, 0));
+                nw[t][0] = v.x; nw[t][1] = v.y;
+            }
+        }
+    }
+    if (finisher) {
+        ew = io.ws[ws_num == 1 ? 0 : ws_group_decode(fin_n, N, ws_num)];
+        if constexpr (EPI == CEPI_RESIDUAL) {
+            eres = io.residual[static_cast<size_t>(fin_m < M ? fin_m : 0) * N + fin_n];
+            enw = io.next_w[fin_n];
+        }
+    }
+    __builtin_amdgcn_s_barrier();                // every cache-resident request of the CU is out
+    u32x4 wq[CT];
+    if (has_work) {
+        const __amdgpu_buffer_rsrc_t rw = make_raw_buffer(packed, static_cast<uint32_t>(N >> 4) * static_cast<uint32_t>(ktiles) * 256u);
+#pragma unroll
+        for (int t = 0; t < CT; ++t) {
+            const int tile0 = uchunk[t] * 4;
+            wq[t] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, uok[t] && tile0 + g < ktiles ? lane * 16 : kBufferOutOfRange,
+                                                                                   (band * ktiles + tile0) * 256, 0));
+        }
+        for (int o = MR * kChainSlabPitch + lane * 16; o < (MR + 1) * kChainSlabPitch; o += 64 * 16) *reinterpret_cast<u32x4*>(slab + o) = u32x4{0u, 0u, 0u, 0u};
+    }
+
+    // ---- (3) the values (CPRO_ATTN: merged and rounded to bf16) and this wave's partial statistics per row
+    float pss[XL], pmx[XL];
+#pragma unroll
+    for (int q = 0; q < XL; ++q) pss[q] = pmx[q] = 0.0f;
+    if (has_work) {
+#pragma unroll
+        for (int t = 0; t < CT; ++t) {
+            if constexpr (PRO == CPRO_ATTN) {
+                float am[kAttentionMaxSplits], al[kAttentionMaxSplits];
+#pragma unroll
+                for (int jj = 0; jj < ASP; ++jj) {
+                    am[jj] = ast[t][jj >> 2][jj & 3];
+                    al[jj] = ast[t][(SQ / 2) + (jj >> 2)][jj & 3];
+                }
+                float m_all = -INFINITY;
+#pragma unroll
+                for (int jj = 0; jj < ASP; ++jj) m_all = fmaxf(m_all, am[jj]);
+                float wj[ASP], den = 0.0f;
+#pragma unroll
+                for (int jj = 0; jj < ASP; ++jj) {
+                    wj[jj] = __expf(am[jj] - m_all);
+                    den = fmaf(wj[jj], al[jj], den);
+                }
+                float merged[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    float num = 0.0f;
+#pragma unroll
+                    for (int jj = 0; jj < ASP; ++jj) num = fmaf(wj[jj], ao[t][jj][c], num);
+                    merged[c] = uok[t] && uchunk[t] * 256 + xcol < K ? num / den : 0.0f;
+                }
+                xr[t][0][0] = pack_bf16x2(merged[0], merged[1]);
+                xr[t][0][1] = pack_bf16x2(merged[2], merged[3]);
+            }
+#pragma unroll
+            for (int q = 0; q < XL; ++q) {
+#pragma unroll
+                for (int j = 0; j < NE / 2; ++j) {
+                    const float f0 = __uint_as_float(xr[t][q][j] << 16), f1 = __uint_as_float(xr[t][q][j] & 0xffff0000u);
+                    const float w0 = __uint_as_float(nw[t][j] << 16), w1 = __uint_as_float(nw[t][j] & 0xffff0000u);
+                    pss[q] = fmaf(f0, f0, pss[q]);
+                    pss[q] = fmaf(f1, f1, pss[q]);
+                    pmx[q] = fmaxf(pmx[q], fmaxf(fabsf(__fmul_rn(f0, w0)), fabsf(__fmul_rn(f1, w1))));
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < XL; ++q) {
+        const float a = group_reduce<LPR, false>(pss[q]);
+        const float b = group_reduce<LPR, true>(pmx[q]);
+        if ((lane % LPR) == 0) part_s[xrow0 + RPL * q][wave] = float2{a, b};
+    }
+    __syncthreads();                             // barrier 1: every wave's partials
+
+    // ---- (4) totals per row -> rstd and the quantisation scale; every wave for itself (lane 16 r + w: row r, wave w)
+    float sval_mine = 0.0f;                      // finishing waves: the bf16 scale of this lane's row fin_m
+#pragma unroll
+    for (int ps = 0; ps < PASSES; ++ps) {
+        const int row = 4 * ps + (lane >> 4);
+        const float2 v = part_s[row < MR ? row : 0][lane & 15];
+        const float total = group_reduce<16, false>(v.x);
+        const float pmax = group_reduce<16, true>(v.y);
+        const float r = rsqrtf(total / static_cast<float>(K) + eps);
+        const float amax_y = fabsf(round_bf16(__fmul_rn(pmax, r)));          // = max |y| of the row, exactly
+        uint16_t sb;
+        const float s_mul = quant_scale(amax_y, quant_mode, &sb);
+        if ((lane & 15) == 0 && row < MR) {
+            stat_w[wave][row][0] = r;
+            stat_w[wave][row][1] = s_mul;
+            if (writer && wave == 0 && io.s_out != nullptr && row < M) io.s_out[row] = sb;
+        }
+        if (ps == wave) sval_mine = bf16_bits_to_float(sb);                  // finishing wave q: rows 4q .. 4q+3 = pass q, same lanes
+    }
+
+    // ---- (5) norm + quantisation into the LDS slot, operands out; then the weights: 2-bit expansion, MFMA
+    i32x4 acc = i32x4{0, 0, 0, 0};
+    if (has_work) {
+        u32x4 bq[CT][4];
+#pragma unroll
+        for (int t = 0; t < CT; ++t) {
+            const int col0 = uchunk[t] * 256;
+#pragma unroll
+            for (int q = 0; q < XL; ++q) {
+                const int row = xrow0 + RPL * q;
+                uint32_t d[NE / 4];
+                chain_quantise<NE>(xr[t][q], nw[t], stat_w[wave][row][0], stat_w[wave][row][1], quant_mode, d);
+                const bool pub = writer && io.xq_out != nullptr && row < M && uok[t] && col0 + xcol < K;
+                if constexpr (NE == 8) {
+                    *reinterpret_cast<u32x2*>(slab + row * kChainSlabPitch + xcol) = u32x2{d[0], d[1]};
+                    if (pub) *reinterpret_cast<u32x2*>(io.xq_out + static_cast<size_t>(row) * K + col0 + xcol) = u32x2{d[0], d[1]};
+                } else {
+                    *reinterpret_cast<uint32_t*>(slab + row * kChainSlabPitch + xcol) = d[0];
+                    if (pub) *reinterpret_cast<uint32_t*>(io.xq_out + static_cast<size_t>(row) * K + col0 + xcol) = d[0];
+                }
+            }
+            const uint8_t* src = slab + (i < MR ? i : MR) * kChainSlabPitch + g * 64;
+#pragma unroll
+            for (int p = 0; p < 4; ++p) bq[t][p] = *reinterpret_cast<const u32x4*>(src + 16 * p);
+        }
+        __builtin_amdgcn_sched_barrier(0);       // nothing that needs a weight word moves up
+#pragma unroll
+        for (int t = 0; t < CT; ++t) {
+            if (t > 0 && !uok[t]) continue;      // scalar
+            const uint32_t wc[4] = {wq[t].x, wq[t].y, wq[t].z, wq[t].w};
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(expand_word_i8(wc[c]), __builtin_bit_cast(i32x4, bq[t][c]), acc, 0, 0, 0);
+        }
+    }
+
+    // ---- (6) accumulators to LDS as [batch row][column], barrier 2, finishing (as terna_chain_chunk_kernel)
+    *reinterpret_cast<i32x4*>(&red[wave][i * 16 + 4 * g]) = acc;
+    if (finisher) asm volatile("" : "+v"(ew), "+v"(eres), "+v"(enw));
+    __syncthreads();
+    if (finisher) {
+        const bool row_ok = fin_m < M;
+        const int* rp = &red[0][64 * wave + lane];
+        int sum = rp[0];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) sum += rp[w * 256];
+        EpilogueRegs e;
+        e.s = sval_mine;
+        e.w[0] = __uint_as_float(ew << 16);
+        const uint16_t o = apply_epilogue<int>(EP_I8_DECODE, e, 0, sum >> kI8WeightShift);
+        const uint32_t o32 = o;
+        const uint32_t op = o32 | (dpp_permute_u32<kDppSwapPairs>(o32) << 16);
+        if constexpr (EPI == CEPI_STORE) {
+            if ((lane & 1) == 0 && row_ok) *reinterpret_cast<uint32_t*>(io.out + static_cast<size_t>(fin_m) * N + fin_n) = op;
+        } else {
+            const float hv = row_ok ? round_bf16(__uint_as_float(eres << 16) + bf16_bits_to_float(o)) : 0.0f;
+            float ssq = hv * hv;
+            float pmax = fabsf(__fmul_rn(hv, __uint_as_float(enw << 16)));
+            ssq = group_reduce<16, false>(ssq);
+            pmax = group_reduce<16, true>(pmax);
+            const uint32_t h32 = float_to_bf16_bits(hv);
+            const uint32_t hp = h32 | (dpp_permute_u32<kDppSwapPairs>(h32) << 16);
+            if (row_ok) {
+                if ((lane & 1) == 0) {
+                    *reinterpret_cast<uint32_t*>(io.out + static_cast<size_t>(fin_m) * N + fin_n) = hp;
+                    if (io.raw_out != nullptr) *reinterpret_cast<uint32_t*>(io.raw_out + static_cast<size_t>(fin_m) * N + fin_n) = op;
+                }
+                if ((lane & 15) == 0) io.stats_out[static_cast<size_t>(fin_m) * (N / 16) + band] = float2{ssq, pmax};
+            }
+        }
+    }
+}
+
 }  // namespace terna
