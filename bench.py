@@ -48,10 +48,10 @@ METRIC = "TernaSpMM GB/s + %HBM roofline (M=8,K=N=2560); 2B-shape decode tok/s"
 # HBM bytes per launch of the small-M P2 kernel on the default workload (M=8, average over the four matrices):
 # a counter measurement, not part of this run -- two rocprofv3 --pmc runs of this file (FETCH_SIZE, WRITE_SIZE),
 # scaled by what the same counters read for a 256 MiB copy.  Quoted with its source; null for any other workload.
-TRAFFIC = {"bytes_per_launch": (19175.4 + 356.0) * 1024 / 4,
-           "source": "profiles/decode_packed_kernel_hbm_traffic.md (two rocprofv3 --pmc runs, FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 by the copy probe)",
-           "measured_at": "the tree of the commit 'Chain at 5-8 rows: norm + quantisation of the down projection's input as one launch ...' "
-                          "(the last change to csrc/decode_packed_kernel.h and launch_decode_packed.hip)"}
+TRAFFIC = {"bytes_per_launch": (19046.0 + 356.0) * 1024 / 4,
+           "source": "profiles/decode_chunk_kernels_hbm_traffic.md (two rocprofv3 --pmc runs, FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 by the copy probe)",
+           "measured_at": "the tree of the commit 'O projection of the chained step in the wide-load form ...' "
+                          "(csrc/decode_chunk_kernel.h and launch_decode_packed.hip as of 'Small-M kernel with four band-tiles per weight load ...')"}
 
 
 def vp(t):
@@ -771,8 +771,8 @@ def main():
                      "traffic": TRAFFIC["bytes_per_launch"] if default_workload else None,
                      "traffic_source": TRAFFIC["source"] if default_workload else None,
                      "traffic_measured_at": TRAFFIC["measured_at"] if default_workload else None,
-                     "kernel": ("terna_decode_packed_kernel<bf16>" if args.layout == "packed"
-                                else "terna_decode_kernel<bf16>"),
+                     "kernel": ("terna_decode_chunk_kernel<bf16> / terna_decode_chunk4_kernel<bf16>" if args.layout == "packed" and args.m <= 16
+                                else ("terna_decode_packed_kernel<bf16>" if args.layout == "packed" else "terna_decode_kernel<bf16>")),
                      "algorithmic_bytes_per_launch": step_bytes / launches_per_step,
                      "avg_launch_us": launch_us},
         "tokens_per_s_linear_layers_only": args.m / (ms_per_step * 1e-3) if args.layers == 30 else None,
