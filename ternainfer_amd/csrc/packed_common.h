@@ -103,12 +103,29 @@ __device__ __forceinline__ unsigned long long repack_fingerprint(const RepackGua
     h ^= fingerprint_mix(b1 + 0xc2b2ae3d27d4eb4full * (lane + 65));
     h ^= fingerprint_mix(b2 + 0x165667b19e3779f9ull * (lane + 129));
     h ^= fingerprint_mix(((s0 << 32) | s1) + 0x27d4eb2f165667c5ull * (lane + 193));
+    // Six exchange steps -- pairs, quads, eights (lane i <-> 7 - i), sixteens (i <-> 15 - i), the 16-lane rows, the halves --
+    // with the data-parallel permutations of the VALU: an LDS-crossbar shuffle costs a hundred cycles a step, and the
+    // workgroup that checks a cached copy must not outlast the ones that do the work.  Lane 0's value depends on all 64.
     uint32_t lo = static_cast<uint32_t>(h), hi32 = static_cast<uint32_t>(h >> 32);
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-        lo += __shfl_xor(lo, off) * 0x85ebca6bu + 1u;          // order-independent within a pair, not across pairs
-        hi32 ^= __shfl_xor(hi32, off);
-    }
+    auto fold = [&](uint32_t partner_lo, uint32_t partner_hi) {
+        lo += partner_lo * 0x85ebca6bu + 1u;                    // not symmetric: the lanes end up with different values
+        hi32 ^= partner_hi;
+    };
+    auto dpp = [](uint32_t v, auto ctrl) {
+        return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), decltype(ctrl)::value, 0xf, 0xf, true));
+    };
+    auto swap_rows = [](uint32_t v, bool halves) {              // the value of lane ^ 16 (lane ^ 32): see cross_row_reduce
+        uint32_t a = v, b = v;
+        if (halves) asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+        else asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+        return a ^ b ^ v;                                       // {a, b} = {own, partner}
+    };
+    fold(dpp(lo, std::integral_constant<int, 0xB1>{}), dpp(hi32, std::integral_constant<int, 0xB1>{}));      // quad_perm [1,0,3,2]
+    fold(dpp(lo, std::integral_constant<int, 0x4E>{}), dpp(hi32, std::integral_constant<int, 0x4E>{}));      // quad_perm [2,3,0,1]
+    fold(dpp(lo, std::integral_constant<int, 0x141>{}), dpp(hi32, std::integral_constant<int, 0x141>{}));    // row_half_mirror
+    fold(dpp(lo, std::integral_constant<int, 0x140>{}), dpp(hi32, std::integral_constant<int, 0x140>{}));    // row_mirror
+    fold(swap_rows(lo, false), swap_rows(hi32, false));
+    fold(swap_rows(lo, true), swap_rows(hi32, true));
     return fingerprint_mix(((static_cast<unsigned long long>(hi32) << 32) | lo) ^ static_cast<unsigned long long>(static_cast<uint32_t>(total)));
 }
 // One wave: compare with the recorded fingerprint; on a mismatch report the copy's id in the host-visible words.
