@@ -106,12 +106,13 @@ __device__ __forceinline__ void chain_quantise(const uint32_t (&hraw)[NE / 2], c
 
 // NBANDS = 1: one band per workgroup, a unit of work is a chunk; CEPI_STORE / CEPI_RESIDUAL.
 // NBANDS = 4: gate+up with the bands of w1 and w3 interleaved (band 2j = rows 16j .. of w1, band 2j+1 the same rows of
-//             w3), two gate / up pairs per workgroup so that one round of workgroups covers 864 bands; a unit of work is
-//             (chunk, pair): unit u is chunk u of pair 0 for u < chunks, chunk u - chunks of pair 1 behind it; CEPI_GATE.
+//             w3), two gate / up pairs per workgroup so that one round of workgroups covers 864 bands; CEPI_GATE.  A unit of
+//             work is (chunk, pair) -- unit u is chunk u of pair 0 for u < chunks, chunk u - chunks of pair 1 behind it --
+//             or, UNIT_BANDS = 4, a chunk with all four bands: its activations are then normed and quantised once.
 // The 16 - M working waves take the units round robin, CT each at most.
 // MR = 1, 2, 4 or 8 >= M: rows of the wave's LDS slot.  One row: 64 lanes x 4 columns; more: 32 lanes x 8 columns, two rows
 // per load.
-template <int NBANDS, int CT, int MR, int EPI>
+template <int NBANDS, int CT, int MR, int EPI, int UNIT_BANDS = (NBANDS == 4 ? 2 : 1)>
 __global__ __launch_bounds__(kChunkWaves * 64) void terna_chain_chunk_kernel(
     const uint16_t* __restrict__ h, const uint16_t* __restrict__ norm_w, const uint32_t* __restrict__ packed,
     const float2* __restrict__ stats_in, int M, int N, int K, int stats_count, float eps, int ws_num, int quant_mode, ChainIo io)
@@ -124,7 +125,9 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_chain_chunk_kernel(
     constexpr int RPL = 64 / LPR;                // rows per load
     constexpr int XL = MR / RPL;                 // activation loads per chunk
     constexpr int FW = (MR + 3) / 4;             // finishing waves per band (pair)
-    constexpr int UB = NBANDS == 4 ? 2 : 1;      // bands per unit of work
+    constexpr int UB = UNIT_BANDS;               // bands per unit of work
+    static_assert(UB == NBANDS || (NBANDS == 4 && UB == 2), "a unit covers the workgroup's bands or one gate / up pair");
+    constexpr int UPAIRS = NBANDS / UB;          // units per chunk
     constexpr int PT = kStatsMaxPartials / 64;
 
     __shared__ int red[WAVES][NBANDS][256];
@@ -148,7 +151,7 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_chain_chunk_kernel(
 #pragma unroll
     for (int t = 0; t < CT; ++t) {
         const int u = wave - M + workers * t;
-        if constexpr (NBANDS == 4) {
+        if constexpr (UPAIRS == 2) {
             upair[t] = u >= chunks ? 1 : 0;
             uchunk[t] = u - upair[t] * chunks;
             uok[t] = !reducer && u < 2 * chunks;
@@ -251,7 +254,7 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_chain_chunk_kernel(
     __syncthreads();                             // barrier 1: the rows' statistics are in LDS
 
     // ---- per unit: norm + quantisation into the LDS slot, operands out, 2-bit expansion, MFMA
-    constexpr int NACC = NBANDS == 4 ? 2 : 1;    // accumulator sets: one per pair
+    constexpr int NACC = UPAIRS;                 // accumulator sets: one per pair that has units of its own
     i32x4 acc[NACC][UB];
 #pragma unroll
     for (int p = 0; p < NACC; ++p)
@@ -290,7 +293,7 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_chain_chunk_kernel(
                         dst[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(expand_word_i8(wc[c]), __builtin_bit_cast(i32x4, bq[c]), dst[b], 0, 0, 0);
                 }
             };
-            if constexpr (NBANDS == 4) {
+            if constexpr (UPAIRS == 2) {
                 if (upair[t] == 0) multiply(acc[0]);             // scalar
                 else multiply(acc[1]);
             } else {

@@ -83,6 +83,7 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_decode_chunk_kernel(
             wq[t] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, tile0 + g < ktiles ? lane * 16 : kBufferOutOfRange,
                                                                                    (band * ktiles + tile0) * 256, 0));
         }
+        __builtin_amdgcn_sched_barrier(0);       // nothing from below is scheduled ahead of the weight requests
     }
     // (A workgroup barrier here, so that every wave's weight requests precede anybody's activation requests, was measured:
     // slower -- the activations then arrive last and everything waits for them.)
@@ -164,7 +165,7 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_decode_chunk_kernel(
         if constexpr (BF16) {
             e.s = 1.0f;
             e.w[0] = __uint_as_float(ew);
-            o = apply_epilogue<float>(ep.kind, e, 0, sum * kBf16WeightUndo);
+            o = apply_epilogue<float>(EP_BF16, e, 0, sum * kBf16WeightUndo);
         } else {
             e.s = __uint_as_float(es << 16);
             e.w[0] = __uint_as_float(ew << 16);
@@ -185,7 +186,11 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_decode_chunk_kernel(
 // (chunks <= 16, so a wave has at most one unit of each pair and every SIMD gets the same number of units).  A wave
 // leaves one accumulator per band in LDS (zeros for a pair it had no unit of); all 16 waves finish: wave 4b + q the
 // accumulators of lanes 16q .. 16q+15 of band b.
-template <typename Act, int MR, bool GUARD = false>
+// UNIT_BANDS = 4: a unit is a chunk with all four bands -- half as many activation loads and stagings, ten working waves
+// instead of sixteen for K = 2560.  Measured on gate+up: the same at 8 rows (5.20 against 5.22 us), slower at 1 - 4 rows
+// (5.06 against 4.83); not instantiated by the launcher.  (In the chained form, where the unit's activations are also
+// normed and quantised, the whole-chunk unit is the faster one: chain_chunk_kernel.h.)
+template <typename Act, int MR, bool GUARD = false, int UNIT_BANDS = 2>
 __global__ __launch_bounds__(kChunkWaves * 64) void terna_decode_chunk4_kernel(
     const Act* __restrict__ x, const uint32_t* __restrict__ packed, uint16_t* __restrict__ out,
     int M, int N, int K, Epilogue ep, RepackGuard guard)
@@ -222,34 +227,44 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_decode_chunk4_kernel(
     const int i = lane & 15, g = lane >> 4;
 
     // this wave's units
-    int upair[2], uchunk[2];
-    bool uok[2];
+    constexpr int UB = UNIT_BANDS;
+    constexpr int UT = 4 / UB;                   // unit slots per wave: two (chunk, pair) units, or one whole chunk
+    static_assert(UB == 2 || UB == 4, "a gate / up pair or all four bands");
+    int upair[UT], uchunk[UT];
+    bool uok[UT];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < UT; ++t) {
         const int u = wave + WAVES * t;
-        upair[t] = u >= chunks ? 1 : 0;
-        uchunk[t] = u - upair[t] * chunks;
-        uok[t] = u < 2 * chunks;
+        if constexpr (UB == 2) {
+            upair[t] = u >= chunks ? 1 : 0;
+            uchunk[t] = u - upair[t] * chunks;
+            uok[t] = u < 2 * chunks;
+        } else {
+            upair[t] = 0;
+            uchunk[t] = u;
+            uok[t] = u < chunks;
+        }
     }
 
     // ---- (1) the weights of both units, at once (a unit the wave does not have: out of range, zeros)
     const __amdgpu_buffer_rsrc_t rw = make_raw_buffer(packed, static_cast<uint32_t>(N >> 4) * static_cast<uint32_t>(ktiles) * 256u);
-    u32x4 wq[2][2];
+    u32x4 wq[UT][UB];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < UT; ++t) {
         const int tile0 = uchunk[t] * 4;
         const int voff = uok[t] && tile0 + g < ktiles ? lane * 16 : kBufferOutOfRange;
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
-            wq[t][b] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, voff, ((band0 + 2 * upair[t] + b) * ktiles + tile0) * 256, 0));
+        for (int b = 0; b < UB; ++b)
+            wq[t][b] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, voff, ((band0 + UB * upair[t] + b) * ktiles + tile0) * 256, 0));
     }
+    __builtin_amdgcn_sched_barrier(0);           // nothing from below is scheduled ahead of the weight requests
     // ---- (2) the activations of the units' chunks
     const int rowbytes = K * SZ;
     const __amdgpu_buffer_rsrc_t rx = make_raw_buffer(x, static_cast<uint32_t>(M) * rowbytes);
     const int xrow = lane / ROWLANES, xcol = (lane % ROWLANES) * 16;
-    u32x4 xr[2][XL];
+    u32x4 xr[UT][XL];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < UT; ++t) {
         const int col0 = uchunk[t] * (256 * SZ);
 #pragma unroll
         for (int h = 0; h < XL; ++h) {
@@ -277,11 +292,11 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_decode_chunk4_kernel(
     if constexpr (MR < 16) {
         for (int o = MR * PITCH + lane * 16; o < SLAB_ROWS * PITCH; o += 64 * 16) *reinterpret_cast<u32x4*>(slab + o) = u32x4{0u, 0u, 0u, 0u};
     }
-    Acc acc[2][2];
+    Acc acc[UT][UB];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        acc[t][0] = Acc{0, 0, 0, 0};
-        acc[t][1] = Acc{0, 0, 0, 0};
+    for (int t = 0; t < UT; ++t) {
+#pragma unroll
+        for (int b = 0; b < UB; ++b) acc[t][b] = Acc{0, 0, 0, 0};
         if (uok[t]) {
 #pragma unroll
             for (int h = 0; h < XL; ++h) *reinterpret_cast<u32x4*>(slab + (xrow + ROWS_PER_LOAD * h) * PITCH + xcol) = xr[t][h];
@@ -290,7 +305,7 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_decode_chunk4_kernel(
 #pragma unroll
             for (int p = 0; p < PIECES; ++p) bq[p] = *reinterpret_cast<const u32x4*>(src + 16 * p);
 #pragma unroll
-            for (int b = 0; b < 2; ++b) {
+            for (int b = 0; b < UB; ++b) {
                 const uint32_t wc[4] = {wq[t][b].x, wq[t][b].y, wq[t][b].z, wq[t][b].w};
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
@@ -307,13 +322,16 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_decode_chunk4_kernel(
         }
     }
     // ---- (5) one accumulator per band into LDS: unit 0 is of pair upair[0], unit 1 (if there is one) of pair 1
-    {
+    if constexpr (UB == 2) {
         const bool first_is_pair0 = upair[0] == 0;                 // scalar
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
             red[wave][b][lane] = first_is_pair0 ? acc[0][b] : Acc{0, 0, 0, 0};
-            red[wave][2 + b][lane] = first_is_pair0 ? acc[1][b] : acc[0][b];
+            red[wave][2 + b][lane] = first_is_pair0 ? acc[UT - 1][b] : acc[0][b];
         }
+    } else {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) red[wave][b][lane] = acc[0][b];
     }
     asm volatile("" : "+v"(es), "+v"(ew));
     __syncthreads();
@@ -327,7 +345,7 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_decode_chunk4_kernel(
         if constexpr (BF16) {
             e.s = 1.0f;
             e.w[0] = __uint_as_float(ew);
-            o = apply_epilogue<float>(ep.kind, e, 0, sum * kBf16WeightUndo);
+            o = apply_epilogue<float>(EP_BF16, e, 0, sum * kBf16WeightUndo);
         } else {
             e.s = __uint_as_float(es << 16);
             e.w[0] = __uint_as_float(ew << 16);
