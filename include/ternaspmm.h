@@ -221,8 +221,10 @@ void ternaspmm_relu2_mul_rmsnorm_quant(const terna_bf16* x13, const terna_bf16* 
  * decode epilogue in ONE launch (x, residual, sum_out, norm_weight, eps as ternaspmm_rmsnorm_quant; packed, out,
  * ws, ws_num as bitlinear_TernaSpMM_packed).  xq_out / s_out are optional copies of the quantised activations
  * (NULL = not written).  sum_out must not alias x or residual (every workgroup reads both).  Supported: M <= 16
- * and K <= 3072 (K <= 2560 when N > 4096); returns 1 when the launch was enqueued, 0 when the shape is outside
- * that range and nothing was done -- the caller then runs ternaspmm_rmsnorm_quant + bitlinear_TernaSpMM_packed.
+ * and K <= 3072 (K <= 2560 when N > 4096); without a residual, M <= 8 and N <= 4096 also K <= 8192 (the kernel of
+ * ternaspmm_fused_linear's NORM prologue serves those).  Returns 1 when the launch was enqueued, 0 when the shape is
+ * outside that range and nothing was done (no argument is read) -- the caller then runs ternaspmm_rmsnorm_quant +
+ * bitlinear_TernaSpMM_packed.
  * Every workgroup repeats the prologue arithmetic (variants for 1, 2, 4, 8 and 16 rows: the lanes of a wave are spread
  * over the rows that exist), so the single launch pays for M = 1 (measured on MI355X: 5.2-5.6 us against 7.2-7.5 us
  * for the pair), still pays for M <= 4 and is no faster than the pair from M = 8 on. */

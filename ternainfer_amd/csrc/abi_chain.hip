@@ -246,6 +246,33 @@ bool chain_chunk_enabled()
 
 }  // namespace
 
+namespace terna {
+
+bool launch_norm_linear_chunk(const uint16_t* x, const uint16_t* norm_w, const uint32_t* packed, uint16_t* out, const uint16_t* ws,
+                              int ws_num, int8_t* xq_out, uint16_t* s_out, int M, int N, int K, float eps, int quant_mode,
+                              hipStream_t st)
+{
+    if (!chain_chunk_enabled() || M < 1 || M > 8 || static_cast<long long>(N) * K / 4 >= (1ll << 31)) return false;
+    ChainArgs a{};
+    a.x = x;
+    a.norm_w = norm_w;
+    a.packed = packed;
+    a.M = M; a.N = N; a.K = K;
+    a.eps = eps;
+    a.out = out;
+    a.ws = ws;
+    a.ws_num = ws_num;
+    a.xq_out = xq_out;
+    a.s_out = s_out;
+    a.qmode = quant_mode;
+    a.ex = FusedExtra{};
+    a.grid = dim3(N / 16);
+    a.st = st;
+    return launch_norm_chunk_by_rows<CEPI_STORE>(a, (K / 64 + 3) / 4);
+}
+
+}  // namespace terna
+
 extern "C" {
 
 int ternaspmm_row_stats_count(int K) { return K < 8 || (K & 7) ? -1 : (K + 511) / 512; }

@@ -9,6 +9,7 @@
 #include "host_util.h"
 #include "norm_quant_kernel.h"
 #include "decode_fused_kernel.h"
+#include "launchers.h"
 
 using namespace terna;
 
@@ -62,6 +63,9 @@ void ternaspmm_relu2_mul_rmsnorm_quant(const terna_bf16* x13, const terna_bf16* 
     if (e != hipSuccess) die("ternaspmm_relu2_mul_rmsnorm_quant", e, __LINE__);
 }
 
+// One band per workgroup repeats the prologue in every workgroup: only where one round of workgroups covers the matrix.
+static bool bands_fit_one_round(int N) { return N / 16 <= 256; }
+
 // mode: FUSED_PLAIN / FUSED_RESIDUAL / FUSED_GLU.  Returns 1 when a launch was enqueued.
 static int launch_decode_fused(int mode, const terna_bf16* x, const terna_bf16* residual, terna_bf16* sum_out,
                                const terna_bf16* norm_weight, float eps, const void* packed, terna_bf16* out,
@@ -69,6 +73,14 @@ static int launch_decode_fused(int mode, const terna_bf16* x, const terna_bf16* 
                                int K, hipStream_t st)
 {
     if (!shape_ok(M, N, K) || !groups_ok(ws_num) || M > 16) return 0;
+    // Rows longer than the per-tile kernels below take (48 band-tiles), no second operand, up to 8 rows: the wide-load
+    // kernel of the chained step's NORM prologue.  For the shorter rows it measured level with the kernels here at
+    // 1-4 rows and 2 % behind at 6-8 rows in a whole decode step, so they keep those.
+    if (mode == FUSED_PLAIN && K / 64 > 16 * 3)
+        return bands_fit_one_round(N) && launch_norm_linear_chunk(x, norm_weight, static_cast<const uint32_t*>(packed), out, ws, ws_num,
+                                                                  xq_out, s_out, M, N, K, eps, quant_mode(), st)
+                   ? 1
+                   : 0;
     const int ktiles = K / 64;
     const int bands = N / 16;
     static const int forced_waves = [] {

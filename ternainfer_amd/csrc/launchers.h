@@ -78,6 +78,12 @@ extern template void launch_prefill_packed<uint16_t>(const uint16_t*, const uint
 extern template PrefillPlan plan_prefill_packed<int8_t>(const void*, int, int, int, const void*, size_t);
 extern template PrefillPlan plan_prefill_packed<uint16_t>(const void*, int, int, int, const void*, size_t);
 
+// norm -> quantisation -> int8 linear on a P2 weight, statistics taken inside, plain store, up to 8 rows, in the
+// wide-load form (chain_chunk_kernel.h; defined in abi_chain.hip).  False where the shape is not covered: nothing enqueued.
+bool launch_norm_linear_chunk(const uint16_t* x, const uint16_t* norm_w, const uint32_t* packed, uint16_t* out, const uint16_t* ws,
+                              int ws_num, int8_t* xq_out, uint16_t* s_out, int M, int N, int K, float eps, int quant_mode,
+                              hipStream_t st);
+
 // Tuning override shared by the two small-M launchers: TERNASPMM_DECODE_WAVES=4|8|16 forces one variant.
 int decode_waves_override();
 

@@ -328,6 +328,17 @@ def _bf16_key(b):
 @pytest.mark.parametrize("n,k,ws_num,res", [(3840, 2560, 3, True), (2560, 2560, 1, False), (13824, 2560, 2, True),
                                             (256, 192, 1, True), (320, 64, 2, False), (4160, 128, 1, False)])
 def test_fused_prologue_linear(lib, m, n, k, ws_num, res):
+    _check_fused_prologue_linear(lib, m, n, k, ws_num, res)
+
+
+@pytest.mark.parametrize("m", [1, 3, 8])
+@pytest.mark.parametrize("n,k,ws_num", [(2560, 6912, 1), (320, 8192, 2), (4096, 3136, 1)])
+def test_fused_prologue_linear_long_rows(lib, m, n, k, ws_num):
+    """Without a residual, up to 8 rows and 4096 outputs the entry point takes rows of up to 8192 columns."""
+    _check_fused_prologue_linear(lib, m, n, k, ws_num, False)
+
+
+def _check_fused_prologue_linear(lib, m, n, k, ws_num, res):
     """One launch: residual add -> norm -> quantise -> ternary matmul -> epilogue.  The published h is exact,
     s and q are what the oracle quantiser gives for a norm output within one bf16 step of the float64 one,
     and the matmul + epilogue on the kernel's own (q, s) is bit-exact."""
@@ -426,7 +437,8 @@ def test_quant_modes_of_the_prologue_kernels(lib, mode):
 
 def test_fused_prologue_linear_declines_what_it_cannot_do(lib):
     z = torch.zeros(64, dtype=torch.int32, device="cuda")
-    for m, n, k in [(17, 256, 192), (8, 2560, 6912), (8, 13824, 3136)]:
+    # declined before any argument is read: the buffers here are far smaller than the shapes
+    for m, n, k in [(17, 256, 192), (8, 2560, 13824), (16, 2560, 6912), (8, 13824, 3136)]:
         assert lib.bitlinear_TernaSpMM_packed_fused(_vp(z), None, None, _vp(z), 1e-5, _vp(z), _vp(z), _vp(z), 1, None, None,
                                                     m, n, k, None) == 0
 
