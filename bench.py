@@ -243,6 +243,8 @@ def measure_model(torch, batch, act="int8", prefetch=True, gen_tokens=256, check
     model.chain = chain
     if os.environ.get("TERNA_BENCH_CHAIN_ROWS"):           # measurement aids
         model.chain_rows = int(os.environ["TERNA_BENCH_CHAIN_ROWS"])
+    if os.environ.get("TERNA_BENCH_SPLIT_ROWS"):
+        model.split_rows = int(os.environ["TERNA_BENCH_SPLIT_ROWS"])
     if os.environ.get("TERNA_BENCH_CHAIN_DOWN_ROWS"):
         for blk in model.layers:
             blk.chain_down_rows = int(os.environ["TERNA_BENCH_CHAIN_DOWN_ROWS"])

@@ -187,6 +187,24 @@ bool launch_chunk_by_rows(const ChainArgs& a, int units)
     return true;
 }
 
+// Activations quantised already (int8 rows + scales), producing epilogue, up to 8 rows: all 16 waves share the units.
+template <int NBANDS, int EPI>
+bool launch_chunk_quantised(const ChainArgs& a, const uint16_t* s_in, int units)
+{
+    ChainIo io{a.out, a.ws, nullptr, nullptr, a.ex.epi_residual, a.ex.epi_next_w, a.ex.stats_out, a.ex.raw_out};
+    io.s_in = s_in;
+    const int ct = (units + kChunkWaves - 1) / kChunkWaves;
+    if (ct > 3 || a.M > 8) return false;
+#define TERNA_CHAIN_XQ(CT)                                                                                              \
+    terna_chain_chunk_kernel<NBANDS, CT, 8, EPI, (NBANDS == 4 ? 2 : 1), true><<<a.grid, dim3(kChunkWaves * 64), 0, a.st>>>( \
+        a.x, nullptr, a.packed, nullptr, a.M, a.N, a.K, 0, 0.0f, a.ws_num, 0, io)
+    if (ct == 1) TERNA_CHAIN_XQ(1);
+    else if (ct == 2) TERNA_CHAIN_XQ(2);
+    else TERNA_CHAIN_XQ(3);
+#undef TERNA_CHAIN_XQ
+    return true;
+}
+
 // The statistics-inside prologues in the wide-load form (terna_chain_norm_kernel): plain rows ...
 template <int EPI>
 bool launch_norm_chunk_by_rows(const ChainArgs& a, int chunks)
@@ -321,18 +339,45 @@ int ternaspmm_fused_linear(const ternaspmm_fused_linear_desc* d, terna_stream st
     const int M = d->M, N = d->N, K = d->K;
     const int pro = d->prologue, epi = d->epilogue;
     if (pro == TERNASPMM_PROLOGUE_QUANTISED) {
-        // activations already quantised (ternaspmm_quant_from_stats, ternaspmm_rmsnorm_quant): the small-M kernel of
-        // bitlinear_TernaSpMM_packed with the producing epilogue
-        if (!shape_ok(M, N, K) || !groups_ok(d->ws_num) || !i8_depth_ok(K) || M > 16 || epi != TERNASPMM_EPILOGUE_RESIDUAL ||
+        // activations already quantised (ternaspmm_quant_from_stats, ternaspmm_rmsnorm_quant): the matmul of
+        // bitlinear_TernaSpMM_packed with a producing epilogue
+        const bool gate = epi == TERNASPMM_EPILOGUE_GATE;
+        const int bands = N / 16, chunks = (K / 64 + 3) / 4;
+        if (!shape_ok(M, N, K) || !groups_ok(d->ws_num) || !i8_depth_ok(K) || M > 16 || (epi != TERNASPMM_EPILOGUE_RESIDUAL && !gate) ||
             d->x == nullptr || d->s_in == nullptr || d->packed == nullptr || d->ws == nullptr || d->out == nullptr ||
-            d->residual == nullptr || d->next_norm_weight == nullptr || d->stats_out == nullptr || N / 16 > kStatsMaxPartials)
+            d->next_norm_weight == nullptr || d->stats_out == nullptr)
             return -1;
-        const Epilogue ep{d->s_in, d->ws, nullptr, d->ws_num, EP_I8_DECODE};
-        launch_decode_packed_producer(static_cast<const int8_t*>(d->x), static_cast<const uint32_t*>(d->packed), d->out, ep, M, N, K,
-                                      d->residual, d->next_norm_weight, d->stats_out, d->raw_out, static_cast<hipStream_t>(stream));
+        if (gate ? (d->ws_num != 2 || bands % 4 != 0 || bands / 2 > kStatsMaxPartials) : (d->residual == nullptr || bands > kStatsMaxPartials))
+            return -1;
+        const hipStream_t st = static_cast<hipStream_t>(stream);
+        ChainArgs a{};
+        a.x = static_cast<const uint16_t*>(d->x);
+        a.packed = static_cast<const uint32_t*>(d->packed);
+        a.M = M; a.N = N; a.K = K;
+        a.out = d->out;
+        a.ws = d->ws;
+        a.ws_num = d->ws_num;
+        a.ex = FusedExtra{nullptr, 0, d->residual, d->next_norm_weight, reinterpret_cast<float2*>(d->stats_out), d->raw_out};
+        a.st = st;
+        const bool wide = chain_chunk_enabled() && static_cast<long long>(N) * K / 4 < (1ll << 31);
+        bool done = false;
+        if (gate) {
+            // four bands (two gate / up pairs) per workgroup, a unit of work is a chunk of one pair
+            a.grid = dim3(bands / 4);
+            done = wide && launch_chunk_quantised<4, CEPI_GATE>(a, d->s_in, 2 * chunks);
+            if (!done) return -1;
+        } else {
+            a.grid = dim3(bands);
+            done = wide && launch_chunk_quantised<1, CEPI_RESIDUAL>(a, d->s_in, chunks);
+            if (!done) {
+                const Epilogue ep{d->s_in, d->ws, nullptr, d->ws_num, EP_I8_DECODE};
+                launch_decode_packed_producer(static_cast<const int8_t*>(d->x), static_cast<const uint32_t*>(d->packed), d->out, ep, M, N, K,
+                                              d->residual, d->next_norm_weight, d->stats_out, d->raw_out, st);
+            }
+        }
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) die("ternaspmm_fused_linear", e, __LINE__);
-        return N / 16;
+        return gate ? bands / 2 : bands;
     }
     if (!shape_ok(M, N, K) || !groups_ok(d->ws_num) || M > 8) return -1;
     const int ktiles = K / 64, bands = N / 16;

@@ -41,6 +41,7 @@ struct ChainIo {
     const uint16_t* next_w;          // producing epilogues: weights of the norm that follows
     float2* stats_out;               // [M][N/16] (CEPI_GATE: [M][N/32])
     uint16_t* raw_out;               // CEPI_RESIDUAL, optional: the linear's own output
+    const uint16_t* s_in = nullptr;  // activations quantised already (XQ): their scales, bf16 [M]
 };
 
 constexpr int kChainSlabPitch = 256 + 16;
@@ -112,9 +113,13 @@ __device__ __forceinline__ void chain_quantise(const uint32_t (&hraw)[NE / 2], c
 // The 16 - M working waves take the units round robin, CT each at most.
 // MR = 1, 2, 4 or 8 >= M: rows of the wave's LDS slot.  One row: 64 lanes x 4 columns; more: 32 lanes x 8 columns, two rows
 // per load.
-template <int NBANDS, int CT, int MR, int EPI, int UNIT_BANDS = (NBANDS == 4 ? 2 : 1)>
+// XQ: the activations are quantised already (`hin` is int8 [M][K], io.s_in their scales; a launch of
+// terna_quant_stats_kernel or of the norm kernel made them): no reducing waves, no statistics, no barrier ahead of the
+// matmul; all 16 waves share the units and a chunk's rows go from the load to the LDS slot as they are (16 bytes per lane,
+// four rows per load).  The producing epilogues are the same.
+template <int NBANDS, int CT, int MR, int EPI, int UNIT_BANDS = (NBANDS == 4 ? 2 : 1), bool XQ = false>
 __global__ __launch_bounds__(kChunkWaves * 64) void terna_chain_chunk_kernel(
-    const uint16_t* __restrict__ h, const uint16_t* __restrict__ norm_w, const uint32_t* __restrict__ packed,
+    const void* __restrict__ hin, const uint16_t* __restrict__ norm_w, const uint32_t* __restrict__ packed,
     const float2* __restrict__ stats_in, int M, int N, int K, int stats_count, float eps, int ws_num, int quant_mode, ChainIo io)
 {
     static_assert((NBANDS == 1 && (EPI == CEPI_STORE || EPI == CEPI_RESIDUAL)) || (NBANDS == 4 && EPI == CEPI_GATE), "see above");
@@ -129,10 +134,12 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_chain_chunk_kernel(
     static_assert(UB == NBANDS || (NBANDS == 4 && UB == 2), "a unit covers the workgroup's bands or one gate / up pair");
     constexpr int UPAIRS = NBANDS / UB;          // units per chunk
     constexpr int PT = kStatsMaxPartials / 64;
+    constexpr int XLQ = (MR + 3) / 4;            // XQ: 16-byte loads per lane and chunk (four rows of 256 bytes each)
 
     __shared__ int red[WAVES][NBANDS][256];
     __shared__ __align__(16) uint8_t slab_all[WAVES][(MR + 1) * kChainSlabPitch];
     __shared__ float rstd_s[8], smul_s[8], sval_s[8];
+    const uint16_t* h = static_cast<const uint16_t*>(hin);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -144,13 +151,14 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_chain_chunk_kernel(
     const bool writer = blockIdx.x == 0;
 
     // this wave's units of work
-    const bool reducer = wave < M;
-    const int workers = WAVES - M;
+    const int reducers = XQ ? 0 : M;
+    const bool reducer = wave < reducers;
+    const int workers = WAVES - reducers;
     int upair[CT], uchunk[CT];
     bool uok[CT];
 #pragma unroll
     for (int t = 0; t < CT; ++t) {
-        const int u = wave - M + workers * t;
+        const int u = wave - reducers + workers * t;
         if constexpr (UPAIRS == 2) {
             upair[t] = u >= chunks ? 1 : 0;
             uchunk[t] = u - upair[t] * chunks;
@@ -184,8 +192,9 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_chain_chunk_kernel(
     const int fin_col = lane & 15;
     const int out_cols = EPI == CEPI_GATE ? N / 2 : N;
     const int fin_n = (EPI == CEPI_GATE ? (static_cast<int>(blockIdx.x) * 2 + fin_p) : band0) * 16 + fin_col;   // output column
-    uint32_t ew = 0u, ew3 = 0u, eres = 0u, enw = 0u;
+    uint32_t ew = 0u, ew3 = 0u, eres = 0u, enw = 0u, es = 0u;
     auto request_epilogue = [&]() {
+        if constexpr (XQ) es = io.s_in[fin_m < M ? fin_m : 0];
         if constexpr (EPI == CEPI_GATE) {
             ew = io.ws[0];                       // gate rows (w1) and up rows (w3): one scale each
             ew3 = io.ws[1];
@@ -199,8 +208,10 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_chain_chunk_kernel(
         }
     };
     u32x4 wq[CT][UB];
-    uint32_t xr[CT][XL][NE / 2], nw[CT][NE / 2];
-    const int xrow0 = lane / LPR, xcol = (lane % LPR) * NE;      // row within a load, first of this lane's columns in the chunk
+    uint32_t xr[XQ ? 1 : CT][XL][NE / 2], nw[XQ ? 1 : CT][NE / 2];
+    u32x4 xq8[XQ ? CT : 1][XLQ];
+    const int xrow0 = XQ ? lane >> 4 : lane / LPR;               // row within a load, first of this lane's columns in the chunk
+    const int xcol = XQ ? (lane & 15) * 16 : (lane % LPR) * NE;
     uint8_t* slab = slab_all[wave];
     if (has_work) {
         const __amdgpu_buffer_rsrc_t rw = make_raw_buffer(packed, static_cast<uint32_t>(N >> 4) * static_cast<uint32_t>(ktiles) * 256u);
@@ -212,6 +223,19 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_chain_chunk_kernel(
             for (int b = 0; b < UB; ++b)
                 wq[t][b] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, voff, ((band0 + UB * upair[t] + b) * ktiles + tile0) * 256, 0));
         }
+        if constexpr (XQ) {
+            const __amdgpu_buffer_rsrc_t rx = make_raw_buffer(hin, static_cast<uint32_t>(M) * K);
+#pragma unroll
+            for (int t = 0; t < CT; ++t) {
+                const int col0 = uchunk[t] * 256;
+                const bool col_ok = uok[t] && col0 + xcol < K;
+#pragma unroll
+                for (int q = 0; q < XLQ; ++q) {
+                    const int row = xrow0 + 4 * q;
+                    xq8[t][q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rx, row < M && col_ok ? row * K + xcol : kBufferOutOfRange, col0, 0));
+                }
+            }
+        } else {
         const __amdgpu_buffer_rsrc_t rx = make_raw_buffer(h, static_cast<uint32_t>(M) * K * 2u);
         const __amdgpu_buffer_rsrc_t rn = make_raw_buffer(norm_w, static_cast<uint32_t>(K) * 2u);
 #pragma unroll
@@ -239,6 +263,7 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_chain_chunk_kernel(
                 nw[t][0] = v.x; nw[t][1] = v.y;
             }
         }
+        }
         if (finisher) request_epilogue();
         // the row of zeros behind the slab's MR rows
         for (int o = MR * kChainSlabPitch + lane * 16; o < (MR + 1) * kChainSlabPitch; o += 64 * 16) *reinterpret_cast<u32x4*>(slab + o) = u32x4{0u, 0u, 0u, 0u};
@@ -251,7 +276,7 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_chain_chunk_kernel(
             request_epilogue();
         }
     }
-    __syncthreads();                             // barrier 1: the rows' statistics are in LDS
+    if constexpr (!XQ) __syncthreads();          // barrier 1: the rows' statistics are in LDS
 
     // ---- per unit: norm + quantisation into the LDS slot, operands out, 2-bit expansion, MFMA
     constexpr int NACC = UPAIRS;                 // accumulator sets: one per pair that has units of its own
@@ -265,6 +290,13 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_chain_chunk_kernel(
         for (int t = 0; t < CT; ++t) {
             if (t > 0 && !uok[t]) continue;      // scalar
             const int col0 = uchunk[t] * 256;
+            if constexpr (XQ) {
+#pragma unroll
+                for (int q = 0; q < XLQ; ++q) {
+                    const int row = xrow0 + 4 * q;
+                    if (row < MR) *reinterpret_cast<u32x4*>(slab + row * kChainSlabPitch + xcol) = xq8[t][q];
+                }
+            } else {
 #pragma unroll
             for (int q = 0; q < XL; ++q) {
                 const int row = xrow0 + RPL * q;
@@ -279,6 +311,7 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_chain_chunk_kernel(
                     *reinterpret_cast<uint32_t*>(slab + row * kChainSlabPitch + xcol) = d[0];
                     if (pub) *reinterpret_cast<uint32_t*>(io.xq_out + static_cast<size_t>(row) * K + col0 + xcol) = d[0];
                 }
+            }
             }
             const uint8_t* src = slab + (i < MR ? i : MR) * kChainSlabPitch + g * 64;
             u32x4 bq[4];
@@ -306,12 +339,12 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_chain_chunk_kernel(
     for (int p = 0; p < NACC; ++p)
 #pragma unroll
         for (int b = 0; b < UB; ++b) *reinterpret_cast<i32x4*>(&red[wave][UB * p + b][i * 16 + 4 * g]) = acc[p][b];
-    if (finisher) asm volatile("" : "+v"(ew), "+v"(ew3), "+v"(eres), "+v"(enw));
+    if (finisher) asm volatile("" : "+v"(ew), "+v"(ew3), "+v"(eres), "+v"(enw), "+v"(es));
     __syncthreads();
     if (finisher) {
         const bool row_ok = fin_m < M;
         EpilogueRegs e;
-        e.s = sval_s[row_ok ? fin_m : 0];
+        e.s = XQ ? __uint_as_float(es << 16) : sval_s[row_ok ? fin_m : 0];
         if constexpr (EPI == CEPI_GATE) {
             const int* rp = &red[0][2 * fin_p][64 * fin_q + lane];
             int sum1 = rp[0], sum3 = rp[256];

@@ -206,13 +206,16 @@ class Block:
             self.w13_interleaved = interleave_gate_up(self.w13.packed, self.w13.n, self.w13.k)
         return self.w13_interleaved
 
-    def forward_chain(self, x, stats, cache_k, cache_v, pos_idx, cos, sin, attn_ws, next_norm):
+    def forward_chain(self, x, stats, cache_k, cache_v, pos_idx, cos, sin, attn_ws, next_norm, split=False):
         """One new token per sequence (up to 8 sequences), the linears chained through producer-side norm statistics:
         `x` is the residual stream INCLUDING the previous block's FFN output and `stats` its partials under this block's
         attention_norm (None: the first block, which takes them inside).  Every linear's epilogue leaves what the next
         launch needs: the O projection adds the stream and leaves the ffn_norm partials, gate+up leaves
         relu(x1)^2 * x3 with the ffn_sub_norm partials, the down projection adds the stream again and leaves the
-        partials under `next_norm` (the next block's attention_norm).  Returns (stream, partials)."""
+        partials under `next_norm` (the next block's attention_norm).  Returns (stream, partials).
+        `split`: the producers are the same, but the norm + quantisation in front of QKV, gate+up and the down projection
+        is a launch of its own from the partials (quant_from_stats: element-wise, no reduction over the row) and the
+        linears take the quantised rows -- for row counts at which every workgroup repeating that work costs more."""
         a = self.args
         bsz = cache_k.shape[0]
         lib = self.wqkv.lib
@@ -225,7 +228,12 @@ class Block:
             if pub:
                 cap.append((name, r[3], r[4], r[2] if r[2] is not None else r[0]))
 
-        if stats is None and not pub:
+        if split:
+            xq, s = quant_from_stats(x, stats, self.attention_norm, a.norm_eps) if stats is not None else rmsnorm_quant(x, self.attention_norm, a.norm_eps)[:2]
+            qkv = self.wqkv.quantised(xq, s)
+            if pub:
+                cap.append(("wqkv", xq, s, qkv))
+        elif stats is None and not pub:
             qkv, _ = rmsnorm_linear_packed(x, self.attention_norm, a.norm_eps, self.wqkv.packed, self.wqkv.ws, self.wqkv.ws_num, self.wqkv.n)
         else:
             if stats is None:                       # (recording: the first block's statistics as a launch of their own)
@@ -266,11 +274,17 @@ class Block:
             r = fused_linear(o, self.attn_sub_norm, a.norm_eps, self.wo.packed, self.wo.ws, self.wo.ws_num, self.wo.n, self.wo.k, **o_kw)
         note("wo", r)
         h, h_stats = r[0], r[1]
-        r = fused_linear(h, self.ffn_norm, a.norm_eps, self.gate_up_interleaved(), self.w13.ws, self.w13.ws_num, self.w13.n, self.w13.k,
-                         stats=h_stats, epilogue=EPILOGUE_GATE, next_norm_weight=self.ffn_sub_norm, publish=pub)
+        if split:
+            xq, s = quant_from_stats(h, h_stats, self.ffn_norm, a.norm_eps)
+            r = fused_linear(xq, None, a.norm_eps, self.gate_up_interleaved(), self.w13.ws, self.w13.ws_num, self.w13.n, self.w13.k,
+                             quantised=s, epilogue=EPILOGUE_GATE, next_norm_weight=self.ffn_sub_norm)
+            r = (r[0], r[1], None, xq, s)
+        else:
+            r = fused_linear(h, self.ffn_norm, a.norm_eps, self.gate_up_interleaved(), self.w13.ws, self.w13.ws_num, self.w13.n, self.w13.k,
+                             stats=h_stats, epilogue=EPILOGUE_GATE, next_norm_weight=self.ffn_sub_norm, publish=pub)
         note("w13", r)
         inner, inner_stats = r[0], r[1]
-        if bsz > self.chain_down_rows:
+        if split or bsz > self.chain_down_rows:
             # K = 6912: from five rows on every workgroup repeating the norm + quantisation of the whole block costs more than
             # one launch that does it once (measured at 8 rows: 10.7 us in one launch, 2.7 + 5.3 us in two)
             xq, s = quant_from_stats(inner, inner_stats, self.ffn_sub_norm, a.norm_eps)
@@ -378,6 +392,10 @@ class Transformer:
     # partials; from five rows on a norm + quantisation launch of its own and the plain small-M kernel are faster
     # (measured at 6 and 8 rows).
     chain_rows = 4
+    # Above that, up to this many sequences, the producing epilogues stay (residual add, gate, partial statistics) and a
+    # small element-wise launch forms the quantised rows from the partials (Block.forward_chain, split): lighter than the
+    # norm kernels, which reduce over the row twice, and the gate+up launch writes F columns instead of 2F.
+    split_rows = 8
 
     def __init__(self, args: ModelArgs, seed: int = 0, act: str = "int8", p_zero: float = 0.40):
         gen = torch.Generator(device="cuda").manual_seed(seed)
@@ -533,13 +551,13 @@ class Transformer:
         if one_launch_attention and self.layers[0].act == "int8" and (bsz == 1 or max_seq > 1024):
             attn_ws = self.attention_partial(bsz, max_seq) or attn_ws
         # one new token for a few sequences: the linears chained through producer-side norm statistics (forward_chain)
-        chain = one_launch_attention and self.layers[0].act == "int8" and bsz <= self.chain_rows and getattr(self, "chain", True) and self.chain_supported()
+        chain = one_launch_attention and self.layers[0].act == "int8" and bsz <= max(self.chain_rows, self.split_rows) and getattr(self, "chain", True) and self.chain_supported()
         stats = None
         for index, (layer, (ck, cv)) in enumerate(zip(self.layers, cache)):
             x_in, pending_in = x, pending
             if chain:
                 nxt = self.layers[index + 1].attention_norm if index + 1 < len(self.layers) else self.norm
-                x, stats = layer.forward_chain(x, stats, ck, cv, pos_idx, cos, sin, attn_ws, nxt)
+                x, stats = layer.forward_chain(x, stats, ck, cv, pos_idx, cos, sin, attn_ws, nxt, split=bsz > self.chain_rows)
             else:
                 x, pending = layer.forward(x, pending, ck, cv, pos_idx, cos, sin, mask, attn_ws)
             if trace is not None:

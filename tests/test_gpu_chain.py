@@ -150,6 +150,12 @@ def test_gate_epilogue_on_interleaved_gate_up(m, f, k):
     want = O.relu2_mul(x13)
     assert inner.shape == (m, f) and (_bits(inner) == want).all()
     _check_stats(st_out.cpu().numpy(), want, nxt, 16)
+    # the same launch fed with activations that are quantised already: the same bits
+    print(f"[case] chain gate+up, quantised activations: m={m} f={f} k={k}", flush=True)
+    r = L.fused_linear(xq, None, 1e-5, inter, _bf(WS), 2, n, k, quantised=s, epilogue=L.EPILOGUE_GATE, next_norm_weight=_bf(nxt))
+    assert r is not None
+    torch.cuda.synchronize()
+    assert torch.equal(r[0], inner) and torch.equal(r[1], st_out)
 
 
 def test_norm_and_attention_prologues_with_the_residual_epilogue():
@@ -240,4 +246,9 @@ def test_unsupported_combinations_are_declined():
     assert L.fused_linear(h, g, 1e-5, packed, _bf(WS), 1, n, k) is None                                    # NORM + STORE: the older entry point
     assert L.fused_linear(h, g, 1e-5, packed, _bf(WS), 1, n, k, stats=L.row_stats(h, g), epilogue=L.EPILOGUE_GATE,
                           next_norm_weight=_bf(_weight(n // 2, 1253))) is None                              # GATE needs two scale groups
+    xq9 = torch.zeros((9, k), dtype=torch.int8, device="cuda")
+    s9 = torch.ones(9, dtype=torch.bfloat16, device="cuda")
+    assert L.fused_linear(xq9, None, 1e-5, packed, _bf(WS), 2, n, k, quantised=s9, epilogue=L.EPILOGUE_GATE,
+                          next_norm_weight=_bf(_weight(n // 2, 1254))) is None                              # GATE on quantised rows: up to 8
+    assert L.fused_linear(xq9, None, 1e-5, packed, _bf(WS), 1, n, k, quantised=s9) is None                 # QUANTISED + STORE: bitlinear_TernaSpMM_packed
     torch.cuda.synchronize()
