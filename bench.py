@@ -245,6 +245,10 @@ def measure_model(torch, batch, act="int8", prefetch=True, gen_tokens=256, check
         model.chain_rows = int(os.environ["TERNA_BENCH_CHAIN_ROWS"])
     if os.environ.get("TERNA_BENCH_SPLIT_ROWS"):
         model.split_rows = int(os.environ["TERNA_BENCH_SPLIT_ROWS"])
+    if os.environ.get("TERNA_BENCH_ATTN_SPLITS"):
+        model.attention_splits = int(os.environ["TERNA_BENCH_ATTN_SPLITS"])
+    if os.environ.get("TERNA_BENCH_SPLIT_MERGE_QUANT"):
+        model.split_merge_quant = os.environ["TERNA_BENCH_SPLIT_MERGE_QUANT"] != "0"
     if os.environ.get("TERNA_BENCH_CHAIN_DOWN_ROWS"):
         for blk in model.layers:
             blk.chain_down_rows = int(os.environ["TERNA_BENCH_CHAIN_DOWN_ROWS"])

@@ -425,6 +425,14 @@ void ternaspmm_rope_decode_attention_partial(const terna_bf16* qkv, const float*
                                              const void* const* pf_ptr, const long long* pf_bytes, const long long* pf_unit_bytes,
                                              int pf_count, terna_stream stream);
 void ternaspmm_attention_merge(const float* partial, int splits, terna_bf16* out, int B, int H, int D, terna_stream stream);
+/* ternaspmm_attention_merge and the ternaspmm_rmsnorm_quant behind it (model.py:236 attn_sub_norm, :120-123 quant_input
+ * of the O projection) in one launch, one workgroup per sequence: (xq_out int8 [B][H*D], s_out bf16 [B]) are the bits of
+ * that pair; o_out (optional, bf16 [B][H*D]) receives the merged attention output.  For a step of several sequences,
+ * whose O projection then takes the quantised rows (ternaspmm_fused_linear, TERNASPMM_PROLOGUE_QUANTISED) instead of
+ * repeating merge, norm and quantisation in every workgroup.  H * D <= 4096, D = 64 or 128, splits 1, 2, 4 or 8;
+ * returns 0, or -1 for anything else (nothing enqueued). */
+int ternaspmm_attention_merge_rmsnorm_quant(const float* partial, int splits, const terna_bf16* norm_weight, float eps, terna_bf16* o_out,
+                                            int8_t* xq_out, terna_bf16* s_out, int B, int H, int D, terna_stream stream);
 
 /* The bookkeeping of one greedy decode step in one launch (generate.py:283-305: argmax, tokens[:, pos] = next_token,
  * the position counters): tok[b] = argmax(logits[b]) as above; if history != NULL and counters[1] < history_len,

@@ -381,4 +381,38 @@ void ternaspmm_attention_merge(const float* partial, int splits, terna_bf16* out
     if (e != hipSuccess) die("ternaspmm_attention_merge", e, __LINE__);
 }
 
+int ternaspmm_attention_merge_rmsnorm_quant(const float* partial, int splits, const terna_bf16* norm_weight, float eps, terna_bf16* o_out,
+                                            int8_t* xq_out, terna_bf16* s_out, int B, int H, int D, terna_stream stream)
+{
+    const long long K = static_cast<long long>(H) * D;
+    if (B < 1 || H < 1 || (D != 64 && D != 128) || (splits != 1 && splits != 2 && splits != 4 && splits != 8) || K > 2048 * 2 ||
+        partial == nullptr || norm_weight == nullptr || xq_out == nullptr || s_out == nullptr)
+        return -1;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int qmode = quant_mode();
+#define TERNA_MERGE_NQ(DIM, SP)                                                                                           \
+    do {                                                                                                                  \
+        if (K <= 2048)                                                                                                    \
+            terna_attention_merge_norm_quant_kernel<DIM, SP, 1><<<dim3(B), dim3(kNormThreads), 0, st>>>(                   \
+                partial, norm_weight, H, B * H, eps, o_out, nullptr, xq_out, s_out, qmode);                               \
+        else                                                                                                              \
+            terna_attention_merge_norm_quant_kernel<DIM, SP, 2><<<dim3(B), dim3(kNormThreads), 0, st>>>(                   \
+                partial, norm_weight, H, B * H, eps, o_out, nullptr, xq_out, s_out, qmode);                               \
+    } while (0)
+#define TERNA_MERGE_NQ_D(DIM)                                                                                             \
+    do {                                                                                                                  \
+        if (splits == 1) TERNA_MERGE_NQ(DIM, 1);                                                                          \
+        else if (splits == 2) TERNA_MERGE_NQ(DIM, 2);                                                                     \
+        else if (splits == 4) TERNA_MERGE_NQ(DIM, 4);                                                                     \
+        else TERNA_MERGE_NQ(DIM, 8);                                                                                      \
+    } while (0)
+    if (D == 128) TERNA_MERGE_NQ_D(128);
+    else TERNA_MERGE_NQ_D(64);
+#undef TERNA_MERGE_NQ_D
+#undef TERNA_MERGE_NQ
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_attention_merge_rmsnorm_quant", e, __LINE__);
+    return 0;
+}
+
 }  // extern "C"

@@ -168,6 +168,83 @@ __global__ __launch_bounds__(D) void terna_attention_merge_kernel(const float* _
     const float* o_head = partial + attention_stat_floats(heads) + static_cast<size_t>(bh) * SP * D;
     out[static_cast<size_t>(bh) * D + threadIdx.x] = float_to_bf16_bits(attention_merge(stat, o_head, SP, D, threadIdx.x));
 }
+// terna_attention_merge_kernel and the norm kernel behind it (norm_quant_kernel.h) as one launch: one workgroup per
+// sequence forms its merged row -- H * D columns, rounded to bf16: the bits the merge kernel stores -- in registers and
+// runs the norm kernel's passes on it.  Everything a thread reads (its heads' statistics, SP partial results of eight
+// columns per vector, the norm weights) is requested before the first use.  o_out (optional): the merged row.
+template <int D, int SP, int NV>
+__global__ __launch_bounds__(kNormThreads) void terna_attention_merge_norm_quant_kernel(
+    const float* __restrict__ partial, const uint16_t* __restrict__ weight, int H, int heads_total, float eps,
+    uint16_t* __restrict__ o_out, uint16_t* __restrict__ y_out, int8_t* __restrict__ xq_out, uint16_t* __restrict__ s_out, int quant_mode)
+{
+    static_assert(D % 8 == 0 && SP >= 1 && SP <= kAttentionMaxSplits && kAttentionMaxSplits == 8, "a vector lies inside one head");
+    const int tid = threadIdx.x;
+    const size_t row = blockIdx.x;
+    const int K = H * D, nvec = K >> 3;
+    u32x4 raw_w[NV];
+    f32x4 st[NV][4], po[NV][SP][2];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int v = tid + i * kNormThreads;
+        const int vc = v < nvec ? v : nvec - 1;
+        const int head = (8 * vc) / D, d = (8 * vc) % D;
+        const size_t bh = row * H + head;
+        raw_w[i] = *reinterpret_cast<const u32x4*>(weight + 8 * vc);
+        const f32x4* sp = reinterpret_cast<const f32x4*>(partial + bh * kAttentionStatFloats);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) st[i][q] = sp[q];
+        const float* op = partial + attention_stat_floats(static_cast<size_t>(heads_total)) + bh * SP * D + d;
+#pragma unroll
+        for (int j = 0; j < SP; ++j) {
+            po[i][j][0] = *reinterpret_cast<const f32x4*>(op + j * D);
+            po[i][j][1] = *reinterpret_cast<const f32x4*>(op + j * D + 4);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        pin_registers(raw_w[i]);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) pin_registers(st[i][q]);
+#pragma unroll
+        for (int j = 0; j < SP; ++j) {
+            pin_registers(po[i][j][0]);
+            pin_registers(po[i][j][1]);
+        }
+    }
+    float h[NV][8];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int v = tid + i * kNormThreads;
+        if (v < nvec) {
+            // attention_merge's arithmetic on the values in registers
+            float mx[SP], dn[SP];
+#pragma unroll
+            for (int j = 0; j < SP; ++j) {
+                mx[j] = st[i][j >> 2][j & 3];
+                dn[j] = st[i][2 + (j >> 2)][j & 3];
+            }
+            float m_all = -INFINITY;
+#pragma unroll
+            for (int j = 0; j < SP; ++j) m_all = fmaxf(m_all, mx[j]);
+            float wj[SP], den = 0.0f;
+#pragma unroll
+            for (int j = 0; j < SP; ++j) {
+                wj[j] = __expf(mx[j] - m_all);
+                den = fmaf(wj[j], dn[j], den);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float num = 0.0f;
+#pragma unroll
+                for (int j = 0; j < SP; ++j) num = fmaf(wj[j], po[i][j][e >> 2][e & 3], num);
+                h[i][e] = round_bf16(num / den);
+            }
+            if (o_out != nullptr) *reinterpret_cast<u32x4*>(o_out + row * K + 8 * v) = pack_bf16x8(h[i]);
+        }
+    }
+    norm_quant_passes<NV>(h, raw_w, K, eps, row, y_out, xq_out, s_out, quant_mode);
+}
+
 // Extra workgroups of the attention launch (blockIdx.x >= heads) that pull up to kAttentionPrefetchRegions regions of
 // device memory through the caches while the heads' workgroups -- one CU each -- do the attention:
 // the weights of the launches that follow.  Unit u of a region goes to a workgroup on XCD (u mod 8),

@@ -95,68 +95,23 @@ __device__ __forceinline__ u32x4 pack_bf16x8(const float f[8])
 }
 __device__ __forceinline__ float round_bf16(float v) { return bf16_bits_to_float(float_to_bf16_bits(v)); }
 
-// GLU = false: x [M][K], optional residual [M][K] and sum_out [M][K].
-// GLU = true : x [M][2K] holding x1 | x3; residual / sum_out unused.
-// NV = 8-element vectors per thread (K <= 2048 NV); SECOND = there is a second operand (the residual, or x3).
-template <bool GLU, int NV = kNormMaxVecs, bool SECOND = true>
-__global__ __launch_bounds__(kNormThreads) void terna_norm_quant_kernel(
-    const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, const uint16_t* __restrict__ weight, int K,
-    float eps, uint16_t* __restrict__ sum_out, uint16_t* __restrict__ y_out, int8_t* __restrict__ xq_out,
-    uint16_t* __restrict__ s_out, int quant_mode)
+// The passes behind the formation of a row, for every kernel that holds one in registers (h[i][j] = element
+// 8 (tid + kNormThreads i) + j, vectors past K / 8 unused; raw_w the norm weights of the same elements): sum of squares
+// -- per thread in element order, the lanes of a wave by group_reduce, the four waves pairwise -- then the norm, the row
+// maximum, the scale and the int8 values.  y_out / xq_out + s_out: optional outputs.
+template <int NV>
+__device__ __forceinline__ void norm_quant_passes(float (&h)[NV][8], const u32x4 (&raw_w)[NV], int K, float eps, size_t row,
+                                                  uint16_t* __restrict__ y_out, int8_t* __restrict__ xq_out,
+                                                  uint16_t* __restrict__ s_out, int quant_mode)
 {
-    static_assert(!GLU || SECOND, "the gate has two operands");
     __shared__ float red[2][kNormThreads / 64];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const size_t row = blockIdx.x;
     const int nvec = K >> 3;
-    const uint16_t* xr = x + row * static_cast<size_t>(GLU ? 2 * K : K);
-
-    // Every global load of the row -- input, second operand, norm weight -- is issued before the
-    // first use: with one row per workgroup the kernel's time is its chain of memory round trips, and the address
-    // unit takes a wave's load in a dozen cycles whatever it fetches: no more loads than the row needs.
-    // The loads are unconditional on clamped addresses (a load inside a branch is waited for at
-    // the join, which would serialise them).
-    u32x4 raw_x[NV], raw_b[NV], raw_w[NV];
-    const uint16_t* br = GLU ? xr + K : (SECOND ? residual + row * K : xr);
-#pragma unroll
-    for (int i = 0; i < NV; ++i) {
-        const int v = tid + i * kNormThreads;
-        const int vc = v < nvec ? v : nvec - 1;
-        raw_x[i] = *reinterpret_cast<const u32x4*>(xr + 8 * vc);
-        if constexpr (SECOND) raw_b[i] = *reinterpret_cast<const u32x4*>(br + 8 * vc);
-        raw_w[i] = *reinterpret_cast<const u32x4*>(weight + 8 * vc);
-    }
-    // pin the loads here: otherwise they are sunk into the branches below, next to their uses
-#pragma unroll
-    for (int i = 0; i < NV; ++i) {
-        pin_registers(raw_x[i]);
-        if constexpr (SECOND) pin_registers(raw_b[i]);
-        pin_registers(raw_w[i]);
-    }
-
-    float h[NV][8];
     float ssq = 0.0f;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-        const int v = tid + i * kNormThreads;
-        if (v < nvec) {
-            unpack_bf16x8(raw_x[i], h[i]);
-            if constexpr (GLU) {
-                float g[8];
-                unpack_bf16x8(raw_b[i], g);
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const float r = fmaxf(h[i][j], 0.0f);
-                    h[i][j] = round_bf16(round_bf16(r * r) * g[j]);
-                }
-            } else if constexpr (SECOND) {
-                float r[8];
-                unpack_bf16x8(raw_b[i], r);
-#pragma unroll
-                for (int j = 0; j < 8; ++j) h[i][j] = round_bf16(h[i][j] + r[j]);
-                if (sum_out != nullptr) *reinterpret_cast<u32x4*>(sum_out + row * K + 8 * v) = pack_bf16x8(h[i]);
-            }
+        if (tid + i * kNormThreads < nvec) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) ssq = fmaf(h[i][j], h[i][j], ssq);
         }
@@ -204,6 +159,70 @@ __global__ __launch_bounds__(kNormThreads) void terna_norm_quant_kernel(
             *reinterpret_cast<u32x2*>(xq_out + row * K + 8 * v) = u32x2{q[0], q[1]};
         }
     }
+}
+
+// GLU = false: x [M][K], optional residual [M][K] and sum_out [M][K].
+// GLU = true : x [M][2K] holding x1 | x3; residual / sum_out unused.
+// NV = 8-element vectors per thread (K <= 2048 NV); SECOND = there is a second operand (the residual, or x3).
+template <bool GLU, int NV = kNormMaxVecs, bool SECOND = true>
+__global__ __launch_bounds__(kNormThreads) void terna_norm_quant_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, const uint16_t* __restrict__ weight, int K,
+    float eps, uint16_t* __restrict__ sum_out, uint16_t* __restrict__ y_out, int8_t* __restrict__ xq_out,
+    uint16_t* __restrict__ s_out, int quant_mode)
+{
+    static_assert(!GLU || SECOND, "the gate has two operands");
+    const int tid = threadIdx.x;
+    const size_t row = blockIdx.x;
+    const int nvec = K >> 3;
+    const uint16_t* xr = x + row * static_cast<size_t>(GLU ? 2 * K : K);
+
+    // Every global load of the row -- input, second operand, norm weight -- is issued before the
+    // first use: with one row per workgroup the kernel's time is its chain of memory round trips, and the address
+    // unit takes a wave's load in a dozen cycles whatever it fetches: no more loads than the row needs.
+    // The loads are unconditional on clamped addresses (a load inside a branch is waited for at
+    // the join, which would serialise them).
+    u32x4 raw_x[NV], raw_b[NV], raw_w[NV];
+    const uint16_t* br = GLU ? xr + K : (SECOND ? residual + row * K : xr);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int v = tid + i * kNormThreads;
+        const int vc = v < nvec ? v : nvec - 1;
+        raw_x[i] = *reinterpret_cast<const u32x4*>(xr + 8 * vc);
+        if constexpr (SECOND) raw_b[i] = *reinterpret_cast<const u32x4*>(br + 8 * vc);
+        raw_w[i] = *reinterpret_cast<const u32x4*>(weight + 8 * vc);
+    }
+    // pin the loads here: otherwise they are sunk into the branches below, next to their uses
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        pin_registers(raw_x[i]);
+        if constexpr (SECOND) pin_registers(raw_b[i]);
+        pin_registers(raw_w[i]);
+    }
+
+    float h[NV][8];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int v = tid + i * kNormThreads;
+        if (v < nvec) {
+            unpack_bf16x8(raw_x[i], h[i]);
+            if constexpr (GLU) {
+                float g[8];
+                unpack_bf16x8(raw_b[i], g);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float r = fmaxf(h[i][j], 0.0f);
+                    h[i][j] = round_bf16(round_bf16(r * r) * g[j]);
+                }
+            } else if constexpr (SECOND) {
+                float r[8];
+                unpack_bf16x8(raw_b[i], r);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) h[i][j] = round_bf16(h[i][j] + r[j]);
+                if (sum_out != nullptr) *reinterpret_cast<u32x4*>(sum_out + row * K + 8 * v) = pack_bf16x8(h[i]);
+            }
+        }
+    }
+    norm_quant_passes<NV>(h, raw_w, K, eps, row, y_out, xq_out, s_out, quant_mode);
 }
 
 }  // namespace terna

@@ -156,6 +156,7 @@ __device__ __forceinline__ void pin_registers(u32x4& v)
 }
 
 __device__ __forceinline__ void pin_registers(u32x2& v) { asm volatile("" : "+v"(v.x), "+v"(v.y)); }
+__device__ __forceinline__ void pin_registers(f32x4& v) { asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w)); }
 __device__ __forceinline__ void pin_registers(float2& v) { asm volatile("" : "+v"(v.x), "+v"(v.y)); }
 
 // max / sum over the four lanes L, L ^ 16, L ^ 32, L ^ 48 with the row-swap permutations of the VALU (gfx950):

@@ -217,6 +217,27 @@ def attention_merge_rmsnorm_linear_packed(partial, splits, heads, head_dim, norm
     return rmsnorm_linear_packed(o, norm_weight, eps, packed, ws, ws_num, out_features)[0]
 
 
+def attention_merge_rmsnorm_quant(partial, splits, heads, head_dim, norm_weight, eps, sequences, want_output=False):
+    """ternaspmm_attention_merge + rmsnorm_quant in one launch (one workgroup per sequence): the quantised input of the O
+    projection from the partial results of a split attention launch.  Returns (xq int8 [sequences, heads * head_dim],
+    s bf16 [sequences], o) -- o the merged attention output with `want_output`, else None -- or None where the library
+    does not take the shape (nothing enqueued)."""
+    lib = _lib.load()
+    k = heads * head_dim
+    need = lib.ternaspmm_attention_partial_bytes(sequences, heads, head_dim)
+    if sequences < 1 or need < 0 or partial.numel() * partial.element_size() < need:
+        raise ValueError(f"partial buffer of {partial.numel() * partial.element_size()} bytes does not hold {sequences} sequences")
+    if norm_weight.numel() != k or norm_weight.dtype != torch.bfloat16:
+        raise ValueError("attention_merge_rmsnorm_quant: the norm weight is a bf16 vector of heads * head_dim elements")
+    dev = partial.device
+    xq = torch.empty((sequences, k), dtype=torch.int8, device=dev)
+    s = torch.empty(sequences, dtype=torch.bfloat16, device=dev)
+    o = torch.empty((sequences, k), dtype=torch.bfloat16, device=dev) if want_output else None
+    rc = lib.ternaspmm_attention_merge_rmsnorm_quant(_p(partial), splits, _p(norm_weight), float(eps), _p(o) if o is not None else None, _p(xq), _p(s), sequences, heads,
+                                                     head_dim, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    return None if rc != 0 else (xq, s, o)
+
+
 def relu2_mul_rmsnorm_linear_packed(x13, norm_weight, eps, packed, ws, ws_num, out_features):
     """squared_relu(x1) * x3 -> RMSNorm -> quant_input -> int8 TernaSpMM on a P2 weight: one launch for up to four
     rows where the library supports the shape, else relu2_mul_rmsnorm_quant + TernaInfer_linear_packed.

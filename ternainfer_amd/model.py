@@ -22,7 +22,7 @@ import torch
 from torch.nn import functional as F
 
 from . import _lib
-from .linear import (EPILOGUE_GATE, EPILOGUE_RESIDUAL, argmax_rows, attention_merge_rmsnorm_linear_packed, fused_linear, get_global_workspace, greedy_step,
+from .linear import (EPILOGUE_GATE, EPILOGUE_RESIDUAL, argmax_rows, attention_merge_rmsnorm_linear_packed, attention_merge_rmsnorm_quant, fused_linear, get_global_workspace, greedy_step,
                      greedy_step_state, interleave_gate_up, lm_head, quant_from_stats, quant_input, row_stats, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant,
                      repack_weight, rmsnorm_linear_packed, rmsnorm_quant)
 
@@ -246,11 +246,22 @@ class Block:
         o_kw = dict(epilogue=EPILOGUE_RESIDUAL, residual=x, next_norm_weight=self.ffn_norm, want_raw=pub, publish=pub)
         if deferred:
             partial, splits = attn_ws
+            pf = self.prefetch if split and self.prefetch is not None else (None, None, None, 0)
             lib.ternaspmm_rope_decode_attention_partial(
                 _p(qkv), _p(cos), _p(sin), _p(pos_idx), per_seq, _p(cache_k), _p(cache_v), _p(partial), splits, bsz, a.n_heads,
-                a.n_kv_heads, a.head_dim, cache_k.shape[2], a.head_dim ** -0.5, int(a.rope_adjacent), None, None, None, 0, stream)
+                a.n_kv_heads, a.head_dim, cache_k.shape[2], a.head_dim ** -0.5, int(a.rope_adjacent), *pf, stream)
             r = None
-            if bsz == 1:
+            if split:
+                # merge + sub-norm + quantisation once per sequence, then the O projection on the quantised rows
+                mq = attention_merge_rmsnorm_quant(partial, splits, a.n_heads, a.head_dim, self.attn_sub_norm, a.norm_eps, bsz, want_output=pub)
+                if mq is not None:
+                    if pub:
+                        cap.append(("attention", None, None, mq[2]))
+                    r = fused_linear(mq[0], None, a.norm_eps, self.wo.packed, self.wo.ws, self.wo.ws_num, self.wo.n, self.wo.k, quantised=mq[1],
+                                     epilogue=EPILOGUE_RESIDUAL, residual=x, next_norm_weight=self.ffn_norm, want_raw=pub)
+                    if r is not None:
+                        r = (r[0], r[1], r[2], mq[0], mq[1])
+            elif bsz == 1:
                 r = fused_linear(partial, self.attn_sub_norm, a.norm_eps, self.wo.packed, self.wo.ws, self.wo.ws_num, self.wo.n, self.wo.k,
                                  attention=(splits, a.head_dim), **o_kw)
             if r is None:
@@ -486,16 +497,16 @@ class Transformer:
             self._rope_tables = tables = (key, torch.stack([ang.cos(), ang.sin()], dim=1).contiguous())
         return tables[1]
 
-    def attention_partial(self, bsz: int, max_seq: int):
+    def attention_partial(self, bsz: int, max_seq: int, single_split: bool = False):
         """(buffer, splits) for the decode step whose attention leaves the merge of its splits to the consumer of its
         output (one sequence: the O projection's prologue; more: a merge launch), or None when that form does not apply
-        (one split recommended; `deferred_attention_merge` False)."""
+        (one split recommended and not `single_split`; `deferred_attention_merge` False)."""
         if not getattr(self, "deferred_attention_merge", True):
             return None
         a = self.args
         lib = _lib.load()
         splits = getattr(self, "attention_splits", None) or lib.ternaspmm_attention_partial_splits(bsz, a.n_heads, max_seq)
-        if splits <= 1:
+        if splits < 1 or (splits == 1 and not single_split):
             return None
         # one buffer per batch size, kept while the model lives: a captured decode graph holds the raw pointer
         held = self.__dict__.setdefault("_attn_partial", {})
@@ -545,19 +556,25 @@ class Transformer:
         x = self.tok_embeddings[tokens.reshape(-1)]
         pending = None
         attn_ws = self.attention_workspace(bsz) if one_launch_attention else None     # layers run one after another: shared
-        # split attention whose merge is left to its consumer: always for one sequence (the O projection's prologue merges);
-        # for more only with long caches, where the shorter attention launch pays for the merge launch (8 sequences at slot
-        # 1500: 1943 -> 1713 us per step; at slot 255 of 384 the pair of launches is 1.5 us slower than the unsplit one)
-        if one_launch_attention and self.layers[0].act == "int8" and (bsz == 1 or max_seq > 1024):
-            attn_ws = self.attention_partial(bsz, max_seq) or attn_ws
         # one new token for a few sequences: the linears chained through producer-side norm statistics (forward_chain)
         chain = one_launch_attention and self.layers[0].act == "int8" and bsz <= max(self.chain_rows, self.split_rows) and getattr(self, "chain", True) and self.chain_supported()
+        split = chain and bsz > self.chain_rows
+        # split attention whose merge is left to its consumer: always for one sequence (the O projection's prologue merges);
+        # for more only with long caches, where the shorter attention launch pays for the merge launch (8 sequences at slot
+        # 1500: 1943 -> 1713 us per step; at slot 255 of 384 the pair of launches is 1.5 us slower than the unsplit one) --
+        # (in the split chain that merge launch also norms and quantises the O projection's input; with short caches
+        # the unsplit launch + the O projection with the norm inside stay ahead there too: 8 sequences, slot 255 of 384,
+        # 1.198 against 1.218 ms per step -- `split_merge_quant` forces the split form)
+        if one_launch_attention and self.layers[0].act == "int8" and (bsz == 1 or max_seq > 1024):
+            attn_ws = self.attention_partial(bsz, max_seq) or attn_ws
+        elif split and getattr(self, "split_merge_quant", False):
+            attn_ws = self.attention_partial(bsz, max_seq, single_split=True) or attn_ws
         stats = None
         for index, (layer, (ck, cv)) in enumerate(zip(self.layers, cache)):
             x_in, pending_in = x, pending
             if chain:
                 nxt = self.layers[index + 1].attention_norm if index + 1 < len(self.layers) else self.norm
-                x, stats = layer.forward_chain(x, stats, ck, cv, pos_idx, cos, sin, attn_ws, nxt, split=bsz > self.chain_rows)
+                x, stats = layer.forward_chain(x, stats, ck, cv, pos_idx, cos, sin, attn_ws, nxt, split=split)
             else:
                 x, pending = layer.forward(x, pending, ck, cv, pos_idx, cos, sin, mask, attn_ws)
             if trace is not None:

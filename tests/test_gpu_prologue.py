@@ -871,3 +871,39 @@ def test_fused_attention_merge_projection(lib, h, kv, d, n_out, s_max, n, splits
     # outside its range: two rows
     assert lib.bitlinear_TernaSpMM_packed_fused_attn(_vp(part), splits, d, _vp(norm_w), 1e-5, _vp(packed), _vp(out2), _vp(ws), 1,
                                                      None, None, 2, n_out, k_in, None) == 0
+
+
+@pytest.mark.parametrize("splits", [1, 2, 4, 8])
+@pytest.mark.parametrize("b,h,kv,d,s_max,lens", [(8, 20, 5, 128, 384, (300, 1, 129, 384, 77, 256, 200, 33)), (3, 4, 2, 64, 64, (5, 64, 17)),
+                                                 (2, 16, 8, 128, 1024, (1000, 600))])
+def test_attention_merge_rmsnorm_quant(lib, b, h, kv, d, s_max, lens, splits):
+    """ternaspmm_attention_merge_rmsnorm_quant (merge of the splits + sub-norm + quantisation, one launch) against
+    ternaspmm_attention_merge followed by ternaspmm_rmsnorm_quant: merged row, int8 values and scales bit-identical."""
+    k_in = h * d
+    qkv = make_bf16_activations(b, (h + 2 * kv) * d, 2100 + b)
+    k0 = make_bf16_activations(b * kv * s_max, d, 2101 + b).reshape(b, kv, s_max, d)
+    v0 = make_bf16_activations(b * kv * s_max, d, 2102 + b, outlier_frac=0.01).reshape(b, kv, s_max, d)
+    pos = np.array(lens, np.int64).reshape(b, 1) - 1
+    cos, sin = _angles(pos.reshape(-1), d)
+    xd, cd, sd, pd, ck, cv = _dev(qkv), _dev(cos), _dev(sin), _dev(pos), _dev(k0), _dev(v0)
+    part = _partial_buffer(lib, b, h, d)
+    lib.ternaspmm_rope_decode_attention_partial(_vp(xd), _vp(cd), _vp(sd), _vp(pd), 1, _vp(ck), _vp(cv), _vp(part), splits,
+                                                b, h, kv, d, s_max, float(d) ** -0.5, 1, None, None, None, 0, None)
+    norm_w = _dev(_weight(k_in, 2103))
+    attn = torch.zeros((b, k_in), dtype=torch.int16, device="cuda")
+    xq1, s1 = torch.zeros((b, k_in), dtype=torch.int8, device="cuda"), torch.zeros(b, dtype=torch.int16, device="cuda")
+    lib.ternaspmm_attention_merge(_vp(part), splits, _vp(attn), b, h, d, None)
+    lib.ternaspmm_rmsnorm_quant(_vp(attn), None, None, _vp(norm_w), 1e-5, None, _vp(xq1), _vp(s1), b, k_in, None)
+    print(f"[case] attention merge + norm + quantise b={b} h={h} d={d} splits={splits}", flush=True)
+    o2 = torch.zeros_like(attn)
+    xq2, s2 = torch.zeros_like(xq1), torch.zeros_like(s1)
+    assert lib.ternaspmm_attention_merge_rmsnorm_quant(_vp(part), splits, _vp(norm_w), 1e-5, _vp(o2), _vp(xq2), _vp(s2), b, h, d, None) == 0
+    xq3, s3 = torch.zeros_like(xq1), torch.zeros_like(s1)
+    assert lib.ternaspmm_attention_merge_rmsnorm_quant(_vp(part), splits, _vp(norm_w), 1e-5, None, _vp(xq3), _vp(s3), b, h, d, None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(o2, attn) and torch.equal(xq2, xq1) and torch.equal(s2, s1)
+    assert torch.equal(xq3, xq1) and torch.equal(s3, s1)
+    assert int(xq2.abs().max().item()) >= 126
+    # outside its range: nothing enqueued
+    assert lib.ternaspmm_attention_merge_rmsnorm_quant(_vp(part), 3, _vp(norm_w), 1e-5, None, _vp(xq3), _vp(s3), b, h, d, None) == -1
+    assert lib.ternaspmm_attention_merge_rmsnorm_quant(_vp(part), splits, _vp(norm_w), 1e-5, None, _vp(xq3), _vp(s3), b, 40, 128, None) == -1
