@@ -416,9 +416,14 @@ void ternaspmm_rope_decode_attention_prefetch(const terna_bf16* qkv, const float
  * inside the O projection's prologue.  The launch boundary takes the place of the arrival counter and of the merging
  * workgroup's dependent reads, which cost the in-launch merge 5 - 6 us whatever the prefix length.
  * ternaspmm_attention_partial_splits(B, H, S): the split count the library recommends (a power of two; 1 when the
- * heads fill the chip anyway).  pf_ptr may be NULL with pf_count = 0. */
+ * heads fill the chip anyway).  pf_ptr may be NULL with pf_count = 0.
+ * Several sequences with 2 or 4 heads per kv head run one workgroup per (sequence, kv head, split): the heads of a kv
+ * group read the same keys and values, which then cross from L2 into a CU once instead of once per head (same bits;
+ * measured, 2B shape, caches of 1656 slots: 8 sequences 1.463 -> 1.351 ms per decode step, 6 sequences 1.405 -> 1.258).
+ * ternaspmm_attention_partial_splits_kv(B, H, KV, S) is the recommendation for that form: it splits from 512 slots on. */
 long long ternaspmm_attention_partial_bytes(int B, int H, int D);
 int ternaspmm_attention_partial_splits(int B, int H, int S);
+int ternaspmm_attention_partial_splits_kv(int B, int H, int KV, int S);   /* the same, knowing the kv heads: see below */
 void ternaspmm_rope_decode_attention_partial(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
                                              int per_sequence, terna_bf16* cache_k, terna_bf16* cache_v, float* partial, int splits,
                                              int B, int H, int KV, int D, int S, float scale, int adjacent,

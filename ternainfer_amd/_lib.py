@@ -55,6 +55,7 @@ PROTOTYPES = {
     "ternaspmm_argmax_bf16": ([_vp, _vp, _ci, _ci, _vp], None),
     "ternaspmm_attention_partial_bytes": ([_ci] * 3, ctypes.c_longlong),
     "ternaspmm_attention_partial_splits": ([_ci] * 3, ctypes.c_int),
+    "ternaspmm_attention_partial_splits_kv": ([_ci] * 4, ctypes.c_int),
     "ternaspmm_rope_decode_attention_partial": ([_vp] * 4 + [_ci] + [_vp] * 3 + [_ci] * 6 + [ctypes.c_float, _ci, _vp, _vp, _vp, _ci, _vp], None),
     "ternaspmm_attention_merge": ([_vp, _ci, _vp, _ci, _ci, _ci, _vp], None),
     "ternaspmm_attention_merge_rmsnorm_quant": ([_vp, _ci, _vp, ctypes.c_float, _vp, _vp, _vp, _ci, _ci, _ci, _vp], ctypes.c_int),

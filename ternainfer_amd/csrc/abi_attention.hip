@@ -11,6 +11,7 @@
 #include "../../include/ternaspmm.h"
 #include "host_util.h"
 #include "attention_kernel.h"
+#include "attention_grouped_kernel.h"
 
 using namespace terna;
 
@@ -119,6 +120,47 @@ void launch_attention_deferred(const uint16_t* qkv, uint16_t* ck, uint16_t* cv, 
     const int slots = grouped ? 8 * (H / KV) * ((B * KV * splits + 7) / 8) : B * H * splits;
     kernel<<<dim3(slots + pf.workgroups), dim3(64 * NW), lds, st>>>(
         qkv, ck, cv, pos, H, KV, S, splits, slots, grouped ? B * KV : 0, per_seq, scale, cos, sin, nullptr, partial, nullptr, pf);
+}
+
+int prefetch_workgroups(const AttentionPrefetch& pf, int slots);
+
+// The deferred-merge launch with one workgroup per (sequence, kv head, split) (attention_grouped_kernel.h).  Returns false
+// where that form does not apply: one head per kv head, a group size other than 2 or 4, a score buffer beyond the LDS.
+template <int D, bool ADJ>
+bool launch_attention_grouped(const uint16_t* qkv, uint16_t* ck, uint16_t* cv, const float* cos, const float* sin, const long long* pos,
+                              int per_seq, float* partial, int splits, int B, int H, int KV, int S, float scale,
+                              const AttentionPrefetch& pf_in, hipStream_t st)
+{
+    static const int waves = [] {
+        // 8 waves: measured ahead of 4 at 2 - 8 sequences with caches of 1656 slots (8 sequences: 1.351 against 1.410 ms
+        // per decode step), level with them at 384 slots
+        const char* v = tuning_env("TERNASPMM_ATTN_GROUPED_WAVES");
+        return v && std::atoi(v) == 4 ? 4 : 8;
+    }();
+    if (KV < 1 || H % KV != 0) return false;
+    const int gq = H / KV;
+    if (gq != 2 && gq != 4) return false;
+    const size_t lds = grouped_attention_lds_bytes(D, waves, gq, S);
+    if (lds > 159 * 1024) return false;          // (160 KB per workgroup, the kernel's static LDS included)
+    AttentionPrefetch pf = pf_in;
+    const int slots = B * KV * splits;
+    pf.workgroups = prefetch_workgroups(pf, slots);
+#define TERNA_GROUPED(NWAVES, GQ)                                                                                          \
+    do {                                                                                                                   \
+        auto kernel = terna_decode_attention_grouped_kernel<D, ADJ, NWAVES, GQ>;                                            \
+        if (lds > 64 * 1024) allow_dynamic_lds(kernel, 159 * 1024, "hipFuncSetAttribute(decode attention, kv groups)", __LINE__); \
+        kernel<<<dim3(slots + pf.workgroups), dim3(64 * NWAVES), lds, st>>>(qkv, ck, cv, pos, KV, S, splits, slots, per_seq, scale, cos, sin, \
+                                                                            partial, pf);                                  \
+    } while (0)
+    if (waves == 8) {
+        if (gq == 4) TERNA_GROUPED(8, 4);
+        else TERNA_GROUPED(8, 2);
+    } else {
+        if (gq == 4) TERNA_GROUPED(4, 4);
+        else TERNA_GROUPED(4, 2);
+    }
+#undef TERNA_GROUPED
+    return true;
 }
 
 template <bool ROPE, bool ADJ>
@@ -337,6 +379,22 @@ int ternaspmm_attention_partial_splits(int B, int H, int S)
     return sp;
 }
 
+int ternaspmm_attention_partial_splits_kv(int B, int H, int KV, int S)
+{
+    if (B < 1 || H < 1 || KV < 1 || H % KV != 0 || S < 1) return -1;
+    const int gq = H / KV;
+    // several sequences whose kv groups share a workgroup (2 or 4 heads per kv head): the grid is B * KV * splits
+    // workgroups, and a cache of more than 512 slots already pays for the split (the unsplit launch requests 512 slots of
+    // keys up front and walks the rest in dependent round trips; measured, 8 sequences of the 2B shape, 856 slots:
+    // 1.316 ms per step unsplit, 1.235 with four splits; 556 slots: 1.204 against 1.219)
+    if (B >= 2 && (gq == 2 || gq == 4) && S > 512 && S <= 1024) {
+        int sp = 1;
+        while (sp < 4 && static_cast<long>(B) * KV * sp * 2 <= 256) sp *= 2;
+        return sp;
+    }
+    return ternaspmm_attention_partial_splits(B, H, S);
+}
+
 void ternaspmm_rope_decode_attention_partial(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,
                                              int per_sequence, terna_bf16* cache_k, terna_bf16* cache_v, float* partial, int splits,
                                              int B, int H, int KV, int D, int S, float scale, int adjacent,
@@ -350,10 +408,27 @@ void ternaspmm_rope_decode_attention_partial(const terna_bf16* qkv, const float*
         return;
     }
     AttentionPrefetch pf = prefetch_regions(pf_ptr, pf_bytes, pf_unit_bytes, pf_count);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // several sequences: the heads of a kv group share a workgroup (TERNASPMM_ATTN_GROUPED=0|1 forces either form)
+    static const int forced_grouped = [] {
+        const char* v = tuning_env("TERNASPMM_ATTN_GROUPED");
+        return v ? std::atoi(v) : -1;
+    }();
+    if (forced_grouped >= 0 ? forced_grouped != 0 : B >= 2) {
+        bool done;
+        if (D == 128) done = adjacent ? launch_attention_grouped<128, true>(qkv, cache_k, cache_v, cos, sin, pos, per_sequence != 0, partial, splits, B, H, KV, S, scale, pf, st)
+                                      : launch_attention_grouped<128, false>(qkv, cache_k, cache_v, cos, sin, pos, per_sequence != 0, partial, splits, B, H, KV, S, scale, pf, st);
+        else done = adjacent ? launch_attention_grouped<64, true>(qkv, cache_k, cache_v, cos, sin, pos, per_sequence != 0, partial, splits, B, H, KV, S, scale, pf, st)
+                             : launch_attention_grouped<64, false>(qkv, cache_k, cache_v, cos, sin, pos, per_sequence != 0, partial, splits, B, H, KV, S, scale, pf, st);
+        if (done) {
+            const hipError_t e = hipGetLastError();
+            if (e != hipSuccess) die("ternaspmm_rope_decode_attention_partial", e, __LINE__);
+            return;
+        }
+    }
     const bool grouped = attention_groups_on(H, KV);
     const int slots = grouped ? 8 * (H / KV) * ((B * KV * splits + 7) / 8) : B * H * splits;
     pf.workgroups = prefetch_workgroups(pf, slots);
-    hipStream_t st = static_cast<hipStream_t>(stream);
 #define TERNA_DEFER(DIM, ADJ) \
     launch_attention_deferred<DIM, ADJ>(qkv, cache_k, cache_v, cos, sin, pos, per_sequence != 0, partial, splits, B, H, KV, S, scale, pf, st)
     if (D == 128) {

@@ -123,6 +123,7 @@ KERNEL_ATTENTION = object()    # in place of a mask: several new tokens, attenti
 
 
 class Block:
+    merge_quant = True             # forward_chain, several sequences, deferred attention merge: the merge launch also norms and quantises
     chain_down_rows = 4            # forward_chain: up to this many rows the down projection normalises + quantises in its own launch
 
     def __init__(self, args: ModelArgs, gen: Optional[torch.Generator], act: str, p_zero: float = 0.40):
@@ -246,12 +247,14 @@ class Block:
         o_kw = dict(epilogue=EPILOGUE_RESIDUAL, residual=x, next_norm_weight=self.ffn_norm, want_raw=pub, publish=pub)
         if deferred:
             partial, splits = attn_ws
-            pf = self.prefetch if split and self.prefetch is not None else (None, None, None, 0)
+            # (weights of the next launches through the caches meanwhile: only next to a short attention -- with caches of
+            # 1656 slots the prefetch cost 2 % of the step, at 856 slots it gains 0.5 %)
+            pf = self.prefetch if split and self.prefetch is not None and cache_k.shape[2] <= 1024 else (None, None, None, 0)
             lib.ternaspmm_rope_decode_attention_partial(
                 _p(qkv), _p(cos), _p(sin), _p(pos_idx), per_seq, _p(cache_k), _p(cache_v), _p(partial), splits, bsz, a.n_heads,
                 a.n_kv_heads, a.head_dim, cache_k.shape[2], a.head_dim ** -0.5, int(a.rope_adjacent), *pf, stream)
             r = None
-            if split:
+            if split or (bsz > 1 and self.merge_quant):
                 # merge + sub-norm + quantisation once per sequence, then the O projection on the quantised rows
                 mq = attention_merge_rmsnorm_quant(partial, splits, a.n_heads, a.head_dim, self.attn_sub_norm, a.norm_eps, bsz, want_output=pub)
                 if mq is not None:
@@ -407,6 +410,7 @@ class Transformer:
     # small element-wise launch forms the quantised rows from the partials (Block.forward_chain, split): lighter than the
     # norm kernels, which reduce over the row twice, and the gate+up launch writes F columns instead of 2F.
     split_rows = 8
+    defer_above = 1024             # cache slots from which on a chained step of 2 .. chain_rows sequences splits its attention
 
     def __init__(self, args: ModelArgs, seed: int = 0, act: str = "int8", p_zero: float = 0.40):
         gen = torch.Generator(device="cuda").manual_seed(seed)
@@ -505,7 +509,7 @@ class Transformer:
             return None
         a = self.args
         lib = _lib.load()
-        splits = getattr(self, "attention_splits", None) or lib.ternaspmm_attention_partial_splits(bsz, a.n_heads, max_seq)
+        splits = getattr(self, "attention_splits", None) or lib.ternaspmm_attention_partial_splits_kv(bsz, a.n_heads, a.n_kv_heads, max_seq)
         if splits < 1 or (splits == 1 and not single_split):
             return None
         # one buffer per batch size, kept while the model lives: a captured decode graph holds the raw pointer
@@ -565,7 +569,7 @@ class Transformer:
         # (in the split chain that merge launch also norms and quantises the O projection's input; with short caches
         # the unsplit launch + the O projection with the norm inside stay ahead there too: 8 sequences, slot 255 of 384,
         # 1.198 against 1.218 ms per step -- `split_merge_quant` forces the split form)
-        if one_launch_attention and self.layers[0].act == "int8" and (bsz == 1 or max_seq > 1024):
+        if one_launch_attention and self.layers[0].act == "int8" and (bsz == 1 or max_seq > (512 if split else self.defer_above)):
             attn_ws = self.attention_partial(bsz, max_seq) or attn_ws
         elif split and getattr(self, "split_merge_quant", False):
             attn_ws = self.attention_partial(bsz, max_seq, single_split=True) or attn_ws
