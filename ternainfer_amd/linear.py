@@ -198,8 +198,9 @@ def attention_merge_rmsnorm_linear_packed(partial, splits, heads, head_dim, norm
                                           sequences=1):
     """The O projection of a decode step fed by the partial results of a split attention launch
     (ternaspmm_rope_decode_attention_partial over `sequences` sequences): for one sequence merge -> RMSNorm -> quant_input
-    -> int8 TernaSpMM in one launch where the library supports the shape, else ternaspmm_attention_merge +
-    rmsnorm_linear_packed (the same bits).  partial: fp32 device buffer of ternaspmm_attention_partial_bytes(sequences, ...);
+    -> int8 TernaSpMM in one launch where the library supports the shape; for more, merge + norm + quantisation in one
+    launch (ternaspmm_attention_merge_rmsnorm_quant) and the linear on its rows; else ternaspmm_attention_merge +
+    rmsnorm_linear_packed.  partial: fp32 device buffer of ternaspmm_attention_partial_bytes(sequences, ...);
     returns out bf16 [sequences, out_features]."""
     lib = _lib.load()
     k = heads * head_dim
@@ -212,6 +213,11 @@ def attention_merge_rmsnorm_linear_packed(partial, splits, heads, head_dim, norm
         if lib.bitlinear_TernaSpMM_packed_fused_attn(_p(partial), splits, head_dim, _p(norm_weight), float(eps), _p(packed), _p(out),
                                                      _p(ws), ws_num, None, None, 1, out_features, k, stream):
             return out
+    else:
+        # several sequences: merge + norm + quantisation once per sequence in one launch, then the linear on the quantised rows
+        mq = attention_merge_rmsnorm_quant(partial, splits, heads, head_dim, norm_weight, eps, sequences)
+        if mq is not None:
+            return TernaInfer_linear_packed(mq[0], packed, mq[1], ws, ws_num, out_features)
     o = torch.empty((sequences, k), dtype=torch.bfloat16, device=partial.device)
     lib.ternaspmm_attention_merge(_p(partial), splits, _p(o), sequences, heads, head_dim, stream)
     return rmsnorm_linear_packed(o, norm_weight, eps, packed, ws, ws_num, out_features)[0]
