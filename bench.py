@@ -295,7 +295,11 @@ def run_model(args, torch):
                                + ("; one sequence: the attention is split over several workgroups per head and the O "
                                   "projection's prologue merges the partial results" if args.batch == 1 else
                                   ("" if args.no_prefetch else "; the idle CUs of the attention launch "
-                                                               "prefetch the weights of the launches that follow")),
+                                                               "prefetch the weights of the launches that follow"))
+                               + ("" if args.no_chain or args.batch > 8 else
+                                  "; the linears are chained through producer-side norm statistics"
+                                  + (" (consumed inside the next linear)" if args.batch <= 4 else
+                                     " (consumed by an element-wise quantise launch in front of the next linear)")),
                    "batch": args.batch, "act": act},
         **{k: fig[k] for k in ("prefill_tokens_per_s", "prefill_ms", "decode_s", "model_build_s", "first_tokens",
                                "graph_equals_eager_first_tokens")}}

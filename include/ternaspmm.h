@@ -419,7 +419,7 @@ void ternaspmm_rope_decode_attention_prefetch(const terna_bf16* qkv, const float
  * heads fill the chip anyway).  pf_ptr may be NULL with pf_count = 0.
  * Several sequences with 2 or 4 heads per kv head run one workgroup per (sequence, kv head, split): the heads of a kv
  * group read the same keys and values, which then cross from L2 into a CU once instead of once per head (same bits;
- * measured, 2B shape, caches of 1656 slots: 8 sequences 1.463 -> 1.351 ms per decode step, 6 sequences 1.405 -> 1.258).
+ * measured, 2B shape, caches of 1528 slots: 8 sequences 1.463 -> 1.351 ms per decode step, 6 sequences 1.405 -> 1.258).
  * ternaspmm_attention_partial_splits_kv(B, H, KV, S) is the recommendation for that form: it splits from 512 slots on. */
 long long ternaspmm_attention_partial_bytes(int B, int H, int D);
 int ternaspmm_attention_partial_splits(int B, int H, int S);

@@ -132,7 +132,7 @@ bool launch_attention_grouped(const uint16_t* qkv, uint16_t* ck, uint16_t* cv, c
                               const AttentionPrefetch& pf_in, hipStream_t st)
 {
     static const int waves = [] {
-        // 8 waves: measured ahead of 4 at 2 - 8 sequences with caches of 1656 slots (8 sequences: 1.351 against 1.410 ms
+        // 8 waves: measured ahead of 4 at 2 - 8 sequences with caches of 1528 slots (8 sequences: 1.351 against 1.410 ms
         // per decode step), level with them at 384 slots
         const char* v = tuning_env("TERNASPMM_ATTN_GROUPED_WAVES");
         return v && std::atoi(v) == 4 ? 4 : 8;
@@ -385,8 +385,8 @@ int ternaspmm_attention_partial_splits_kv(int B, int H, int KV, int S)
     const int gq = H / KV;
     // several sequences whose kv groups share a workgroup (2 or 4 heads per kv head): the grid is B * KV * splits
     // workgroups, and a cache of more than 512 slots already pays for the split (the unsplit launch requests 512 slots of
-    // keys up front and walks the rest in dependent round trips; measured, 8 sequences of the 2B shape, 856 slots:
-    // 1.316 ms per step unsplit, 1.235 with four splits; 556 slots: 1.204 against 1.219)
+    // keys up front and walks the rest in dependent round trips; measured, 8 sequences of the 2B shape, 728 slots:
+    // 1.316 ms per step unsplit, 1.235 with four splits; 428 slots: 1.204 against 1.219)
     if (B >= 2 && (gq == 2 || gq == 4) && S > 512 && S <= 1024) {
         int sp = 1;
         while (sp < 4 && static_cast<long>(B) * KV * sp * 2 <= 256) sp *= 2;

@@ -248,7 +248,7 @@ class Block:
         if deferred:
             partial, splits = attn_ws
             # (weights of the next launches through the caches meanwhile: only next to a short attention -- with caches of
-            # 1656 slots the prefetch cost 2 % of the step, at 856 slots it gains 0.5 %)
+            # 1528 slots the prefetch cost 2 % of the step, at 728 slots it gains 0.5 %)
             pf = self.prefetch if split and self.prefetch is not None and cache_k.shape[2] <= 1024 else (None, None, None, 0)
             lib.ternaspmm_rope_decode_attention_partial(
                 _p(qkv), _p(cos), _p(sin), _p(pos_idx), per_seq, _p(cache_k), _p(cache_v), _p(partial), splits, bsz, a.n_heads,
@@ -411,8 +411,8 @@ class Transformer:
     # norm kernels, which reduce over the row twice, and the gate+up launch writes F columns instead of 2F.
     split_rows = 8
     # Cache slots from which on a chained step of 2 .. chain_rows sequences splits its attention and leaves the merge to a
-    # launch of its own (measured, 4 sequences: 556 slots 1.041 ms per step unsplit against 1.115, 856 slots 1.154 against 1.120)
-    defer_above = 768
+    # launch of its own (measured, 4 sequences: 428 slots 1.041 ms per step unsplit against 1.115, 728 slots 1.154 against 1.120)
+    defer_above = 640
 
     def __init__(self, args: ModelArgs, seed: int = 0, act: str = "int8", p_zero: float = 0.40):
         gen = torch.Generator(device="cuda").manual_seed(seed)
