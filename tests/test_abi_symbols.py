@@ -97,6 +97,17 @@ def test_host_side_size_and_policy_functions():
     assert lib.ternaspmm_attention_partial_splits(1, 20, 64) == 2
     assert lib.ternaspmm_attention_partial_splits(1, 20, 128) == 4
     assert lib.ternaspmm_attention_workspace_bytes(1, 20, 128) > 0
+    # knowing the kv heads: several sequences with 2 or 4 heads per kv head split from 512 slots on (one workgroup per kv head)
+    assert lib.ternaspmm_attention_partial_splits_kv(8, 20, 5, 384) == 1
+    assert lib.ternaspmm_attention_partial_splits_kv(8, 20, 5, 728) == 4
+    assert lib.ternaspmm_attention_partial_splits_kv(16, 20, 5, 728) == 2
+    assert lib.ternaspmm_attention_partial_splits_kv(8, 20, 5, 2048) == lib.ternaspmm_attention_partial_splits(8, 20, 2048)
+    assert lib.ternaspmm_attention_partial_splits_kv(1, 20, 5, 728) == lib.ternaspmm_attention_partial_splits(1, 20, 728)
+    assert lib.ternaspmm_attention_partial_splits_kv(8, 20, 20, 728) == lib.ternaspmm_attention_partial_splits(8, 20, 728)
+    assert lib.ternaspmm_attention_partial_splits_kv(8, 20, 3, 728) == -1
+    # refused on the host, nothing enqueued: split counts and row lengths the merge + norm + quantise launch does not take
+    assert lib.ternaspmm_attention_merge_rmsnorm_quant(None, 3, None, 1e-5, None, None, None, 8, 20, 128, None) == -1
+    assert lib.ternaspmm_attention_merge_rmsnorm_quant(None, 4, None, 1e-5, None, None, None, 8, 40, 128, None) == -1
 
 
 def test_python_wrappers_refuse_mismatched_tensors_on_the_host():
