@@ -283,8 +283,9 @@ int bitlinear_TernaSpMM_packed_fused_glu(const terna_bf16* x13, const terna_bf16
  * combination or the shape is not supported and nothing was enqueued (supported: K <= 2560 for every combination,
  * K <= 7168 for TERNASPMM_PROLOGUE_STATS with STORE / RESIDUAL, K <= 8192 for PROLOGUE_NORM, K <= 4096 for
  * PROLOGUE_ATTENTION; GATE needs PROLOGUE_STATS; PROLOGUE_NORM here only with EPILOGUE_RESIDUAL).  out must not alias x or
- * residual.  Only enqueues.  Every workgroup of such a launch repeats the norm + quantisation of all M rows: measured on
- * the 2B shapes the chain pays up to 4 rows; above, ternaspmm_rmsnorm_quant + bitlinear_TernaSpMM_packed is faster. */
+ * residual.  Only enqueues.  Every workgroup of a launch with a NORM / ATTENTION / STATS prologue repeats the norm +
+ * quantisation of all M rows: measured on the 2B shapes that pays up to 4 rows; above, ternaspmm_quant_from_stats in front
+ * of a PROLOGUE_QUANTISED launch (or of bitlinear_TernaSpMM_packed) consumes the producer's partials faster. */
 enum { TERNASPMM_PROLOGUE_NORM = 0, TERNASPMM_PROLOGUE_ATTENTION = 1, TERNASPMM_PROLOGUE_STATS = 2, TERNASPMM_PROLOGUE_QUANTISED = 3 };
 enum { TERNASPMM_EPILOGUE_STORE = 0, TERNASPMM_EPILOGUE_RESIDUAL = 1, TERNASPMM_EPILOGUE_GATE = 2 };
 typedef struct ternaspmm_fused_linear_desc {

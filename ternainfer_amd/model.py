@@ -401,10 +401,10 @@ class Block:
 class Transformer:
     """Random-init decoder; `act` selects int8-quantised (reference semantics) or bf16 activations."""
 
-    # Up to this many sequences a one-token step chains its linears (Block.forward_chain).  Every workgroup of a chained
-    # linear normalises and quantises the whole activation matrix again, and one of its waves per row only adds up
-    # partials; from five rows on a norm + quantisation launch of its own and the plain small-M kernel are faster
-    # (measured at 6 and 8 rows).
+    # Up to this many sequences a one-token step chains its linears with the norm + quantisation inside the consuming
+    # linear (Block.forward_chain).  Every workgroup of such a linear normalises and quantises the whole activation matrix
+    # again, and one of its waves per row only adds up partials; from five rows on that costs more than a launch that does
+    # it once (measured at 5, 6 and 8 rows).
     chain_rows = 4
     # Above that, up to this many sequences, the producing epilogues stay (residual add, gate, partial statistics) and a
     # small element-wise launch forms the quantised rows from the partials (Block.forward_chain, split): lighter than the
