@@ -258,8 +258,8 @@ def measure_model(torch, batch, act="int8", prefetch=True, gen_tokens=256, check
         for blk in model.layers:
             blk.chain_down_rows = int(os.environ["TERNA_BENCH_CHAIN_DOWN_ROWS"])
     model.enable_prefetch(False)
-    if prefetch:     # weights of the following launches, pulled through the caches during the attention launch
-        model.enable_prefetch(True, ("wo", "w13", "w2", "next_wqkv", "norms") if batch <= 2 else ("wo", "w13", "norms"))
+    if prefetch and batch <= 2:     # weights of the following launches, pulled through the caches during the attention launch
+        model.enable_prefetch(True, ("wo", "w13", "w2", "next_wqkv", "norms"))
     torch.cuda.synchronize()
     build_s = time.perf_counter() - t0
     gen = torch.Generator(device="cuda").manual_seed(20260501)
@@ -294,8 +294,8 @@ def run_model(args, torch):
                                "sampling are library kernels; the prompt pass is one HIP graph too"
                                + ("; one sequence: the attention is split over several workgroups per head and the O "
                                   "projection's prologue merges the partial results" if args.batch == 1 else
-                                  ("" if args.no_prefetch else "; the idle CUs of the attention launch "
-                                                               "prefetch the weights of the launches that follow"))
+                                  ("" if args.no_prefetch or args.batch > 2 else "; the idle CUs of the attention launch "
+                                                                                 "prefetch the weights of the launches that follow"))
                                + ("" if args.no_chain or args.batch > 8 else
                                   "; the linears are chained through producer-side norm statistics"
                                   + (" (consumed inside the next linear)" if args.batch <= 4 else

@@ -399,7 +399,8 @@ void ternaspmm_rope_decode_attention(const terna_bf16* qkv, const float* cos, co
  * kernel reads: bands per workgroup x K/64 x 256 bytes -- so that a unit lands in the L2 its consumer will use;
  * pf_unit_bytes[r] = 0 marks a small region (at most 1 MiB: norm weights, scales) that every workgroup of the
  * consumers reads and every XCD therefore fetches whole.
- * A region that breaks one of these rules is skipped.
+ * A region that breaks one of these rules is skipped; nothing is prefetched when the attention leaves fewer than 96
+ * CUs idle (the few prefetching workgroups would outlast it).
  * pf_ptr / pf_bytes / pf_unit_bytes are host arrays of pf_count entries, read during the call.  Results are those of
  * ternaspmm_rope_decode_attention; nothing depends on where the prefetched bytes end up. */
 void ternaspmm_rope_decode_attention_prefetch(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,

@@ -210,7 +210,9 @@ int prefetch_workgroups(const AttentionPrefetch& pf, int slots)
         const char* v = tuning_env("TERNASPMM_ATTN_PREFETCH_WGS");
         return v ? std::atoi(v) / 8 * 8 : -1;
     }();
-    return pf.count > 0 && slots < 232 ? (forced_wgs >= 0 ? forced_wgs : (256 - slots) / 8 * 8) : 0;
+    // With fewer than 96 CUs left the few prefetching workgroups outlast the attention (measured, 2B shape, regions of
+    // 10 MB: 9 - 11 sequences -- 64 and 32 workgroups -- ran 10 - 20 % slower per step than without prefetch).
+    return pf.count > 0 && slots <= 160 ? (forced_wgs >= 0 ? forced_wgs : (256 - slots) / 8 * 8) : 0;
 }
 
 }  // namespace

@@ -453,8 +453,10 @@ class Transformer:
     def enable_prefetch(self, on: bool = True, which=("wo", "w13", "w2", "next_wqkv", "norms")) -> None:
         """Single-token steps: while a block's attention runs (one workgroup per head), extra workgroups of that
         launch prefetch the weights of its O, gate+up and down projections and of the next block's QKV projection
-        (`which` picks among them).  Measured on MI355X: +6 % tokens/s at batch 1 with all four; at batch 8, where
-        the heads leave fewer CUs idle, ("wo", "w13") gives +1 % and more than that costs time."""
+        (`which` picks among them).  Measured on MI355X with the unsplit attention launch: +6 % tokens/s at batch 1 with
+        all four.  With the step as it is now -- one sequence runs the split attention, which passes no regions -- it pays
+        for two sequences (+1 %); from three on the step is 1.4 - 1.7 % faster without, and where few CUs are left idle the
+        prefetching workgroups become the launch's critical path (nine to eleven sequences: 10 - 20 % slower)."""
         for n, blk in enumerate(self.layers):
             if not on:
                 blk.prefetch = None
