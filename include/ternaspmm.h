@@ -266,7 +266,7 @@ int bitlinear_TernaSpMM_packed_fused_glu(const terna_bf16* x13, const terna_bf16
  *                                           (stats_count <= 448), as a producing epilogue or ternaspmm_row_stats left them
  *             TERNASPMM_PROLOGUE_QUANTISED  x = int8 [M][K] with its scales s_in bf16 [M] (ternaspmm_quant_from_stats,
  *                                           ternaspmm_rmsnorm_quant): no prologue; with TERNASPMM_EPILOGUE_RESIDUAL
- *                                           (M <= 16, any K the int8 kernels take) or TERNASPMM_EPILOGUE_GATE (M <= 8,
+ *                                           (M <= 16, any K the int8 kernels take) or TERNASPMM_EPILOGUE_GATE (M <= 16,
  *                                           K <= 6144).  From five rows on this pair -- the element-wise quantise launch,
  *                                           then the linear on its rows -- is the faster way to consume a producer's
  *                                           partials (measured, 2B shapes, 8 rows: 6706 against 6498 tokens/s for the

@@ -187,20 +187,28 @@ bool launch_chunk_by_rows(const ChainArgs& a, int units)
     return true;
 }
 
-// Activations quantised already (int8 rows + scales), producing epilogue, up to 8 rows: all 16 waves share the units.
+// Activations quantised already (int8 rows + scales), producing epilogue, up to 16 rows: all 16 waves share the units.
 template <int NBANDS, int EPI>
 bool launch_chunk_quantised(const ChainArgs& a, const uint16_t* s_in, int units)
 {
     ChainIo io{a.out, a.ws, nullptr, nullptr, a.ex.epi_residual, a.ex.epi_next_w, a.ex.stats_out, a.ex.raw_out};
     io.s_in = s_in;
     const int ct = (units + kChunkWaves - 1) / kChunkWaves;
-    if (ct > 3 || a.M > 8) return false;
-#define TERNA_CHAIN_XQ(CT)                                                                                              \
-    terna_chain_chunk_kernel<NBANDS, CT, 8, EPI, (NBANDS == 4 ? 2 : 1), true><<<a.grid, dim3(kChunkWaves * 64), 0, a.st>>>( \
-        a.x, nullptr, a.packed, nullptr, a.M, a.N, a.K, 0, 0.0f, a.ws_num, 0, io)
-    if (ct == 1) TERNA_CHAIN_XQ(1);
-    else if (ct == 2) TERNA_CHAIN_XQ(2);
-    else TERNA_CHAIN_XQ(3);
+    if (ct > 3 || a.M > 16) return false;
+#define TERNA_CHAIN_XQ(CT, MR)                                                                                          \
+    do {                                                                                                                \
+        auto kernel = terna_chain_chunk_kernel<NBANDS, CT, MR, EPI, (NBANDS == 4 ? 2 : 1), true>;                         \
+        kernel<<<a.grid, dim3(kChunkWaves * 64), 0, a.st>>>(a.x, nullptr, a.packed, nullptr, a.M, a.N, a.K, 0, 0.0f, a.ws_num, 0, io); \
+    } while (0)
+#define TERNA_CHAIN_XQ_CT(MR)                                                                                           \
+    do {                                                                                                                \
+        if (ct == 1) TERNA_CHAIN_XQ(1, MR);                                                                             \
+        else if (ct == 2) TERNA_CHAIN_XQ(2, MR);                                                                        \
+        else TERNA_CHAIN_XQ(3, MR);                                                                                     \
+    } while (0)
+    if (a.M <= 8) TERNA_CHAIN_XQ_CT(8);
+    else TERNA_CHAIN_XQ_CT(16);
+#undef TERNA_CHAIN_XQ_CT
 #undef TERNA_CHAIN_XQ
     return true;
 }

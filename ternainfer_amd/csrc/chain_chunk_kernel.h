@@ -116,14 +116,14 @@ __device__ __forceinline__ void chain_quantise(const uint32_t (&hraw)[NE / 2], c
 // XQ: the activations are quantised already (`hin` is int8 [M][K], io.s_in their scales; a launch of
 // terna_quant_stats_kernel or of the norm kernel made them): no reducing waves, no statistics, no barrier ahead of the
 // matmul; all 16 waves share the units and a chunk's rows go from the load to the LDS slot as they are (16 bytes per lane,
-// four rows per load).  The producing epilogues are the same.
+// four rows per load).  The producing epilogues are the same.  MR = 16 exists in this form only.
 template <int NBANDS, int CT, int MR, int EPI, int UNIT_BANDS = (NBANDS == 4 ? 2 : 1), bool XQ = false>
 __global__ __launch_bounds__(kChunkWaves * 64) void terna_chain_chunk_kernel(
     const void* __restrict__ hin, const uint16_t* __restrict__ norm_w, const uint32_t* __restrict__ packed,
     const float2* __restrict__ stats_in, int M, int N, int K, int stats_count, float eps, int ws_num, int quant_mode, ChainIo io)
 {
     static_assert((NBANDS == 1 && (EPI == CEPI_STORE || EPI == CEPI_RESIDUAL)) || (NBANDS == 4 && EPI == CEPI_GATE), "see above");
-    static_assert(MR == 1 || MR == 2 || MR == 4 || MR == 8, "rows of the slab");
+    static_assert(MR == 1 || MR == 2 || MR == 4 || MR == 8 || (XQ && MR == 16), "rows of the slab (sixteen: quantised rows only)");
     constexpr int WAVES = kChunkWaves;
     constexpr int NE = MR == 1 ? 4 : 8;          // columns per lane and load
     constexpr int LPR = 256 / NE;                // lanes along a chunk row

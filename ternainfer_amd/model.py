@@ -208,7 +208,7 @@ class Block:
         return self.w13_interleaved
 
     def forward_chain(self, x, stats, cache_k, cache_v, pos_idx, cos, sin, attn_ws, next_norm, split=False):
-        """One new token per sequence (up to 8 sequences), the linears chained through producer-side norm statistics:
+        """One new token per sequence (up to 16 sequences), the linears chained through producer-side norm statistics:
         `x` is the residual stream INCLUDING the previous block's FFN output and `stats` its partials under this block's
         attention_norm (None: the first block, which takes them inside).  Every linear's epilogue leaves what the next
         launch needs: the O projection adds the stream and leaves the ffn_norm partials, gate+up leaves
@@ -285,7 +285,14 @@ class Block:
                                                     a.head_dim ** -0.5, int(a.rope_adjacent), _p(attn_ws), stream)
             if pub:
                 cap.append(("attention", None, None, o))
-            r = fused_linear(o, self.attn_sub_norm, a.norm_eps, self.wo.packed, self.wo.ws, self.wo.ws_num, self.wo.n, self.wo.k, **o_kw)
+            r = None
+            if bsz <= 8:                         # the sub-norm's statistics taken inside the O projection
+                r = fused_linear(o, self.attn_sub_norm, a.norm_eps, self.wo.packed, self.wo.ws, self.wo.ws_num, self.wo.n, self.wo.k, **o_kw)
+            if r is None:                        # more rows: the norm kernel, then the O projection on its quantised rows
+                xq, s, _ = rmsnorm_quant(o, self.attn_sub_norm, a.norm_eps)
+                r = fused_linear(xq, None, a.norm_eps, self.wo.packed, self.wo.ws, self.wo.ws_num, self.wo.n, self.wo.k, quantised=s,
+                                 epilogue=EPILOGUE_RESIDUAL, residual=x, next_norm_weight=self.ffn_norm, want_raw=pub)
+                r = (r[0], r[1], r[2], xq, s)
         note("wo", r)
         h, h_stats = r[0], r[1]
         if split:
@@ -409,7 +416,7 @@ class Transformer:
     # Above that, up to this many sequences, the producing epilogues stay (residual add, gate, partial statistics) and a
     # small element-wise launch forms the quantised rows from the partials (Block.forward_chain, split): lighter than the
     # norm kernels, which reduce over the row twice, and the gate+up launch writes F columns instead of 2F.
-    split_rows = 8
+    split_rows = 16
     # Cache slots from which on a chained step of 2 .. chain_rows sequences splits its attention and leaves the merge to a
     # launch of its own (measured, 4 sequences: 428 slots 1.041 ms per step unsplit against 1.115, 728 slots 1.154 against 1.120)
     defer_above = 640

@@ -158,6 +158,26 @@ def test_gate_epilogue_on_interleaved_gate_up(m, f, k):
     assert torch.equal(r[0], inner) and torch.equal(r[1], st_out)
 
 
+@pytest.mark.parametrize("m", [9, 11, 16])
+@pytest.mark.parametrize("f,k", [(6912, 2560), (128, 192), (64, 6144)])
+def test_gate_epilogue_on_quantised_rows_above_eight(m, f, k):
+    """The gate epilogue fed with quantised rows takes up to 16 of them (the statistics-fed prologue stops at 8): the norm
+    kernel's (xq, s) in, relu(x1)^2 * x3 and its partials out, against the oracle on the ordinary [w1; w3] matrix."""
+    n = 2 * f
+    w13 = make_ternary(n, k, 0.40, 1270 + m + f)
+    inter = L.interleave_gate_up(_packed(w13), n, k)
+    h = make_bf16_activations(m, k, 1271 + m + k, outlier_frac=0.01)
+    g, nxt = _weight(k, 1272 + k), _weight(f, 1273 + f)
+    xq, s, _ = L.rmsnorm_quant(_bf(h), _bf(g), 1e-5)
+    print(f"[case] chain gate+up, quantised activations: m={m} f={f} k={k}", flush=True)
+    r = L.fused_linear(xq, None, 1e-5, inter, _bf(WS), 2, n, k, quantised=s, epilogue=L.EPILOGUE_GATE, next_norm_weight=_bf(nxt))
+    assert r is not None
+    torch.cuda.synchronize()
+    want = O.relu2_mul(O.spmm_i8(xq.cpu().numpy(), w13, _bits(s), WS, 2, 0))
+    assert r[0].shape == (m, f) and (_bits(r[0]) == want).all()
+    _check_stats(r[1].cpu().numpy(), want, nxt, 16)
+
+
 def test_norm_and_attention_prologues_with_the_residual_epilogue():
     """The prologues that take their statistics inside, now with the producing epilogue: the raw output must be the
     bits of the existing entry points (same kernel arithmetic), the stream their residual sum."""
@@ -202,7 +222,7 @@ def test_norm_and_attention_prologues_with_the_residual_epilogue():
     _check_stats(st.cpu().numpy(), h_next, nxt, 16)
 
 
-@pytest.mark.parametrize("m", [1, 5, 8, 16])
+@pytest.mark.parametrize("m", [1, 5, 8, 11, 16])
 @pytest.mark.parametrize("n,k", [(2560, 6912), (2560, 2560), (8256, 192)])
 def test_quantise_launch_and_quantised_prologue(m, n, k):
     """The norm + quantisation as a launch of its own from the producer's partials, and the small-M linear on its output
@@ -246,9 +266,9 @@ def test_unsupported_combinations_are_declined():
     assert L.fused_linear(h, g, 1e-5, packed, _bf(WS), 1, n, k) is None                                    # NORM + STORE: the older entry point
     assert L.fused_linear(h, g, 1e-5, packed, _bf(WS), 1, n, k, stats=L.row_stats(h, g), epilogue=L.EPILOGUE_GATE,
                           next_norm_weight=_bf(_weight(n // 2, 1253))) is None                              # GATE needs two scale groups
-    xq9 = torch.zeros((9, k), dtype=torch.int8, device="cuda")
-    s9 = torch.ones(9, dtype=torch.bfloat16, device="cuda")
+    xq9 = torch.zeros((17, k), dtype=torch.int8, device="cuda")
+    s9 = torch.ones(17, dtype=torch.bfloat16, device="cuda")
     assert L.fused_linear(xq9, None, 1e-5, packed, _bf(WS), 2, n, k, quantised=s9, epilogue=L.EPILOGUE_GATE,
-                          next_norm_weight=_bf(_weight(n // 2, 1254))) is None                              # GATE on quantised rows: up to 8
+                          next_norm_weight=_bf(_weight(n // 2, 1254))) is None                              # GATE on quantised rows: up to 16
     assert L.fused_linear(xq9, None, 1e-5, packed, _bf(WS), 1, n, k, quantised=s9) is None                 # QUANTISED + STORE: bitlinear_TernaSpMM_packed
     torch.cuda.synchronize()
