@@ -251,6 +251,9 @@ def measure_model(torch, batch, act="int8", prefetch=True, gen_tokens=256, check
         model.split_merge_quant = os.environ["TERNA_BENCH_SPLIT_MERGE_QUANT"] != "0"
     if os.environ.get("TERNA_BENCH_DEFER_ABOVE"):
         model.defer_above = int(os.environ["TERNA_BENCH_DEFER_ABOVE"])
+    if os.environ.get("TERNA_BENCH_ATTENTION_STATS"):
+        for blk in model.layers:
+            blk.attention_stats = os.environ["TERNA_BENCH_ATTENTION_STATS"] != "0"
     if os.environ.get("TERNA_BENCH_O_NORM_ROWS"):
         for blk in model.layers:
             blk.o_norm_rows = int(os.environ["TERNA_BENCH_O_NORM_ROWS"])

@@ -391,6 +391,15 @@ void ternaspmm_rope_decode_attention(const terna_bf16* qkv, const float* cos, co
                                      int per_sequence, terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV,
                                      int D, int S, float scale, int adjacent, void* workspace, terna_stream stream);
 
+/* ternaspmm_rope_decode_attention (always the unsplit launch) as a producer for the chained step: next to out it leaves,
+ * per sequence and head, the partial statistics of the norm that reads the attention output (model.py:236
+ * attn_sub_norm, norm_weight bf16 [H * D]): stats_out fp32 [B][H][2] = (sum of o^2, max |o * norm_weight|) over the
+ * head's D columns of the stored bf16 row -- what ternaspmm_quant_from_stats (stats_count = H) or a
+ * TERNASPMM_PROLOGUE_STATS launch adds up.  Returns H, or -1 for unsupported arguments (nothing enqueued). */
+int ternaspmm_rope_decode_attention_stats(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos, int per_sequence,
+                                          terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV, int D, int S,
+                                          float scale, int adjacent, const terna_bf16* norm_weight, float* stats_out, terna_stream stream);
+
 /* ternaspmm_rope_decode_attention with up to six prefetch regions (no counterpart in the reference).  The attention
  * of a decode step occupies one CU per (sequence, head); this variant adds workgroups on the CUs that stay idle, which
  * read pf_bytes[r] bytes (at most 1 GiB) at pf_ptr[r] (16-byte aligned device memory) and discard them: the weights of the launches that

@@ -60,6 +60,7 @@ PROTOTYPES = {
     "ternaspmm_attention_merge": ([_vp, _ci, _vp, _ci, _ci, _ci, _vp], None),
     "ternaspmm_attention_merge_rmsnorm_quant": ([_vp, _ci, _vp, ctypes.c_float, _vp, _vp, _vp, _ci, _ci, _ci, _vp], ctypes.c_int),
     "ternaspmm_rope_kv_store": ([_vp] * 4 + [_ci] + [_vp] * 3 + [_ci] * 7 + [_vp], None),
+    "ternaspmm_rope_decode_attention_stats": ([_vp] * 4 + [_ci] + [_vp] * 3 + [_ci] * 5 + [ctypes.c_float, _ci, _vp, _vp, _vp], ctypes.c_int),
     "ternaspmm_rope_decode_attention": ([_vp] * 4 + [_ci] + [_vp] * 3 + [_ci] * 5 + [ctypes.c_float, _ci, _vp, _vp], None),
     "ternaspmm_decode_attention": ([_vp] * 4 + [_ci, _vp] + [_ci] * 5 + [ctypes.c_float, _vp, _vp], None),
     "ternaspmm_prefill_attention": ([_vp] * 4 + [_ci, _vp] + [_ci] * 6 + [ctypes.c_float, _vp], None),

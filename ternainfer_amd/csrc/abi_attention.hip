@@ -91,8 +91,9 @@ int attention_splits(int B, int H, int S, const AttentionScratch& scratch)
 template <int D, bool ROPE, bool ADJ, int NW, bool SPLIT>
 void launch_attention_as(const uint16_t* q, uint16_t* ck, uint16_t* cv, const float* cos, const float* sin,
                          const long long* pos, int per_seq, uint16_t* out, int B, int H, int KV, int S, float scale, int splits,
-                         const AttentionScratch& scratch, const AttentionPrefetch& pf_in, hipStream_t st)
+                         const AttentionScratch& scratch, const AttentionPrefetch& pf_in, hipStream_t st, AttentionStats stats)
 {
+    if (stats.norm_w == nullptr || stats.out == nullptr) stats = AttentionStats{q, nullptr};   // (the kernel loads norm_w unconditionally)
     AttentionPrefetch pf = pf_in;
     if (splits > 1) pf.workgroups = 0;                       // the split grid is two-dimensional: no extra workgroups
     auto kernel = terna_decode_attention_kernel<D, ROPE, ADJ, NW, SPLIT>;
@@ -101,7 +102,7 @@ void launch_attention_as(const uint16_t* q, uint16_t* ck, uint16_t* cv, const fl
     const int slots = attention_slots(B, H, KV);
     kernel<<<dim3(slots + pf.workgroups, splits), dim3(64 * NW), lds, st>>>(
         q, ck, cv, pos, H, KV, S, splits, slots, attention_groups_on(H, KV) ? B * KV : 0, per_seq, scale, cos, sin, out, scratch.partial,
-        scratch.arrived, pf);
+        scratch.arrived, pf, stats);
 }
 
 // The split with the merge left to the next launch (DEFER): one-dimensional grid of (sequence, head, split) workgroups,
@@ -119,7 +120,7 @@ void launch_attention_deferred(const uint16_t* qkv, uint16_t* ck, uint16_t* cv, 
     const bool grouped = attention_groups_on(H, KV);
     const int slots = grouped ? 8 * (H / KV) * ((B * KV * splits + 7) / 8) : B * H * splits;
     kernel<<<dim3(slots + pf.workgroups), dim3(64 * NW), lds, st>>>(
-        qkv, ck, cv, pos, H, KV, S, splits, slots, grouped ? B * KV : 0, per_seq, scale, cos, sin, nullptr, partial, nullptr, pf);
+        qkv, ck, cv, pos, H, KV, S, splits, slots, grouped ? B * KV : 0, per_seq, scale, cos, sin, nullptr, partial, nullptr, pf, AttentionStats{qkv, nullptr});
 }
 
 int prefetch_workgroups(const AttentionPrefetch& pf, int slots);
@@ -166,12 +167,13 @@ bool launch_attention_grouped(const uint16_t* qkv, uint16_t* ck, uint16_t* cv, c
 template <bool ROPE, bool ADJ>
 void launch_attention(const uint16_t* q, uint16_t* ck, uint16_t* cv, const float* cos, const float* sin,
                              const long long* pos, int per_seq, uint16_t* out, int B, int H, int KV, int D, int S, float scale,
-                             const AttentionScratch& scratch, const AttentionPrefetch& pf, hipStream_t st)
+                             const AttentionScratch& scratch, const AttentionPrefetch& pf, hipStream_t st,
+                             AttentionStats stats = AttentionStats{nullptr, nullptr})
 {
     const int splits = attention_splits(B, H, S, scratch);
     const int nw = splits > 1 ? 4 : attention_waves(B, H);       // a split is a short prefix: the narrow workgroup
 #define TERNA_ATTN(DIM, NWAVES, SPLIT) \
-    launch_attention_as<DIM, ROPE, ADJ, NWAVES, SPLIT>(q, ck, cv, cos, sin, pos, per_seq, out, B, H, KV, S, scale, splits, scratch, pf, st)
+    launch_attention_as<DIM, ROPE, ADJ, NWAVES, SPLIT>(q, ck, cv, cos, sin, pos, per_seq, out, B, H, KV, S, scale, splits, scratch, pf, st, stats)
     if (D == 128) {
         if (splits > 1) TERNA_ATTN(128, 4, true);
         else if (nw == 8) TERNA_ATTN(128, 8, false);
@@ -337,6 +339,22 @@ void ternaspmm_rope_decode_attention(const terna_bf16* qkv, const float* cos, co
     else launch_attention<true, false>(qkv, cache_k, cache_v, cos, sin, pos, per_sequence != 0, out, B, H, KV, D, S, scale, scratch, AttentionPrefetch{}, st);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_rope_decode_attention", e, __LINE__);
+}
+
+int ternaspmm_rope_decode_attention_stats(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos, int per_sequence,
+                                          terna_bf16* cache_k, terna_bf16* cache_v, terna_bf16* out, int B, int H, int KV, int D, int S,
+                                          float scale, int adjacent, const terna_bf16* norm_weight, float* stats_out, terna_stream stream)
+{
+    if (!attention_args_ok("ternaspmm_rope_decode_attention_stats", B, H, KV, D, S)) return -1;
+    if (norm_weight == nullptr || stats_out == nullptr || H > 448) return -1;      // (448: partials per row a consumer adds up)
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const AttentionStats stats{norm_weight, reinterpret_cast<float2*>(stats_out)};
+    // no workspace: the unsplit launch, whose workgroups hold whole output rows of their heads
+    if (adjacent) launch_attention<true, true>(qkv, cache_k, cache_v, cos, sin, pos, per_sequence != 0, out, B, H, KV, D, S, scale, AttentionScratch{}, AttentionPrefetch{}, st, stats);
+    else launch_attention<true, false>(qkv, cache_k, cache_v, cos, sin, pos, per_sequence != 0, out, B, H, KV, D, S, scale, AttentionScratch{}, AttentionPrefetch{}, st, stats);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_rope_decode_attention_stats", e, __LINE__);
+    return H;
 }
 
 void ternaspmm_rope_decode_attention_prefetch(const terna_bf16* qkv, const float* cos, const float* sin, const long long* pos,

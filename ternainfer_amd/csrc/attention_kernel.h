@@ -325,6 +325,15 @@ __device__ __forceinline__ void attention_prefetch_role(const AttentionPrefetch&
     if (seen == 0xffffffffu && pf.count > kAttentionPrefetchRegions) *const_cast<u32x4*>(pf.base[0]) = u32x4{seen, 0u, 0u, 0u};   // never true: keeps the loads
 }
 
+// The unsplit launch as a producer: per (sequence, head) the partial statistics of the norm that reads the attention
+// output -- (sum of o^2, max |o * norm_w|) over the head's D columns of the stored bf16 row, the form
+// terna_quant_stats_kernel adds up (H partials per row).  norm_w is loaded unconditionally and must always point at H * D
+// readable elements (the launcher passes q when no statistics are wanted); out = nullptr: none written.
+struct AttentionStats {
+    const uint16_t* norm_w;
+    float2* out;                  // [B][H]
+};
+
 constexpr size_t decode_attention_lds_bytes(int D, int NW, int S)
 {
     return (static_cast<size_t>(S) + (64 * NW / (D / 8)) * D + 64 * NW) * sizeof(float);
@@ -336,7 +345,7 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
     const long long* __restrict__ pos, int H, int KV, int S, int splits, int heads, int groups, int per_seq, float scale,
     const float* __restrict__ cosv_all, const float* __restrict__ sinv_all, uint16_t* __restrict__ out,
-    float* partial, int* arrived, AttentionPrefetch pf)
+    float* partial, int* arrived, AttentionPrefetch pf, AttentionStats stats)
 {
     static_assert(D == 64 || D == 128, "head dimension");
     constexpr int CH = D / 8;                    // 8-dimension chunks of a row
@@ -457,6 +466,8 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
             sn[1] = *reinterpret_cast<const f32x4*>(sinv + 8 * ca + 4);
         }
     }
+    uint32_t nw_raw = 0u;                        // this thread's norm weight (unsplit launch: the statistics of the output row)
+    if constexpr (!SPLIT && !DEFER) nw_raw = stats.norm_w[h * D + (tid & (D - 1))];
     __builtin_amdgcn_sched_barrier(0);           // the requests above stay above the ones below
 #pragma unroll
     for (int t = 0; t < KT; ++t) load_keys(wave + NW * t, kr[t]);
@@ -629,7 +640,30 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     }
     uint16_t* orow = out + (static_cast<size_t>(b) * H + h) * D;
     if ((!SPLIT || SP == 1) && !DEFER) {        // (DEFER has no output row: `out` is NULL there, also with one split)
-        if (tid < D) orow[tid] = float_to_bf16_bits(o / sum);
+        float v = 0.0f;
+        if (tid < D) {
+            const uint16_t ob = float_to_bf16_bits(o / sum);
+            orow[tid] = ob;
+            v = bf16_bits_to_float(ob);
+        }
+        if constexpr (!SPLIT) {
+            if (stats.out != nullptr) {          // uniform: the row's statistics under the next norm, D columns = D / 64 waves
+                float ssq = v * v;
+                float pm = tid < D ? fabsf(__fmul_rn(v, __uint_as_float(nw_raw << 16))) : 0.0f;
+                ssq = wave_sum(ssq);
+                pm = wave_max(pm);
+                if (lane == 0 && wave < D / 64) {
+                    red[wave] = ssq;
+                    red[NW + wave] = pm;
+                }
+                __syncthreads();
+                if (tid == 0) {
+                    float2 r{red[0], red[NW]};
+                    if constexpr (D == 128) r = float2{red[0] + red[1], fmaxf(red[NW], red[NW + 1])};
+                    stats.out[bh] = r;
+                }
+            }
+        }
         return;
     }
 

@@ -907,3 +907,48 @@ def test_attention_merge_rmsnorm_quant(lib, b, h, kv, d, s_max, lens, splits):
     # outside its range: nothing enqueued
     assert lib.ternaspmm_attention_merge_rmsnorm_quant(_vp(part), 3, _vp(norm_w), 1e-5, None, _vp(xq3), _vp(s3), b, h, d, None) == -1
     assert lib.ternaspmm_attention_merge_rmsnorm_quant(_vp(part), splits, _vp(norm_w), 1e-5, None, _vp(xq3), _vp(s3), b, 40, 128, None) == -1
+
+
+@pytest.mark.parametrize("b,h,kv,d,s_max,lens", [(8, 20, 5, 128, 384, (300, 1, 129, 384, 77, 256, 200, 33)), (3, 4, 2, 64, 64, (5, 64, 17)),
+                                                 (12, 20, 5, 128, 256, tuple(range(20, 260, 20)))])
+def test_rope_decode_attention_with_norm_statistics(lib, b, h, kv, d, s_max, lens):
+    """ternaspmm_rope_decode_attention_stats: the output row and the caches are those of ternaspmm_rope_decode_attention
+    (no workspace: the unsplit launch); the statistics are, per sequence and head, the sum of squares (fp32 accuracy) and
+    the exact max |o * w| of the stored bf16 row; ternaspmm_quant_from_stats on them agrees with the norm kernel's scales
+    up to one bf16 step."""
+    k_in = h * d
+    qkv = make_bf16_activations(b, (h + 2 * kv) * d, 2200 + b)
+    k0 = make_bf16_activations(b * kv * s_max, d, 2201 + b).reshape(b, kv, s_max, d)
+    v0 = make_bf16_activations(b * kv * s_max, d, 2202 + b, outlier_frac=0.01).reshape(b, kv, s_max, d)
+    pos = np.array(lens, np.int64).reshape(b, 1) - 1
+    cos, sin = _angles(pos.reshape(-1), d)
+    w = _weight(k_in, 2203)
+    xd, cd, sd, pd, wd = _dev(qkv), _dev(cos), _dev(sin), _dev(pos), _dev(w)
+    ck1, cv1, ck2, cv2 = _dev(k0), _dev(v0), _dev(k0), _dev(v0)
+    o1 = torch.zeros((b, k_in), dtype=torch.int16, device="cuda")
+    o2 = torch.zeros_like(o1)
+    st = torch.full((b, h, 2), float("nan"), dtype=torch.float32, device="cuda")
+    print(f"[case] attention with norm statistics b={b} h={h} d={d}", flush=True)
+    lib.ternaspmm_rope_decode_attention(_vp(xd), _vp(cd), _vp(sd), _vp(pd), 1, _vp(ck1), _vp(cv1), _vp(o1), b, h, kv, d, s_max,
+                                        float(d) ** -0.5, 1, None, None)
+    assert lib.ternaspmm_rope_decode_attention_stats(_vp(xd), _vp(cd), _vp(sd), _vp(pd), 1, _vp(ck2), _vp(cv2), _vp(o2), b, h, kv, d, s_max,
+                                                     float(d) ** -0.5, 1, _vp(wd), _vp(st), None) == h
+    torch.cuda.synchronize()
+    assert torch.equal(o1, o2) and torch.equal(ck1, ck2) and torch.equal(cv1, cv2)
+    o = O.bf16_bits_to_f32(o2.cpu().numpy().view(np.uint16)).reshape(b, h, d)
+    wf = O.bf16_bits_to_f32(w).reshape(1, h, d)
+    got = st.cpu().numpy()
+    assert (got[:, :, 1] == np.abs(o * wf).max(axis=2)).all()
+    assert np.allclose(got[:, :, 0], (o.astype(np.float64) ** 2).sum(axis=2), rtol=2e-6, atol=1e-30)
+    # the consumer: quantised rows from these partials against the norm kernel on the same row
+    xq1, s1 = torch.zeros((b, k_in), dtype=torch.int8, device="cuda"), torch.zeros(b, dtype=torch.int16, device="cuda")
+    xq2, s2 = torch.zeros_like(xq1), torch.zeros_like(s1)
+    lib.ternaspmm_rmsnorm_quant(_vp(o2), None, None, _vp(wd), 1e-5, None, _vp(xq1), _vp(s1), b, k_in, None)
+    assert lib.ternaspmm_quant_from_stats(_vp(o2), _vp(st), h, _vp(wd), 1e-5, _vp(xq2), _vp(s2), b, k_in, None) == 0
+    torch.cuda.synchronize()
+    assert np.abs(_bf16_key(s1.cpu().numpy().view(np.uint16)) - _bf16_key(s2.cpu().numpy().view(np.uint16))).max() <= 1
+    same = (s1 == s2).cpu().numpy()
+    dq = np.abs(xq1.cpu().numpy().astype(np.int32) - xq2.cpu().numpy().astype(np.int32))[same]
+    assert dq.size and dq.max() <= 1 and (dq != 0).mean() < 0.02
+    assert lib.ternaspmm_rope_decode_attention_stats(_vp(xd), _vp(cd), _vp(sd), _vp(pd), 1, _vp(ck2), _vp(cv2), _vp(o2), b, h, kv, d, s_max,
+                                                     float(d) ** -0.5, 1, None, _vp(st), None) == -1
