@@ -254,6 +254,9 @@ def measure_model(torch, batch, act="int8", prefetch=True, gen_tokens=256, check
     if os.environ.get("TERNA_BENCH_ATTENTION_STATS"):
         for blk in model.layers:
             blk.attention_stats = os.environ["TERNA_BENCH_ATTENTION_STATS"] != "0"
+    if os.environ.get("TERNA_BENCH_ATTENTION_STATS_CHAIN"):
+        for blk in model.layers:
+            blk.attention_stats_chain = os.environ["TERNA_BENCH_ATTENTION_STATS_CHAIN"] != "0"
     if os.environ.get("TERNA_BENCH_O_NORM_ROWS"):
         for blk in model.layers:
             blk.o_norm_rows = int(os.environ["TERNA_BENCH_O_NORM_ROWS"])

@@ -127,6 +127,7 @@ class Block:
     # and the O projection on its quantised rows (measured: 4 sequences 3917 against 3769 tokens/s, 5 sequences 4285
     # against 4343, 8 sequences 6708 against 6849)
     o_norm_rows = 4
+    attention_stats_chain = True   # the same for 2 .. o_norm_rows sequences, consumed by the O projection's STATS prologue (+1 - 1.6 %)
     attention_stats = True         # ... and the unsplit attention launch leaves the sub-norm's partial statistics (see forward_chain)
     merge_quant = True             # forward_chain, several sequences, deferred attention merge: the merge launch also norms and quantises
     chain_down_rows = 4            # forward_chain: up to this many rows the down projection normalises + quantises in its own launch
@@ -285,7 +286,7 @@ class Block:
                     _p(qkv), _p(cos), _p(sin), _p(pos_idx), per_seq, _p(cache_k), _p(cache_v), _p(o), bsz, a.n_heads, a.n_kv_heads,
                     a.head_dim, cache_k.shape[2], a.head_dim ** -0.5, int(a.rope_adjacent), _p(attn_ws), ptrs, sizes, units,
                     count, stream)
-            elif bsz > self.o_norm_rows and self.attention_stats:
+            elif (bsz > self.o_norm_rows or (bsz > 1 and self.attention_stats_chain)) and self.attention_stats:
                 # the unsplit launch also leaves the sub-norm's partial statistics per head: the quantised rows of the O
                 # projection then come from the element-wise launch instead of the norm kernel
                 o_stats = torch.empty((bsz, a.n_heads, 2), dtype=torch.float32, device=x.device)
@@ -300,8 +301,9 @@ class Block:
             if pub:
                 cap.append(("attention", None, None, o))
             r = None
-            if bsz <= self.o_norm_rows:          # the sub-norm's statistics taken inside the O projection
-                r = fused_linear(o, self.attn_sub_norm, a.norm_eps, self.wo.packed, self.wo.ws, self.wo.ws_num, self.wo.n, self.wo.k, **o_kw)
+            if bsz <= self.o_norm_rows:          # the sub-norm's statistics taken inside the O projection (or given by the attention)
+                r = fused_linear(o, self.attn_sub_norm, a.norm_eps, self.wo.packed, self.wo.ws, self.wo.ws_num, self.wo.n, self.wo.k,
+                                 stats=o_stats, **o_kw)
             if r is None:                        # more rows: the norm kernel (or the quantise launch), then the O projection on quantised rows
                 if o_stats is not None:
                     xq, s = quant_from_stats(o, o_stats, self.attn_sub_norm, a.norm_eps)
