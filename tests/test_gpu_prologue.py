@@ -952,3 +952,36 @@ def test_rope_decode_attention_with_norm_statistics(lib, b, h, kv, d, s_max, len
     assert dq.size and dq.max() <= 1 and (dq != 0).mean() < 0.02
     assert lib.ternaspmm_rope_decode_attention_stats(_vp(xd), _vp(cd), _vp(sd), _vp(pd), 1, _vp(ck2), _vp(cv2), _vp(o2), b, h, kv, d, s_max,
                                                      float(d) ** -0.5, 1, None, _vp(st), None) == -1
+
+
+@pytest.mark.parametrize("splits", [1, 4])
+@pytest.mark.parametrize("b,h,kv,d,s_max,n", [(2, 4, 2, 64, 300, 17), (8, 20, 5, 128, 384, 300), (2, 16, 8, 128, 100, 77), (1, 20, 5, 128, 384, 200)])
+def test_rope_decode_attention_partial_rotate_half(lib, b, h, kv, d, s_max, n, splits):
+    """The deferred-merge launches with the rotate-half pairing of RoPE (adjacent = 0; several sequences with 2 or 4 heads
+    per kv head run one workgroup per kv head): caches bit-identical to ternaspmm_rope_decode_attention, merged output
+    within the attention tolerance of the unsplit launch."""
+    lens = [max(1, n - 5 * i) for i in range(b)]
+    qkv = make_bf16_activations(b, (h + 2 * kv) * d, 2301 + n)
+    k0 = make_bf16_activations(b * kv * s_max, d, 2302 + n).reshape(b, kv, s_max, d)
+    v0 = make_bf16_activations(b * kv * s_max, d, 2303 + n, outlier_frac=0.01).reshape(b, kv, s_max, d)
+    pos = np.array(lens, np.int64) - 1
+    cos, sin = _angles(pos, d)
+    xd, cd, sd, pd = _dev(qkv), _dev(cos), _dev(sin), _dev(pos)
+    scale = float(d) ** -0.5
+    ck1, cv1, ck2, cv2 = _dev(k0), _dev(v0), _dev(k0), _dev(v0)
+    o1 = torch.zeros((b, h * d), dtype=torch.int16, device="cuda")
+    o2 = torch.zeros_like(o1)
+    print(f"[case] attention partial + merge, rotate-half b={b} h={h} kv={kv} d={d} n={n} splits={splits}", flush=True)
+    lib.ternaspmm_rope_decode_attention(_vp(xd), _vp(cd), _vp(sd), _vp(pd), 1, _vp(ck1), _vp(cv1), _vp(o1), b, h, kv, d, s_max,
+                                        scale, 0, None, None)
+    part = _partial_buffer(lib, b, h, d)
+    lib.ternaspmm_rope_decode_attention_partial(_vp(xd), _vp(cd), _vp(sd), _vp(pd), 1, _vp(ck2), _vp(cv2), _vp(part), splits,
+                                                b, h, kv, d, s_max, scale, 0, None, None, None, 0, None)
+    lib.ternaspmm_attention_merge(_vp(part), splits, _vp(o2), b, h, d, None)
+    torch.cuda.synchronize()
+    assert torch.equal(ck1, ck2) and torch.equal(cv1, cv2)
+    got = O.bf16_bits_to_f32(o2.cpu().numpy().view(np.uint16)).reshape(b, h, d).astype(np.float64)
+    unsplit = O.bf16_bits_to_f32(o1.cpu().numpy().view(np.uint16)).reshape(b, h, d).astype(np.float64)
+    tol = 2.0 ** -7 * np.abs(unsplit).max(axis=-1, keepdims=True) + 1e-6
+    assert np.isfinite(got).all()
+    assert (np.abs(got - unsplit) <= 2 * tol).all(), float((np.abs(got - unsplit) / tol).max())
