@@ -95,32 +95,36 @@ def test_toy_model_greedy_decode_graph_equals_eager():
     assert torch.equal(a, c)
 
 
-@pytest.mark.parametrize("bsz", [3, 6, 12, 16])
-def test_toy_model_decode_step_forms_agree(bsz):
+@pytest.mark.parametrize("bsz,plen,slots", [(3, 20, 40), (6, 20, 40), (12, 20, 40), (16, 20, 40), (6, 560, 600), (12, 1040, 1100), (2, 700, 720)])
+def test_toy_model_decode_step_forms_agree(bsz, plen, slots):
     """One-token steps of several sequences: the chained forms (up to four sequences the statistics are consumed inside the
     next linear, above by the element-wise quantise launch; from nine on the O projection takes the norm kernel's rows)
-    against the step of plain launches; greedy tokens of the replayed graph against eager execution."""
+    against the step of plain launches; greedy tokens of the replayed graph against eager execution.  With the longer caches
+    the chained steps split their attention (one workgroup per kv head) and leave the merge to the launch that also norms
+    and quantises the O projection's input."""
     from ternainfer_amd.model import ModelArgs, Transformer, greedy_decode
     args = ModelArgs(dim=256, n_layers=3, n_heads=4, n_kv_heads=2, vocab_size=1024, ffn_dim=384)
     model = Transformer(args, seed=61, act="int8")
     assert model.chain_supported()
-    plen = 20
     prompt = torch.randint(0, args.vocab_size, (bsz, plen), generator=torch.Generator().manual_seed(62 + bsz)).cuda()
-    print(f"[case] toy model, {bsz} sequences: chained decode step against plain launches", flush=True)
+    print(f"[case] toy model, {bsz} sequences, {slots} cache slots: chained decode step against plain launches", flush=True)
     outs = []
     with torch.inference_mode():
         for chain in (True, False):
             model.chain = chain
-            cache = model.make_cache(bsz, 40)
+            cache = model.make_cache(bsz, slots)
             model.forward(prompt, cache, torch.arange(plen, device="cuda"))
             outs.append(model.forward(prompt[:, -1:].contiguous(), cache, torch.tensor([plen], device="cuda")).float())
     model.chain = True
+    if slots > 512 and bsz > 1:
+        assert model.attention_partial(bsz, slots) is not None             # the split attention is the path that ran
     assert outs[0].shape == (bsz, args.vocab_size)
     err = (outs[0] - outs[1]).abs().max().item()
     assert err <= 3e-2 * outs[1].abs().max().item(), err
     assert torch.nn.functional.cosine_similarity(outs[0].flatten(), outs[1].flatten(), dim=0).item() > 0.9995
-    a, _, _ = greedy_decode(model, prompt, 10, use_graph=True)
-    b, _, _ = greedy_decode(model, prompt, 10, use_graph=False)
+    gen = min(10, slots - plen)
+    a, _, _ = greedy_decode(model, prompt, gen, use_graph=True)
+    b, _, _ = greedy_decode(model, prompt, gen, use_graph=False)
     assert torch.equal(a, b)
 
 
