@@ -34,8 +34,10 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_decode_chunk_kernel(
     const Act* __restrict__ x, const uint32_t* __restrict__ packed, uint16_t* __restrict__ out,
     int M, int N, int K, Epilogue ep, RepackGuard guard)
 {
-    if constexpr (GUARD) {                       // the extra workgroup past the last band: see decode_packed_kernel.h
-        if (static_cast<int>(blockIdx.x) * 16 >= N) {
+    // GUARD: one extra workgroup checks the cached copy's fingerprint (decode_packed_kernel.h).  It is the FIRST of the grid:
+    // its check is two dependent memory round trips, longer than a band's work, and starts ahead of the bands' dispatch.
+    if constexpr (GUARD) {
+        if (blockIdx.x == 0) {
             if (threadIdx.x < 64) repack_guard_role(guard, threadIdx.x);
             return;
         }
@@ -59,7 +61,7 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_decode_chunk_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int band = blockIdx.x;
+    const int band = static_cast<int>(blockIdx.x) - (GUARD ? 1 : 0);
     const int ktiles = K >> 6;
     const int i = lane & 15, g = lane >> 4;
 
@@ -195,8 +197,8 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_decode_chunk4_kernel(
     const Act* __restrict__ x, const uint32_t* __restrict__ packed, uint16_t* __restrict__ out,
     int M, int N, int K, Epilogue ep, RepackGuard guard)
 {
-    if constexpr (GUARD) {
-        if (static_cast<int>(blockIdx.x) * 64 >= N) {
+    if constexpr (GUARD) {                       // the checking workgroup comes first (see above)
+        if (blockIdx.x == 0) {
             if (threadIdx.x < 64) repack_guard_role(guard, threadIdx.x);
             return;
         }
@@ -221,7 +223,7 @@ __global__ __launch_bounds__(kChunkWaves * 64) void terna_decode_chunk4_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int band0 = blockIdx.x * 4;
+    const int band0 = (static_cast<int>(blockIdx.x) - (GUARD ? 1 : 0)) * 4;
     const int ktiles = K >> 6;
     const int chunks = (ktiles + 3) >> 2;
     const int i = lane & 15, g = lane >> 4;

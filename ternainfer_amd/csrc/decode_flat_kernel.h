@@ -46,8 +46,8 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_flat_kernel(
     const Act* __restrict__ x, const uint32_t* __restrict__ packed, uint16_t* __restrict__ out,
     int M, int N, int K, Epilogue ep, RepackGuard guard)
 {
-    if constexpr (GUARD) {                       // the extra workgroup past the last band: see decode_packed_kernel.h
-        if (static_cast<int>(blockIdx.x) * (16 * NB) >= N) {
+    if constexpr (GUARD) {                       // the extra, checking workgroup is the first of the grid: see decode_packed_kernel.h
+        if (blockIdx.x == 0) {
             if (threadIdx.x < 64) repack_guard_role(guard, threadIdx.x);
             return;
         }
@@ -66,7 +66,7 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_flat_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int band0 = blockIdx.x * NB;
+    const int band0 = (static_cast<int>(blockIdx.x) - (GUARD ? 1 : 0)) * NB;
     const int ktiles = K >> 6;
     const int i = lane & 15, g = lane >> 4;
 

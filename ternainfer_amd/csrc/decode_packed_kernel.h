@@ -46,10 +46,13 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
     int M, int N, int K, Epilogue ep, RepackGuard guard, PackedProducer prod)
 {
     static_assert(!RES || (MB == 1 && sizeof(Act) == 1), "the producing epilogue: int8 activations, up to 16 rows");
-    // A launch on a cached P2 copy carries one extra workgroup in x -- the one past the last band -- that checks, next to
-    // the others and off their critical path, that the copy still belongs to the caller's tensors.
+    // A launch on a cached P2 copy carries one extra workgroup in x that checks, next to the others, that the copy still
+    // belongs to the caller's tensors.  It is the FIRST workgroup of the grid: the check is two dependent memory round trips
+    // (the stream's total, then the samples), longer than a band's work at small M, and as the last workgroup it started
+    // behind the dispatch of all the others and ended the launch (the 2B layer set through the reference symbols: 0.541 ms
+    // per step with the check last, 0.504 with it first, 0.500 without a check).
     if constexpr (GUARD) {
-        if (static_cast<int>(blockIdx.x) * (16 * NB) >= N) {
+        if (blockIdx.x == 0) {
             if (blockIdx.y == 0 && threadIdx.x < 64) repack_guard_role(guard, threadIdx.x);
             return;
         }
@@ -68,7 +71,7 @@ __global__ __launch_bounds__(WAVES * 64) void terna_decode_packed_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int band0 = blockIdx.x * NB;
+    const int band0 = (static_cast<int>(blockIdx.x) - (GUARD ? 1 : 0)) * NB;
     const int m_base = blockIdx.y * (16 * MB);
     const int ktiles = K >> 6;
     const int i = lane & 15, g = lane >> 4;
