@@ -54,13 +54,16 @@ int prefill_splits(long tiles, int steps, int M, int N, size_t scratch_bytes)
 
 template <typename Act, int MB, int NA>
 void launch_prefill_packed_dma_as(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M,
-                                  int N, int K, const PrefillPlan& plan, void* scratch, hipStream_t st)
+                                  int N, int K, const PrefillPlan& plan, void* scratch, hipStream_t st, const RepackGuard* guard)
 {
     using S = PackedPrefillDmaSmem<MB>;
     auto kernel = terna_prefill_packed_dma_kernel<Act, MB, NA>;
     allow_dynamic_lds(kernel, S::kBytes, "hipFuncSetAttribute(prefill packed dma)", __LINE__);
-    const dim3 grid(plan.grid_x, plan.grid_y, plan.splits);
     const int splits = plan.splits;
+    // The check of a cached copy rides in the launch: as one more row of workgroups in y, or -- with split-K planes, whose
+    // workgroup -> XCD pattern an extra row per plane would shift -- as the first workgroup of the reduce launch.
+    const bool guard_row = guard != nullptr && splits == 1;
+    const dim3 grid(plan.grid_x, plan.grid_y + (guard_row ? 1 : 0), plan.splits);
     static const int xcd_forced = [] {
         const char* v = tuning_env("TERNASPMM_PREFILL_XCD_MAP");
         return v ? std::atoi(v) : -1;
@@ -69,13 +72,15 @@ void launch_prefill_packed_dma_as(const Act* x, const uint32_t* packed, uint16_t
     // below that the default order, which fetches every weight tile on one XCD only, moves less data.
     // TERNASPMM_PREFILL_XCD_MAP=0|1 forces it off / on (tuning aid).
     const bool big_x = static_cast<size_t>(M) * K * sizeof(Act) > (4u << 20);
-    const int xcd_map = (grid.y % 8 == 0) && (xcd_forced < 0 ? big_x : xcd_forced != 0);
-    kernel<<<grid, dim3(256), S::kBytes, st>>>(x, packed, out, ep, M, N, K, xcd_map, splits, splits > 1 ? scratch : nullptr);
+    const int xcd_map = (plan.grid_y % 8 == 0) && (xcd_forced < 0 ? big_x : xcd_forced != 0);
+    kernel<<<grid, dim3(256), S::kBytes, st>>>(x, packed, out, ep, M, N, K, xcd_map, splits, splits > 1 ? scratch : nullptr,
+                                               guard_row ? 1 : 0, guard_row ? *guard : RepackGuard{});
     if (splits > 1) {
         using AccT = typename std::conditional<sizeof(Act) == 1, int, float>::type;
         const long quads = static_cast<long>(M) * (N >> 2);
-        terna_splitk_reduce_kernel<AccT><<<dim3(static_cast<unsigned>((quads + 255) / 256)), dim3(256), 0, st>>>(
-            static_cast<const AccT*>(scratch), out, ep, M, N, splits);
+        const bool guard_first = guard != nullptr;
+        terna_splitk_reduce_kernel<AccT><<<dim3(static_cast<unsigned>((quads + 255) / 256) + (guard_first ? 1 : 0)), dim3(256), 0, st>>>(
+            static_cast<const AccT*>(scratch), out, ep, M, N, splits, guard_first ? 1 : 0, guard_first ? *guard : RepackGuard{});
     }
 }
 
@@ -133,26 +138,28 @@ PrefillPlan plan_prefill_packed(const void* x, int M, int N, int K, const void* 
 }
 
 template <typename Act>
-void launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
-                           void* scratch, size_t scratch_bytes, hipStream_t st)
+bool launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                           void* scratch, size_t scratch_bytes, hipStream_t st, const RepackGuard* guard)
 {
     const PrefillPlan plan = plan_prefill_packed<Act>(x, M, N, K, scratch, scratch_bytes);
     if (plan.direct_lds) {
-        if (plan.bm == 64 && plan.bn == 128) launch_prefill_packed_dma_as<Act, 2, 1>(x, packed, out, ep, M, N, K, plan, scratch, st);
-        else if (plan.bm == 128 && plan.bn == 128) launch_prefill_packed_dma_as<Act, 4, 1>(x, packed, out, ep, M, N, K, plan, scratch, st);
-        else if (plan.bm == 128) launch_prefill_packed_dma_as<Act, 4, 2>(x, packed, out, ep, M, N, K, plan, scratch, st);
-        else launch_prefill_packed_dma_as<Act, 2, 2>(x, packed, out, ep, M, N, K, plan, scratch, st);
-        return;
+        if (plan.grid_y >= 65535u) guard = nullptr;         // (no room for the checking row: the caller launches the check itself)
+        if (plan.bm == 64 && plan.bn == 128) launch_prefill_packed_dma_as<Act, 2, 1>(x, packed, out, ep, M, N, K, plan, scratch, st, guard);
+        else if (plan.bm == 128 && plan.bn == 128) launch_prefill_packed_dma_as<Act, 4, 1>(x, packed, out, ep, M, N, K, plan, scratch, st, guard);
+        else if (plan.bm == 128) launch_prefill_packed_dma_as<Act, 4, 2>(x, packed, out, ep, M, N, K, plan, scratch, st, guard);
+        else launch_prefill_packed_dma_as<Act, 2, 2>(x, packed, out, ep, M, N, K, plan, scratch, st, guard);
+        return guard != nullptr;
     }
     if (plan.bm == 64 && plan.bn == 128) launch_prefill_packed_as<Act, 2, 1>(x, packed, out, ep, M, N, K, st);
     else if (plan.bm == 256) launch_prefill_packed_as<Act, 8>(x, packed, out, ep, M, N, K, st);
     else if (plan.bm == 96) launch_prefill_packed_as<Act, 3>(x, packed, out, ep, M, N, K, st);
     else if (plan.bm == 128) launch_prefill_packed_as<Act, 4>(x, packed, out, ep, M, N, K, st);
     else launch_prefill_packed_as<Act, 2>(x, packed, out, ep, M, N, K, st);
+    return false;
 }
 
-template void launch_prefill_packed<TERNA_PREFILL_ACT>(const TERNA_PREFILL_ACT*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int,
-                                                       void*, size_t, hipStream_t);
+template bool launch_prefill_packed<TERNA_PREFILL_ACT>(const TERNA_PREFILL_ACT*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int,
+                                                       void*, size_t, hipStream_t, const RepackGuard*);
 template PrefillPlan plan_prefill_packed<TERNA_PREFILL_ACT>(const void*, int, int, int, const void*, size_t);
 
 }  // namespace terna

@@ -44,10 +44,11 @@ void launch_decode_packed_producer(const int8_t* x, const uint32_t* packed, uint
 void launch_repack_fingerprint(const RepackGuard& guard, unsigned long long* out, hipStream_t st);
 void launch_repack_guard(const RepackGuard* guard, hipStream_t st);
 // `scratch` (may be NULL; 16-byte aligned, scratch_bytes long): room for split-K partial sums when the shape has few
-// output tiles for the chip; the call then enqueues two launches.
+// output tiles for the chip; the call then enqueues two launches.  `guard` (may be NULL): the check of a cached copy;
+// returns true when the launch carried it, false when the caller has to enqueue it (launch_repack_guard).
 template <typename Act>
-void launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
-                           void* scratch, size_t scratch_bytes, hipStream_t st);
+bool launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
+                           void* scratch, size_t scratch_bytes, hipStream_t st, const RepackGuard* guard = nullptr);
 // What launch_prefill_packed does with a call (host arithmetic only, nothing is enqueued): the output tile, the
 // grid, the split-K count and how many bytes of `scratch` the partial planes take (0 without a split; never more than
 // scratch_bytes).
@@ -70,10 +71,10 @@ extern template void launch_decode_packed<int8_t>(const int8_t*, const uint32_t*
                                                   const RepackGuard*);
 extern template void launch_decode_packed<uint16_t>(const uint16_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, hipStream_t,
                                                     const RepackGuard*);
-extern template void launch_prefill_packed<int8_t>(const int8_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, void*, size_t,
-                                                   hipStream_t);
-extern template void launch_prefill_packed<uint16_t>(const uint16_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, void*, size_t,
-                                                     hipStream_t);
+extern template bool launch_prefill_packed<int8_t>(const int8_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, void*, size_t,
+                                                   hipStream_t, const RepackGuard*);
+extern template bool launch_prefill_packed<uint16_t>(const uint16_t*, const uint32_t*, uint16_t*, const Epilogue&, int, int, int, void*, size_t,
+                                                     hipStream_t, const RepackGuard*);
 
 extern template PrefillPlan plan_prefill_packed<int8_t>(const void*, int, int, int, const void*, size_t);
 extern template PrefillPlan plan_prefill_packed<uint16_t>(const void*, int, int, int, const void*, size_t);

@@ -436,8 +436,16 @@ struct PackedPrefillDmaSmem {
 template <typename Act, int MB, int NA>
 __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) void terna_prefill_packed_dma_kernel(
     const Act* __restrict__ x, const uint32_t* __restrict__ packed, uint16_t* __restrict__ out,
-    Epilogue ep, int M, int N, int K, int xcd_map, int splits, void* __restrict__ partial)
+    Epilogue ep, int M, int N, int K, int xcd_map, int splits, void* __restrict__ partial, int guard_on, RepackGuard guard)
 {
+    // guard_on: the launch runs on a cached copy of a caller's weight and carries one extra row of workgroups in y, the
+    // first of which checks the copy's fingerprint next to the others (a launch of its own cost 1.5 - 2 us per call: 11 %
+    // of a step at M = 256); the rest of that row leaves at once.
+    const int tile_rows = static_cast<int>(gridDim.y) - (guard_on ? 1 : 0);
+    if (guard_on && static_cast<int>(blockIdx.y) == tile_rows) {
+        if (blockIdx.x == 0 && blockIdx.z == 0 && threadIdx.x < 64) repack_guard_role(guard, threadIdx.x);
+        return;
+    }
     using S = PackedPrefillDmaSmem<MB>;
     constexpr int BN = 128 * NA, BM = S::BM;
     // One step is 128 bytes of every activation row: 64 bf16 columns (one 64-column weight tile,
@@ -461,7 +469,7 @@ __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) voi
     int n_tile = blockIdx.x, m_tile = blockIdx.y;
     if (xcd_map) {
         const int linear = blockIdx.y * gridDim.x + blockIdx.x;
-        const int per_xcd = gridDim.y >> 3;          // batch tiles per XCD
+        const int per_xcd = tile_rows >> 3;          // batch tiles per XCD
         const int xcd = linear & 7, idx = linear >> 3;
         m_tile = xcd * per_xcd + idx % per_xcd;
         n_tile = idx / per_xcd;
@@ -648,11 +656,16 @@ __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) voi
 // family: weights were +-2, the sum is halved first, as in the unsplit epilogue).  One thread per four columns.
 template <typename AccT>
 __global__ __launch_bounds__(256) void terna_splitk_reduce_kernel(const AccT* __restrict__ partial, uint16_t* __restrict__ out,
-                                                                  Epilogue ep, int M, int N, int splits)
+                                                                  Epilogue ep, int M, int N, int splits, int guard_on, RepackGuard guard)
 {
+    // guard_on: the first workgroup of the grid checks the cached copy the planes were computed from (see the main kernel)
+    if (guard_on && blockIdx.x == 0) {
+        if (threadIdx.x < 64) repack_guard_role(guard, threadIdx.x);
+        return;
+    }
     typedef AccT V4 __attribute__((ext_vector_type(4)));
     const int quads = N >> 2;
-    const long idx = static_cast<long>(blockIdx.x) * 256 + threadIdx.x;
+    const long idx = (static_cast<long>(blockIdx.x) - (guard_on ? 1 : 0)) * 256 + threadIdx.x;
     if (idx >= static_cast<long>(M) * quads) return;
     const int m = static_cast<int>(idx / quads), n0 = static_cast<int>(idx - static_cast<long>(m) * quads) * 4;
     const size_t at = static_cast<size_t>(m) * N + n0, plane = static_cast<size_t>(M) * N;

@@ -248,8 +248,8 @@ void run_planned(const CallPlan& plan, const Act* x, const Weights& w, const Rep
         launch_decode_packed<Act>(x, cached.packed, out, ep, M, N, K, st, &cached.guard);
         break;
     case CALL_P2_LARGE:
-        launch_prefill_packed<Act>(x, cached.packed, out, ep, M, N, K, scratch, plan.scratch_bytes, st);
-        launch_repack_guard(&cached.guard, st);
+        if (!launch_prefill_packed<Act>(x, cached.packed, out, ep, M, N, K, scratch, plan.scratch_bytes, st, &cached.guard))
+            launch_repack_guard(&cached.guard, st);
         break;
     case CALL_REF_SMALL:
         launch_decode<Act>(x, w, out, ep, M, N, K, st);

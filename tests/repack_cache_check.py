@@ -31,29 +31,36 @@ def _stats(lib):
 
 def stale() -> int:
     lib = _lib.load()
-    n, k = 320, 192
-    # the replacement is sparser: its sign stream is shorter than the one the copy's check was set up for
-    a, b = DeviceFormat(make_ternary(n, k, 0.30, 980)), DeviceFormat(make_ternary(n, k, 0.70, 981))
-    assert b.vals.numel() < a.vals.numel()
-    xq, s = make_int8_activations(8, k, 982)
-    for _ in range(2):                           # first sight (copy made), cached sight
-        if not (run_i8(lib, a, xq, s, WS, 1) == O.spmm_i8(xq, a.w, s, WS, 1, 0)).all():
-            print("int8 mismatch before the rewrite")
-            return 1
-    assert _stats(lib)[0] == 1
-    a.bm.copy_(b.bm); a.off.copy_(b.off); a.med.copy_(b.med)
-    a.vals.zero_(); a.vals[: b.vals.numel()].copy_(b.vals)
-    torch.cuda.synchronize()
-    print("[case] rewritten under the same pointers, no clear", flush=True)
-    run_i8(lib, a, xq, s, WS, 1)                 # this launch reports the stale copy (its result is the old weight's)
-    torch.cuda.synchronize()
-    want = O.spmm_i8(xq, b.w, s, WS, 1, 0)
-    for sight in range(3):                       # dropped + rebuilt (first sight again), then cached sights
-        if not (run_i8(lib, a, xq, s, WS, 1) == want).all():
-            print("the new weight is not served correctly after the stale copy was dropped", sight)
-            return 1
-    st = _stats(lib)
-    assert st[0] == 1 and st[2] == 1, st
+    # which launch carries the check: the small-M kernel (an extra workgroup, first of the grid), the MFMA-tiled kernel
+    # (an extra row of workgroups), or -- with split-K planes in the workspace -- the launch that adds the planes up
+    cases = [("small-M kernel", 320, 192, 8, 3, False), ("MFMA-tiled kernel", 320, 192, 300, 4, False),
+             ("MFMA-tiled kernel + split-K", 256, 3328, 256, 4, True)]
+    for index, (what, n, k, m, kernel, split) in enumerate(cases):
+        # the replacement is sparser: its sign stream is shorter than the one the copy's check was set up for
+        a, b = DeviceFormat(make_ternary(n, k, 0.30, 980 + index)), DeviceFormat(make_ternary(n, k, 0.70, 990 + index))
+        assert b.vals.numel() < a.vals.numel()
+        xq, s = make_int8_activations(m, k, 982 + index)
+        used = ctypes.c_longlong(0)
+        assert lib.ternaspmm_plan_reference_call(1, 0, m, n, k, 7, ctypes.c_void_p(4096), 1, ctypes.byref(used)) == kernel, what
+        assert (used.value > 0) == split, (what, used.value)
+        for _ in range(2):                           # first sight (copy made), cached sight
+            if not (run_i8(lib, a, xq, s, WS, 1) == O.spmm_i8(xq, a.w, s, WS, 1, 0 if m <= 64 else 1)).all():
+                print("int8 mismatch before the rewrite", what)
+                return 1
+        before = _stats(lib)
+        a.bm.copy_(b.bm); a.off.copy_(b.off); a.med.copy_(b.med)
+        a.vals.zero_(); a.vals[: b.vals.numel()].copy_(b.vals)
+        torch.cuda.synchronize()
+        print(f"[case] rewritten under the same pointers, no clear: the check rides in the {what}", flush=True)
+        run_i8(lib, a, xq, s, WS, 1)                 # this launch reports the stale copy (its result is the old weight's)
+        torch.cuda.synchronize()
+        want = O.spmm_i8(xq, b.w, s, WS, 1, 0 if m <= 64 else 1)
+        for sight in range(3):                       # dropped + rebuilt (first sight again), then cached sights
+            if not (run_i8(lib, a, xq, s, WS, 1) == want).all():
+                print("the new weight is not served correctly after the stale copy was dropped", what, sight)
+                return 1
+        st = _stats(lib)
+        assert st[2] == before[2] + 1, (what, before, st)
     print("stale copy dropped and rebuilt ok")
     return 0
 
