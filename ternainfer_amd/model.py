@@ -130,7 +130,7 @@ class Block:
     attention_stats_chain = True   # the same for 2 .. o_norm_rows sequences, consumed by the O projection's STATS prologue (+1 - 1.6 %)
     attention_stats = True         # ... and the unsplit attention launch leaves the sub-norm's partial statistics (see forward_chain)
     merge_quant = True             # forward_chain, several sequences, deferred attention merge: the merge launch also norms and quantises
-    chain_down_rows = 4            # forward_chain: up to this many rows the down projection normalises + quantises in its own launch
+    chain_down_rows = 2            # forward_chain: up to this many rows the down projection (K = ffn_dim) norms + quantises inside its launch
 
     def __init__(self, args: ModelArgs, gen: Optional[torch.Generator], act: str, p_zero: float = 0.40):
         self.args = args
@@ -325,8 +325,8 @@ class Block:
         note("w13", r)
         inner, inner_stats = r[0], r[1]
         if split or bsz > self.chain_down_rows:
-            # K = 6912: from five rows on every workgroup repeating the norm + quantisation of the whole block costs more than
-            # one launch that does it once (measured at 8 rows: 10.7 us in one launch, 2.7 + 5.3 us in two)
+            # K = 6912: from three rows on every workgroup repeating the norm + quantisation of the whole block costs more than
+            # one launch that does it once (measured: 3 sequences 2972 -> 3031 tokens/s, 4 3976 -> 4004; 2 sequences 2094 against 2082)
             xq, s = quant_from_stats(inner, inner_stats, self.ffn_sub_norm, a.norm_eps)
             r = fused_linear(xq, None, a.norm_eps, self.w2.packed, self.w2.ws, self.w2.ws_num, self.w2.n, self.w2.k, quantised=s,
                              epilogue=EPILOGUE_RESIDUAL, residual=h, next_norm_weight=next_norm, want_raw=pub)
