@@ -88,7 +88,7 @@ int attention_splits(int B, int H, int S, const AttentionScratch& scratch)
     return sp;
 }
 
-template <int D, bool ROPE, bool ADJ, int NW, bool SPLIT>
+template <int D, bool ROPE, bool ADJ, int NW, bool SPLIT, int KT = 4>
 void launch_attention_as(const uint16_t* q, uint16_t* ck, uint16_t* cv, const float* cos, const float* sin,
                          const long long* pos, int per_seq, uint16_t* out, int B, int H, int KV, int S, float scale, int splits,
                          const AttentionScratch& scratch, const AttentionPrefetch& pf_in, hipStream_t st, AttentionStats stats)
@@ -96,9 +96,9 @@ void launch_attention_as(const uint16_t* q, uint16_t* ck, uint16_t* cv, const fl
     if (stats.norm_w == nullptr || stats.out == nullptr) stats = AttentionStats{q, nullptr};   // (the kernel loads norm_w unconditionally)
     AttentionPrefetch pf = pf_in;
     if (splits > 1) pf.workgroups = 0;                       // the split grid is two-dimensional: no extra workgroups
-    auto kernel = terna_decode_attention_kernel<D, ROPE, ADJ, NW, SPLIT>;
+    auto kernel = terna_decode_attention_kernel<D, ROPE, ADJ, NW, SPLIT, false, KT>;
     const size_t lds = decode_attention_lds_bytes(D, NW, S);
-    if (lds > 64 * 1024) allow_dynamic_lds(kernel, 160 * 1024, "hipFuncSetAttribute(decode attention)", __LINE__);
+    if (lds > 64 * 1024) allow_dynamic_lds(kernel, 159 * 1024, "hipFuncSetAttribute(decode attention)", __LINE__);
     const int slots = attention_slots(B, H, KV);
     kernel<<<dim3(slots + pf.workgroups, splits), dim3(64 * NW), lds, st>>>(
         q, ck, cv, pos, H, KV, S, splits, slots, attention_groups_on(H, KV) ? B * KV : 0, per_seq, scale, cos, sin, out, scratch.partial,
@@ -174,15 +174,28 @@ void launch_attention(const uint16_t* q, uint16_t* ck, uint16_t* cv, const float
     const int nw = splits > 1 ? 4 : attention_waves(B, H);       // a split is a short prefix: the narrow workgroup
 #define TERNA_ATTN(DIM, NWAVES, SPLIT) \
     launch_attention_as<DIM, ROPE, ADJ, NWAVES, SPLIT>(q, ck, cv, cos, sin, pos, per_seq, out, B, H, KV, S, scale, splits, scratch, pf, st, stats)
+    // the wide unsplit workgroup: as many key tiles in flight per wave as cover the cache (128 slots each), four at most
+    static const bool all_tiles = [] {               // TERNASPMM_ATTN_KEY_TILES=4: always four (tuning aid)
+        const char* v = tuning_env("TERNASPMM_ATTN_KEY_TILES");
+        return v && std::atoi(v) == 4;
+    }();
+#define TERNA_ATTN_WIDE(DIM)                                                                                                         \
+    do {                                                                                                                             \
+        if (all_tiles) TERNA_ATTN(DIM, 8, false);                                                                                    \
+        else if (S <= 256) launch_attention_as<DIM, ROPE, ADJ, 8, false, 2>(q, ck, cv, cos, sin, pos, per_seq, out, B, H, KV, S, scale, splits, scratch, pf, st, stats); \
+        else if (S <= 384) launch_attention_as<DIM, ROPE, ADJ, 8, false, 3>(q, ck, cv, cos, sin, pos, per_seq, out, B, H, KV, S, scale, splits, scratch, pf, st, stats); \
+        else TERNA_ATTN(DIM, 8, false);                                                                                              \
+    } while (0)
     if (D == 128) {
         if (splits > 1) TERNA_ATTN(128, 4, true);
-        else if (nw == 8) TERNA_ATTN(128, 8, false);
+        else if (nw == 8) TERNA_ATTN_WIDE(128);
         else TERNA_ATTN(128, 4, false);
     } else {
         if (splits > 1) TERNA_ATTN(64, 4, true);
-        else if (nw == 8) TERNA_ATTN(64, 8, false);
+        else if (nw == 8) TERNA_ATTN_WIDE(64);
         else TERNA_ATTN(64, 4, false);
     }
+#undef TERNA_ATTN_WIDE
 #undef TERNA_ATTN
 }
 

@@ -339,7 +339,7 @@ constexpr size_t decode_attention_lds_bytes(int D, int NW, int S)
     return (static_cast<size_t>(S) + (64 * NW / (D / 8)) * D + 64 * NW) * sizeof(float);
 }
 
-template <int D, bool ROPE, bool ADJACENT = false, int NW = 4, bool SPLIT = false, bool DEFER = false>
+template <int D, bool ROPE, bool ADJACENT = false, int NW = 4, bool SPLIT = false, bool DEFER = false, int KT = 4>
 __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     // what the first loads depend on comes first: the leading sixteen dwords of the arguments arrive in scalar registers
     const uint16_t* __restrict__ q, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
@@ -423,7 +423,11 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     // partial score of row i and a slot's score is the sum over its R rows: the accumulator puts
     // them in R neighbouring lanes (columns 0 .. R-1), one quad permutation or two add them up.
     constexpr int NJ = D / 32;                   // MFMAs (32 dimensions each) per tile
-    constexpr int KT = 4;                        // key tiles in flight per wave: slots 0 .. 255
+    // KT key tiles in flight per wave (slots 0 .. 64 NW KT - 1 of the split; tiles beyond go through the loop below, one
+    // dependent round trip each).  The launcher picks KT so that the requests just cover the cache: every request costs the
+    // CU's address unit a slot whatever it returns, and a test in the kernel -- even a wave-uniform one on a kernel argument
+    // -- made the waits around the requests conservative (8 sequences, caches of 384 slots: four tiles 6951 tokens/s,
+    // three 7001, four with the fourth behind such a test 6919).
     constexpr int VU = 8;                        // value rows in flight per thread
     const int r16 = lane & 15, kblk = lane >> 4;
     const int chunk = tid % CH, slice = tid / CH;
@@ -432,11 +436,15 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
     const int rr = r16 % R, sl = r16 / R;
     const int piece = rr + R * kblk;             // this lane's 16 bytes (8 dimensions) of a key row, and of q
     u32x4 kr[KT][NJ], vr[VU], qb;
+    // Cache rows come through raw buffer loads over the kv head's S rows: a slot past the cache costs an instruction slot
+    // but neither a memory access nor a returned kilobyte (a clamped address did both).
+    const __amdgpu_buffer_rsrc_t rk = make_raw_buffer(kbase, static_cast<uint32_t>(S) * D * 2u);
+    const __amdgpu_buffer_rsrc_t rv = make_raw_buffer(vbase, static_cast<uint32_t>(S) * D * 2u);
     auto load_keys = [&](int ltile, u32x4 (&dst)[NJ]) {
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
             const int sk = 16 * (ltile * SP + sp) + SPM * j + sl;
-            dst[j] = *reinterpret_cast<const u32x4*>(kbase + static_cast<size_t>(sk < S ? sk : 0) * D + 8 * piece);
+            dst[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rk, (sk * D + 8 * piece) * 2, 0, 0));
         }
     };
     // Order of the requests: the new token's own row pieces and angles first (ROPE) -- loads return in order, so
@@ -474,7 +482,7 @@ __global__ __launch_bounds__(64 * NW) void terna_decode_attention_kernel(
 #pragma unroll
     for (int u = 0; u < VU; ++u) {
         const int sv = cache_slot(slice + u * SLICES);
-        vr[u] = *reinterpret_cast<const u32x4*>(vbase + static_cast<size_t>(sv < S ? sv : 0) * D + chunk * 8);
+        vr[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rv, (sv * D + chunk * 8) * 2, 0, 0));
     }
     __builtin_amdgcn_sched_barrier(0);           // everything is requested; only now the position is looked at
     // Prefix length: slots 0 .. pos.  It comes from device memory the host cannot check, so it is clamped to the

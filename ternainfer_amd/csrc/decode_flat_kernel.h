@@ -24,14 +24,6 @@
 
 namespace terna {
 
-constexpr int kBufferRsrcFlags = 0x00020000;                    // raw buffer, 32-bit data format
-constexpr int kBufferOutOfRange = static_cast<int>(0x80000000u);   // a lane offset no buffer reaches
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_raw_buffer(const void* base, uint32_t bytes)
-{
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), kBufferRsrcFlags);
-}
-
 // The weight-scale group of one output column (the rule of ws_group_decode4 / ws_group_prefill for a single column).
 __device__ __forceinline__ int ws_group_of(int n, int N, int ws_num, int kind)
 {

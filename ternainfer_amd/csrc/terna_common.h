@@ -148,6 +148,16 @@ struct EpilogueRegs {
     float w[4];     // weight-group scale of each column (bf16 family: the fp32 scale)
 };
 
+// Raw buffer loads: a resource (base, byte range) in scalar registers, a per-lane byte offset and a scalar offset.  A lane
+// whose offset lies past the range gets zeros and touches no memory -- no clamped address, no masked branch.
+constexpr int kBufferRsrcFlags = 0x00020000;                    // raw buffer, 32-bit data format
+constexpr int kBufferOutOfRange = static_cast<int>(0x80000000u);   // a lane offset no buffer reaches
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_raw_buffer(const void* base, uint32_t bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), kBufferRsrcFlags);
+}
+
 // Makes the value live in registers at this point of the program: a load that produced it cannot be sunk
 // past here (into a branch, next to its use), and is waited for here.
 __device__ __forceinline__ void pin_registers(u32x4& v)
