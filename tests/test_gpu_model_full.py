@@ -132,14 +132,21 @@ class Worst:
 
 
 def check_quantiser(tag, y_twin, xq, s, worst, max_step, max_frac):
-    """The GPU's (xq, s) against the quantisation of the twin's float64 norm output: the scale within one bf16 step;
+    """The GPU's (xq, s) against the quantisation of the twin's float64 norm output: the scale within one bf16 step (or
+    the scale of a row maximum one bf16 step beside the twin's);
     on rows whose scale agrees the integers within `max_step`, differing on at most `max_frac` of the elements.
-    Observed worst over both batch sizes, 30 layers and 3 passes: one step on 5e-5 of the elements where the norm's
+    Observed worst over the batch sizes, 30 layers and 3 passes: one step on 5e-5 of the elements where the norm's
     input is known exactly (bound 2e-3), on 8e-4 behind the attention that is merged inside the O projection, where
     the twin's input comes from its own float64 attention (bound 1e-2)."""
     q_t, s_t = cpu_quant(y_twin)
     ds = bf16_steps(s, s_t)
-    assert int(ds.max()) <= 1, f"{tag}: activation scale {int(ds.max())} bf16 steps off"
+    # The fp32 norm may round a row's largest element to the bf16 neighbour of the float64 norm's; where that value's
+    # mantissa is near 1 and the scale's near 2, one step of the maximum is two steps of 127 / maximum.  So a scale more
+    # than one step off must be the exact scale of a maximum one bf16 step beside the twin's.
+    top = y_twin.float().abs().amax(-1).to(torch.bfloat16).view(torch.int16).to(torch.int32)
+    beside = [(127.0 / (top + d).to(torch.int16).view(torch.bfloat16).float().clamp(min=1e-5)).to(torch.bfloat16) for d in (-1, 1)]
+    ok = (ds <= 1) | (s == beside[0]) | (s == beside[1])
+    assert bool(ok.all()), f"{tag}: activation scale {int(ds[~ok].max())} bf16 steps off"
     same = ds == 0
     assert bool(same.any()), f"{tag}: no row with an agreeing scale"
     dq = (xq[same].to(torch.int32) - q_t[same].to(torch.int32)).abs()
@@ -243,7 +250,7 @@ def full_model():
     return (args,) + build_model(args, seed=20260500)
 
 
-@pytest.mark.parametrize("bsz", [1, 8])
+@pytest.mark.parametrize("bsz", [1, 8, 12, 16])
 def test_full_size_blocks_match_cpu_twin_layer_by_layer(full_model, bsz):
     args, model, host = full_model
     gen = torch.Generator().manual_seed(20260500 + bsz)
@@ -306,7 +313,7 @@ def test_full_size_blocks_match_cpu_twin_layer_by_layer(full_model, bsz):
             print(f"[info] batch {bsz} pass {pi} logits: {r}", flush=True)
 
 
-@pytest.mark.parametrize("bsz", [1, 8])
+@pytest.mark.parametrize("bsz", [1, 8, 12, 16])
 def test_full_size_decode_graph_gives_the_tokens_of_eager_execution(full_model, bsz):
     from ternainfer_amd.model import greedy_decode
     args, model, _ = full_model
