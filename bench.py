@@ -16,7 +16,7 @@ dense matrix -- divided by the measured time.  `roofline` prices the same bytes 
 layer of the same workload and doubles as the correctness gate of the run.
 
 The default run (`--workload decode`) also measures, in the same process and into the same line,
-the other figures the path is judged on: the literal single-matrix configuration (`config1`),
+the other figures of the path: the literal single-matrix configuration (`config1`),
 the layer set at M = 1 and 16, the same launches without the dependence between them (`launches_overlapped`,
 evidence only), the unmodified call site (`drop_in_reference_format`), the prefill
 shapes at M = 2048 for both activation types (`prefill_m2048`), the 2B-shaped model's decode
@@ -729,8 +729,8 @@ def main():
     ap.add_argument("--m", type=int, default=8, help="activation rows per call (decode batch)")
     ap.add_argument("--layers", type=int, default=30, help="distinct weight copies per matrix")
     ap.add_argument("--workload", choices=["decode", "prefill", "model", "sweep", "midm"], default="decode",
-                    help="decode: the headline small-M HBM-bound pass (plus, unless --no-extras, every other figure the "
-                         "path is judged on); prefill: the M>=256 MFMA-bound pass; model: random-init BitNet-2B-shaped "
+                    help="decode: the headline small-M HBM-bound pass (plus, unless --no-extras, every other figure of the "
+                         "path); prefill: the M>=256 MFMA-bound pass; model: random-init BitNet-2B-shaped "
                          "decoder, 128-token prompt + 256 greedy tokens; sweep: the sparsity / structure sweep at M=16; "
                          "midm: both kernel families at the batch sizes between decode and prefill")
     ap.add_argument("--batch", type=int, default=1, help="sequences decoded together (model workload)")
