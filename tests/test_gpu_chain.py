@@ -82,6 +82,27 @@ def test_row_stats(m, k):
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 8])
 @pytest.mark.parametrize("n,k,ws_num", [(3840, 2560, 3), (2560, 2560, 1), (2560, 6912, 1), (256, 192, 2)])
 def test_stats_prologue_with_store_and_residual_epilogues(m, n, k, ws_num):
+    _stats_prologue_case(m, n, k, ws_num)
+
+
+def _random_chain_shapes(count, seed):
+    """Seeded shapes nobody tuned for: 1 - 8 rows, N and K any multiple of 64 (K up to 112 k-tiles, the longest the
+    statistics-given kernels take), weight-scale groups that divide N."""
+    rng = np.random.default_rng(seed)
+    shapes = []
+    for _ in range(count):
+        n = 64 * int(rng.integers(1, 33))
+        k = 64 * int(rng.choice([rng.integers(1, 13), rng.integers(13, 41), rng.integers(41, 113)]))
+        shapes.append((int(rng.integers(1, 9)), n, k, int(rng.choice([g for g in (1, 2, 3, 4) if n % g == 0]))))
+    return shapes
+
+
+@pytest.mark.parametrize("m,n,k,ws_num", _random_chain_shapes(16, 20260901))
+def test_stats_prologue_random_shapes(m, n, k, ws_num):
+    _stats_prologue_case(m, n, k, ws_num)
+
+
+def _stats_prologue_case(m, n, k, ws_num):
     w = make_ternary(n, k, 0.40, 1210 + m + n)
     packed = _packed(w)
     h = make_bf16_activations(m, k, 1211 + m + k, outlier_frac=0.01)
@@ -110,7 +131,7 @@ def test_stats_prologue_with_store_and_residual_epilogues(m, n, k, ws_num):
     assert (_bits(out2) == h_next).all()
     _check_stats(st_out.cpu().numpy(), h_next, nxt, 16)
     # ... and the consumer of THAT: statistics from the producing epilogue, not from ternaspmm_row_stats
-    if n in (2560,):
+    if n <= 2560:
         w2 = make_ternary(256, n, 0.40, 1215 + m)
         p2 = _packed(w2)
         r = L.fused_linear(out2, _bf(nxt), 1e-5, p2, ws, 1, 256, n, stats=st_out, publish=True)

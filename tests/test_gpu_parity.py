@@ -516,6 +516,43 @@ def test_packed_kernel_choice_boundaries(lib, m, n, k, ws_num, with_ws):
     _check_bf16(_run_packed_ws(lib, "bf16", packed, n, x, None, scale, ws_num, 0, work)[:, cols], ref)
 
 
+def _random_shapes(count, seed):
+    """Seeded shapes off the beaten track: N and K any multiple of 64 (N up to 1536: 96 bands, K up to 40 k-tiles), M on
+    both sides of every kernel cut, one to four weight-scale groups."""
+    rng = np.random.default_rng(seed)
+    shapes = []
+    for i in range(count):
+        n = 64 * int(rng.integers(1, 25))
+        k = 64 * int(rng.integers(1, 41))
+        m = int(rng.choice([rng.integers(1, 17), rng.integers(17, 65), rng.integers(65, 200), rng.integers(200, 420)]))
+        ws_num = int(rng.choice([g for g in (1, 2, 3, 4) if n % g == 0]))          # groups that divide N, as every caller's do
+        shapes.append((m, n, k, ws_num, float(rng.choice([0.2, 0.4, 0.6])), 9000 + i))
+    return shapes
+
+
+@pytest.mark.parametrize("m,n,k,ws_num,p0,seed", _random_shapes(24, 20260900))
+def test_random_shapes_int8_bit_exact_on_every_route(lib, m, n, k, ws_num, p0, seed):
+    """Shapes nobody tuned for, through the reference's entry point (with and without its workspace) and through the P2
+    entry points (default route with and without scratch, both forced kernels): the integers of every route are the
+    oracle's, bit for bit, under the epilogue rule that route follows."""
+    w = make_ternary(n, k, p0, seed)
+    fmt = DeviceFormat(w)
+    xq, s = make_int8_activations(m, k, seed + 1)
+    if m > 2:
+        s = s.copy()
+        s[m // 3] = 0                                                    # a row whose scale is zero
+    by_m = O.spmm_i8(xq, w, s, WS, ws_num, 0 if m <= 64 else 1)
+    for workspace in (True, False):
+        assert (run_i8(lib, fmt, xq, s, WS, ws_num, workspace=workspace) == by_m).all(), f"reference entry point, workspace={workspace}"
+    packed = repack(lib, fmt)
+    work = torch.empty(8 * m * n * 4, dtype=torch.int8, device="cuda")
+    assert (_run_packed_ws(lib, "int8", packed, n, xq, s, WS, ws_num, 0, None) == by_m).all(), "P2, default route"
+    assert (_run_packed_ws(lib, "int8", packed, n, xq, s, WS, ws_num, 0, work) == by_m).all(), "P2, default route, scratch"
+    assert (run_i8_packed(lib, packed, n, xq, s, WS, ws_num, 1) == O.spmm_i8(xq, w, s, WS, ws_num, 1)).all(), "P2, MFMA-tiled kernel"
+    if m <= 64:
+        assert (run_i8_packed(lib, packed, n, xq, s, WS, ws_num, 2) == by_m).all(), "P2, small-M kernel"
+
+
 # ------------------------------------------------------------------------------- P2 layout (load-time repack)
 @pytest.mark.parametrize("kind", ["iid40", "skewed", "dense", "empty", "sparse97"])
 def test_repack_is_bit_exact(lib, kind):
