@@ -141,7 +141,17 @@ template <typename Act>
 bool launch_prefill_packed(const Act* x, const uint32_t* packed, uint16_t* out, const Epilogue& ep, int M, int N, int K,
                            void* scratch, size_t scratch_bytes, hipStream_t st, const RepackGuard* guard)
 {
-    const PrefillPlan plan = plan_prefill_packed<Act>(x, M, N, K, scratch, scratch_bytes);
+    PrefillPlan plan = plan_prefill_packed<Act>(x, M, N, K, scratch, scratch_bytes);
+    if (plan.direct_lds && !(plan.bm == 64 && plan.bn == 128) && !epilogue_scales_per_tile(ep, N)) {
+        // weight-scale groups that change inside a 32-feature tile: only the 128 x 64 instantiation carries the per-column
+        // epilogue (unsplit: it then uses no more scratch than the plan reported)
+        plan.bm = 64;
+        plan.bn = 128;
+        plan.grid_x = static_cast<unsigned>((N + 127) / 128);
+        plan.grid_y = static_cast<unsigned>((M + 63) / 64);
+        plan.splits = 1;
+        plan.scratch_used = 0;
+    }
     if (plan.direct_lds) {
         if (plan.grid_y >= 65535u) guard = nullptr;         // (no room for the checking row: the caller launches the check itself)
         if (plan.bm == 64 && plan.bn == 128) launch_prefill_packed_dma_as<Act, 2, 1>(x, packed, out, ep, M, N, K, plan, scratch, st, guard);

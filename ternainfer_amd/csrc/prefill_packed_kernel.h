@@ -62,7 +62,17 @@ struct OutTile {
 // twice the true sum (weights were +-2; x0.5 is exact); an integer one is the sum times 64 (weights were +-64; >> 6 is exact).
 // `tile`: this wave's OutTile<NA>::kBytes of LDS (results leave as whole rows; needs out and N * 2 to be multiples of
 // 16 bytes), or nullptr (every lane stores its 8-byte pieces itself).
-template <int MB, int NA, typename AccV>
+// One weight-group scale per 32-feature tile: always under the per-128-column rule of the prefill epilogue and with one
+// group, otherwise when the group boundaries fall on multiples of 32.  (Host and device: the launcher picks a kernel by it.)
+__host__ __device__ inline bool epilogue_scales_per_tile(const Epilogue& ep, int N)
+{
+    return ep.kind == EP_I8_PREFILL || ep.ws_num == 1 || (N == 3840 && ep.ws_num == 3) || (N / ep.ws_num) % 32 == 0;
+}
+
+// COLS = false leaves out the per-column path (scales that change inside a 32-feature tile): unrolled next to 64 - 128 live
+// accumulators it spilled up to 88 registers, so every launch of the larger tiles carried scratch memory for a path that
+// almost no call takes.  The launcher sends such calls to the 128 x 64 instantiation, which keeps the path.
+template <int MB, int NA, typename AccV, bool COLS = true>
 __device__ __forceinline__ void packed_prefill_epilogue(AccV (&acc)[NA][MB], uint16_t* __restrict__ out,
                                                         const Epilogue& ep, int M, int N, int n_wave, int m0, int lane,
                                                         uint8_t* tile = nullptr)
@@ -116,8 +126,7 @@ __device__ __forceinline__ void packed_prefill_epilogue(AccV (&acc)[NA][MB], uin
     // 32 (always for the per-128-column rule of the prefill epilogue): the per-element work is then
     // one multiply (bf16 family, prefill rule) or one divide and one multiply (decode rule), with
     // the same operations in the same order as apply_epilogue.
-    const bool tile_groups = ep.kind == EP_I8_PREFILL || ep.ws_num == 1 || (N == 3840 && ep.ws_num == 3) ||
-                             (N / ep.ws_num) % 32 == 0;
+    const bool tile_groups = !COLS || epilogue_scales_per_tile(ep, N);
     if (tile_groups) {
         float w_of[NA];
         static_for<0, NA>([&](auto ac) {
@@ -161,7 +170,7 @@ __device__ __forceinline__ void packed_prefill_epilogue(AccV (&acc)[NA][MB], uin
         return;
     }
     // group boundaries inside a tile: per-column scales
-    static_for<0, MB>([&](auto bc) {
+    if constexpr (COLS) static_for<0, MB>([&](auto bc) {
         constexpr int b = decltype(bc)::value;
         static_for<0, 4 * NA>([&](auto tc) {
             constexpr int a = decltype(tc)::value >> 2, vq = decltype(tc)::value & 3;
@@ -647,8 +656,8 @@ __global__ __launch_bounds__(256, MB * NA <= 4 ? 4 : (MB * NA <= 8 ? 2 : 1)) voi
     }
     // ... for the final results whenever 16-byte stores can address the output
     const bool rows_ok = ((reinterpret_cast<uintptr_t>(out) | (static_cast<uintptr_t>(N) * 2)) & 15) == 0;
-    packed_prefill_epilogue<MB, NA>(acc, out, ep, M, N, n0 + 32 * NA * wave, m0, lane,
-                                    rows_ok ? smem + wave * OutTile<NA>::kBytes : nullptr);
+    packed_prefill_epilogue<MB, NA, AccV, MB == 2 && NA == 1>(acc, out, ep, M, N, n0 + 32 * NA * wave, m0, lane,
+                                                                rows_ok ? smem + wave * OutTile<NA>::kBytes : nullptr);
 }
 
 // Second launch of a split-K call: out[m][n0 .. n0+3] = epilogue(sum over the splits, in split order, of partial[z][m][n]).

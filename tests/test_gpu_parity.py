@@ -634,6 +634,25 @@ def test_packed_bf16_2b_layer_shapes(lib, m, n, k):
     _check_bf16(got[:, cols], ref)
 
 
+@pytest.mark.parametrize("m,with_ws", [(2560, False), (2560, True), (300, True)])
+def test_packed_bf16_scale_groups_inside_a_tile_at_large_m(lib, m, with_ws):
+    """Four weight-scale groups of 1072 features: the boundaries fall in the middle of a 32-feature tile, so every
+    column takes its own scale.  Only the 128 x 64 tile of the MFMA kernel carries that epilogue; a call the planner would
+    give 256-wide tiles (M = 2560: 680 of them) or split-K planes (M = 300 with scratch) must end up there too."""
+    n, k, ws_num = 4288, 128, 4
+    w = make_ternary(n, k, 0.40, 480 + m)
+    packed = repack(lib, DeviceFormat(w))
+    x = make_bf16_activations(m, k, 481 + m)
+    scale = np.array([0.7, 1.9, 1.3, 0.45], np.float32)
+    work = torch.empty(8 * m * n * 4, dtype=torch.int8, device="cuda") if with_ws else None
+    got = _run_packed_ws(lib, "bf16", packed, n, x, None, scale, ws_num, 1, work)
+    near = np.concatenate([np.arange(b - 40, b + 40) for b in (1072, 2144, 3216)])
+    cols = np.unique(np.concatenate([near, np.random.default_rng(482).permutation(n)[:128], [0, n - 1]]))
+    ref = O.bf16_bits_to_f32(x).astype(np.float64) @ w[cols].astype(np.float64).T * \
+        scale[O.ws_group_decode(cols, n, ws_num)].astype(np.float64)[None, :]
+    _check_bf16(got[:, cols], ref)
+
+
 def test_large_m_with_workspace_matches_without(lib):
     """The transcode-into-workspace route and the fused route compute the same sums in a different
     order; both must sit within tolerance of the golden, and the int8 family must agree bit for bit."""
