@@ -292,6 +292,24 @@ def test_prefill_attention(lib, b, h, kv, d, s_max, first, t):
     prefill_attention_case(lib, b, h, kv, d, s_max, first, t)
 
 
+def _random_prefill_attention_shapes(count, seed):
+    rng = np.random.default_rng(seed)
+    shapes = []
+    for _ in range(count):
+        kv, group = int(rng.choice([1, 2, 3, 5])), int(rng.choice([1, 2, 3, 4, 8]))
+        t = int(rng.choice([rng.integers(1, 17), rng.integers(17, 130), rng.integers(130, 400)]))
+        first = int(rng.choice([0, rng.integers(1, 300)]))
+        shapes.append((int(rng.integers(1, 4)), kv * group, kv, int(rng.choice([64, 128])), first + t + int(rng.integers(0, 40)), first, t))
+    return shapes
+
+
+@pytest.mark.parametrize("b,h,kv,d,s_max,first,t", _random_prefill_attention_shapes(12, 20260904))
+def test_prefill_attention_random_shapes(lib, b, h, kv, d, s_max, first, t):
+    """Seeded shapes nobody tuned for: 1 - 8 query heads per kv head (3: the one-wave-per-head kernel), 1 - 400 new tokens
+    behind prefixes of 0 - 300 slots, caches that end anywhere."""
+    prefill_attention_case(lib, b, h, kv, d, s_max, first, t)
+
+
 def test_prefill_attention_kernels_give_the_same_bits(lib):
     """The grouped kernel (query heads of a kv head in one workgroup, keys / values through LDS) against the one-wave
     kernel, which a child process selects through the tuning override: same arithmetic in the same order, so the
