@@ -278,6 +278,60 @@ def test_quantise_launch_and_quantised_prologue(m, n, k):
     _check_stats(st.cpu().numpy(), h_next, nxt, 16)
 
 
+def _random_quantised_shapes(count, seed, gate):
+    """Seeded shapes for the linears on quantised rows: 1 - 16 rows, N any multiple of 64 (gate: F any multiple of 32, N = 2 F),
+    K any multiple of 64 up to what the epilogue takes (gate: 6144)."""
+    rng = np.random.default_rng(seed)
+    shapes = []
+    for _ in range(count):
+        m = int(rng.choice([rng.integers(1, 9), rng.integers(9, 17)]))
+        k = 64 * int(rng.choice([rng.integers(1, 13), rng.integers(13, 97 if gate else 113)]))
+        shapes.append((m, 32 * int(rng.integers(1, 65)) if gate else 64 * int(rng.integers(1, 41)), k))
+    return shapes
+
+
+@pytest.mark.parametrize("m,n,k", _random_quantised_shapes(12, 20260905, False))
+def test_quantised_prologue_residual_random_shapes(m, n, k):
+    """ternaspmm_quant_from_stats + the linear on its rows with the residual epilogue, on shapes nobody tuned for: the
+    integers exact on the published (xq, s), the stream and the partials of the next norm as for the other producers."""
+    w = make_ternary(n, k, 0.40, 1280 + m + n)
+    packed = _packed(w)
+    h = make_bf16_activations(m, k, 1281 + m + k, outlier_frac=0.01)
+    g, nxt = _weight(k, 1282 + k), _weight(n, 1283 + n)
+    res = make_bf16_activations(m, n, 1284 + m + n)
+    xq, s = L.quant_from_stats(_bf(h), L.row_stats(_bf(h), _bf(g)), _bf(g), 1e-5)
+    print(f"[case] quantised prologue, residual epilogue, random shape: m={m} n={n} k={k}", flush=True)
+    r = L.fused_linear(xq, None, 1e-5, packed, _bf(WS), 1, n, k, quantised=s, epilogue=L.EPILOGUE_RESIDUAL, residual=_bf(res),
+                       next_norm_weight=_bf(nxt), want_raw=True)
+    assert r is not None
+    out, st, raw, _, _ = r
+    torch.cuda.synchronize()
+    q, sb = xq.cpu().numpy(), _bits(s)
+    _check_quantiser(h, g, q, sb)
+    want = O.spmm_i8(q, w, sb, WS, 1, 0)
+    assert (_bits(raw) == want).all()
+    h_next = O.residual_add(res, want)
+    assert (_bits(out) == h_next).all()
+    _check_stats(st.cpu().numpy(), h_next, nxt, 16)
+
+
+@pytest.mark.parametrize("m,f,k", _random_quantised_shapes(12, 20260906, True))
+def test_quantised_prologue_gate_random_shapes(m, f, k):
+    n = 2 * f
+    w13 = make_ternary(n, k, 0.40, 1290 + m + f)
+    inter = L.interleave_gate_up(_packed(w13), n, k)
+    h = make_bf16_activations(m, k, 1291 + m + k, outlier_frac=0.01)
+    g, nxt = _weight(k, 1292 + k), _weight(f, 1293 + f)
+    xq, s, _ = L.rmsnorm_quant(_bf(h), _bf(g), 1e-5)
+    print(f"[case] quantised prologue, gate epilogue, random shape: m={m} f={f} k={k}", flush=True)
+    r = L.fused_linear(xq, None, 1e-5, inter, _bf(WS), 2, n, k, quantised=s, epilogue=L.EPILOGUE_GATE, next_norm_weight=_bf(nxt))
+    assert r is not None
+    torch.cuda.synchronize()
+    want = O.relu2_mul(O.spmm_i8(xq.cpu().numpy(), w13, _bits(s), WS, 2, 0))
+    assert r[0].shape == (m, f) and (_bits(r[0]) == want).all()
+    _check_stats(r[1].cpu().numpy(), want, nxt, 16)
+
+
 def test_unsupported_combinations_are_declined():
     n, k = 256, 192
     packed = _packed(make_ternary(n, k, 0.4, 1250))
