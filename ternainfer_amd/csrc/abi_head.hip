@@ -49,7 +49,13 @@ void ternaspmm_lm_head_bf16(const terna_bf16* x, const terna_bf16* w, terna_bf16
         std::fprintf(stderr, "ternaspmm_lm_head_bf16: unsupported arguments (M=%d V=%d K=%d)\n", M, V, K);
         return;
     }
-    const size_t lds = lm_head_lds_bytes(M, K);
+    // the unpadded layout where it buys a second workgroup per CU (TERNASPMM_LM_HEAD_SWIZZLE=0 keeps the padded one)
+    static const bool swizzle_on = [] {
+        const char* v = tuning_env("TERNASPMM_LM_HEAD_SWIZZLE");
+        return !(v && std::atoi(v) == 0);
+    }();
+    const bool swizzled = swizzle_on && M > 4 && (K & 63) == 0 && lm_head_lds_bytes(M, K) > 80 * 1024 && lm_head_lds_bytes_swizzled(M, K) <= 80 * 1024;
+    const size_t lds = swizzled ? lm_head_lds_bytes_swizzled(M, K) : lm_head_lds_bytes(M, K);
     if (lds > 160 * 1024) {
         std::fprintf(stderr, "ternaspmm_lm_head_bf16: M=%d rows of K=%d do not fit the 160 KB of LDS\n", M, K);
         return;
@@ -79,7 +85,7 @@ void ternaspmm_lm_head_bf16(const terna_bf16* x, const terna_bf16* w, terna_bf16
             terna_lm_head_quad_kernel<8><<<qgrid, dim3(kLmWaves * 64), lds, static_cast<hipStream_t>(stream)>>>(x, w, logits, M, V, K);
         }
     } else {
-        terna_lm_head_kernel<<<dim3(grid), dim3(kLmWaves * 64), lds, static_cast<hipStream_t>(stream)>>>(x, w, logits, M, V, K);
+        terna_lm_head_kernel<<<dim3(grid), dim3(kLmWaves * 64), lds, static_cast<hipStream_t>(stream)>>>(x, w, logits, M, V, K, swizzled ? 1 : 0);
     }
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_lm_head_bf16", e, __LINE__);

@@ -19,26 +19,34 @@ constexpr int kLmWaves = 4;
 constexpr int kLmUnroll = 16;                    // k-steps of 32 in flight per lane (16 bytes each)
 
 constexpr size_t lm_head_lds_bytes(int M, int K) { return static_cast<size_t>(M) * (K * 2 + 16); }
+// Rows without padding, the 16-byte piece c of row r at position c ^ (r & 7) instead (the same spread over the banks; K a
+// multiple of 64 so that a piece's partner is in the row): 16 rows of K = 2560 are then 80 KB, and two workgroups fit a CU.
+constexpr size_t lm_head_lds_bytes_swizzled(int M, int K) { return static_cast<size_t>(M) * K * 2; }
 
 __global__ __launch_bounds__(kLmWaves * 64) void terna_lm_head_kernel(const uint16_t* __restrict__ x,
                                                                       const uint16_t* __restrict__ w,
-                                                                      uint16_t* __restrict__ logits, int M, int V, int K)
+                                                                      uint16_t* __restrict__ logits, int M, int V, int K, int swizzled)
 {
-    extern __shared__ __align__(16) uint8_t xs[];            // [M][K * 2 + 16]: padded pitch
+    extern __shared__ __align__(16) uint8_t xs[];            // [M][K * 2 + 16]: padded pitch, or [M][K * 2] swizzled
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int pitch = K * 2 + 16;
+    const int pitch = swizzled ? K * 2 : K * 2 + 16;
     const int row_vecs = K >> 3;                             // 16-byte pieces per row
     for (int p = tid; p < M * row_vecs; p += kLmWaves * 64) {
         const int r = p / row_vecs, c = p - r * row_vecs;
-        *reinterpret_cast<u32x4*>(xs + r * pitch + 16 * c) = *reinterpret_cast<const u32x4*>(x + static_cast<size_t>(r) * K + 8 * c);
+        *reinterpret_cast<u32x4*>(xs + r * pitch + 16 * (swizzled ? c ^ (r & 7) : c)) =
+            *reinterpret_cast<const u32x4*>(x + static_cast<size_t>(r) * K + 8 * c);
     }
     __syncthreads();
 
     const int i = lane & 15, kg = lane >> 4;
     const int steps = K >> 5;
     const bool live = i < M;
-    const uint8_t* xrow = xs + (live ? i : 0) * pitch + 16 * kg;   // B operand: batch row i, chunk kg of each step
+    // B operand: batch row i, chunk kg of each step = piece 4 s + kg of the row; swizzled: (4 s + kg) ^ (i & 7), i.e. chunk
+    // kg ^ (i & 3) of step s ^ ((i >> 2) & 1)
+    const int row_b = live ? i : 0;
+    const uint8_t* xrow = xs + row_b * pitch + 16 * (swizzled ? kg ^ (row_b & 3) : kg);
+    const int step_flip = swizzled ? (row_b >> 2) & 1 : 0;
     const int blocks = (V + 15) >> 4;
     const bool wide_store = (V & 3) == 0 && (reinterpret_cast<uintptr_t>(logits) & 7) == 0;   // 8-byte stores of four logits
     for (int blk = blockIdx.x * kLmWaves + wave; blk < blocks; blk += gridDim.x * kLmWaves) {
@@ -55,7 +63,7 @@ __global__ __launch_bounds__(kLmWaves * 64) void terna_lm_head_kernel(const uint
 #pragma unroll
             for (int u = 0; u < kLmUnroll; ++u) {
                 const int s = s0 + u;
-                u32x4 b = *reinterpret_cast<const u32x4*>(xrow + 64 * (s < steps ? s : steps - 1));
+                u32x4 b = *reinterpret_cast<const u32x4*>(xrow + 64 * ((s < steps ? s : steps - 1) ^ step_flip));
                 if (s >= steps || !live) b = u32x4{0u, 0u, 0u, 0u};
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[u]), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
             }
