@@ -74,7 +74,21 @@ void ternaspmm_lm_head_bf16(const terna_bf16* x, const terna_bf16* w, terna_bf16
         return v ? std::atoi(v) : 1;
     }();
     const int ksteps = K / 128;
-    if (quad && M <= 4 && (K & 127) == 0) {
+    static const bool quad32 = [] {                     // TERNASPMM_LM_HEAD_QUAD32=0: 5 - 8 rows through the 16-row kernel
+        const char* v = tuning_env("TERNASPMM_LM_HEAD_QUAD32");
+        return !(v && std::atoi(v) == 0);
+    }();
+    if (quad && quad32 && M > 4 && M <= 8 && (K & 63) == 0) {
+        const int qwgs = ((V + 7) / 8 + kLmWaves - 1) / kLmWaves;
+        const dim3 qgrid(qwgs < cap ? qwgs : cap);
+        if ((K / 64) % 10 == 0) {
+            if (lds > 64 * 1024) allow_dynamic_lds(terna_lm_head_quad32_kernel<10>, 160 * 1024, "hipFuncSetAttribute(lm head)", __LINE__);
+            terna_lm_head_quad32_kernel<10><<<qgrid, dim3(kLmWaves * 64), lds, static_cast<hipStream_t>(stream)>>>(x, w, logits, M, V, K);
+        } else {
+            if (lds > 64 * 1024) allow_dynamic_lds(terna_lm_head_quad32_kernel<8>, 160 * 1024, "hipFuncSetAttribute(lm head)", __LINE__);
+            terna_lm_head_quad32_kernel<8><<<qgrid, dim3(kLmWaves * 64), lds, static_cast<hipStream_t>(stream)>>>(x, w, logits, M, V, K);
+        }
+    } else if (quad && M <= 4 && (K & 127) == 0) {
         const int qwgs = ((V + 3) / 4 + kLmWaves - 1) / kLmWaves;
         const dim3 qgrid(qwgs < cap ? qwgs : cap);
         if (ksteps % 10 == 0) {

@@ -142,4 +142,67 @@ __global__ __launch_bounds__(kLmWaves * 64) void terna_lm_head_quad_kernel(const
     }
 }
 
+// Five to eight rows of activations: the same trick on the 32 x 32 x 16 MFMA, whose 32 columns hold eight batch rows of four
+// partials each.  Row i of A: vocabulary row i / 4 (eight per operand), the 16-byte pieces (i % 4) + 4 (L >> 5) of a
+// 128-byte step; column 4 m + r of B: batch row m's pieces r + 4 (L >> 5); out[i][4 m + i % 4] is a partial logit, and the
+// four partials of (vocabulary row, batch row) meet in the four lanes of a quad.  Four consecutive lanes load 64 consecutive
+// bytes, as above.  UNROLL loads of a lane are in flight; it should divide K / 64.
+template <int UNROLL>
+__global__ __launch_bounds__(kLmWaves * 64) void terna_lm_head_quad32_kernel(const uint16_t* __restrict__ x,
+                                                                             const uint16_t* __restrict__ w,
+                                                                             uint16_t* __restrict__ logits, int M, int V, int K)
+{
+    extern __shared__ __align__(16) uint8_t xs[];            // [M][K * 2 + 16]: padded pitch
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int pitch = K * 2 + 16;
+    const int row_vecs = K >> 3;
+    for (int p = tid; p < M * row_vecs; p += kLmWaves * 64) {
+        const int r = p / row_vecs, c = p - r * row_vecs;
+        *reinterpret_cast<u32x4*>(xs + r * pitch + 16 * c) = *reinterpret_cast<const u32x4*>(x + static_cast<size_t>(r) * K + 8 * c);
+    }
+    __syncthreads();
+
+    const int i = lane & 31, hb = lane >> 5;
+    const int piece = (i & 3) + 4 * hb;                      // 16 bytes of a 128-byte step of a row (A and B alike)
+    const int steps = K >> 6;
+    const int m = i >> 2;                                    // B column i: batch row i / 4
+    const bool live = m < M;
+    const uint8_t* xrow = xs + (live ? m : 0) * pitch + 16 * piece;
+    const int blocks = (V + 7) >> 3;
+    for (int blk = blockIdx.x * kLmWaves + wave; blk < blocks; blk += gridDim.x * kLmWaves) {
+        const int row = blk * 8 + (i >> 2);
+        const uint16_t* wrow = w + static_cast<size_t>(row < V ? row : V - 1) * K + 8 * piece;
+        f32x16 acc;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[e] = 0.0f;
+        for (int s0 = 0; s0 < steps; s0 += UNROLL) {
+            u32x4 a[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const int s = s0 + u < steps ? s0 + u : steps - 1;
+                a[u] = *reinterpret_cast<const u32x4*>(wrow + 64 * s);
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const int s = s0 + u;
+                u32x4 b = *reinterpret_cast<const u32x4*>(xrow + 128 * (s < steps ? s : steps - 1));
+                if (s >= steps || !live) b = u32x4{0u, 0u, 0u, 0u};
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[u]), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
+            }
+        }
+        // lane (column i, half hb) holds rows (e & 3) + 8 (e >> 2) + 4 hb: row 4 q + r with r = e & 3, q = 2 (e >> 2) + hb, i.e.
+        // vocabulary row blk * 8 + q, pieces r (mod 4): its partial for batch row m is in column 4 m + r -- element r + 4 t
+        // of the lane whose column has i % 4 == r
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            float part = (i & 3) == 0 ? acc[4 * t] : (i & 3) == 1 ? acc[4 * t + 1] : (i & 3) == 2 ? acc[4 * t + 2] : acc[4 * t + 3];
+            part += dpp_permute<kDppSwapPairs>(part);
+            part += dpp_permute<kDppSwapHalfQuads>(part);
+            const int v = blk * 8 + 2 * t + hb;
+            if ((i & 3) == 0 && live && v < V) logits[static_cast<size_t>(m) * V + v] = float_to_bf16_bits(part);
+        }
+    }
+}
+
 }  // namespace terna

@@ -162,12 +162,13 @@ def test_argmax_rows(lib, b, v):
 
 @pytest.mark.parametrize("m,v,k", [(1, 128256, 2560), (8, 128256, 2560), (16, 4096, 2560), (3, 1003, 64), (2, 50, 32),
                                    (5, 8200, 6912), (16, 640, 4128), (3, 1003, 384), (4, 8200, 6912), (1, 50, 128),
-                                   (4, 128256, 2560), (2, 4098, 2176)])
+                                   (4, 128256, 2560), (2, 4098, 2176), (7, 1003, 192), (6, 4098, 2176), (5, 50, 64)])
 def test_lm_head_against_fp64(lib, m, v, k):
     """bf16 LM head: within the bf16 GEMM bar of the fp64 product (max|err| <= 1e-2 max|ref|, median <= 1 ULP
     of the bf16 result), also for V not a multiple of 16 or 4, K that is not a multiple of the unrolled
     depth, and K whose 16 activation rows need more than 64 KB of LDS.  Up to four rows with K a multiple of 128
-    take the kernel whose quads of lanes load 64 contiguous bytes, everything else the plain one."""
+    take the kernel whose quads of lanes load 64 contiguous bytes, five to eight rows with K a multiple of 64 its form on
+    the 32 x 32 MFMA, everything else the plain one."""
     import ternainfer_amd as T
     rng = np.random.default_rng(4100 + m + v + k)
     x = O.f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
