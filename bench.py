@@ -263,6 +263,8 @@ def measure_model(torch, batch, act="int8", prefetch=True, gen_tokens=256, check
         model.attention_splits = int(os.environ["TERNA_BENCH_ATTN_SPLITS"])
     if os.environ.get("TERNA_BENCH_SPLIT_MERGE_QUANT"):
         model.split_merge_quant = os.environ["TERNA_BENCH_SPLIT_MERGE_QUANT"] != "0"
+    if os.environ.get("TERNA_BENCH_STEP_INPUTS"):
+        model.step_inputs = os.environ["TERNA_BENCH_STEP_INPUTS"] != "0"
     if os.environ.get("TERNA_BENCH_DEFER_ABOVE"):
         model.defer_above = int(os.environ["TERNA_BENCH_DEFER_ABOVE"])
     if os.environ.get("TERNA_BENCH_ATTENTION_STATS"):

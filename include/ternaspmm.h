@@ -324,6 +324,17 @@ int ternaspmm_quant_from_stats(const terna_bf16* h, const float* stats, int stat
 int ternaspmm_row_stats_count(int K);
 int ternaspmm_row_stats(const terna_bf16* h, const terna_bf16* norm_weight, float* stats_out, int M, int K, terna_stream stream);
 
+/* The inputs of a single-token step in one launch (the reference: the embedding lookup of model.py:367's tied matrix and
+ * the rows of the RoPE table, two framework launches): x_out bf16 [B][K] = embedding[tokens[b]] (embedding bf16 [V][K]) with
+ * its partials stats_out fp32 [B][ternaspmm_row_stats_count(K)][2] under norm_weight, exactly as ternaspmm_row_stats leaves
+ * them, and rope_out fp32 [2][B][rope_half] = the cos rows, then the sin rows, of rope_table fp32 [S][2][rope_half] at
+ * pos[b] (per_sequence) or pos[0] (tokens, pos: int64 in device memory; values outside their table are clamped).
+ * K a multiple of 8, rope_half a multiple of 4 up to 512, 16-byte aligned tables and outputs.  Returns the partial count or
+ * -1.  Only enqueues. */
+int ternaspmm_step_inputs(const long long* tokens, const long long* pos, int per_sequence, const terna_bf16* embedding, int V, int K,
+                          const float* rope_table, int S, int rope_half, const terna_bf16* norm_weight, terna_bf16* x_out,
+                          float* stats_out, float* rope_out, int B, terna_stream stream);
+
 /* Load time: band permutation of a P2 gate+up matrix [w1; w3] ([N][K], N = 2F) for TERNASPMM_EPILOGUE_GATE -- band 2j <-
  * rows 16j .. 16j+15 of w1, band 2j+1 <- the same rows of w3.  packed_out: N*K/4 bytes, not `packed`.  Returns 0 / -1. */
 int ternaspmm_interleave_gate_up(const void* packed, void* packed_out, int N, int K, terna_stream stream);

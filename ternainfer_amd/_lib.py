@@ -84,6 +84,7 @@ PROTOTYPES = {
     "ternaspmm_row_stats_count": ([_ci], _ci),
     "ternaspmm_row_stats": ([_vp, _vp, _vp, _ci, _ci, _vp], _ci),
     "ternaspmm_interleave_gate_up": ([_vp, _vp, _ci, _ci, _vp], _ci),
+    "ternaspmm_step_inputs": ([_vp, _vp, _ci, _vp, _ci, _ci, _vp, _ci, _ci, _vp, _vp, _vp, _vp, _ci, _vp], _ci),
     "ternaspmm_version": ([], ctypes.c_char_p),
 }
 

@@ -43,6 +43,48 @@ __global__ __launch_bounds__(256) void terna_row_stats_kernel(const uint16_t* __
     }
 }
 
+// The inputs of a single-token step in one launch: x_out[b] = embedding[tokens[b]] with its partials under norm_w (as
+// terna_row_stats_kernel leaves them), and the rows of the RoPE table at the sequences' positions, cos rows then sin rows
+// (rope_out [2][B][half]; table [S][2][half]).  A token or position outside its table is clamped (device memory the host
+// cannot check).  One workgroup of 256 threads per sequence.
+__global__ __launch_bounds__(256) void terna_step_inputs_kernel(const long long* __restrict__ tokens, const long long* __restrict__ pos,
+                                                                 int per_seq, const uint16_t* __restrict__ embedding, int V, int K,
+                                                                 const float* __restrict__ rope_table, int S, int half,
+                                                                 const uint16_t* __restrict__ norm_w, uint16_t* __restrict__ x_out,
+                                                                 float2* __restrict__ stats_out, float* __restrict__ rope_out, int count)
+{
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int b = blockIdx.x, B = gridDim.x;
+    long long t = tokens[b], p = pos[per_seq ? b : 0];
+    t = t < 0 ? 0 : (t >= V ? V - 1 : t);
+    p = p < 0 ? 0 : (p >= S ? S - 1 : p);
+    const uint16_t* row = embedding + static_cast<size_t>(t) * K;
+    if (tid < 2 * half / 4) {                           // half is a multiple of 4: 16-byte pieces, cos row then sin row
+        const int which = tid / (half / 4), piece = tid - which * (half / 4);
+        const f32x4 v = *reinterpret_cast<const f32x4*>(rope_table + (static_cast<size_t>(p) * 2 + which) * half + 4 * piece);
+        *reinterpret_cast<f32x4*>(rope_out + (static_cast<size_t>(which) * B + b) * half + 4 * piece) = v;
+    }
+    for (int part = wave; part < count; part += 4) {
+        const int c = part * 512 + lane * 8;
+        float ssq = 0.0f, pmax = 0.0f;
+        if (c < K) {                                    // K is a multiple of 8
+            const u32x4 hv = *reinterpret_cast<const u32x4*>(row + c);
+            *reinterpret_cast<u32x4*>(x_out + static_cast<size_t>(b) * K + c) = hv;
+            float f[8], w[8];
+            unpack_bf16x8(hv, f);
+            unpack_bf16x8(*reinterpret_cast<const u32x4*>(norm_w + c), w);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                ssq = fmaf(f[e], f[e], ssq);
+                pmax = fmaxf(pmax, fabsf(__fmul_rn(f[e], w[e])));
+            }
+        }
+        ssq = wave_sum(ssq);
+        pmax = wave_max(pmax);
+        if (lane == 0) stats_out[static_cast<size_t>(b) * count + part] = float2{ssq, pmax};
+    }
+}
+
 // Band permutation of a P2 gate+up matrix ([w1; w3], N = 2F rows) for the FEPI_GLU epilogue: band 2j <- band j (rows
 // 16j .. of w1), band 2j + 1 <- band F/16 + j (the same rows of w3).  One workgroup per destination band.
 __global__ __launch_bounds__(256) void terna_interleave_gate_up_kernel(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst,
@@ -313,6 +355,27 @@ int ternaspmm_row_stats(const terna_bf16* h, const terna_bf16* norm_weight, floa
     terna_row_stats_kernel<<<dim3(M), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(h, norm_weight, reinterpret_cast<float2*>(stats_out), K, count);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) die("ternaspmm_row_stats", e, __LINE__);
+    return count;
+}
+
+int ternaspmm_step_inputs(const long long* tokens, const long long* pos, int per_sequence, const terna_bf16* embedding, int V, int K,
+                          const float* rope_table, int S, int rope_half, const terna_bf16* norm_weight, terna_bf16* x_out,
+                          float* stats_out, float* rope_out, int B, terna_stream stream)
+{
+    const int count = ternaspmm_row_stats_count(K);
+    if (B < 1 || B > 65535 || V < 1 || S < 1 || count < 1 || count > kStatsMaxPartials || rope_half < 4 || (rope_half & 3) || rope_half > 512 ||
+        tokens == nullptr || pos == nullptr || embedding == nullptr || rope_table == nullptr || norm_weight == nullptr || x_out == nullptr ||
+        stats_out == nullptr || rope_out == nullptr ||
+        ((reinterpret_cast<uintptr_t>(embedding) | reinterpret_cast<uintptr_t>(x_out) | reinterpret_cast<uintptr_t>(norm_weight) |
+          reinterpret_cast<uintptr_t>(rope_table) | reinterpret_cast<uintptr_t>(rope_out)) & 15)) {
+        std::fprintf(stderr, "ternaspmm_step_inputs: unsupported arguments (B=%d V=%d K=%d S=%d rope_half=%d)\n", B, V, K, S, rope_half);
+        return -1;
+    }
+    terna_step_inputs_kernel<<<dim3(B), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+        tokens, pos, per_sequence != 0, embedding, V, K, rope_table, S, rope_half, norm_weight, x_out, reinterpret_cast<float2*>(stats_out),
+        rope_out, count);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) die("ternaspmm_step_inputs", e, __LINE__);
     return count;
 }
 

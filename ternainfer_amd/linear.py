@@ -307,6 +307,32 @@ def row_stats(h, norm_weight):
     return out
 
 
+def step_inputs(tokens, pos, embedding, rope_table, norm_weight):
+    """The inputs of a single-token step in one launch (ternaspmm_step_inputs): tokens int64 [B] (any shape with B
+    elements), pos int64 [1] (one position for all) or [B], embedding bf16 [V, K], rope_table fp32 [S, 2, half].
+    Returns (x bf16 [B, K], partials fp32 [B, count, 2] under `norm_weight`, cos fp32 [B, half], sin fp32 [B, half])."""
+    b = tokens.numel()
+    v, k = embedding.shape
+    s_len, two, half = rope_table.shape
+    if tokens.dtype != torch.int64 or pos.dtype != torch.int64 or pos.numel() not in (1, b) or two != 2 or rope_table.dtype != torch.float32 \
+            or embedding.dtype != torch.bfloat16 or not (tokens.is_contiguous() and pos.is_contiguous() and embedding.is_contiguous()
+                                                         and rope_table.is_contiguous()):
+        raise ValueError("step_inputs: tokens / pos int64, embedding bf16 [V, K], rope_table fp32 [S, 2, half], all contiguous")
+    _check_rows("step_inputs", embedding, norm_weight=(norm_weight, k))
+    lib = _lib.load()
+    count = lib.ternaspmm_row_stats_count(k)
+    if count < 1:
+        raise ValueError(f"step_inputs: unsupported K={k}")
+    x = torch.empty((b, k), dtype=torch.bfloat16, device=embedding.device)
+    stats = torch.empty((b, count, 2), dtype=torch.float32, device=embedding.device)
+    rope = torch.empty((2, b, half), dtype=torch.float32, device=embedding.device)
+    got = lib.ternaspmm_step_inputs(_p(tokens), _p(pos), int(pos.numel() == b and b > 1), _p(embedding), v, k, _p(rope_table), s_len, half,
+                                    _p(norm_weight), _p(x), _p(stats), _p(rope), b, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    if got != count:
+        raise ValueError(f"step_inputs: the library refused the launch (B={b} V={v} K={k} S={s_len} half={half})")
+    return x, stats, rope[0], rope[1]
+
+
 def quant_from_stats(h, stats, norm_weight, eps):
     """Norm + quant_input of h bf16 [M, K] from the partials its producer left (ternaspmm_quant_from_stats):
     (xq int8 [M, K], s bf16 [M])."""

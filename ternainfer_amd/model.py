@@ -23,7 +23,7 @@ from torch.nn import functional as F
 
 from . import _lib
 from .linear import (EPILOGUE_GATE, EPILOGUE_RESIDUAL, argmax_rows, attention_merge_rmsnorm_linear_packed, attention_merge_rmsnorm_quant, fused_linear, get_global_workspace, greedy_step,
-                     greedy_step_state, interleave_gate_up, lm_head, quant_from_stats, quant_input, row_stats, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant,
+                     greedy_step_state, interleave_gate_up, lm_head, quant_from_stats, quant_input, row_stats, relu2_mul_rmsnorm_linear_packed, relu2_mul_rmsnorm_quant, step_inputs,
                      repack_weight, rmsnorm_linear_packed, rmsnorm_quant)
 
 
@@ -576,22 +576,27 @@ class Transformer:
         bsz, t = tokens.shape
         max_seq = cache[0][0].shape[2]
         dev = tokens.device
-        rows = self.rope_tables(max_seq, dev).index_select(0, pos_idx.reshape(-1))   # fp32 [T | B*T, 2, head_dim / 2]
-        cos, sin = rows[:, 0].contiguous(), rows[:, 1].contiguous()           # views when one row
         mask = None
         kernels_fit = self.layers[0].fused and a.head_dim in (64, 128) and max_seq <= 8192 and tokens.is_cuda
         one_launch_attention = kernels_fit and t == 1
+        # one new token for a few sequences: the linears chained through producer-side norm statistics (forward_chain)
+        chain = one_launch_attention and self.layers[0].act == "int8" and bsz <= max(self.chain_rows, self.split_rows) and getattr(self, "chain", True) and self.chain_supported()
+        stats = None
+        if chain and getattr(self, "step_inputs", True):
+            # embedding rows, their partials under the first block's norm and the RoPE rows of the positions: one launch
+            x, stats, cos, sin = step_inputs(tokens, pos_idx.reshape(-1), self.tok_embeddings, self.rope_tables(max_seq, dev), self.layers[0].attention_norm)
+        else:
+            rows = self.rope_tables(max_seq, dev).index_select(0, pos_idx.reshape(-1))   # fp32 [T | B*T, 2, head_dim / 2]
+            cos, sin = rows[:, 0].contiguous(), rows[:, 1].contiguous()       # views when one row
+            x = self.tok_embeddings[tokens.reshape(-1)]
         if kernels_fit and t > 1 and getattr(self, "kernel_prefill_attention", True):
             mask = KERNEL_ATTENTION
         elif not one_launch_attention:
             # causal over cache slots: new token at slot p sees slots <= p
             seen = torch.arange(max_seq, device=dev) <= pos_idx[..., None]    # [T | B, T][S]
             mask = seen[:, None] if pos_idx.dim() == 2 else seen[None, None]
-        x = self.tok_embeddings[tokens.reshape(-1)]
         pending = None
         attn_ws = self.attention_workspace(bsz) if one_launch_attention else None     # layers run one after another: shared
-        # one new token for a few sequences: the linears chained through producer-side norm statistics (forward_chain)
-        chain = one_launch_attention and self.layers[0].act == "int8" and bsz <= max(self.chain_rows, self.split_rows) and getattr(self, "chain", True) and self.chain_supported()
         split = chain and bsz > self.chain_rows
         # split attention whose merge is left to its consumer: always for one sequence (the O projection's prologue merges);
         # for more only with long caches, where the shorter attention launch pays for the merge launch (8 sequences at slot
@@ -603,7 +608,6 @@ class Transformer:
             attn_ws = self.attention_partial(bsz, max_seq) or attn_ws
         elif split and getattr(self, "split_merge_quant", False):
             attn_ws = self.attention_partial(bsz, max_seq, single_split=True) or attn_ws
-        stats = None
         for index, (layer, (ck, cv)) in enumerate(zip(self.layers, cache)):
             x_in, pending_in = x, pending
             if chain:

@@ -79,6 +79,30 @@ def test_row_stats(m, k):
     _check_stats(st, h, g, 512)
 
 
+@pytest.mark.parametrize("b,v,k,s_len,half,per_seq", [(1, 128256, 2560, 384, 64, False), (8, 128256, 2560, 384, 64, False),
+                                                       (5, 1000, 520, 40, 32, True), (16, 300, 64, 2048, 64, True), (3, 50, 6912, 7, 4, True)])
+def test_step_inputs(b, v, k, s_len, half, per_seq):
+    """ternaspmm_step_inputs against the three launches it stands for: the embedding rows (bit copies), their partials
+    exactly as ternaspmm_row_stats leaves them, the RoPE-table rows of the positions (shared or per sequence)."""
+    gen = torch.Generator().manual_seed(1300 + b + k)
+    emb = (torch.randn((v, k), generator=gen) * 0.02).to(torch.bfloat16).cuda()
+    table = torch.randn((s_len, 2, half), generator=gen).cuda()
+    g = _weight(k, 1301 + k)
+    tokens = torch.randint(0, v, (b, 1), generator=gen).cuda()
+    tokens[0, 0] = v - 1
+    pos = torch.randint(0, s_len, (b if per_seq else 1,), generator=gen).cuda()
+    pos[-1] = s_len - 1
+    print(f"[case] step inputs b={b} v={v} k={k} S={s_len} half={half} per_seq={per_seq}", flush=True)
+    x, stats, cos, sin = L.step_inputs(tokens, pos, emb, table, _bf(g))
+    torch.cuda.synchronize()
+    want = emb[tokens.reshape(-1)]
+    assert torch.equal(x, want)
+    assert torch.equal(stats, L.row_stats(want, _bf(g)))
+    rows = table.index_select(0, pos.expand(b) if not per_seq else pos)
+    assert torch.equal(cos, rows[:, 0]) and torch.equal(sin, rows[:, 1])
+    assert cos.is_contiguous() and sin.is_contiguous()
+
+
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 8])
 @pytest.mark.parametrize("n,k,ws_num", [(3840, 2560, 3), (2560, 2560, 1), (2560, 6912, 1), (256, 192, 2)])
 def test_stats_prologue_with_store_and_residual_epilogues(m, n, k, ws_num):
