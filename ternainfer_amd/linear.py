@@ -314,10 +314,10 @@ def step_inputs(tokens, pos, embedding, rope_table, norm_weight):
     b = tokens.numel()
     v, k = embedding.shape
     s_len, two, half = rope_table.shape
+    tokens, pos = tokens.reshape(-1).contiguous(), pos.reshape(-1).contiguous()      # (copies only where a caller passed a strided view)
     if tokens.dtype != torch.int64 or pos.dtype != torch.int64 or pos.numel() not in (1, b) or two != 2 or rope_table.dtype != torch.float32 \
-            or embedding.dtype != torch.bfloat16 or not (tokens.is_contiguous() and pos.is_contiguous() and embedding.is_contiguous()
-                                                         and rope_table.is_contiguous()):
-        raise ValueError("step_inputs: tokens / pos int64, embedding bf16 [V, K], rope_table fp32 [S, 2, half], all contiguous")
+            or embedding.dtype != torch.bfloat16 or not (embedding.is_contiguous() and rope_table.is_contiguous()):
+        raise ValueError("step_inputs: tokens / pos int64, embedding bf16 [V, K] and rope_table fp32 [S, 2, half] contiguous")
     _check_rows("step_inputs", embedding, norm_weight=(norm_weight, k))
     lib = _lib.load()
     count = lib.ternaspmm_row_stats_count(k)
