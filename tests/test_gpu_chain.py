@@ -103,6 +103,32 @@ def test_step_inputs(b, v, k, s_len, half, per_seq):
     assert cos.is_contiguous() and sin.is_contiguous()
 
 
+def test_step_inputs_clamps_and_refuses():
+    """Tokens and positions come from device memory the host cannot check: values outside their tables are clamped, not
+    followed.  Shapes and pointers the kernel cannot take are refused on the host (-1, nothing launched)."""
+    import ctypes
+    from ternainfer_amd import _lib
+    lib = _lib.load()
+    v, k, s_len, half = 40, 128, 16, 8
+    emb = (torch.randn((v, k)) * 0.02).to(torch.bfloat16).cuda()
+    table = torch.randn((s_len, 2, half)).cuda()
+    g = _bf(_weight(k, 1310))
+    tokens = torch.tensor([[-5], [v + 100], [7]], dtype=torch.int64).cuda()
+    pos = torch.tensor([s_len + 3, -1, 2], dtype=torch.int64).cuda()
+    x, stats, cos, sin = L.step_inputs(tokens, pos, emb, table, g)
+    torch.cuda.synchronize()
+    assert torch.equal(x, emb[torch.tensor([0, v - 1, 7]).cuda()])
+    assert torch.equal(cos, table[torch.tensor([s_len - 1, 0, 2]).cuda(), 0]) and torch.equal(sin, table[torch.tensor([s_len - 1, 0, 2]).cuda(), 1])
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    xo, so, ro = torch.empty_like(x), torch.empty_like(stats), torch.empty((2, 3, half), device="cuda")
+    ok = lambda **kw: lib.ternaspmm_step_inputs(p(tokens), p(pos), 1, kw.get("emb", p(emb)), v, kw.get("k", k), p(table), s_len, kw.get("half", half),
+                                                p(g), p(xo), p(so), kw.get("rope", p(ro)), kw.get("b", 3), None)
+    assert ok() == 1
+    assert ok(k=124) == -1 and ok(half=6) == -1 and ok(b=0) == -1 and ok(emb=None) == -1
+    assert ok(rope=ctypes.c_void_p(ro.data_ptr() + 4)) == -1
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 8])
 @pytest.mark.parametrize("n,k,ws_num", [(3840, 2560, 3), (2560, 2560, 1), (2560, 6912, 1), (256, 192, 2)])
 def test_stats_prologue_with_store_and_residual_epilogues(m, n, k, ws_num):
